@@ -1,0 +1,326 @@
+"""TEST INFRASTRUCTURE — ctypes access to the CPU oracle.
+
+Two libraries sit behind this module:
+
+* ``liboracle.so``      — the plain-C restatement of the reference's CPU algorithm (``bb_oracle.c``).
+* ``_ref/libbbref.so``  — the reference's own CPU headers compiled behind ``ref_shim.cpp`` (present only where it
+  was built from the reference tree).
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this module; the
+shipped package never does.  Arrays are numpy, node-major / frame-minor, C-contiguous: fp32 buffers are
+``[nodes, stride]`` float32, bit buffers ``[nodes, stride_words]`` int32 with frame f at word f>>5, bit f&31.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ORACLE_SO = os.path.join(_HERE, "liboracle.so")
+_REF_SO = os.path.join(_HERE, "_ref", "libbbref.so")
+
+_f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+
+
+def build(force=False):
+    """Compile liboracle.so (and _ref/libbbref.so where the reference tree is present)."""
+    if force or not os.path.exists(_ORACLE_SO):
+        subprocess.check_call(["make", "-C", _HERE, "liboracle.so"] + (["-B"] if force else []))
+    if os.path.isdir("/root/reference/include/bb") and (force or not os.path.exists(_REF_SO)):
+        subprocess.check_call(["make", "-C", _HERE, "ref"])
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_ORACLE_SO):
+            build()
+        _lib = C.CDLL(_ORACLE_SO)
+    return _lib
+
+
+def have_ref():
+    return os.path.exists(_REF_SO)
+
+
+def ref():
+    global _ref
+    if _ref is None:
+        _ref = C.CDLL(_REF_SO)
+    return _ref
+
+
+def _c(a, dt):
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+# ----------------------------------------------------------------------------------------------
+#  restatement (liboracle.so)
+# ----------------------------------------------------------------------------------------------
+
+def vector_clamp(src, lo=0.0, hi=1.0):
+    src = _c(src, np.float32)
+    dst = np.empty_like(src)
+    lib().oracle_fp32_Vector_clamp(_ptr(dst), _ptr(src), C.c_float(lo), C.c_float(hi), C.c_int(src.size))
+    return dst
+
+
+def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, simd=True):
+    """fp32 x [I, stride] -> y [O, stride] (padding columns zero)."""
+    x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]; stride = x.shape[1]
+    y = np.zeros((O, stride), np.float32)
+    lib().oracle_fp32_StochasticLut_Forward(C.c_int(n), _ptr(x), _ptr(y), _ptr(idx), _ptr(W), C.c_int(O), C.c_int(frame_size),
+                                            C.c_int(stride), C.c_int(int(input_binary)), C.c_int(int(lut_binarize)),
+                                            C.c_float(bias), C.c_int(int(simd)))
+    return y
+
+
+def bit_stochastic_lut_forward(n, xbits, idx, W, frame_size, y_stride, lut_binarize=False, bias=0.25):
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]
+    y = np.zeros((O, y_stride), np.float32)
+    lib().oracle_bit_fp32_StochasticLut_Forward(C.c_int(n), _ptr(xbits), _ptr(y), _ptr(idx), _ptr(W), C.c_int(O),
+                                                C.c_int(frame_size), C.c_int(y_stride), C.c_int(xbits.shape[1]),
+                                                C.c_int(int(lut_binarize)), C.c_float(bias))
+    return y
+
+
+def bit_bit_stochastic_lut_forward(n, xbits, idx, W, frame_size, lut_binarize=False, bias=0.25):
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]
+    y = np.zeros((O, xbits.shape[1]), np.int32)
+    lib().oracle_bit_bit_fp32_StochasticLut_Forward(C.c_int(n), _ptr(xbits), _ptr(y), _ptr(idx), _ptr(W), C.c_int(O),
+                                                    C.c_int(frame_size), C.c_int(xbits.shape[1]),
+                                                    C.c_int(int(lut_binarize)), C.c_float(bias))
+    return y
+
+
+def stochastic_lut_backward(n, x, dy, idx, W, frame_size, dW_init=None, input_binary=False, lut_binarize=False,
+                            bias=0.25, simd=True):
+    """returns (dx [I, stride], dW [O, 2^n]); dW starts from dW_init (zeros when None)."""
+    x = _c(x, np.float32); dy = _c(dy, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    I, stride = x.shape; O = idx.shape[0]
+    dx = np.zeros((I, stride), np.float32)
+    dW = np.zeros((O, 1 << n), np.float32) if dW_init is None else _c(dW_init, np.float32).copy()
+    lib().oracle_fp32_StochasticLut_Backward(C.c_int(n), _ptr(x), _ptr(dy), _ptr(dx), _ptr(idx), _ptr(W), _ptr(dW),
+                                             C.c_int(I), C.c_int(O), C.c_int(frame_size), C.c_int(stride),
+                                             C.c_int(int(input_binary)), C.c_int(int(lut_binarize)), C.c_float(bias),
+                                             C.c_int(int(simd)))
+    return dx, dW
+
+
+def bit_stochastic_lut_backward(n, xbits, dy, idx, W, frame_size, dW_init=None, lut_binarize=False, bias=0.25):
+    xbits = _c(xbits, np.int32); dy = _c(dy, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    I = xbits.shape[0]; O = idx.shape[0]; stride = dy.shape[1]
+    dx = np.zeros((I, stride), np.float32)
+    dW = np.zeros((O, 1 << n), np.float32) if dW_init is None else _c(dW_init, np.float32).copy()
+    lib().oracle_bit_fp32_StochasticLut_Backward(C.c_int(n), _ptr(xbits), _ptr(dy), _ptr(dx), _ptr(idx), _ptr(W), _ptr(dW),
+                                                 C.c_int(I), C.c_int(O), C.c_int(frame_size), C.c_int(stride),
+                                                 C.c_int(xbits.shape[1]), C.c_int(int(lut_binarize)), C.c_float(bias))
+    return dx, dW
+
+
+def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
+                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True):
+    """fp32 x. returns (y, mean, rstd, running_mean, running_var)."""
+    x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]; stride = x.shape[1]
+    y = np.zeros((O, stride), np.float32)
+    mean = np.zeros(O, np.float32); rstd = np.zeros(O, np.float32)
+    rm = _c(running_mean, np.float32).copy(); rv = _c(running_var, np.float32).copy()
+    lib().oracle_fp32_DifferentiableLutN_ForwardTraining(
+        C.c_int(n), _ptr(x), _ptr(y), _ptr(idx), _ptr(W), _ptr(mean), _ptr(rstd), _ptr(rm), _ptr(rv),
+        C.c_float(gamma), C.c_float(beta), C.c_float(momentum), C.c_float(bias),
+        C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(int(lut_binarize)), C.c_int(int(binary_mode)))
+    return y, mean, rstd, rm, rv
+
+
+def bit_differentiable_lut_forward_training(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
+                                            momentum=0.9, bias=0.25, lut_binarize=False):
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]; stride = xbits.shape[1]
+    y = np.zeros((O, stride), np.int32)
+    mean = np.zeros(O, np.float32); rstd = np.zeros(O, np.float32)
+    rm = _c(running_mean, np.float32).copy(); rv = _c(running_var, np.float32).copy()
+    lib().oracle_bit_fp32_DifferentiableLutN_ForwardTraining(
+        C.c_int(n), _ptr(xbits), _ptr(y), _ptr(idx), _ptr(W), _ptr(mean), _ptr(rstd), _ptr(rm), _ptr(rv),
+        C.c_float(gamma), C.c_float(beta), C.c_float(momentum), C.c_float(bias),
+        C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(int(lut_binarize)))
+    return y, mean, rstd, rm, rv
+
+
+def differentiable_lut_forward_inference(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
+                                         bias=0.25, lut_binarize=False, binary_mode=True):
+    x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]; stride = x.shape[1]
+    y = np.zeros((O, stride), np.float32)
+    rm = _c(running_mean, np.float32); rv = _c(running_var, np.float32)
+    lib().oracle_fp32_DifferentiableLutN_ForwardInference(
+        C.c_int(n), _ptr(x), _ptr(y), _ptr(idx), _ptr(W), _ptr(rm), _ptr(rv),
+        C.c_float(gamma), C.c_float(beta), C.c_float(bias),
+        C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(int(lut_binarize)), C.c_int(int(binary_mode)))
+    return y
+
+
+def bit_differentiable_lut_forward_inference(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3,
+                                             beta=0.5, bias=0.25, lut_binarize=False):
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]; stride = xbits.shape[1]
+    y = np.zeros((O, stride), np.int32)
+    rm = _c(running_mean, np.float32); rv = _c(running_var, np.float32)
+    lib().oracle_bit_fp32_DifferentiableLutN_ForwardInference(
+        C.c_int(n), _ptr(xbits), _ptr(y), _ptr(idx), _ptr(W), _ptr(rm), _ptr(rv),
+        C.c_float(gamma), C.c_float(beta), C.c_float(bias),
+        C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(int(lut_binarize)))
+    return y
+
+
+def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_binarize=False, binary_mode=True):
+    x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    O = idx.shape[0]; stride = x.shape[1]
+    y = np.zeros((O, stride), np.float32)
+    lib().oracle_fp32_DifferentiableLutN_ForwardNoBn(
+        C.c_int(n), _ptr(x), _ptr(y), _ptr(idx), _ptr(W), C.c_float(bias),
+        C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(int(lut_binarize)), C.c_int(int(binary_mode)))
+    return y
+
+
+def differentiable_lut_backward(n, x, dy, idx, W, frame_size, mean, rstd, dW_init=None, gamma=0.3, beta=0.5, bias=0.25,
+                                lut_binarize=False, binary_mode=True):
+    x = _c(x, np.float32); dy = _c(dy, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    I, stride = x.shape; O = idx.shape[0]
+    dx = np.zeros((I, stride), np.float32)
+    dW = np.zeros((O, 1 << n), np.float32) if dW_init is None else _c(dW_init, np.float32).copy()
+    lib().oracle_fp32_DifferentiableLutN_Backward(
+        C.c_int(n), _ptr(x), _ptr(dy), _ptr(dx), _ptr(idx), _ptr(W), _ptr(dW), _ptr(_c(mean, np.float32)),
+        _ptr(_c(rstd, np.float32)), C.c_float(gamma), C.c_float(beta), C.c_float(bias),
+        C.c_int(I), C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(int(lut_binarize)), C.c_int(int(binary_mode)))
+    return dx, dW
+
+
+def bit_differentiable_lut_backward(n, xbits, dy, idx, W, frame_size, mean, rstd, dW_init=None, gamma=0.3, beta=0.5,
+                                    bias=0.25, lut_binarize=False):
+    xbits = _c(xbits, np.int32); dy = _c(dy, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    I = xbits.shape[0]; O = idx.shape[0]; stride = dy.shape[1]
+    dx = np.zeros((I, stride), np.float32)
+    dW = np.zeros((O, 1 << n), np.float32) if dW_init is None else _c(dW_init, np.float32).copy()
+    lib().oracle_bit_fp32_DifferentiableLutN_Backward(
+        C.c_int(n), _ptr(xbits), _ptr(dy), _ptr(dx), _ptr(idx), _ptr(W), _ptr(dW), _ptr(_c(mean, np.float32)),
+        _ptr(_c(rstd, np.float32)), C.c_float(gamma), C.c_float(beta), C.c_float(bias),
+        C.c_int(I), C.c_int(O), C.c_int(frame_size), C.c_int(stride), C.c_int(xbits.shape[1]), C.c_int(int(lut_binarize)))
+    return dx, dW
+
+
+def binary_lut6_forward(xbits, idx, table, frame_size, words=False):
+    """packed x [I, stride_words] int32 -> packed y [O, stride_words]; bits of frames >= frame_size stay zero
+    (generic loop) or are computed from the padding (words=True, the AVX2-shaped loop)."""
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); table = _c(table, np.int32)
+    O = idx.shape[0]; stride = xbits.shape[1]
+    y = np.zeros((O, stride), np.int32)
+    if words:
+        lib().oracle_bit_BinaryLut6_Forward_words(_ptr(xbits), _ptr(y), _ptr(idx), _ptr(table), C.c_int(O),
+                                                  C.c_int((frame_size + 31) // 32), C.c_int(stride))
+    else:
+        lib().oracle_bit_BinaryLut6_Forward(_ptr(xbits), _ptr(y), _ptr(idx), _ptr(table), C.c_int(O),
+                                            C.c_int(frame_size), C.c_int(stride))
+    return y
+
+
+def reverse_table(n, idx, input_node_size):
+    idx = _c(idx, np.int32)
+    O = idx.shape[0]
+    f = lib().oracle_ReverseTable
+    f.restype = C.c_int
+    stride = f(C.c_int(n), _ptr(idx), C.c_int(input_node_size), C.c_int(O), None, C.c_int(0))
+    rev = np.zeros((input_node_size, stride), np.int32)
+    f(C.c_int(n), _ptr(idx), C.c_int(input_node_size), C.c_int(O), _ptr(rev), C.c_int(rev.size))
+    return rev
+
+
+# ----------------------------------------------------------------------------------------------
+#  the real reference headers (oracle/_ref/libbbref.so) — dense [nodes, frames] arrays, no stride
+# ----------------------------------------------------------------------------------------------
+
+def ref_stochastic_lut(n, x, idx, W, dy=None, dW_init=None, bit_input=False, binary_mode=False, lut_binarize=False,
+                       host_simd=True, frame_size=None):
+    """Runs bb::StochasticLutN<n,...>::Forward (+Backward). Returns dict(y, W, dx, dW)."""
+    idx = _c(idx, np.int32); W = _c(W, np.float32).copy()
+    O = idx.shape[0]
+    if bit_input:
+        x = _c(x, np.int32); I = x.shape[0]; F = frame_size
+        assert x.shape[1] == (F + 31) // 32
+    else:
+        x = _c(x, np.float32); I, F = x.shape
+    y = np.zeros((O, F), np.float32)
+    dx = np.zeros((I, F), np.float32) if dy is not None else None
+    dW = None
+    if dy is not None:
+        dy = _c(dy, np.float32)
+        dW = np.zeros((O, 1 << n), np.float32) if dW_init is None else _c(dW_init, np.float32).copy()
+    rc = ref().bbref_StochasticLut(C.c_int(n), C.c_int(int(bit_input)), C.c_int(I), C.c_int(O), C.c_int(F),
+                                   _ptr(x), _ptr(idx), _ptr(W), _ptr(dy), _ptr(y), _ptr(dx), _ptr(dW),
+                                   C.c_int(int(binary_mode)), C.c_int(int(lut_binarize)), C.c_int(int(host_simd)))
+    assert rc == 0
+    return dict(y=y, W=W, dx=dx, dW=dW)
+
+
+def ref_differentiable_lut(n, x, idx, W, running_mean, running_var, dy=None, dW_init=None, bit_input=False,
+                           gamma=0.3, beta=0.5, momentum=0.9, batch_norm=True, binary_mode=True, lut_binarize=False,
+                           train=True, frame_size=None):
+    idx = _c(idx, np.int32); W = _c(W, np.float32).copy()
+    O = idx.shape[0]
+    if bit_input:
+        x = _c(x, np.int32); I = x.shape[0]; F = frame_size
+        y = np.zeros((O, (F + 31) // 32), np.int32)
+    else:
+        x = _c(x, np.float32); I, F = x.shape
+        y = np.zeros((O, F), np.float32)
+    dx = np.zeros((I, F), np.float32) if dy is not None else None
+    dW = None
+    if dy is not None:
+        dy = _c(dy, np.float32)
+        dW = np.zeros((O, 1 << n), np.float32) if dW_init is None else _c(dW_init, np.float32).copy()
+    mean = np.zeros(O, np.float32); rstd = np.zeros(O, np.float32)
+    rm = _c(running_mean, np.float32).copy(); rv = _c(running_var, np.float32).copy()
+    rc = ref().bbref_DifferentiableLut(C.c_int(n), C.c_int(int(bit_input)), C.c_int(I), C.c_int(O), C.c_int(F),
+                                       _ptr(x), _ptr(idx), _ptr(W), _ptr(dy), _ptr(y), _ptr(dx), _ptr(dW),
+                                       _ptr(mean), _ptr(rstd), _ptr(rm), _ptr(rv),
+                                       C.c_float(gamma), C.c_float(beta), C.c_float(momentum),
+                                       C.c_int(int(batch_norm)), C.c_int(int(binary_mode)), C.c_int(int(lut_binarize)),
+                                       C.c_int(int(train)))
+    assert rc == 0
+    return dict(y=y, W=W, dx=dx, dW=dW, mean=mean, rstd=rstd, running_mean=rm, running_var=rv)
+
+
+def ref_binary_lut6(xbits, idx, table, frame_size, host_simd=True):
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); table = _c(table, np.int32)
+    I = xbits.shape[0]; O = idx.shape[0]
+    assert xbits.shape[1] == (frame_size + 31) // 32
+    y = np.zeros((O, xbits.shape[1]), np.int32)
+    rc = ref().bbref_BinaryLut6(C.c_int(I), C.c_int(O), C.c_int(frame_size), _ptr(xbits), _ptr(idx), _ptr(table), _ptr(y),
+                                C.c_int(int(host_simd)))
+    assert rc == 0
+    return y
+
+
+def ref_reverse_table6(idx, input_node_size):
+    idx = _c(idx, np.int32)
+    O = idx.shape[0]
+    f = ref().bbref_ReverseTable6
+    f.restype = C.c_int
+    stride = f(C.c_int(input_node_size), C.c_int(O), _ptr(idx), None, C.c_int(0))
+    rev = np.zeros((input_node_size, stride), np.int32)
+    f(C.c_int(input_node_size), C.c_int(O), _ptr(idx), _ptr(rev), C.c_int(rev.size))
+    return rev

@@ -1,0 +1,640 @@
+/*
+ * TEST INFRASTRUCTURE — CPU oracle for the differentiable-LUT hot path.
+ *
+ * This file is a plain-C restatement of BinaryBrain's *CPU* implementation of
+ * StochasticLutN / DifferentiableLutN / BinaryLutN<6> and of the connection
+ * reverse table.  It exists so that parity tests, the smoke check and the
+ * cpu_baseline leg of the benchmark have a fixed side to compare the HIP
+ * library against on machines where the reference tree is absent.  Nothing in
+ * the shipped library may call it.
+ *
+ * Build: gcc -O2 -mavx2 -mfma -fopenmp -ffp-contract=off (see oracle/Makefile).
+ * -ffp-contract=off keeps every multiply/add a separate IEEE operation; fused
+ * multiply-adds appear only where the reference uses _mm256_fmadd_ps and are
+ * written as fmaf().
+ *
+ * How each function is pinned (tests/test_oracle_*.py):
+ *   - *_StochasticLut_Forward/Backward, simd order : bit-exact against the real
+ *     reference headers (oracle/_ref) where that library is built, against the
+ *     committed vectors in tests/golden/ elsewhere, plus closed forms
+ *     (x in {0,1}^N picks W[index]; constant W; sum_i dW[i] = sum_f dy;
+ *     multilinear finite differences for dx) and an fp64 brute force.
+ *   - generic order, DifferentiableLutN *: same vectors with a few-ulp
+ *     tolerance (the reference's generic loops are subject to the compiler's
+ *     contraction choices), textbook mean/variance, BN gradient invariants.
+ *   - BinaryLut6, reverse table: bit-exact against oracle/_ref and golden
+ *     vectors; BinaryLut6 also against StochasticLut with W,x in {0,1}.
+ *
+ * Array conventions (the reference's FrameBuffer layout, include/bb/FrameBuffer.h:28-46,
+ * 927-939): node-major, frame-minor; element (node n, frame f) of an fp32
+ * buffer is p[n*stride + f]; of a bit buffer, bit (f & 31) of the 32-bit word
+ * p[n*stride_words + (f >> 5)] (include/bb/DataType.h:612-647).
+ */
+
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define MAXN   6
+#define MAXNN  64
+
+static inline float clamp01(float v) { return fminf(1.0f, fmaxf(0.0f, v)); }
+
+/* include/bb/StochasticOperation.h:95-114 */
+static inline float lut_forward_generic(float const *x, float const *W, int N)
+{
+    float acc = 0.0f;
+    for (int i = 0; i < (1 << N); ++i) {
+        float w = W[i];
+        for (int j = 0; j < N; ++j) {
+            w *= ((i >> j) & 1) ? x[j] : (1.0f - x[j]);
+        }
+        acc += w;
+    }
+    return acc;
+}
+
+/* include/bb/StochasticOperation.h:118-152 */
+static inline void lut_backward_generic(float const *x, float *dx, float dy, float const *W, float *dW, int N)
+{
+    for (int i = 0; i < (1 << N); ++i) {
+        float dw = dy;
+        for (int j = 0; j < N; ++j) {
+            dw *= ((i >> j) & 1) ? x[j] : (1.0f - x[j]);
+        }
+        dW[i] += dw;
+    }
+    for (int i = 0; i < N; ++i) {
+        dx[i] = 0;
+        for (int j = 0; j < (1 << N); ++j) {
+            float w = ((j >> i) & 1) ? +W[j] : -W[j];
+            for (int k = 0; k < N; ++k) {
+                if (i != k) {
+                    w *= ((j >> k) & 1) ? x[k] : (1.0f - x[k]);
+                }
+            }
+            dx[i] += w;
+        }
+        dx[i] *= dy;
+    }
+}
+
+/* One frame of simd_fp32_StochasticLut6_Forward (include/bb/StochasticLutSimd.h:77-154):
+ * pair products xk_ab = x[2k+1]? * x[2k]?, then y = W0*(x2*(x1*x0)) followed by 63 fmadd in index order. */
+static inline float lut6_forward_simd_order(float const xp[6], float const W[64])
+{
+    float xn[6], pr[3][4];
+    for (int i = 0; i < 6; ++i) { xn[i] = 1.0f - xp[i]; }
+    for (int k = 0; k < 3; ++k) {
+        pr[k][0] = xn[2 * k + 1] * xn[2 * k];
+        pr[k][1] = xn[2 * k + 1] * xp[2 * k];
+        pr[k][2] = xp[2 * k + 1] * xn[2 * k];
+        pr[k][3] = xp[2 * k + 1] * xp[2 * k];
+    }
+    float y = 0.0f;
+    for (int i = 0; i < 64; ++i) {
+        float p = pr[2][(i >> 4) & 3] * (pr[1][(i >> 2) & 3] * pr[0][i & 3]);
+        y = (i == 0) ? (W[0] * p) : fmaf(W[i], p, y);
+    }
+    return y;
+}
+
+/* One frame of simd_fp32_StochasticLut6_Backward (StochasticLutSimd.h:240-433). dWacc is the per-lane accumulator. */
+static inline void lut6_backward_simd_order(float const xp[6], float grad, float const W[64], float dWacc[64], float dx[6])
+{
+    float xn[6], pr[3][4], d[3][4];
+    for (int i = 0; i < 6; ++i) { xn[i] = 1.0f - xp[i]; }
+    for (int k = 0; k < 3; ++k) {
+        pr[k][0] = xn[2 * k + 1] * xn[2 * k];
+        pr[k][1] = xn[2 * k + 1] * xp[2 * k];
+        pr[k][2] = xp[2 * k + 1] * xn[2 * k];
+        pr[k][3] = xp[2 * k + 1] * xp[2 * k];
+        d[k][0] = d[k][1] = d[k][2] = d[k][3] = 0.0f;
+    }
+    for (int i = 0; i < 64; ++i) {
+        float p = pr[2][(i >> 4) & 3] * (pr[1][(i >> 2) & 3] * pr[0][i & 3]);
+        dWacc[i] = fmaf(grad, p, dWacc[i]);
+    }
+    for (int i = 0; i < 64; ++i) {
+        int a = i & 3, b = (i >> 2) & 3, c = (i >> 4) & 3;
+        float dxi = W[i] * grad;
+        d[0][a] = fmaf(dxi, pr[2][c] * pr[1][b], d[0][a]);
+        d[1][b] = fmaf(dxi, pr[2][c] * pr[0][a], d[1][b]);
+        d[2][c] = fmaf(dxi, pr[1][b] * pr[0][a], d[2][c]);
+    }
+    for (int k = 0; k < 3; ++k) {
+        /* even input of the pair (StochasticLutSimd.h:399-403, 411-415, 423-427) */
+        float dxn = d[k][0] * xn[2 * k + 1];
+        dxn = fmaf(d[k][2], xp[2 * k + 1], dxn);
+        float dxp = d[k][1] * xn[2 * k + 1];
+        dxp = fmaf(d[k][3], xp[2 * k + 1], dxp);
+        dx[2 * k] = dxp - dxn;
+        /* odd input of the pair (:405-409, 417-421, 429-433) */
+        dxn = d[k][0] * xn[2 * k];
+        dxn = fmaf(d[k][1], xp[2 * k], dxn);
+        dxp = d[k][2] * xn[2 * k];
+        dxp = fmaf(d[k][3], xp[2 * k], dxp);
+        dx[2 * k + 1] = dxp - dxn;
+    }
+}
+
+/* bb_mm256_hsum_ps (include/bb/SimdSupport.h:93-100): ((a0+a1)+(a2+a3)) + ((a4+a5)+(a6+a7)) */
+static inline float hsum8(float const a[8])
+{
+    return ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+}
+
+static inline float read_x_fp32(float const *row, int f, int input_binary, float bias)
+{
+    float v = row[f];
+    if (input_binary) { return 0.5f + ((v > 0.5f) ? +bias : -bias); }
+    return clamp01(v);
+}
+
+static inline int read_bit(int32_t const *row, int f)
+{
+    return (int)(((uint32_t)row[f >> 5] >> (f & 31)) & 1u);
+}
+
+static inline float read_x_bit(int32_t const *row, int f, float bias)
+{
+    float v = read_bit(row, f) ? 1.0f : 0.0f;
+    return 0.5f + ((v > 0.5f) ? +bias : -bias);
+}
+
+static inline void write_bit(int32_t *row, int f, int v)
+{
+    uint32_t m = 1u << (f & 31);
+    uint32_t w = (uint32_t)row[f >> 5];
+    row[f >> 5] = (int32_t)(v ? (w | m) : (w & ~m));
+}
+
+static void load_W(float *Wl, float const *W, int node, int NN, int lut_binarize)
+{
+    for (int i = 0; i < NN; ++i) {
+        float w = W[(size_t)node * NN + i];
+        if (lut_binarize) { w = (w > 0.5f) ? 1.0f : 0.0f; }
+        Wl[i] = w;
+    }
+}
+
+
+/* Tensor::Clamp_inplace as used on W (include/bb/StochasticLutN.h:451) */
+void oracle_fp32_Vector_clamp(float *dst, float const *src, float lo, float hi, int size)
+{
+    for (int i = 0; i < size; ++i) { dst[i] = fminf(hi, fmaxf(lo, src[i])); }
+}
+
+
+/* StochasticLutN<N,float>::Forward, host path (include/bb/StochasticLutN.h:504-559).
+ * simd != 0 and n == 6 selects the AVX2 association (StochasticLutSimd.h:25-163). W is used as given. */
+void oracle_fp32_StochasticLut_Forward(int n, float const *x, float *y, int32_t const *idx, float const *W,
+                                       int node_size, int frame_size, int frame_stride,
+                                       int input_binary, int lut_binarize, float bias, int simd)
+{
+    int const NN = 1 << n;
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        float Wl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = read_x_fp32(x + (size_t)idx[node * n + i] * frame_stride, f, input_binary, bias);
+            }
+            float v = (simd && n == 6) ? lut6_forward_simd_order(xv, Wl) : lut_forward_generic(xv, Wl, n);
+            if (simd && n == 6) { v = fminf(fmaxf(v, 0.0f), 1.0f); }       /* StochasticLutSimd.h:157-158 */
+            else                { v = fmaxf(0.0f, v); v = fminf(1.0f, v); } /* StochasticLutN.h:551-552 */
+            y[(size_t)node * frame_stride + f] = v;
+        }
+    }
+}
+
+/* StochasticLutN<N,Bit>::Forward generic path: x bit-packed, y fp32 (StochasticLutN.h:512-559) */
+void oracle_bit_fp32_StochasticLut_Forward(int n, int32_t const *x, float *y, int32_t const *idx, float const *W,
+                                           int node_size, int frame_size, int frame_stride, int bin_frame_stride,
+                                           int lut_binarize, float bias)
+{
+    int const NN = 1 << n;
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        float Wl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = read_x_bit(x + (size_t)idx[node * n + i] * bin_frame_stride, f, bias);
+            }
+            float v = lut_forward_generic(xv, Wl, n);
+            v = fmaxf(0.0f, v); v = fminf(1.0f, v);
+            y[(size_t)node * frame_stride + f] = v;
+        }
+    }
+}
+
+/* DifferentiableLutN<N,Bit> forward without batch-norm: bit in, bit out, y = (LUT > 0.5)
+ * (include/bb/DifferentiableLutN.h:959-1008 with BinType = Bit). Bits of frames >= frame_size are left untouched. */
+void oracle_bit_bit_fp32_StochasticLut_Forward(int n, int32_t const *x, int32_t *y, int32_t const *idx, float const *W,
+                                               int node_size, int frame_size, int frame_stride,
+                                               int lut_binarize, float bias)
+{
+    int const NN = 1 << n;
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        float Wl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = read_x_bit(x + (size_t)idx[node * n + i] * frame_stride, f, bias);
+            }
+            float v = lut_forward_generic(xv, Wl, n);
+            write_bit(y + (size_t)node * frame_stride, f, v > 0.5f);
+        }
+    }
+}
+
+
+static void backward_core(int n, float const *x_fp32, int32_t const *x_bit, float const *dy, float *dx,
+                          int32_t const *idx, float const *W, float *dW,
+                          int input_node_size, int output_node_size, int frame_size,
+                          int frame_stride, int bin_frame_stride,
+                          int input_binary, int lut_binarize, float bias, int simd)
+{
+    int const NN = 1 << n;
+    size_t const tmp_rows = (size_t)output_node_size * n;
+    float *tmp = (float *)malloc(sizeof(float) * tmp_rows * (size_t)frame_size);
+
+    #pragma omp parallel for
+    for (int node = 0; node < output_node_size; ++node) {
+        float Wl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        if (simd && n == 6 && !x_bit) {
+            /* StochasticLutSimd.h:195-440: 8 independent lanes over frames, horizontal sum at the end */
+            float acc[8][64];
+            memset(acc, 0, sizeof(acc));
+            for (int f = 0; f < frame_size; ++f) {
+                float xv[6], dxv[6];
+                for (int i = 0; i < 6; ++i) {
+                    xv[i] = read_x_fp32(x_fp32 + (size_t)idx[node * 6 + i] * frame_stride, f, input_binary, bias);
+                }
+                lut6_backward_simd_order(xv, dy[(size_t)node * frame_stride + f], Wl, acc[f & 7], dxv);
+                for (int i = 0; i < 6; ++i) { tmp[((size_t)node * 6 + i) * frame_size + f] = dxv[i]; }
+            }
+            for (int i = 0; i < 64; ++i) {
+                float lanes[8];
+                for (int l = 0; l < 8; ++l) { lanes[l] = acc[l][i]; }
+                dW[(size_t)node * 64 + i] += hsum8(lanes);
+            }
+        }
+        else {
+            /* StochasticLutN.h:692-736 */
+            float dWl[MAXNN];
+            memset(dWl, 0, sizeof(dWl));
+            for (int f = 0; f < frame_size; ++f) {
+                float xv[MAXN], dxv[MAXN];
+                for (int i = 0; i < n; ++i) {
+                    int in = idx[node * n + i];
+                    xv[i] = x_bit ? read_x_bit(x_bit + (size_t)in * bin_frame_stride, f, bias)
+                                  : read_x_fp32(x_fp32 + (size_t)in * frame_stride, f, input_binary, bias);
+                }
+                lut_backward_generic(xv, dxv, dy[(size_t)node * frame_stride + f], Wl, dWl, n);
+                for (int i = 0; i < n; ++i) { tmp[((size_t)node * n + i) * frame_size + f] = dxv[i]; }
+            }
+            for (int i = 0; i < NN; ++i) { dW[(size_t)node * NN + i] += dWl[i]; }
+        }
+    }
+
+    /* integrate: zero-filled dx, contributions added in ascending (node, input) order
+     * (StochasticLutSimd.h:179, 442-454; StochasticLutN.h:680, 738-749) */
+    for (int in = 0; in < input_node_size; ++in) {
+        memset(dx + (size_t)in * frame_stride, 0, sizeof(float) * (size_t)frame_size);
+    }
+    #pragma omp parallel for
+    for (int f = 0; f < frame_size; ++f) {
+        for (int node = 0; node < output_node_size; ++node) {
+            for (int i = 0; i < n; ++i) {
+                dx[(size_t)idx[node * n + i] * frame_stride + f] += tmp[((size_t)node * n + i) * frame_size + f];
+            }
+        }
+    }
+    free(tmp);
+}
+
+/* StochasticLutN<N,float>::Backward host path (StochasticLutN.h:668-752). dW accumulates; dx is overwritten. */
+void oracle_fp32_StochasticLut_Backward(int n, float const *x, float const *dy, float *dx, int32_t const *idx,
+                                        float const *W, float *dW,
+                                        int input_node_size, int output_node_size, int frame_size, int frame_stride,
+                                        int input_binary, int lut_binarize, float bias, int simd)
+{
+    backward_core(n, x, NULL, dy, dx, idx, W, dW, input_node_size, output_node_size, frame_size,
+                  frame_stride, 0, input_binary, lut_binarize, bias, simd);
+}
+
+/* StochasticLutN<N,Bit>::Backward generic path */
+void oracle_bit_fp32_StochasticLut_Backward(int n, int32_t const *x, float const *dy, float *dx, int32_t const *idx,
+                                            float const *W, float *dW,
+                                            int input_node_size, int output_node_size, int frame_size,
+                                            int frame_stride, int bin_frame_stride, int lut_binarize, float bias)
+{
+    backward_core(n, NULL, x, dy, dx, idx, W, dW, input_node_size, output_node_size, frame_size,
+                  frame_stride, bin_frame_stride, 1, lut_binarize, bias, 0);
+}
+
+
+/* ---- DifferentiableLutN ------------------------------------------------------------------ */
+
+static inline float dl_read_x(float const *x_fp32, int32_t const *x_bit, int in, int f,
+                              int frame_stride, int bin_frame_stride, int binary_mode, float bias)
+{
+    float v = x_bit ? (read_bit(x_bit + (size_t)in * bin_frame_stride, f) ? 1.0f : 0.0f)
+                    : x_fp32[(size_t)in * frame_stride + f];
+    if (binary_mode) { return 0.5f + ((v > 0.5f) ? +bias : -bias); }
+    return clamp01(v);
+}
+
+static inline float dl_activate(float v, int binary_mode)
+{
+    if (binary_mode) { return (v > 0.5f) ? 1.0f : 0.0f; }
+    v = fminf(v, 1.0f);
+    v = fmaxf(v, 0.0f);
+    return v;
+}
+
+static void dl_forward_core(int n, float const *x_fp32, int32_t const *x_bit, float *y_fp32, int32_t *y_bit,
+                            int32_t const *idx, float const *W,
+                            float *mean_out, float *rstd_out, float *running_mean, float *running_var,
+                            float gamma, float beta, float momentum, float bias,
+                            int node_size, int frame_size, int frame_stride, int bin_frame_stride,
+                            int lut_binarize, int binary_mode, int train)
+{
+    int const NN = 1 << n;
+    float const reciprocal_frame_size = 1.0f / (float)frame_size;
+
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        float Wl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        float mean, rstd;
+        if (train) {
+            /* include/bb/DifferentiableLutN.h:775-812: Kahan-compensated sums in frame order */
+            float s1 = 0, c1 = 0, y1, t1;
+            float s2 = 0, c2 = 0, y2, t2;
+            for (int f = 0; f < frame_size; ++f) {
+                float xv[MAXN];
+                for (int i = 0; i < n; ++i) {
+                    xv[i] = dl_read_x(x_fp32, x_bit, idx[node * n + i], f, frame_stride, bin_frame_stride, binary_mode, bias);
+                }
+                float v = lut_forward_generic(xv, Wl, n);
+                y1 = v - c1;       t1 = s1 + y1; c1 = (t1 - s1) - y1; s1 = t1;
+                y2 = (v * v) - c2; t2 = s2 + y2; c2 = (t2 - s2) - y2; s2 = t2;
+            }
+            mean = s1 * reciprocal_frame_size;
+            float var = fmaxf(1.0e-5f, (s2 * reciprocal_frame_size) - (mean * mean));
+            rstd = 1.0f / sqrtf(var);
+            running_mean[node] = running_mean[node] * momentum + mean * (1.0f - momentum);
+            running_var[node]  = running_var[node]  * momentum + var  * (1.0f - momentum);
+            mean_out[node] = mean;
+            rstd_out[node] = rstd;
+        }
+        else {
+            /* :866-868 */
+            mean = running_mean[node];
+            rstd = 1.0f / sqrtf(running_var[node]);
+        }
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = dl_read_x(x_fp32, x_bit, idx[node * n + i], f, frame_stride, bin_frame_stride, binary_mode, bias);
+            }
+            float v = lut_forward_generic(xv, Wl, n);
+            v = (v - mean) * rstd;
+            v = v * gamma + beta;
+            v = dl_activate(v, binary_mode);
+            if (y_bit) { write_bit(y_bit + (size_t)node * bin_frame_stride, f, v != 0.0f); }
+            else       { y_fp32[(size_t)node * frame_stride + f] = v; }
+        }
+    }
+}
+
+/* DifferentiableLutN<N,float>::Forward(train=true), batch_norm on (DifferentiableLutN.h:754-847) */
+void oracle_fp32_DifferentiableLutN_ForwardTraining(int n, float const *x, float *y, int32_t const *idx, float const *W,
+        float *mean, float *rstd, float *running_mean, float *running_var,
+        float gamma, float beta, float momentum, float bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode)
+{
+    dl_forward_core(n, x, NULL, y, NULL, idx, W, mean, rstd, running_mean, running_var, gamma, beta, momentum, bias,
+                    node_size, frame_size, frame_stride, 0, lut_binarize, binary_mode, 1);
+}
+
+/* DifferentiableLutN<N,Bit>::Forward(train=true): bit in, bit out; binary_mode is forced on for Bit (:116-118) */
+void oracle_bit_fp32_DifferentiableLutN_ForwardTraining(int n, int32_t const *x, int32_t *y, int32_t const *idx, float const *W,
+        float *mean, float *rstd, float *running_mean, float *running_var,
+        float gamma, float beta, float momentum, float bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize)
+{
+    dl_forward_core(n, NULL, x, NULL, y, idx, W, mean, rstd, running_mean, running_var, gamma, beta, momentum, bias,
+                    node_size, frame_size, 0, frame_stride, lut_binarize, 1, 1);
+}
+
+/* DifferentiableLutN::Forward(train=false), batch_norm on (:848-902) */
+void oracle_fp32_DifferentiableLutN_ForwardInference(int n, float const *x, float *y, int32_t const *idx, float const *W,
+        float const *running_mean, float const *running_var,
+        float gamma, float beta, float bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode)
+{
+    dl_forward_core(n, x, NULL, y, NULL, idx, W, NULL, NULL, (float *)running_mean, (float *)running_var, gamma, beta, 0.0f, bias,
+                    node_size, frame_size, frame_stride, 0, lut_binarize, binary_mode, 0);
+}
+
+void oracle_bit_fp32_DifferentiableLutN_ForwardInference(int n, int32_t const *x, int32_t *y, int32_t const *idx, float const *W,
+        float const *running_mean, float const *running_var,
+        float gamma, float beta, float bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize)
+{
+    dl_forward_core(n, NULL, x, NULL, y, idx, W, NULL, NULL, (float *)running_mean, (float *)running_var, gamma, beta, 0.0f, bias,
+                    node_size, frame_size, 0, frame_stride, lut_binarize, 1, 0);
+}
+
+/* DifferentiableLutN<N,float> forward without batch-norm (:959-1008): out = binary ? (y > 0.5) : clip(y, 0, 1) */
+void oracle_fp32_DifferentiableLutN_ForwardNoBn(int n, float const *x, float *y, int32_t const *idx, float const *W,
+        float bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode)
+{
+    int const NN = 1 << n;
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        float Wl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = dl_read_x(x, NULL, idx[node * n + i], f, frame_stride, 0, binary_mode, bias);
+            }
+            y[(size_t)node * frame_stride + f] = dl_activate(lut_forward_generic(xv, Wl, n), binary_mode);
+        }
+    }
+}
+
+static void dl_backward_core(int n, float const *x_fp32, int32_t const *x_bit, float const *dy, float *dx,
+                             int32_t const *idx, float const *W, float *dW,
+                             float const *mean_in, float const *rstd_in,
+                             float gamma, float beta, float bias,
+                             int input_node_size, int output_node_size, int frame_size,
+                             int frame_stride, int bin_frame_stride, int lut_binarize, int binary_mode)
+{
+    /* include/bb/DifferentiableLutN.h:1157-1266: single-threaded in the reference; kept sequential here so the
+     * dx accumulation order (node, frame, input) is the reference's. */
+    int const NN = 1 << n;
+    float const reciprocal_frame_size = 1.0f / (float)frame_size;
+
+    for (int in = 0; in < input_node_size; ++in) {
+        memset(dx + (size_t)in * frame_stride, 0, sizeof(float) * (size_t)frame_size);
+    }
+    for (int node = 0; node < output_node_size; ++node) {
+        float Wl[MAXNN], dWl[MAXNN];
+        load_W(Wl, W, node, NN, lut_binarize);
+        memset(dWl, 0, sizeof(dWl));
+
+        float mean = mean_in[node];
+        float rstd = rstd_in[node];
+        float rstd2 = rstd * rstd;
+        float dmeanx = 0;
+        float dstd = 0;
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = dl_read_x(x_fp32, x_bit, idx[node * n + i], f, frame_stride, bin_frame_stride, binary_mode, bias);
+            }
+            float v = lut_forward_generic(xv, Wl, n);
+            float tanh_x = ((v - mean) * rstd) * gamma + beta;
+            float g = dy[(size_t)node * frame_stride + f];
+            if (tanh_x <= 0.0f) { g = 0.0f; }
+            if (tanh_x >= 1.0f) { g = 0.0f; }
+            float xc = v - mean;
+            float dxn = gamma * g;
+            dstd   += -(dxn * xc * rstd2);
+            dmeanx += -(dxn * rstd);
+        }
+        float dvar  = dstd * rstd;
+        float dmean = (dmeanx - (mean * dvar)) * reciprocal_frame_size;
+
+        for (int f = 0; f < frame_size; ++f) {
+            float xv[MAXN], dxv[MAXN];
+            for (int i = 0; i < n; ++i) {
+                xv[i] = dl_read_x(x_fp32, x_bit, idx[node * n + i], f, frame_stride, bin_frame_stride, binary_mode, bias);
+            }
+            float v = lut_forward_generic(xv, Wl, n);
+            float tanh_x = ((v - mean) * rstd) * gamma + beta;
+            float g = dy[(size_t)node * frame_stride + f];
+            if (tanh_x <= 0.0f) { g = 0.0f; }
+            if (tanh_x >= 1.0f) { g = 0.0f; }
+            float dxn = g * gamma;
+            float dxc = dxn * rstd;
+            float d   = dxc + dmean + (v * dvar * reciprocal_frame_size);
+            lut_backward_generic(xv, dxv, d, Wl, dWl, n);
+            for (int i = 0; i < n; ++i) {
+                dx[(size_t)idx[node * n + i] * frame_stride + f] += dxv[i];
+            }
+        }
+        for (int i = 0; i < NN; ++i) { dW[(size_t)node * NN + i] += dWl[i]; }
+    }
+}
+
+/* DifferentiableLutN<N,float>::Backward with batch-norm (:1157-1266); mean/rstd are the values Forward(train) stored */
+void oracle_fp32_DifferentiableLutN_Backward(int n, float const *x, float const *dy, float *dx, int32_t const *idx,
+        float const *W, float *dW, float const *mean, float const *rstd,
+        float gamma, float beta, float bias,
+        int input_node_size, int output_node_size, int frame_size, int frame_stride,
+        int lut_binarize, int binary_mode)
+{
+    dl_backward_core(n, x, NULL, dy, dx, idx, W, dW, mean, rstd, gamma, beta, bias,
+                     input_node_size, output_node_size, frame_size, frame_stride, 0, lut_binarize, binary_mode);
+}
+
+void oracle_bit_fp32_DifferentiableLutN_Backward(int n, int32_t const *x, float const *dy, float *dx, int32_t const *idx,
+        float const *W, float *dW, float const *mean, float const *rstd,
+        float gamma, float beta, float bias,
+        int input_node_size, int output_node_size, int frame_size, int frame_stride, int x_frame_stride,
+        int lut_binarize)
+{
+    dl_backward_core(n, NULL, x, dy, dx, idx, W, dW, mean, rstd, gamma, beta, bias,
+                     input_node_size, output_node_size, frame_size, frame_stride, x_frame_stride, lut_binarize, 1);
+}
+
+
+/* ---- BinaryLutN<6> ------------------------------------------------------------------------- */
+
+/* Generic loop of BinaryLutN<6,Bit>::Forward (include/bb/BinaryLutN.h:436-463): input k is table-index bit k,
+ * entries 0-31 live in table word 0 (:170-171, 279-284). Only bits of frames < frame_size are written. */
+void oracle_bit_BinaryLut6_Forward(int32_t const *x, int32_t *y, int32_t const *idx, int32_t const *table,
+                                   int node_size, int frame_size, int frame_stride)
+{
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            int index = 0, mask = 1;
+            for (int i = 0; i < 6; ++i) {
+                if (read_bit(x + (size_t)idx[node * 6 + i] * frame_stride, f)) { index |= mask; }
+                mask <<= 1;
+            }
+            int v = (int)(((uint32_t)table[node * 2 + (index >> 5)] >> (index & 31)) & 1u);
+            write_bit(y + (size_t)node * frame_stride, f, v);
+        }
+    }
+}
+
+/* Word-parallel form of the AVX2 loop (BinaryLutN.h:322-433): y = OR_k (T_k & AND_j (bit_j(k) ? x_j : ~x_j)),
+ * evaluated on whole 32-bit words, padding bits included — used as the timed CPU baseline. */
+void oracle_bit_BinaryLut6_Forward_words(int32_t const *x, int32_t *y, int32_t const *idx, int32_t const *table,
+                                         int node_size, int word_size, int frame_stride)
+{
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        uint32_t const t0 = (uint32_t)table[node * 2 + 0], t1 = (uint32_t)table[node * 2 + 1];
+        uint32_t const *xr[6];
+        for (int i = 0; i < 6; ++i) { xr[i] = (uint32_t const *)x + (size_t)idx[node * 6 + i] * frame_stride; }
+        uint32_t *yr = (uint32_t *)y + (size_t)node * frame_stride;
+        for (int w = 0; w < word_size; ++w) {
+            uint32_t xv[6];
+            for (int i = 0; i < 6; ++i) { xv[i] = xr[i][w]; }
+            uint32_t acc = 0;
+            for (int k = 0; k < 64; ++k) {
+                uint32_t lut = (((k < 32 ? t0 : t1) >> (k & 31)) & 1u) ? 0xffffffffu : 0u;
+                for (int j = 0; j < 6; ++j) { lut &= ((k >> j) & 1) ? xv[j] : ~xv[j]; }
+                acc |= lut;
+            }
+            yr[w] = acc;
+        }
+    }
+}
+
+
+/* ---- connection tables --------------------------------------------------------------------- */
+
+/* FixedSizeConnectionTable<N>::BuildReverseTable (include/bb/FixedSizeConnectionTable.h:180-215).
+ * Returns the row stride 1 + max fan-out. When rev != NULL and stride*input_node_size <= rev_cap the table is
+ * written: row r = [count, node*N+input ... in ascending (node,input) order, zero tail]. */
+int oracle_ReverseTable(int n, int32_t const *idx, int input_node_size, int output_node_size, int32_t *rev, int rev_cap)
+{
+    int *cnt = (int *)calloc((size_t)input_node_size, sizeof(int));
+    for (int node = 0; node < output_node_size; ++node) {
+        for (int i = 0; i < n; ++i) { cnt[idx[node * n + i]]++; }
+    }
+    int max_n = 0;
+    for (int r = 0; r < input_node_size; ++r) { if (cnt[r] > max_n) { max_n = cnt[r]; } }
+    free(cnt);
+    int stride = max_n + 1;
+    if (rev && (long long)stride * input_node_size <= rev_cap) {
+        memset(rev, 0, sizeof(int32_t) * (size_t)stride * (size_t)input_node_size);
+        for (int node = 0; node < output_node_size; ++node) {
+            for (int i = 0; i < n; ++i) {
+                int32_t r = idx[node * n + i];
+                int32_t c = rev[(size_t)r * stride] + 1;
+                rev[(size_t)r * stride]     = c;
+                rev[(size_t)r * stride + c] = (int32_t)(node * n + i);
+            }
+        }
+    }
+    return stride;
+}

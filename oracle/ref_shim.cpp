@@ -1,0 +1,261 @@
+// TEST INFRASTRUCTURE — not part of the shipped library.
+//
+// Thin extern "C" harness around the *unmodified* BinaryBrain CPU headers
+// (compiled with -I/root/reference/include, no BB_WITH_CUDA).  It lets the
+// parity tests and the CPU-baseline leg of bench.py run the reference's own
+// host implementation of the three LUT layers on caller-provided dense
+// arrays.  Every array is node-major, frame-minor: element (node n, frame f)
+// of an fp32 buffer is p[n*frames + f]; bit buffers are rows of `words`
+// 32-bit words per node, frame f at word f>>5 bit f&31 (the reference's own
+// packing, include/bb/DataType.h:612-647).
+//
+// Built only where the reference tree is present; see oracle/Makefile.
+
+#include <cstring>
+#include <cstdint>
+#include <vector>
+#include <string>
+
+#include "bb/StochasticLutN.h"
+#include "bb/DifferentiableLutN.h"
+#include "bb/BinaryLutN.h"
+#include "bb/FixedSizeConnectionTable.h"
+
+namespace {
+
+using bb::index_t;
+
+void put_fp32(bb::FrameBuffer &buf, float const *src, index_t nodes, index_t frames)
+{
+    auto ptr = buf.Lock<float>(true);
+    index_t stride = buf.GetFrameStride() / (index_t)sizeof(float);
+    for (index_t n = 0; n < nodes; ++n) {
+        float *row = ptr.GetAddr(n);
+        std::memcpy(row, src + n * frames, sizeof(float) * (size_t)frames);
+        for (index_t f = frames; f < stride; ++f) { row[f] = 0.0f; }
+    }
+}
+
+void get_fp32(bb::FrameBuffer &buf, float *dst, index_t nodes, index_t frames)
+{
+    auto ptr = buf.LockConst<float>();
+    for (index_t n = 0; n < nodes; ++n) {
+        std::memcpy(dst + n * frames, ptr.GetAddr(n), sizeof(float) * (size_t)frames);
+    }
+}
+
+void put_bit(bb::FrameBuffer &buf, std::int32_t const *src, index_t nodes, index_t words)
+{
+    auto ptr = buf.Lock<bb::Bit>(true);
+    index_t stride_bytes = buf.GetFrameStride();
+    for (index_t n = 0; n < nodes; ++n) {
+        auto *row = (std::uint8_t *)ptr.GetAddr(n);
+        std::memset(row, 0, (size_t)stride_bytes);
+        index_t nbytes = std::min(stride_bytes, words * 4);
+        std::memcpy(row, src + n * words, (size_t)nbytes);
+    }
+}
+
+void get_bit(bb::FrameBuffer &buf, std::int32_t *dst, index_t nodes, index_t words)
+{
+    auto ptr = buf.LockConst<bb::Bit>();
+    index_t stride_bytes = buf.GetFrameStride();
+    for (index_t n = 0; n < nodes; ++n) {
+        auto const *row = (std::uint8_t const *)ptr.GetAddr(n);
+        std::memset(dst + n * words, 0, (size_t)words * 4);
+        index_t nbytes = std::min(stride_bytes, words * 4);
+        std::memcpy(dst + n * words, row, (size_t)nbytes);
+    }
+}
+
+std::string onoff(int v) { return v ? "true" : "false"; }
+
+template <int N, typename BinType>
+int run_stochastic(int I, int O, int F, void const *x, std::int32_t const *idx, float *W,
+                   float const *dy, float *y, float *dx, float *dW,
+                   int binary_mode, int lut_binarize, int host_simd)
+{
+    auto lut = bb::StochasticLutN<N, BinType, float>::Create((index_t)O);
+    lut->SendCommand("host_only true");
+    lut->SendCommand("host_simd " + onoff(host_simd));
+    lut->SendCommand("lut_binarize " + onoff(lut_binarize));
+    lut->SendCommand("binary " + onoff(binary_mode));
+
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer x_buf((index_t)F, {(index_t)I}, xtype, true);
+    lut->SetInputShape(x_buf.GetShape());
+    for (int n = 0; n < O; ++n) {
+        for (int i = 0; i < N; ++i) { lut->SetNodeConnectionIndex(n, i, idx[n * N + i]); }
+    }
+    {
+        auto Wp = lut->lock_W();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { Wp(n, i) = W[n * (1 << N) + i]; }
+    }
+    if (dW) {
+        auto dWp = lut->lock_dW();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { dWp(n, i) = dW[n * (1 << N) + i]; }
+    }
+    if (xtype == BB_TYPE_BIT) { put_bit(x_buf, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(x_buf, (float const *)x, I, F); }
+
+    auto y_buf = lut->Forward(x_buf, dy != nullptr);
+    get_fp32(y_buf, y, O, F);
+    {
+        auto Wp = lut->lock_W_const();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { W[n * (1 << N) + i] = Wp(n, i); }
+    }
+    if (dy) {
+        bb::FrameBuffer dy_buf((index_t)F, {(index_t)O}, BB_TYPE_FP32, true);
+        put_fp32(dy_buf, dy, O, F);
+        auto dx_buf = lut->Backward(dy_buf);
+        get_fp32(dx_buf, dx, I, F);
+        auto dWp = lut->lock_dW_const();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { dW[n * (1 << N) + i] = dWp(n, i); }
+    }
+    return 0;
+}
+
+template <int N, typename BinType>
+int run_differentiable(int I, int O, int F, void const *x, std::int32_t const *idx, float *W,
+                       float const *dy, void *y, float *dx, float *dW,
+                       float *mean, float *rstd, float *running_mean, float *running_var,
+                       float gamma, float beta, float momentum,
+                       int batch_norm, int binary_mode, int lut_binarize, int train)
+{
+    typename bb::DifferentiableLutN<N, BinType, float>::create_t cr;
+    cr.output_shape = {(index_t)O};
+    cr.batch_norm   = batch_norm != 0;
+    cr.binary       = binary_mode != 0;
+    cr.momentum     = momentum;
+    cr.gamma        = gamma;
+    cr.beta         = beta;
+    auto lut = bb::DifferentiableLutN<N, BinType, float>::Create(cr);
+    lut->SendCommand("host_only true");
+    lut->SendCommand("lut_binarize " + onoff(lut_binarize));
+
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer x_buf((index_t)F, {(index_t)I}, xtype, true);
+    lut->SetInputShape(x_buf.GetShape());
+    for (int n = 0; n < O; ++n) {
+        for (int i = 0; i < N; ++i) { lut->SetNodeConnectionIndex(n, i, idx[n * N + i]); }
+    }
+    {
+        auto Wp = lut->lock_W();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { Wp(n, i) = W[n * (1 << N) + i]; }
+    }
+    if (dW) {
+        auto dWp = lut->lock_dW();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { dWp(n, i) = dW[n * (1 << N) + i]; }
+    }
+    {
+        auto rm = lut->lock_mean();
+        auto rv = lut->lock_var();
+        for (int n = 0; n < O; ++n) { rm[n] = running_mean[n]; rv[n] = running_var[n]; }
+    }
+    if (xtype == BB_TYPE_BIT) { put_bit(x_buf, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(x_buf, (float const *)x, I, F); }
+
+    auto y_buf = lut->Forward(x_buf, train != 0);
+    if (xtype == BB_TYPE_BIT) { get_bit(y_buf, (std::int32_t *)y, O, (F + 31) / 32); }
+    else                      { get_fp32(y_buf, (float *)y, O, F); }
+    {
+        auto rm = lut->lock_mean_const();
+        auto rv = lut->lock_var_const();
+        for (int n = 0; n < O; ++n) { running_mean[n] = rm[n]; running_var[n] = rv[n]; }
+    }
+    if (batch_norm && train) {
+        auto tm = lut->lock_tmp_mean_const();
+        auto tr = lut->lock_tmp_rstd_const();
+        for (int n = 0; n < O; ++n) { mean[n] = tm[n]; rstd[n] = tr[n]; }
+    }
+    if (dy) {
+        bb::FrameBuffer dy_buf((index_t)F, {(index_t)O}, BB_TYPE_FP32, true);
+        put_fp32(dy_buf, dy, O, F);
+        auto dx_buf = lut->Backward(dy_buf);
+        get_fp32(dx_buf, dx, I, F);
+        auto dWp = lut->lock_dW_const();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < (1 << N); ++i) { dW[n * (1 << N) + i] = dWp(n, i); }
+    }
+    return 0;
+}
+
+}  // namespace
+
+
+extern "C" {
+
+// StochasticLutN<N,float|Bit,float>::Forward (+Backward when dy != NULL) on the host-only path.
+// W is clamped in place exactly as Forward does (include/bb/StochasticLutN.h:451).
+int bbref_StochasticLut(int n, int bit_input, int I, int O, int F,
+                        void const *x, std::int32_t const *idx, float *W,
+                        float const *dy, float *y, float *dx, float *dW,
+                        int binary_mode, int lut_binarize, int host_simd)
+{
+#define BBREF_CASE(NN) \
+    case NN: return bit_input ? run_stochastic<NN, bb::Bit>(I, O, F, x, idx, W, dy, y, dx, dW, binary_mode, lut_binarize, host_simd) \
+                              : run_stochastic<NN, float  >(I, O, F, x, idx, W, dy, y, dx, dW, binary_mode, lut_binarize, host_simd);
+    switch (n) { BBREF_CASE(2) BBREF_CASE(3) BBREF_CASE(4) BBREF_CASE(5) BBREF_CASE(6) default: return -1; }
+#undef BBREF_CASE
+}
+
+// DifferentiableLutN<N,float|Bit,float>::Forward (+Backward when dy != NULL), host-only generic path.
+int bbref_DifferentiableLut(int n, int bit_input, int I, int O, int F,
+                            void const *x, std::int32_t const *idx, float *W,
+                            float const *dy, void *y, float *dx, float *dW,
+                            float *mean, float *rstd, float *running_mean, float *running_var,
+                            float gamma, float beta, float momentum,
+                            int batch_norm, int binary_mode, int lut_binarize, int train)
+{
+#define BBREF_CASE(NN) \
+    case NN: return bit_input ? run_differentiable<NN, bb::Bit>(I, O, F, x, idx, W, dy, y, dx, dW, mean, rstd, running_mean, running_var, gamma, beta, momentum, batch_norm, binary_mode, lut_binarize, train) \
+                              : run_differentiable<NN, float  >(I, O, F, x, idx, W, dy, y, dx, dW, mean, rstd, running_mean, running_var, gamma, beta, momentum, batch_norm, binary_mode, lut_binarize, train);
+    switch (n) { BBREF_CASE(2) BBREF_CASE(4) BBREF_CASE(6) default: return -1; }
+#undef BBREF_CASE
+}
+
+// BinaryLutN<6,Bit>::Forward, host-only; host_simd selects the AVX2 or the generic loop.
+int bbref_BinaryLut6(int I, int O, int F, std::int32_t const *x, std::int32_t const *idx,
+                     std::int32_t const *table /*[O][2]*/, std::int32_t *y, int host_simd)
+{
+    auto lut = bb::BinaryLutN<6, bb::Bit, float>::Create((index_t)O);
+    lut->SendCommand("host_only true");
+    lut->SendCommand("host_simd " + onoff(host_simd));
+    bb::FrameBuffer x_buf((index_t)F, {(index_t)I}, BB_TYPE_BIT, true);
+    lut->SetInputShape(x_buf.GetShape());
+    for (int nd = 0; nd < O; ++nd) {
+        for (int i = 0; i < 6; ++i) { lut->SetNodeConnectionIndex(nd, i, idx[nd * 6 + i]); }
+        for (int b = 0; b < 64; ++b) { lut->SetLutTable(nd, b, ((table[nd * 2 + (b >> 5)] >> (b & 31)) & 1) != 0); }
+    }
+    put_bit(x_buf, x, I, (F + 31) / 32);
+    auto y_buf = lut->Forward(x_buf, false);
+    get_bit(y_buf, y, O, (F + 31) / 32);
+    return 0;
+}
+
+// FixedSizeConnectionTable<6>: reverse table for a given input table.
+// Returns the row stride (1 + max fan-out); fills rev (capacity rev_cap int32) when it fits.
+int bbref_ReverseTable6(int I, int O, std::int32_t const *idx, std::int32_t *rev, int rev_cap)
+{
+    bb::FixedSizeConnectionTable<6> tbl;
+    tbl.SetShape({(index_t)I}, {(index_t)O});
+    for (int nd = 0; nd < O; ++nd) for (int i = 0; i < 6; ++i) { tbl.SetInputConnection(nd, i, idx[nd * 6 + i]); }
+    auto ptr = tbl.LockConst_ReverseTable();
+    int stride = (int)tbl.GetReverseTableStride();
+    if ((long long)stride * I <= rev_cap) {
+        for (int r = 0; r < I; ++r) for (int c = 0; c < stride; ++c) { rev[r * stride + c] = ptr(r, c); }
+    }
+    return stride;
+}
+
+// Seeded default wiring of StochasticLutN<6>::SetInputShape (random ShuffleSet policy) — used only
+// to check that injected wiring satisfies the same invariants (distinct inputs per node).
+int bbref_DefaultWiring6(int I, int O, std::uint64_t seed, std::int32_t *idx)
+{
+    auto lut = bb::StochasticLutN<6, float, float>::Create((index_t)O, "", seed);
+    lut->SendCommand("host_only true");
+    lut->SetInputShape({(index_t)I});
+    for (int nd = 0; nd < O; ++nd) for (int i = 0; i < 6; ++i) { idx[nd * 6 + i] = (std::int32_t)lut->GetNodeConnectionIndex(nd, i); }
+    return 0;
+}
+
+}  // extern "C"

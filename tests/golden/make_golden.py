@@ -1,0 +1,118 @@
+"""Writes tests/golden/*.npz: input/output vectors produced by the reference's own CPU headers.
+
+Run in a container that holds the reference tree and a built ``oracle/_ref/libbbref.so``
+(``make -C oracle ref``):  ``python tests/golden/make_golden.py``.
+The files hold data only (inputs, flags and the arrays the reference returned); padding bits of packed outputs
+are masked to zero because the reference leaves them undefined.
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+import oracle                               # noqa: E402
+from binarybrain_amd import synth          # noqa: E402
+
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+
+def mask_bits(packed, frames):
+    return synth.pack_bits(synth.unpack_bits(packed, frames), packed.shape[1])
+
+
+def stochastic_cases():
+    rng = np.random.default_rng(20240601)
+    cases = {}
+    k = 0
+    for (n, I, O, F, simd) in [(6, 32, 16, 64, 1), (6, 14, 16, 8, 1), (6, 13, 17, 29, 0), (4, 20, 16, 40, 0), (2, 9, 8, 24, 0)]:
+        for (binary_mode, lut_binarize) in [(0, 0), (0, 1), (1, 0)]:
+            idx = synth.wiring(rng, I, O, n)
+            W = synth.lut_tables(rng, O, n, -0.1, 1.1)
+            x = synth.uniform_frames(rng, I, F, stride=F, lo=-0.1, hi=1.1)
+            dy = synth.normal_frames(rng, O, F, stride=F)
+            dW0 = rng.standard_normal((O, 1 << n)).astype(np.float32)
+            r = oracle.ref_stochastic_lut(n, x, idx, W, dy=dy, dW_init=dW0, binary_mode=binary_mode,
+                                          lut_binarize=lut_binarize, host_simd=simd)
+            p = "c%d_" % k
+            cases.update({p + "meta": np.array([n, I, O, F, simd, binary_mode, lut_binarize], np.int32),
+                          p + "idx": idx, p + "W": W, p + "x": x, p + "dy": dy, p + "dW0": dW0,
+                          p + "Wc": r["W"], p + "y": r["y"], p + "dx": r["dx"], p + "dW": r["dW"]})
+            k += 1
+    # bit-packed input
+    for (n, I, O, F) in [(6, 24, 16, 70), (4, 12, 8, 33)]:
+        for lut_binarize in (0, 1):
+            idx = synth.wiring(rng, I, O, n)
+            W = synth.lut_tables(rng, O, n)
+            xb = synth.bernoulli_bits(rng, I, F)
+            dy = synth.normal_frames(rng, O, F, stride=F)
+            r = oracle.ref_stochastic_lut(n, xb, idx, W, dy=dy, bit_input=True, lut_binarize=lut_binarize, frame_size=F)
+            p = "c%d_" % k
+            cases.update({p + "meta": np.array([n, I, O, F, -1, 1, lut_binarize], np.int32),
+                          p + "idx": idx, p + "W": W, p + "xbits": xb, p + "dy": dy,
+                          p + "Wc": r["W"], p + "y": r["y"], p + "dx": r["dx"], p + "dW": r["dW"]})
+            k += 1
+    cases["count"] = np.array([k], np.int32)
+    np.savez_compressed(os.path.join(OUT, "stochastic_lut.npz"), **cases)
+
+
+def differentiable_cases():
+    rng = np.random.default_rng(20240602)
+    cases = {}
+    k = 0
+    for (n, I, O, F) in [(6, 20, 16, 40), (6, 16, 8, 131), (4, 20, 16, 39), (2, 10, 8, 64)]:
+        for (bit, binary_mode, lut_binarize, batch_norm) in [(0, 1, 0, 1), (0, 0, 0, 1), (0, 1, 1, 1), (1, 1, 0, 1),
+                                                              (0, 1, 0, 0), (0, 0, 0, 0), (1, 1, 0, 0)]:
+            idx = synth.wiring(rng, I, O, n)
+            W = synth.lut_tables(rng, O, n)
+            dy = synth.normal_frames(rng, O, F, stride=F)
+            rm = rng.random(O).astype(np.float32)
+            rv = (rng.random(O) + 0.5).astype(np.float32)
+            x = synth.bernoulli_bits(rng, I, F) if bit else synth.uniform_frames(rng, I, F, stride=F, lo=-0.1, hi=1.1)
+            kw = dict(bit_input=bool(bit), batch_norm=bool(batch_norm), binary_mode=bool(binary_mode),
+                      lut_binarize=bool(lut_binarize), frame_size=F, gamma=0.3, beta=0.5, momentum=0.9)
+            r = oracle.ref_differentiable_lut(n, x, idx, W, rm, rv, dy=dy, train=True, **kw)
+            ri = oracle.ref_differentiable_lut(n, x, idx, W, rm, rv, train=False, **kw)
+            y, yi = r["y"], ri["y"]
+            if bit:
+                y, yi = mask_bits(y, F), mask_bits(yi, F)
+            p = "c%d_" % k
+            cases.update({p + "meta": np.array([n, I, O, F, bit, binary_mode, lut_binarize, batch_norm], np.int32),
+                          p + "idx": idx, p + "W": W, p + "x": x, p + "dy": dy, p + "rm": rm, p + "rv": rv,
+                          p + "y": y, p + "y_inf": yi, p + "dx": r["dx"], p + "dW": r["dW"],
+                          p + "mean": r["mean"], p + "rstd": r["rstd"],
+                          p + "rm_out": r["running_mean"], p + "rv_out": r["running_var"]})
+            k += 1
+    cases["count"] = np.array([k], np.int32)
+    np.savez_compressed(os.path.join(OUT, "differentiable_lut.npz"), **cases)
+
+
+def binary_cases():
+    rng = np.random.default_rng(20240603)
+    cases = {}
+    k = 0
+    for (I, O, F) in [(16, 16, 32), (64, 32, 512), (70, 33, 1000), (8, 5, 7)]:
+        idx = synth.wiring(rng, I, O, 6)
+        T = synth.truth_tables(rng, O)
+        xb = synth.bernoulli_bits(rng, I, F)
+        y_simd = mask_bits(oracle.ref_binary_lut6(xb, idx, T, F, host_simd=True), F)
+        y_gen = mask_bits(oracle.ref_binary_lut6(xb, idx, T, F, host_simd=False), F)
+        assert np.array_equal(y_simd, y_gen)
+        rev = oracle.ref_reverse_table6(idx, I)
+        p = "c%d_" % k
+        cases.update({p + "meta": np.array([I, O, F], np.int32), p + "idx": idx, p + "table": T, p + "xbits": xb,
+                      p + "y": y_simd, p + "rev": rev})
+        k += 1
+    cases["count"] = np.array([k], np.int32)
+    np.savez_compressed(os.path.join(OUT, "binary_lut6.npz"), **cases)
+
+
+if __name__ == "__main__":
+    assert oracle.have_ref(), "build oracle/_ref first (make -C oracle ref)"
+    stochastic_cases()
+    differentiable_cases()
+    binary_cases()
+    for f in sorted(os.listdir(OUT)):
+        if f.endswith(".npz"):
+            print(f, os.path.getsize(os.path.join(OUT, f)), "bytes")
