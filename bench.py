@@ -1,0 +1,139 @@
+"""Benchmark of the differentiable-LUT hot path on one MI355X.
+
+A step is one pass of StochasticLut6 over one batch of synthetic input: clamp W, forward, backward (dW and dx), fp32,
+4096 input nodes -> 4096 output nodes, 8192 frames.  Inputs are resident in HBM before the timed region.
+Prints ONE JSON line: node-evaluations per second (one node-eval = one (output node, frame) pair taken through forward
+and backward), the HBM roofline of the dominant kernel, and the CPU reference timed on this host's cores.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
+
+
+def algorithmic_bytes(I, O, F):
+    """every tensor touched once per pass, index and table traffic included (fp32, N = 6)"""
+    fwd = 4 * F * (I + O) + 256 * O + 24 * O
+    bwd = 4 * F * (2 * I + O) + 3 * 256 * O + 24 * O
+    return fwd, bwd
+
+
+def cpu_baseline(I, O, frames, threads, reps=9):
+    """Forward+backward of the same layer on the host cores: the reference's own AVX2/OpenMP path when oracle/_ref is
+    present ("reference"), else the C restatement ("port").  Timed around Forward+Backward only; median of reps."""
+    import numpy as np
+    os.environ["OMP_NUM_THREADS"] = str(threads)
+    import oracle
+    from binarybrain_amd import synth
+    rng = np.random.default_rng(1)
+    idx = synth.wiring(rng, I, O)
+    W = synth.lut_tables(rng, O)
+    x = synth.uniform_frames(rng, I, frames, frames)
+    dy = synth.normal_frames(rng, O, frames, frames)
+    secs, kind = oracle.time_stochastic_lut6(x, dy, idx, W, reps)
+    med = float(np.median(secs))
+    return {"value": O * frames / med / 1e9, "unit": "G node-evals/s", "cores": threads, "kind": kind,
+            "sample": "StochasticLut6 fwd+bwd (AVX2+OpenMP host path), %d->%d nodes, %d frames, 1 warm-up + median of %d"
+                      % (I, O, frames, reps)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "1")),
+                    help="0: deterministic dx through dx_tmp + reverse table; 1: fp32 atomics")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-frames", type=int, default=8192)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards over frames, "
+              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from binarybrain_amd import capi, ops, synth
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    lib = capi.lib()
+    I = O = 4096
+    F = 8192
+    rng = np.random.default_rng(0)
+    idx_h = synth.wiring(rng, I, O)
+    idx = torch.from_numpy(idx_h).cuda()
+    W = torch.from_numpy(synth.lut_tables(rng, O)).cuda()
+    x = torch.from_numpy(synth.uniform_frames(rng, I, F, F)).cuda()
+    dy = torch.from_numpy(synth.normal_frames(rng, O, F, F)).cuda()
+    dW = torch.zeros((O, 64), device="cuda")
+    y = torch.empty((O, F), device="cuda")
+    dx = torch.empty((I, F), device="cuda")
+    ops.set_dx_mode(args.dx_mode)
+    rev = ops.reverse_table(idx, I) if args.dx_mode == 0 else None
+    dx_tmp = None
+    tmp_frames = None
+    if args.dx_mode == 0:
+        tmp_frames = ops._tmp_frames(O, 6, F)
+        dx_tmp = torch.empty((O * 6, ((tmp_frames + 63) // 64) * 64), device="cuda")
+
+    def step():
+        ops.vector_clamp_(W)                                    # StochasticLutN::Forward clamps W first
+        ops.stochastic_lut_forward(6, x, idx, W, F, out=y)
+        ops.stochastic_lut_backward(6, x, dy, idx, W, dW, F, rev, dx_tmp=dx_tmp, tmp_frame_size=tmp_frames, out=dx)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.bbhip_KernelTimer_Enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lib.bbhip_KernelTimer_Enable(0)
+
+    ms = C.c_float(); cnt = C.c_int()
+    capi.check(lib.bbhip_KernelTimer_Read(0, C.byref(ms), C.byref(cnt)))
+    fwd_ms = ms.value / max(cnt.value, 1)
+    capi.check(lib.bbhip_KernelTimer_Read(1, C.byref(ms), C.byref(cnt)))
+    bwd_launches = cnt.value
+    bwd_ms = ms.value / max(cnt.value, 1)
+
+    fwd_b, bwd_b = algorithmic_bytes(I, O, F)
+    launches_per_step = bwd_launches / args.steps
+    bwd_bytes_per_launch = bwd_b / launches_per_step
+    achieved = bwd_bytes_per_launch / (bwd_ms * 1e-3) / 1e9
+    node_evals = O * F
+    ms_per_step = dt / args.steps * 1e3
+    out = {
+        "metric": "G node-evals/s StochasticLut6 fp32 fwd+bwd (8192 frames x 4096 nodes)",
+        "value": node_evals / (dt / args.steps) / 1e9,
+        "unit": "G node-evals/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "StochasticLut6 fwd+bwd fp32, 4096 in x 4096 out x 8192 frames, uniform random 6-of-4096 wiring",
+                   "dx_mode": "atomic" if args.dx_mode else "deterministic (dx_tmp + reverse table)",
+                   "lut_binarize": False, "binary": False},
+        "hbm_frac_step": (fwd_b + bwd_b) / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "lut_backward_kernel<6>", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "launches_per_step": launches_per_step, "avg_launch_ms": bwd_ms,
+                     "forward_kernel_ms": fwd_ms,
+                     "forward_kernel_frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(I, O, args.cpu_frames, os.cpu_count() if (os.cpu_count() or 1) <= 16 else 16)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

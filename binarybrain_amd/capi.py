@@ -1,0 +1,82 @@
+"""ctypes binding of the C ABI in include/bbhip.h.  Device memory and streams come from torch; nothing here computes."""
+import ctypes as C
+import os
+
+from .build import LIB_PATH
+
+_lib = None
+
+_vp, _i, _f = C.c_void_p, C.c_int, C.c_float
+
+_SIGNATURES = {
+    "bbhip_GetDeviceCount": (C.c_int, []),
+    "bbhip_GetDevice": (C.c_int, []),
+    "bbhip_SetDevice": (None, [_i]),
+    "bbhip_SetHostOnly": (None, [_i]),
+    "bbhip_IsHostOnly": (C.c_int, []),
+    "bbhip_IsDeviceAvailable": (C.c_int, []),
+    "bbhip_GetLastErrorString": (C.c_char_p, []),
+    "bbhip_LocalHeap_Malloc": (C.c_void_p, [C.c_size_t]),
+    "bbhip_LocalHeap_Free": (None, [_vp]),
+    "bbhip_LocalHeap_GetMaxAllocSize": (C.c_size_t, []),
+    "bbhip_LocalHeap_GetAllocatedSize": (C.c_size_t, []),
+    "bbhip_LocalHeap_GarbageCollect": (None, []),
+    "bbhip_KernelTimer_Enable": (None, [_i]),
+    "bbhip_KernelTimer_Read": (C.c_int, [_i, C.POINTER(C.c_float), C.POINTER(C.c_int)]),
+    "bbhip_SetDxMode": (None, [_i]),
+    "bbhip_GetDxMode": (C.c_int, []),
+    "bbhip_fp32_Vector_set": (C.c_int, [_vp, _f, _i, _vp]),
+    "bbhip_fp32_Vector_clamp": (C.c_int, [_vp, _vp, _f, _f, _i, _vp]),
+    "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
+    "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
+    "bbhip_bit_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
+    "bbhip_bit_bit_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp]),
+    "bbhip_fp32_StochasticLut_Backward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 9 + [_f, _vp]),
+    "bbhip_bit_fp32_StochasticLut_Backward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 9 + [_f, _vp]),
+    "bbhip_fp32_DifferentiableLutN_ForwardTraining": (C.c_int, [_i] + [_vp] * 8 + [_f] * 4 + [_i] * 5 + [_vp]),
+    "bbhip_bit_fp32_DifferentiableLutN_ForwardTraining": (C.c_int, [_i] + [_vp] * 8 + [_f] * 4 + [_i] * 4 + [_vp]),
+    "bbhip_fp32_DifferentiableLutN_ForwardInference": (C.c_int, [_i] + [_vp] * 6 + [_f] * 3 + [_i] * 5 + [_vp]),
+    "bbhip_bit_fp32_DifferentiableLutN_ForwardInference": (C.c_int, [_i] + [_vp] * 6 + [_f] * 3 + [_i] * 4 + [_vp]),
+    "bbhip_fp32_DifferentiableLutN_Backward": (C.c_int, [_i] + [_vp] * 12 + [_f] * 3 + [_i] * 9 + [_vp]),
+    "bbhip_bit_fp32_DifferentiableLutN_Backward": (C.c_int, [_i] + [_vp] * 12 + [_f] * 3 + [_i] * 9 + [_vp]),
+    "bbhip_fp32_DifferentiableLutN_ForwardNoBn": (C.c_int, [_i] + [_vp] * 4 + [_f] + [_i] * 5 + [_vp]),
+    "bbhip_bit_BinaryLut6_Forward": (C.c_int, [_vp] * 4 + [_i] * 3 + [_vp]),
+}
+
+
+class BbhipError(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded library. Fails loudly when it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise BbhipError("%s is missing: build it with `python -m binarybrain_amd.build` "
+                             "(or __graft_entry__.build())" % LIB_PATH)
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def check(rc):
+    if rc != 0:
+        raise BbhipError(lib().bbhip_GetLastErrorString().decode())
+
+
+def ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def stream_ptr():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)

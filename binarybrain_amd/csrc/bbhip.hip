@@ -1,0 +1,781 @@
+// Host side of the C ABI declared in include/bbhip.h: argument checks, scratch management and kernel launches.
+// The kernels themselves are in lut_kernels.hpp; the arithmetic they share in lut_math.hpp.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/bbhip.h"
+#include "lut_kernels.hpp"
+
+using namespace bbhip;
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+//  errors
+// ------------------------------------------------------------------------------------------------
+thread_local std::string g_last_error;
+
+int fail(char const *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return 1;
+}
+
+#define BBHIP_TRY(expr)                                                                              \
+    do {                                                                                             \
+        hipError_t e_ = (expr);                                                                      \
+        if (e_ != hipSuccess) { return fail("%s: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); } \
+    } while (0)
+
+#define BBHIP_REQUIRE(cond)                                                                          \
+    do {                                                                                             \
+        if (!(cond)) { return fail("%s: rejected argument: %s", __func__, #cond); }                  \
+    } while (0)
+
+#define BBHIP_LAUNCH_CHECK() BBHIP_TRY(hipGetLastError())
+
+// ------------------------------------------------------------------------------------------------
+//  global switches
+// ------------------------------------------------------------------------------------------------
+bool g_host_only = false;
+int  g_dx_mode   = 0;
+
+// ------------------------------------------------------------------------------------------------
+//  optional kernel timer: HIP events around the dominant kernel of each entry point, on the launch stream
+// ------------------------------------------------------------------------------------------------
+enum TimedKernel : int { kTimeForward = 0, kTimeBackward = 1, kTimeBinary = 2, kTimedKinds = 3 };
+struct TimedLaunch { hipEvent_t start, stop; int which; };
+bool g_timer_on = false;
+std::vector<TimedLaunch> g_timed;
+
+struct ScopedTimer {
+    hipStream_t st; bool on; TimedLaunch t;
+    ScopedTimer(int which, hipStream_t s) : st(s), on(g_timer_on)
+    {
+        if (!on) { return; }
+        t.which = which;
+        if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { on = false; return; }
+        (void)hipEventRecord(t.start, st);
+    }
+    ~ScopedTimer()
+    {
+        if (!on) { return; }
+        (void)hipEventRecord(t.stop, st);
+        g_timed.push_back(t);
+    }
+};
+
+int env_int(char const *name, int def)
+{
+    char const *s = getenv(name);
+    if (!s || !*s) { return def; }
+    int v = atoi(s);
+    return v > 0 ? v : def;
+}
+
+// frames per unit; both are rounded to wavefront multiples where used
+int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 256); return ((v + 63) / 64) * 64; }
+int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 512);  return ((v + 63) / 64) * 64; }
+int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
+
+// ------------------------------------------------------------------------------------------------
+//  scratch arena: one growing device buffer per device, reused by every call
+// ------------------------------------------------------------------------------------------------
+constexpr int kMaxDevices = 64;
+struct Arena { void *ptr = nullptr; size_t cap = 0; };
+Arena g_arena[kMaxDevices];
+
+int arena_get(size_t bytes, char **out)
+{
+    int dev = 0;
+    BBHIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) { return fail("device index %d out of range", dev); }
+    Arena &a = g_arena[dev];
+    if (a.cap < bytes) {
+        if (a.ptr) {
+            BBHIP_TRY(hipDeviceSynchronize());
+            BBHIP_TRY(hipFree(a.ptr));
+            a.ptr = nullptr;
+            a.cap = 0;
+        }
+        size_t want = bytes + bytes / 2 + (1u << 20);
+        BBHIP_TRY(hipMalloc(&a.ptr, want));
+        a.cap = want;
+    }
+    *out = static_cast<char *>(a.ptr);
+    return 0;
+}
+
+inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// ------------------------------------------------------------------------------------------------
+//  dispatch helpers
+// ------------------------------------------------------------------------------------------------
+#define BBHIP_SWITCH_N(n, EXPR)                       \
+    switch (n) {                                      \
+    case 2: { constexpr int N = 2; EXPR; } break;     \
+    case 3: { constexpr int N = 3; EXPR; } break;     \
+    case 4: { constexpr int N = 4; EXPR; } break;     \
+    case 5: { constexpr int N = 5; EXPR; } break;     \
+    case 6: { constexpr int N = 6; EXPR; } break;     \
+    default: return fail("LUT width n=%d not in 2..6", n); \
+    }
+
+template <int N>
+void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st)
+{
+    int const total = node_size * (1 << N);
+    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize);
+}
+
+template <int N, int XMODE, int YMODE, int KIND>
+void launch_forward(FwdArgs const &a, hipStream_t st)
+{
+    hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND>), dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, st, a);
+}
+
+// xmode / ymode / kind are runtime values here; the combinations that exist are enumerated explicitly
+template <int N>
+int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, hipStream_t st)
+{
+#define BBHIP_FWD_CASE(X, Y, K) if (xmode == X && ymode == Y && kind == K) { launch_forward<N, X, Y, K>(a, st); return 0; }
+    BBHIP_FWD_CASE(kXClamp,  kYClamp,    0)
+    BBHIP_FWD_CASE(kXBinary, kYClamp,    0)
+    BBHIP_FWD_CASE(kXBit,    kYClamp,    0)
+    BBHIP_FWD_CASE(kXBit,    kYBit,      0)
+    BBHIP_FWD_CASE(kXBinary, kYBinarize, 0)
+    BBHIP_FWD_CASE(kXClamp,  kYClamp,    1)
+    BBHIP_FWD_CASE(kXBinary, kYBinarize, 1)
+    BBHIP_FWD_CASE(kXBit,    kYBit,      1)
+    BBHIP_FWD_CASE(kXClamp,  kYClamp,    2)
+    BBHIP_FWD_CASE(kXBinary, kYClamp,    2)
+    BBHIP_FWD_CASE(kXBit,    kYClamp,    2)
+#undef BBHIP_FWD_CASE
+    return fail("forward variant (x=%d, y=%d, kind=%d) not built", xmode, ymode, kind);
+}
+
+template <int N>
+int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStream_t st)
+{
+    dim3 const grid(a.slab_count * a.tile_count), block(kBlock);
+#define BBHIP_BWD_CASE(X, K, M) if (xmode == X && kind == K && dxmode == M) { hipLaunchKernelGGL((lut_backward_kernel<N, X, K, M>), grid, block, 0, st, a); return 0; }
+    BBHIP_BWD_CASE(kXClamp,  0, kDxAtomic) BBHIP_BWD_CASE(kXClamp,  0, kDxTmp)
+    BBHIP_BWD_CASE(kXBinary, 0, kDxAtomic) BBHIP_BWD_CASE(kXBinary, 0, kDxTmp)
+    BBHIP_BWD_CASE(kXBit,    0, kDxAtomic) BBHIP_BWD_CASE(kXBit,    0, kDxTmp)
+    BBHIP_BWD_CASE(kXClamp,  1, kDxAtomic) BBHIP_BWD_CASE(kXClamp,  1, kDxTmp)
+    BBHIP_BWD_CASE(kXBinary, 1, kDxAtomic) BBHIP_BWD_CASE(kXBinary, 1, kDxTmp)
+    BBHIP_BWD_CASE(kXBit,    1, kDxAtomic) BBHIP_BWD_CASE(kXBit,    1, kDxTmp)
+    BBHIP_BWD_CASE(kXClamp,  2, kDxTmp)
+    BBHIP_BWD_CASE(kXBinary, 2, kDxTmp)
+    BBHIP_BWD_CASE(kXBit,    2, kDxTmp)
+#undef BBHIP_BWD_CASE
+    return fail("backward variant (x=%d, kind=%d, dx=%d) not built", xmode, kind, dxmode);
+}
+
+// ------------------------------------------------------------------------------------------------
+//  forward driver
+// ------------------------------------------------------------------------------------------------
+struct ForwardCall {
+    int n;
+    void const *x; void *y; int const *idx; float const *W;
+    int node_size, frame_size, x_stride, y_stride;
+    int xmode, ymode;
+    int lut_binarize; float bias;
+    // batch-norm
+    int bn;                      // 0 none, 1 training, 2 inference
+    float *mean, *rstd, *running_mean, *running_var;
+    float gamma, beta, momentum;
+};
+
+int check_forward(ForwardCall const &c)
+{
+    if (!(c.x && c.y && c.idx && c.W))               { return fail("forward: null buffer"); }
+    if (!(c.node_size > 0 && c.frame_size > 0))      { return fail("forward: node_size=%d frame_size=%d must be positive", c.node_size, c.frame_size); }
+    int const x_need = (c.xmode == kXBit) ? (c.frame_size + 31) / 32 : c.frame_size;
+    int const y_need = (c.ymode == kYBit) ? (c.frame_size + 31) / 32 : c.frame_size;
+    if (c.x_stride < x_need || c.y_stride < y_need)  { return fail("forward: frame stride (x %d, y %d) shorter than the frames (%d, %d)", c.x_stride, c.y_stride, x_need, y_need); }
+    if ((long long)c.node_size * (1 << c.n) > 0x7fffffffLL) { return fail("forward: node_size too large"); }
+    if (c.bn == 1 && !(c.mean && c.rstd && c.running_mean && c.running_var)) { return fail("forward: null statistics buffer"); }
+    if (c.bn == 2 && !(c.running_mean && c.running_var))                      { return fail("forward: null statistics buffer"); }
+    return 0;
+}
+
+template <int N>
+int run_forward(ForwardCall const &c, hipStream_t st)
+{
+    constexpr int NN = 1 << N;
+    int const chunk       = fwd_chunk_frames();
+    int const chunk_count = ceil_div(c.frame_size, chunk);
+    int const tile_count  = ceil_div(c.node_size, kWavesPerBlk);
+    if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("forward: grid too large"); }
+
+    size_t const c_bytes    = align256((size_t)c.node_size * NN * sizeof(float));
+    size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
+    size_t const rstd_bytes = (c.bn == 2) ? align256((size_t)c.node_size * sizeof(float)) : 0;
+    char *base = nullptr;
+    if (arena_get(c_bytes + stat_bytes + rstd_bytes, &base)) { return 1; }
+    float *C        = reinterpret_cast<float *>(base);
+    float *stat     = reinterpret_cast<float *>(base + c_bytes);
+    float *rstd_tmp = reinterpret_cast<float *>(base + c_bytes + stat_bytes);
+
+    launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st);
+    BBHIP_LAUNCH_CHECK();
+
+    FwdArgs a{};
+    a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C;
+    a.node_size = c.node_size; a.frame_size = c.frame_size;
+    a.x_stride = c.x_stride; a.y_stride = c.y_stride;
+    a.chunk = chunk; a.chunk_count = chunk_count; a.tile_count = tile_count;
+    a.bias = c.bias; a.gamma = c.gamma; a.beta = c.beta;
+
+    int kind = 0;
+    if (c.bn == 1) {
+        a.stat_partial = stat;
+        if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, st)) { return 1; }
+        BBHIP_LAUNCH_CHECK();
+        hipLaunchKernelGGL(bn_forward_finalize_kernel, dim3(ceil_div(c.node_size, kBlock)), dim3(kBlock), 0, st,
+                           stat, C, NN, c.mean, c.rstd, c.running_mean, c.running_var, c.momentum,
+                           c.node_size, chunk_count, c.frame_size);
+        BBHIP_LAUNCH_CHECK();
+        a.mean = c.mean; a.rstd = c.rstd;
+        kind = 1;
+    }
+    else if (c.bn == 2) {
+        hipLaunchKernelGGL(rsqrt_kernel, dim3(ceil_div(c.node_size, kBlock)), dim3(kBlock), 0, st,
+                           c.running_var, rstd_tmp, c.node_size);
+        BBHIP_LAUNCH_CHECK();
+        a.mean = c.running_mean; a.rstd = rstd_tmp;
+        kind = 1;
+    }
+    {
+        ScopedTimer tm(kTimeForward, st);
+        if (dispatch_forward<N>(c.xmode, c.ymode, kind, a, st)) { return 1; }
+    }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int forward_entry(ForwardCall const &c, void *stream)
+{
+    if (check_forward(c)) { return 1; }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, st));
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+//  backward driver
+// ------------------------------------------------------------------------------------------------
+struct BackwardCall {
+    int n;
+    void const *x; float const *dy; float *dx; float *dx_tmp;
+    int const *idx; int const *rev; float const *W; float *dW;
+    int rev_stride, input_node_size, output_node_size, frame_size;
+    int x_stride, frame_stride, tmp_frame_size, tmp_frame_stride;
+    int xmode, lut_binarize; float bias;
+    int bn;
+    float const *mean, *rstd; float *dmean_tmp, *dvar_tmp;
+    float gamma, beta;
+};
+
+int check_backward(BackwardCall const &c, int dxmode)
+{
+    if (!(c.x && c.dy && c.dx && c.idx && c.W && c.dW)) { return fail("backward: null buffer"); }
+    if (!(c.input_node_size > 0 && c.output_node_size > 0 && c.frame_size > 0)) { return fail("backward: sizes must be positive"); }
+    int const x_need = (c.xmode == kXBit) ? (c.frame_size + 31) / 32 : c.frame_size;
+    if (c.x_stride < x_need || c.frame_stride < c.frame_size) { return fail("backward: frame stride shorter than the frames"); }
+    if ((long long)c.output_node_size * (1 << c.n) > 0x7fffffffLL) { return fail("backward: node_size too large"); }
+    if (dxmode == kDxTmp) {
+        if (!(c.dx_tmp && c.rev))                        { return fail("backward: deterministic dx needs dx_tmp and reverse_index (or bbhip_SetDxMode(1))"); }
+        if (c.tmp_frame_size <= 0)                       { return fail("backward: tmp_frame_size=%d must be positive", c.tmp_frame_size); }
+        int const span = c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size;
+        if (c.tmp_frame_stride < span)                   { return fail("backward: tmp_frame_stride=%d shorter than tmp_frame_size", c.tmp_frame_stride); }
+        if (c.rev_stride < 1)                            { return fail("backward: reverse_index_stride=%d", c.rev_stride); }
+    }
+    if (c.bn && !(c.mean && c.rstd && c.dmean_tmp && c.dvar_tmp)) { return fail("backward: null statistics buffer"); }
+    return 0;
+}
+
+template <int N>
+int run_backward(BackwardCall const &c, hipStream_t st)
+{
+    constexpr int NN = 1 << N;
+    int const dxmode = g_dx_mode ? kDxAtomic : kDxTmp;
+    if (check_backward(c, dxmode)) { return 1; }
+
+    int const tile_count = ceil_div(c.output_node_size, kWavesPerBlk);
+    int const range      = (dxmode == kDxTmp) ? (c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size) : c.frame_size;
+    int const range_count = ceil_div(c.frame_size, range);
+
+    // slab length: a wavefront multiple; long enough that the per-slab partial tables stay below 256 MiB
+    int slab = bwd_slab_frames();
+    for (;;) {
+        long long slabs = (long long)range_count * ceil_div(range, slab);
+        if (slabs * c.output_node_size * NN * (long long)sizeof(float) <= (256LL << 20) || slab >= range) { break; }
+        slab *= 2;
+    }
+    // total number of slabs over all ranges (the last range may be shorter)
+    int slab_total = 0;
+    for (int r = 0; r < range_count; ++r) {
+        int const len = (r + 1 < range_count) ? range : (c.frame_size - r * range);
+        slab_total += ceil_div(len, slab);
+    }
+    if ((long long)slab_total * tile_count > 0x7fffffffLL) { return fail("backward: grid too large"); }
+
+    size_t const c_bytes    = align256((size_t)c.output_node_size * NN * sizeof(float));
+    size_t const part_bytes = align256((size_t)slab_total * c.output_node_size * NN * sizeof(float));
+    size_t const stat_bytes = c.bn ? align256((size_t)slab_total * c.output_node_size * 2 * sizeof(float)) : 0;
+    char *base = nullptr;
+    if (arena_get(c_bytes + part_bytes + stat_bytes, &base)) { return 1; }
+    float *C    = reinterpret_cast<float *>(base);
+    float *part = reinterpret_cast<float *>(base + c_bytes);
+    float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
+
+    launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
+    BBHIP_LAUNCH_CHECK();
+
+    BwdArgs a{};
+    a.x = c.x; a.dy = c.dy; a.idx = c.idx; a.C = C;
+    a.dw_partial = part; a.stat_partial = stat;
+    a.mean = c.mean; a.rstd = c.rstd; a.dmean = c.dmean_tmp; a.dvar = c.dvar_tmp;
+    a.node_size = c.output_node_size; a.frame_size = c.frame_size;
+    a.x_stride = c.x_stride; a.dy_stride = c.frame_stride;
+    a.slab = slab; a.tile_count = tile_count;
+    a.bias = c.bias; a.gamma = c.gamma; a.beta = c.beta; a.inv_frames = 1.0f / (float)c.frame_size;
+
+    if (c.bn) {
+        // phase 0: per-node sums over ALL frames, then dmean / dvar
+        a.f_base = 0; a.f_limit = c.frame_size; a.slab_first = 0;
+        a.slab_count = ceil_div(c.frame_size, slab);
+        a.dx = nullptr; a.dx_stride = 0;
+        if (dispatch_backward<N>(c.xmode, 2, kDxTmp, a, st)) { return 1; }
+        BBHIP_LAUNCH_CHECK();
+        hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, kBlock)), dim3(kBlock), 0, st,
+                           stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, a.slab_count, c.frame_size);
+        BBHIP_LAUNCH_CHECK();
+    }
+
+    if (dxmode == kDxAtomic) {
+        size_t const count = (size_t)c.input_node_size * c.frame_stride;
+        hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((count + kBlock * 4 - 1) / (kBlock * 4))), dim3(kBlock), 0, st, c.dx, 0.0f, count);
+        BBHIP_LAUNCH_CHECK();
+    }
+
+    int slab_first = 0;
+    for (int r = 0; r < range_count; ++r) {
+        a.f_base     = r * range;
+        a.f_limit    = (a.f_base + range < c.frame_size) ? a.f_base + range : c.frame_size;
+        a.slab_first = slab_first;
+        a.slab_count = ceil_div(a.f_limit - a.f_base, slab);
+        if (dxmode == kDxAtomic) { a.dx = c.dx;     a.dx_stride = c.frame_stride; }
+        else                     { a.dx = c.dx_tmp; a.dx_stride = c.tmp_frame_stride; }
+        {
+            ScopedTimer tm(kTimeBackward, st);
+            if (dispatch_backward<N>(c.xmode, c.bn ? 1 : 0, dxmode, a, st)) { return 1; }
+        }
+        BBHIP_LAUNCH_CHECK();
+        if (dxmode == kDxTmp) {
+            dim3 const grid(ceil_div(a.f_limit - a.f_base, kBlock), c.input_node_size < 65535 ? c.input_node_size : 65535);
+            hipLaunchKernelGGL(dx_gather_kernel, grid, dim3(kBlock), 0, st, c.dx_tmp, c.dx, c.rev, c.rev_stride,
+                               c.input_node_size, a.f_base, a.f_limit, c.frame_stride, c.tmp_frame_stride);
+            BBHIP_LAUNCH_CHECK();
+        }
+        slab_first += a.slab_count;
+    }
+
+    int const total = c.output_node_size * NN;
+    hipLaunchKernelGGL(dw_finalize_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, part, c.dW, c.output_node_size, slab_total);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int backward_entry(BackwardCall const &c, void *stream)
+{
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st));
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+//  caching allocator
+// ------------------------------------------------------------------------------------------------
+struct LocalHeap {
+    std::mutex mtx;
+    std::map<void *, size_t>      used;
+    std::multimap<size_t, void *> spare;
+    size_t allocated = 0, reserved = 0, max_alloc = 0;
+
+    void *alloc(size_t size)
+    {
+        if (size == 0) { size = 1; }
+        size = (size + 255) & ~(size_t)255;
+        std::lock_guard<std::mutex> lk(mtx);
+        auto it = spare.lower_bound(size);
+        if (it != spare.end() && it->first <= size + size / 2) {        // best fit within 1.5x
+            void *p = it->second;
+            size_t sz = it->first;
+            spare.erase(it);
+            used[p] = sz;
+            allocated += sz;
+            if (allocated > max_alloc) { max_alloc = allocated; }
+            return p;
+        }
+        void *p = nullptr;
+        if (hipMalloc(&p, size) != hipSuccess) {
+            (void)hipGetLastError();
+            collect_locked();
+            if (hipMalloc(&p, size) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        }
+        used[p] = size;
+        allocated += size;
+        reserved += size;
+        if (allocated > max_alloc) { max_alloc = allocated; }
+        return p;
+    }
+
+    void release(void *p)
+    {
+        if (!p) { return; }
+        std::lock_guard<std::mutex> lk(mtx);
+        auto it = used.find(p);
+        if (it == used.end()) { return; }
+        size_t sz = it->second;
+        used.erase(it);
+        allocated -= sz;
+        spare.emplace(sz, p);
+        if (reserved > max_alloc + max_alloc / 2) { collect_locked(); }   // keep the reserve within 1.5x of the high-water mark
+    }
+
+    void collect_locked(void)
+    {
+        for (auto &kv : spare) { (void)hipFree(kv.second); reserved -= kv.first; }
+        spare.clear();
+    }
+};
+
+LocalHeap &heap(void) { static LocalHeap h; return h; }
+
+}  // namespace
+
+
+// ================================================================================================
+//  exported entry points
+// ================================================================================================
+extern "C" {
+
+int bbhip_GetDeviceCount(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return n;
+}
+
+int bbhip_GetDevice(void)
+{
+    int d = 0;
+    if (hipGetDevice(&d) != hipSuccess) { (void)hipGetLastError(); return -1; }
+    return d;
+}
+
+void bbhip_SetDevice(int device) { if (hipSetDevice(device) != hipSuccess) { fail("hipSetDevice(%d) failed", device); (void)hipGetLastError(); } }
+void bbhip_SetHostOnly(int host_only) { g_host_only = host_only != 0; }
+int  bbhip_IsHostOnly(void) { return g_host_only ? 1 : 0; }
+int  bbhip_IsDeviceAvailable(void) { return (!g_host_only && bbhip_GetDeviceCount() > 0) ? 1 : 0; }
+const char *bbhip_GetLastErrorString(void) { return g_last_error.c_str(); }
+
+void  *bbhip_LocalHeap_Malloc(size_t size) { return heap().alloc(size); }
+void   bbhip_LocalHeap_Free(void *ptr) { heap().release(ptr); }
+size_t bbhip_LocalHeap_GetMaxAllocSize(void) { return heap().max_alloc; }
+size_t bbhip_LocalHeap_GetAllocatedSize(void) { return heap().allocated; }
+void   bbhip_LocalHeap_GarbageCollect(void) { std::lock_guard<std::mutex> lk(heap().mtx); heap().collect_locked(); }
+
+void bbhip_KernelTimer_Enable(int enable) { g_timer_on = enable != 0; }
+
+int bbhip_KernelTimer_Read(int which, float *total_ms, int *launches)
+{
+    BBHIP_REQUIRE(which >= 0 && which < kTimedKinds && total_ms != nullptr && launches != nullptr);
+    float total = 0.0f;
+    int count = 0;
+    std::vector<TimedLaunch> keep;
+    for (auto &t : g_timed) {
+        if (t.which != which) { keep.push_back(t); continue; }
+        float ms = 0.0f;
+        BBHIP_TRY(hipEventSynchronize(t.stop));
+        BBHIP_TRY(hipEventElapsedTime(&ms, t.start, t.stop));
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+        total += ms;
+        ++count;
+    }
+    g_timed.swap(keep);
+    *total_ms = total;
+    *launches = count;
+    return 0;
+}
+
+void bbhip_SetDxMode(int mode) { g_dx_mode = mode ? 1 : 0; }
+int  bbhip_GetDxMode(void) { return g_dx_mode; }
+
+int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)
+{
+    BBHIP_REQUIRE(dev_dst != nullptr && size >= 0);
+    if (size == 0) { return 0; }
+    hipLaunchKernelGGL(fill_kernel, dim3(ceil_div(size, kBlock * 4)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, a, (size_t)size);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, float hi, int size, void *stream)
+{
+    BBHIP_REQUIRE(dev_dst != nullptr && dev_src != nullptr && size >= 0);
+    if (size == 0) { return 0; }
+    hipLaunchKernelGGL(clamp_kernel, dim3(ceil_div(size, kBlock)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, dev_src, lo, hi, size);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
+                             int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream)
+{
+    BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr);
+    BBHIP_REQUIRE(node_size > 0 && node_size <= 65535 * 1024 && frame_size > 0);
+    BBHIP_REQUIRE(x_frame_stride >= (frame_size + 31) / 32 && y_frame_stride >= frame_size);
+    // grid.y is limited to 65535 rows per launch
+    for (int n0 = 0; n0 < node_size; n0 += 65535) {
+        int const rows = (node_size - n0 < 65535) ? node_size - n0 : 65535;
+        hipLaunchKernelGGL(conv_bit_to_real_kernel, dim3(ceil_div(frame_size, kBlock), rows), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                           reinterpret_cast<uint32_t const *>(dev_x_buf) + (size_t)n0 * x_frame_stride,
+                           dev_y_buf + (size_t)n0 * y_frame_stride, value0, value1, frame_size, x_frame_stride, y_frame_stride);
+        BBHIP_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+// ---- StochasticLut ---------------------------------------------------------------------------------
+
+int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                     float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                     int input_binary, int lut_binarize, float unbinarize_bias, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = input_binary ? kXBinary : kXClamp; c.ymode = kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return forward_entry(c, stream);
+}
+
+int bbhip_bit_fp32_StochasticLut_Forward(int n, int const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                         float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                         int bin_frame_stride, int lut_binarize, float unbinarize_bias, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = bin_frame_stride; c.y_stride = frame_stride;
+    c.xmode = kXBit; c.ymode = kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return forward_entry(c, stream);
+}
+
+int bbhip_bit_bit_fp32_StochasticLut_Forward(int n, int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index,
+                                             float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                             int lut_binarize, float unbinarize_bias, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = kXBit; c.ymode = kYBit;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return forward_entry(c, stream);
+}
+
+int bbhip_fp32_DifferentiableLutN_ForwardNoBn(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float unbinarize_bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = binary_mode ? kXBinary : kXClamp; c.ymode = binary_mode ? kYBinarize : kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return forward_entry(c, stream);
+}
+
+int bbhip_fp32_StochasticLut_Backward(int n, float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+                                      float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index,
+                                      float const *dev_W, float *dev_dW, int reverse_index_stride,
+                                      int input_node_size, int output_node_size, int frame_size, int frame_stride,
+                                      int tmp_frame_size, int tmp_frame_stride, int input_binary, int lut_binarize,
+                                      float unbinarize_bias, void *stream)
+{
+    BackwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.dy = dev_dy_buf; c.dx = dev_dx_buf; c.dx_tmp = dev_dx_tmp;
+    c.idx = dev_input_index; c.rev = dev_reverse_index; c.W = dev_W; c.dW = dev_dW;
+    c.rev_stride = reverse_index_stride; c.input_node_size = input_node_size; c.output_node_size = output_node_size;
+    c.frame_size = frame_size; c.x_stride = frame_stride; c.frame_stride = frame_stride;
+    c.tmp_frame_size = tmp_frame_size; c.tmp_frame_stride = tmp_frame_stride;
+    c.xmode = input_binary ? kXBinary : kXClamp; c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return backward_entry(c, stream);
+}
+
+int bbhip_bit_fp32_StochasticLut_Backward(int n, int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+                                          float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index,
+                                          float const *dev_W, float *dev_dW, int reverse_index_stride,
+                                          int input_node_size, int output_node_size, int frame_size, int frame_stride,
+                                          int bin_frame_stride, int tmp_frame_size, int tmp_frame_stride,
+                                          int lut_binarize, float unbinarize_bias, void *stream)
+{
+    BackwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.dy = dev_dy_buf; c.dx = dev_dx_buf; c.dx_tmp = dev_dx_tmp;
+    c.idx = dev_input_index; c.rev = dev_reverse_index; c.W = dev_W; c.dW = dev_dW;
+    c.rev_stride = reverse_index_stride; c.input_node_size = input_node_size; c.output_node_size = output_node_size;
+    c.frame_size = frame_size; c.x_stride = bin_frame_stride; c.frame_stride = frame_stride;
+    c.tmp_frame_size = tmp_frame_size; c.tmp_frame_stride = tmp_frame_stride;
+    c.xmode = kXBit; c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return backward_entry(c, stream);
+}
+
+// ---- DifferentiableLut -----------------------------------------------------------------------------
+
+int bbhip_fp32_DifferentiableLutN_ForwardTraining(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode,
+        void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = binary_mode ? kXBinary : kXClamp; c.ymode = binary_mode ? kYBinarize : kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.running_mean = dev_running_mean_buf; c.running_var = dev_running_var_buf;
+    c.gamma = gamma; c.beta = beta; c.momentum = momentum;
+    return forward_entry(c, stream);
+}
+
+int bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(int n, int const *dev_x_buf, int *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = kXBit; c.ymode = kYBit;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.running_mean = dev_running_mean_buf; c.running_var = dev_running_var_buf;
+    c.gamma = gamma; c.beta = beta; c.momentum = momentum;
+    return forward_entry(c, stream);
+}
+
+int bbhip_fp32_DifferentiableLutN_ForwardInference(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float const *dev_running_mean_buf,
+        float const *dev_running_var_buf, float gamma, float beta, float unbinarize_bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = binary_mode ? kXBinary : kXClamp; c.ymode = binary_mode ? kYBinarize : kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 2; c.running_mean = const_cast<float *>(dev_running_mean_buf); c.running_var = const_cast<float *>(dev_running_var_buf);
+    c.gamma = gamma; c.beta = beta;
+    return forward_entry(c, stream);
+}
+
+int bbhip_bit_fp32_DifferentiableLutN_ForwardInference(int n, int const *dev_x_buf, int *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float const *dev_running_mean_buf,
+        float const *dev_running_var_buf, float gamma, float beta, float unbinarize_bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, void *stream)
+{
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = kXBit; c.ymode = kYBit;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 2; c.running_mean = const_cast<float *>(dev_running_mean_buf); c.running_var = const_cast<float *>(dev_running_var_buf);
+    c.gamma = gamma; c.beta = beta;
+    return forward_entry(c, stream);
+}
+
+int bbhip_fp32_DifferentiableLutN_Backward(int n, float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+        float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index, float const *dev_W,
+        float *dev_dW, float const *dev_mean_buf, float const *dev_rstd_buf, float *dev_dmean_tmp,
+        float *dev_dvar_tmp, float gamma, float beta, float unbinarize_bias, int reverse_index_stride,
+        int input_node_size, int output_node_size, int frame_size, int frame_stride, int tmp_frame_size,
+        int tmp_frame_stride, int lut_binarize, int binary_mode, void *stream)
+{
+    BackwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.dy = dev_dy_buf; c.dx = dev_dx_buf; c.dx_tmp = dev_dx_tmp;
+    c.idx = dev_input_index; c.rev = dev_reverse_index; c.W = dev_W; c.dW = dev_dW;
+    c.rev_stride = reverse_index_stride; c.input_node_size = input_node_size; c.output_node_size = output_node_size;
+    c.frame_size = frame_size; c.x_stride = frame_stride; c.frame_stride = frame_stride;
+    c.tmp_frame_size = tmp_frame_size; c.tmp_frame_stride = tmp_frame_stride;
+    c.xmode = binary_mode ? kXBinary : kXClamp; c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.dmean_tmp = dev_dmean_tmp; c.dvar_tmp = dev_dvar_tmp;
+    c.gamma = gamma; c.beta = beta;
+    return backward_entry(c, stream);
+}
+
+int bbhip_bit_fp32_DifferentiableLutN_Backward(int n, int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+        float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index, float const *dev_W,
+        float *dev_dW, float const *dev_mean_buf, float const *dev_rstd_buf, float *dev_dmean_tmp,
+        float *dev_dvar_tmp, float gamma, float beta, float unbinarize_bias, int reverse_index_stride,
+        int input_node_size, int output_node_size, int frame_size, int frame_stride, int x_frame_stride,
+        int tmp_frame_size, int tmp_frame_stride, int lut_binarize, void *stream)
+{
+    BackwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.dy = dev_dy_buf; c.dx = dev_dx_buf; c.dx_tmp = dev_dx_tmp;
+    c.idx = dev_input_index; c.rev = dev_reverse_index; c.W = dev_W; c.dW = dev_dW;
+    c.rev_stride = reverse_index_stride; c.input_node_size = input_node_size; c.output_node_size = output_node_size;
+    c.frame_size = frame_size; c.x_stride = x_frame_stride; c.frame_stride = frame_stride;
+    c.tmp_frame_size = tmp_frame_size; c.tmp_frame_stride = tmp_frame_stride;
+    c.xmode = kXBit; c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.dmean_tmp = dev_dmean_tmp; c.dvar_tmp = dev_dvar_tmp;
+    c.gamma = gamma; c.beta = beta;
+    return backward_entry(c, stream);
+}
+
+// ---- BinaryLut6 ------------------------------------------------------------------------------------
+
+int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
+                                 int node_size, int frame_size, int frame_stride, void *stream)
+{
+    BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr && dev_input_index != nullptr && dev_table != nullptr);
+    BBHIP_REQUIRE(node_size > 0 && frame_size > 0);
+    BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);
+    BinArgs a{};
+    a.x = reinterpret_cast<uint32_t const *>(dev_x_buf);
+    a.y = reinterpret_cast<uint32_t *>(dev_y_buf);
+    a.idx = dev_input_index; a.table = dev_table;
+    a.node_size = node_size; a.frame_size = frame_size; a.stride = frame_stride;
+    a.word_count = (frame_size + 31) / 32;
+    a.chunk = bin_chunk_words();
+    a.chunk_count = ceil_div(a.word_count, a.chunk);
+    a.tile_count = ceil_div(node_size, kWavesPerBlk);
+    BBHIP_REQUIRE((long long)a.chunk_count * a.tile_count <= 0x7fffffffLL);
+    {
+        ScopedTimer tm(kTimeBinary, static_cast<hipStream_t>(stream));
+        hipLaunchKernelGGL(binary_lut6_kernel<1>, dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, static_cast<hipStream_t>(stream), a);
+    }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,543 @@
+// HIP kernels of the differentiable-LUT path for gfx950 (wave64).
+//
+// Data layout (the FrameBuffer layout of the reference, include/bb/FrameBuffer.h:28-46): node-major, frame-minor.
+// Element (node n, frame f) of an fp32 buffer is p[n*stride + f]; of a packed buffer, bit (f & 31) of word
+// p[n*stride_words + (f >> 5)].  A wavefront always works on 64 consecutive frames of ONE output node: the node's
+// table and its N connection indices are wave-uniform (scalar registers / scalar loads), the N gathered input rows
+// are read as coalesced 256-byte segments, and the result row is written the same way.
+//
+// Work decomposition: a *unit* is (output node, chunk of frames); a workgroup of 4 waves takes 4 consecutive nodes of
+// one chunk.  Workgroups are numbered so that the ones an XCD receives (hardware deals consecutive workgroup ids
+// round-robin over the 8 XCDs) cover a contiguous range of chunks: every input row segment is then gathered by one
+// XCD only and the ~N-fold re-reads of a row by its consumers are served by that XCD's L2.
+#pragma once
+
+#include "lut_math.hpp"
+
+namespace bbhip {
+
+constexpr int kBlock        = 256;                 // threads per workgroup
+constexpr int kWavesPerBlk  = kBlock / kWave;      // = nodes per workgroup
+constexpr int kXcd          = 8;
+
+// logical workgroup index for hardware workgroup id b of a grid of B: XCD x (= b % 8) owns a contiguous range
+__device__ __forceinline__ int xcd_remap(int b, int B)
+{
+    int const q = B / kXcd, r = B % kXcd;
+    int const x = b % kXcd, k = b / kXcd;
+    return x * q + (x < r ? x : r) + k;
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { v += __shfl_xor(v, o, 64); }
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+//  table preparation: C = centred-monomial coefficients of W' (W' = lut_binarize ? W > 0.5 : W)
+// ------------------------------------------------------------------------------------------------
+template <int N>
+__global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
+                                                           int node_size, int lut_binarize)
+{
+    constexpr int NN = 1 << N;
+    int const t = blockIdx.x * kBlock + threadIdx.x;
+    int const total = node_size * NN;
+    float v = 0.0f;
+    if (t < total) {
+        v = W[t];
+        if (lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+    }
+    int const i = t & (NN - 1);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float const o = __shfl_xor(v, 1 << j, 64);
+        v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f;
+    }
+    if (t < total) { C[t] = v; }
+}
+
+// dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order)
+template <int N>
+__global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__restrict__ partial, float *__restrict__ dW,
+                                                            int node_size, int slab_count)
+{
+    constexpr int NN = 1 << N;
+    int const t = blockIdx.x * kBlock + threadIdx.x;
+    int const total = node_size * NN;
+    float v = 0.0f;
+    if (t < total) {
+        for (int s = 0; s < slab_count; ++s) { v += partial[(size_t)s * total + t]; }
+    }
+    int const i = t & (NN - 1);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float const o = __shfl_xor(v, 1 << j, 64);
+        v = ((i >> j) & 1) ? (o * 0.5f + v) : (v * 0.5f - o);
+    }
+    if (t < total) { dW[t] += v; }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  gather of one frame's inputs
+// ------------------------------------------------------------------------------------------------
+template <int N, int XMODE>
+struct Gather {
+    // rows[k]: wave-uniform pointer to the input row of connection k (float rows, or packed words for kXBit)
+    __device__ __forceinline__ static void load(void const *(&rows)[N], int f, bool ok, float bias, float (&z)[N])
+    {
+        if (XMODE == kXBit) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                uint32_t const w = ok ? reinterpret_cast<uint32_t const *>(rows[k])[f >> 5] : 0u;
+                z[k] = centre_bit(w, f & 31, bias);
+            }
+        }
+        else {
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                float const v = ok ? reinterpret_cast<float const *>(rows[k])[f] : 0.0f;
+                z[k] = centre<XMODE>(v, bias);
+            }
+        }
+    }
+};
+
+struct FwdArgs {
+    void const  *x;
+    void        *y;
+    int const   *idx;
+    float const *C;             // [O][2^N] centred coefficients
+    float const *mean;          // BN: per node (nullptr otherwise)
+    float const *rstd;
+    float       *stat_partial;  // STATS: [chunk][O][2] partial sums of (v - C0), (v - C0)^2
+    int   node_size, frame_size;
+    int   x_stride, y_stride;   // elements per node row (floats or words)
+    int   chunk;                // frames per unit, multiple of 64
+    int   chunk_count, tile_count;
+    float bias, gamma, beta;
+};
+
+// FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only
+template <int N, int XMODE, int YMODE, int FWD_KIND>
+__global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
+{
+    using D = LutDims<N>;
+    int const B    = a.chunk_count * a.tile_count;
+    int const lid  = xcd_remap(blockIdx.x, B);
+    int const ck   = lid / a.tile_count;
+    int const tile = lid - ck * a.tile_count;
+    int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
+    if (node >= a.node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    float C[D::NN];
+    LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
+    void const *rows[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        int const in = a.idx[node * N + k];
+        rows[k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
+                                   : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
+    }
+    float mean = 0.0f, rstd = 1.0f;
+    if (FWD_KIND == 1) { mean = a.mean[node]; rstd = a.rstd[node]; }
+    float const c0 = C[0];
+
+    int const f_begin = ck * a.chunk;
+    int const f_end   = min(f_begin + a.chunk, a.frame_size);
+    float s1 = 0.0f, s2 = 0.0f;
+
+    for (int f0 = f_begin; f0 < f_end; f0 += kWave) {
+        int const  f  = f0 + lane;
+        bool const ok = f < f_end;
+        float z[N];
+        Gather<N, XMODE>::load(rows, f, ok, a.bias, z);
+        float v = LutEval<N>::forward(C, z);
+
+        if (FWD_KIND == 2) {
+            float const d = ok ? (v - c0) : 0.0f;
+            s1 += d;
+            s2 = __builtin_fmaf(d, d, s2);
+            continue;
+        }
+        if (FWD_KIND == 1) {
+            v = (v - mean) * rstd;
+            v = v * a.gamma + a.beta;
+        }
+        if (YMODE == kYBit) {
+            uint64_t const m = __ballot(ok && (v > 0.5f));
+            uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
+            if (lane == 0)                          { yr[0] = (uint32_t)m; }
+            if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
+        }
+        else {
+            if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+            else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+            if (ok) { reinterpret_cast<float *>(a.y)[(size_t)node * a.y_stride + f] = v; }
+        }
+    }
+
+    if (FWD_KIND == 2) {
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        if (lane == 0) {
+            float *p = a.stat_partial + ((size_t)ck * a.node_size + node) * 2;
+            p[0] = s1;
+            p[1] = s2;
+        }
+    }
+}
+
+// per node: mean, var (>= 1e-5), rstd, running statistics (reference: include/bb/DifferentiableLutN.h:804-812)
+__global__ __launch_bounds__(kBlock) void bn_forward_finalize_kernel(float const *__restrict__ stat_partial, float const *__restrict__ C, int nn,
+                                                                    float *__restrict__ mean, float *__restrict__ rstd,
+                                                                    float *__restrict__ running_mean, float *__restrict__ running_var,
+                                                                    float momentum, int node_size, int chunk_count, int frame_size)
+{
+    int const node = blockIdx.x * kBlock + threadIdx.x;
+    if (node >= node_size) { return; }
+    float s1 = 0.0f, s2 = 0.0f;
+    for (int c = 0; c < chunk_count; ++c) {
+        float const *p = stat_partial + ((size_t)c * node_size + node) * 2;
+        s1 += p[0];
+        s2 += p[1];
+    }
+    float const r  = 1.0f / (float)frame_size;
+    float const m0 = s1 * r;                                  // mean of (v - C0)
+    float const m  = C[(size_t)node * nn] + m0;
+    float const var = fmaxf(1.0e-5f, s2 * r - m0 * m0);
+    float const rs  = 1.0f / sqrtf(var);
+    running_mean[node] = running_mean[node] * momentum + m   * (1.0f - momentum);
+    running_var[node]  = running_var[node]  * momentum + var * (1.0f - momentum);
+    mean[node] = m;
+    rstd[node] = rs;
+}
+
+// rstd = 1/sqrt(var) for inference (reference: DifferentiableLutN.h:866-868)
+__global__ __launch_bounds__(kBlock) void rsqrt_kernel(float const *__restrict__ var, float *__restrict__ rstd, int size)
+{
+    int const i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < size) { rstd[i] = 1.0f / sqrtf(var[i]); }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  backward
+// ------------------------------------------------------------------------------------------------
+struct BwdArgs {
+    void const  *x;
+    float const *dy;
+    float       *dx;            // DX_ATOMIC: [I][stride], zero-filled;  DX_TMP: dx_tmp [O*N][tmp_stride]
+    int const   *idx;
+    float const *C;
+    float       *dw_partial;    // [slab][O][2^N]   (BWD_KIND 0,1)
+    float const *mean;          // BN
+    float const *rstd;
+    float const *dmean;         // BN phase 1
+    float const *dvar;
+    float       *stat_partial;  // BN phase 0: [slab][O][2]
+    int   node_size, frame_size;
+    int   x_stride, dy_stride, dx_stride;
+    int   f_base, f_limit;      // frame range handled by this launch
+    int   slab;                 // frames per unit, multiple of 64
+    int   slab_first;           // index of the first slab of this launch in dw_partial
+    int   slab_count, tile_count;
+    float bias, gamma, beta, inv_frames;
+};
+
+enum DxMode : int { kDxAtomic = 0, kDxTmp = 1 };
+
+// BWD_KIND: 0 = plain LUT backward, 1 = backward through batch-norm (phase 1), 2 = batch-norm statistics (phase 0)
+template <int N, int XMODE, int BWD_KIND, int DXMODE>
+__global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
+{
+    using D = LutDims<N>;
+    __shared__ float red[kWavesPerBlk][16][kWave + 1];
+
+    int const B    = a.slab_count * a.tile_count;
+    int const lid  = xcd_remap(blockIdx.x, B);
+    int const sl   = lid / a.tile_count;
+    int const tile = lid - sl * a.tile_count;
+    int const wv   = threadIdx.x / kWave;
+    int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + wv);
+    if (node >= a.node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    float C[D::NN];
+    LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
+    void const *rows[N];
+    int ins[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        ins[k] = a.idx[node * N + k];
+        rows[k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)ins[k] * a.x_stride)
+                                   : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)ins[k] * a.x_stride);
+    }
+    float const *__restrict__ dyr = a.dy + (size_t)node * a.dy_stride;
+
+    float mean = 0.0f, rstd = 1.0f, dmean = 0.0f, dvarf = 0.0f;
+    if (BWD_KIND != 0) { mean = a.mean[node]; rstd = a.rstd[node]; }
+    if (BWD_KIND == 1) { dmean = a.dmean[node]; dvarf = a.dvar[node] * a.inv_frames; }
+    float const grs = a.gamma * rstd;
+
+    int const f_begin = a.f_base + sl * a.slab;
+    int const f_end   = min(f_begin + a.slab, a.f_limit);
+
+    float acc[D::NN];
+#pragma unroll
+    for (int i = 0; i < D::NN; ++i) { acc[i] = 0.0f; }
+    float s0 = 0.0f, s1 = 0.0f;
+
+    for (int f0 = f_begin; f0 < f_end; f0 += kWave) {
+        int const  f  = f0 + lane;
+        bool const ok = f < f_end;
+        float z[N];
+        Gather<N, XMODE>::load(rows, f, ok, a.bias, z);
+        float d = ok ? dyr[f] : 0.0f;
+
+        float zl[D::NL], zh[D::NH];
+#pragma unroll
+        for (int k = 0; k < D::NL; ++k) { zl[k] = z[k]; }
+#pragma unroll
+        for (int k = 0; k < D::NH; ++k) { zh[k] = z[D::NL + k]; }
+        float l[D::L], h[D::H], q[D::H];
+        monomials<D::NL>(zl, l);
+        monomials<D::NH>(zh, h);
+        LutEval<N>::partial_q(C, l, q);
+
+        if (BWD_KIND != 0) {
+            // hard-tanh window on the batch-norm output (reference: DifferentiableLutN.h:1206-1211, 1241-1246)
+            float const v = LutEval<N>::combine(h, q);
+            float const t = ((v - mean) * rstd) * a.gamma + a.beta;
+            if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
+            if (BWD_KIND == 2) {
+                s0 += d;
+                s1 = __builtin_fmaf(d, v - mean, s1);
+                continue;
+            }
+            // dL/d(LUT output) (reference: DifferentiableLutN.h:1248-1250)
+            d = ok ? (__builtin_fmaf(d, grs, dmean) + v * dvarf) : 0.0f;
+        }
+
+        float g[D::H];
+        g[0] = d;
+#pragma unroll
+        for (int j = 1; j < D::H; ++j) { g[j] = d * h[j]; }
+
+        // table gradient in the centred basis
+#pragma unroll
+        for (int j = 0; j < D::H; ++j) {
+            acc[j * D::L] += g[j];
+#pragma unroll
+            for (int i = 1; i < D::L; ++i) { acc[j * D::L + i] = __builtin_fmaf(g[j], l[i], acc[j * D::L + i]); }
+        }
+
+        // input gradients
+        float p[D::L];
+#pragma unroll
+        for (int i = 0; i < D::L; ++i) {
+            float s = g[0] * C[i];
+#pragma unroll
+            for (int j = 1; j < D::H; ++j) { s = __builtin_fmaf(g[j], C[j * D::L + i], s); }
+            p[i] = s;
+        }
+        float dxl[D::NL], dxh[D::NH];
+        LutEval<N>::template group_grad<D::NL>(l, p, dxl);
+        LutEval<N>::template group_grad<D::NH>(h, q, dxh);
+#pragma unroll
+        for (int k = 0; k < D::NH; ++k) { dxh[k] *= d; }
+
+        if (ok) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                float const val = (k < D::NL) ? dxl[k < D::NL ? k : 0] : dxh[k >= D::NL ? k - D::NL : 0];
+                if (DXMODE == kDxAtomic) {
+                    unsafeAtomicAdd(a.dx + (size_t)ins[k] * a.dx_stride + f, val);
+                }
+                else {
+                    a.dx[(size_t)(node * N + k) * a.dx_stride + (f - a.f_base)] = val;
+                }
+            }
+        }
+    }
+
+    if (BWD_KIND == 2) {
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        if (lane == 0) {
+            float *pp = a.stat_partial + ((size_t)(a.slab_first + sl) * a.node_size + node) * 2;
+            pp[0] = s0;
+            pp[1] = s1;
+        }
+        return;
+    }
+
+    // frame reduction of the 2^N per-lane accumulators through LDS, 16 at a time:
+    // lane i sums accumulator (i / 4), lanes (i % 4) * 16 .. + 15, then the 4 quarter sums are combined.
+    float *out = a.dw_partial + ((size_t)(a.slab_first + sl) * a.node_size + node) * D::NN;
+    constexpr int PASS = (D::NN + 15) / 16;
+#pragma unroll
+    for (int ps = 0; ps < PASS; ++ps) {
+        constexpr int CNT = D::NN < 16 ? D::NN : 16;
+#pragma unroll
+        for (int r = 0; r < CNT; ++r) { red[wv][r][lane] = acc[ps * 16 + r]; }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        int const r  = lane >> 2;
+        int const qd = lane & 3;
+        float s = 0.0f;
+        if (r < CNT) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t) { s += red[wv][r][qd * 16 + t]; }
+        }
+        s += __shfl_xor(s, 1, 64);
+        s += __shfl_xor(s, 2, 64);
+        if (qd == 0 && r < CNT) { out[ps * 16 + r] = s; }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// per node: dvar, dmean from the phase-0 sums (reference: DifferentiableLutN.h:1218-1222)
+__global__ __launch_bounds__(kBlock) void bn_backward_finalize_kernel(float const *__restrict__ stat_partial,
+                                                                     float const *__restrict__ mean, float const *__restrict__ rstd,
+                                                                     float *__restrict__ dmean, float *__restrict__ dvar,
+                                                                     float gamma, int node_size, int slab_count, int frame_size)
+{
+    int const node = blockIdx.x * kBlock + threadIdx.x;
+    if (node >= node_size) { return; }
+    float s0 = 0.0f, s1 = 0.0f;
+    for (int s = 0; s < slab_count; ++s) {
+        float const *p = stat_partial + ((size_t)s * node_size + node) * 2;
+        s0 += p[0];
+        s1 += p[1];
+    }
+    float const rs = rstd[node];
+    float const dstd   = -(gamma * s1) * (rs * rs);
+    float const dmeanx = -(gamma * s0) * rs;
+    float const dv = dstd * rs;
+    dvar[node]  = dv;
+    dmean[node] = (dmeanx - mean[node] * dv) * (1.0f / (float)frame_size);
+}
+
+// dx[in][f] = sum_k tmp[rev[in][k]][f - base], k = 1 .. rev[in][0]  (the reference's reverse-table order,
+// cuda/Common.cuh:174-202 and include/bb/FixedSizeConnectionTable.h:198-214); overwrites dx
+__global__ __launch_bounds__(kBlock) void dx_gather_kernel(float const *__restrict__ tmp, float *__restrict__ dx,
+                                                          int const *__restrict__ rev, int rev_stride, int input_node_size,
+                                                          int f_base, int f_limit, int dx_stride, int tmp_stride)
+{
+    int const f  = f_base + blockIdx.x * kBlock + threadIdx.x;
+    if (f >= f_limit) { return; }
+    for (int in = blockIdx.y; in < input_node_size; in += gridDim.y) {
+        int const *r = rev + (size_t)in * rev_stride;
+        int const cnt = r[0];
+        float s = 0.0f;
+        for (int k = 1; k <= cnt; ++k) { s += tmp[(size_t)r[k] * tmp_stride + (f - f_base)]; }
+        dx[(size_t)in * dx_stride + f] = s;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  elementwise helpers
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void fill_kernel(float *__restrict__ dst, float v, size_t size)
+{
+    size_t const i4 = ((size_t)blockIdx.x * kBlock + threadIdx.x) * 4;
+    if (i4 + 3 < size && ((uintptr_t)dst & 15) == 0) {
+        *reinterpret_cast<float4 *>(dst + i4) = make_float4(v, v, v, v);
+    }
+    else {
+        for (size_t i = i4; i < size && i < i4 + 4; ++i) { dst[i] = v; }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void clamp_kernel(float *__restrict__ dst, float const *__restrict__ src, float lo, float hi, int size)
+{
+    int const i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < size) { dst[i] = fminf(hi, fmaxf(lo, src[i])); }
+}
+
+// packed bits -> fp32 values (reference: cuda/ConvBitToReal.cu, include/bb/FrameBuffer.h:850-866)
+__global__ __launch_bounds__(kBlock) void conv_bit_to_real_kernel(uint32_t const *__restrict__ x, float *__restrict__ y, float v0, float v1,
+                                                                 int frame_size, int x_stride, int y_stride)
+{
+    int const f    = blockIdx.x * kBlock + threadIdx.x;
+    int const node = blockIdx.y;
+    if (f >= frame_size) { return; }
+    uint32_t const w = x[(size_t)node * x_stride + (f >> 5)];
+    y[(size_t)node * y_stride + f] = ((w >> (f & 31)) & 1u) ? v1 : v0;
+}
+
+// ------------------------------------------------------------------------------------------------
+//  BinaryLut6: y = table[x5 x4 x3 x2 x1 x0] on 32 frames per word, as a 6-level multiplexer tree of bit-selects
+//  (reference semantics: include/bb/BinaryLutN.h:436-463 — input k is index bit k, entries 0-31 in table word 0)
+// ------------------------------------------------------------------------------------------------
+struct BinArgs {
+    uint32_t const *x;
+    uint32_t       *y;
+    int const      *idx;
+    int const      *table;      // [O][2]
+    int node_size, frame_size, stride;   // stride in words
+    int word_count;             // (frame_size + 31) / 32
+    int chunk;                  // words per unit, multiple of 64
+    int chunk_count, tile_count;
+};
+
+__device__ __forceinline__ uint32_t bitsel(uint32_t s, uint32_t hi, uint32_t lo) { return (s & hi) | (~s & lo); }
+
+template <int WPL>   // words per lane per step
+__global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
+{
+    int const B    = a.chunk_count * a.tile_count;
+    int const lid  = xcd_remap(blockIdx.x, B);
+    int const ck   = lid / a.tile_count;
+    int const tile = lid - ck * a.tile_count;
+    int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
+    if (node >= a.node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    uint32_t const *rows[6];
+#pragma unroll
+    for (int k = 0; k < 6; ++k) { rows[k] = a.x + (size_t)a.idx[node * 6 + k] * a.stride; }
+    uint32_t *yr = a.y + (size_t)node * a.stride;
+
+    uint32_t const t0 = (uint32_t)a.table[node * 2 + 0], t1 = (uint32_t)a.table[node * 2 + 1];
+    uint32_t m[64];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+        m[k]      = ((t0 >> k) & 1u) ? 0xffffffffu : 0u;
+        m[k + 32] = ((t1 >> k) & 1u) ? 0xffffffffu : 0u;
+    }
+
+    int const w_begin = ck * a.chunk;
+    int const w_end   = min(w_begin + a.chunk, a.word_count);
+    uint32_t const tail_mask = (a.frame_size & 31) ? ((1u << (a.frame_size & 31)) - 1u) : 0xffffffffu;
+
+    for (int w0 = w_begin; w0 < w_end; w0 += kWave * WPL) {
+#pragma unroll
+        for (int u = 0; u < WPL; ++u) {
+            int const w = w0 + u * kWave + lane;
+            bool const ok = w < w_end;
+            uint32_t xv[6];
+#pragma unroll
+            for (int k = 0; k < 6; ++k) { xv[k] = ok ? rows[k][w] : 0u; }
+            uint32_t t[32];
+#pragma unroll
+            for (int k = 0; k < 32; ++k) { t[k] = bitsel(xv[0], m[2 * k + 1], m[2 * k]); }
+#pragma unroll
+            for (int lv = 1; lv < 6; ++lv) {
+#pragma unroll
+                for (int k = 0; k < (32 >> lv); ++k) { t[k] = bitsel(xv[lv], t[2 * k + 1], t[2 * k]); }
+            }
+            uint32_t r = t[0];
+            if (w == a.word_count - 1) { r &= tail_mask; }
+            if (ok) { yr[w] = r; }
+        }
+    }
+}
+
+}  // namespace bbhip

@@ -1,0 +1,238 @@
+"""Functional layer over the C ABI: torch device tensors in, torch device tensors out.
+
+Every function is a direct call of one entry point of include/bbhip.h on the current torch stream.  Buffers follow
+the FrameBuffer layout: ``[nodes, stride]`` float32 rows (stride >= frames) or ``[nodes, stride_words]`` int32 rows of
+packed bits.  Nothing here has a CPU fallback: without the built library, or off a GPU, calls raise.
+"""
+import torch
+
+from . import capi
+from .capi import check, lib, ptr, stream_ptr
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise capi.BbhipError("bbhip ops need device tensors")
+        if t is not None and not t.is_contiguous():
+            raise capi.BbhipError("bbhip ops need contiguous tensors")
+
+
+def set_dx_mode(mode):
+    """0: deterministic dx (dx_tmp + reverse table); 1: fp32 atomics."""
+    lib().bbhip_SetDxMode(int(mode))
+
+
+def vector_clamp_(t, lo=0.0, hi=1.0):
+    _dev(t)
+    check(lib().bbhip_fp32_Vector_clamp(ptr(t), ptr(t), lo, hi, t.numel(), stream_ptr()))
+    return t
+
+
+def vector_set_(t, value):
+    _dev(t)
+    check(lib().bbhip_fp32_Vector_set(ptr(t), value, t.numel(), stream_ptr()))
+    return t
+
+
+def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
+    _dev(xbits)
+    y = torch.empty((xbits.shape[0], y_stride), dtype=torch.float32, device=xbits.device)
+    check(lib().bbhip_fp32_ConvBitToReal(ptr(xbits), ptr(y), value0, value1, xbits.shape[0], frame_size,
+                                         xbits.shape[1], y_stride, stream_ptr()))
+    return y
+
+
+def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None):
+    _dev(x, idx, W, out)
+    O = idx.shape[0]
+    y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
+    check(lib().bbhip_fp32_StochasticLut_Forward(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, frame_size, x.shape[1],
+                                                 int(input_binary), int(lut_binarize), bias, stream_ptr()))
+    return y
+
+
+def bit_stochastic_lut_forward(n, xbits, idx, W, frame_size, y_stride, lut_binarize=False, bias=0.25):
+    _dev(xbits, idx, W)
+    O = idx.shape[0]
+    y = torch.empty((O, y_stride), dtype=torch.float32, device=xbits.device)
+    check(lib().bbhip_bit_fp32_StochasticLut_Forward(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), O, frame_size, y_stride,
+                                                     xbits.shape[1], int(lut_binarize), bias, stream_ptr()))
+    return y
+
+
+def bit_bit_stochastic_lut_forward(n, xbits, idx, W, frame_size, lut_binarize=False, bias=0.25):
+    _dev(xbits, idx, W)
+    O = idx.shape[0]
+    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    check(lib().bbhip_bit_bit_fp32_StochasticLut_Forward(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), O, frame_size,
+                                                         xbits.shape[1], int(lut_binarize), bias, stream_ptr()))
+    return y
+
+
+def _tmp_frames(output_nodes, n, frame_size, max_tmp_bytes=256 * 1024 * 1024):
+    """Frames per dx_tmp pass, as the reference sizes its scratch (include/bb/StochasticLutN.h:584-587)."""
+    t = max_tmp_bytes // (4 * output_nodes * n)
+    t = max(t, 32)
+    t = (t + 31) & ~0x1f
+    return min(t, frame_size)
+
+
+def _tmp_for(output_nodes, n, frame_size, device, max_tmp_bytes):
+    tf = _tmp_frames(output_nodes, n, frame_size, max_tmp_bytes)
+    ts = ((tf + 63) // 64) * 64
+    return torch.empty((output_nodes * n, ts), dtype=torch.float32, device=device), tf, ts
+
+
+def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_binary=False, lut_binarize=False, bias=0.25,
+                            dx_tmp=None, tmp_frame_size=None, max_tmp_bytes=256 * 1024 * 1024, out=None):
+    """dW is accumulated in place; returns dx [I, stride]. ``rev`` (reverse table) and dx_tmp are used by the
+    deterministic dx mode only."""
+    _dev(x, dy, idx, W, dW, rev, dx_tmp, out)
+    I = x.shape[0]; O = idx.shape[0]
+    dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
+    tf = ts = 0
+    if lib().bbhip_GetDxMode() == 0:
+        if dx_tmp is None:
+            dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
+        else:
+            ts = dx_tmp.shape[1]
+            tf = min(ts, frame_size) if tmp_frame_size is None else tmp_frame_size
+    check(lib().bbhip_fp32_StochasticLut_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
+                                                  0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,
+                                                  int(input_binary), int(lut_binarize), bias, stream_ptr()))
+    return dx
+
+
+def bit_stochastic_lut_backward(n, xbits, dy, idx, W, dW, frame_size, rev=None, lut_binarize=False, bias=0.25,
+                                max_tmp_bytes=256 * 1024 * 1024):
+    _dev(xbits, dy, idx, W, dW, rev)
+    I = xbits.shape[0]; O = idx.shape[0]
+    dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    dx_tmp, tf, ts = (None, 0, 0)
+    if lib().bbhip_GetDxMode() == 0:
+        dx_tmp, tf, ts = _tmp_for(O, n, frame_size, dy.device, max_tmp_bytes)
+    check(lib().bbhip_bit_fp32_StochasticLut_Backward(n, ptr(xbits), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
+                                                      0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1],
+                                                      xbits.shape[1], tf, ts, int(lut_binarize), bias, stream_ptr()))
+    return dx
+
+
+def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
+                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True):
+    """fp32 frames. running_mean / running_var are updated in place. returns (y, mean, rstd)."""
+    _dev(x, idx, W, running_mean, running_var)
+    O = idx.shape[0]
+    y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    mean = torch.empty(O, dtype=torch.float32, device=x.device)
+    rstd = torch.empty(O, dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_DifferentiableLutN_ForwardTraining(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
+                                                              ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
+                                                              O, frame_size, x.shape[1], int(lut_binarize), int(binary_mode),
+                                                              stream_ptr()))
+    return y, mean, rstd
+
+
+def bit_differentiable_lut_forward_training(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
+                                            momentum=0.9, bias=0.25, lut_binarize=False):
+    _dev(xbits, idx, W, running_mean, running_var)
+    O = idx.shape[0]
+    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    mean = torch.empty(O, dtype=torch.float32, device=xbits.device)
+    rstd = torch.empty(O, dtype=torch.float32, device=xbits.device)
+    check(lib().bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
+                                                                  ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
+                                                                  O, frame_size, xbits.shape[1], int(lut_binarize), stream_ptr()))
+    return y, mean, rstd
+
+
+def differentiable_lut_forward_inference(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
+                                         bias=0.25, lut_binarize=False, binary_mode=True):
+    _dev(x, idx, W, running_mean, running_var)
+    O = idx.shape[0]
+    y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_DifferentiableLutN_ForwardInference(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(running_mean),
+                                                               ptr(running_var), gamma, beta, bias, O, frame_size, x.shape[1],
+                                                               int(lut_binarize), int(binary_mode), stream_ptr()))
+    return y
+
+
+def bit_differentiable_lut_forward_inference(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3,
+                                             beta=0.5, bias=0.25, lut_binarize=False):
+    _dev(xbits, idx, W, running_mean, running_var)
+    O = idx.shape[0]
+    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    check(lib().bbhip_bit_fp32_DifferentiableLutN_ForwardInference(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), ptr(running_mean),
+                                                                   ptr(running_var), gamma, beta, bias, O, frame_size,
+                                                                   xbits.shape[1], int(lut_binarize), stream_ptr()))
+    return y
+
+
+def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_binarize=False, binary_mode=True):
+    _dev(x, idx, W)
+    O = idx.shape[0]
+    y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_DifferentiableLutN_ForwardNoBn(n, ptr(x), ptr(y), ptr(idx), ptr(W), bias, O, frame_size, x.shape[1],
+                                                          int(lut_binarize), int(binary_mode), stream_ptr()))
+    return y
+
+
+def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, rev=None, gamma=0.3, beta=0.5, bias=0.25,
+                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024):
+    _dev(x, dy, idx, W, dW, mean, rstd, rev)
+    I = x.shape[0]; O = idx.shape[0]
+    dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=x.device)
+    dmean = torch.empty(O, dtype=torch.float32, device=x.device)
+    dvar = torch.empty(O, dtype=torch.float32, device=x.device)
+    dx_tmp, tf, ts = (None, 0, 0)
+    if lib().bbhip_GetDxMode() == 0:
+        dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
+    check(lib().bbhip_fp32_DifferentiableLutN_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
+                                                       ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
+                                                       0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,
+                                                       int(lut_binarize), int(binary_mode), stream_ptr()))
+    return dx
+
+
+def bit_differentiable_lut_backward(n, xbits, dy, idx, W, dW, frame_size, mean, rstd, rev=None, gamma=0.3, beta=0.5,
+                                    bias=0.25, lut_binarize=False, max_tmp_bytes=256 * 1024 * 1024):
+    _dev(xbits, dy, idx, W, dW, mean, rstd, rev)
+    I = xbits.shape[0]; O = idx.shape[0]
+    dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    dmean = torch.empty(O, dtype=torch.float32, device=dy.device)
+    dvar = torch.empty(O, dtype=torch.float32, device=dy.device)
+    dx_tmp, tf, ts = (None, 0, 0)
+    if lib().bbhip_GetDxMode() == 0:
+        dx_tmp, tf, ts = _tmp_for(O, n, frame_size, dy.device, max_tmp_bytes)
+    check(lib().bbhip_bit_fp32_DifferentiableLutN_Backward(n, ptr(xbits), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W),
+                                                           ptr(dW), ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
+                                                           0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1],
+                                                           xbits.shape[1], tf, ts, int(lut_binarize), stream_ptr()))
+    return dx
+
+
+def binary_lut6_forward(xbits, idx, table, frame_size, out=None):
+    _dev(xbits, idx, table, out)
+    O = idx.shape[0]
+    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device) if out is None else out
+    check(lib().bbhip_bit_BinaryLut6_Forward(ptr(xbits), ptr(y), ptr(idx), ptr(table), O, frame_size, xbits.shape[1], stream_ptr()))
+    return y
+
+
+def reverse_table(idx, input_nodes):
+    """Reverse connection table as the reference builds it (include/bb/FixedSizeConnectionTable.h:180-215):
+    ``[input_nodes, 1 + max fan-out]`` int32, row r = [count, node*n + input ... ascending, zero tail].
+    Built on the host with numpy (index bookkeeping, not on the timed path); returned on idx's device."""
+    import numpy as np
+    h = idx.detach().cpu().numpy().astype(np.int64)
+    O, n = h.shape
+    flat = h.reshape(-1)
+    counts = np.bincount(flat, minlength=input_nodes)
+    stride = int(counts.max()) + 1 if flat.size else 1
+    order = np.argsort(flat, kind="stable")                      # ascending (node, input) within each input row
+    starts = np.concatenate([[0], np.cumsum(counts)[:-1]])
+    rev = np.zeros((input_nodes, stride), np.int32)
+    rev[:, 0] = counts
+    pos = np.arange(flat.size) - np.repeat(starts, counts)
+    rev[flat[order], 1 + pos] = order.astype(np.int32)
+    return torch.from_numpy(rev).to(idx.device)

@@ -1,0 +1,155 @@
+/*
+ * bbhip — C ABI of the MI355X (gfx950) differentiable-LUT library.
+ *
+ * Every entry point replaces one device entry point of BinaryBrain's CUDA library (declared in the reference's
+ * include/bbcu/bbcu.h; the file:line each one replaces is cited below).  The reference's entry points are C++
+ * function templates on the LUT width N; here N is the leading `int n` argument (2..6).  Otherwise the argument
+ * lists, their order and meaning are the reference's.
+ *
+ * Conventions (identical to the reference unless noted):
+ *   - all pointers are DEVICE pointers; the caller owns every buffer;
+ *   - frame buffers are node-major, frame-minor: element (node, frame) of an fp32 buffer is p[node*frame_stride + frame];
+ *     of a bit-packed buffer, bit (frame & 31) of the 32-bit word p[node*frame_stride + (frame >> 5)];
+ *     `frame_stride` counts elements (floats or 32-bit words) per node row;
+ *   - W and dW are [node_size][2^n] row-major fp32, input_index is [node_size][n] int32;
+ *   - y and dx are write-only, dW accumulates (dW += ...), running_mean/running_var are read-modify-write;
+ *   - the last argument is a hipStream_t passed as void* (NULL = the default stream); launches are asynchronous;
+ *   - return value: 0 on success; non-zero on a rejected argument or a HIP error (the reference prints and blocks on
+ *     stdin instead, include/bbcu/bbcu_util.h:17-36) — bbhip_GetLastErrorString() describes the last failure.
+ *
+ * Internal scratch (transformed tables, per-slab partial sums) comes from a library-owned arena that grows with
+ * hipMalloc on demand and is reused by later calls; calls that overlap on one device (different host threads or
+ * streams) race on it, exactly as the reference's allocator singleton is not thread-safe (cuda/LocalHeap.cu:174).
+ */
+#ifndef BBHIP_H_
+#define BBHIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- device runtime shim (reference: include/bbcu/bbcu.h:49-55, cuda/Manager.cu) ---- */
+int  bbhip_GetDeviceCount(void);
+int  bbhip_GetDevice(void);
+void bbhip_SetDevice(int device);
+void bbhip_SetHostOnly(int host_only);
+int  bbhip_IsHostOnly(void);
+int  bbhip_IsDeviceAvailable(void);
+const char *bbhip_GetLastErrorString(void);
+
+/* ---- caching device allocator (reference: include/bbcu/bbcu.h:63-67, cuda/LocalHeap.cu:88-139) ---- */
+void  *bbhip_LocalHeap_Malloc(size_t size);
+void   bbhip_LocalHeap_Free(void *ptr);
+size_t bbhip_LocalHeap_GetMaxAllocSize(void);
+size_t bbhip_LocalHeap_GetAllocatedSize(void);
+void   bbhip_LocalHeap_GarbageCollect(void);
+
+/* ---- how dx is accumulated over the fan-out of an input node (no counterpart in the reference) ----
+ * 0 (default): deterministic — per-connection gradients go to dx_tmp and are summed through reverse_index in the
+ *              reference's order (cuda/Common.cuh:174-202); needs dx_tmp and reverse_index.
+ * 1          : fp32 atomic adds into a zero-filled dx; dx_tmp and reverse_index may be NULL; summation order is
+ *              not reproducible between runs. */
+void bbhip_SetDxMode(int mode);
+int  bbhip_GetDxMode(void);
+
+/* ---- kernel timer (instrumentation; no counterpart in the reference) ----
+ * While enabled, every call brackets its dominant kernel (which: 0 = LUT forward kernel, 1 = LUT backward kernel,
+ * 2 = BinaryLut6 kernel) with HIP events on the launch stream.  Read waits for the recorded launches of one kind,
+ * returns their summed duration and count, and forgets them. */
+void bbhip_KernelTimer_Enable(int enable);
+int  bbhip_KernelTimer_Read(int which, float *total_ms, int *launches);
+
+/* ---- elementwise helpers ---- */
+/* bbcu_fp32_Vector_set, include/bbcu/bbcu.h:89-94 */
+int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream);
+/* bbcu_fp32_Vector_clamp, include/bbcu/bbcu.h:191-198 (W is clamped to [0,1] before every StochasticLut forward,
+ * include/bb/StochasticLutN.h:451) */
+int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, float hi, int size, void *stream);
+/* bbcu_ConvBitToReal<float>, include/bbcu/bbcu.h:246-258 */
+int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
+                             int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream);
+
+/* ---- StochasticLut ---- */
+/* bbcu_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:667-681 */
+int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                     float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                     int input_binary, int lut_binarize, float unbinarize_bias, void *stream);
+/* bbcu_bit_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:683-697 */
+int bbhip_bit_fp32_StochasticLut_Forward(int n, int const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                         float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                         int bin_frame_stride, int lut_binarize, float unbinarize_bias, void *stream);
+/* bbcu_bit_bit_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:699-712 */
+int bbhip_bit_bit_fp32_StochasticLut_Forward(int n, int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index,
+                                             float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                             int lut_binarize, float unbinarize_bias, void *stream);
+/* bbcu_fp32_StochasticLut_Backward<N>, include/bbcu/bbcu.h:715-737 */
+int bbhip_fp32_StochasticLut_Backward(int n, float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+                                      float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index,
+                                      float const *dev_W, float *dev_dW, int reverse_index_stride,
+                                      int input_node_size, int output_node_size, int frame_size, int frame_stride,
+                                      int tmp_frame_size, int tmp_frame_stride, int input_binary, int lut_binarize,
+                                      float unbinarize_bias, void *stream);
+/* bbcu_bit_fp32_StochasticLut_Backward<N>, include/bbcu/bbcu.h:739-761 */
+int bbhip_bit_fp32_StochasticLut_Backward(int n, int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+                                          float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index,
+                                          float const *dev_W, float *dev_dW, int reverse_index_stride,
+                                          int input_node_size, int output_node_size, int frame_size, int frame_stride,
+                                          int bin_frame_stride, int tmp_frame_size, int tmp_frame_stride,
+                                          int lut_binarize, float unbinarize_bias, void *stream);
+
+/* ---- DifferentiableLut (LUT fused with per-node batch normalisation and binarize / hard-tanh) ---- */
+/* bbcu_fp32_DifferentiableLutN_ForwardTraining<N>, include/bbcu/bbcu.h:518-539 */
+int bbhip_fp32_DifferentiableLutN_ForwardTraining(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode,
+        void *stream);
+/* bbcu_bit_fp32_DifferentiableLutN_ForwardTraining<N>, include/bbcu/bbcu.h:541-561 */
+int bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(int n, int const *dev_x_buf, int *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, void *stream);
+/* bbcu_fp32_DifferentiableLutN_ForwardInference<N>, include/bbcu/bbcu.h:563-581
+ * (rstd = 1/sqrt(running_var) and the hard-tanh clip follow the reference's CPU path, include/bb/DifferentiableLutN.h:866-897) */
+int bbhip_fp32_DifferentiableLutN_ForwardInference(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float const *dev_running_mean_buf,
+        float const *dev_running_var_buf, float gamma, float beta, float unbinarize_bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode, void *stream);
+/* bbcu_bit_fp32_DifferentiableLutN_ForwardInference<N>, include/bbcu/bbcu.h:583-600 */
+int bbhip_bit_fp32_DifferentiableLutN_ForwardInference(int n, int const *dev_x_buf, int *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float const *dev_running_mean_buf,
+        float const *dev_running_var_buf, float gamma, float beta, float unbinarize_bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, void *stream);
+/* bbcu_fp32_DifferentiableLutN_Backward<N>, include/bbcu/bbcu.h:602-630 */
+int bbhip_fp32_DifferentiableLutN_Backward(int n, float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+        float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index, float const *dev_W,
+        float *dev_dW, float const *dev_mean_buf, float const *dev_rstd_buf, float *dev_dmean_tmp,
+        float *dev_dvar_tmp, float gamma, float beta, float unbinarize_bias, int reverse_index_stride,
+        int input_node_size, int output_node_size, int frame_size, int frame_stride, int tmp_frame_size,
+        int tmp_frame_stride, int lut_binarize, int binary_mode, void *stream);
+/* bbcu_bit_fp32_DifferentiableLutN_Backward<N>, include/bbcu/bbcu.h:632-660 */
+int bbhip_bit_fp32_DifferentiableLutN_Backward(int n, int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+        float *dev_dx_tmp, int const *dev_input_index, int const *dev_reverse_index, float const *dev_W,
+        float *dev_dW, float const *dev_mean_buf, float const *dev_rstd_buf, float *dev_dmean_tmp,
+        float *dev_dvar_tmp, float gamma, float beta, float unbinarize_bias, int reverse_index_stride,
+        int input_node_size, int output_node_size, int frame_size, int frame_stride, int x_frame_stride,
+        int tmp_frame_size, int tmp_frame_stride, int lut_binarize, void *stream);
+/* DifferentiableLutN<N,float>::Forward without batch-norm on the reference's CPU path binarizes the output in binary
+ * mode (include/bb/DifferentiableLutN.h:994-1002); its CUDA path calls bbcu_fp32_StochasticLut_Forward, which only clips.
+ * This entry point gives the CPU behaviour: y = binary_mode ? (LUT > 0.5) : clip(LUT, 0, 1). */
+int bbhip_fp32_DifferentiableLutN_ForwardNoBn(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float const *dev_W, float unbinarize_bias,
+        int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode, void *stream);
+
+/* ---- BinaryLut6 ---- */
+/* bbcu_bit_BinatyLut6_Forward [sic], include/bbcu/bbcu.h:285-295. Bits of the last word beyond frame_size are written as 0. */
+int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
+                                 int node_size, int frame_size, int frame_stride, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif  /* BBHIP_H_ */

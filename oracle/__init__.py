@@ -324,3 +324,25 @@ def ref_reverse_table6(idx, input_node_size):
     rev = np.zeros((input_node_size, stride), np.int32)
     f(C.c_int(input_node_size), C.c_int(O), _ptr(idx), _ptr(rev), C.c_int(rev.size))
     return rev
+
+
+# ----------------------------------------------------------------------------------------------
+#  timed CPU baselines (used by bench.py only)
+# ----------------------------------------------------------------------------------------------
+
+def time_stochastic_lut6(x, dy, idx, W, reps=3, use_ref=None):
+    """Seconds per StochasticLut6 forward+backward on the host, one value per repetition (after one warm-up).
+    use_ref=True times the reference's own AVX2/OpenMP path, False the C restatement; None picks the reference when built."""
+    x = _c(x, np.float32); dy = _c(dy, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
+    I, F = x.shape; O = idx.shape[0]
+    secs = np.zeros(reps, np.float64)
+    if use_ref is None:
+        use_ref = have_ref()
+    if use_ref:
+        rc = ref().bbref_StochasticLut6_Time(C.c_int(I), C.c_int(O), C.c_int(F), _ptr(x), _ptr(idx), _ptr(W), _ptr(dy),
+                                             C.c_int(0), C.c_int(reps), _ptr(secs))
+        assert rc == 0
+    else:
+        lib().oracle_fp32_StochasticLut6_Time(_ptr(x), _ptr(dy), _ptr(idx), _ptr(W), C.c_int(I), C.c_int(O), C.c_int(F),
+                                              C.c_int(reps), _ptr(secs))
+    return secs, ("reference" if use_ref else "port")

@@ -638,3 +638,26 @@ int oracle_ReverseTable(int n, int32_t const *idx, int input_node_size, int outp
     }
     return stride;
 }
+
+
+/* ---- timed CPU baseline (port) ----------------------------------------------------------------- */
+#include <time.h>
+
+/* One warm-up, then `reps` repetitions of StochasticLut6 forward+backward (AVX2 association), wall-clock around the
+ * two calls only. */
+void oracle_fp32_StochasticLut6_Time(float const *x, float const *dy, int32_t const *idx, float const *W,
+                                     int input_node_size, int output_node_size, int frame_size, int reps, double *seconds)
+{
+    float *y  = (float *)malloc(sizeof(float) * (size_t)output_node_size * frame_size);
+    float *dx = (float *)malloc(sizeof(float) * (size_t)input_node_size * frame_size);
+    float *dW = (float *)calloc((size_t)output_node_size * 64, sizeof(float));
+    for (int r = -1; r < reps; ++r) {
+        struct timespec t0, t1;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        oracle_fp32_StochasticLut_Forward(6, x, y, idx, W, output_node_size, frame_size, frame_size, 0, 0, 0.25f, 1);
+        oracle_fp32_StochasticLut_Backward(6, x, dy, dx, idx, W, dW, input_node_size, output_node_size, frame_size, frame_size, 0, 0, 0.25f, 1);
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        if (r >= 0) { seconds[r] = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec); }
+    }
+    free(y); free(dx); free(dW);
+}

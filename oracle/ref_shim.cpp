@@ -11,6 +11,7 @@
 //
 // Built only where the reference tree is present; see oracle/Makefile.
 
+#include <chrono>
 #include <cstring>
 #include <cstdint>
 #include <vector>
@@ -196,6 +197,34 @@ int bbref_StochasticLut(int n, int bit_input, int I, int O, int F,
                               : run_stochastic<NN, float  >(I, O, F, x, idx, W, dy, y, dx, dW, binary_mode, lut_binarize, host_simd);
     switch (n) { BBREF_CASE(2) BBREF_CASE(3) BBREF_CASE(4) BBREF_CASE(5) BBREF_CASE(6) default: return -1; }
 #undef BBREF_CASE
+}
+
+// Times StochasticLutN<6,float>::Forward + Backward (AVX2/OpenMP host path) on caller data: one warm-up, then
+// `reps` repetitions timed with steady_clock around Forward+Backward only; seconds[r] receives each repetition.
+int bbref_StochasticLut6_Time(int I, int O, int F, float const *x, std::int32_t const *idx, float const *W,
+                              float const *dy, int lut_binarize, int reps, double *seconds)
+{
+    auto lut = bb::StochasticLutN<6, float, float>::Create((index_t)O);
+    lut->SendCommand("host_only true");
+    lut->SendCommand("lut_binarize " + onoff(lut_binarize));
+    bb::FrameBuffer x_buf((index_t)F, {(index_t)I}, BB_TYPE_FP32, true);
+    lut->SetInputShape(x_buf.GetShape());
+    for (int n = 0; n < O; ++n) for (int i = 0; i < 6; ++i) { lut->SetNodeConnectionIndex(n, i, idx[n * 6 + i]); }
+    {
+        auto Wp = lut->lock_W();
+        for (int n = 0; n < O; ++n) for (int i = 0; i < 64; ++i) { Wp(n, i) = W[n * 64 + i]; }
+    }
+    put_fp32(x_buf, x, I, F);
+    bb::FrameBuffer dy_buf((index_t)F, {(index_t)O}, BB_TYPE_FP32, true);
+    put_fp32(dy_buf, dy, O, F);
+    for (int r = -1; r < reps; ++r) {
+        auto t0 = std::chrono::steady_clock::now();
+        auto y_buf  = lut->Forward(x_buf, true);
+        auto dx_buf = lut->Backward(dy_buf);
+        auto t1 = std::chrono::steady_clock::now();
+        if (r >= 0) { seconds[r] = std::chrono::duration<double>(t1 - t0).count(); }
+    }
+    return 0;
 }
 
 // DifferentiableLutN<N,float|Bit,float>::Forward (+Backward when dy != NULL), host-only generic path.

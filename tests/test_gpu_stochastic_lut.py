@@ -1,0 +1,191 @@
+"""GPU parity of the StochasticLut entry points (through the C ABI) against the CPU oracle.
+
+Shapes follow the reference's own parity test (tests/gtest/StochasticLutNTest.cpp:235-246) plus the CPU-runnable
+benchmark configuration (784 -> 1024 nodes, 64 frames) and ragged frame counts.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from binarybrain_amd import synth
+from util import assert_bwd, assert_fwd, dev, host, rel_err
+
+pytestmark = pytest.mark.gpu
+
+REF_SHAPES = [(6, 1, 1), (14, 16, 8), (14, 1024, 8), (14, 1024, 3), (13, 17, 1529), (784, 1024, 64), (40, 33, 300)]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from binarybrain_amd import ops as o
+    yield o
+    o.set_dx_mode(0)
+
+
+def _case(rng, n, I, O, F, lo=-0.1, hi=1.1):
+    stride = synth.frame_stride_fp32(F)
+    idx = synth.wiring(rng, I, O, n)
+    W = oracle.vector_clamp(synth.lut_tables(rng, O, n, -0.2, 1.2))
+    x = synth.uniform_frames(rng, I, F, stride, lo, hi)
+    dy = synth.normal_frames(rng, O, F, stride)
+    return stride, idx, W, x, dy
+
+
+@pytest.mark.parametrize("shape", REF_SHAPES)
+@pytest.mark.parametrize("lut_binarize", [0, 1])
+@pytest.mark.parametrize("input_binary", [0, 1])
+def test_lut6_forward_backward(ops, shape, lut_binarize, input_binary):
+    I, O, F = shape
+    rng = np.random.default_rng(hash((I, O, F, lut_binarize, input_binary)) & 0xffff)
+    stride, idx, W, x, dy = _case(rng, 6, I, O, F)
+    dW0 = rng.standard_normal((O, 64)).astype(np.float32)
+    y_ref = oracle.stochastic_lut_forward(6, x, idx, W, F, input_binary, lut_binarize, 0.25, F % 8 == 0)
+    dx_ref, dW_ref = oracle.stochastic_lut_backward(6, x, dy, idx, W, F, dW0, input_binary, lut_binarize, 0.25, F % 8 == 0)
+
+    y = ops.stochastic_lut_forward(6, dev(x), dev(idx), dev(W), F, input_binary, lut_binarize)
+    assert_fwd(host(y)[:, :F], y_ref[:, :F], "y")
+    rev = ops.reverse_table(dev(idx), I)
+    assert np.array_equal(host(rev), oracle.reverse_table(6, idx, I))
+    for mode in (0, 1):
+        ops.set_dx_mode(mode)
+        dW = dev(dW0.copy())
+        dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, input_binary, lut_binarize)
+        assert_bwd(host(dx)[:, :F], dx_ref[:, :F], "dx mode %d" % mode)
+        assert_bwd(host(dW), dW_ref, "dW mode %d" % mode)
+    ops.set_dx_mode(0)
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 5])
+def test_other_widths(ops, n):
+    rng = np.random.default_rng(100 + n)
+    for (I, O, F) in [(12, 9, 70), (30, 64, 256)]:
+        for lut_binarize in (0, 1):
+            stride, idx, W, x, dy = _case(rng, n, I, O, F)
+            y_ref = oracle.stochastic_lut_forward(n, x, idx, W, F, 0, lut_binarize, 0.25, False)
+            dx_ref, dW_ref = oracle.stochastic_lut_backward(n, x, dy, idx, W, F, None, 0, lut_binarize, 0.25, False)
+            y = ops.stochastic_lut_forward(n, dev(x), dev(idx), dev(W), F, False, lut_binarize)
+            assert_fwd(host(y)[:, :F], y_ref[:, :F])
+            rev = ops.reverse_table(dev(idx), I)
+            for mode in (0, 1):
+                ops.set_dx_mode(mode)
+                dW = dev(np.zeros((O, 1 << n), np.float32))
+                dx = ops.stochastic_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, False, lut_binarize)
+                assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
+    ops.set_dx_mode(0)
+
+
+@pytest.mark.parametrize("n", [6, 4, 2])
+def test_bit_input(ops, n):
+    rng = np.random.default_rng(200 + n)
+    for (I, O, F) in [(24, 16, 70), (64, 40, 2048 + 33)]:
+        for lut_binarize in (0, 1):
+            idx = synth.wiring(rng, I, O, n); W = synth.lut_tables(rng, O, n)
+            xs = synth.frame_stride_bit(F); ys = synth.frame_stride_fp32(F)
+            xb = synth.bernoulli_bits(rng, I, F, xs); dy = synth.normal_frames(rng, O, F, ys)
+            y_ref = oracle.bit_stochastic_lut_forward(n, xb, idx, W, F, ys, lut_binarize)
+            dx_ref, dW_ref = oracle.bit_stochastic_lut_backward(n, xb, dy, idx, W, F, None, lut_binarize)
+            yb_ref = oracle.bit_bit_stochastic_lut_forward(n, xb, idx, W, F, lut_binarize)
+            y = ops.bit_stochastic_lut_forward(n, dev(xb), dev(idx), dev(W), F, ys, lut_binarize)
+            assert_fwd(host(y)[:, :F], y_ref[:, :F])
+            yb = ops.bit_bit_stochastic_lut_forward(n, dev(xb), dev(idx), dev(W), F, lut_binarize)
+            # inputs take two values, so the LUT output takes at most 2^n values per node: a threshold flip needs an
+            # exact tie at 0.5, which random tables do not produce -> bit-exact
+            assert np.array_equal(synth.unpack_bits(host(yb), F), synth.unpack_bits(yb_ref, F))
+            rev = ops.reverse_table(dev(idx), I)
+            for mode in (0, 1):
+                ops.set_dx_mode(mode)
+                dW = dev(np.zeros((O, 1 << n), np.float32))
+                dx = ops.bit_stochastic_lut_backward(n, dev(xb), dev(dy), dev(idx), dev(W), dW, F, rev, lut_binarize)
+                assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
+    ops.set_dx_mode(0)
+
+
+def test_golden_vectors_on_gpu(ops):
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "stochastic_lut.npz"))
+    for k in range(int(g["count"][0])):
+        p = "c%d_" % k
+        n, I, O, F, simd, binary_mode, lut_binarize = [int(v) for v in g[p + "meta"]]
+        if simd < 0:
+            continue
+        stride = synth.frame_stride_fp32(F)
+        x = np.zeros((I, stride), np.float32); x[:, :F] = g[p + "x"]
+        dy = np.zeros((O, stride), np.float32); dy[:, :F] = g[p + "dy"]
+        W = dev(g[p + "W"])
+        ops.vector_clamp_(W)
+        assert np.array_equal(host(W), g[p + "Wc"])
+        y = ops.stochastic_lut_forward(n, dev(x), dev(g[p + "idx"]), W, F, binary_mode, lut_binarize)
+        assert_fwd(host(y)[:, :F], g[p + "y"])
+        dW = dev(g[p + "dW0"])
+        rev = ops.reverse_table(dev(g[p + "idx"]), I)
+        dx = ops.stochastic_lut_backward(n, dev(x), dev(dy), dev(g[p + "idx"]), W, dW, F, rev, binary_mode, lut_binarize)
+        assert_bwd(host(dx)[:, :F], g[p + "dx"]); assert_bwd(host(dW), g[p + "dW"])
+
+
+def test_tmp_chunking_and_strides(ops):
+    # dx_tmp smaller than the frame range: the deterministic path walks the frames in several passes
+    rng = np.random.default_rng(5)
+    I, O, F = 50, 37, 1000
+    stride, idx, W, x, dy = _case(rng, 6, I, O, F)
+    dx_ref, dW_ref = oracle.stochastic_lut_backward(6, x, dy, idx, W, F, None, 0, 0, 0.25, True)
+    rev = ops.reverse_table(dev(idx), I)
+    ops.set_dx_mode(0)
+    dW = dev(np.zeros((O, 64), np.float32))
+    dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, max_tmp_bytes=4 * O * 6 * 96)
+    assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
+    # deterministic mode is reproducible bit for bit
+    dW2 = dev(np.zeros((O, 64), np.float32))
+    dx2 = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW2, F, rev, max_tmp_bytes=4 * O * 6 * 96)
+    assert np.array_equal(host(dx)[:, :F], host(dx2)[:, :F]) and np.array_equal(host(dW), host(dW2))
+
+
+def test_rejected_arguments(ops):
+    import torch
+    from binarybrain_amd.capi import BbhipError
+    x = torch.zeros((8, 64), device="cuda"); idx = torch.zeros((4, 6), dtype=torch.int32, device="cuda")
+    W = torch.zeros((4, 64), device="cuda")
+    with pytest.raises(BbhipError):
+        ops.stochastic_lut_forward(7, x, idx, W, 64)            # width outside 2..6
+    with pytest.raises(BbhipError):
+        ops.stochastic_lut_forward(6, x, idx, W, 65)            # stride shorter than the frames
+    with pytest.raises(BbhipError):
+        ops.stochastic_lut_forward(6, x, idx, W, 0)             # empty frame range
+    ops.set_dx_mode(0)
+    with pytest.raises(BbhipError):                              # deterministic dx without a reverse table
+        ops.stochastic_lut_backward(6, x, x[:4].contiguous(), idx, W, torch.zeros_like(W), 64, rev=None)
+
+
+def test_full_size_properties(ops):
+    """4096 -> 4096 nodes, 8192 frames: the oracle checks a slice of nodes; size-independent rules check the rest."""
+    import torch
+    rng = np.random.default_rng(42)
+    I = O = 4096; F = 8192
+    idx = synth.wiring(rng, I, O); W = synth.lut_tables(rng, O)
+    x = synth.uniform_frames(rng, I, F, F); dy = synth.normal_frames(rng, O, F, F)
+    xd, dyd, idxd, Wd = dev(x), dev(dy), dev(idx), dev(W)
+    y = ops.stochastic_lut_forward(6, xd, idxd, Wd, F)
+    sel = np.arange(0, O, 64)
+    y_ref = oracle.stochastic_lut_forward(6, x, idx[sel], W[sel], F)
+    assert_fwd(host(y)[sel], y_ref)
+    ops.set_dx_mode(1)
+    dW = torch.zeros((O, 64), device="cuda")
+    dx = ops.stochastic_lut_backward(6, xd, dyd, idxd, Wd, dW, F)
+    # sum_i prod_i = 1  =>  sum_i dW[o, i] = sum_f dy[o, f]
+    s = dy.astype(np.float64).sum(1)
+    assert np.abs(host(dW).astype(np.float64).sum(1) - s).max() <= 1e-4 * np.abs(s).max()
+    # dW of the selected nodes against the oracle (dW of a node depends on that node only)
+    _, dW_ref = oracle.stochastic_lut_backward(6, x, dy[sel], idx[sel], W[sel], F)
+    assert_bwd(host(dW)[sel], dW_ref)
+    # dx: deterministic and atomic accumulation agree, dx is linear in dy, and a slice of frames matches the oracle
+    ops.set_dx_mode(0)
+    rev = ops.reverse_table(idxd, I)
+    dWb = torch.zeros((O, 64), device="cuda")
+    dxb = ops.stochastic_lut_backward(6, xd, dyd, idxd, Wd, dWb, F, rev)
+    assert rel_err(host(dx), host(dxb)) <= 1e-5 and rel_err(host(dW), host(dWb)) <= 1e-5
+    dWc = torch.zeros((O, 64), device="cuda")
+    dxc = ops.stochastic_lut_backward(6, xd, (dyd * 2.0).contiguous(), idxd, Wd, dWc, F, rev)
+    assert rel_err(host(dxc), 2.0 * host(dxb)) <= 1e-6
+    fs = 256
+    dx_ref, _ = oracle.stochastic_lut_backward(6, np.ascontiguousarray(x[:, :fs]), np.ascontiguousarray(dy[:, :fs]), idx, W, fs)
+    assert_bwd(host(dxb)[:, :fs], dx_ref)
