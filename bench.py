@@ -51,7 +51,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "1")),
-                    help="0: deterministic dx through dx_tmp + reverse table; 1: fp32 atomics")
+                    help="0: deterministic input-centric dx; 1: fp32 atomics; 2: dx_tmp + reverse table")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -78,10 +78,10 @@ def main():
     y = torch.empty((O, F), device="cuda")
     dx = torch.empty((I, F), device="cuda")
     ops.set_dx_mode(args.dx_mode)
-    rev = ops.reverse_table(idx, I) if args.dx_mode == 0 else None
+    rev = ops.reverse_table(idx, I) if args.dx_mode != 1 else None
     dx_tmp = None
     tmp_frames = None
-    if args.dx_mode == 0:
+    if args.dx_mode == 2:
         tmp_frames = ops._tmp_frames(O, 6, F)
         dx_tmp = torch.empty((O * 6, ((tmp_frames + 63) // 64) * 64), device="cuda")
 
@@ -121,7 +121,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "StochasticLut6 fwd+bwd fp32, 4096 in x 4096 out x 8192 frames, uniform random 6-of-4096 wiring",
-                   "dx_mode": "atomic" if args.dx_mode else "deterministic (dx_tmp + reverse table)",
+                   "dx_mode": ["deterministic (input-centric, reverse table)", "atomic", "dx_tmp + reverse table"][args.dx_mode],
                    "lut_binarize": False, "binary": False},
         "hbm_frac_step": (fwd_b + bwd_b) / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": "lut_backward_kernel<6>", "achieved": achieved, "peak": HBM_PEAK_GBS,

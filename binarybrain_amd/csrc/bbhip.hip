@@ -57,7 +57,7 @@ int  g_dx_mode   = 0;
 // ------------------------------------------------------------------------------------------------
 //  optional kernel timer: HIP events around the dominant kernel of each entry point, on the launch stream
 // ------------------------------------------------------------------------------------------------
-enum TimedKernel : int { kTimeForward = 0, kTimeBackward = 1, kTimeBinary = 2, kTimedKinds = 3 };
+enum TimedKernel : int { kTimeForward = 0, kTimeBackward = 1, kTimeBinary = 2, kTimeDx = 3, kTimedKinds = 4 };
 struct TimedLaunch { hipEvent_t start, stop; int which; };
 bool g_timer_on = false;
 std::vector<TimedLaunch> g_timed;
@@ -88,8 +88,9 @@ int env_int(char const *name, int def)
 }
 
 // frames per unit; both are rounded to wavefront multiples where used
-int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 256); return ((v + 63) / 64) * 64; }
+int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 512); return ((v + 63) / 64) * 64; }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 512);  return ((v + 63) / 64) * 64; }
+int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return (v <= 64) ? 64 : (v <= 128) ? 128 : 256; }
 int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
 
 // ------------------------------------------------------------------------------------------------
@@ -181,11 +182,37 @@ int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStre
     BBHIP_BWD_CASE(kXClamp,  1, kDxAtomic) BBHIP_BWD_CASE(kXClamp,  1, kDxTmp)
     BBHIP_BWD_CASE(kXBinary, 1, kDxAtomic) BBHIP_BWD_CASE(kXBinary, 1, kDxTmp)
     BBHIP_BWD_CASE(kXBit,    1, kDxAtomic) BBHIP_BWD_CASE(kXBit,    1, kDxTmp)
+    BBHIP_BWD_CASE(kXClamp,  0, kDxNone) BBHIP_BWD_CASE(kXClamp,  1, kDxNone)
+    BBHIP_BWD_CASE(kXBinary, 0, kDxNone) BBHIP_BWD_CASE(kXBinary, 1, kDxNone)
+    BBHIP_BWD_CASE(kXBit,    0, kDxNone) BBHIP_BWD_CASE(kXBit,    1, kDxNone)
     BBHIP_BWD_CASE(kXClamp,  2, kDxTmp)
     BBHIP_BWD_CASE(kXBinary, 2, kDxTmp)
     BBHIP_BWD_CASE(kXBit,    2, kDxTmp)
 #undef BBHIP_BWD_CASE
     return fail("backward variant (x=%d, kind=%d, dx=%d) not built", xmode, kind, dxmode);
+}
+
+template <int N, int U>
+int dispatch_dx_u(int xmode, DxArgs const &a, hipStream_t st)
+{
+    dim3 const grid(a.chunk_count * a.tile_count), block(kBlock);
+    switch (xmode) {
+    case kXClamp:  hipLaunchKernelGGL((lut_dx_kernel<N, kXClamp, U>),  grid, block, 0, st, a); return 0;
+    case kXBinary: hipLaunchKernelGGL((lut_dx_kernel<N, kXBinary, U>), grid, block, 0, st, a); return 0;
+    case kXBit:    hipLaunchKernelGGL((lut_dx_kernel<N, kXBit, U>),    grid, block, 0, st, a); return 0;
+    }
+    return fail("dx variant (x=%d) not built", xmode);
+}
+
+template <int N>
+int dispatch_dx(int xmode, DxArgs const &a, hipStream_t st)
+{
+    switch (a.chunk) {
+    case 64:  return dispatch_dx_u<N, 1>(xmode, a, st);
+    case 128: return dispatch_dx_u<N, 2>(xmode, a, st);
+    case 256: return dispatch_dx_u<N, 4>(xmode, a, st);
+    }
+    return fail("dx chunk %d not built", a.chunk);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -301,8 +328,12 @@ int check_backward(BackwardCall const &c, int dxmode)
     int const x_need = (c.xmode == kXBit) ? (c.frame_size + 31) / 32 : c.frame_size;
     if (c.x_stride < x_need || c.frame_stride < c.frame_size) { return fail("backward: frame stride shorter than the frames"); }
     if ((long long)c.output_node_size * (1 << c.n) > 0x7fffffffLL) { return fail("backward: node_size too large"); }
+    if (dxmode == kDxNone) {
+        if (!c.rev)                                      { return fail("backward: deterministic dx needs reverse_index (or bbhip_SetDxMode(1))"); }
+        if (c.rev_stride < 1)                            { return fail("backward: reverse_index_stride=%d", c.rev_stride); }
+    }
     if (dxmode == kDxTmp) {
-        if (!(c.dx_tmp && c.rev))                        { return fail("backward: deterministic dx needs dx_tmp and reverse_index (or bbhip_SetDxMode(1))"); }
+        if (!(c.dx_tmp && c.rev))                        { return fail("backward: scratch-buffer dx needs dx_tmp and reverse_index"); }
         if (c.tmp_frame_size <= 0)                       { return fail("backward: tmp_frame_size=%d must be positive", c.tmp_frame_size); }
         int const span = c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size;
         if (c.tmp_frame_stride < span)                   { return fail("backward: tmp_frame_stride=%d shorter than tmp_frame_size", c.tmp_frame_stride); }
@@ -316,7 +347,7 @@ template <int N>
 int run_backward(BackwardCall const &c, hipStream_t st)
 {
     constexpr int NN = 1 << N;
-    int const dxmode = g_dx_mode ? kDxAtomic : kDxTmp;
+    int const dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
     if (check_backward(c, dxmode)) { return 1; }
 
     int const tile_count = ceil_div(c.output_node_size, kWavesPerBlk);
@@ -338,17 +369,30 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     }
     if ((long long)slab_total * tile_count > 0x7fffffffLL) { return fail("backward: grid too large"); }
 
+    size_t const conn       = (size_t)c.output_node_size * N;
     size_t const c_bytes    = align256((size_t)c.output_node_size * NN * sizeof(float));
     size_t const part_bytes = align256((size_t)slab_total * c.output_node_size * NN * sizeof(float));
     size_t const stat_bytes = c.bn ? align256((size_t)slab_total * c.output_node_size * 2 * sizeof(float)) : 0;
+    size_t const dtab_bytes = (dxmode == kDxNone) ? align256(conn * (NN / 2) * sizeof(float)) : 0;
+    size_t const otab_bytes = (dxmode == kDxNone) ? align256(conn * (N - 1) * sizeof(int)) : 0;
+    size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + part_bytes + stat_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes + dyh_bytes, &base)) { return 1; }
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
+    float *Dtab = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes);
+    int   *Otab = reinterpret_cast<int *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
+    float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes);
 
     launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
     BBHIP_LAUNCH_CHECK();
+    if (dxmode == kDxNone) {
+        size_t const total = conn * (NN / 2);
+        if (total > 0x7fffffffULL) { return fail("backward: node_size too large"); }
+        hipLaunchKernelGGL(deriv_table_kernel<N>, dim3(ceil_div((int)total, kBlock)), dim3(kBlock), 0, st, C, c.idx, Dtab, Otab, c.output_node_size);
+        BBHIP_LAUNCH_CHECK();
+    }
 
     BwdArgs a{};
     a.x = c.x; a.dy = c.dy; a.idx = c.idx; a.C = C;
@@ -383,8 +427,9 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         a.f_limit    = (a.f_base + range < c.frame_size) ? a.f_base + range : c.frame_size;
         a.slab_first = slab_first;
         a.slab_count = ceil_div(a.f_limit - a.f_base, slab);
-        if (dxmode == kDxAtomic) { a.dx = c.dx;     a.dx_stride = c.frame_stride; }
-        else                     { a.dx = c.dx_tmp; a.dx_stride = c.tmp_frame_stride; }
+        if (dxmode == kDxAtomic)    { a.dx = c.dx;     a.dx_stride = c.frame_stride; }
+        else if (dxmode == kDxTmp)  { a.dx = c.dx_tmp; a.dx_stride = c.tmp_frame_stride; }
+        else                        { a.dx = dyh;      a.dx_stride = c.frame_stride; }
         {
             ScopedTimer tm(kTimeBackward, st);
             if (dispatch_backward<N>(c.xmode, c.bn ? 1 : 0, dxmode, a, st)) { return 1; }
@@ -397,6 +442,23 @@ int run_backward(BackwardCall const &c, hipStream_t st)
             BBHIP_LAUNCH_CHECK();
         }
         slab_first += a.slab_count;
+    }
+
+    if (dxmode == kDxNone) {
+        DxArgs d{};
+        d.x = c.x; d.dy = c.bn ? dyh : c.dy; d.dx = c.dx; d.rev = c.rev; d.Dtab = Dtab; d.Otab = Otab;
+        d.rev_stride = c.rev_stride; d.input_node_size = c.input_node_size; d.frame_size = c.frame_size;
+        d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
+        d.chunk = dx_chunk_frames();                    // 64 frames x {1, 2, 4} wavefront-steps
+        d.chunk_count = ceil_div(c.frame_size, d.chunk);
+        d.tile_count  = ceil_div(c.input_node_size, kWavesPerBlk);
+        if ((long long)d.chunk_count * d.tile_count > 0x7fffffffLL) { return fail("backward: grid too large"); }
+        d.bias = c.bias;
+        {
+            ScopedTimer tm(kTimeDx, st);
+            if (dispatch_dx<N>(c.xmode, d, st)) { return 1; }
+        }
+        BBHIP_LAUNCH_CHECK();
     }
 
     int const total = c.output_node_size * NN;
@@ -529,7 +591,7 @@ int bbhip_KernelTimer_Read(int which, float *total_ms, int *launches)
     return 0;
 }
 
-void bbhip_SetDxMode(int mode) { g_dx_mode = mode ? 1 : 0; }
+void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
 int  bbhip_GetDxMode(void) { return g_dx_mode; }
 
 int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)

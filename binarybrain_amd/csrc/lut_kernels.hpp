@@ -85,22 +85,25 @@ __global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__rest
 // ------------------------------------------------------------------------------------------------
 template <int N, int XMODE>
 struct Gather {
-    // rows[k]: wave-uniform pointer to the input row of connection k (float rows, or packed words for kXBit)
-    __device__ __forceinline__ static void load(void const *(&rows)[N], int f, bool ok, float bias, float (&z)[N])
+    // rows[k]: wave-uniform pointer to the input row of connection k (float rows, or packed words for kXBit).
+    // fs is a frame index already clamped into the buffer, so every lane loads unconditionally and the N loads
+    // are issued back to back.
+    // The element offset is an unsigned 32-bit byte offset from the wave-uniform row pointer, which lets the load use the
+    // scalar-base + vector-offset addressing form (no per-load 64-bit vector add).
+    __device__ __forceinline__ static void load_raw(void const *(&rows)[N], int fs, uint32_t (&raw)[N])
     {
-        if (XMODE == kXBit) {
+        uint32_t const off = ((XMODE == kXBit) ? (uint32_t)(fs >> 5) : (uint32_t)fs) * 4u;
 #pragma unroll
-            for (int k = 0; k < N; ++k) {
-                uint32_t const w = ok ? reinterpret_cast<uint32_t const *>(rows[k])[f >> 5] : 0u;
-                z[k] = centre_bit(w, f & 31, bias);
-            }
+        for (int k = 0; k < N; ++k) {
+            raw[k] = *reinterpret_cast<uint32_t const *>(reinterpret_cast<char const *>(rows[k]) + off);
         }
-        else {
+    }
+
+    __device__ __forceinline__ static void centre_all(uint32_t const (&raw)[N], int fs, float bias, float (&z)[N])
+    {
 #pragma unroll
-            for (int k = 0; k < N; ++k) {
-                float const v = ok ? reinterpret_cast<float const *>(rows[k])[f] : 0.0f;
-                z[k] = centre<XMODE>(v, bias);
-            }
+        for (int k = 0; k < N; ++k) {
+            z[k] = (XMODE == kXBit) ? centre_bit(raw[k], fs & 31, bias) : centre<XMODE>(__uint_as_float(raw[k]), bias);
         }
     }
 };
@@ -133,8 +136,9 @@ __global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
-    float C[D::NN];
+    float C[D::NN], cv[D::H];
     LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
+    LutEval<N>::pin_constants(C, cv);
     void const *rows[N];
 #pragma unroll
     for (int k = 0; k < N; ++k) {
@@ -150,33 +154,45 @@ __global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
     int const f_end   = min(f_begin + a.chunk, a.frame_size);
     float s1 = 0.0f, s2 = 0.0f;
 
-    for (int f0 = f_begin; f0 < f_end; f0 += kWave) {
-        int const  f  = f0 + lane;
-        bool const ok = f < f_end;
-        float z[N];
-        Gather<N, XMODE>::load(rows, f, ok, a.bias, z);
-        float v = LutEval<N>::forward(C, z);
+    constexpr int U = 4;                         // wavefront-steps whose loads are issued together
+    int const f_last = a.frame_size - 1;
+    for (int fb = f_begin; fb < f_end; fb += kWave * U) {
+        uint32_t raw[U][N];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            Gather<N, XMODE>::load_raw(rows, min(fb + u * kWave + lane, f_last), raw[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int const f0 = fb + u * kWave;
+            if (f0 >= f_end) { break; }
+            int const  f  = f0 + lane;
+            bool const ok = f < f_end;
+            float z[N];
+            Gather<N, XMODE>::centre_all(raw[u], min(f, f_last), a.bias, z);
+            float v = LutEval<N>::forward(C, cv, z);
 
-        if (FWD_KIND == 2) {
-            float const d = ok ? (v - c0) : 0.0f;
-            s1 += d;
-            s2 = __builtin_fmaf(d, d, s2);
-            continue;
-        }
-        if (FWD_KIND == 1) {
-            v = (v - mean) * rstd;
-            v = v * a.gamma + a.beta;
-        }
-        if (YMODE == kYBit) {
-            uint64_t const m = __ballot(ok && (v > 0.5f));
-            uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
-            if (lane == 0)                          { yr[0] = (uint32_t)m; }
-            if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
-        }
-        else {
-            if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
-            else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
-            if (ok) { reinterpret_cast<float *>(a.y)[(size_t)node * a.y_stride + f] = v; }
+            if (FWD_KIND == 2) {
+                float const d = ok ? (v - c0) : 0.0f;
+                s1 += d;
+                s2 = __builtin_fmaf(d, d, s2);
+                continue;
+            }
+            if (FWD_KIND == 1) {
+                v = (v - mean) * rstd;
+                v = v * a.gamma + a.beta;
+            }
+            if (YMODE == kYBit) {
+                uint64_t const m = __ballot(ok && (v > 0.5f));
+                uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
+                if (lane == 0)                          { yr[0] = (uint32_t)m; }
+                if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
+            }
+            else {
+                if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+                else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+                if (ok) { reinterpret_cast<float *>(a.y)[(size_t)node * a.y_stride + f] = v; }
+            }
         }
     }
 
@@ -229,7 +245,8 @@ __global__ __launch_bounds__(kBlock) void rsqrt_kernel(float const *__restrict__
 struct BwdArgs {
     void const  *x;
     float const *dy;
-    float       *dx;            // DX_ATOMIC: [I][stride], zero-filled;  DX_TMP: dx_tmp [O*N][tmp_stride]
+    float       *dx;            // kDxAtomic: dx [I][stride], zero-filled;  kDxTmp: dx_tmp [O*N][tmp_stride];
+                                // kDxNone + batch-norm: dL/d(LUT output) [O][dx_stride] for the input-centric dx kernel
     int const   *idx;
     float const *C;
     float       *dw_partial;    // [slab][O][2^N]   (BWD_KIND 0,1)
@@ -247,9 +264,10 @@ struct BwdArgs {
     float bias, gamma, beta, inv_frames;
 };
 
-enum DxMode : int { kDxAtomic = 0, kDxTmp = 1 };
+enum DxMode : int { kDxAtomic = 0, kDxTmp = 1, kDxNone = 2 };
 
 // BWD_KIND: 0 = plain LUT backward, 1 = backward through batch-norm (phase 1), 2 = batch-norm statistics (phase 0)
+// DXMODE  : how (whether) the per-connection input gradients leave the kernel
 template <int N, int XMODE, int BWD_KIND, int DXMODE>
 __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 {
@@ -265,8 +283,9 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
-    float C[D::NN];
+    float C[D::NN], cv[D::H];
     LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
+    LutEval<N>::pin_constants(C, cv);
     void const *rows[N];
     int ins[N];
 #pragma unroll
@@ -284,80 +303,98 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 
     int const f_begin = a.f_base + sl * a.slab;
     int const f_end   = min(f_begin + a.slab, a.f_limit);
+    int const f_last  = a.frame_size - 1;
 
     float acc[D::NN];
 #pragma unroll
     for (int i = 0; i < D::NN; ++i) { acc[i] = 0.0f; }
     float s0 = 0.0f, s1 = 0.0f;
 
-    for (int f0 = f_begin; f0 < f_end; f0 += kWave) {
-        int const  f  = f0 + lane;
-        bool const ok = f < f_end;
-        float z[N];
-        Gather<N, XMODE>::load(rows, f, ok, a.bias, z);
-        float d = ok ? dyr[f] : 0.0f;
-
-        float zl[D::NL], zh[D::NH];
+    constexpr int U = 2;                         // wavefront-steps whose loads are issued together
+    for (int fb = f_begin; fb < f_end; fb += kWave * U) {
+        uint32_t raw[U][N];
+        float dyv[U];
 #pragma unroll
-        for (int k = 0; k < D::NL; ++k) { zl[k] = z[k]; }
-#pragma unroll
-        for (int k = 0; k < D::NH; ++k) { zh[k] = z[D::NL + k]; }
-        float l[D::L], h[D::H], q[D::H];
-        monomials<D::NL>(zl, l);
-        monomials<D::NH>(zh, h);
-        LutEval<N>::partial_q(C, l, q);
-
-        if (BWD_KIND != 0) {
-            // hard-tanh window on the batch-norm output (reference: DifferentiableLutN.h:1206-1211, 1241-1246)
-            float const v = LutEval<N>::combine(h, q);
-            float const t = ((v - mean) * rstd) * a.gamma + a.beta;
-            if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
-            if (BWD_KIND == 2) {
-                s0 += d;
-                s1 = __builtin_fmaf(d, v - mean, s1);
-                continue;
-            }
-            // dL/d(LUT output) (reference: DifferentiableLutN.h:1248-1250)
-            d = ok ? (__builtin_fmaf(d, grs, dmean) + v * dvarf) : 0.0f;
+        for (int u = 0; u < U; ++u) {
+            int const fs = min(fb + u * kWave + lane, f_last);
+            Gather<N, XMODE>::load_raw(rows, fs, raw[u]);
+            dyv[u] = *reinterpret_cast<float const *>(reinterpret_cast<char const *>(dyr) + (uint32_t)fs * 4u);
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int const f0 = fb + u * kWave;
+            if (f0 >= f_end) { break; }
+            int const  f  = f0 + lane;
+            bool const ok = f < f_end;
+            float z[N];
+            Gather<N, XMODE>::centre_all(raw[u], min(f, f_last), a.bias, z);
+            float d = ok ? dyv[u] : 0.0f;
 
-        float g[D::H];
-        g[0] = d;
+            float zl[D::NL], zh[D::NH];
 #pragma unroll
-        for (int j = 1; j < D::H; ++j) { g[j] = d * h[j]; }
+            for (int k = 0; k < D::NL; ++k) { zl[k] = z[k]; }
+#pragma unroll
+            for (int k = 0; k < D::NH; ++k) { zh[k] = z[D::NL + k]; }
+            float l[D::L], h[D::H], q[D::H];
+            monomials<D::NL>(zl, l);
+            monomials<D::NH>(zh, h);
+            if (BWD_KIND != 0 || DXMODE != kDxNone) { LutEval<N>::partial_q(C, cv, l, q); }
 
-        // table gradient in the centred basis
-#pragma unroll
-        for (int j = 0; j < D::H; ++j) {
-            acc[j * D::L] += g[j];
-#pragma unroll
-            for (int i = 1; i < D::L; ++i) { acc[j * D::L + i] = __builtin_fmaf(g[j], l[i], acc[j * D::L + i]); }
-        }
-
-        // input gradients
-        float p[D::L];
-#pragma unroll
-        for (int i = 0; i < D::L; ++i) {
-            float s = g[0] * C[i];
-#pragma unroll
-            for (int j = 1; j < D::H; ++j) { s = __builtin_fmaf(g[j], C[j * D::L + i], s); }
-            p[i] = s;
-        }
-        float dxl[D::NL], dxh[D::NH];
-        LutEval<N>::template group_grad<D::NL>(l, p, dxl);
-        LutEval<N>::template group_grad<D::NH>(h, q, dxh);
-#pragma unroll
-        for (int k = 0; k < D::NH; ++k) { dxh[k] *= d; }
-
-        if (ok) {
-#pragma unroll
-            for (int k = 0; k < N; ++k) {
-                float const val = (k < D::NL) ? dxl[k < D::NL ? k : 0] : dxh[k >= D::NL ? k - D::NL : 0];
-                if (DXMODE == kDxAtomic) {
-                    unsafeAtomicAdd(a.dx + (size_t)ins[k] * a.dx_stride + f, val);
+            if (BWD_KIND != 0) {
+                // hard-tanh window on the batch-norm output (reference: DifferentiableLutN.h:1206-1211, 1241-1246)
+                float const v = LutEval<N>::combine(h, q);
+                float const t = ((v - mean) * rstd) * a.gamma + a.beta;
+                if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
+                if (BWD_KIND == 2) {
+                    s0 += d;
+                    s1 = __builtin_fmaf(d, v - mean, s1);
+                    continue;
                 }
-                else {
-                    a.dx[(size_t)(node * N + k) * a.dx_stride + (f - a.f_base)] = val;
+                // dL/d(LUT output) (reference: DifferentiableLutN.h:1248-1250)
+                d = ok ? (__builtin_fmaf(d, grs, dmean) + v * dvarf) : 0.0f;
+                if (DXMODE == kDxNone && ok) { a.dx[(size_t)node * a.dx_stride + f] = d; }
+            }
+
+            float g[D::H];
+            g[0] = d;
+#pragma unroll
+            for (int j = 1; j < D::H; ++j) { g[j] = d * h[j]; }
+
+            // table gradient in the centred basis
+#pragma unroll
+            for (int j = 0; j < D::H; ++j) {
+                acc[j * D::L] += g[j];
+#pragma unroll
+                for (int i = 1; i < D::L; ++i) { acc[j * D::L + i] = __builtin_fmaf(g[j], l[i], acc[j * D::L + i]); }
+            }
+
+            if (DXMODE == kDxNone) { continue; }
+
+            // input gradients
+            float p[D::L];
+#pragma unroll
+            for (int i = 0; i < D::L; ++i) {
+                float s = g[0] * C[i];
+#pragma unroll
+                for (int j = 1; j < D::H; ++j) { s = __builtin_fmaf(g[j], C[j * D::L + i], s); }
+                p[i] = s;
+            }
+            float dxl[D::NL], dxh[D::NH];
+            LutEval<N>::template group_grad<D::NL>(l, p, dxl);
+            LutEval<N>::template group_grad<D::NH>(h, q, dxh);
+#pragma unroll
+            for (int k = 0; k < D::NH; ++k) { dxh[k] *= d; }
+
+            if (ok) {
+#pragma unroll
+                for (int k = 0; k < N; ++k) {
+                    float const val = (k < D::NL) ? dxl[k < D::NL ? k : 0] : dxh[k >= D::NL ? k - D::NL : 0];
+                    if (DXMODE == kDxAtomic) {
+                        unsafeAtomicAdd(a.dx + (size_t)ins[k] * a.dx_stride + f, val);
+                    }
+                    else {
+                        a.dx[(size_t)(node * N + k) * a.dx_stride + (f - a.f_base)] = val;
+                    }
                 }
             }
         }
@@ -399,6 +436,129 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  input-centric dx: one wavefront owns dx[input node][64 frames x U] and walks the node's fan-out list
+//  (the reverse table, in its ascending (node, input) order), re-evaluating dy/dx_k of each consumer from that
+//  consumer's other N-1 inputs.  By multilinearity dy/dx_k is itself a LUT over the other inputs whose
+//  centred coefficients are the entries of C with bit k set:  Dk[s] = C[insert_zero_bit(s, k) | (1 << k)].
+//  No scratch, no atomics; every dx element is written exactly once, summed in the reference's order.
+// ------------------------------------------------------------------------------------------------
+
+// per connection e = node*N + k:  coefficient table Dk [2^(N-1)] and the N-1 other input nodes
+template <int N>
+__global__ __launch_bounds__(kBlock) void deriv_table_kernel(float const *__restrict__ C, int const *__restrict__ idx,
+                                                            float *__restrict__ Dtab, int *__restrict__ Otab, int node_size)
+{
+    constexpr int NN = 1 << N, HN = NN / 2;
+    int const t = blockIdx.x * kBlock + threadIdx.x;
+    int const total = node_size * N * HN;
+    if (t >= total) { return; }
+    int const s = t % HN;
+    int const e = t / HN;
+    int const k = e % N;
+    int const node = e / N;
+    int const lo = s & ((1 << k) - 1);
+    int const hi = s >> k;
+    Dtab[t] = C[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)];
+    if (s < N - 1) {
+        int const j = (s < k) ? s : s + 1;           // the s-th other connection
+        Otab[(size_t)e * (N - 1) + s] = idx[node * N + j];
+    }
+}
+
+struct DxArgs {
+    void const  *x;
+    float const *dy;            // dL/d(LUT output) [O][dy_stride]
+    float       *dx;            // [I][dx_stride]
+    int const   *rev;           // reverse table [I][rev_stride]: count, then connection ids node*N + k
+    float const *Dtab;          // [O*N][2^(N-1)]
+    int const   *Otab;          // [O*N][N-1]
+    int   rev_stride, input_node_size, frame_size;
+    int   x_stride, dy_stride, dx_stride;
+    int   chunk, chunk_count, tile_count;
+    float bias;
+};
+
+template <int N, int XMODE, int U>          // U wavefront-steps per unit: chunk = 64 * U frames
+__global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
+{
+    constexpr int M  = N - 1;                 // variables of the derivative LUT
+    constexpr int ML = M / 2, MH = M - ML;
+    constexpr int L = 1 << ML, H = 1 << MH, HN = 1 << M;
+
+    int const B    = a.chunk_count * a.tile_count;
+    int const lid  = xcd_remap(blockIdx.x, B);
+    int const ck   = lid / a.tile_count;
+    int const tile = lid - ck * a.tile_count;
+    int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
+    if (in >= a.input_node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    int const f_begin = ck * a.chunk;
+    int const f_last  = a.frame_size - 1;
+    int fs[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) { fs[u] = min(f_begin + u * kWave + lane, f_last); }
+
+    float acc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
+
+    int const *__restrict__ r = a.rev + (size_t)in * a.rev_stride;
+    int const cnt = r[0];
+    for (int t = 1; t <= cnt; ++t) {
+        int const e    = r[t];
+        int const node = e / N;
+        float Dk[HN];
+#pragma unroll
+        for (int s = 0; s < HN; ++s) { Dk[s] = a.Dtab[(size_t)e * HN + s]; }
+        void const *rows[M];
+#pragma unroll
+        for (int j = 0; j < M; ++j) {
+            int const o = a.Otab[(size_t)e * M + j];
+            rows[j] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)o * a.x_stride)
+                                       : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)o * a.x_stride);
+        }
+        float const *__restrict__ dyr = a.dy + (size_t)node * a.dy_stride;
+
+        uint32_t raw[U][M];
+        float dyv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            Gather<M, XMODE>::load_raw(rows, fs[u], raw[u]);
+            dyv[u] = *reinterpret_cast<float const *>(reinterpret_cast<char const *>(dyr) + (uint32_t)fs[u] * 4u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float z[M];
+            Gather<M, XMODE>::centre_all(raw[u], fs[u], a.bias, z);
+            float zl[ML > 0 ? ML : 1], zh[MH];
+#pragma unroll
+            for (int k = 0; k < ML; ++k) { zl[k] = z[k]; }
+#pragma unroll
+            for (int k = 0; k < MH; ++k) { zh[k] = z[ML + k]; }
+            float l[L], h[H];
+            monomials<ML>(zl, l);
+            monomials<MH>(zh, h);
+            float v = 0.0f;
+#pragma unroll
+            for (int j = 0; j < H; ++j) {
+                float q = Dk[j * L];
+#pragma unroll
+                for (int i = 1; i < L; ++i) { q = __builtin_fmaf(l[i], Dk[j * L + i], q); }
+                v = (j == 0) ? q : __builtin_fmaf(h[j], q, v);
+            }
+            acc[u] = __builtin_fmaf(dyv[u], v, acc[u]);
+        }
+    }
+
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        int const f = f_begin + u * kWave + lane;
+        if (f < a.frame_size) { a.dx[(size_t)in * a.dx_stride + f] = acc[u]; }
     }
 }
 

@@ -94,12 +94,24 @@ struct LutEval {
         for (int i = 0; i < D::NN; ++i) { C[i] = Cg[i]; }
     }
 
-    // q[j] = sum_i C[j*L+i] * l[i]
-    __device__ __forceinline__ static void partial_q(float const (&C)[D::NN], float const (&l)[D::L], float (&q)[D::H])
+    // Vector-register copies of the H constant terms C[j*L].  A fused multiply-add may read only one scalar
+    // register, so "C[j*L] + l[1]*C[j*L+1]" needs one of the two coefficients in a vector register; copying them once
+    // per unit (instead of once per frame step) takes H moves out of the frame loop.  The asm keeps the compiler from
+    // re-materialising the copy inside the loop.
+    __device__ __forceinline__ static void pin_constants(float const (&C)[D::NN], float (&cv)[D::H])
     {
 #pragma unroll
         for (int j = 0; j < D::H; ++j) {
-            float a = C[j * D::L];
+            asm volatile("v_mov_b32 %0, %1" : "=v"(cv[j]) : "s"(C[j * D::L]));
+        }
+    }
+
+    // q[j] = sum_i C[j*L+i] * l[i], cv[j] = C[j*L] held in a vector register
+    __device__ __forceinline__ static void partial_q(float const (&C)[D::NN], float const (&cv)[D::H], float const (&l)[D::L], float (&q)[D::H])
+    {
+#pragma unroll
+        for (int j = 0; j < D::H; ++j) {
+            float a = cv[j];
 #pragma unroll
             for (int i = 1; i < D::L; ++i) {
                 a = __builtin_fmaf(l[i], C[j * D::L + i], a);
@@ -119,7 +131,7 @@ struct LutEval {
     }
 
     // y for one frame from the centred inputs z[0..N-1]
-    __device__ __forceinline__ static float forward(float const (&C)[D::NN], float const (&z)[N])
+    __device__ __forceinline__ static float forward(float const (&C)[D::NN], float const (&cv)[D::H], float const (&z)[N])
     {
         float zl[D::NL > 0 ? D::NL : 1], zh[D::NH];
 #pragma unroll
@@ -129,7 +141,7 @@ struct LutEval {
         float l[D::L], h[D::H], q[D::H];
         monomials<D::NL>(zl, l);
         monomials<D::NH>(zh, h);
-        partial_q(C, l, q);
+        partial_q(C, cv, l, q);
         return combine(h, q);
     }
 

@@ -19,7 +19,8 @@ def _dev(*ts):
 
 
 def set_dx_mode(mode):
-    """0: deterministic dx (dx_tmp + reverse table); 1: fp32 atomics."""
+    """0: deterministic dx, input-centric re-evaluation through the reverse table (default); 1: fp32 atomics;
+    2: the reference's scheme (per-connection gradients in dx_tmp, summed through the reverse table)."""
     lib().bbhip_SetDxMode(int(mode))
 
 
@@ -86,13 +87,13 @@ def _tmp_for(output_nodes, n, frame_size, device, max_tmp_bytes):
 
 def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_binary=False, lut_binarize=False, bias=0.25,
                             dx_tmp=None, tmp_frame_size=None, max_tmp_bytes=256 * 1024 * 1024, out=None):
-    """dW is accumulated in place; returns dx [I, stride]. ``rev`` (reverse table) and dx_tmp are used by the
-    deterministic dx mode only."""
+    """dW is accumulated in place; returns dx [I, stride]. ``rev`` (reverse table) is needed by dx modes 0 and 2,
+    dx_tmp by mode 2 only (allocated here when not given)."""
     _dev(x, dy, idx, W, dW, rev, dx_tmp, out)
     I = x.shape[0]; O = idx.shape[0]
     dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
     tf = ts = 0
-    if lib().bbhip_GetDxMode() == 0:
+    if lib().bbhip_GetDxMode() == 2:
         if dx_tmp is None:
             dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
         else:
@@ -110,7 +111,7 @@ def bit_stochastic_lut_backward(n, xbits, dy, idx, W, dW, frame_size, rev=None, 
     I = xbits.shape[0]; O = idx.shape[0]
     dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=dy.device)
     dx_tmp, tf, ts = (None, 0, 0)
-    if lib().bbhip_GetDxMode() == 0:
+    if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, dy.device, max_tmp_bytes)
     check(lib().bbhip_bit_fp32_StochasticLut_Backward(n, ptr(xbits), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                       0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1],
@@ -185,7 +186,7 @@ def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, re
     dmean = torch.empty(O, dtype=torch.float32, device=x.device)
     dvar = torch.empty(O, dtype=torch.float32, device=x.device)
     dx_tmp, tf, ts = (None, 0, 0)
-    if lib().bbhip_GetDxMode() == 0:
+    if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
     check(lib().bbhip_fp32_DifferentiableLutN_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                        ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
@@ -202,7 +203,7 @@ def bit_differentiable_lut_backward(n, xbits, dy, idx, W, dW, frame_size, mean, 
     dmean = torch.empty(O, dtype=torch.float32, device=dy.device)
     dvar = torch.empty(O, dtype=torch.float32, device=dy.device)
     dx_tmp, tf, ts = (None, 0, 0)
-    if lib().bbhip_GetDxMode() == 0:
+    if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, dy.device, max_tmp_bytes)
     check(lib().bbhip_bit_fp32_DifferentiableLutN_Backward(n, ptr(xbits), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W),
                                                            ptr(dW), ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,

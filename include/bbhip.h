@@ -47,16 +47,19 @@ size_t bbhip_LocalHeap_GetAllocatedSize(void);
 void   bbhip_LocalHeap_GarbageCollect(void);
 
 /* ---- how dx is accumulated over the fan-out of an input node (no counterpart in the reference) ----
- * 0 (default): deterministic — per-connection gradients go to dx_tmp and are summed through reverse_index in the
- *              reference's order (cuda/Common.cuh:174-202); needs dx_tmp and reverse_index.
+ * 0 (default): deterministic, no scratch — one wavefront per (input node, frame chunk) walks reverse_index in the
+ *              reference's order (cuda/Common.cuh:174-202, include/bb/FixedSizeConnectionTable.h:198-214) and
+ *              re-evaluates each consumer's dy/dx from that consumer's other inputs; needs reverse_index, ignores dx_tmp.
  * 1          : fp32 atomic adds into a zero-filled dx; dx_tmp and reverse_index may be NULL; summation order is
- *              not reproducible between runs. */
+ *              not reproducible between runs.
+ * 2          : the reference's scheme — per-connection gradients go to dx_tmp ([output_node_size*n][tmp_frame_stride],
+ *              tmp_frame_size frames per pass) and are summed through reverse_index; deterministic. */
 void bbhip_SetDxMode(int mode);
 int  bbhip_GetDxMode(void);
 
 /* ---- kernel timer (instrumentation; no counterpart in the reference) ----
  * While enabled, every call brackets its dominant kernel (which: 0 = LUT forward kernel, 1 = LUT backward kernel,
- * 2 = BinaryLut6 kernel) with HIP events on the launch stream.  Read waits for the recorded launches of one kind,
+ * 2 = BinaryLut6 kernel, 3 = input-centric dx kernel) with HIP events on the launch stream.  Read waits for the recorded launches of one kind,
  * returns their summed duration and count, and forgets them. */
 void bbhip_KernelTimer_Enable(int enable);
 int  bbhip_KernelTimer_Read(int which, float *total_ms, int *launches);

@@ -83,7 +83,7 @@ def test_fp32_training_inference_backward(ops, n, F):
         dx_ref, dW_ref = oracle.differentiable_lut_backward(n, x, dy, idx, W, F, mean_ref, rstd_ref, None, gamma, beta, 0.25,
                                                             lut_binarize, binary_mode)
         rev = ops.reverse_table(dev(idx), I)
-        for mode in (0, 1):
+        for mode in (0, 1, 2):
             ops.set_dx_mode(mode)
             dW = dev(np.zeros((O, 1 << n), np.float32))
             dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev,
@@ -149,7 +149,7 @@ def test_bit_variants(ops, n):
             _check_binary(synth.unpack_bits(host(yi), F), synth.unpack_bits(yi_ref, F), pre, "bit inference")
             dx_ref, dW_ref = oracle.bit_differentiable_lut_backward(n, xb, dy, idx, W, F, mean_ref, rstd_ref, lut_binarize=lut_binarize)
             rev = ops.reverse_table(dev(idx), I)
-            for mode in (0, 1):
+            for mode in (0, 1, 2):
                 ops.set_dx_mode(mode)
                 dW = dev(np.zeros((O, 1 << n), np.float32))
                 dx = ops.bit_differentiable_lut_backward(n, dev(xb), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev,

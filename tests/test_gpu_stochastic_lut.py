@@ -48,7 +48,7 @@ def test_lut6_forward_backward(ops, shape, lut_binarize, input_binary):
     assert_fwd(host(y)[:, :F], y_ref[:, :F], "y")
     rev = ops.reverse_table(dev(idx), I)
     assert np.array_equal(host(rev), oracle.reverse_table(6, idx, I))
-    for mode in (0, 1):
+    for mode in (0, 1, 2):
         ops.set_dx_mode(mode)
         dW = dev(dW0.copy())
         dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, input_binary, lut_binarize)
@@ -68,7 +68,7 @@ def test_other_widths(ops, n):
             y = ops.stochastic_lut_forward(n, dev(x), dev(idx), dev(W), F, False, lut_binarize)
             assert_fwd(host(y)[:, :F], y_ref[:, :F])
             rev = ops.reverse_table(dev(idx), I)
-            for mode in (0, 1):
+            for mode in (0, 1, 2):
                 ops.set_dx_mode(mode)
                 dW = dev(np.zeros((O, 1 << n), np.float32))
                 dx = ops.stochastic_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, False, lut_binarize)
@@ -94,7 +94,7 @@ def test_bit_input(ops, n):
             # exact tie at 0.5, which random tables do not produce -> bit-exact
             assert np.array_equal(synth.unpack_bits(host(yb), F), synth.unpack_bits(yb_ref, F))
             rev = ops.reverse_table(dev(idx), I)
-            for mode in (0, 1):
+            for mode in (0, 1, 2):
                 ops.set_dx_mode(mode)
                 dW = dev(np.zeros((O, 1 << n), np.float32))
                 dx = ops.bit_stochastic_lut_backward(n, dev(xb), dev(dy), dev(idx), dev(W), dW, F, rev, lut_binarize)
@@ -123,21 +123,37 @@ def test_golden_vectors_on_gpu(ops):
         assert_bwd(host(dx)[:, :F], g[p + "dx"]); assert_bwd(host(dW), g[p + "dW"])
 
 
-def test_tmp_chunking_and_strides(ops):
-    # dx_tmp smaller than the frame range: the deterministic path walks the frames in several passes
+def test_tmp_chunking_and_determinism(ops):
     rng = np.random.default_rng(5)
     I, O, F = 50, 37, 1000
     stride, idx, W, x, dy = _case(rng, 6, I, O, F)
     dx_ref, dW_ref = oracle.stochastic_lut_backward(6, x, dy, idx, W, F, None, 0, 0, 0.25, True)
     rev = ops.reverse_table(dev(idx), I)
-    ops.set_dx_mode(0)
+    # mode 2 with a dx_tmp smaller than the frame range: the frames are walked in several passes
+    ops.set_dx_mode(2)
     dW = dev(np.zeros((O, 64), np.float32))
     dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, max_tmp_bytes=4 * O * 6 * 96)
     assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
-    # deterministic mode is reproducible bit for bit
-    dW2 = dev(np.zeros((O, 64), np.float32))
-    dx2 = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW2, F, rev, max_tmp_bytes=4 * O * 6 * 96)
-    assert np.array_equal(host(dx)[:, :F], host(dx2)[:, :F]) and np.array_equal(host(dW), host(dW2))
+    # the deterministic modes are reproducible bit for bit
+    for mode in (0, 2):
+        ops.set_dx_mode(mode)
+        outs = []
+        for _ in range(2):
+            dW = dev(np.zeros((O, 64), np.float32))
+            dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev)
+            outs.append((host(dx)[:, :F].copy(), host(dW).copy()))
+        assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    ops.set_dx_mode(0)
+    # an input node nobody reads gets dx = 0
+    idx2 = idx.copy(); idx2[idx2 == 7] = 8
+    for o in range(O):                       # keep the 6 inputs of a node distinct
+        while len(set(idx2[o])) < 6:
+            idx2[o] = synth.wiring(rng, I, 1)[0]; idx2[o][idx2[o] == 7] = 9
+    rev2 = ops.reverse_table(dev(idx2), I)
+    dW = dev(np.zeros((O, 64), np.float32))
+    dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx2), dev(W), dW, F, rev2)
+    if not (idx2 == 7).any():
+        assert np.array_equal(host(dx)[7, :F], np.zeros(F, np.float32))
 
 
 def test_rejected_arguments(ops):
