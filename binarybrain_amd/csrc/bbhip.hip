@@ -90,7 +90,8 @@ int env_int(char const *name, int def)
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 512); return ((v + 63) / 64) * 64; }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 512);  return ((v + 63) / 64) * 64; }
-int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return (v <= 64) ? 64 : (v <= 128) ? 128 : 256; }
+int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 256); return ((v + 63) / 64) * 64; }
+int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 4); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
 int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
 
 // ------------------------------------------------------------------------------------------------
@@ -205,14 +206,14 @@ int dispatch_dx_u(int xmode, DxArgs const &a, hipStream_t st)
 }
 
 template <int N>
-int dispatch_dx(int xmode, DxArgs const &a, hipStream_t st)
+int dispatch_dx(int xmode, int steps, DxArgs const &a, hipStream_t st)
 {
-    switch (a.chunk) {
-    case 64:  return dispatch_dx_u<N, 1>(xmode, a, st);
-    case 128: return dispatch_dx_u<N, 2>(xmode, a, st);
-    case 256: return dispatch_dx_u<N, 4>(xmode, a, st);
+    switch (steps) {
+    case 1: return dispatch_dx_u<N, 1>(xmode, a, st);
+    case 2: return dispatch_dx_u<N, 2>(xmode, a, st);
+    case 4: return dispatch_dx_u<N, 4>(xmode, a, st);
     }
-    return fail("dx chunk %d not built", a.chunk);
+    return fail("dx kernel with %d wavefront-steps per pass not built", steps);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -369,28 +370,27 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     }
     if ((long long)slab_total * tile_count > 0x7fffffffLL) { return fail("backward: grid too large"); }
 
-    size_t const conn       = (size_t)c.output_node_size * N;
     size_t const c_bytes    = align256((size_t)c.output_node_size * NN * sizeof(float));
     size_t const part_bytes = align256((size_t)slab_total * c.output_node_size * NN * sizeof(float));
     size_t const stat_bytes = c.bn ? align256((size_t)slab_total * c.output_node_size * 2 * sizeof(float)) : 0;
-    size_t const dtab_bytes = (dxmode == kDxNone) ? align256(conn * (NN / 2) * sizeof(float)) : 0;
-    size_t const otab_bytes = (dxmode == kDxNone) ? align256(conn * (N - 1) * sizeof(int)) : 0;
+    size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;
+    size_t const dtab_bytes = align256(term_count * sizeof(int));
+    size_t const otab_bytes = 0;
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     char *base = nullptr;
     if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes + dyh_bytes, &base)) { return 1; }
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
-    float *Dtab = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes);
-    int   *Otab = reinterpret_cast<int *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
+    int   *term = reinterpret_cast<int *>(base + c_bytes + part_bytes + stat_bytes);
     float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes);
 
     launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
     BBHIP_LAUNCH_CHECK();
-    if (dxmode == kDxNone) {
-        size_t const total = conn * (NN / 2);
-        if (total > 0x7fffffffULL) { return fail("backward: node_size too large"); }
-        hipLaunchKernelGGL(deriv_table_kernel<N>, dim3(ceil_div((int)total, kBlock)), dim3(kBlock), 0, st, C, c.idx, Dtab, Otab, c.output_node_size);
+    if (dxmode == kDxNone && term_count > 0) {
+        size_t const blocks = (term_count + kBlock - 1) / kBlock;
+        if (blocks > 0x7fffffffULL) { return fail("backward: reverse table too large"); }
+        hipLaunchKernelGGL(term_table_kernel<N>, dim3((unsigned)blocks), dim3(kBlock), 0, st, C, c.idx, c.rev, c.rev_stride, c.input_node_size, term);
         BBHIP_LAUNCH_CHECK();
     }
 
@@ -446,17 +446,18 @@ int run_backward(BackwardCall const &c, hipStream_t st)
 
     if (dxmode == kDxNone) {
         DxArgs d{};
-        d.x = c.x; d.dy = c.bn ? dyh : c.dy; d.dx = c.dx; d.rev = c.rev; d.Dtab = Dtab; d.Otab = Otab;
+        d.x = c.x; d.dy = c.bn ? dyh : c.dy; d.dx = c.dx; d.rev = c.rev; d.term = term;
         d.rev_stride = c.rev_stride; d.input_node_size = c.input_node_size; d.frame_size = c.frame_size;
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
-        d.chunk = dx_chunk_frames();                    // 64 frames x {1, 2, 4} wavefront-steps
+        int const steps = dx_pass_steps();              // wavefront-steps per pass: {1, 2, 4}
+        d.chunk = ((dx_chunk_frames() + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
         d.chunk_count = ceil_div(c.frame_size, d.chunk);
         d.tile_count  = ceil_div(c.input_node_size, kWavesPerBlk);
         if ((long long)d.chunk_count * d.tile_count > 0x7fffffffLL) { return fail("backward: grid too large"); }
         d.bias = c.bias;
         {
             ScopedTimer tm(kTimeDx, st);
-            if (dispatch_dx<N>(c.xmode, d, st)) { return 1; }
+            if (dispatch_dx<N>(c.xmode, steps, d, st)) { return 1; }
         }
         BBHIP_LAUNCH_CHECK();
     }

@@ -447,26 +447,43 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 //  No scratch, no atomics; every dx element is written exactly once, summed in the reference's order.
 // ------------------------------------------------------------------------------------------------
 
-// per connection e = node*N + k:  coefficient table Dk [2^(N-1)] and the N-1 other input nodes
+// Term table for the input-centric dx kernel: for input node `in` and its t-th consumer connection (t-th entry of
+// the reverse-table row, e = node*N + k) one record of kTermHead + 2^(N-1) dwords at
+// ((in * max_fan + t) * record):  [0 .. N-2] the consumer's other input nodes (ascending connection order, k skipped),
+// [N-1] the consumer node, rest of the head unused, then the 2^(N-1) coefficients Dk.  All records of one input
+// node are contiguous, so a wavefront reads its whole work list from one base address with scalar loads.
+constexpr int kTermHead = 8;
+
 template <int N>
-__global__ __launch_bounds__(kBlock) void deriv_table_kernel(float const *__restrict__ C, int const *__restrict__ idx,
-                                                            float *__restrict__ Dtab, int *__restrict__ Otab, int node_size)
+__global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restrict__ C, int const *__restrict__ idx,
+                                                           int const *__restrict__ rev, int rev_stride, int input_node_size,
+                                                           int *__restrict__ term)
 {
-    constexpr int NN = 1 << N, HN = NN / 2;
-    int const t = blockIdx.x * kBlock + threadIdx.x;
-    int const total = node_size * N * HN;
+    constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN;
+    int const max_fan = rev_stride - 1;
+    long long const t = (long long)blockIdx.x * kBlock + threadIdx.x;
+    long long const total = (long long)input_node_size * max_fan * REC;
     if (t >= total) { return; }
-    int const s = t % HN;
-    int const e = t / HN;
-    int const k = e % N;
-    int const node = e / N;
-    int const lo = s & ((1 << k) - 1);
-    int const hi = s >> k;
-    Dtab[t] = C[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)];
-    if (s < N - 1) {
-        int const j = (s < k) ? s : s + 1;           // the s-th other connection
-        Otab[(size_t)e * (N - 1) + s] = idx[node * N + j];
+    int const w    = (int)(t % REC);
+    long long const rec = t / REC;
+    int const slot = (int)(rec % max_fan);
+    int const in   = (int)(rec / max_fan);
+    int const *r = rev + (size_t)in * rev_stride;
+    int v = 0;
+    if (slot < r[0]) {
+        int const e = r[1 + slot];
+        int const k = e % N;
+        int const node = e / N;
+        if (w < N - 1)            { v = idx[node * N + ((w < k) ? w : w + 1)]; }
+        else if (w == N - 1)      { v = node; }
+        else if (w >= kTermHead)  {
+            int const sidx = w - kTermHead;
+            int const lo = sidx & ((1 << k) - 1);
+            int const hi = sidx >> k;
+            v = __float_as_int(C[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)]);
+        }
     }
+    term[t] = v;
 }
 
 struct DxArgs {
@@ -474,67 +491,59 @@ struct DxArgs {
     float const *dy;            // dL/d(LUT output) [O][dy_stride]
     float       *dx;            // [I][dx_stride]
     int const   *rev;           // reverse table [I][rev_stride]: count, then connection ids node*N + k
-    float const *Dtab;          // [O*N][2^(N-1)]
-    int const   *Otab;          // [O*N][N-1]
+    int const   *term;          // term table, see term_table_kernel
     int   rev_stride, input_node_size, frame_size;
     int   x_stride, dy_stride, dx_stride;
     int   chunk, chunk_count, tile_count;
     float bias;
 };
 
+// ------------------------------------------------------------------------------------------------
+//  input-centric dx: one wavefront owns dx[input node][64 frames x U] and walks the node's fan-out list
+//  (the reverse table, in its ascending (node, input) order), re-evaluating dy/dx_k of each consumer from that
+//  consumer's other N-1 inputs.  By multilinearity dy/dx_k is itself a LUT over the other inputs whose
+//  centred coefficients are the entries of C with bit k set:  Dk[s] = C[insert_zero_bit(s, k) | (1 << k)].
+//  No scratch traffic, no atomics; every dx element is written exactly once, summed in the reference's order.
+// ------------------------------------------------------------------------------------------------
 template <int N, int XMODE, int U>          // U wavefront-steps per unit: chunk = 64 * U frames
-__global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
-{
-    constexpr int M  = N - 1;                 // variables of the derivative LUT
-    constexpr int ML = M / 2, MH = M - ML;
-    constexpr int L = 1 << ML, H = 1 << MH, HN = 1 << M;
+struct DxTerm {
+    static constexpr int M  = N - 1;        // variables of the derivative LUT
+    static constexpr int ML = M / 2, MH = M - ML;
+    static constexpr int L = 1 << ML, H = 1 << MH, HN = 1 << M, REC = kTermHead + HN;
 
-    int const B    = a.chunk_count * a.tile_count;
-    int const lid  = xcd_remap(blockIdx.x, B);
-    int const ck   = lid / a.tile_count;
-    int const tile = lid - ck * a.tile_count;
-    int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
-    if (in >= a.input_node_size) { return; }
-    int const lane = threadIdx.x & (kWave - 1);
+    float    Dk[HN];
+    uint32_t raw[U][M];
+    float    dyv[U];
 
-    int const f_begin = ck * a.chunk;
-    int const f_last  = a.frame_size - 1;
-    int fs[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) { fs[u] = min(f_begin + u * kWave + lane, f_last); }
-
-    float acc[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
-
-    int const *__restrict__ r = a.rev + (size_t)in * a.rev_stride;
-    int const cnt = r[0];
-    for (int t = 1; t <= cnt; ++t) {
-        int const e    = r[t];
-        int const node = e / N;
-        float Dk[HN];
-#pragma unroll
-        for (int s = 0; s < HN; ++s) { Dk[s] = a.Dtab[(size_t)e * HN + s]; }
+    // scalar loads of one record, then the vector loads of its U x (M + 1) operands
+    __device__ __forceinline__ void fetch(DxArgs const &a, int const *__restrict__ rec, int const (&fs)[U])
+    {
         void const *rows[M];
 #pragma unroll
         for (int j = 0; j < M; ++j) {
-            int const o = a.Otab[(size_t)e * M + j];
+            int const o = rec[j];
             rows[j] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)o * a.x_stride)
                                        : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)o * a.x_stride);
         }
-        float const *__restrict__ dyr = a.dy + (size_t)node * a.dy_stride;
-
-        uint32_t raw[U][M];
-        float dyv[U];
+        float const *dyr = a.dy + (size_t)rec[M] * a.dy_stride;
+#pragma unroll
+        for (int sidx = 0; sidx < HN; ++sidx) { Dk[sidx] = __int_as_float(rec[kTermHead + sidx]); }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             Gather<M, XMODE>::load_raw(rows, fs[u], raw[u]);
             dyv[u] = *reinterpret_cast<float const *>(reinterpret_cast<char const *>(dyr) + (uint32_t)fs[u] * 4u);
         }
+    }
+
+    __device__ __forceinline__ void accumulate(int const (&fs)[U], float bias, float (&acc)[U]) const
+    {
+        float cv[H];
+#pragma unroll
+        for (int j = 0; j < H; ++j) { asm("v_mov_b32 %0, %1" : "=v"(cv[j]) : "s"(Dk[j * L])); }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float z[M];
-            Gather<M, XMODE>::centre_all(raw[u], fs[u], a.bias, z);
+            Gather<M, XMODE>::centre_all(raw[u], fs[u], bias, z);
             float zl[ML > 0 ? ML : 1], zh[MH];
 #pragma unroll
             for (int k = 0; k < ML; ++k) { zl[k] = z[k]; }
@@ -546,7 +555,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
             float v = 0.0f;
 #pragma unroll
             for (int j = 0; j < H; ++j) {
-                float q = Dk[j * L];
+                float q = cv[j];
 #pragma unroll
                 for (int i = 1; i < L; ++i) { q = __builtin_fmaf(l[i], Dk[j * L + i], q); }
                 v = (j == 0) ? q : __builtin_fmaf(h[j], q, v);
@@ -554,11 +563,44 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
             acc[u] = __builtin_fmaf(dyv[u], v, acc[u]);
         }
     }
+};
+
+template <int N, int XMODE, int U>
+__global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
+{
+    using T = DxTerm<N, XMODE, U>;
+    int const B    = a.chunk_count * a.tile_count;
+    int const lid  = xcd_remap(blockIdx.x, B);
+    int const ck   = lid / a.tile_count;
+    int const tile = lid - ck * a.tile_count;
+    int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
+    if (in >= a.input_node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    int const cnt = a.rev[(size_t)in * a.rev_stride];
+    int const *__restrict__ rec = a.term + (size_t)in * (a.rev_stride - 1) * T::REC;
+    int const f_last = a.frame_size - 1;
+
+    // a unit is a.chunk frames = several passes of 64 * U frames; the node's work list is walked once per pass
+    for (int f_begin = ck * a.chunk; f_begin < min((ck + 1) * a.chunk, a.frame_size); f_begin += kWave * U) {
+        int fs[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { fs[u] = min(f_begin + u * kWave + lane, f_last); }
+        float acc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
+
+        for (int t = 0; t < cnt; ++t) {
+            T tm;
+            tm.fetch(a, rec + (size_t)t * T::REC, fs);
+            tm.accumulate(fs, a.bias, acc);
+        }
 
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        int const f = f_begin + u * kWave + lane;
-        if (f < a.frame_size) { a.dx[(size_t)in * a.dx_stride + f] = acc[u]; }
+        for (int u = 0; u < U; ++u) {
+            int const f = f_begin + u * kWave + lane;
+            if (f < a.frame_size) { a.dx[(size_t)in * a.dx_stride + f] = acc[u]; }
+        }
     }
 }
 

@@ -102,7 +102,7 @@ struct LutEval {
     {
 #pragma unroll
         for (int j = 0; j < D::H; ++j) {
-            asm volatile("v_mov_b32 %0, %1" : "=v"(cv[j]) : "s"(C[j * D::L]));
+            asm("v_mov_b32 %0, %1" : "=v"(cv[j]) : "s"(C[j * D::L]));
         }
     }
 
