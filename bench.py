@@ -72,11 +72,12 @@ def main():
     idx_h = synth.wiring(rng, I, O)
     idx = torch.from_numpy(idx_h).cuda()
     W = torch.from_numpy(synth.lut_tables(rng, O)).cuda()
-    x = torch.from_numpy(synth.uniform_frames(rng, I, F, F)).cuda()
-    dy = torch.from_numpy(synth.normal_frames(rng, O, F, F)).cuda()
+    S = synth.frame_stride_fp32(F)                     # node rows padded off a power-of-two pitch
+    x = torch.from_numpy(synth.uniform_frames(rng, I, F, S)).cuda()
+    dy = torch.from_numpy(synth.normal_frames(rng, O, F, S)).cuda()
     dW = torch.zeros((O, 64), device="cuda")
-    y = torch.empty((O, F), device="cuda")
-    dx = torch.empty((I, F), device="cuda")
+    y = torch.empty((O, S), device="cuda")
+    dx = torch.empty((I, S), device="cuda")
     ops.set_dx_mode(args.dx_mode)
     rev = ops.reverse_table(idx, I) if args.dx_mode != 1 else None
     dx_tmp = None

@@ -821,12 +821,18 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
                                  int node_size, int frame_size, int frame_stride, void *stream)
 {
     BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr && dev_input_index != nullptr && dev_table != nullptr);
-    BBHIP_REQUIRE(node_size > 0 && frame_size > 0);
+    BBHIP_REQUIRE(node_size > 0 && node_size <= (0x7fffffff >> 6) && frame_size > 0);
     BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    char *base = nullptr;
+    if (arena_get(align256((size_t)node_size * 64 * sizeof(uint32_t)), &base)) { return 1; }
+    uint32_t *mask = reinterpret_cast<uint32_t *>(base);
+    hipLaunchKernelGGL(binary_mask_kernel, dim3(ceil_div(node_size * 64, kBlock)), dim3(kBlock), 0, st, dev_table, mask, node_size);
+    BBHIP_LAUNCH_CHECK();
     BinArgs a{};
     a.x = reinterpret_cast<uint32_t const *>(dev_x_buf);
     a.y = reinterpret_cast<uint32_t *>(dev_y_buf);
-    a.idx = dev_input_index; a.table = dev_table;
+    a.idx = dev_input_index; a.mask = mask;
     a.node_size = node_size; a.frame_size = frame_size; a.stride = frame_stride;
     a.word_count = (frame_size + 31) / 32;
     a.chunk = bin_chunk_words();
@@ -834,8 +840,9 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     a.tile_count = ceil_div(node_size, kWavesPerBlk);
     BBHIP_REQUIRE((long long)a.chunk_count * a.tile_count <= 0x7fffffffLL);
     {
-        ScopedTimer tm(kTimeBinary, static_cast<hipStream_t>(stream));
-        hipLaunchKernelGGL(binary_lut6_kernel<1>, dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, static_cast<hipStream_t>(stream), a);
+        ScopedTimer tm(kTimeBinary, st);
+        if (a.chunk % 128 == 0) { hipLaunchKernelGGL(binary_lut6_kernel<2>, dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, st, a); }
+        else                    { hipLaunchKernelGGL(binary_lut6_kernel<1>, dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, st, a); }
     }
     BBHIP_LAUNCH_CHECK();
     return 0;

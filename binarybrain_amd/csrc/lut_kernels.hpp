@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
             else {
                 if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
                 else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
-                if (ok) { reinterpret_cast<float *>(a.y)[(size_t)node * a.y_stride + f] = v; }
+                if (ok) { __builtin_nontemporal_store(v, reinterpret_cast<float *>(a.y) + (size_t)node * a.y_stride + f); }
             }
         }
     }
@@ -599,7 +599,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             int const f = f_begin + u * kWave + lane;
-            if (f < a.frame_size) { a.dx[(size_t)in * a.dx_stride + f] = acc[u]; }
+            if (f < a.frame_size) { __builtin_nontemporal_store(acc[u], a.dx + (size_t)in * a.dx_stride + f); }
         }
     }
 }
@@ -682,14 +682,37 @@ struct BinArgs {
     uint32_t const *x;
     uint32_t       *y;
     int const      *idx;
-    int const      *table;      // [O][2]
+    uint32_t const *mask;       // [O][64]: table bit k expanded to 0 / 0xffffffff (binary_mask_kernel)
     int node_size, frame_size, stride;   // stride in words
     int word_count;             // (frame_size + 31) / 32
     int chunk;                  // words per unit, multiple of 64
     int chunk_count, tile_count;
 };
 
-__device__ __forceinline__ uint32_t bitsel(uint32_t s, uint32_t hi, uint32_t lo) { return (s & hi) | (~s & lo); }
+// table [O][2] (entries 0-31 in word 0) -> mask [O][64]
+__global__ __launch_bounds__(kBlock) void binary_mask_kernel(int const *__restrict__ table, uint32_t *__restrict__ mask, int node_size)
+{
+    int const t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= node_size * 64) { return; }
+    int const node = t >> 6, k = t & 63;
+    uint32_t const w = (uint32_t)table[node * 2 + (k >> 5)];
+    mask[t] = ((w >> (k & 31)) & 1u) ? 0xffffffffu : 0u;
+}
+
+// bit-select d = (s & hi) | (~s & lo): one instruction per multiplexer of the tree
+__device__ __forceinline__ uint32_t bfi_vvv(uint32_t s, uint32_t hi, uint32_t lo)
+{
+    uint32_t d;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "v"(s), "v"(hi), "v"(lo));
+    return d;
+}
+// same with the "hi" operand wave-uniform (scalar register)
+__device__ __forceinline__ uint32_t bfi_vsv(uint32_t s, uint32_t hi, uint32_t lo)
+{
+    uint32_t d;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "v"(s), "s"(hi), "v"(lo));
+    return d;
+}
 
 template <int WPL>   // words per lane per step
 __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
@@ -702,42 +725,49 @@ __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
+    // level-0 multiplexers select between two table entries: entry 2k+1 stays in a scalar register, entry 2k is
+    // copied once per unit into a vector register (an instruction may read one scalar register only)
+    uint32_t const *__restrict__ mg = a.mask + (size_t)node * 64;
+    uint32_t m_hi[32], m_lo[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+        m_hi[k] = mg[2 * k + 1];
+        uint32_t const lo = mg[2 * k];
+        asm("v_mov_b32 %0, %1" : "=v"(m_lo[k]) : "s"(lo));
+    }
+
     uint32_t const *rows[6];
 #pragma unroll
     for (int k = 0; k < 6; ++k) { rows[k] = a.x + (size_t)a.idx[node * 6 + k] * a.stride; }
     uint32_t *yr = a.y + (size_t)node * a.stride;
 
-    uint32_t const t0 = (uint32_t)a.table[node * 2 + 0], t1 = (uint32_t)a.table[node * 2 + 1];
-    uint32_t m[64];
-#pragma unroll
-    for (int k = 0; k < 32; ++k) {
-        m[k]      = ((t0 >> k) & 1u) ? 0xffffffffu : 0u;
-        m[k + 32] = ((t1 >> k) & 1u) ? 0xffffffffu : 0u;
-    }
-
     int const w_begin = ck * a.chunk;
     int const w_end   = min(w_begin + a.chunk, a.word_count);
+    int const w_last  = a.word_count - 1;
     uint32_t const tail_mask = (a.frame_size & 31) ? ((1u << (a.frame_size & 31)) - 1u) : 0xffffffffu;
 
     for (int w0 = w_begin; w0 < w_end; w0 += kWave * WPL) {
+        uint32_t xv[WPL][6];
+#pragma unroll
+        for (int u = 0; u < WPL; ++u) {
+            uint32_t const off = (uint32_t)min(w0 + u * kWave + lane, w_last) * 4u;
+#pragma unroll
+            for (int k = 0; k < 6; ++k) { xv[u][k] = *reinterpret_cast<uint32_t const *>(reinterpret_cast<char const *>(rows[k]) + off); }
+        }
 #pragma unroll
         for (int u = 0; u < WPL; ++u) {
             int const w = w0 + u * kWave + lane;
-            bool const ok = w < w_end;
-            uint32_t xv[6];
-#pragma unroll
-            for (int k = 0; k < 6; ++k) { xv[k] = ok ? rows[k][w] : 0u; }
             uint32_t t[32];
 #pragma unroll
-            for (int k = 0; k < 32; ++k) { t[k] = bitsel(xv[0], m[2 * k + 1], m[2 * k]); }
+            for (int k = 0; k < 32; ++k) { t[k] = bfi_vsv(xv[u][0], m_hi[k], m_lo[k]); }
 #pragma unroll
             for (int lv = 1; lv < 6; ++lv) {
 #pragma unroll
-                for (int k = 0; k < (32 >> lv); ++k) { t[k] = bitsel(xv[lv], t[2 * k + 1], t[2 * k]); }
+                for (int k = 0; k < (32 >> lv); ++k) { t[k] = bfi_vvv(xv[u][lv], t[2 * k + 1], t[2 * k]); }
             }
             uint32_t r = t[0];
-            if (w == a.word_count - 1) { r &= tail_mask; }
-            if (ok) { yr[w] = r; }
+            if (w == w_last) { r &= tail_mask; }
+            if (w < w_end) { __builtin_nontemporal_store(r, yr + w); }     // streamed once: keep it from displacing x rows in L2
         }
     }
 }

@@ -11,13 +11,21 @@ WAVE = 64
 
 
 def frame_stride_fp32(frames, multiple=WAVE):
-    """Row length (floats) of an fp32 frame buffer: frames rounded up to a wavefront multiple."""
-    return ((frames + multiple - 1) // multiple) * multiple
+    """Row length (floats) of an fp32 frame buffer: frames rounded up to a wavefront multiple; rows whose byte length
+    would be a multiple of 2 KiB get 128 more floats, because node rows that are a power of two apart fall into
+    the same few L2 sets and the gathered rows then evict each other."""
+    s = ((frames + multiple - 1) // multiple) * multiple
+    if (s * 4) % 2048 == 0:
+        s += 128
+    return s
 
 
 def frame_stride_bit(frames, multiple_bits=WAVE * 32):
-    """Row length (32-bit words) of a bit-packed frame buffer: rounded so that a wavefront reads whole words."""
-    return ((frames + multiple_bits - 1) // multiple_bits) * (multiple_bits // 32)
+    """Row length (32-bit words) of a bit-packed frame buffer: whole words for a wavefront, same de-aliasing pad."""
+    s = ((frames + multiple_bits - 1) // multiple_bits) * (multiple_bits // 32)
+    if (s * 4) % 2048 == 0:
+        s += 96
+    return s
 
 
 def wiring(rng, input_nodes, output_nodes, n=6):
