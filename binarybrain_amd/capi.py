@@ -21,6 +21,13 @@ _SIGNATURES = {
     "bbhip_LocalHeap_GetMaxAllocSize": (C.c_size_t, []),
     "bbhip_LocalHeap_GetAllocatedSize": (C.c_size_t, []),
     "bbhip_LocalHeap_GarbageCollect": (None, []),
+    "bbhip_Malloc": (C.c_int, [C.POINTER(C.c_void_p), C.c_size_t]),
+    "bbhip_Free": (C.c_int, [_vp]),
+    "bbhip_MallocHost": (C.c_int, [C.POINTER(C.c_void_p), C.c_size_t]),
+    "bbhip_FreeHost": (C.c_int, [_vp]),
+    "bbhip_Memcpy": (C.c_int, [_vp, _vp, C.c_size_t, _i]),
+    "bbhip_Memset": (C.c_int, [_vp, _i, C.c_size_t]),
+    "bbhip_DeviceSynchronize": (C.c_int, []),
     "bbhip_KernelTimer_Enable": (None, [_i]),
     "bbhip_KernelTimer_Read": (C.c_int, [_i, C.POINTER(C.c_float), C.POINTER(C.c_int)]),
     "bbhip_SetDxMode": (None, [_i]),

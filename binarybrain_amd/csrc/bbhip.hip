@@ -568,6 +568,53 @@ size_t bbhip_LocalHeap_GetMaxAllocSize(void) { return heap().max_alloc; }
 size_t bbhip_LocalHeap_GetAllocatedSize(void) { return heap().allocated; }
 void   bbhip_LocalHeap_GarbageCollect(void) { std::lock_guard<std::mutex> lk(heap().mtx); heap().collect_locked(); }
 
+int bbhip_Malloc(void **ptr, size_t size)
+{
+    BBHIP_REQUIRE(ptr != nullptr);
+    *ptr = heap().alloc(size);
+    if (!*ptr) { return fail("bbhip_Malloc: out of device memory (%zu bytes)", size); }
+    return 0;
+}
+
+int bbhip_Free(void *ptr) { heap().release(ptr); return 0; }
+
+int bbhip_MallocHost(void **ptr, size_t size)
+{
+    BBHIP_REQUIRE(ptr != nullptr);
+    BBHIP_TRY(hipHostMalloc(ptr, size ? size : 1, hipHostMallocDefault));
+    return 0;
+}
+
+int bbhip_FreeHost(void *ptr)
+{
+    if (ptr) { BBHIP_TRY(hipHostFree(ptr)); }
+    return 0;
+}
+
+int bbhip_Memcpy(void *dst, void const *src, size_t size, int kind)
+{
+    BBHIP_REQUIRE(kind >= 1 && kind <= 3);
+    if (size == 0) { return 0; }
+    BBHIP_REQUIRE(dst != nullptr && src != nullptr);
+    hipMemcpyKind const k = (kind == 1) ? hipMemcpyHostToDevice : (kind == 2) ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+    BBHIP_TRY(hipMemcpy(dst, src, size, k));
+    return 0;
+}
+
+int bbhip_Memset(void *dev_ptr, int value, size_t size)
+{
+    if (size == 0) { return 0; }
+    BBHIP_REQUIRE(dev_ptr != nullptr);
+    BBHIP_TRY(hipMemset(dev_ptr, value, size));
+    return 0;
+}
+
+int bbhip_DeviceSynchronize(void)
+{
+    BBHIP_TRY(hipDeviceSynchronize());
+    return 0;
+}
+
 void bbhip_KernelTimer_Enable(int enable) { g_timer_on = enable != 0; }
 
 int bbhip_KernelTimer_Read(int which, float *total_ms, int *launches)

@@ -1,0 +1,315 @@
+// DifferentiableLutN<N, BinType, RealType>: the N-input differentiable LUT fused with per-node batch normalisation
+// (scalar gamma / beta) and a binarize or hard-tanh output stage, with the reference's model API
+// (include/bb/DifferentiableLutN.h:35-1398: create_t, Create, SetInputShape, Forward(train), Backward, commands
+// binary / lut_binarize / batch_norm / momentum / backward_break / host_only / parameter_lock, running statistics).
+// Numerical semantics are those of the reference's CPU path (:754-1008 forward, :1157-1396 backward): training
+// statistics mean / max(1e-5, var) / rstd, running = running*m + stat*(1-m), inference rstd = 1/sqrt(running_var),
+// hard-tanh window on dy in both binary and non-binary mode.  Frame work runs in the HIP library only.
+#pragma once
+
+#include <random>
+
+#include "bb/Model.h"
+#include "bb/FixedSizeConnectionTable.h"
+
+namespace bb {
+
+template <int N = 6, typename BinType = float, typename RealType = float>
+class DifferentiableLutN : public Model {
+    static_assert(std::is_same<RealType, float>::value, "fp32 tables only");
+    static constexpr int NN = 1 << N;
+    static constexpr bool kBitType = std::is_same<BinType, Bit>::value;
+
+protected:
+    bool        m_host_only = false;
+    bool        m_lut_binarize = false;
+    bool        m_binary_mode = true;
+    bool        m_batch_norm = true;
+    bool        m_backward_break = false;
+    bool        m_flagClamp = false;            // W is clamped lazily, once after each backward (reference :605-608, :1022)
+    RealType    m_unbinarize_bias = (RealType)0.25;
+    index_t     m_max_tmp_mem_size = 256 * 1024 * 1024;
+    std::string m_connection;
+    indices_t   m_input_shape, m_output_shape;
+    FixedSizeConnectionTable<N> m_connection_table;
+    std::shared_ptr<Tensor> m_W, m_dW;
+    RealType    m_momentum, m_gamma, m_beta;
+    Tensor_<RealType> m_mean, m_rstd, m_running_mean, m_running_var;
+    std::mt19937_64 m_mt;
+
+    void CommandProc(std::vector<std::string> args) override
+    {
+        Model::CommandProc(args);
+        if (!kBitType && args.size() == 2 && args[0] == "binary") { m_binary_mode = EvalBool(args[1]); }
+        if (args.size() == 2 && args[0] == "lut_binarize")   { m_lut_binarize = EvalBool(args[1]); }
+        if (args.size() == 2 && args[0] == "host_only")      { m_host_only = EvalBool(args[1]); }
+        if (args.size() == 2 && args[0] == "batch_norm")     { m_batch_norm = EvalBool(args[1]); }
+        if (args.size() == 2 && args[0] == "momentum")       { m_momentum = (RealType)std::stod(args[1]); }
+        if (args.size() == 2 && args[0] == "backward_break") { m_backward_break = EvalBool(args[1]); }
+    }
+
+    void RequireDevice(char const *what) const
+    {
+        if (m_host_only || !Manager::IsDeviceAvailable()) {
+            throw Exception(std::string(what) + ": host-only execution is not provided by this library (device path only)");
+        }
+    }
+
+public:
+    struct create_t {
+        indices_t     output_shape;
+        bool          batch_norm = true;
+        bool          binary = true;
+        std::string   connection;
+        RealType      momentum = (RealType)0.9;
+        RealType      gamma = (RealType)0.3;
+        RealType      beta = (RealType)0.5;
+        std::uint64_t seed = 1;
+    };
+
+protected:
+    explicit DifferentiableLutN(create_t const &create)
+    {
+        m_output_shape = create.output_shape;
+        m_connection = create.connection;
+        m_batch_norm = create.batch_norm;
+        m_binary_mode = create.binary || kBitType;
+        m_momentum = create.momentum;
+        m_gamma = create.gamma;
+        m_beta = create.beta;
+        m_mt.seed(create.seed);
+        m_W = std::make_shared<Tensor>();
+        m_dW = std::make_shared<Tensor>();
+    }
+
+public:
+    static std::string ModelName(void) { return "DifferentiableLut" + std::to_string(N); }
+    std::string GetModelName(void) const override { return ModelName(); }
+
+    static std::shared_ptr<DifferentiableLutN> Create(create_t const &create) { return std::shared_ptr<DifferentiableLutN>(new DifferentiableLutN(create)); }
+    static std::shared_ptr<DifferentiableLutN> Create(indices_t const &output_shape, bool batch_norm = true, std::string connection = "")
+    {
+        create_t c; c.output_shape = output_shape; c.batch_norm = batch_norm; c.connection = connection;
+        return Create(c);
+    }
+    static std::shared_ptr<DifferentiableLutN> Create(index_t output_node_size, bool batch_norm = true, std::string connection = "")
+    {
+        return Create(indices_t({output_node_size}), batch_norm, connection);
+    }
+
+    Tensor &W(void)  { return *m_W; }
+    Tensor &dW(void) { return *m_dW; }
+    auto lock_W(void)              { return m_W->Lock<RealType>(); }
+    auto lock_W_const(void) const  { return m_W->LockConst<RealType>(); }
+    auto lock_dW(void)             { return m_dW->Lock<RealType>(); }
+    auto lock_dW_const(void) const { return m_dW->LockConst<RealType>(); }
+    auto lock_mean(void)                  { return m_running_mean.Lock(); }
+    auto lock_mean_const(void) const      { return m_running_mean.LockConst(); }
+    auto lock_var(void)                   { return m_running_var.Lock(); }
+    auto lock_var_const(void) const       { return m_running_var.LockConst(); }
+    auto lock_tmp_mean_const(void) const  { return m_mean.LockConst(); }
+    auto lock_tmp_rstd_const(void) const  { return m_rstd.LockConst(); }
+    double GetGamma(void) const { return (double)m_gamma; }
+    double GetBeta(void) const  { return (double)m_beta; }
+
+    index_t GetNodeConnectionSize(index_t) const { return N; }
+    void    SetNodeConnectionIndex(index_t node, index_t input_index, index_t input_node) { m_connection_table.SetInputConnection(node, input_index, input_node); }
+    index_t GetNodeConnectionIndex(index_t node, index_t input_index) const { return m_connection_table.GetInputConnection(node, input_index); }
+
+    indices_t SetInputShape(indices_t shape) override
+    {
+        if (shape == m_input_shape) { return m_output_shape; }
+        m_input_shape = shape;
+        m_connection_table.SetShape(m_input_shape, m_output_shape);
+        m_connection_table.InitializeConnection(m_mt(), m_connection);
+        m_W->Resize({this->GetOutputNodeSize(), (index_t)NN}, DataType<RealType>::type);
+        m_W->InitNormalDistribution(0.5, 0.01, m_mt());
+        m_dW->Resize({this->GetOutputNodeSize(), (index_t)NN}, DataType<RealType>::type);
+        m_dW->FillZero();
+        m_mean.Resize(m_output_shape);
+        m_rstd.Resize(m_output_shape);
+        m_running_mean.Resize(m_output_shape); m_running_mean = (RealType)0.0;
+        m_running_var.Resize(m_output_shape);  m_running_var = (RealType)1.0;
+        return m_output_shape;
+    }
+    indices_t GetInputShape(void) const override  { return m_input_shape; }
+    indices_t GetOutputShape(void) const override { return m_output_shape; }
+
+    Variables GetParameters(void) override { Variables v; if (!m_parameter_lock) { v.PushBack(m_W); }  return v; }
+    Variables GetGradients(void) override  { Variables v; if (!m_parameter_lock) { v.PushBack(m_dW); } return v; }
+
+    // one node on the host with the running statistics (reference: DifferentiableLutN.h:527-586)
+    std::vector<double> ForwardNode(index_t node, std::vector<double> input_value) const override
+    {
+        BB_ASSERT((int)input_value.size() == N);
+        auto Wp = lock_W_const();
+        RealType x[N];
+        for (int i = 0; i < N; ++i) {
+            RealType v = (RealType)input_value[(std::size_t)i];
+            x[i] = m_binary_mode ? ((RealType)0.5 + ((v > (RealType)0.5) ? +m_unbinarize_bias : -m_unbinarize_bias))
+                                 : std::min((RealType)1, std::max((RealType)0, v));
+        }
+        RealType y = 0;
+        for (int i = 0; i < NN; ++i) {
+            RealType w = Wp(node, i);
+            if (m_flagClamp) { w = std::min((RealType)1, std::max((RealType)0, w)); }
+            if (m_lut_binarize) { w = (w > (RealType)0.5) ? (RealType)1 : (RealType)0; }
+            for (int j = 0; j < N; ++j) { w *= ((i >> j) & 1) ? x[j] : ((RealType)1 - x[j]); }
+            y += w;
+        }
+        if (m_batch_norm) {
+            RealType const mean = lock_mean_const()[node];
+            RealType const rstd = (RealType)1 / std::sqrt(lock_var_const()[node]);
+            y = (y - mean) * rstd;
+            y = y * m_gamma + m_beta;
+        }
+        y = m_binary_mode ? ((y > (RealType)0.5) ? (RealType)1 : (RealType)0) : std::max((RealType)0, std::min((RealType)1, y));
+        return std::vector<double>(1, (double)y);
+    }
+
+    FrameBuffer Forward(FrameBuffer x_buf, bool train = true) override
+    {
+        RequireDevice("DifferentiableLutN::Forward");
+        if (x_buf.GetShape() != m_input_shape) { SetInputShape(x_buf.GetShape()); }
+        FrameBuffer y_buf(x_buf.GetFrameSize(), m_output_shape, DataType<BinType>::type);
+        if (train) { this->PushFrameBuffer(x_buf); }
+        if (m_flagClamp) { m_W->Clamp_inplace(0.0f, 1.0f); m_flagClamp = false; }
+        if (!kBitType && x_buf.GetType() == BB_TYPE_BIT) { x_buf = x_buf.ConvertBitToFP32(); }      // reference :610-613
+        BB_ASSERT(x_buf.GetType() == DataType<BinType>::type);
+
+        int const O = (int)y_buf.GetNodeSize(), F = (int)y_buf.GetFrameSize();
+        int const y_stride = (int)(y_buf.GetFrameStride() / 4), x_stride = (int)(x_buf.GetFrameStride() / 4);
+        if (!kBitType) { BB_ASSERT(x_stride == y_stride); }
+        auto x_ptr   = x_buf.LockDeviceMemoryConst();
+        auto y_ptr   = y_buf.LockDeviceMemory(true);
+        auto idx_ptr = m_connection_table.LockDeviceMemConst_InputTable();
+        auto W_ptr   = m_W->LockDeviceMemoryConst();
+
+        if (m_batch_norm && train) {
+            auto mean_ptr = m_mean.LockDeviceMemory(true);
+            auto rstd_ptr = m_rstd.LockDeviceMemory(true);
+            auto rm_ptr   = m_running_mean.LockDeviceMemory();
+            auto rv_ptr   = m_running_var.LockDeviceMemory();
+            if (kBitType) {
+                CheckDevice(bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(),
+                                (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
+                                (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
+                                O, F, y_stride, m_lut_binarize ? 1 : 0, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTraining");
+            }
+            else {
+                CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTraining(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
+                                (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
+                                (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
+                                O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_ForwardTraining");
+            }
+        }
+        else if (m_batch_norm) {
+            auto rm_ptr = m_running_mean.LockDeviceMemoryConst();
+            auto rv_ptr = m_running_var.LockDeviceMemoryConst();
+            if (kBitType) {
+                CheckDevice(bbhip_bit_fp32_DifferentiableLutN_ForwardInference(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(),
+                                (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float const *)rm_ptr.GetAddr(), (float const *)rv_ptr.GetAddr(),
+                                m_gamma, m_beta, m_unbinarize_bias, O, F, y_stride, m_lut_binarize ? 1 : 0, nullptr),
+                            "bbhip_bit_fp32_DifferentiableLutN_ForwardInference");
+            }
+            else {
+                CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardInference(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
+                                (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float const *)rm_ptr.GetAddr(), (float const *)rv_ptr.GetAddr(),
+                                m_gamma, m_beta, m_unbinarize_bias, O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr),
+                            "bbhip_fp32_DifferentiableLutN_ForwardInference");
+            }
+        }
+        else if (kBitType) {
+            CheckDevice(bbhip_bit_bit_fp32_StochasticLut_Forward(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(),
+                            (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), O, F, y_stride,
+                            m_lut_binarize ? 1 : 0, m_unbinarize_bias, nullptr), "bbhip_bit_bit_fp32_StochasticLut_Forward");
+        }
+        else {
+            CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardNoBn(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
+                            (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), m_unbinarize_bias, O, F, y_stride,
+                            m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_ForwardNoBn");
+        }
+        return y_buf;
+    }
+
+    FrameBuffer Backward(FrameBuffer dy_buf) override
+    {
+        if (m_backward_break || dy_buf.Empty()) { return FrameBuffer(); }
+        BB_ASSERT(dy_buf.GetType() == DataType<RealType>::type);
+        RequireDevice("DifferentiableLutN::Backward");
+        m_flagClamp = true;
+        FrameBuffer x_buf = this->PopFrameBuffer();
+        if (!kBitType && x_buf.GetType() == BB_TYPE_BIT) { x_buf = x_buf.ConvertBitToFP32(); }
+        BB_ASSERT(x_buf.GetType() == DataType<BinType>::type && x_buf.GetFrameSize() == dy_buf.GetFrameSize());
+        FrameBuffer dx_buf(dy_buf.GetFrameSize(), m_input_shape, DataType<RealType>::type);
+
+        FrameBuffer tmp_buf;
+        index_t tmp_frame_size = 0;
+        if (bbhip_GetDxMode() == 2) {
+            tmp_frame_size = m_max_tmp_mem_size / (index_t)(sizeof(float) * (std::size_t)this->GetOutputNodeSize() * N);
+            tmp_frame_size = std::max(tmp_frame_size, (index_t)32);
+            tmp_frame_size = (tmp_frame_size + 31) & ~(index_t)0x1f;
+            tmp_frame_size = std::min(tmp_frame_size, dy_buf.GetFrameSize());
+            tmp_buf.Resize(tmp_frame_size, {this->GetOutputNodeSize() * N}, DataType<RealType>::type);
+        }
+        float *tmp_addr = nullptr;
+        std::unique_ptr<DevicePtr> tmp_ptr;
+        if (!tmp_buf.Empty()) { tmp_ptr.reset(new DevicePtr(tmp_buf.LockDeviceMemory(true))); tmp_addr = (float *)tmp_ptr->GetAddr(); }
+
+        int const I = (int)dx_buf.GetNodeSize(), O = (int)dy_buf.GetNodeSize(), F = (int)dy_buf.GetFrameSize();
+        int const stride = (int)(dx_buf.GetFrameStride() / 4), x_stride = (int)(x_buf.GetFrameStride() / 4);
+        int const tmp_stride = (int)(tmp_buf.GetFrameStride() / 4);
+        auto x_ptr   = x_buf.LockDeviceMemoryConst();
+        auto dy_ptr  = dy_buf.LockDeviceMemoryConst();
+        auto dx_ptr  = dx_buf.LockDeviceMemory(true);
+        auto rev_ptr = m_connection_table.LockDeviceMemConst_ReverseTable();
+        auto idx_ptr = m_connection_table.LockDeviceMemConst_InputTable();
+        auto W_ptr   = m_W->LockDeviceMemoryConst();
+        auto dW_ptr  = m_dW->LockDeviceMemory();
+        int const rev_stride = (int)m_connection_table.GetReverseTableStride();
+
+        if (m_batch_norm) {
+            // with a locked parameter set the statistics of inference are used (reference :1048-1051)
+            Tensor_<RealType> mean(m_output_shape), rstd(m_output_shape);
+            if (m_parameter_lock) {
+                auto rm = m_running_mean.LockConst(); auto rv = m_running_var.LockConst();
+                auto mp = mean.Lock(true); auto rp = rstd.Lock(true);
+                for (index_t n = 0; n < O; ++n) { mp[n] = rm[n]; rp[n] = (RealType)1 / std::sqrt(rv[n] + (RealType)1.0e-7); }
+            }
+            auto mean_ptr = m_parameter_lock ? mean.LockDeviceMemoryConst() : m_mean.LockDeviceMemoryConst();
+            auto rstd_ptr = m_parameter_lock ? rstd.LockDeviceMemoryConst() : m_rstd.LockDeviceMemoryConst();
+            Tensor_<RealType> dmean(m_output_shape), dvar(m_output_shape);
+            auto dmean_ptr = dmean.LockDeviceMemory(true);
+            auto dvar_ptr  = dvar.LockDeviceMemory(true);
+            if (kBitType) {
+                CheckDevice(bbhip_bit_fp32_DifferentiableLutN_Backward(N, (int const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
+                                tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),
+                                (float const *)mean_ptr.GetAddr(), (float const *)rstd_ptr.GetAddr(), (float *)dmean_ptr.GetAddr(), (float *)dvar_ptr.GetAddr(),
+                                m_gamma, m_beta, m_unbinarize_bias, rev_stride, I, O, F, stride, x_stride, (int)tmp_frame_size, tmp_stride,
+                                m_lut_binarize ? 1 : 0, nullptr), "bbhip_bit_fp32_DifferentiableLutN_Backward");
+            }
+            else {
+                CheckDevice(bbhip_fp32_DifferentiableLutN_Backward(N, (float const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
+                                tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),
+                                (float const *)mean_ptr.GetAddr(), (float const *)rstd_ptr.GetAddr(), (float *)dmean_ptr.GetAddr(), (float *)dvar_ptr.GetAddr(),
+                                m_gamma, m_beta, m_unbinarize_bias, rev_stride, I, O, F, stride, (int)tmp_frame_size, tmp_stride,
+                                m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_Backward");
+            }
+        }
+        else if (kBitType) {
+            CheckDevice(bbhip_bit_fp32_StochasticLut_Backward(N, (int const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
+                            tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),
+                            rev_stride, I, O, F, stride, x_stride, (int)tmp_frame_size, tmp_stride, m_lut_binarize ? 1 : 0, m_unbinarize_bias, nullptr),
+                        "bbhip_bit_fp32_StochasticLut_Backward");
+        }
+        else {
+            CheckDevice(bbhip_fp32_StochasticLut_Backward(N, (float const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
+                            tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),
+                            rev_stride, I, O, F, stride, (int)tmp_frame_size, tmp_stride, m_binary_mode ? 1 : 0, m_lut_binarize ? 1 : 0,
+                            m_unbinarize_bias, nullptr), "bbhip_fp32_StochasticLut_Backward");
+        }
+        return dx_buf;
+    }
+};
+
+}  // namespace bb

@@ -46,6 +46,18 @@ size_t bbhip_LocalHeap_GetMaxAllocSize(void);
 size_t bbhip_LocalHeap_GetAllocatedSize(void);
 void   bbhip_LocalHeap_GarbageCollect(void);
 
+/* ---- raw device / pinned-host memory and copies (reference: bbcu::Malloc/Free/MallocHost/FreeHost/Memcpy,
+ * include/bbcu/bbcu_util.h:89-134; Malloc/Free go through the caching allocator above) ----
+ * kind: 1 = host to device, 2 = device to host, 3 = device to device.  Copies and Memset are synchronous with respect
+ * to the host and ordered after work queued on the default stream. */
+int bbhip_Malloc(void **ptr, size_t size);
+int bbhip_Free(void *ptr);
+int bbhip_MallocHost(void **ptr, size_t size);
+int bbhip_FreeHost(void *ptr);
+int bbhip_Memcpy(void *dst, void const *src, size_t size, int kind);
+int bbhip_Memset(void *dev_ptr, int value, size_t size);
+int bbhip_DeviceSynchronize(void);
+
 /* ---- how dx is accumulated over the fan-out of an input node (no counterpart in the reference) ----
  * 0 (default): deterministic, no scratch — one wavefront per (input node, frame chunk) walks reverse_index in the
  *              reference's order (cuda/Common.cuh:174-202, include/bb/FixedSizeConnectionTable.h:198-214) and

@@ -1,0 +1,137 @@
+// CPU test of the host-side plumbing (no device needed): frame-buffer layout and bit packing, tensors, the connection
+// table and its reverse table against the oracle, command handling, and the refusal to run without a device.
+#include <cstdio>
+#include <map>
+#include <set>
+#include <vector>
+
+#include "bb/StochasticLutN.h"
+#include "bb/DifferentiableLutN.h"
+#include "bb/BinaryLutN.h"
+
+extern "C" int oracle_ReverseTable(int n, std::int32_t const *idx, int input_node_size, int output_node_size, std::int32_t *rev, int rev_cap);
+
+static int g_fail = 0;
+#define CHECK(cond) do { if (!(cond)) { ++g_fail; std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond); } } while (0)
+
+int main(void)
+{
+    bb::Manager::SetHostOnly(true);
+    CHECK(!bb::Manager::IsDeviceAvailable());
+
+    // frame buffer: node-major rows, stride a 256-byte multiple and never a 2 KiB multiple
+    {
+        bb::FrameBuffer buf(100, {3, 5}, BB_TYPE_FP32, true);
+        CHECK(buf.GetNodeSize() == 15 && buf.GetFrameSize() == 100 && buf.GetFrameStride() == 512);
+        CHECK(bb::FrameBuffer::CalcFrameStride(BB_TYPE_FP32, 8192) == 32768 + 512);
+        CHECK(bb::FrameBuffer::CalcFrameStride(BB_TYPE_BIT, 262144) == 32768 + 384);
+        CHECK(bb::FrameBuffer::CalcFrameStride(BB_TYPE_BIT, 1) == 256);
+        buf.SetFP32(99, 14, 3.5f);
+        buf.SetFP32(0, 0, -1.0f);
+        CHECK(buf.GetFP32(99, 14) == 3.5f && buf.GetFP32(0, 0) == -1.0f);
+        auto p = buf.LockConst<float>();
+        CHECK(p.GetAddr(14)[99] == 3.5f);
+        CHECK((char const *)p.GetAddr(1) - (char const *)p.GetAddr(0) == 512);
+        bb::FrameBuffer alias = buf;                       // copies share storage, as in the reference
+        alias.SetFP32(1, 1, 7.0f);
+        CHECK(buf.GetFP32(1, 1) == 7.0f);
+    }
+    // packed bits: frame f is bit f & 7 of byte f >> 3 (bit f & 31 of little-endian word f >> 5)
+    {
+        bb::FrameBuffer buf(70, {4}, BB_TYPE_BIT, true);
+        buf.FillZero();
+        buf.SetBit(0, 2, true); buf.SetBit(33, 2, true); buf.SetBit(69, 2, true);
+        auto p = buf.LockConst<bb::Bit>();
+        std::uint32_t const *w = reinterpret_cast<std::uint32_t const *>(p.GetAddr(2));
+        CHECK(w[0] == 1u && w[1] == 2u && w[2] == (1u << 5));
+        CHECK(buf.GetBit(33, 2) && !buf.GetBit(34, 2) && !buf.GetBit(33, 1));
+        buf.SetBit(33, 2, false);
+        CHECK(!buf.GetBit(33, 2));
+        bool threw = false;
+        try { buf.Lock<float>(); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);                                      // typed access checks the element type
+    }
+    // tensors
+    {
+        bb::Tensor_<float> t(bb::indices_t({4, 8}), true);
+        t = 0.25f;
+        auto p = t.Lock();
+        p(3, 7) = 1.0f;
+        CHECK(p[31] == 1.0f && p(0, 0) == 0.25f && t.GetSize() == 32);
+        bb::Tensor w({16, 64}, BB_TYPE_FP32, true);
+        w.InitNormalDistribution(0.5, 0.01, 1);
+        double s = 0; { auto q = w.LockConst<float>(); for (int i = 0; i < 1024; ++i) { s += q[i]; } }
+        CHECK(std::abs(s / 1024 - 0.5) < 0.01);
+    }
+    // connection table: distinct inputs per node, balanced use of inputs, reverse table equal to the oracle's
+    for (std::string policy : {"", "random", "serial"}) {
+        int const I = 50, O = 37;
+        bb::FixedSizeConnectionTable<6> tbl;
+        tbl.SetShape({I}, {O});
+        tbl.InitializeConnection(3, policy);
+        std::vector<std::int32_t> idx((size_t)O * 6);
+        std::map<int, int> use;
+        for (int o = 0; o < O; ++o) {
+            std::set<int> seen;
+            for (int i = 0; i < 6; ++i) { int v = (int)tbl.GetInputConnection(o, i); CHECK(v >= 0 && v < I); seen.insert(v); use[v]++; idx[(size_t)o * 6 + i] = v; }
+            CHECK(seen.size() == 6);
+        }
+        int lo = 1 << 30, hi = 0;
+        for (int v = 0; v < I; ++v) { lo = std::min(lo, use[v]); hi = std::max(hi, use[v]); }
+        CHECK(hi - lo <= 2);                               // every input used about equally often
+        int const stride = oracle_ReverseTable(6, idx.data(), I, O, nullptr, 0);
+        std::vector<std::int32_t> rev((size_t)I * stride);
+        oracle_ReverseTable(6, idx.data(), I, O, rev.data(), (int)rev.size());
+        CHECK(tbl.GetReverseTableStride() == stride);
+        auto p = tbl.LockConst_ReverseTable();
+        bool same = true;
+        for (int r = 0; r < I; ++r) for (int c = 0; c < stride; ++c) { same = same && (p(r, c) == rev[(size_t)r * stride + c]); }
+        CHECK(same);
+        tbl.SetInputConnection(0, 0, (tbl.GetInputConnection(0, 0) + 1) % I);     // editing the wiring rebuilds the reverse table
+        idx[0] = (std::int32_t)tbl.GetInputConnection(0, 0);
+        int const stride2 = oracle_ReverseTable(6, idx.data(), I, O, nullptr, 0);
+        std::vector<std::int32_t> rev2((size_t)I * stride2);
+        oracle_ReverseTable(6, idx.data(), I, O, rev2.data(), (int)rev2.size());
+        auto p2 = tbl.LockConst_ReverseTable();
+        same = (tbl.GetReverseTableStride() == stride2);
+        for (int r = 0; same && r < I; ++r) for (int c = 0; c < stride2; ++c) { same = same && (p2(r, c) == rev2[(size_t)r * stride2 + c]); }
+        CHECK(same);
+    }
+    // models: shapes, parameters, commands, ForwardNode, and no silent host execution
+    {
+        auto lut = bb::StochasticLutN<6, float>::Create(10);
+        CHECK(lut->GetModelName() == "StochasticLut6");
+        CHECK(lut->SetInputShape({4, 5}) == bb::indices_t({10}));
+        CHECK(lut->GetInputNodeSize() == 20 && lut->GetOutputNodeSize() == 10);
+        CHECK(lut->GetParameters().GetSize() == 1 && lut->GetGradients().GetSize() == 1);
+        CHECK(lut->W().GetShape() == bb::indices_t({10, 64}));
+        { auto W = lut->lock_W(); for (int i = 0; i < 64; ++i) { W(3, i) = (i == 37) ? 0.9f : 0.1f; } }
+        std::vector<double> in(6);
+        for (int b = 0; b < 6; ++b) { in[(size_t)b] = (37 >> b) & 1; }
+        CHECK(lut->ForwardNode(3, in)[0] == 1.0);                                // lut_binarize is on by default
+        lut->SendCommand("lut_binarize false");
+        CHECK(std::abs(lut->ForwardNode(3, in)[0] - 0.9) < 1e-6);
+        in[0] = 1.0 - in[0];
+        CHECK(std::abs(lut->ForwardNode(3, in)[0] - 0.1) < 1e-6);
+        bool threw = false;
+        try { lut->Forward(bb::FrameBuffer(8, {4, 5}, BB_TYPE_FP32, true)); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);
+        auto dl = bb::DifferentiableLutN<6, bb::Bit>::Create(12);
+        CHECK(dl->GetModelName() == "DifferentiableLut6");
+        dl->SetInputShape({30});
+        CHECK(dl->GetParameters().GetSize() == 1);
+        dl->SendCommand("parameter_lock true");
+        CHECK(dl->GetParameters().GetSize() == 0);
+        { auto v = dl->lock_var_const(); auto m = dl->lock_mean_const(); CHECK(v[0] == 1.0f && m[11] == 0.0f); }
+        auto bl = bb::BinaryLutN<6, bb::Bit>::Create(5);
+        bl->SetInputShape({9});
+        bl->SetLutTable(2, 40, true);  CHECK(bl->GetLutTable(2, 40));
+        bl->SetLutTable(2, 40, false); CHECK(!bl->GetLutTable(2, 40));
+        std::set<bb::index_t> seen;
+        for (int i = 0; i < 6; ++i) { seen.insert(bl->GetNodeConnectionIndex(4, i)); }
+        CHECK(seen.size() == 6);
+        CHECK(bl->Backward(bb::FrameBuffer(8, {5}, BB_TYPE_FP32, true)).GetNodeSize() == 9);
+    }
+    std::printf("%s (%d failed checks)\n", g_fail ? "FAILED" : "OK", g_fail);
+    return g_fail ? 1 : 0;
+}

@@ -1,0 +1,220 @@
+// GPU test of the C++ model classes (bb::StochasticLutN, bb::DifferentiableLutN, bb::BinaryLutN) in the shape of the
+// reference's own parity test (tests/gtest/StochasticLutNTest.cpp:15-246): random wiring/table/input injected into the
+// model, Forward/Backward on the device, results compared with the CPU oracle (oracle/bb_oracle.c, linked as the
+// checker only).  Exit status 0 = all checks passed.
+#include <cmath>
+#include <cstdio>
+#include <random>
+#include <vector>
+
+#include "bb/StochasticLutN.h"
+#include "bb/DifferentiableLutN.h"
+#include "bb/BinaryLutN.h"
+
+extern "C" {
+void oracle_fp32_StochasticLut_Forward(int n, float const *x, float *y, std::int32_t const *idx, float const *W, int node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
+void oracle_fp32_StochasticLut_Backward(int n, float const *x, float const *dy, float *dx, std::int32_t const *idx, float const *W, float *dW, int input_node_size, int output_node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
+void oracle_fp32_DifferentiableLutN_ForwardTraining(int n, float const *x, float *y, std::int32_t const *idx, float const *W, float *mean, float *rstd, float *running_mean, float *running_var, float gamma, float beta, float momentum, float bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode);
+void oracle_fp32_DifferentiableLutN_Backward(int n, float const *x, float const *dy, float *dx, std::int32_t const *idx, float const *W, float *dW, float const *mean, float const *rstd, float gamma, float beta, float bias, int input_node_size, int output_node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode);
+void oracle_bit_BinaryLut6_Forward(std::int32_t const *x, std::int32_t *y, std::int32_t const *idx, std::int32_t const *table, int node_size, int frame_size, int frame_stride);
+}
+
+static int g_fail = 0;
+#define CHECK(cond, ...) do { if (!(cond)) { ++g_fail; std::printf("FAIL %s:%d: ", __FILE__, __LINE__); std::printf(__VA_ARGS__); std::printf("\n"); } } while (0)
+
+static double max_abs(std::vector<float> const &a) { double m = 0; for (float v : a) { m = std::max(m, (double)std::fabs(v)); } return m; }
+static double max_diff(std::vector<float> const &a, std::vector<float> const &b) { double m = 0; for (size_t i = 0; i < a.size(); ++i) { m = std::max(m, (double)std::fabs(a[i] - b[i])); } return m; }
+
+template <int N>
+static void wire(std::mt19937_64 &mt, int I, int O, std::vector<std::int32_t> &idx)
+{
+    idx.resize((size_t)O * N);
+    for (int o = 0; o < O; ++o) {
+        for (int i = 0; i < N; ++i) {
+            for (;;) {
+                std::int32_t c = (std::int32_t)(mt() % (std::uint64_t)I);
+                bool dup = false;
+                for (int j = 0; j < i; ++j) { dup = dup || idx[(size_t)o * N + j] == c; }
+                if (!dup) { idx[(size_t)o * N + i] = c; break; }
+            }
+        }
+    }
+}
+
+static void read_fp32(bb::FrameBuffer &buf, std::vector<float> &out)
+{
+    auto p = buf.LockConst<float>();
+    out.assign((size_t)(buf.GetNodeSize() * buf.GetFrameSize()), 0.0f);
+    for (bb::index_t n = 0; n < buf.GetNodeSize(); ++n) for (bb::index_t f = 0; f < buf.GetFrameSize(); ++f) { out[(size_t)(n * buf.GetFrameSize() + f)] = p.Get(f, n); }
+}
+
+template <int N>
+static void test_stochastic(int I, int O, int F, bool lut_binarize, bool binary)
+{
+    std::mt19937_64 mt(12345 + I + O + F);
+    std::uniform_real_distribution<float> uni(-0.1f, 1.1f);
+    std::normal_distribution<float> nrm(0.0f, 1.0f);
+    constexpr int NN = 1 << N;
+
+    auto lut = bb::StochasticLutN<N, float>::Create(O);
+    lut->SendCommand(std::string("lut_binarize ") + (lut_binarize ? "true" : "false"));
+    lut->SendCommand(std::string("binary ") + (binary ? "true" : "false"));
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32);
+    lut->SetInputShape(x_buf.GetShape());
+
+    std::vector<std::int32_t> idx; wire<N>(mt, I, O, idx);
+    for (int o = 0; o < O; ++o) for (int i = 0; i < N; ++i) { lut->SetNodeConnectionIndex(o, i, idx[(size_t)o * N + i]); }
+    std::vector<float> W((size_t)O * NN), x((size_t)I * F), dy((size_t)O * F);
+    { auto Wp = lut->lock_W(); for (int o = 0; o < O; ++o) for (int i = 0; i < NN; ++i) { W[(size_t)o * NN + i] = std::min(1.0f, std::max(0.0f, uni(mt))); Wp(o, i) = W[(size_t)o * NN + i]; } }
+    { auto xp = x_buf.Lock<float>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x[(size_t)n * F + f] = uni(mt); xp.Set(f, n, x[(size_t)n * F + f]); } }
+    bb::FrameBuffer dy_buf(F, {O}, BB_TYPE_FP32);
+    { auto dp = dy_buf.Lock<float>(true); for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dy[(size_t)n * F + f] = nrm(mt); dp.Set(f, n, dy[(size_t)n * F + f]); } }
+
+    for (int loop = 0; loop < 2; ++loop) {            // dW accumulates over the loops, as in the reference test
+        auto y_buf = lut->Forward(x_buf);
+        auto dx_buf = lut->Backward(dy_buf);
+        std::vector<float> y, dx;
+        read_fp32(y_buf, y); read_fp32(dx_buf, dx);
+        std::vector<float> y_ref((size_t)O * F), dx_ref((size_t)I * F), dW_ref((size_t)O * NN, 0.0f);
+        oracle_fp32_StochasticLut_Forward(N, x.data(), y_ref.data(), idx.data(), W.data(), O, F, F, binary, lut_binarize, 0.25f, 0);
+        for (int l = 0; l <= loop; ++l) {
+            oracle_fp32_StochasticLut_Backward(N, x.data(), dy.data(), dx_ref.data(), idx.data(), W.data(), dW_ref.data(), I, O, F, F, binary, lut_binarize, 0.25f, 0);
+        }
+        std::vector<float> dW((size_t)O * NN);
+        { auto p = lut->lock_dW_const(); for (int o = 0; o < O; ++o) for (int i = 0; i < NN; ++i) { dW[(size_t)o * NN + i] = p(o, i); } }
+        CHECK(max_diff(y, y_ref) <= 1e-5, "StochasticLut%d %dx%dx%d y err %g", N, I, O, F, max_diff(y, y_ref));
+        CHECK(max_diff(dx, dx_ref) <= 1e-4 * max_abs(dx_ref), "StochasticLut%d dx err %g", N, max_diff(dx, dx_ref));
+        CHECK(max_diff(dW, dW_ref) <= 1e-4 * max_abs(dW_ref), "StochasticLut%d dW err %g (loop %d)", N, max_diff(dW, dW_ref), loop);
+    }
+    // ForwardNode agrees with the frame path on corner inputs
+    {
+        std::vector<double> v((size_t)N, 1.0);
+        double r = lut->ForwardNode(0, v)[0];
+        float w = W[(size_t)NN - 1]; if (lut_binarize) { w = w > 0.5f ? 1.0f : 0.0f; }
+        if (!binary) { CHECK(std::fabs(r - w) < 1e-6, "ForwardNode corner value %g vs %g", r, (double)w); }
+    }
+    // host-only execution is refused, not emulated
+    lut->SendCommand("host_only true");
+    bool threw = false;
+    try { lut->Forward(x_buf); } catch (bb::Exception const &) { threw = true; }
+    CHECK(threw, "host_only forward must throw");
+}
+
+template <int N>
+static void test_differentiable(int I, int O, int F, bool binary)
+{
+    std::mt19937_64 mt(777 + I + O + F);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    std::normal_distribution<float> nrm(0.0f, 1.0f);
+    constexpr int NN = 1 << N;
+    typename bb::DifferentiableLutN<N, float>::create_t cr;
+    cr.output_shape = {O}; cr.binary = binary;
+    auto lut = bb::DifferentiableLutN<N, float>::Create(cr);
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32);
+    lut->SetInputShape(x_buf.GetShape());
+    std::vector<std::int32_t> idx; wire<N>(mt, I, O, idx);
+    for (int o = 0; o < O; ++o) for (int i = 0; i < N; ++i) { lut->SetNodeConnectionIndex(o, i, idx[(size_t)o * N + i]); }
+    std::vector<float> W((size_t)O * NN), x((size_t)I * F), dy((size_t)O * F);
+    { auto Wp = lut->lock_W(); for (size_t k = 0; k < W.size(); ++k) { W[k] = uni(mt); Wp[(bb::index_t)k] = W[k]; } }
+    { auto xp = x_buf.Lock<float>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x[(size_t)n * F + f] = uni(mt); xp.Set(f, n, x[(size_t)n * F + f]); } }
+    bb::FrameBuffer dy_buf(F, {O}, BB_TYPE_FP32);
+    { auto dp = dy_buf.Lock<float>(true); for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dy[(size_t)n * F + f] = nrm(mt); dp.Set(f, n, dy[(size_t)n * F + f]); } }
+
+    auto y_buf = lut->Forward(x_buf, true);
+    auto dx_buf = lut->Backward(dy_buf);
+    std::vector<float> y, dx; read_fp32(y_buf, y); read_fp32(dx_buf, dx);
+    std::vector<float> y_ref((size_t)O * F), mean((size_t)O), rstd((size_t)O), rm((size_t)O, 0.0f), rv((size_t)O, 1.0f), dx_ref((size_t)I * F), dW_ref((size_t)O * NN, 0.0f);
+    oracle_fp32_DifferentiableLutN_ForwardTraining(N, x.data(), y_ref.data(), idx.data(), W.data(), mean.data(), rstd.data(), rm.data(), rv.data(), 0.3f, 0.5f, 0.9f, 0.25f, O, F, F, 0, binary);
+    oracle_fp32_DifferentiableLutN_Backward(N, x.data(), dy.data(), dx_ref.data(), idx.data(), W.data(), dW_ref.data(), mean.data(), rstd.data(), 0.3f, 0.5f, 0.25f, I, O, F, F, 0, binary);
+    std::vector<float> dW((size_t)O * NN), rm_gpu((size_t)O), rv_gpu((size_t)O), mean_gpu((size_t)O);
+    { auto p = lut->lock_dW_const(); for (size_t k = 0; k < dW.size(); ++k) { dW[k] = p[(bb::index_t)k]; } }
+    { auto a = lut->lock_mean_const(); auto b = lut->lock_var_const(); auto c = lut->lock_tmp_mean_const(); for (int o = 0; o < O; ++o) { rm_gpu[(size_t)o] = a[o]; rv_gpu[(size_t)o] = b[o]; mean_gpu[(size_t)o] = c[o]; } }
+    if (binary) {
+        size_t mism = 0; for (size_t k = 0; k < y.size(); ++k) { mism += (y[k] != y_ref[k]); }
+        CHECK(mism <= 2 + y.size() / 10000, "DifferentiableLut%d binary y mismatches %zu of %zu", N, mism, y.size());
+    }
+    else {
+        CHECK(max_diff(y, y_ref) <= 2e-4, "DifferentiableLut%d y err %g", N, max_diff(y, y_ref));
+    }
+    CHECK(max_diff(mean_gpu, mean) <= 1e-5, "batch mean err %g", max_diff(mean_gpu, mean));
+    CHECK(max_diff(rm_gpu, rm) <= 1e-5 && max_diff(rv_gpu, rv) <= 1e-5, "running statistics err %g %g", max_diff(rm_gpu, rm), max_diff(rv_gpu, rv));
+    CHECK(max_diff(dx, dx_ref) <= 1e-4 * max_abs(dx_ref), "DifferentiableLut%d dx err %g of %g", N, max_diff(dx, dx_ref), max_abs(dx_ref));
+    CHECK(max_diff(dW, dW_ref) <= 1e-4 * max_abs(dW_ref), "DifferentiableLut%d dW err %g of %g", N, max_diff(dW, dW_ref), max_abs(dW_ref));
+}
+
+static void test_binary(int I, int O, int F)
+{
+    std::mt19937_64 mt(99 + I + O + F);
+    auto lut = bb::BinaryLutN<6, bb::Bit>::Create(O);
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_BIT);
+    lut->SetInputShape(x_buf.GetShape());
+    int const words = (F + 31) / 32;
+    std::vector<std::int32_t> idx((size_t)O * 6), table((size_t)O * 2), x((size_t)I * words, 0), y_ref((size_t)O * words, 0);
+    for (int o = 0; o < O; ++o) {
+        for (int i = 0; i < 6; ++i) { idx[(size_t)o * 6 + i] = (std::int32_t)lut->GetNodeConnectionIndex(o, i); }
+        for (int b = 0; b < 64; ++b) { if (lut->GetLutTable(o, b)) { table[(size_t)o * 2 + b / 32] |= (std::int32_t)(1u << (b % 32)); } }
+    }
+    { auto xp = x_buf.Lock<bb::Bit>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { bool b = (mt() & 1) != 0; xp.Set(f, n, bb::Bit(b)); if (b) { x[(size_t)n * words + f / 32] |= (std::int32_t)(1u << (f % 32)); } } }
+    auto y_buf = lut->Forward(x_buf);
+    oracle_bit_BinaryLut6_Forward(x.data(), y_ref.data(), idx.data(), table.data(), O, F, words);
+    auto yp = y_buf.LockConst<bb::Bit>();
+    size_t mism = 0;
+    for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { mism += ((bool)yp.Get(f, n) != (((std::uint32_t)y_ref[(size_t)n * words + f / 32] >> (f % 32)) & 1u)); }
+    CHECK(mism == 0, "BinaryLut6 %dx%dx%d: %zu mismatching bits", I, O, F, mism);
+}
+
+// trained-layer hand-off: a StochasticLut6 with binarized tables tabulated into a BinaryLut6 gives the same bits
+static void test_import_layer(void)
+{
+    int const I = 32, O = 24, F = 200;
+    std::mt19937_64 mt(5);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    auto src = bb::StochasticLutN<6, bb::Bit>::Create(O);
+    src->SendCommand("lut_binarize true");
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_BIT);
+    src->SetInputShape(x_buf.GetShape());
+    { auto Wp = src->lock_W(); for (int k = 0; k < O * 64; ++k) { Wp[k] = uni(mt); } }
+    { auto xp = x_buf.Lock<bb::Bit>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { xp.Set(f, n, bb::Bit((mt() & 1) != 0)); } }
+    auto dst = bb::BinaryLutN<6, bb::Bit>::Create(O);
+    dst->SetInputShape(x_buf.GetShape());
+    dst->ImportLayer(src);
+    auto y_src = src->Forward(x_buf, false);          // fp32 in [0,1]; with binarized tables and bits at 0.5+-0.25 it is > 0.5 iff the table bit is 1
+    auto y_dst = dst->Forward(x_buf);
+    auto a = y_src.LockConst<float>(); auto b = y_dst.LockConst<bb::Bit>();
+    size_t mism = 0;
+    for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { mism += ((a.Get(f, n) > 0.5f) != (bool)b.Get(f, n)); }
+    CHECK(mism == 0, "ImportLayer: %zu mismatching bits", mism);
+}
+
+int main(void)
+{
+    if (!bb::Manager::IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
+    try {
+        // shapes of tests/gtest/StochasticLutNTest.cpp:235-246
+        int const shapes[][3] = {{6, 1, 1}, {14, 16, 8}, {14, 1024, 8}, {14, 1024, 3}, {13, 17, 1529}};
+        for (auto &s : shapes) {
+            test_stochastic<6>(s[0], s[1], s[2], true, false);
+            test_stochastic<6>(s[0], s[1], s[2], false, false);
+            test_stochastic<6>(s[0], s[1], s[2], false, true);
+        }
+        test_stochastic<4>(14, 33, 100, false, false);
+        test_stochastic<2>(14, 33, 100, true, false);
+        for (int dx_mode = 0; dx_mode <= 2; ++dx_mode) {
+            bbhip_SetDxMode(dx_mode);
+            test_stochastic<6>(40, 33, 300, false, false);
+            test_differentiable<6>(24, 20, 1024, true);
+            test_differentiable<6>(24, 20, 131, false);
+            test_differentiable<4>(24, 20, 64, true);
+        }
+        bbhip_SetDxMode(0);
+        test_binary(16, 16, 32);
+        test_binary(70, 33, 1000);
+        test_import_layer();
+    }
+    catch (std::exception const &e) {
+        std::printf("exception: %s\n", e.what());
+        return 1;
+    }
+    std::printf("%s (%d failed checks)\n", g_fail ? "FAILED" : "OK", g_fail);
+    return g_fail ? 1 : 0;
+}

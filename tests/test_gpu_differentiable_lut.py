@@ -89,9 +89,10 @@ def test_fp32_training_inference_backward(ops, n, F):
             dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev,
                                                  gamma, beta, 0.25, lut_binarize, binary_mode)
             if np.abs(dx_ref).max() > 0:
-                # hard-tanh gating flips for pre-activations within rounding of 0 or 1; allow for those frames
-                assert rel_err(host(dx)[:, :F], dx_ref[:, :F]) <= 1e-4 or F <= 39
-                assert rel_err(host(dW), dW_ref) <= 1e-4 or F <= 39
+                assert_bwd(host(dx)[:, :F], dx_ref[:, :F], "dx mode %d" % mode)
+                assert_bwd(host(dW), dW_ref, "dW mode %d" % mode)
+            else:       # a single frame: the batch statistics remove the whole gradient
+                assert np.abs(host(dx)[:, :F]).max() <= 1e-5 and np.abs(host(dW)).max() <= 1e-5
         ops.set_dx_mode(0)
 
 
@@ -118,8 +119,6 @@ def test_larger_layer(ops, n):
         dW = dev(np.zeros((O, 1 << n), np.float32))
         dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, mean, rstd, rev, binary_mode=binary_mode)
         assert_bwd(host(dx), dx_ref); assert_bwd(host(dW), dW_ref)
-        # batch-norm removes mean and scale from the gradient: sum_i dW = 0 and sum_i W dW = 0 up to the gated frames
-        assert np.abs(host(dW).astype(np.float64).sum(1)).max() <= 1e-3 * np.abs(dW_ref).max() * 64 or True
 
 
 @pytest.mark.parametrize("n", [6, 4])
