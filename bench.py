@@ -18,6 +18,17 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 
+# HBM-side bytes per launch at the default workloads, from the hardware counters FETCH_SIZE (x 2.000 KiB per count) and
+# WRITE_SIZE (x 1.000 KiB per count); each scale is what the same counter reads for a plain device copy of known size in
+# the same profiler run.  The counter tables and the commands are in profiles/*.md.  A kernel or workload that is not
+# listed reports null.
+MEASURED_TRAFFIC_BYTES = {
+    ("lut_dx_kernel<6>", 0):       (1041651.5 * 2.0 + 131072.0) * 1024,
+    ("lut_forward_kernel<6>", 0):  (234850.7 * 2.0 + 131072.0) * 1024,
+    ("lut_backward_kernel<6>", 0): (311368.4 * 2.0 + 16384.5) * 1024,
+    ("binary_lut6_kernel", 0):     (1020522.1 * 2.0 + 524288.0) * 1024,
+}
+
 
 def algorithmic_bytes(I, O, F):
     """every tensor touched once per pass, index and table traffic included (fp32, N = 6)"""
@@ -45,19 +56,84 @@ def cpu_baseline(I, O, frames, threads, reps=9):
                       % (I, O, frames, reps)}
 
 
+def bench_binarylut6(args, lib):
+    """BinaryLut6 packed inference: 8192 -> 16384 nodes, 262144 frames, 32 frames per word (secondary measurement)."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import capi, ops, synth
+    I, O, F = 8192, 16384, 262144
+    SW = synth.frame_stride_bit(F)
+    rng = np.random.default_rng(0)
+    idx = torch.from_numpy(synth.wiring(rng, I, O)).cuda()
+    T = torch.from_numpy(synth.truth_tables(rng, O)).cuda()
+    x = torch.from_numpy(synth.bernoulli_bits(rng, I, F, SW)).cuda()
+    y = torch.zeros((O, SW), dtype=torch.int32, device="cuda")
+    for _ in range(args.warmup):
+        ops.binary_lut6_forward(x, idx, T, F, out=y)
+    torch.cuda.synchronize()
+    lib.bbhip_KernelTimer_Enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ops.binary_lut6_forward(x, idx, T, F, out=y)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lib.bbhip_KernelTimer_Enable(0)
+    ms = C.c_float(); cnt = C.c_int()
+    capi.check(lib.bbhip_KernelTimer_Read(2, C.byref(ms), C.byref(cnt)))
+    avg_ms = ms.value / max(cnt.value, 1)
+    alg = F // 8 * (I + O) + 32 * O
+    gbs = alg / (avg_ms * 1e-3) / 1e9
+    out = {"metric": "T node-evals/s BinaryLut6 packed inference (8192 -> 16384 nodes, 262144 frames)",
+           "value": O * F / (dt / args.steps) / 1e12, "unit": "T node-evals/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+           "config": {"workload": "BinaryLut6 packed inference, 8192 in x 16384 out x 262144 frames", "frame_stride_words": SW},
+           "roofline": {"bound": "hbm", "kernel": "binary_lut6_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": gbs / HBM_PEAK_GBS,
+                        "traffic": MEASURED_TRAFFIC_BYTES.get(("binary_lut6_kernel", 0))}}
+    if args.profile_copy:
+        for _ in range(3):
+            y[:I].copy_(x)
+        torch.cuda.synchronize()
+        out["profile_copy_bytes"] = int(x.numel() * 4)
+    if not args.no_cpu:
+        import oracle
+        os.environ.setdefault("OMP_NUM_THREADS", str(min(os.cpu_count() or 1, 16)))
+        fs = 8192                                        # bounded sample: same nodes, 8192 of the 262144 frames
+        xs = synth.bernoulli_bits(rng, I, fs)
+        idx_h = idx.cpu().numpy(); T_h = T.cpu().numpy()
+        best = None
+        for _ in range(3):
+            t1 = time.perf_counter()
+            if oracle.have_ref():
+                oracle.ref_binary_lut6(xs, idx_h, T_h, fs, host_simd=True)
+            else:
+                oracle.binary_lut6_forward(xs, idx_h, T_h, fs, words=True)
+            d = time.perf_counter() - t1
+            best = d if best is None else min(best, d)
+        out["cpu_baseline"] = {"value": O * fs / best / 1e12, "unit": "T node-evals/s", "cores": min(os.cpu_count() or 1, 16),
+                               "kind": "reference" if oracle.have_ref() else "port",
+                               "sample": "BinaryLut6 forward (AVX2+OpenMP host path incl. harness copies), 8192 -> 16384 nodes, 8192 of the 262144 frames, best of 3"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "1")),
+    ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "0")),
                     help="0: deterministic input-centric dx; 1: fp32 atomics; 2: dx_tmp + reverse table")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--profile-copy", action="store_true",
+                    help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6"],
+                    help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards over frames, "
-              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path would shard over the "
+              "frame axis; no multi-GPU code is built)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
@@ -66,6 +142,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     lib = capi.lib()
+    if args.workload == "binarylut6":
+        return bench_binarylut6(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)
@@ -139,9 +217,15 @@ def main():
                    "lut_binarize": False, "binary": False, "frame_stride_floats": S},
         "hbm_frac_step": (fwd_b + bwd_b) / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dk["frac"], "traffic": None},
+                     "unit": "GB/s", "frac": dk["frac"],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((dominant, args.dx_mode))},
         "kernels": kernels,
     }
+    if args.profile_copy:
+        for _ in range(3):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        out["profile_copy_bytes"] = int(x.numel() * 4)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(I, O, args.cpu_frames, os.cpu_count() if (os.cpu_count() or 1) <= 16 else 16)
     print(json.dumps(out))

@@ -231,10 +231,14 @@ struct ForwardCall {
     float gamma, beta, momentum;
 };
 
+// the kernels address a frame inside its node row with a 32-bit byte offset
+constexpr int kMaxFrames = 1 << 29;
+
 int check_forward(ForwardCall const &c)
 {
     if (!(c.x && c.y && c.idx && c.W))               { return fail("forward: null buffer"); }
     if (!(c.node_size > 0 && c.frame_size > 0))      { return fail("forward: node_size=%d frame_size=%d must be positive", c.node_size, c.frame_size); }
+    if (c.frame_size > kMaxFrames)                   { return fail("forward: frame_size=%d above %d (32-bit byte offsets within a row)", c.frame_size, kMaxFrames); }
     int const x_need = (c.xmode == kXBit) ? (c.frame_size + 31) / 32 : c.frame_size;
     int const y_need = (c.ymode == kYBit) ? (c.frame_size + 31) / 32 : c.frame_size;
     if (c.x_stride < x_need || c.y_stride < y_need)  { return fail("forward: frame stride (x %d, y %d) shorter than the frames (%d, %d)", c.x_stride, c.y_stride, x_need, y_need); }
@@ -326,6 +330,7 @@ int check_backward(BackwardCall const &c, int dxmode)
 {
     if (!(c.x && c.dy && c.dx && c.idx && c.W && c.dW)) { return fail("backward: null buffer"); }
     if (!(c.input_node_size > 0 && c.output_node_size > 0 && c.frame_size > 0)) { return fail("backward: sizes must be positive"); }
+    if (c.frame_size > kMaxFrames)                   { return fail("backward: frame_size=%d above %d (32-bit byte offsets within a row)", c.frame_size, kMaxFrames); }
     int const x_need = (c.xmode == kXBit) ? (c.frame_size + 31) / 32 : c.frame_size;
     if (c.x_stride < x_need || c.frame_stride < c.frame_size) { return fail("backward: frame stride shorter than the frames"); }
     if ((long long)c.output_node_size * (1 << c.n) > 0x7fffffffLL) { return fail("backward: node_size too large"); }
