@@ -89,7 +89,7 @@ int env_int(char const *name, int def)
 
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 512); return ((v + 63) / 64) * 64; }
-int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 512);  return ((v + 63) / 64) * 64; }
+int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 1024);  return ((v + 63) / 64) * 64; }
 int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 256); return ((v + 63) / 64) * 64; }
 int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 4); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
 int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
@@ -139,11 +139,11 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
     default: return fail("LUT width n=%d not in 2..6", n); \
     }
 
-template <int N>
+template <int N, bool PLAIN = false>
 void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st)
 {
     int const total = node_size * (1 << N);
-    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize);
+    hipLaunchKernelGGL((table_prep_kernel<N, PLAIN>), dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize);
 }
 
 template <int N, int XMODE, int YMODE, int KIND>
@@ -380,7 +380,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     size_t const stat_bytes = c.bn ? align256((size_t)slab_total * c.output_node_size * 2 * sizeof(float)) : 0;
     size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;
     size_t const dtab_bytes = align256(term_count * sizeof(int));
-    size_t const otab_bytes = 0;
+    size_t const otab_bytes = (dxmode == kDxNone) ? c_bytes : 0;        // plain-basis coefficients for the dx kernel
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     char *base = nullptr;
     if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes + dyh_bytes, &base)) { return 1; }
@@ -388,14 +388,17 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
     int   *term = reinterpret_cast<int *>(base + c_bytes + part_bytes + stat_bytes);
+    float *P    = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
     float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes);
 
     launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
     BBHIP_LAUNCH_CHECK();
     if (dxmode == kDxNone && term_count > 0) {
+        launch_table_prep<N, true>(c.W, P, c.output_node_size, c.lut_binarize, st);
+        BBHIP_LAUNCH_CHECK();
         size_t const blocks = (term_count + kBlock - 1) / kBlock;
         if (blocks > 0x7fffffffULL) { return fail("backward: reverse table too large"); }
-        hipLaunchKernelGGL(term_table_kernel<N>, dim3((unsigned)blocks), dim3(kBlock), 0, st, C, c.idx, c.rev, c.rev_stride, c.input_node_size, term);
+        hipLaunchKernelGGL(term_table_kernel<N>, dim3((unsigned)blocks), dim3(kBlock), 0, st, P, c.idx, c.rev, c.rev_stride, c.input_node_size, term);
         BBHIP_LAUNCH_CHECK();
     }
 

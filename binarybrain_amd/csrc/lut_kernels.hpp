@@ -36,9 +36,11 @@ __device__ __forceinline__ float wave_sum(float v)
 }
 
 // ------------------------------------------------------------------------------------------------
-//  table preparation: C = centred-monomial coefficients of W' (W' = lut_binarize ? W > 0.5 : W)
+//  table preparation from W' (W' = lut_binarize ? W > 0.5 : W):
+//    PLAIN = false: C = coefficients in the centred monomial basis,  y = sum_S C[S] prod_{j in S} (x_j - 1/2)
+//    PLAIN = true : P = coefficients in the plain monomial basis,    y = sum_S P[S] prod_{j in S} x_j
 // ------------------------------------------------------------------------------------------------
-template <int N>
+template <int N, bool PLAIN>
 __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
                                                            int node_size, int lut_binarize)
 {
@@ -54,7 +56,8 @@ __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restr
 #pragma unroll
     for (int j = 0; j < N; ++j) {
         float const o = __shfl_xor(v, 1 << j, 64);
-        v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f;
+        if (PLAIN) { v = ((i >> j) & 1) ? (v - o) : v; }
+        else       { v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f; }
     }
     if (t < total) { C[t] = v; }
 }
@@ -125,7 +128,7 @@ struct FwdArgs {
 
 // FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only
 template <int N, int XMODE, int YMODE, int FWD_KIND>
-__global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void lut_forward_kernel(FwdArgs a)
 {
     using D = LutDims<N>;
     int const B    = a.chunk_count * a.tile_count;
@@ -136,9 +139,17 @@ __global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
-    float C[D::NN], cv[D::H];
-    LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
-    LutEval<N>::pin_constants(C, cv);
+    constexpr bool kMatrix = LutMatrixQ<N>::kUsable;
+    float C[kMatrix ? 1 : D::NN], cv[D::H];
+    LutMatrixQ<N> mq;
+    if constexpr (kMatrix) {
+        mq.load(a.C + (size_t)node * D::NN, lane);
+        C[0] = a.C[(size_t)node * D::NN];
+    }
+    else {
+        LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
+        LutEval<N>::pin_constants(C, cv);
+    }
     void const *rows[N];
 #pragma unroll
     for (int k = 0; k < N; ++k) {
@@ -160,7 +171,9 @@ __global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
         uint32_t raw[U][N];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            Gather<N, XMODE>::load_raw(rows, min(fb + u * kWave + lane, f_last), raw[u]);
+            if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
+                Gather<N, XMODE>::load_raw(rows, min(fb + u * kWave + lane, f_last), raw[u]);
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -170,7 +183,9 @@ __global__ __launch_bounds__(kBlock) void lut_forward_kernel(FwdArgs a)
             bool const ok = f < f_end;
             float z[N];
             Gather<N, XMODE>::centre_all(raw[u], min(f, f_last), a.bias, z);
-            float v = LutEval<N>::forward(C, cv, z);
+            float v;
+            if constexpr (kMatrix) { v = mq.forward(z); }
+            else                   { v = LutEval<N>::forward(C, cv, z); }
 
             if (FWD_KIND == 2) {
                 float const d = ok ? (v - c0) : 0.0f;
@@ -439,23 +454,15 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     }
 }
 
-// ------------------------------------------------------------------------------------------------
-//  input-centric dx: one wavefront owns dx[input node][64 frames x U] and walks the node's fan-out list
-//  (the reverse table, in its ascending (node, input) order), re-evaluating dy/dx_k of each consumer from that
-//  consumer's other N-1 inputs.  By multilinearity dy/dx_k is itself a LUT over the other inputs whose
-//  centred coefficients are the entries of C with bit k set:  Dk[s] = C[insert_zero_bit(s, k) | (1 << k)].
-//  No scratch, no atomics; every dx element is written exactly once, summed in the reference's order.
-// ------------------------------------------------------------------------------------------------
-
 // Term table for the input-centric dx kernel: for input node `in` and its t-th consumer connection (t-th entry of
 // the reverse-table row, e = node*N + k) one record of kTermHead + 2^(N-1) dwords at
 // ((in * max_fan + t) * record):  [0 .. N-2] the consumer's other input nodes (ascending connection order, k skipped),
-// [N-1] the consumer node, rest of the head unused, then the 2^(N-1) coefficients Dk.  All records of one input
+// [N-1] the consumer node, rest of the head unused, then the 2^(N-1) coefficients Dk (taken from the plain-basis table P).  All records of one input
 // node are contiguous, so a wavefront reads its whole work list from one base address with scalar loads.
 constexpr int kTermHead = 8;
 
 template <int N>
-__global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restrict__ C, int const *__restrict__ idx,
+__global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restrict__ P, int const *__restrict__ idx,
                                                            int const *__restrict__ rev, int rev_stride, int input_node_size,
                                                            int *__restrict__ term)
 {
@@ -480,7 +487,7 @@ __global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restr
             int const sidx = w - kTermHead;
             int const lo = sidx & ((1 << k) - 1);
             int const hi = sidx >> k;
-            v = __float_as_int(C[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)]);
+            v = __float_as_int(P[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)]);
         }
     }
     term[t] = v;
@@ -501,11 +508,33 @@ struct DxArgs {
 // ------------------------------------------------------------------------------------------------
 //  input-centric dx: one wavefront owns dx[input node][64 frames x U] and walks the node's fan-out list
 //  (the reverse table, in its ascending (node, input) order), re-evaluating dy/dx_k of each consumer from that
-//  consumer's other N-1 inputs.  By multilinearity dy/dx_k is itself a LUT over the other inputs whose
-//  centred coefficients are the entries of C with bit k set:  Dk[s] = C[insert_zero_bit(s, k) | (1 << k)].
-//  No scratch traffic, no atomics; every dx element is written exactly once, summed in the reference's order.
+//  consumer's other N-1 inputs.  By multilinearity dy/dx_k is itself a LUT over the other inputs; in the plain
+//  monomial basis  y = sum_S P[S] prod_{j in S} x_j  its coefficients are the entries of P with bit k set:
+//  Dk[s] = P[insert_zero_bit(s, k) | (1 << k)].  This kernel uses the plain basis (no centring subtraction per
+//  operand; |P| <= 2^N |W| keeps the rounding error of the 2^(N-1)-term sum near 1e-6 of the gradient scale).
+//  The low ML variables are expanded into monomials (wave-uniform coefficients, one FMA each), the high MH variables
+//  are folded by Horner's rule.  No scratch traffic, no atomics; every dx element is written exactly once, summed in
+//  the reference's order.
+//
+//  Rows are read through buffer descriptors (base = the row, extent = its valid bytes): the vector offset stays a
+//  32-bit register shared by all loads of a pass, and lanes beyond the last frame read 0 instead of needing a clamp.
 // ------------------------------------------------------------------------------------------------
-template <int N, int XMODE, int U>          // U wavefront-steps per unit: chunk = 64 * U frames
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(void const *base, int row, int stride_elems, uint32_t row_bytes)
+{
+    char const *p = reinterpret_cast<char const *>(base) + (size_t)row * (size_t)stride_elems * 4u;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p), 0, (int)row_bytes, 0x00020000);
+}
+
+// value of one input as the LUT sees it (reference: include/bb/StochasticLutN.h:536-553)
+template <int XMODE>
+__device__ __forceinline__ float input_value(uint32_t raw, int bit, float lo, float hi)
+{
+    if (XMODE == kXClamp)  { return __builtin_amdgcn_fmed3f(__uint_as_float(raw), 0.0f, 1.0f); }
+    if (XMODE == kXBinary) { return (__uint_as_float(raw) > 0.5f) ? hi : lo; }
+    return ((raw >> bit) & 1u) ? hi : lo;
+}
+
+template <int N, int XMODE, int U>          // U wavefront-steps per pass
 struct DxTerm {
     static constexpr int M  = N - 1;        // variables of the derivative LUT
     static constexpr int ML = M / 2, MH = M - ML;
@@ -515,52 +544,59 @@ struct DxTerm {
     uint32_t raw[U][M];
     float    dyv[U];
 
-    // scalar loads of one record, then the vector loads of its U x (M + 1) operands
-    __device__ __forceinline__ void fetch(DxArgs const &a, int const *__restrict__ rec, int const (&fs)[U])
+    // scalar loads of one record, then the vector loads of its U x (M + 1) operands.
+    // xoff / yoff: byte offset of this lane's element (word for packed rows) in the first step of the pass
+    __device__ __forceinline__ void fetch(DxArgs const &a, int const *__restrict__ rec, uint32_t xoff, uint32_t yoff,
+                                          uint32_t x_row_bytes, uint32_t y_row_bytes)
     {
-        void const *rows[M];
+        __amdgpu_buffer_rsrc_t rows[M];
 #pragma unroll
-        for (int j = 0; j < M; ++j) {
-            int const o = rec[j];
-            rows[j] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)o * a.x_stride)
-                                       : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)o * a.x_stride);
-        }
-        float const *dyr = a.dy + (size_t)rec[M] * a.dy_stride;
+        for (int j = 0; j < M; ++j) { rows[j] = row_descriptor(a.x, rec[j], a.x_stride, x_row_bytes); }
+        __amdgpu_buffer_rsrc_t const dyr = row_descriptor(a.dy, rec[M], a.dy_stride, y_row_bytes);
 #pragma unroll
         for (int sidx = 0; sidx < HN; ++sidx) { Dk[sidx] = __int_as_float(rec[kTermHead + sidx]); }
+        constexpr uint32_t xstep = (XMODE == kXBit) ? (kWave / 32) * 4u : kWave * 4u;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            Gather<M, XMODE>::load_raw(rows, fs[u], raw[u]);
-            dyv[u] = *reinterpret_cast<float const *>(reinterpret_cast<char const *>(dyr) + (uint32_t)fs[u] * 4u);
+#pragma unroll
+            for (int j = 0; j < M; ++j) { raw[u][j] = __builtin_amdgcn_raw_buffer_load_b32(rows[j], xoff + u * xstep, 0, 0); }
+            dyv[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0));
         }
     }
 
-    __device__ __forceinline__ void accumulate(int const (&fs)[U], float bias, float (&acc)[U]) const
+    __device__ __forceinline__ void accumulate(int bit, float lo, float hi, float (&acc)[U]) const
     {
+        // constant terms of the H partial sums in vector registers: an FMA reads at most one scalar register
         float cv[H];
+        if (L > 1) {
 #pragma unroll
-        for (int j = 0; j < H; ++j) { asm("v_mov_b32 %0, %1" : "=v"(cv[j]) : "s"(Dk[j * L])); }
+            for (int j = 0; j < H; ++j) { asm("v_mov_b32 %0, %1" : "=v"(cv[j]) : "s"(Dk[j * L])); }
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            float z[M];
-            Gather<M, XMODE>::centre_all(raw[u], fs[u], bias, z);
-            float zl[ML > 0 ? ML : 1], zh[MH];
+            float xv[M];
 #pragma unroll
-            for (int k = 0; k < ML; ++k) { zl[k] = z[k]; }
+            for (int k = 0; k < M; ++k) { xv[k] = input_value<XMODE>(raw[u][k], bit, lo, hi); }
+            float xl[ML > 0 ? ML : 1];
 #pragma unroll
-            for (int k = 0; k < MH; ++k) { zh[k] = z[ML + k]; }
-            float l[L], h[H];
-            monomials<ML>(zl, l);
-            monomials<MH>(zh, h);
-            float v = 0.0f;
+            for (int k = 0; k < ML; ++k) { xl[k] = xv[k]; }
+            float l[L];
+            monomials<ML>(xl, l);
+            float q[H];
 #pragma unroll
             for (int j = 0; j < H; ++j) {
-                float q = cv[j];
+                float s = (L > 1) ? cv[j] : Dk[j * L];
 #pragma unroll
-                for (int i = 1; i < L; ++i) { q = __builtin_fmaf(l[i], Dk[j * L + i], q); }
-                v = (j == 0) ? q : __builtin_fmaf(h[j], q, v);
+                for (int i = 1; i < L; ++i) { s = __builtin_fmaf(l[i], Dk[j * L + i], s); }
+                q[j] = s;
             }
-            acc[u] = __builtin_fmaf(dyv[u], v, acc[u]);
+            // Horner over the high variables: bit v of j belongs to xv[ML + v]
+#pragma unroll
+            for (int v = 0; v < MH; ++v) {
+#pragma unroll
+                for (int s = 0; s < (H >> (v + 1)); ++s) { q[s] = __builtin_fmaf(xv[ML + v], q[2 * s + 1], q[2 * s]); }
+            }
+            acc[u] = __builtin_fmaf(dyv[u], q[0], acc[u]);
         }
     }
 };
@@ -579,21 +615,23 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 
     int const cnt = a.rev[(size_t)in * a.rev_stride];
     int const *__restrict__ rec = a.term + (size_t)in * (a.rev_stride - 1) * T::REC;
-    int const f_last = a.frame_size - 1;
+    uint32_t const y_row_bytes = (uint32_t)a.frame_size * 4u;
+    uint32_t const x_row_bytes = (XMODE == kXBit) ? (uint32_t)((a.frame_size + 31) >> 5) * 4u : y_row_bytes;
+    float const lo = 0.5f - a.bias, hi = 0.5f + a.bias;
 
     // a unit is a.chunk frames = several passes of 64 * U frames; the node's work list is walked once per pass
     for (int f_begin = ck * a.chunk; f_begin < min((ck + 1) * a.chunk, a.frame_size); f_begin += kWave * U) {
-        int fs[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) { fs[u] = min(f_begin + u * kWave + lane, f_last); }
+        uint32_t const f0   = (uint32_t)(f_begin + lane);
+        uint32_t const yoff = f0 * 4u;
+        uint32_t const xoff = (XMODE == kXBit) ? (f0 >> 5) * 4u : yoff;
         float acc[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
 
         for (int t = 0; t < cnt; ++t) {
             T tm;
-            tm.fetch(a, rec + (size_t)t * T::REC, fs);
-            tm.accumulate(fs, a.bias, acc);
+            tm.fetch(a, rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes);
+            tm.accumulate(lane & 31, lo, hi, acc);
         }
 
 #pragma unroll

@@ -138,11 +138,22 @@ struct LutEval {
         for (int k = 0; k < D::NL; ++k) { zl[k] = z[k]; }
 #pragma unroll
         for (int k = 0; k < D::NH; ++k) { zh[k] = z[D::NL + k]; }
-        float l[D::L], h[D::H], q[D::H];
+        float l[D::L], q[D::H];
         monomials<D::NL>(zl, l);
-        monomials<D::NH>(zh, h);
         partial_q(C, cv, l, q);
-        return combine(h, q);
+        return fold_high(zh, q);
+    }
+
+    // Horner's rule over the high variables: sum_j h[j] q[j] with h the monomials of zh, bit v of j belonging to zh[v];
+    // H - 1 fused multiply-adds and no monomial products.  q is consumed.
+    __device__ __forceinline__ static float fold_high(float const (&zh)[D::NH], float (&q)[D::H])
+    {
+#pragma unroll
+        for (int v = 0; v < D::NH; ++v) {
+#pragma unroll
+            for (int s = 0; s < (D::H >> (v + 1)); ++s) { q[s] = __builtin_fmaf(zh[v], q[2 * s + 1], q[2 * s]); }
+        }
+        return q[0];
     }
 
     // d(sum)/dz for the variables of one group: out[k] = sum_{i : bit k} m[i ^ (1<<k)] * v[i]
@@ -163,6 +174,66 @@ struct LutEval {
             }
             out[k] = a;
         }
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+//  The partial sums q[j] = sum_i C[j*L + i] * l[i] on the matrix unit.
+//
+//  v_mfma_f32_4x4x1_16b_f32 performs, for each of the 16 lane quads b of a wavefront, the rank-1 update
+//      D_b[r][c] += A_b[r] * B_b[c],      A_b[r] = srcA of lane 4b + r,   B_b[c] = srcB of lane 4b + c,
+//  and returns D_b[r][c] in result register r of lane 4b + c.  With srcB = l[i] of the lane's own frame and
+//  srcA = C[(4g + r)*L + i] (the same in every quad), L - 1 such updates starting from the constant terms leave
+//  q[4g + r] of the lane's own frame in result register r: 4 coefficients per lane and instruction instead of 1,
+//  with the frames staying one per lane and no data movement between lanes.
+// ------------------------------------------------------------------------------------------------
+typedef float mfma_f4 __attribute__((ext_vector_type(4)));
+
+template <int N>
+struct LutMatrixQ {
+    using D = LutDims<N>;
+    static constexpr bool kUsable = (D::H % 4 == 0) && (D::L >= 4);
+    static constexpr int  G = (D::H >= 4) ? D::H / 4 : 1;     // groups of 4 partial sums
+
+    float   a[G][D::L];      // a[g][i]: coefficient C[(4g + lane%4)*L + i]   (i >= 1 used)
+    mfma_f4 c0[G];           // c0[g][r]: constant term C[(4g + r)*L], identical in all lanes
+
+    __device__ __forceinline__ void load(float const *__restrict__ Cg, int lane)
+    {
+        int const r = lane & 3;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int i = 1; i < D::L; ++i) { a[g][i] = Cg[(4 * g + r) * D::L + i]; }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) { c0[g][v] = Cg[(4 * g + v) * D::L]; }
+        }
+    }
+
+    __device__ __forceinline__ void partial_q(float const (&l)[D::L], float (&q)[D::H]) const
+    {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            mfma_f4 acc = c0[g];
+#pragma unroll
+            for (int i = 1; i < D::L; ++i) { acc = __builtin_amdgcn_mfma_f32_4x4x1f32(a[g][i], l[i], acc, 0, 0, 0); }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) { q[4 * g + v] = acc[v]; }
+        }
+    }
+
+    // y for one frame from the centred inputs z[0..N-1]
+    __device__ __forceinline__ float forward(float const (&z)[N]) const
+    {
+        float zl[D::NL > 0 ? D::NL : 1], zh[D::NH];
+#pragma unroll
+        for (int k = 0; k < D::NL; ++k) { zl[k] = z[k]; }
+#pragma unroll
+        for (int k = 0; k < D::NH; ++k) { zh[k] = z[D::NL + k]; }
+        float l[D::L], q[D::H];
+        monomials<D::NL>(zl, l);
+        partial_q(l, q);
+        return LutEval<N>::fold_high(zh, q);
     }
 };
 
