@@ -453,15 +453,16 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     }
 
     if (dxmode == kDxNone) {
+        int const steps = dx_pass_steps();              // wavefront-steps per pass: {1, 2, 4}
+        int const chunk = ((dx_chunk_frames() + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
+        int const chunk_count = ceil_div(c.frame_size, chunk);
+        int const in_tiles    = ceil_div(c.input_node_size, kWavesPerBlk);
+        if ((long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
         DxArgs d{};
         d.x = c.x; d.dy = c.bn ? dyh : c.dy; d.dx = c.dx; d.rev = c.rev; d.term = term;
         d.rev_stride = c.rev_stride; d.input_node_size = c.input_node_size; d.frame_size = c.frame_size;
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
-        int const steps = dx_pass_steps();              // wavefront-steps per pass: {1, 2, 4}
-        d.chunk = ((dx_chunk_frames() + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
-        d.chunk_count = ceil_div(c.frame_size, d.chunk);
-        d.tile_count  = ceil_div(c.input_node_size, kWavesPerBlk);
-        if ((long long)d.chunk_count * d.tile_count > 0x7fffffffLL) { return fail("backward: grid too large"); }
+        d.chunk = chunk; d.chunk_count = chunk_count; d.tile_count = in_tiles;
         d.bias = c.bias;
         {
             ScopedTimer tm(kTimeDx, st);
