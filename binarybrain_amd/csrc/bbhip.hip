@@ -90,8 +90,8 @@ int env_int(char const *name, int def)
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 512); return ((v + 63) / 64) * 64; }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 1024);  return ((v + 63) / 64) * 64; }
-int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 256); return ((v + 63) / 64) * 64; }
-int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 4); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
+int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
+int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 2); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
 int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
 
 // ------------------------------------------------------------------------------------------------
@@ -398,7 +398,9 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         BBHIP_LAUNCH_CHECK();
         size_t const blocks = (term_count + kBlock - 1) / kBlock;
         if (blocks > 0x7fffffffULL) { return fail("backward: reverse table too large"); }
-        hipLaunchKernelGGL(term_table_kernel<N>, dim3((unsigned)blocks), dim3(kBlock), 0, st, P, c.idx, c.rev, c.rev_stride, c.input_node_size, term);
+        hipLaunchKernelGGL(term_table_kernel<N>, dim3((unsigned)blocks), dim3(kBlock), 0, st, P, c.idx, c.rev, c.rev_stride, c.input_node_size,
+                           (unsigned long long)(uintptr_t)c.x, (unsigned long long)c.x_stride * 4ULL,
+                           (unsigned long long)(uintptr_t)(c.bn ? (void const *)dyh : (void const *)c.dy), (unsigned long long)c.frame_stride * 4ULL, term);
         BBHIP_LAUNCH_CHECK();
     }
 

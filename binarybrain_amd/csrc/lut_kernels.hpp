@@ -456,16 +456,21 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 
 // Term table for the input-centric dx kernel: for input node `in` and its t-th consumer connection (t-th entry of
 // the reverse-table row, e = node*N + k) one record of kTermHead + 2^(N-1) dwords at
-// ((in * max_fan + t) * record):  [0 .. N-2] the consumer's other input nodes (ascending connection order, k skipped),
-// [N-1] the consumer node, rest of the head unused, then the 2^(N-1) coefficients Dk (taken from the plain-basis table P).  All records of one input
-// node are contiguous, so a wavefront reads its whole work list from one base address with scalar loads.
-constexpr int kTermHead = 8;
+// ((in * max_fan + t) * record):  dwords [2j, 2j+1], j < N-1: the 64-bit device address of the row of the consumer's
+// other input j (ascending connection order, k skipped); dwords [2(N-1), 2(N-1)+1]: the address of the consumer's dy
+// row; rest of the head unused; then the 2^(N-1) coefficients Dk (taken from the plain-basis table P).  The addresses
+// are final, so the dx kernel spends no scalar arithmetic on them.  All records of one input node are contiguous, so a
+// wavefront reads its whole work list from one base address with scalar loads.
+constexpr int kTermHead = 12;
 
 template <int N>
 __global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restrict__ P, int const *__restrict__ idx,
                                                            int const *__restrict__ rev, int rev_stride, int input_node_size,
+                                                           unsigned long long x_base, unsigned long long x_row_pitch_bytes,
+                                                           unsigned long long dy_base, unsigned long long dy_row_pitch_bytes,
                                                            int *__restrict__ term)
 {
+    static_assert(2 * N <= kTermHead, "head too small");
     constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN;
     int const max_fan = rev_stride - 1;
     long long const t = (long long)blockIdx.x * kBlock + threadIdx.x;
@@ -476,19 +481,25 @@ __global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restr
     int const slot = (int)(rec % max_fan);
     int const in   = (int)(rec / max_fan);
     int const *r = rev + (size_t)in * rev_stride;
+    bool const live = slot < r[0];
+    int const e    = live ? r[1 + slot] : 0;
+    int const k    = e % N;
+    int const node = e / N;
     int v = 0;
-    if (slot < r[0]) {
-        int const e = r[1 + slot];
-        int const k = e % N;
-        int const node = e / N;
-        if (w < N - 1)            { v = idx[node * N + ((w < k) ? w : w + 1)]; }
-        else if (w == N - 1)      { v = node; }
-        else if (w >= kTermHead)  {
-            int const sidx = w - kTermHead;
-            int const lo = sidx & ((1 << k) - 1);
-            int const hi = sidx >> k;
-            v = __float_as_int(P[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)]);
+    if (w < 2 * N) {
+        int const j = w >> 1;
+        unsigned long long addr = (j < N - 1) ? x_base : dy_base;          // unused slots point at valid memory
+        if (live) {
+            addr = (j < N - 1) ? x_base + (unsigned long long)idx[node * N + ((j < k) ? j : j + 1)] * x_row_pitch_bytes
+                               : dy_base + (unsigned long long)node * dy_row_pitch_bytes;
         }
+        v = (w & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
+    }
+    else if (w >= kTermHead && live) {
+        int const sidx = w - kTermHead;
+        int const lo = sidx & ((1 << k) - 1);
+        int const hi = sidx >> k;
+        v = __float_as_int(P[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)]);
     }
     term[t] = v;
 }
@@ -525,6 +536,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(void const *bas
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p), 0, (int)row_bytes, 0x00020000);
 }
 
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t address_descriptor(uint32_t addr_lo, uint32_t addr_hi, uint32_t row_bytes)
+{
+    uint64_t const p = ((uint64_t)addr_hi << 32) | addr_lo;
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char *>(p), 0, (int)row_bytes, 0x00020000);
+}
+
 // value of one input as the LUT sees it (reference: include/bb/StochasticLutN.h:536-553)
 template <int XMODE>
 __device__ __forceinline__ float input_value(uint32_t raw, int bit, float lo, float hi)
@@ -534,37 +551,45 @@ __device__ __forceinline__ float input_value(uint32_t raw, int bit, float lo, fl
     return ((raw >> bit) & 1u) ? hi : lo;
 }
 
+// One term of the work list.  The gathered rows live in a Stage (vector registers); the coefficients are fetched
+// into scalar registers right before the term is evaluated.
 template <int N, int XMODE, int U>          // U wavefront-steps per pass
 struct DxTerm {
     static constexpr int M  = N - 1;        // variables of the derivative LUT
     static constexpr int ML = M / 2, MH = M - ML;
     static constexpr int L = 1 << ML, H = 1 << MH, HN = 1 << M, REC = kTermHead + HN;
 
-    float    Dk[HN];
-    uint32_t raw[U][M];
-    float    dyv[U];
+    struct Stage {
+        uint32_t raw[U][M];
+        float    dyv[U];
+    };
 
-    // scalar loads of one record, then the vector loads of its U x (M + 1) operands.
+    // vector loads of the U x (M + 1) operands of the record at rec (its head is read with scalar loads).
     // xoff / yoff: byte offset of this lane's element (word for packed rows) in the first step of the pass
-    __device__ __forceinline__ void fetch(DxArgs const &a, int const *__restrict__ rec, uint32_t xoff, uint32_t yoff,
-                                          uint32_t x_row_bytes, uint32_t y_row_bytes)
+    template <typename RecPtr>
+    __device__ __forceinline__ static void issue(RecPtr rec, uint32_t xoff, uint32_t yoff,
+                                                 uint32_t x_row_bytes, uint32_t y_row_bytes, Stage &st)
     {
-        __amdgpu_buffer_rsrc_t rows[M];
-#pragma unroll
-        for (int j = 0; j < M; ++j) { rows[j] = row_descriptor(a.x, rec[j], a.x_stride, x_row_bytes); }
-        __amdgpu_buffer_rsrc_t const dyr = row_descriptor(a.dy, rec[M], a.dy_stride, y_row_bytes);
-#pragma unroll
-        for (int sidx = 0; sidx < HN; ++sidx) { Dk[sidx] = __int_as_float(rec[kTermHead + sidx]); }
         constexpr uint32_t xstep = (XMODE == kXBit) ? (kWave / 32) * 4u : kWave * 4u;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
+        for (int j = 0; j < M; ++j) {
+            __amdgpu_buffer_rsrc_t const r = address_descriptor((uint32_t)rec[2 * j], (uint32_t)rec[2 * j + 1], x_row_bytes);
 #pragma unroll
-            for (int j = 0; j < M; ++j) { raw[u][j] = __builtin_amdgcn_raw_buffer_load_b32(rows[j], xoff + u * xstep, 0, 0); }
-            dyv[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0));
+            for (int u = 0; u < U; ++u) { st.raw[u][j] = __builtin_amdgcn_raw_buffer_load_b32(r, xoff + u * xstep, 0, 0); }
         }
+        __amdgpu_buffer_rsrc_t const dyr = address_descriptor((uint32_t)rec[2 * M], (uint32_t)rec[2 * M + 1], y_row_bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) { st.dyv[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0)); }
     }
 
-    __device__ __forceinline__ void accumulate(int bit, float lo, float hi, float (&acc)[U]) const
+    template <typename RecPtr>
+    __device__ __forceinline__ static void load_coefficients(RecPtr rec, float (&Dk)[HN])
+    {
+#pragma unroll
+        for (int sidx = 0; sidx < HN; ++sidx) { Dk[sidx] = __int_as_float(rec[kTermHead + sidx]); }
+    }
+
+    __device__ __forceinline__ static void accumulate(Stage const &st, float const (&Dk)[HN], int bit, float lo, float hi, float (&acc)[U])
     {
         // constant terms of the H partial sums in vector registers: an FMA reads at most one scalar register
         float cv[H];
@@ -576,7 +601,7 @@ struct DxTerm {
         for (int u = 0; u < U; ++u) {
             float xv[M];
 #pragma unroll
-            for (int k = 0; k < M; ++k) { xv[k] = input_value<XMODE>(raw[u][k], bit, lo, hi); }
+            for (int k = 0; k < M; ++k) { xv[k] = input_value<XMODE>(st.raw[u][k], bit, lo, hi); }
             float xl[ML > 0 ? ML : 1];
 #pragma unroll
             for (int k = 0; k < ML; ++k) { xl[k] = xv[k]; }
@@ -596,7 +621,7 @@ struct DxTerm {
 #pragma unroll
                 for (int s = 0; s < (H >> (v + 1)); ++s) { q[s] = __builtin_fmaf(xv[ML + v], q[2 * s + 1], q[2 * s]); }
             }
-            acc[u] = __builtin_fmaf(dyv[u], q[0], acc[u]);
+            acc[u] = __builtin_fmaf(st.dyv[u], q[0], acc[u]);
         }
     }
 };
@@ -614,12 +639,19 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
     int const lane = threadIdx.x & (kWave - 1);
 
     int const cnt = a.rev[(size_t)in * a.rev_stride];
-    int const *__restrict__ rec = a.term + (size_t)in * (a.rev_stride - 1) * T::REC;
+    // The term table is read through the constant address space: its wave-uniform loads stay scalar loads wherever
+    // they are placed relative to the stores of this kernel (the table is written by an earlier kernel).
+    typedef __attribute__((address_space(4))) int const const_int;
+    const_int *rec = (const_int *)(a.term + (size_t)in * (a.rev_stride - 1) * T::REC);
     uint32_t const y_row_bytes = (uint32_t)a.frame_size * 4u;
     uint32_t const x_row_bytes = (XMODE == kXBit) ? (uint32_t)((a.frame_size + 31) >> 5) * 4u : y_row_bytes;
     float const lo = 0.5f - a.bias, hi = 0.5f + a.bias;
+    int const bit = lane & 31;
 
-    // a unit is a.chunk frames = several passes of 64 * U frames; the node's work list is walked once per pass
+    // a unit is a.chunk frames = several passes of 64 * U frames; the node's work list is walked once per pass.
+    // (Requesting the operands of later terms ahead of time — a ring of stages — was measured slower at every depth:
+    // with 8 wavefronts per SIMD the other wavefronts already cover the latency, and more loads in flight only
+    // lengthen the queues.)
     for (int f_begin = ck * a.chunk; f_begin < min((ck + 1) * a.chunk, a.frame_size); f_begin += kWave * U) {
         uint32_t const f0   = (uint32_t)(f_begin + lane);
         uint32_t const yoff = f0 * 4u;
@@ -629,9 +661,11 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
         for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
 
         for (int t = 0; t < cnt; ++t) {
-            T tm;
-            tm.fetch(a, rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes);
-            tm.accumulate(lane & 31, lo, hi, acc);
+            typename T::Stage st;
+            float Dk[T::HN];
+            T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
+            T::load_coefficients(rec + (size_t)t * T::REC, Dk);
+            T::accumulate(st, Dk, bit, lo, hi, acc);
         }
 
 #pragma unroll

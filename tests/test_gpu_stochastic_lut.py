@@ -205,3 +205,67 @@ def test_full_size_properties(ops):
     fs = 256
     dx_ref, _ = oracle.stochastic_lut_backward(6, np.ascontiguousarray(x[:, :fs]), np.ascontiguousarray(dy[:, :fs]), idx, W, fs)
     assert_bwd(host(dxb)[:, :fs], dx_ref)
+
+
+def _adversarial_tables(n):
+    """Tables whose monomial coefficients are as large as a [0,1] table allows: parity, AND, OR, single spikes."""
+    nn = 1 << n
+    i = np.arange(nn)
+    pop = np.array([bin(v).count("1") for v in i])
+    t = [
+        (pop & 1).astype(np.float32),                 # parity: plain-basis coefficients (-2)^(|S|-1)
+        1.0 - (pop & 1).astype(np.float32),
+        (i == nn - 1).astype(np.float32),             # AND
+        (i != 0).astype(np.float32),                  # OR
+        np.ones(nn, np.float32),
+        np.zeros(nn, np.float32),
+        ((i >> (n - 1)) & 1).astype(np.float32),      # projection on the last input
+        (i == 5 % nn).astype(np.float32),             # one spike
+    ]
+    return np.stack(t)
+
+
+@pytest.mark.parametrize("n", [6, 5, 4, 3, 2])
+def test_adversarial_tables(ops, n):
+    """Worst cases for a monomial-basis evaluation: extreme tables with inputs at and near the corners of the cube.
+    The oracle here is the defining formula in fp64 (sum of 2^n products), not an fp32 association."""
+    rng = np.random.default_rng(700 + n)
+    T = _adversarial_tables(n)
+    O = T.shape[0] * 4
+    I, F = 16, 192
+    W = np.tile(T, (4, 1)).astype(np.float32)
+    idx = synth.wiring(rng, I, O, n)
+    stride = synth.frame_stride_fp32(F)
+    x = np.zeros((I, stride), np.float32)
+    x[:, :64] = rng.integers(0, 2, (I, 64)).astype(np.float32)                     # corners
+    x[:, 64:128] = np.clip(rng.integers(0, 2, (I, 64)) + rng.normal(0, 1e-3, (I, 64)), 0, 1)   # next to corners
+    x[:, 128:F] = rng.random((I, F - 128))
+    dy = synth.normal_frames(rng, O, F, stride)
+
+    xs = x[idx][:, :, :F].astype(np.float64)                                       # [O][n][F]
+    y64 = np.zeros((O, F)); dW64 = np.zeros((O, 1 << n)); dx64 = np.zeros((I, F))
+    for i in range(1 << n):
+        fac = [xs[:, j] if (i >> j) & 1 else 1.0 - xs[:, j] for j in range(n)]
+        prod = np.prod(fac, axis=0)
+        y64 += W[:, i:i + 1] * prod
+        dW64[:, i] = (dy[:, :F] * prod).sum(axis=1)
+        for j in range(n):
+            others = np.prod([fac[k] for k in range(n) if k != j], axis=0) if n > 1 else 1.0
+            g = W[:, i:i + 1] * others * dy[:, :F] * (1.0 if (i >> j) & 1 else -1.0)
+            np.add.at(dx64, idx[:, j], g)
+
+    y = ops.stochastic_lut_forward(n, dev(x), dev(idx), dev(W), F, False, False)
+    assert_fwd(host(y)[:, :F], np.clip(y64, 0, 1), "y")
+    rev = ops.reverse_table(dev(idx), I)
+    for mode in (0, 1, 2):
+        ops.set_dx_mode(mode)
+        dW = dev(np.zeros((O, 1 << n), np.float32))
+        dx = ops.stochastic_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, False, False)
+        assert_bwd(host(dx)[:, :F], dx64, "dx mode %d" % mode)
+        assert_bwd(host(dW), dW64, "dW mode %d" % mode)
+    ops.set_dx_mode(0)
+    # the exact corner frames reproduce the table entries themselves
+    corner = host(y)[:, :64]
+    sel = (xs[:, :, :64] > 0.5).astype(np.int64)
+    code = sum(sel[:, j] << j for j in range(n))
+    assert np.array_equal(corner, np.take_along_axis(W, code, axis=1))
