@@ -88,7 +88,7 @@ int env_int(char const *name, int def)
 }
 
 // frames per unit; both are rounded to wavefront multiples where used
-int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 512); return ((v + 63) / 64) * 64; }
+int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 256); return ((v + 63) / 64) * 64; }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 1024);  return ((v + 63) / 64) * 64; }
 int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
 int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 2); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
@@ -149,7 +149,7 @@ void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize
 template <int N, int XMODE, int YMODE, int KIND>
 void launch_forward(FwdArgs const &a, hipStream_t st)
 {
-    hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND>), dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, st, a);
+    hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND>), dim3(a.chunk_count * a.tiles.count), dim3(kBlock), 0, st, a);
 }
 
 // xmode / ymode / kind are runtime values here; the combinations that exist are enumerated explicitly
@@ -175,7 +175,7 @@ int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, hipStream
 template <int N>
 int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStream_t st)
 {
-    dim3 const grid(a.slab_count * a.tile_count), block(kBlock);
+    dim3 const grid(a.slab_count * a.tiles.count), block(kBlock);
 #define BBHIP_BWD_CASE(X, K, M) if (xmode == X && kind == K && dxmode == M) { hipLaunchKernelGGL((lut_backward_kernel<N, X, K, M>), grid, block, 0, st, a); return 0; }
     BBHIP_BWD_CASE(kXClamp,  0, kDxAtomic) BBHIP_BWD_CASE(kXClamp,  0, kDxTmp)
     BBHIP_BWD_CASE(kXBinary, 0, kDxAtomic) BBHIP_BWD_CASE(kXBinary, 0, kDxTmp)
@@ -196,7 +196,7 @@ int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStre
 template <int N, int U>
 int dispatch_dx_u(int xmode, DxArgs const &a, hipStream_t st)
 {
-    dim3 const grid(a.chunk_count * a.tile_count), block(kBlock);
+    dim3 const grid(a.chunk_count * a.tiles.count), block(kBlock);
     switch (xmode) {
     case kXClamp:  hipLaunchKernelGGL((lut_dx_kernel<N, kXClamp, U>),  grid, block, 0, st, a); return 0;
     case kXBinary: hipLaunchKernelGGL((lut_dx_kernel<N, kXBinary, U>), grid, block, 0, st, a); return 0;
@@ -273,7 +273,7 @@ int run_forward(ForwardCall const &c, hipStream_t st)
     a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C;
     a.node_size = c.node_size; a.frame_size = c.frame_size;
     a.x_stride = c.x_stride; a.y_stride = c.y_stride;
-    a.chunk = chunk; a.chunk_count = chunk_count; a.tile_count = tile_count;
+    a.chunk = chunk; a.chunk_count = chunk_count; a.tiles = make_tile_divisor(tile_count);
     a.bias = c.bias; a.gamma = c.gamma; a.beta = c.beta;
 
     int kind = 0;
@@ -410,7 +410,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     a.mean = c.mean; a.rstd = c.rstd; a.dmean = c.dmean_tmp; a.dvar = c.dvar_tmp;
     a.node_size = c.output_node_size; a.frame_size = c.frame_size;
     a.x_stride = c.x_stride; a.dy_stride = c.frame_stride;
-    a.slab = slab; a.tile_count = tile_count;
+    a.slab = slab; a.tiles = make_tile_divisor(tile_count);
     a.bias = c.bias; a.gamma = c.gamma; a.beta = c.beta; a.inv_frames = 1.0f / (float)c.frame_size;
 
     if (c.bn) {
@@ -464,7 +464,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         d.x = c.x; d.dy = c.bn ? dyh : c.dy; d.dx = c.dx; d.rev = c.rev; d.term = term;
         d.rev_stride = c.rev_stride; d.input_node_size = c.input_node_size; d.frame_size = c.frame_size;
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
-        d.chunk = chunk; d.chunk_count = chunk_count; d.tile_count = in_tiles;
+        d.chunk = chunk; d.chunk_count = chunk_count; d.tiles = make_tile_divisor(in_tiles);
         d.bias = c.bias;
         {
             ScopedTimer tm(kTimeDx, st);
@@ -895,12 +895,12 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     a.word_count = (frame_size + 31) / 32;
     a.chunk = bin_chunk_words();
     a.chunk_count = ceil_div(a.word_count, a.chunk);
-    a.tile_count = ceil_div(node_size, kWavesPerBlk);
-    BBHIP_REQUIRE((long long)a.chunk_count * a.tile_count <= 0x7fffffffLL);
+    a.tiles = make_tile_divisor(ceil_div(node_size, kWavesPerBlk));
+    BBHIP_REQUIRE((long long)a.chunk_count * a.tiles.count <= 0x7fffffffLL);
     {
         ScopedTimer tm(kTimeBinary, st);
-        if (a.chunk % 128 == 0) { hipLaunchKernelGGL(binary_lut6_kernel<2>, dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, st, a); }
-        else                    { hipLaunchKernelGGL(binary_lut6_kernel<1>, dim3(a.chunk_count * a.tile_count), dim3(kBlock), 0, st, a); }
+        if (a.chunk % 128 == 0) { hipLaunchKernelGGL(binary_lut6_kernel<2>, dim3(a.chunk_count * a.tiles.count), dim3(kBlock), 0, st, a); }
+        else                    { hipLaunchKernelGGL(binary_lut6_kernel<1>, dim3(a.chunk_count * a.tiles.count), dim3(kBlock), 0, st, a); }
     }
     BBHIP_LAUNCH_CHECK();
     return 0;

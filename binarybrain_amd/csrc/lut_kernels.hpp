@@ -13,6 +13,7 @@
 #pragma once
 
 #include "lut_math.hpp"
+#include "tile_divisor.hpp"
 
 namespace bbhip {
 
@@ -122,7 +123,8 @@ struct FwdArgs {
     int   node_size, frame_size;
     int   x_stride, y_stride;   // elements per node row (floats or words)
     int   chunk;                // frames per unit, multiple of 64
-    int   chunk_count, tile_count;
+    int   chunk_count;
+    TileDivisor tiles;
     float bias, gamma, beta;
 };
 
@@ -131,10 +133,10 @@ template <int N, int XMODE, int YMODE, int FWD_KIND>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void lut_forward_kernel(FwdArgs a)
 {
     using D = LutDims<N>;
-    int const B    = a.chunk_count * a.tile_count;
+    int const B    = a.chunk_count * a.tiles.count;
     int const lid  = xcd_remap(blockIdx.x, B);
-    int const ck   = lid / a.tile_count;
-    int const tile = lid - ck * a.tile_count;
+    int ck, tile;
+    split_tile(lid, a.tiles, ck, tile);
     int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
@@ -275,7 +277,8 @@ struct BwdArgs {
     int   f_base, f_limit;      // frame range handled by this launch
     int   slab;                 // frames per unit, multiple of 64
     int   slab_first;           // index of the first slab of this launch in dw_partial
-    int   slab_count, tile_count;
+    int   slab_count;
+    TileDivisor tiles;
     float bias, gamma, beta, inv_frames;
 };
 
@@ -289,10 +292,10 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     using D = LutDims<N>;
     __shared__ float red[kWavesPerBlk][16][kWave + 1];
 
-    int const B    = a.slab_count * a.tile_count;
+    int const B    = a.slab_count * a.tiles.count;
     int const lid  = xcd_remap(blockIdx.x, B);
-    int const sl   = lid / a.tile_count;
-    int const tile = lid - sl * a.tile_count;
+    int sl, tile;
+    split_tile(lid, a.tiles, sl, tile);
     int const wv   = threadIdx.x / kWave;
     int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + wv);
     if (node >= a.node_size) { return; }
@@ -512,7 +515,8 @@ struct DxArgs {
     int const   *term;          // term table, see term_table_kernel
     int   rev_stride, input_node_size, frame_size;
     int   x_stride, dy_stride, dx_stride;
-    int   chunk, chunk_count, tile_count;
+    int   chunk, chunk_count;
+    TileDivisor tiles;
     float bias;
 };
 
@@ -630,10 +634,10 @@ template <int N, int XMODE, int U>
 __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 {
     using T = DxTerm<N, XMODE, U>;
-    int const B    = a.chunk_count * a.tile_count;
+    int const B    = a.chunk_count * a.tiles.count;
     int const lid  = xcd_remap(blockIdx.x, B);
-    int const ck   = lid / a.tile_count;
-    int const tile = lid - ck * a.tile_count;
+    int ck, tile;
+    split_tile(lid, a.tiles, ck, tile);
     int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
     if (in >= a.input_node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
@@ -758,7 +762,8 @@ struct BinArgs {
     int node_size, frame_size, stride;   // stride in words
     int word_count;             // (frame_size + 31) / 32
     int chunk;                  // words per unit, multiple of 64
-    int chunk_count, tile_count;
+    int chunk_count;
+    TileDivisor tiles;
 };
 
 // table [O][2] (entries 0-31 in word 0) -> mask [O][64]
@@ -789,10 +794,10 @@ __device__ __forceinline__ uint32_t bfi_vsv(uint32_t s, uint32_t hi, uint32_t lo
 template <int WPL>   // words per lane per step
 __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
 {
-    int const B    = a.chunk_count * a.tile_count;
+    int const B    = a.chunk_count * a.tiles.count;
     int const lid  = xcd_remap(blockIdx.x, B);
-    int const ck   = lid / a.tile_count;
-    int const tile = lid - ck * a.tile_count;
+    int ck, tile;
+    split_tile(lid, a.tiles, ck, tile);
     int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);

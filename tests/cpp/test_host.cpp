@@ -8,6 +8,7 @@
 #include "bb/StochasticLutN.h"
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
+#include "../../binarybrain_amd/csrc/tile_divisor.hpp"
 
 extern "C" int oracle_ReverseTable(int n, std::int32_t const *idx, int input_node_size, int output_node_size, std::int32_t *rev, int rev_cap);
 
@@ -132,6 +133,31 @@ int main(void)
         CHECK(seen.size() == 6);
         CHECK(bl->Backward(bb::FrameBuffer(8, {5}, BB_TYPE_FP32, true)).GetNodeSize() == 9);
     }
+    // workgroup index -> (frame chunk, node tile) without an integer division: exact for every index below 2^31
+    {
+        int const divisors[] = {1, 2, 3, 5, 7, 64, 255, 256, 257, 1000, 1024, 1536, 4096, 65535, 1 << 20, (1 << 20) + 1, 0x3fffffff, 0x7fffffff};
+        std::uint64_t state = 0x9e3779b97f4a7c15ull;
+        for (int d : divisors) {
+            bbhip::TileDivisor const t = bbhip::make_tile_divisor(d);
+            auto check = [&](std::uint32_t n) {
+                int outer, tile;
+                bbhip::split_tile((int)n, t, outer, tile);
+                if (outer != (int)(n / (std::uint32_t)d) || tile != (int)(n % (std::uint32_t)d)) { CHECK(!"split_tile"); }
+            };
+            for (std::uint32_t n = 0; n < 70000; ++n) { check(n); }
+            for (std::uint32_t k = 1; k < 200; ++k) {                 // around multiples of d and at the top of the range
+                std::uint64_t const m = (std::uint64_t)k * (std::uint64_t)d;
+                if (m < 0x7fffffffull) { check((std::uint32_t)m); check((std::uint32_t)m - 1); check((std::uint32_t)m + 1 < 0x80000000u ? (std::uint32_t)m + 1 : 0); }
+                check(0x7fffffffu - k);
+            }
+            for (int i = 0; i < 200000; ++i) {
+                state ^= state << 13; state ^= state >> 7; state ^= state << 17;
+                check((std::uint32_t)(state >> 33));
+            }
+            check(0x7fffffffu);
+        }
+    }
+
     std::printf("%s (%d failed checks)\n", g_fail ? "FAILED" : "OK", g_fail);
     return g_fail ? 1 : 0;
 }
