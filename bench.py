@@ -23,9 +23,9 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # the same profiler run.  The counter tables and the commands are in profiles/*.md.  A kernel or workload that is not
 # listed reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("lut_dx_kernel<6>", 0):       (1051926.5 * 2.0 + 131072.0) * 1024,
-    ("lut_forward_kernel<6>", 0):  (235452.5 * 2.0 + 131072.0) * 1024,
-    ("lut_backward_kernel<6>", 0): (350947.5 * 2.0 + 8192.3) * 1024,
+    ("lut_dx_kernel<6>", 0):       (657246.3 * 2.0 + 131072.0) * 1024,
+    ("lut_forward_kernel<6>", 0):  (135308.5 * 2.0 + 131072.0) * 1024,
+    ("lut_backward_kernel<6>", 0): (351931.7 * 2.0 + 8192.4) * 1024,
     ("binary_lut6_kernel", 0):     (1020522.1 * 2.0 + 524288.0) * 1024,
 }
 
