@@ -56,6 +56,51 @@ def cpu_baseline(I, O, frames, threads, reps=9):
                       % (I, O, frames, reps)}
 
 
+def bench_adam(args, lib):
+    """One Adam update of a parameter list (secondary measurement): the three W tables of the MNIST-shaped LUT network
+    (6144, 1024 and 70 nodes x 64 entries) followed by four 16 Mi-element tensors, so that the call is bandwidth-bound.
+    Algorithmic bytes: 28 per element (read p, g, m, v; write p, m, v)."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import ops
+    sizes = [6144 * 64, 1024 * 64, 70 * 64] + [1 << 24] * 4
+    g = torch.Generator(device="cuda"); g.manual_seed(0)
+    params = [torch.rand(n, device="cuda", generator=g) for n in sizes]
+    grads = [torch.randn(n, device="cuda", generator=g) * 0.1 for n in sizes]
+    st = ops.AdamState(params, grads)
+    for _ in range(args.warmup):
+        st.step()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        st.step()
+    e1.record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    kernel_ms = e0.elapsed_time(e1) / args.steps          # back-to-back launches of the one kernel on the current stream
+    total = sum(sizes)
+    gbs = 28.0 * total / (kernel_ms * 1e-3) / 1e9
+    out = {"metric": "G parameter updates/s, Adam fp32", "value": total / (dt / args.steps) / 1e9, "unit": "G updates/s",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "Adam step over %d tensors, %d elements" % (len(sizes), total)},
+           "roofline": {"bound": "hbm", "kernel": "adam_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+    if not args.no_cpu:
+        import oracle
+        n = 1 << 22
+        rng = np.random.default_rng(0)
+        p = rng.random(n).astype(np.float32); gr = rng.standard_normal(n).astype(np.float32)
+        oracle.adam_steps(p, [gr])
+        t = time.perf_counter(); reps = 20
+        oracle.adam_steps(p, [gr] * reps)
+        out["cpu_baseline"] = {"value": n * reps / (time.perf_counter() - t) / 1e9, "unit": "G updates/s", "cores": 1, "kind": "port",
+                               "sample": "C restatement of the reference's host update, one tensor of %d elements, %d steps" % (n, reps)}
+    print(json.dumps(out))
+
+
 def bench_binarylut6(args, lib):
     """BinaryLut6 packed inference: 8192 -> 16384 nodes, 262144 frames, 32 frames per word (secondary measurement)."""
     import numpy as np
@@ -127,7 +172,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "adam"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -144,6 +189,8 @@ def main():
     lib = capi.lib()
     if args.workload == "binarylut6":
         return bench_binarylut6(args, lib)
+    if args.workload == "adam":
+        return bench_adam(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)

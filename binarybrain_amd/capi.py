@@ -34,6 +34,16 @@ _SIGNATURES = {
     "bbhip_GetDxMode": (C.c_int, []),
     "bbhip_fp32_Vector_set": (C.c_int, [_vp, _f, _i, _vp]),
     "bbhip_fp32_Vector_clamp": (C.c_int, [_vp, _vp, _f, _f, _i, _vp]),
+    "bbhip_fp32_Vector_add_ex": (C.c_int, [_vp, _vp, _vp, _f, _f, _f, _i, _vp]),
+    "bbhip_fp32_Vector_mul_ex": (C.c_int, [_vp, _vp, _vp, _f, _f, _i, _vp]),
+    "bbhip_fp32_Vector_div_ex": (C.c_int, [_vp, _vp, _vp, _f, _f, _f, _f, _i, _vp]),
+    "bbhip_fp32_Vector_sqrt": (C.c_int, [_vp, _vp, _i, _vp]),
+    "bbhip_fp32_Vector_exp": (C.c_int, [_vp, _vp, _i, _vp]),
+    "bbhip_fp32_Vector_min": (C.c_int, [_vp, _vp, _vp, _i, _vp]),
+    "bbhip_fp32_Vector_min_v": (C.c_int, [_vp, _vp, _f, _i, _vp]),
+    "bbhip_fp32_Vector_max": (C.c_int, [_vp, _vp, _vp, _i, _vp]),
+    "bbhip_fp32_Vector_max_v": (C.c_int, [_vp, _vp, _f, _i, _vp]),
+    "bbhip_fp32_OptimizerAdam": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _vp]),
     "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "bbhip_bit_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),

@@ -14,6 +14,7 @@
 
 #include "../../include/bbhip.h"
 #include "lut_kernels.hpp"
+#include "vector_kernels.hpp"
 
 using namespace bbhip;
 
@@ -545,6 +546,24 @@ struct LocalHeap {
 
 LocalHeap &heap(void) { static LocalHeap h; return h; }
 
+constexpr int kAdamBlocksPerTensor = 1024;
+
+template <int OP>
+int vector_op(float *dst, float const *src0, float const *src1, float a, float b, float c, float d, int size, void *stream, char const *name)
+{
+    if (!(dst != nullptr && src0 != nullptr && (src1 != nullptr || !vec_binary<OP>()) && size >= 0)) {
+        return fail("%s: rejected argument (null pointer or negative size)", name);
+    }
+    if (size == 0) { return 0; }
+    int const aligned = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src0) |
+                          (vec_binary<OP>() ? reinterpret_cast<uintptr_t>(src1) : 0)) & 15) == 0;
+    size_t const blocks = ((size_t)size + kVecBlock * 4 - 1) / (kVecBlock * 4);
+    hipLaunchKernelGGL(vector_op_kernel<OP>, dim3((unsigned)blocks), dim3(kVecBlock), 0, static_cast<hipStream_t>(stream),
+                       dst, src0, src1, a, b, c, d, (size_t)size, aligned);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 }  // namespace
 
 
@@ -667,6 +686,40 @@ int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, floa
     BBHIP_REQUIRE(dev_dst != nullptr && dev_src != nullptr && size >= 0);
     if (size == 0) { return 0; }
     hipLaunchKernelGGL(clamp_kernel, dim3(ceil_div(size, kBlock)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, dev_src, lo, hi, size);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_Vector_add_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c, int size, void *stream)
+{ return vector_op<kVecAddEx>(dev_dst, dev_src0, dev_src1, a, b, c, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_mul_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, int size, void *stream)
+{ return vector_op<kVecMulEx>(dev_dst, dev_src0, dev_src1, a, b, 0.0f, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_div_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c, float d, int size, void *stream)
+{ return vector_op<kVecDivEx>(dev_dst, dev_src0, dev_src1, a, b, c, d, size, stream, __func__); }
+int bbhip_fp32_Vector_sqrt(float *dev_dst, float const *dev_src, int size, void *stream)
+{ return vector_op<kVecSqrt>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_exp(float *dev_dst, float const *dev_src, int size, void *stream)
+{ return vector_op<kVecExp>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_min(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream)
+{ return vector_op<kVecMin>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_min_v(float *dev_dst, float const *dev_src, float a, int size, void *stream)
+{ return vector_op<kVecMinV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_max(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream)
+{ return vector_op<kVecMax>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+int bbhip_fp32_Vector_max_v(float *dev_dst, float const *dev_src, float a, int size, void *stream)
+{ return vector_op<kVecMaxV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+
+int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
+                             float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
+{
+    BBHIP_REQUIRE(size >= 0 && size <= 65535);
+    if (size == 0) { return 0; }
+    BBHIP_REQUIRE(dev_size_table != nullptr && dev_params_buf_table != nullptr && dev_grads_buf_table != nullptr &&
+                  dev_m_buf_table != nullptr && dev_v_buf_table != nullptr);
+    // the element counts live on the device: a fixed number of blocks per tensor strides over its elements
+    hipLaunchKernelGGL(adam_kernel, dim3(kAdamBlocksPerTensor, (unsigned)size), dim3(kVecBlock), 0, static_cast<hipStream_t>(stream),
+                       dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table,
+                       lr_t, 1.0f - beta1, 1.0f - beta2);
     BBHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -36,6 +36,81 @@ def vector_set_(t, value):
     return t
 
 
+def _out(dst, like):
+    return torch.empty_like(like) if dst is None else dst
+
+
+def vector_add_ex(src0, src1, a=1.0, b=1.0, c=0.0, out=None):
+    """a * src0 + b * src1 + c"""
+    dst = _out(out, src0); _dev(src0, src1, dst)
+    check(lib().bbhip_fp32_Vector_add_ex(ptr(dst), ptr(src0), ptr(src1), a, b, c, src0.numel(), stream_ptr()))
+    return dst
+
+
+def vector_mul_ex(src0, src1, a=1.0, b=0.0, out=None):
+    """a * src0 * src1 + b"""
+    dst = _out(out, src0); _dev(src0, src1, dst)
+    check(lib().bbhip_fp32_Vector_mul_ex(ptr(dst), ptr(src0), ptr(src1), a, b, src0.numel(), stream_ptr()))
+    return dst
+
+
+def vector_div_ex(src0, src1, a=1.0, b=0.0, c=1.0, d=0.0, out=None):
+    """(a * src0 + b) / (c * src1 + d)"""
+    dst = _out(out, src0); _dev(src0, src1, dst)
+    check(lib().bbhip_fp32_Vector_div_ex(ptr(dst), ptr(src0), ptr(src1), a, b, c, d, src0.numel(), stream_ptr()))
+    return dst
+
+
+def vector_unary(name, src, out=None):
+    """name in {"sqrt", "exp"}"""
+    dst = _out(out, src); _dev(src, dst)
+    check(getattr(lib(), "bbhip_fp32_Vector_" + name)(ptr(dst), ptr(src), src.numel(), stream_ptr()))
+    return dst
+
+
+def vector_minmax(name, src0, src1, out=None):
+    """name in {"min", "max"}; src1 is a tensor or a Python float (the *_v entry points)"""
+    dst = _out(out, src0)
+    if isinstance(src1, torch.Tensor):
+        _dev(src0, src1, dst)
+        check(getattr(lib(), "bbhip_fp32_Vector_" + name)(ptr(dst), ptr(src0), ptr(src1), src0.numel(), stream_ptr()))
+    else:
+        _dev(src0, dst)
+        check(getattr(lib(), "bbhip_fp32_Vector_%s_v" % name)(ptr(dst), ptr(src0), float(src1), src0.numel(), stream_ptr()))
+    return dst
+
+
+class AdamState:
+    """Device-side tables of one parameter list for bbhip_fp32_OptimizerAdam, with the bias-correction products kept
+    on the host as the reference does (include/bb/OptimizerAdam.h:104-110, 166-180)."""
+
+    def __init__(self, params, grads, learning_rate=0.001, beta1=0.9, beta2=0.999):
+        import numpy as np
+        _dev(*params, *grads)
+        self.params, self.grads = list(params), list(grads)
+        self.m = [torch.zeros_like(p) for p in params]
+        self.v = [torch.zeros_like(p) for p in params]
+        dev = params[0].device
+        table = lambda ts: torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=dev)
+        self.t_params, self.t_grads, self.t_m, self.t_v = table(self.params), table(self.grads), table(self.m), table(self.v)
+        self.t_size = torch.tensor([p.numel() for p in params], dtype=torch.int32, device=dev)
+        f32 = np.float32
+        self.lr, self.beta1, self.beta2 = f32(learning_rate), f32(beta1), f32(beta2)
+        self.b1, self.b2 = f32(beta1), f32(beta2)
+
+    def lr_t(self):
+        import numpy as np
+        one = np.float32(1.0)
+        return np.float32(np.float32(self.lr * np.sqrt(one - self.b2, dtype=np.float32)) / (one - self.b1))
+
+    def step(self):
+        check(lib().bbhip_fp32_OptimizerAdam(len(self.params), ptr(self.t_size), ptr(self.t_params), ptr(self.t_grads),
+                                             ptr(self.t_m), ptr(self.t_v), float(self.lr_t()), float(self.beta1),
+                                             float(self.beta2), stream_ptr()))
+        self.b1 = self.b1 * self.beta1
+        self.b2 = self.b2 * self.beta2
+
+
 def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
     _dev(xbits)
     y = torch.empty((xbits.shape[0], y_stride), dtype=torch.float32, device=xbits.device)

@@ -82,6 +82,39 @@ int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream);
 /* bbcu_fp32_Vector_clamp, include/bbcu/bbcu.h:191-198 (W is clamped to [0,1] before every StochasticLut forward,
  * include/bb/StochasticLutN.h:451) */
 int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, float hi, int size, void *stream);
+/* bbcu_fp32_Vector_add_ex, include/bbcu/bbcu.h:96-107:  dst = a * src0 + b * src1 + c.
+ * These elementwise operations evaluate the reference's C++ expressions (include/bb/TensorOperator.h:41-238) in fp32
+ * operation by operation (no fused multiply-add); dst may alias a source. */
+int bbhip_fp32_Vector_add_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c,
+                             int size, void *stream);
+/* bbcu_fp32_Vector_mul_ex, include/bbcu/bbcu.h:109-119:  dst = a * src0 * src1 + b */
+int bbhip_fp32_Vector_mul_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b,
+                             int size, void *stream);
+/* bbcu_fp32_Vector_div_ex, include/bbcu/bbcu.h:121-132:  dst = (a * src0 + b) / (c * src1 + d) */
+int bbhip_fp32_Vector_div_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c,
+                             float d, int size, void *stream);
+/* bbcu_fp32_Vector_sqrt, include/bbcu/bbcu.h:134-140 (the reference launches one block of 1024 threads and so only
+ * handles the first 1024 elements, cuda/Vector.cu:233; here every element is processed, as on its CPU path) */
+int bbhip_fp32_Vector_sqrt(float *dev_dst, float const *dev_src, int size, void *stream);
+/* bbcu_fp32_Vector_exp, include/bbcu/bbcu.h:143-149 (same remark) */
+int bbhip_fp32_Vector_exp(float *dev_dst, float const *dev_src, int size, void *stream);
+/* bbcu_fp32_Vector_min / min_v / max / max_v, include/bbcu/bbcu.h:152-189; std::min / std::max semantics of the CPU
+ * path (include/bb/TensorOperator.h:170-222): a NaN in the second operand is dropped, in the first it propagates */
+int bbhip_fp32_Vector_min(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream);
+int bbhip_fp32_Vector_min_v(float *dev_dst, float const *dev_src, float a, int size, void *stream);
+int bbhip_fp32_Vector_max(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream);
+int bbhip_fp32_Vector_max_v(float *dev_dst, float const *dev_src, float a, int size, void *stream);
+
+/* ---- Adam ---- */
+/* bbcu_fp32_OptimizerAdam, include/bbcu/bbcu.h:1560-1572 (cuda/OptimizerAdam.cu:12-84).  One update of `size` tensors:
+ * the four pointer tables and the element-count table are DEVICE arrays of `size` entries.  lr_t is the
+ * bias-corrected rate the caller computes (include/bb/OptimizerAdam.h:171).  Per element, each step rounded to fp32:
+ *     m += (1-beta1)*(g - m);   v += (1-beta2)*(g*g - v);   p -= (lr_t*m) / (sqrt(v) + 1e-7)
+ * (the reference's host path, include/bb/OptimizerAdam.h:173-176; its CUDA kernel adds the 1e-7 in double). */
+int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *dev_params_buf_table,
+                             float *const *dev_grads_buf_table, float *const *dev_m_buf_table,
+                             float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream);
+
 /* bbcu_ConvBitToReal<float>, include/bbcu/bbcu.h:246-258 */
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
                              int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream);

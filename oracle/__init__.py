@@ -76,6 +76,38 @@ def vector_clamp(src, lo=0.0, hi=1.0):
     return dst
 
 
+_VEC_OPS = {"add_ex": 0, "mul_ex": 1, "div_ex": 2, "sqrt": 3, "exp": 4, "min": 5, "min_v": 6, "max": 7, "max_v": 8}
+
+
+def vector_op(name, src0, src1=None, a=0.0, b=0.0, c=0.0, d=0.0):
+    """Elementwise fp32 vector operation ``name`` of the reference's Tensor arithmetic."""
+    src0 = _c(src0, np.float32)
+    src1 = None if src1 is None else _c(src1, np.float32)
+    dst = np.empty_like(src0)
+    lib().oracle_fp32_Vector_op(C.c_int(_VEC_OPS[name]), _ptr(dst), _ptr(src0), _ptr(src1), C.c_float(a), C.c_float(b),
+                                C.c_float(c), C.c_float(d), C.c_int(src0.size))
+    return dst
+
+
+def adam_lr_t(learning_rate, b1, b2):
+    """Bias-corrected rate in fp32, as include/bb/OptimizerAdam.h:171 computes it."""
+    one = np.float32(1.0)
+    return np.float32(np.float32(np.float32(learning_rate) * np.sqrt(one - np.float32(b2), dtype=np.float32)) / (one - np.float32(b1)))
+
+
+def adam_steps(param, grads, learning_rate=0.001, beta1=0.9, beta2=0.999):
+    """Run len(grads) Adam updates on one tensor; returns (param, m, v) after the last step."""
+    p = _c(param, np.float32).copy()
+    m = np.zeros_like(p); v = np.zeros_like(p)
+    b1 = np.float32(beta1); b2 = np.float32(beta2)
+    for g in grads:
+        g = _c(g, np.float32)
+        lib().oracle_fp32_OptimizerAdam(C.c_int(p.size), _ptr(p), _ptr(g), _ptr(m), _ptr(v), C.c_float(adam_lr_t(learning_rate, b1, b2)),
+                                        C.c_float(beta1), C.c_float(beta2))
+        b1 = np.float32(b1 * np.float32(beta1)); b2 = np.float32(b2 * np.float32(beta2))
+    return p, m, v
+
+
 def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, simd=True):
     """fp32 x [I, stride] -> y [O, stride] (padding columns zero)."""
     x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
@@ -329,6 +361,26 @@ def ref_reverse_table6(idx, input_node_size):
 # ----------------------------------------------------------------------------------------------
 #  timed CPU baselines (used by bench.py only)
 # ----------------------------------------------------------------------------------------------
+
+def ref_adam_steps(param, grads, learning_rate=0.001, beta1=0.9, beta2=0.999):
+    """bb::OptimizerAdam<float> of the reference (host path): param after len(grads) updates."""
+    p = _c(param, np.float32).copy()
+    g = _c(np.stack([np.asarray(x, np.float32).ravel() for x in grads]), np.float32)
+    rc = ref().bbref_OptimizerAdam(C.c_int(p.size), C.c_int(g.shape[0]), _ptr(p), _ptr(g), C.c_float(learning_rate),
+                                   C.c_float(beta1), C.c_float(beta2))
+    assert rc == 0
+    return p
+
+
+def ref_vector_op(name, src0, src1=None, a=0.0, b=0.0, c=0.0, d=0.0):
+    src0 = _c(src0, np.float32)
+    src1 = None if src1 is None else _c(src1, np.float32)
+    dst = np.empty_like(src0)
+    rc = ref().bbref_Vector_op(C.c_int(_VEC_OPS[name]), _ptr(dst), _ptr(src0), _ptr(src1), C.c_float(a), C.c_float(b),
+                               C.c_float(c), C.c_float(d), C.c_int(src0.size))
+    assert rc == 0
+    return dst
+
 
 def time_stochastic_lut6(x, dy, idx, W, reps=3, use_ref=None):
     """Seconds per StochasticLut6 forward+backward on the host, one value per repetition (after one warm-up).

@@ -661,3 +661,46 @@ void oracle_fp32_StochasticLut6_Time(float const *x, float const *dy, int32_t co
     }
     free(y); free(dx); free(dW);
 }
+
+/* ------------------------------------------------------------------------------------------------
+ * Elementwise vector operations of the reference's Tensor arithmetic (include/bb/TensorOperator.h:41-238) and the
+ * Adam update (include/bb/OptimizerAdam.h:166-180, host path).  Evaluated in fp32 operation by operation (this file
+ * is built with -ffp-contract=off).  Pinned by: numpy closed forms in fp32 (tests/test_oracle.py), the reference's
+ * own Tensor operators and OptimizerAdam through oracle/_ref where it is built, the model in the reference's
+ * optimizer test (tests/gtest/OptimizerAdamTest.cpp:10-40) restated in the test, and tests/golden/adam.npz.
+ * op: 0 add_ex, 1 mul_ex, 2 div_ex, 3 sqrt, 4 exp, 5 min, 6 min_v, 7 max, 8 max_v (std::min / std::max semantics)
+ * ------------------------------------------------------------------------------------------------ */
+void oracle_fp32_Vector_op(int op, float *dst, float const *src0, float const *src1, float a, float b, float c, float d, int size)
+{
+    for (int i = 0; i < size; ++i) {
+        float const x = src0[i];
+        float const y = src1 ? src1[i] : 0.0f;
+        float r;
+        switch (op) {
+        case 0:  r = a * x + b * y + c; break;                       /* TensorOperator.h:54 */
+        case 1:  r = a * x * y + b; break;                           /* :91 */
+        case 2:  r = (a * x + b) / (c * y + d); break;               /* :110 */
+        case 3:  r = sqrtf(x); break;                                /* :137 */
+        case 4:  r = expf(x); break;                                 /* :164 */
+        case 5:  r = (y < x) ? y : x; break;                         /* :179 std::min(src0, src1) */
+        case 6:  r = (a < x) ? a : x; break;                         /* :193 */
+        case 7:  r = (x < y) ? y : x; break;                         /* :208 std::max(src0, src1) */
+        default: r = (x < a) ? a : x; break;                         /* :222 */
+        }
+        dst[i] = r;
+    }
+}
+
+/* One Adam step on one tensor; lr_t is computed by the caller as the reference does (OptimizerAdam.h:171). */
+void oracle_fp32_OptimizerAdam(int size, float *param, float const *grad, float *m, float *v, float lr_t, float beta1, float beta2)
+{
+    float const nb1 = 1.0f - beta1, nb2 = 1.0f - beta2;
+    for (int i = 0; i < size; ++i) {
+        float const g = grad[i];
+        float t = g - m[i];          t = nb1 * t;   m[i] = m[i] + t;          /* m += (1-b1)*(g - m)   :173 */
+        float u = g * g;  u = u - v[i]; u = nb2 * u; v[i] = v[i] + u;         /* v += (1-b2)*(g*g - v) :174 */
+        float num = lr_t * m[i];
+        float den = sqrtf(v[i]) + 1.0e-7f;
+        param[i] = param[i] - num / den;                                       /* p -= lr_t*m/(sqrt(v)+1e-7) :176 */
+    }
+}

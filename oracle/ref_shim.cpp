@@ -21,6 +21,8 @@
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
 #include "bb/FixedSizeConnectionTable.h"
+#include "bb/OptimizerAdam.h"
+#include "bb/TensorOperator.h"
 
 namespace {
 
@@ -285,6 +287,46 @@ int bbref_DefaultWiring6(int I, int O, std::uint64_t seed, std::int32_t *idx)
     lut->SetInputShape({(index_t)I});
     for (int nd = 0; nd < O; ++nd) for (int i = 0; i < 6; ++i) { idx[nd * 6 + i] = (std::int32_t)lut->GetNodeConnectionIndex(nd, i); }
     return 0;
+}
+
+
+// bb::OptimizerAdam<float> (host path, include/bb/OptimizerAdam.h:142-180): `steps` updates of one fp32 tensor of
+// `size` elements; grads is [steps][size]; param is updated in place.
+int bbref_OptimizerAdam(int size, int steps, float *param, float const *grads, float learning_rate, float beta1, float beta2)
+{
+    auto opt = bb::OptimizerAdam<float>::Create(learning_rate, beta1, beta2);
+    auto p = std::shared_ptr<bb::Tensor>(new bb::Tensor(bb::indices_t({(bb::index_t)size}), BB_TYPE_FP32, true));
+    auto g = std::shared_ptr<bb::Tensor>(new bb::Tensor(bb::indices_t({(bb::index_t)size}), BB_TYPE_FP32, true));
+    bb::Variables pv, gv;
+    pv.PushBack(p);
+    gv.PushBack(g);
+    opt->SetVariables(pv, gv);
+    { auto ptr = p->Lock<float>(); for (int i = 0; i < size; ++i) { ptr(i) = param[i]; } }
+    for (int s = 0; s < steps; ++s) {
+        { auto ptr = g->Lock<float>(); for (int i = 0; i < size; ++i) { ptr(i) = grads[(size_t)s * size + i]; } }
+        opt->Update();
+    }
+    { auto ptr = p->LockConst<float>(); for (int i = 0; i < size; ++i) { param[i] = ptr(i); } }
+    return 0;
+}
+
+// The reference's elementwise kernels of its Tensor arithmetic, host versions (include/bb/TensorOperator.h:41-238).
+// op: 0 add_ex, 1 mul_ex, 2 div_ex, 3 sqrt, 4 exp, 5 min, 6 min_v, 7 max, 8 max_v
+int bbref_Vector_op(int op, float *dst, float const *src0, float const *src1, float a, float b, float c, float d, int size)
+{
+    bb::index_t const n = size;
+    switch (op) {
+    case 0: bb::Tensor_Vector_add_ex<float>(dst, src0, src1, a, b, c, n); return 0;
+    case 1: bb::Tensor_Vector_mul_ex<float>(dst, src0, src1, a, b, n); return 0;
+    case 2: bb::Tensor_Vector_div_ex<float>(dst, src0, src1, a, b, c, d, n); return 0;
+    case 3: bb::Tensor_Vector_sqrt<float>(dst, src0, n); return 0;
+    case 4: bb::Tensor_Vector_exp<float>(dst, src0, n); return 0;
+    case 5: bb::Tensor_Vector_min<float>(dst, src0, src1, n); return 0;
+    case 6: bb::Tensor_Vector_min_v<float>(dst, src0, a, n); return 0;
+    case 7: bb::Tensor_Vector_max<float>(dst, src0, src1, n); return 0;
+    case 8: bb::Tensor_Vector_max_v<float>(dst, src0, a, n); return 0;
+    }
+    return -1;
 }
 
 }  // extern "C"

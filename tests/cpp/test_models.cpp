@@ -10,8 +10,10 @@
 #include "bb/StochasticLutN.h"
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
+#include "bb/OptimizerAdam.h"
 
 extern "C" {
+void oracle_fp32_OptimizerAdam(int size, float *param, float const *grad, float *m, float *v, float lr_t, float beta1, float beta2);
 void oracle_fp32_StochasticLut_Forward(int n, float const *x, float *y, std::int32_t const *idx, float const *W, int node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
 void oracle_fp32_StochasticLut_Backward(int n, float const *x, float const *dy, float *dx, std::int32_t const *idx, float const *W, float *dW, int input_node_size, int output_node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
 void oracle_fp32_DifferentiableLutN_ForwardTraining(int n, float const *x, float *y, std::int32_t const *idx, float const *W, float *mean, float *rstd, float *running_mean, float *running_var, float gamma, float beta, float momentum, float bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode);
@@ -186,6 +188,51 @@ static void test_import_layer(void)
     CHECK(mism == 0, "ImportLayer: %zu mismatching bits", mism);
 }
 
+// Shaped like the reference's optimizer test (tests/gtest/OptimizerAdamTest.cpp:44-96): parameters follow a model of the
+// update step by step; here the model is the CPU oracle and the list holds several tensors of different sizes.
+static void test_adam(void)
+{
+    float const lr = 0.001f, beta1 = 0.9f, beta2 = 0.999f;
+    int const sizes[] = {1, 70 * 64, 1024 * 64, 5};
+    auto opt = bb::OptimizerAdam<float>::Create(lr, beta1, beta2);
+    std::vector<std::shared_ptr<bb::Tensor>> params, grads;
+    bb::Variables pv, gv;
+    std::mt19937_64 mt(1);
+    std::normal_distribution<float> norm(0.0001f, 2.0f);
+    std::vector<std::vector<float>> p_ref, m_ref, v_ref;
+    for (int n : sizes) {
+        auto p = std::make_shared<bb::Tensor>(bb::indices_t({(bb::index_t)n}), BB_TYPE_FP32);
+        auto g = std::make_shared<bb::Tensor>(bb::indices_t({(bb::index_t)n}), BB_TYPE_FP32);
+        std::vector<float> init((size_t)n);
+        { auto ptr = p->Lock<float>(true); for (int i = 0; i < n; ++i) { init[(size_t)i] = ptr[i] = 0.1f + 0.001f * (float)(i % 97); } }
+        g->FillZero();
+        params.push_back(p); grads.push_back(g); pv.PushBack(p); gv.PushBack(g);
+        p_ref.push_back(init); m_ref.emplace_back((size_t)n, 0.0f); v_ref.emplace_back((size_t)n, 0.0f);
+    }
+    opt->SetVariables(pv, gv);
+    float b1 = beta1, b2 = beta2;
+    for (int step = 0; step < 10; ++step) {
+        float const lr_t = lr * std::sqrt(1.0f - b2) / (1.0f - b1);
+        for (size_t t = 0; t < params.size(); ++t) {
+            int const n = sizes[t];
+            std::vector<float> g((size_t)n);
+            for (auto &x : g) { x = norm(mt); }
+            { auto ptr = grads[t]->Lock<float>(true); for (int i = 0; i < n; ++i) { ptr[i] = g[(size_t)i]; } }
+            oracle_fp32_OptimizerAdam(n, p_ref[t].data(), g.data(), m_ref[t].data(), v_ref[t].data(), lr_t, beta1, beta2);
+        }
+        opt->Update();
+        b1 *= beta1; b2 *= beta2;
+        for (size_t t = 0; t < params.size(); ++t) {
+            auto ptr = params[t]->LockConst<float>();
+            size_t bad = 0;
+            for (int i = 0; i < sizes[t]; ++i) { bad += (ptr[i] != p_ref[t][(size_t)i]); }
+            CHECK(bad == 0, "Adam step %d tensor %zu: %zu of %d parameters differ from the oracle", step, t, bad, sizes[t]);
+            auto gp = grads[t]->LockConst<float>();
+            CHECK(gp[0] == 0.0f && gp[sizes[t] - 1] == 0.0f, "Update must clear the gradients");
+        }
+    }
+}
+
 int main(void)
 {
     if (!bb::Manager::IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
@@ -210,6 +257,7 @@ int main(void)
         test_binary(16, 16, 32);
         test_binary(70, 33, 1000);
         test_import_layer();
+        test_adam();
     }
     catch (std::exception const &e) {
         std::printf("exception: %s\n", e.what());

@@ -108,11 +108,45 @@ def binary_cases():
     np.savez_compressed(os.path.join(OUT, "binary_lut6.npz"), **cases)
 
 
+def adam_cases():
+    """bb::OptimizerAdam<float> and the elementwise Tensor kernels of the reference (host path)."""
+    rng = np.random.default_rng(20240604)
+    cases = {}
+    k = 0
+    for (size, steps, lr, b1, b2) in [(1, 10, 0.001, 0.9, 0.999), (257, 12, 0.001, 0.9, 0.999), (64, 5, 0.01, 0.8, 0.99)]:
+        p0 = rng.standard_normal(size).astype(np.float32)
+        g = (rng.standard_normal((steps, size)) * 2.0 + 0.0001).astype(np.float32)
+        if size > 8:
+            g[:, 3] = 0.0                                   # a parameter that never receives a gradient
+        p1 = oracle.ref_adam_steps(p0, list(g), lr, b1, b2)
+        q = "a%d_" % k
+        cases.update({q + "hyper": np.array([lr, b1, b2], np.float64), q + "p0": p0, q + "g": g, q + "p": p1})
+        k += 1
+    cases["adam_count"] = np.array([k], np.int32)
+    x = (rng.standard_normal(301) * 3.0).astype(np.float32)
+    y = (rng.standard_normal(301) * 3.0).astype(np.float32)
+    pos = np.abs(x) + np.float32(0.01)
+    cases.update({"vx": x, "vy": y, "vpos": pos, "coef": np.array([1.5, -0.75, 0.25, 2.0], np.float32)})
+    a, b, c, d = [float(v) for v in cases["coef"]]
+    cases["add_ex"] = oracle.ref_vector_op("add_ex", x, y, a, b, c)
+    cases["mul_ex"] = oracle.ref_vector_op("mul_ex", x, y, a, b)
+    cases["div_ex"] = oracle.ref_vector_op("div_ex", x, pos, a, b, c, d)
+    cases["sqrt"] = oracle.ref_vector_op("sqrt", pos)
+    cases["exp"] = oracle.ref_vector_op("exp", x)
+    cases["min"] = oracle.ref_vector_op("min", x, y)
+    cases["min_v"] = oracle.ref_vector_op("min_v", x, None, 0.3)
+    cases["max"] = oracle.ref_vector_op("max", x, y)
+    cases["max_v"] = oracle.ref_vector_op("max_v", x, None, 0.3)
+    np.savez_compressed(os.path.join(OUT, "adam.npz"), **cases)
+
+
 if __name__ == "__main__":
     assert oracle.have_ref(), "build oracle/_ref first (make -C oracle ref)"
-    stochastic_cases()
-    differentiable_cases()
-    binary_cases()
+    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam"]
+    if "stochastic" in which: stochastic_cases()
+    if "differentiable" in which: differentiable_cases()
+    if "binary" in which: binary_cases()
+    if "adam" in which: adam_cases()
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)), "bytes")
