@@ -101,6 +101,61 @@ def bench_adam(args, lib):
     print(json.dumps(out))
 
 
+def bench_conv(args, lib):
+    """The permutation kernels around the LUT layers of a conv block (secondary measurement), at the shapes of the
+    CIFAR-like configuration: 256 images of 3 x 32 x 32, 3 x 3 valid filter (27 taps, 230400 window frames), 36 output
+    channels of 30 x 30, 2 x 2 pooling.  Algorithmic bytes: every element of input and output once."""
+    import torch
+    from binarybrain_amd import ops, synth
+    F, C, H, W, FH, FW, CO = 256, 3, 32, 32, 3, 3, 36
+    OH, OW = H - FH + 1, W - FW + 1
+    g = torch.Generator(device="cuda"); g.manual_seed(0)
+    img = torch.rand((C * H * W, synth.frame_stride_fp32(F)), device="cuda", generator=g)
+    cols = ops.im2col_forward(img, C, H, W, F, FH, FW)
+    dcols = torch.rand_like(cols)
+    act = torch.rand((CO, synth.frame_stride_fp32(F * OH * OW)), device="cuda", generator=g)
+    maps = ops.col2im_forward(act, CO, OH, OW, F)
+    dmaps = torch.rand_like(maps)
+    pooled = ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F)
+    dpooled = torch.rand_like(pooled)
+    e = 4
+    cases = [
+        ("im2col_forward_kernel", lambda: ops.im2col_forward(img, C, H, W, F, FH, FW), e * F * (C * H * W + C * FH * FW * OH * OW)),
+        ("im2col_backward_kernel", lambda: ops.im2col_backward(dcols, C, H, W, F, FH, FW), e * F * (C * H * W + C * FH * FW * OH * OW)),
+        ("col2im_kernel<forward>", lambda: ops.col2im_forward(act, CO, OH, OW, F), 2 * e * F * CO * OH * OW),
+        ("col2im_kernel<backward>", lambda: ops.col2im_backward(dmaps, CO, OH, OW, F), 2 * e * F * CO * OH * OW),
+        ("stochastic_maxpool2x2_forward_kernel", lambda: ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F), e * F * CO * (OH * OW + (OH // 2) * (OW // 2))),
+        ("stochastic_maxpool2x2_backward_kernel", lambda: ops.stochastic_maxpool2x2_backward(maps, dpooled, CO, OH, OW, F),
+         e * F * CO * (2 * OH * OW + (OH // 2) * (OW // 2))),
+    ]
+    kernels = {}
+    total_ms = 0.0
+    for name, fn, nbytes in cases:
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        # the wrappers allocate their result from torch's caching allocator (no device call): events around single launches
+        ms = []
+        for _ in range(args.steps):
+            e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+            out = fn(); del out
+            torch.cuda.synchronize()
+            e0.record(); out = fn(); e1.record(); torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        med = sorted(ms)[len(ms) // 2]
+        total_ms += med
+        kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
+    dom = max(kernels, key=lambda k: kernels[k]["ms"])
+    out = {"metric": "conv-block permutation kernels, ms per pass over 256 images (fwd+bwd)", "value": total_ms, "unit": "ms",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": total_ms, "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "Im2Col 3x32x32 (3x3 valid) / Col2Im 36x30x30 / StochasticMaxPooling2x2, 256 images"},
+           "roofline": {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},
+           "kernels": kernels}
+    print(json.dumps(out))
+
+
 def bench_binarylut6(args, lib):
     """BinaryLut6 packed inference: 8192 -> 16384 nodes, 262144 frames, 32 frames per word (secondary measurement)."""
     import numpy as np
@@ -172,7 +227,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "adam"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "adam", "conv"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -191,6 +246,8 @@ def main():
         return bench_binarylut6(args, lib)
     if args.workload == "adam":
         return bench_adam(args, lib)
+    if args.workload == "conv":
+        return bench_conv(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)

@@ -44,6 +44,14 @@ _SIGNATURES = {
     "bbhip_fp32_Vector_max": (C.c_int, [_vp, _vp, _vp, _i, _vp]),
     "bbhip_fp32_Vector_max_v": (C.c_int, [_vp, _vp, _f, _i, _vp]),
     "bbhip_fp32_OptimizerAdam": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _vp]),
+    "bbhip_fp32_Im2Col_Forward": (C.c_int, [_vp, _vp] + [_i] * 15 + [_f, _vp]),
+    "bbhip_bit_Im2Col_Forward": (C.c_int, [_vp, _vp] + [_i] * 15 + [_vp]),
+    "bbhip_fp32_Im2Col_Backward": (C.c_int, [_vp, _vp] + [_i] * 14 + [_vp]),
+    "bbhip_fp32_Col2Im_Forward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_bit_Col2Im_Forward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_fp32_Col2Im_Backward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_fp32_StochasticMaxPooling2x2_Forward": (C.c_int, [_vp, _vp] + [_i] * 7 + [_vp]),
+    "bbhip_fp32_StochasticMaxPooling2x2_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 7 + [_vp]),
     "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "bbhip_bit_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),

@@ -15,6 +15,7 @@
 #include "../../include/bbhip.h"
 #include "lut_kernels.hpp"
 #include "vector_kernels.hpp"
+#include "conv_kernels.hpp"
 
 using namespace bbhip;
 
@@ -546,6 +547,29 @@ struct LocalHeap {
 
 LocalHeap &heap(void) { static LocalHeap h; return h; }
 
+int check_im2col(Im2ColArgs const &a, bool bit, char const *name)
+{
+    if (!(a.x && a.y)) { return fail("%s: null buffer", name); }
+    if (!(a.c > 0 && a.h > 0 && a.w > 0 && a.fh > 0 && a.fw > 0 && a.oh > 0 && a.ow > 0 && a.input_frame_size > 0)) {
+        return fail("%s: sizes must be positive", name);
+    }
+    if (!(a.x_stride > 0 && a.y_stride > 0 && a.x_offset >= 0 && a.y_offset >= 0)) { return fail("%s: bad stride or offset", name); }
+    if (a.border_mode < 0 || a.border_mode > 4) { return fail("%s: border_mode=%d not in 0..4", name, a.border_mode); }
+    // border modes fold an out-of-range tap back once: it must land inside the image
+    if (a.border_mode != 0 &&
+        (a.x_offset >= a.w || a.y_offset >= a.h || a.fw - 1 - a.x_offset + (a.ow - 1) * a.x_stride > 2 * a.w - 2 ||
+         a.fh - 1 - a.y_offset + (a.oh - 1) * a.y_stride > 2 * a.h - 2)) {
+        return fail("%s: filter reaches a full image size beyond the border", name);
+    }
+    long long const out_frames = (long long)a.input_frame_size * a.oh * a.ow;
+    if (out_frames > 0x7fffffffLL) { return fail("%s: %lld output frames do not fit an int", name, out_frames); }
+    long long const in_need  = bit ? (a.input_frame_size + 31) / 32 : a.input_frame_size;
+    long long const out_need = bit ? (out_frames + 31) / 32 : out_frames;
+    if (a.input_frame_stride < in_need || a.output_frame_stride < out_need) { return fail("%s: frame stride shorter than the frames", name); }
+    if ((long long)a.c * a.h * a.w > 0x7fffffffLL || (long long)a.c * a.fh * a.fw > 0x7fffffffLL) { return fail("%s: too many nodes", name); }
+    return 0;
+}
+
 constexpr int kAdamBlocksPerTensor = 1024;
 
 template <int OP>
@@ -722,6 +746,145 @@ int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *
                        lr_t, 1.0f - beta1, 1.0f - beta2);
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+
+int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
+                              int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size,
+                              int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
+                              int border_mode, float border_value, void *stream)
+{
+    Im2ColArgs a{dev_x_buf, dev_y_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
+                 input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
+                 border_mode, border_value, 0, 0};
+    if (check_im2col(a, false, __func__)) { return 1; }
+    a.ox_tiles = ceil_div(a.ow, kTile);
+    a.f_tiles  = ceil_div(a.input_frame_size, kTile);
+    long long const blocks = (long long)a.c * a.fh * a.fw * a.oh * a.ox_tiles * a.f_tiles;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(im2col_forward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_bit_Im2Col_Forward(int const *dev_x_buf, int *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
+                             int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size,
+                             int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
+                             int border_mode, void *stream)
+{
+    Im2ColArgs a{dev_x_buf, dev_y_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
+                 input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
+                 border_mode, 0.0f, 0, 0};
+    if (check_im2col(a, true, __func__)) { return 1; }
+    long long const out_frames = (long long)a.input_frame_size * a.oh * a.ow;
+    int const words = (int)((out_frames + 31) / 32);
+    long long const total = (long long)a.c * a.fh * a.fw * words;
+    long long const blocks = (total + kConvBlock - 1) / kConvBlock;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(im2col_forward_bit_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, words, total);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_Im2Col_Backward(float const *dev_dy_buf, float *dev_dx_buf, int x_stride, int y_stride, int x_offset, int y_offset,
+                               int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size,
+                               int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
+                               void *stream)
+{
+    Im2ColArgs a{dev_dy_buf, dev_dx_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
+                 input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
+                 0, 0.0f, 0, 0};
+    if (check_im2col(a, false, __func__)) { return 1; }
+    int const x_tiles = ceil_div(a.w, kTile);
+    a.f_tiles = ceil_div(a.input_frame_size, kTile);
+    long long const blocks = (long long)a.c * a.h * x_tiles * a.f_tiles;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(im2col_backward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, x_tiles);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int check_col2im(void const *p, void const *q, int w, int h, int c, int narrow_stride, int frames, int wide_stride, bool bit, char const *name)
+{
+    if (!(p && q)) { return fail("%s: null buffer", name); }
+    if (!(w > 0 && h > 0 && c > 0 && frames > 0)) { return fail("%s: sizes must be positive", name); }
+    long long const narrow = (long long)frames * h * w;
+    if (narrow > 0x7fffffffLL) { return fail("%s: %lld input frames do not fit an int", name, narrow); }
+    if (narrow_stride < (bit ? (narrow + 31) / 32 : narrow) || wide_stride < (bit ? (frames + 31) / 32 : frames)) {
+        return fail("%s: frame stride shorter than the frames", name);
+    }
+    if ((long long)c * h * w > 0x7fffffffLL) { return fail("%s: too many nodes", name); }
+    return 0;
+}
+
+int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
+                              int output_frame_size, int output_frame_stride, void *stream)
+{
+    if (check_col2im(dev_x_buf, dev_y_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, false, __func__)) { return 1; }
+    int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
+    long long const blocks = (long long)c_size * xy_tiles * f_tiles;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(col2im_kernel<true>, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream),
+                       dev_x_buf, dev_y_buf, hw, c_size, input_frame_stride, output_frame_size, output_frame_stride, xy_tiles, f_tiles);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w_size, int h_size, int c_size, int input_frame_stride,
+                               int output_frame_size, int output_frame_stride, void *stream)
+{
+    if (check_col2im(dev_dy_buf, dev_dx_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, false, __func__)) { return 1; }
+    int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
+    long long const blocks = (long long)c_size * xy_tiles * f_tiles;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(col2im_kernel<false>, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream),
+                       dev_dy_buf, dev_dx_buf, hw, c_size, input_frame_stride, output_frame_size, output_frame_stride, xy_tiles, f_tiles);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_bit_Col2Im_Forward(int const *dev_x_buf, int *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
+                             int output_frame_size, int output_frame_stride, void *stream)
+{
+    if (check_col2im(dev_x_buf, dev_y_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, true, __func__)) { return 1; }
+    int const hw = h_size * w_size, words = (output_frame_size + 31) / 32;
+    long long const total = (long long)c_size * hw * words;
+    long long const blocks = (total + kConvBlock - 1) / kConvBlock;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(col2im_forward_bit_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<uint32_t const *>(dev_x_buf), reinterpret_cast<uint32_t *>(dev_y_buf), hw, input_frame_stride,
+                       output_frame_size, output_frame_stride, words, total);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int launch_pool(PoolArgs const &a, bool backward, void *stream, char const *name)
+{
+    if (!(a.x && a.out && (a.dy || !backward))) { return fail("%s: null buffer", name); }
+    if (!(a.w > 0 && a.h > 0 && a.c > 0 && a.frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (a.ow != (a.w + 1) / 2 || a.oh != (a.h + 1) / 2) { return fail("%s: output size must be ceil(input / 2)", name); }
+    if (a.frame_stride < a.frame_size) { return fail("%s: frame stride shorter than the frames", name); }
+    int const f_blocks = ceil_div(a.frame_size, kConvBlock);
+    long long const blocks = (long long)a.c * a.oh * a.ow * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    if (backward) { hipLaunchKernelGGL(stochastic_maxpool2x2_backward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, f_blocks); }
+    else          { hipLaunchKernelGGL(stochastic_maxpool2x2_forward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, f_blocks); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_StochasticMaxPooling2x2_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size,
+                                               int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride, void *stream)
+{
+    PoolArgs a{dev_x_buf, nullptr, dev_y_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
+    return launch_pool(a, false, stream, __func__);
+}
+
+int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int input_w_size,
+                                                int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                                int frame_stride, void *stream)
+{
+    PoolArgs a{dev_x_buf, dev_dy_buf, dev_dx_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
+    return launch_pool(a, true, stream, __func__);
 }
 
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,

@@ -1,0 +1,284 @@
+// Convolution plumbing around the LUT layers: Im2Col, Col2Im, StochasticMaxPooling2x2.
+//
+// A convolution in this framework is Im2Col -> LUT layers -> Col2Im: Im2Col turns every filter window position of every
+// image into its own frame (frame' = (frame, oy, ox), node' = (c, fy, fx)), Col2Im turns them back into pixels
+// (node = (c, y, x)).  Both are permutations between the pixel index and the frame index of node-major, frame-minor
+// buffers, i.e. transposes whose two sides are contiguous along different indices.  The fp32 kernels stage 64 x 64
+// tiles through LDS so that reads and writes are both made of contiguous runs; the packed-bit kernels assemble each
+// output word from 32 single-bit gathers.  (Reference semantics: the host paths of include/bb/ConvolutionIm2Col.h:370-452,
+// ConvolutionCol2Im.h:203-293, StochasticMaxPooling2x2.h:190-306.)
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "vector_kernels.hpp"
+
+namespace bbhip {
+
+constexpr int kConvBlock = 256;
+constexpr int kTile = 64;
+
+struct Im2ColArgs {
+    void const *x;          // [c*h*w][input_frame_stride]
+    void       *y;          // [c*fh*fw][output_frame_stride], frames*oh*ow frames
+    int x_stride, y_stride, x_offset, y_offset;
+    int input_frame_size, input_frame_stride;
+    int w, h, c, ow, oh, output_frame_stride, fw, fh;
+    int border_mode;
+    float border_value;
+    int ox_tiles, f_tiles;
+};
+
+// include/bb/ConvolutionIm2Col.h:251-286
+__device__ __forceinline__ bool im2col_border(int mode, int &x, int &y, int w, int h)
+{
+    switch (mode) {
+    case 1: if (x < 0) { x = -x - 1; } if (y < 0) { y = -y - 1; } if (x >= w) { x = (w - 1) - (x - w); } if (y >= h) { y = (h - 1) - (y - h); } return true;
+    case 2: if (x < 0) { x = -x; }     if (y < 0) { y = -y; }     if (x >= w) { x = (w - 2) - (x - w); } if (y >= h) { y = (h - 2) - (y - h); } return true;
+    case 3: if (x < 0) { x = 0; }      if (y < 0) { y = 0; }      if (x >= w) { x = w - 1; }             if (y >= h) { y = h - 1; }             return true;
+    case 4: if (x < 0) { x += w; }     if (y < 0) { y += h; }     if (x >= w) { x -= w; }                if (y >= h) { y -= h; }                return true;
+    default: return false;
+    }
+}
+
+// input pixel of window position (oy, ox), tap (fy, fx); false = the constant border value applies
+__device__ __forceinline__ bool im2col_source(Im2ColArgs const &a, int oy, int ox, int fy, int fx, int &iy, int &ix)
+{
+    iy = oy * a.y_stride - a.y_offset + fy;
+    ix = ox * a.x_stride - a.x_offset + fx;
+    if (iy >= 0 && iy < a.h && ix >= 0 && ix < a.w) { return true; }
+    return im2col_border(a.border_mode, ix, iy, a.w, a.h);
+}
+
+// block = (output node, oy, 64 window columns, 64 input frames)
+__global__ __launch_bounds__(kConvBlock) void im2col_forward_kernel(Im2ColArgs a)
+{
+    __shared__ float tile[kTile][kTile + 1];                 // [ox][frame]
+    int b = blockIdx.x;
+    int const ft = b % a.f_tiles;  b /= a.f_tiles;
+    int const xt = b % a.ox_tiles; b /= a.ox_tiles;
+    int const oy = b % a.oh;       b /= a.oh;
+    int const node = b;                                      // (c*fh + fy)*fw + fx
+    int const fx = node % a.fw, fy = (node / a.fw) % a.fh, c = node / (a.fw * a.fh);
+    int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int const f0 = ft * kTile, ox0 = xt * kTile;
+    float const *x = static_cast<float const *>(a.x);
+    float *y = static_cast<float *>(a.y);
+
+    for (int i = wave; i < kTile; i += kConvBlock / 64) {
+        int const ox = ox0 + i;
+        if (ox >= a.ow) { break; }
+        int iy, ix;
+        bool const have = im2col_source(a, oy, ox, fy, fx, iy, ix);      // wave-uniform
+        float v = a.border_value;
+        if (have && f0 + lane < a.input_frame_size) {
+            v = x[((size_t)(c * a.h + iy) * a.w + ix) * a.input_frame_stride + f0 + lane];
+        }
+        tile[i][lane] = v;
+    }
+    __syncthreads();
+    size_t const plane = (size_t)a.oh * a.ow;
+    for (int f = wave; f < kTile; f += kConvBlock / 64) {
+        if (f0 + f >= a.input_frame_size) { break; }
+        if (ox0 + lane < a.ow) {
+            y[(size_t)node * a.output_frame_stride + (size_t)(f0 + f) * plane + (size_t)oy * a.ow + ox0 + lane] = tile[lane][f];
+        }
+    }
+}
+
+// one thread per output word (32 consecutive output frames of one node)
+__global__ __launch_bounds__(kConvBlock) void im2col_forward_bit_kernel(Im2ColArgs a, int words_per_node, long long total_words)
+{
+    long long const t = (long long)blockIdx.x * kConvBlock + threadIdx.x;
+    if (t >= total_words) { return; }
+    int const wd = (int)(t % words_per_node);
+    int const node = (int)(t / words_per_node);
+    int const fx = node % a.fw, fy = (node / a.fw) % a.fh, c = node / (a.fw * a.fh);
+    uint32_t const *x = static_cast<uint32_t const *>(a.x);
+    long long const plane = (long long)a.oh * a.ow;
+    long long const frames = (long long)a.input_frame_size * plane;
+    uint32_t out = 0;
+    for (int bit = 0; bit < 32; ++bit) {
+        long long const of = (long long)wd * 32 + bit;
+        if (of >= frames) { break; }
+        int const in_frame = (int)(of / plane);
+        int const f = (int)(of % plane);
+        int iy, ix;
+        if (im2col_source(a, f / a.ow, f % a.ow, fy, fx, iy, ix)) {
+            uint32_t const word = x[((size_t)(c * a.h + iy) * a.w + ix) * a.input_frame_stride + (in_frame >> 5)];
+            out |= ((word >> (in_frame & 31)) & 1u) << bit;
+        }
+    }
+    static_cast<uint32_t *>(a.y)[(size_t)node * a.output_frame_stride + wd] = out;
+}
+
+// dx[(c, y, x)][f] = sum over the taps (fy, fx) whose window holds (y, x), in (fy, fx) order, of dy[(c, fy, fx)][(f, oy, ox)]
+// (include/bb/ConvolutionIm2Col.h:411-452: border replicas carry no gradient).  block = (c, y, 64 columns, 64 frames);
+// the sums are formed with one lane per column (runs along ox are contiguous in dy) and transposed through LDS.
+__global__ __launch_bounds__(kConvBlock) void im2col_backward_kernel(Im2ColArgs a, int x_tiles)
+{
+    __shared__ float tile[kTile][kTile + 1];                 // [x][frame]
+    int b = blockIdx.x;
+    int const ft = b % a.f_tiles; b /= a.f_tiles;
+    int const xt = b % x_tiles;   b /= x_tiles;
+    int const y  = b % a.h;       b /= a.h;
+    int const c  = b;
+    int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int const f0 = ft * kTile, x0 = xt * kTile;
+    int const x = x0 + lane;
+    float const *dy = static_cast<float const *>(a.x);       // the gradient buffer comes in through the first slot
+    float *dx = static_cast<float *>(a.y);
+    constexpr int kPer = kTile / (kConvBlock / 64);          // frames per thread
+    float acc[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) { acc[j] = 0.0f; }
+
+    int const iy_limit = (a.oh - 1) * a.y_stride, ix_limit = (a.ow - 1) * a.x_stride;
+    size_t const plane = (size_t)a.oh * a.ow;
+    if (x < a.w) {
+        int const x_align = x % a.x_stride, y_align = y % a.y_stride;
+        for (int fy = y_align; fy < a.fh; fy += a.y_stride) {
+            int const iy = y - fy + a.y_offset;
+            if (iy < 0 || iy > iy_limit) { continue; }
+            for (int fx = x_align; fx < a.fw; fx += a.x_stride) {
+                int const ix = x - fx + a.x_offset;
+                if (ix < 0 || ix > ix_limit) { continue; }
+                float const *row = dy + (size_t)((c * a.fh + fy) * a.fw + fx) * a.output_frame_stride
+                                      + (size_t)(iy / a.y_stride) * a.ow + (ix / a.x_stride);
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) {
+                    int const f = f0 + wave + j * (kConvBlock / 64);
+                    if (f < a.input_frame_size) { acc[j] += row[(size_t)f * plane]; }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) { tile[lane][wave + j * (kConvBlock / 64)] = acc[j]; }
+    __syncthreads();
+    for (int i = wave; i < kTile; i += kConvBlock / 64) {
+        if (x0 + i >= a.w) { break; }
+        if (f0 + lane < a.input_frame_size) {
+            dx[((size_t)(c * a.h + y) * a.w + x0 + i) * a.input_frame_stride + f0 + lane] = tile[i][lane];
+        }
+    }
+}
+
+// y[(c, xy)][f] = x[c][f*hw + xy]  (forward)  /  dx[c][f*hw + xy] = dy[(c, xy)][f]  (backward): a [frames][hw] <-> [hw][frames]
+// transpose per channel.  block = (c, 64 pixels, 64 frames).  `narrow` is the [c][frames*hw] side, `wide` the [c*hw][frames] side.
+template <bool FORWARD>
+__global__ __launch_bounds__(kConvBlock) void col2im_kernel(float const *__restrict__ src, float *__restrict__ dst, int hw, int c_size,
+                                                           int narrow_stride, int frames, int wide_stride, int xy_tiles, int f_tiles)
+{
+    __shared__ float tile[kTile][kTile + 1];
+    int b = blockIdx.x;
+    int const ft = b % f_tiles;  b /= f_tiles;
+    int const xt = b % xy_tiles; b /= xy_tiles;
+    int const c = b;
+    int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int const f0 = ft * kTile, xy0 = xt * kTile;
+    if (FORWARD) {
+        for (int f = wave; f < kTile && f0 + f < frames; f += kConvBlock / 64) {          // lanes along xy: contiguous in src
+            if (xy0 + lane < hw) { tile[f][lane] = src[(size_t)c * narrow_stride + (size_t)(f0 + f) * hw + xy0 + lane]; }
+        }
+        __syncthreads();
+        for (int i = wave; i < kTile && xy0 + i < hw; i += kConvBlock / 64) {             // lanes along frames: contiguous in dst
+            if (f0 + lane < frames) { dst[((size_t)c * hw + xy0 + i) * wide_stride + f0 + lane] = tile[lane][i]; }
+        }
+    }
+    else {
+        for (int i = wave; i < kTile && xy0 + i < hw; i += kConvBlock / 64) {
+            if (f0 + lane < frames) { tile[i][lane] = src[((size_t)c * hw + xy0 + i) * wide_stride + f0 + lane]; }
+        }
+        __syncthreads();
+        for (int f = wave; f < kTile && f0 + f < frames; f += kConvBlock / 64) {
+            if (xy0 + lane < hw) { dst[(size_t)c * narrow_stride + (size_t)(f0 + f) * hw + xy0 + lane] = tile[lane][f]; }
+        }
+    }
+}
+
+// one thread per output word of the [c*hw][frames] side
+__global__ __launch_bounds__(kConvBlock) void col2im_forward_bit_kernel(uint32_t const *__restrict__ x, uint32_t *__restrict__ y, int hw,
+                                                                       int input_frame_stride, int frames, int output_frame_stride,
+                                                                       int words_per_node, long long total_words)
+{
+    long long const t = (long long)blockIdx.x * kConvBlock + threadIdx.x;
+    if (t >= total_words) { return; }
+    int const wd = (int)(t % words_per_node);
+    long long const node = t / words_per_node;           // c*hw + xy
+    int const xy = (int)(node % hw);
+    long long const c = node / hw;
+    uint32_t out = 0;
+    for (int bit = 0; bit < 32; ++bit) {
+        int const f = wd * 32 + bit;
+        if (f >= frames) { break; }
+        long long const in_frame = (long long)f * hw + xy;
+        uint32_t const word = x[(size_t)c * input_frame_stride + (in_frame >> 5)];
+        out |= ((word >> (in_frame & 31)) & 1u) << bit;
+    }
+    y[(size_t)node * output_frame_stride + wd] = out;
+}
+
+struct PoolArgs {
+    float const *x;
+    float const *dy;
+    float       *out;       // y (forward) or dx (backward)
+    int w, h, ow, oh, c, frame_size, frame_stride;
+};
+
+// y = 1 - prod over the window taps inside the image, (fy, fx) ascending, of (1 - x): the probability that at least one
+// of four independent binary inputs is 1 (include/bb/StochasticMaxPooling2x2.h:190-218).  One thread per (output node, frame).
+__global__ __launch_bounds__(kConvBlock) void stochastic_maxpool2x2_forward_kernel(PoolArgs a, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kConvBlock + threadIdx.x;
+    int const node = blockIdx.x / f_blocks;
+    if (f >= a.frame_size) { return; }
+    int const ox = node % a.ow, oy = (node / a.ow) % a.oh, c = node / (a.ow * a.oh);
+    float out = 1.0f;
+#pragma unroll
+    for (int fy = 0; fy < 2; ++fy) {
+#pragma unroll
+        for (int fx = 0; fx < 2; ++fx) {
+            int const iy = oy * 2 + fy, ix = ox * 2 + fx;
+            // the product is rounded on its own (not fused into the final 1 - out)
+            if (iy < a.h && ix < a.w) { out = rounded_mul(out, 1.0f - a.x[((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride + f]); }
+        }
+    }
+    a.out[(size_t)node * a.frame_stride + f] = 1.0f - out;
+}
+
+// dx of each tap = dy * prod over the other three taps of (1 - x), the product evaluated in double and rounded once, taps
+// outside the image reading as 0 (include/bb/StochasticMaxPooling2x2.h:262-306)
+__global__ __launch_bounds__(kConvBlock) void stochastic_maxpool2x2_backward_kernel(PoolArgs a, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kConvBlock + threadIdx.x;
+    int const node = blockIdx.x / f_blocks;
+    if (f >= a.frame_size) { return; }
+    int const ox = node % a.ow, oy = (node / a.ow) % a.oh, c = node / (a.ow * a.oh);
+    double in[2][2] = {{0.0, 0.0}, {0.0, 0.0}};
+#pragma unroll
+    for (int fy = 0; fy < 2; ++fy) {
+#pragma unroll
+        for (int fx = 0; fx < 2; ++fx) {
+            int const iy = oy * 2 + fy, ix = ox * 2 + fx;
+            if (iy < a.h && ix < a.w) { in[fy][fx] = (double)a.x[((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride + f]; }
+        }
+    }
+    double const g = (double)a.dy[(size_t)node * a.frame_stride + f];
+    float gr[2][2];
+    gr[0][0] = (float)(g * (1.0 - in[0][1]) * (1.0 - in[1][0]) * (1.0 - in[1][1]));
+    gr[0][1] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[1][0]) * (1.0 - in[1][1]));
+    gr[1][0] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[0][1]) * (1.0 - in[1][1]));
+    gr[1][1] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[0][1]) * (1.0 - in[1][0]));
+#pragma unroll
+    for (int fy = 0; fy < 2; ++fy) {
+#pragma unroll
+        for (int fx = 0; fx < 2; ++fx) {
+            int const iy = oy * 2 + fy, ix = ox * 2 + fx;
+            if (iy < a.h && ix < a.w) { a.out[((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride + f] = gr[fy][fx]; }
+        }
+    }
+}
+
+}  // namespace bbhip

@@ -111,6 +111,81 @@ class AdamState:
         self.b2 = self.b2 * self.beta2
 
 
+BORDER_MODES = {"constant": 0, "reflect": 1, "reflect_101": 2, "replicate": 3, "wrap": 4}
+
+
+def im2col_geometry(h, w, fh, fw, ys=1, xs=1, padding="valid"):
+    """(oh, ow, y_offset, x_offset) of a filter fh x fw stepping by (ys, xs) (reference: include/bb/ConvolutionIm2Col.h:183-198)"""
+    if padding == "valid":
+        return ((h - fh + 1) + (ys - 1)) // ys, ((w - fw + 1) + (xs - 1)) // xs, 0, 0
+    if padding != "same":
+        raise capi.BbhipError("padding must be 'valid' or 'same'")
+    return (h + ys - 1) // ys, (w + xs - 1) // xs, (fh - 1) // 2, (fw - 1) // 2
+
+
+def _stride_for(frames, bit):
+    from . import synth
+    return synth.frame_stride_bit(frames) if bit else synth.frame_stride_fp32(frames)
+
+
+def im2col_forward(x, c, h, w, frames, fh, fw, ys=1, xs=1, padding="valid", border="reflect_101", border_value=0.0):
+    """x [c*h*w, stride] float32 or packed int32 -> y [c*fh*fw, stride'] holding frames*oh*ow frames"""
+    _dev(x)
+    bit = x.dtype == torch.int32
+    oh, ow, yo, xo = im2col_geometry(h, w, fh, fw, ys, xs, padding)
+    of = frames * oh * ow
+    y = (torch.zeros if bit else torch.empty)((c * fh * fw, _stride_for(of, bit)), dtype=x.dtype, device=x.device)
+    if bit:
+        check(lib().bbhip_bit_Im2Col_Forward(ptr(x), ptr(y), xs, ys, xo, yo, frames, x.shape[1], w, h, c, ow, oh, y.shape[1], fw, fh,
+                                             BORDER_MODES[border], stream_ptr()))
+    else:
+        check(lib().bbhip_fp32_Im2Col_Forward(ptr(x), ptr(y), xs, ys, xo, yo, frames, x.shape[1], w, h, c, ow, oh, y.shape[1], fw, fh,
+                                              BORDER_MODES[border], border_value, stream_ptr()))
+    return y
+
+
+def im2col_backward(dy, c, h, w, frames, fh, fw, ys=1, xs=1, padding="valid"):
+    _dev(dy)
+    oh, ow, yo, xo = im2col_geometry(h, w, fh, fw, ys, xs, padding)
+    dx = torch.empty((c * h * w, _stride_for(frames, False)), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_Im2Col_Backward(ptr(dy), ptr(dx), xs, ys, xo, yo, frames, dx.shape[1], w, h, c, ow, oh, dy.shape[1], fw, fh,
+                                           stream_ptr()))
+    return dx
+
+
+def col2im_forward(x, c, h, w, frames):
+    """x [c, stride] over frames*h*w frames -> y [c*h*w, stride'] over frames frames"""
+    _dev(x)
+    bit = x.dtype == torch.int32
+    y = (torch.zeros if bit else torch.empty)((c * h * w, _stride_for(frames, bit)), dtype=x.dtype, device=x.device)
+    fn = lib().bbhip_bit_Col2Im_Forward if bit else lib().bbhip_fp32_Col2Im_Forward
+    check(fn(ptr(x), ptr(y), w, h, c, x.shape[1], frames, y.shape[1], stream_ptr()))
+    return y
+
+
+def col2im_backward(dy, c, h, w, frames):
+    _dev(dy)
+    dx = torch.empty((c, _stride_for(frames * h * w, False)), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_Col2Im_Backward(ptr(dy), ptr(dx), w, h, c, dx.shape[1], frames, dy.shape[1], stream_ptr()))
+    return dx
+
+
+def stochastic_maxpool2x2_forward(x, c, h, w, frames):
+    _dev(x)
+    oh, ow = (h + 1) // 2, (w + 1) // 2
+    y = torch.empty((c * oh * ow, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_StochasticMaxPooling2x2_Forward(ptr(x), ptr(y), w, h, ow, oh, c, frames, x.shape[1], stream_ptr()))
+    return y
+
+
+def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
+    _dev(x, dy)
+    oh, ow = (h + 1) // 2, (w + 1) // 2
+    dx = torch.empty_like(x)
+    check(lib().bbhip_fp32_StochasticMaxPooling2x2_Backward(ptr(x), ptr(dy), ptr(dx), w, h, ow, oh, c, frames, x.shape[1], stream_ptr()))
+    return dx
+
+
 def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
     _dev(xbits)
     y = torch.empty((xbits.shape[0], y_stride), dtype=torch.float32, device=xbits.device)

@@ -119,6 +119,48 @@ int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
                              int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream);
 
+/* ---- convolution plumbing: Im2Col, Col2Im, StochasticMaxPooling2x2 ----
+ * A convolution is Im2Col -> LUT layers -> Col2Im.  Buffers are node-major / frame-minor as everywhere; nodes are
+ * (c, y, x) row-major pixels or (c, fy, fx) filter taps; Im2Col's output frame is (input frame, oy, ox) row-major.
+ * Results follow the reference's host paths (include/bb/ConvolutionIm2Col.h:370-452, ConvolutionCol2Im.h:203-293,
+ * StochasticMaxPooling2x2.h:190-306) bit for bit. */
+/* bbcu_fp32_Im2Col_Forward, include/bbcu/bbcu.h:1076-1097.  x_stride / y_stride are the window steps, x_offset / y_offset
+ * the padding ((filter-1)/2 for "same", 0 for "valid"); border_mode 0 constant (border_value), 1 reflect, 2 reflect_101,
+ * 3 replicate, 4 wrap (include/bb/DataType.h BB_BORDER_*). */
+int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
+                              int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size,
+                              int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
+                              int border_mode, float border_value, void *stream);
+/* bbcu_bit_Im2Col_Forward, include/bbcu/bbcu.h:1099-1119 (packed bits; strides in 32-bit words; constant border = 0) */
+int bbhip_bit_Im2Col_Forward(int const *dev_x_buf, int *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
+                             int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size,
+                             int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
+                             int border_mode, void *stream);
+/* bbcu_fp32_Im2Col_Backward, include/bbcu/bbcu.h:1122-1141: dx is overwritten; only taps inside the image carry gradient */
+int bbhip_fp32_Im2Col_Backward(float const *dev_dy_buf, float *dev_dx_buf, int x_stride, int y_stride, int x_offset, int y_offset,
+                               int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size,
+                               int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
+                               void *stream);
+/* bbcu_fp32_Col2Im_Forward, include/bbcu/bbcu.h:1148-1159: y[(c, xy)][f] = x[c][f*h*w + xy]; input_* describe the
+ * [c][frames*h*w] buffer, output_* the [c*h*w][frames] buffer (also in Backward, where the first is dx) */
+int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
+                              int output_frame_size, int output_frame_stride, void *stream);
+/* bbcu_bit_Col2Im_Forward, include/bbcu/bbcu.h:1161-1172 */
+int bbhip_bit_Col2Im_Forward(int const *dev_x_buf, int *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
+                             int output_frame_size, int output_frame_stride, void *stream);
+/* bbcu_fp32_Col2Im_Backward, include/bbcu/bbcu.h:1175-1186 */
+int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w_size, int h_size, int c_size, int input_frame_stride,
+                               int output_frame_size, int output_frame_stride, void *stream);
+/* bbcu_fp32_StochasticMaxPooling2x2_Forward, include/bbcu/bbcu.h:768-780: y = 1 - prod over the 2 x 2 window of (1 - x);
+ * output sizes are ceil(input / 2), window taps outside the image are skipped */
+int bbhip_fp32_StochasticMaxPooling2x2_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size,
+                                               int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride,
+                                               void *stream);
+/* bbcu_fp32_StochasticMaxPooling2x2_Backward, include/bbcu/bbcu.h:783-796 */
+int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int input_w_size,
+                                                int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                                int frame_stride, void *stream);
+
 /* ---- StochasticLut ---- */
 /* bbcu_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:667-681 */
 int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,

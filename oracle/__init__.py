@@ -108,6 +108,85 @@ def adam_steps(param, grads, learning_rate=0.001, beta1=0.9, beta2=0.999):
     return p, m, v
 
 
+BORDER_MODES = {"constant": 0, "reflect": 1, "reflect_101": 2, "replicate": 3, "wrap": 4}
+
+
+def im2col_geometry(h, w, fh, fw, ys=1, xs=1, padding="valid"):
+    """(oh, ow, y_offset, x_offset) as include/bb/ConvolutionIm2Col.h:183-198 computes them."""
+    if padding == "valid":
+        return ((h - fh + 1) + (ys - 1)) // ys, ((w - fw + 1) + (xs - 1)) // xs, 0, 0
+    assert padding == "same"
+    return (h + ys - 1) // ys, (w + xs - 1) // xs, (fh - 1) // 2, (fw - 1) // 2
+
+
+def im2col_forward(x, c, h, w, frames, fh, fw, ys=1, xs=1, padding="valid", border="reflect_101", border_value=0.0, bit=False):
+    """x: [c*h*w, stride] fp32 (or packed int32 words when bit) -> y: [c*fh*fw, stride'] over frames*oh*ow frames."""
+    oh, ow, yo, xo = im2col_geometry(h, w, fh, fw, ys, xs, padding)
+    of = frames * oh * ow
+    if bit:
+        x = _c(x, np.int32)
+        y = np.zeros((c * fh * fw, (of + 31) // 32), np.int32)
+        lib().oracle_bit_Im2Col_Forward(_ptr(x), _ptr(y), C.c_int(xs), C.c_int(ys), C.c_int(xo), C.c_int(yo), C.c_int(frames),
+                                        C.c_int(x.shape[1]), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(ow), C.c_int(oh),
+                                        C.c_int(y.shape[1]), C.c_int(fw), C.c_int(fh), C.c_int(BORDER_MODES[border]))
+    else:
+        x = _c(x, np.float32)
+        y = np.zeros((c * fh * fw, of), np.float32)
+        lib().oracle_fp32_Im2Col_Forward(_ptr(x), _ptr(y), C.c_int(xs), C.c_int(ys), C.c_int(xo), C.c_int(yo), C.c_int(frames),
+                                         C.c_int(x.shape[1]), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(ow), C.c_int(oh),
+                                         C.c_int(y.shape[1]), C.c_int(fw), C.c_int(fh), C.c_int(BORDER_MODES[border]),
+                                         C.c_float(border_value))
+    return y
+
+
+def im2col_backward(dy, c, h, w, frames, fh, fw, ys=1, xs=1, padding="valid"):
+    oh, ow, yo, xo = im2col_geometry(h, w, fh, fw, ys, xs, padding)
+    dy = _c(dy, np.float32)
+    dx = np.zeros((c * h * w, frames), np.float32)
+    lib().oracle_fp32_Im2Col_Backward(_ptr(dy), _ptr(dx), C.c_int(xs), C.c_int(ys), C.c_int(xo), C.c_int(yo), C.c_int(frames),
+                                      C.c_int(frames), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(ow), C.c_int(oh),
+                                      C.c_int(dy.shape[1]), C.c_int(fw), C.c_int(fh))
+    return dx
+
+
+def col2im_forward(x, c, h, w, frames, bit=False):
+    """x: [c, frames*h*w] -> y: [c*h*w, frames]"""
+    if bit:
+        x = _c(x, np.int32)
+        y = np.zeros((c * h * w, (frames + 31) // 32), np.int32)
+        lib().oracle_bit_Col2Im_Forward(_ptr(x), _ptr(y), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(x.shape[1]), C.c_int(frames), C.c_int(y.shape[1]))
+    else:
+        x = _c(x, np.float32)
+        y = np.zeros((c * h * w, frames), np.float32)
+        lib().oracle_fp32_Col2Im_Forward(_ptr(x), _ptr(y), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(x.shape[1]), C.c_int(frames), C.c_int(frames))
+    return y
+
+
+def col2im_backward(dy, c, h, w, frames):
+    dy = _c(dy, np.float32)
+    dx = np.zeros((c, frames * h * w), np.float32)
+    lib().oracle_fp32_Col2Im_Backward(_ptr(dy), _ptr(dx), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(dx.shape[1]), C.c_int(frames), C.c_int(dy.shape[1]))
+    return dx
+
+
+def stochastic_maxpool2x2_forward(x, c, h, w, frames):
+    x = _c(x, np.float32)
+    oh, ow = (h + 1) // 2, (w + 1) // 2
+    y = np.zeros((c * oh * ow, x.shape[1]), np.float32)
+    lib().oracle_fp32_StochasticMaxPooling2x2_Forward(_ptr(x), _ptr(y), C.c_int(w), C.c_int(h), C.c_int(ow), C.c_int(oh), C.c_int(c),
+                                                      C.c_int(frames), C.c_int(x.shape[1]))
+    return y
+
+
+def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
+    x = _c(x, np.float32); dy = _c(dy, np.float32)
+    oh, ow = (h + 1) // 2, (w + 1) // 2
+    dx = np.zeros_like(x)
+    lib().oracle_fp32_StochasticMaxPooling2x2_Backward(_ptr(x), _ptr(dy), _ptr(dx), C.c_int(w), C.c_int(h), C.c_int(ow), C.c_int(oh),
+                                                       C.c_int(c), C.c_int(frames), C.c_int(x.shape[1]))
+    return dx
+
+
 def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, simd=True):
     """fp32 x [I, stride] -> y [O, stride] (padding columns zero)."""
     x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
@@ -380,6 +459,48 @@ def ref_vector_op(name, src0, src1=None, a=0.0, b=0.0, c=0.0, d=0.0):
                                C.c_float(c), C.c_float(d), C.c_int(src0.size))
     assert rc == 0
     return dst
+
+
+def ref_im2col(x, c, h, w, frames, fh, fw, ys=1, xs=1, padding="valid", border="reflect_101", dy=None, bit=False):
+    """The reference's ConvolutionIm2Col (host path): returns (y, dx or None).  Dense arrays: fp32 [nodes, frames] or
+    packed [nodes, ceil(frames/32)]."""
+    oh, ow, _, _ = im2col_geometry(h, w, fh, fw, ys, xs, padding)
+    of = frames * oh * ow
+    if bit:
+        x = _c(x, np.int32); y = np.zeros((c * fh * fw, (of + 31) // 32), np.int32)
+    else:
+        x = _c(x, np.float32); y = np.zeros((c * fh * fw, of), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((c * h * w, frames), np.float32)
+    hw = (C.c_int * 2)()
+    got = ref().bbref_Im2Col(C.c_int(int(bit)), C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(frames), C.c_int(fh), C.c_int(fw),
+                             C.c_int(ys), C.c_int(xs), padding.encode(), border.encode(), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx), hw)
+    assert got == of and (hw[0], hw[1]) == (oh, ow)
+    return y, dx
+
+
+def ref_col2im(x, c, h, w, frames, dy=None, bit=False):
+    if bit:
+        x = _c(x, np.int32); y = np.zeros((c * h * w, (frames + 31) // 32), np.int32)
+    else:
+        x = _c(x, np.float32); y = np.zeros((c * h * w, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((c, frames * h * w), np.float32)
+    assert ref().bbref_Col2Im(C.c_int(int(bit)), C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(frames), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx)) == 0
+    return y, dx
+
+
+def ref_stochastic_maxpool2x2(x, c, h, w, frames, dy=None):
+    x = _c(x, np.float32)
+    oh, ow = (h + 1) // 2, (w + 1) // 2
+    y = np.zeros((c * oh * ow, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((c * h * w, frames), np.float32)
+    assert ref().bbref_StochasticMaxPooling2x2(C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(frames), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx)) == 0
+    return y, dx
 
 
 def time_stochastic_lut6(x, dy, idx, W, reps=3, use_ref=None):

@@ -704,3 +704,216 @@ void oracle_fp32_OptimizerAdam(int size, float *param, float const *grad, float 
         param[i] = param[i] - num / den;                                       /* p -= lr_t*m/(sqrt(v)+1e-7) :176 */
     }
 }
+
+
+/* ------------------------------------------------------------------------------------------------
+ * Convolution plumbing around the LUT layers: Im2Col, Col2Im, StochasticMaxPooling2x2 (host paths of
+ * include/bb/ConvolutionIm2Col.h:317-470, ConvolutionCol2Im.h:203-300, StochasticMaxPooling2x2.h:190-320).
+ * Buffers are node-major, frame-minor with explicit strides (floats, or 32-bit words for packed bits).
+ * Pinned by: the known answers of the reference's tests (tests/gtest/ConvolutionIm2ColTest.cpp:20-200,
+ * ConvolutionCol2ImTest.cpp), restated in tests/test_oracle_conv.py; the reference's own classes through
+ * oracle/_ref where built; tests/golden/conv.npz; permutation identities (Col2Im backward inverts forward,
+ * Im2Col backward = transpose of forward on constant borders, pooling = 1 - prod(1 - x)).
+ * border_mode: 0 constant, 1 reflect, 2 reflect_101, 3 replicate, 4 wrap (include/bb/DataType.h BB_BORDER_*).
+ * ------------------------------------------------------------------------------------------------ */
+static int im2col_border(int mode, int *x, int *y, int w, int h)        /* ConvolutionIm2Col.h:251-286 */
+{
+    switch (mode) {
+    case 1: if (*x < 0) { *x = -*x - 1; } if (*y < 0) { *y = -*y - 1; }
+            if (*x >= w) { *x = (w - 1) - (*x - w); } if (*y >= h) { *y = (h - 1) - (*y - h); } return 1;
+    case 2: if (*x < 0) { *x = -*x; } if (*y < 0) { *y = -*y; }
+            if (*x >= w) { *x = (w - 2) - (*x - w); } if (*y >= h) { *y = (h - 2) - (*y - h); } return 1;
+    case 3: if (*x < 0) { *x = 0; } if (*y < 0) { *y = 0; } if (*x >= w) { *x = w - 1; } if (*y >= h) { *y = h - 1; } return 1;
+    case 4: if (*x < 0) { *x += w; } if (*y < 0) { *y += h; } if (*x >= w) { *x -= w; } if (*y >= h) { *y -= h; } return 1;
+    default: return 0;
+    }
+}
+
+static int get_bit(int const *row, long long f) { return (row[f >> 5] >> (f & 31)) & 1; }
+static void set_bit(int *row, long long f, int v)
+{
+    unsigned int const m = 1u << (f & 31);
+    unsigned int w = (unsigned int)row[f >> 5];
+    w = v ? (w | m) : (w & ~m);
+    row[f >> 5] = (int)w;
+}
+
+/* is_bit = 0: fp32 buffers; 1: packed bits (border_value is then 0/1) */
+static void im2col_forward(int is_bit, void const *x, void *y, int x_stride, int y_stride, int x_offset, int y_offset,
+                           int input_frame_size, int input_frame_stride, int w, int h, int c_size, int ow, int oh,
+                           int output_frame_stride, int fw, int fh, int border_mode, float border_value)
+{
+    long long const output_size = (long long)oh * ow;
+    long long const output_frame_size = (long long)input_frame_size * output_size;
+    for (int c = 0; c < c_size; ++c) {
+        for (int fy = 0; fy < fh; ++fy) {
+            for (int fx = 0; fx < fw; ++fx) {
+                long long const out_node = ((long long)c * fh + fy) * fw + fx;
+                for (long long of = 0; of < output_frame_size; ++of) {
+                    long long const in_frame = of / output_size;
+                    long long const f = of % output_size;
+                    int iy = (int)(f / ow) * y_stride - y_offset + fy;
+                    int ix = (int)(f % ow) * x_stride - x_offset + fx;
+                    int have = (iy >= 0 && iy < h && ix >= 0 && ix < w);
+                    if (!have) { have = im2col_border(border_mode, &ix, &iy, w, h); }
+                    long long const in_node = ((long long)c * h + iy) * w + ix;
+                    if (is_bit) {
+                        int const v = have ? get_bit((int const *)x + in_node * input_frame_stride, in_frame) : (border_value > 0.5f);
+                        set_bit((int *)y + out_node * output_frame_stride, of, v);
+                    }
+                    else {
+                        float const v = have ? ((float const *)x)[in_node * input_frame_stride + in_frame] : border_value;
+                        ((float *)y)[out_node * output_frame_stride + of] = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+void oracle_fp32_Im2Col_Forward(float const *x, float *y, int x_stride, int y_stride, int x_offset, int y_offset,
+                                int input_frame_size, int input_frame_stride, int w, int h, int c, int ow, int oh,
+                                int output_frame_stride, int fw, int fh, int border_mode, float border_value)
+{
+    im2col_forward(0, x, y, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, w, h, c, ow, oh,
+                   output_frame_stride, fw, fh, border_mode, border_value);
+}
+
+void oracle_bit_Im2Col_Forward(int const *x, int *y, int x_stride, int y_stride, int x_offset, int y_offset,
+                               int input_frame_size, int input_frame_stride, int w, int h, int c, int ow, int oh,
+                               int output_frame_stride, int fw, int fh, int border_mode)
+{
+    im2col_forward(1, x, y, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, w, h, c, ow, oh,
+                   output_frame_stride, fw, fh, border_mode, 0.0f);
+}
+
+/* ConvolutionIm2Col.h:411-452: only in-range taps contribute (border replicas carry no gradient); sums in (fy, fx) order */
+void oracle_fp32_Im2Col_Backward(float const *dy, float *dx, int x_stride, int y_stride, int x_offset, int y_offset,
+                                 int input_frame_size, int input_frame_stride, int w, int h, int c_size, int ow, int oh,
+                                 int output_frame_stride, int fw, int fh)
+{
+    int const iy_limit = (oh - 1) * y_stride, ix_limit = (ow - 1) * x_stride;
+    for (int c = 0; c < c_size; ++c) {
+        for (int y = 0; y < h; ++y) {
+            for (int x = 0; x < w; ++x) {
+                long long const in_node = ((long long)c * h + y) * w + x;
+                int const x_align = x % x_stride, y_align = y % y_stride;
+                for (int f = 0; f < input_frame_size; ++f) {
+                    float s = 0.0f;
+                    for (int fy = y_align; fy < fh; fy += y_stride) {
+                        int const iy = y - fy + y_offset;
+                        if (iy < 0 || iy > iy_limit) { continue; }
+                        for (int fx = x_align; fx < fw; fx += x_stride) {
+                            int const ix = x - fx + x_offset;
+                            if (ix < 0 || ix > ix_limit) { continue; }
+                            long long const of = ((long long)f * oh + (iy / y_stride)) * ow + (ix / x_stride);
+                            long long const out_node = ((long long)c * fh + fy) * fw + fx;
+                            s += dy[out_node * output_frame_stride + of];
+                        }
+                    }
+                    dx[in_node * input_frame_stride + f] = s;
+                }
+            }
+        }
+    }
+}
+
+/* ConvolutionCol2Im.h:203-217: y[(c, xy)][f] = x[c][f*hw + xy] */
+void oracle_fp32_Col2Im_Forward(float const *x, float *y, int w, int h, int c_size, int input_frame_stride,
+                                int output_frame_size, int output_frame_stride)
+{
+    long long const hw = (long long)h * w;
+    for (int c = 0; c < c_size; ++c) {
+        for (long long xy = 0; xy < hw; ++xy) {
+            for (int f = 0; f < output_frame_size; ++f) {
+                y[(c * hw + xy) * output_frame_stride + f] = x[(long long)c * input_frame_stride + f * hw + xy];
+            }
+        }
+    }
+}
+
+void oracle_bit_Col2Im_Forward(int const *x, int *y, int w, int h, int c_size, int input_frame_stride,
+                               int output_frame_size, int output_frame_stride)
+{
+    long long const hw = (long long)h * w;
+    for (int c = 0; c < c_size; ++c) {
+        for (long long xy = 0; xy < hw; ++xy) {
+            for (int f = 0; f < output_frame_size; ++f) {
+                set_bit(y + (c * hw + xy) * output_frame_stride, f, get_bit(x + (long long)c * input_frame_stride, f * hw + xy));
+            }
+        }
+    }
+}
+
+/* ConvolutionCol2Im.h:279-293: dx[c][f*hw + xy] = dy[(c, xy)][f].  input_* describe dx, output_* describe dy. */
+void oracle_fp32_Col2Im_Backward(float const *dy, float *dx, int w, int h, int c_size, int input_frame_stride,
+                                 int output_frame_size, int output_frame_stride)
+{
+    long long const hw = (long long)h * w;
+    for (int c = 0; c < c_size; ++c) {
+        for (long long xy = 0; xy < hw; ++xy) {
+            for (int f = 0; f < output_frame_size; ++f) {
+                dx[(long long)c * input_frame_stride + f * hw + xy] = dy[(c * hw + xy) * output_frame_stride + f];
+            }
+        }
+    }
+}
+
+/* StochasticMaxPooling2x2.h:190-218: y = 1 - prod over the window (taps inside the image, (fy, fx) ascending) of (1 - x) */
+void oracle_fp32_StochasticMaxPooling2x2_Forward(float const *x, float *y, int w, int h, int ow, int oh, int c_size,
+                                                 int frame_size, int frame_stride)
+{
+    for (int c = 0; c < c_size; ++c) {
+        for (int oy = 0; oy < oh; ++oy) {
+            for (int ox = 0; ox < ow; ++ox) {
+                for (int f = 0; f < frame_size; ++f) {
+                    float out = 1.0f;
+                    for (int fy = 0; fy < 2; ++fy) {
+                        int const iy = oy * 2 + fy;
+                        if (iy >= h) { continue; }
+                        for (int fx = 0; fx < 2; ++fx) {
+                            int const ix = ox * 2 + fx;
+                            if (ix >= w) { continue; }
+                            out *= (1.0f - x[(((long long)c * h + iy) * w + ix) * frame_stride + f]);
+                        }
+                    }
+                    y[(((long long)c * oh + oy) * ow + ox) * frame_stride + f] = 1.0f - out;
+                }
+            }
+        }
+    }
+}
+
+/* StochasticMaxPooling2x2.h:262-306: in_grad = (float)(dy * (1.0 - other taps ...)) evaluated in double; taps outside the
+ * image read as 0 */
+void oracle_fp32_StochasticMaxPooling2x2_Backward(float const *x, float const *dy, float *dx, int w, int h, int ow, int oh,
+                                                  int c_size, int frame_size, int frame_stride)
+{
+    for (int c = 0; c < c_size; ++c) {
+        for (int oy = 0; oy < oh; ++oy) {
+            for (int ox = 0; ox < ow; ++ox) {
+                for (int f = 0; f < frame_size; ++f) {
+                    float in[2][2] = {{0, 0}, {0, 0}};
+                    for (int fy = 0; fy < 2; ++fy) {
+                        for (int fx = 0; fx < 2; ++fx) {
+                            int const iy = oy * 2 + fy, ix = ox * 2 + fx;
+                            if (iy < h && ix < w) { in[fy][fx] = x[(((long long)c * h + iy) * w + ix) * frame_stride + f]; }
+                        }
+                    }
+                    float const g = dy[(((long long)c * oh + oy) * ow + ox) * frame_stride + f];
+                    float gr[2][2];
+                    gr[0][0] = (float)(g * (1.0 - in[0][1]) * (1.0 - in[1][0]) * (1.0 - in[1][1]));
+                    gr[0][1] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[1][0]) * (1.0 - in[1][1]));
+                    gr[1][0] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[0][1]) * (1.0 - in[1][1]));
+                    gr[1][1] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[0][1]) * (1.0 - in[1][0]));
+                    for (int fy = 0; fy < 2; ++fy) {
+                        for (int fx = 0; fx < 2; ++fx) {
+                            int const iy = oy * 2 + fy, ix = ox * 2 + fx;
+                            if (iy < h && ix < w) { dx[(((long long)c * h + iy) * w + ix) * frame_stride + f] = gr[fy][fx]; }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}

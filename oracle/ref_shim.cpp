@@ -22,6 +22,9 @@
 #include "bb/BinaryLutN.h"
 #include "bb/FixedSizeConnectionTable.h"
 #include "bb/OptimizerAdam.h"
+#include "bb/ConvolutionIm2Col.h"
+#include "bb/ConvolutionCol2Im.h"
+#include "bb/StochasticMaxPooling2x2.h"
 #include "bb/TensorOperator.h"
 
 namespace {
@@ -329,4 +332,97 @@ int bbref_Vector_op(int op, float *dst, float const *src0, float const *src1, fl
     return -1;
 }
 
+
 }  // extern "C"
+
+// ConvolutionIm2Col<float|Bit, float> (host path).  x: [c*h*w][frames] dense (fp32) or [c*h*w][words] (bits);
+// y: [c*fh*fw][frames*oh*ow]; when dy != NULL (fp32 only) Backward is run and dx [c*h*w][frames] is returned.
+// out_hw receives {oh, ow}.
+template <typename FT>
+static int run_im2col(int c, int h, int w, int frames, int fh, int fw, int ys, int xs, char const *padding, char const *border,
+                      void const *x, void *y, float const *dy, float *dx, int *out_hw)
+{
+    auto m = bb::ConvolutionIm2Col<FT, float>::Create(fh, fw, ys, xs, padding, border);
+    m->SendCommand("host_only true");
+    bb::indices_t shape({(index_t)c, (index_t)h, (index_t)w});
+    bb::FrameBuffer xb(frames, shape, bb::DataType<FT>::type, true);
+    index_t const in_nodes = (index_t)c * h * w;
+    if (std::is_same<FT, bb::Bit>::value) { put_bit(xb, (std::int32_t const *)x, in_nodes, (frames + 31) / 32); }
+    else                                   { put_fp32(xb, (float const *)x, in_nodes, frames); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    index_t const out_nodes = (index_t)c * fh * fw;
+    index_t const out_frames = yb.GetFrameSize();
+    index_t const o = out_frames / frames;            // oh * ow
+    (void)o;
+    if (std::is_same<FT, bb::Bit>::value) { get_bit(yb, (std::int32_t *)y, out_nodes, (out_frames + 31) / 32); }
+    else                                   { get_fp32(yb, (float *)y, out_nodes, out_frames); }
+    if (dy) {
+        bb::FrameBuffer dyb(out_frames, bb::indices_t({(index_t)c, (index_t)fh, (index_t)fw}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, out_nodes, out_frames);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, in_nodes, frames);
+    }
+    if (out_hw) {
+        std::string pad(padding);
+        out_hw[0] = pad == "same" ? (h + ys - 1) / ys : ((h - fh + 1) + (ys - 1)) / ys;
+        out_hw[1] = pad == "same" ? (w + xs - 1) / xs : ((w - fw + 1) + (xs - 1)) / xs;
+    }
+    return (int)out_frames;
+}
+
+extern "C" int bbref_Im2Col(int bit, int c, int h, int w, int frames, int fh, int fw, int ys, int xs, char const *padding, char const *border,
+                 void const *x, void *y, float const *dy, float *dx, int *out_hw)
+{
+    return bit ? run_im2col<bb::Bit>(c, h, w, frames, fh, fw, ys, xs, padding, border, x, y, dy, dx, out_hw)
+               : run_im2col<float>(c, h, w, frames, fh, fw, ys, xs, padding, border, x, y, dy, dx, out_hw);
+}
+
+// ConvolutionCol2Im<float|Bit, float> (host path).  x: [c][frames*h*w]; y: [c*h*w][frames]; dy/dx likewise (fp32).
+template <typename FT>
+static int run_col2im(int c, int h, int w, int frames, void const *x, void *y, float const *dy, float *dx)
+{
+    auto m = bb::ConvolutionCol2Im<FT, float>::Create(h, w);
+    m->SendCommand("host_only true");
+    m->SetInputShape(bb::indices_t({(index_t)c}));      // Forward does not derive the channel count itself
+    index_t const in_frames = (index_t)frames * h * w;
+    bb::FrameBuffer xb(in_frames, bb::indices_t({(index_t)c}), bb::DataType<FT>::type, true);
+    if (std::is_same<FT, bb::Bit>::value) { put_bit(xb, (std::int32_t const *)x, c, (in_frames + 31) / 32); }
+    else                                   { put_fp32(xb, (float const *)x, c, in_frames); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    index_t const out_nodes = (index_t)c * h * w;
+    if (std::is_same<FT, bb::Bit>::value) { get_bit(yb, (std::int32_t *)y, out_nodes, (frames + 31) / 32); }
+    else                                   { get_fp32(yb, (float *)y, out_nodes, frames); }
+    if (dy) {
+        bb::FrameBuffer dyb(frames, bb::indices_t({(index_t)c, (index_t)h, (index_t)w}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, out_nodes, frames);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, c, in_frames);
+    }
+    return 0;
+}
+
+extern "C" int bbref_Col2Im(int bit, int c, int h, int w, int frames, void const *x, void *y, float const *dy, float *dx)
+{
+    return bit ? run_col2im<bb::Bit>(c, h, w, frames, x, y, dy, dx) : run_col2im<float>(c, h, w, frames, x, y, dy, dx);
+}
+
+// StochasticMaxPooling2x2<float, float> (host path).  x: [c*h*w][frames]; y: [c*oh*ow][frames]
+extern "C" int bbref_StochasticMaxPooling2x2(int c, int h, int w, int frames, float const *x, float *y, float const *dy, float *dx)
+{
+    auto m = bb::StochasticMaxPooling2x2<float, float>::Create();
+    m->SendCommand("host_only true");
+    bb::FrameBuffer xb(frames, bb::indices_t({(index_t)c, (index_t)h, (index_t)w}), BB_TYPE_FP32, true);
+    put_fp32(xb, x, (index_t)c * h * w, frames);
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    int const oh = (h + 1) / 2, ow = (w + 1) / 2;
+    get_fp32(yb, y, (index_t)c * oh * ow, frames);
+    if (dy) {
+        bb::FrameBuffer dyb(frames, bb::indices_t({(index_t)c, (index_t)oh, (index_t)ow}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, (index_t)c * oh * ow, frames);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, (index_t)c * h * w, frames);
+    }
+    return 0;
+}
+
+  // extern "C"

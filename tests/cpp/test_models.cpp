@@ -11,8 +11,15 @@
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
 #include "bb/OptimizerAdam.h"
+#include "bb/ConvolutionIm2Col.h"
+#include "bb/ConvolutionCol2Im.h"
+#include "bb/StochasticMaxPooling2x2.h"
 
 extern "C" {
+void oracle_fp32_Im2Col_Backward(float const *dy, float *dx, int x_stride, int y_stride, int x_offset, int y_offset, int input_frame_size,
+                                 int input_frame_stride, int w, int h, int c, int ow, int oh, int output_frame_stride, int fw, int fh);
+void oracle_fp32_StochasticMaxPooling2x2_Forward(float const *x, float *y, int w, int h, int ow, int oh, int c, int frame_size, int frame_stride);
+void oracle_fp32_StochasticMaxPooling2x2_Backward(float const *x, float const *dy, float *dx, int w, int h, int ow, int oh, int c, int frame_size, int frame_stride);
 void oracle_fp32_OptimizerAdam(int size, float *param, float const *grad, float *m, float *v, float lr_t, float beta1, float beta2);
 void oracle_fp32_StochasticLut_Forward(int n, float const *x, float *y, std::int32_t const *idx, float const *W, int node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
 void oracle_fp32_StochasticLut_Backward(int n, float const *x, float const *dy, float *dx, std::int32_t const *idx, float const *W, float *dW, int input_node_size, int output_node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
@@ -233,6 +240,65 @@ static void test_adam(void)
     }
 }
 
+// The reference's Im2Col test (tests/gtest/ConvolutionIm2ColTest.cpp:19-190): 2 frames of {2, 3, 4} images whose pixels
+// encode their own coordinates, filter 2 x 3; then a conv block Im2Col -> Col2Im -> pooling against the oracle.
+static void test_conv_plumbing(void)
+{
+    auto im2col = bb::ConvolutionIm2Col<>::Create(2, 3);
+    bb::FrameBuffer x(2, {2, 3, 4}, BB_TYPE_FP32);
+    for (int f = 0; f < 2; ++f) for (int c = 0; c < 2; ++c) for (int y = 0; y < 3; ++y) for (int xx = 0; xx < 4; ++xx) {
+        x.SetFP32(f, (c * 3 + y) * 4 + xx, (float)(1000 * f + 100 * c + 10 * y + xx));
+    }
+    bb::FrameBuffer y = im2col->Forward(x);
+    CHECK(y.GetFrameSize() == 8 && y.GetNodeSize() == 12, "Im2Col output %d frames x %d nodes", (int)y.GetFrameSize(), (int)y.GetNodeSize());
+    int const base[8] = {0, 1, 10, 11, 1000, 1001, 1010, 1011};
+    size_t bad = 0;
+    for (int of = 0; of < 8; ++of) for (int c = 0; c < 2; ++c) for (int fy = 0; fy < 2; ++fy) for (int fx = 0; fx < 3; ++fx) {
+        bad += (y.GetFP32(of, (c * 2 + fy) * 3 + fx) != (float)(base[of] + 100 * c + 10 * fy + fx));
+    }
+    CHECK(bad == 0, "Im2Col known answers: %zu wrong", bad);
+    bb::FrameBuffer dy(8, {2, 2, 3}, BB_TYPE_FP32);
+    std::vector<float> dyv(12 * 8);
+    for (int of = 0; of < 8; ++of) for (int n = 0; n < 12; ++n) { dyv[(size_t)n * 8 + of] = (float)(1000 * of + n); dy.SetFP32(of, n, dyv[(size_t)n * 8 + of]); }
+    bb::FrameBuffer dx = im2col->Backward(dy);
+    std::vector<float> dx_ref(24 * 2);
+    oracle_fp32_Im2Col_Backward(dyv.data(), dx_ref.data(), 1, 1, 0, 0, 2, 2, 4, 3, 2, 2, 2, 8, 3, 2);
+    bad = 0;
+    for (int f = 0; f < 2; ++f) for (int n = 0; n < 24; ++n) { bad += (dx.GetFP32(f, n) != dx_ref[(size_t)n * 2 + f]); }
+    CHECK(bad == 0, "Im2Col backward: %zu wrong", bad);
+
+    // 1 x 1 Im2Col and Col2Im invert each other; pooling against the oracle
+    int const C = 3, H = 5, W = 7, F = 70;
+    std::mt19937_64 mt(5);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    bb::FrameBuffer img(F, {C, H, W}, BB_TYPE_FP32);
+    std::vector<float> dense((size_t)C * H * W * F);
+    for (int n = 0; n < C * H * W; ++n) for (int f = 0; f < F; ++f) { dense[(size_t)n * F + f] = uni(mt); img.SetFP32(f, n, dense[(size_t)n * F + f]); }
+    auto one = bb::ConvolutionIm2Col<>::Create(1, 1);
+    auto col2im = bb::ConvolutionCol2Im<>::Create(H, W);
+    bb::FrameBuffer back = col2im->Forward(one->Forward(img));
+    bad = 0;
+    for (int n = 0; n < C * H * W; ++n) for (int f = 0; f < F; ++f) { bad += (back.GetFP32(f, n) != dense[(size_t)n * F + f]); }
+    CHECK(bad == 0 && back.GetShape() == bb::indices_t({C, H, W}), "Im2Col(1x1) -> Col2Im round trip: %zu wrong", bad);
+    auto pool = bb::StochasticMaxPooling2x2<>::Create();
+    bb::FrameBuffer py = pool->Forward(img);
+    int const OH = 3, OW = 4;
+    std::vector<float> py_ref((size_t)C * OH * OW * F), pdy((size_t)C * OH * OW * F), pdx_ref(dense.size());
+    oracle_fp32_StochasticMaxPooling2x2_Forward(dense.data(), py_ref.data(), W, H, OW, OH, C, F, F);
+    bb::FrameBuffer pdy_buf(F, {C, OH, OW}, BB_TYPE_FP32);
+    bad = 0;
+    for (int n = 0; n < C * OH * OW; ++n) for (int f = 0; f < F; ++f) {
+        bad += (py.GetFP32(f, n) != py_ref[(size_t)n * F + f]);
+        pdy[(size_t)n * F + f] = uni(mt) - 0.5f; pdy_buf.SetFP32(f, n, pdy[(size_t)n * F + f]);
+    }
+    CHECK(bad == 0, "StochasticMaxPooling2x2 forward: %zu wrong", bad);
+    bb::FrameBuffer pdx = pool->Backward(pdy_buf);
+    oracle_fp32_StochasticMaxPooling2x2_Backward(dense.data(), pdy.data(), pdx_ref.data(), W, H, OW, OH, C, F, F);
+    bad = 0;
+    for (int n = 0; n < C * H * W; ++n) for (int f = 0; f < F; ++f) { bad += (pdx.GetFP32(f, n) != pdx_ref[(size_t)n * F + f]); }
+    CHECK(bad == 0, "StochasticMaxPooling2x2 backward: %zu wrong", bad);
+}
+
 int main(void)
 {
     if (!bb::Manager::IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
@@ -258,6 +324,7 @@ int main(void)
         test_binary(70, 33, 1000);
         test_import_layer();
         test_adam();
+        test_conv_plumbing();
     }
     catch (std::exception const &e) {
         std::printf("exception: %s\n", e.what());

@@ -140,13 +140,61 @@ def adam_cases():
     np.savez_compressed(os.path.join(OUT, "adam.npz"), **cases)
 
 
+def conv_cases():
+    """ConvolutionIm2Col, ConvolutionCol2Im and StochasticMaxPooling2x2 of the reference (host paths)."""
+    rng = np.random.default_rng(20240605)
+    cases = {}
+    k = 0
+    for (c, h, w, F, fh, fw, ys, xs, pad, border) in [(2, 3, 4, 2, 2, 3, 1, 1, "valid", "reflect_101"),
+                                                      (3, 7, 6, 5, 3, 3, 1, 1, "same", "reflect_101"),
+                                                      (2, 8, 9, 3, 3, 3, 2, 2, "same", "replicate"),
+                                                      (1, 5, 5, 4, 3, 3, 2, 1, "valid", "constant"),
+                                                      (2, 6, 7, 3, 3, 5, 1, 1, "same", "wrap"),
+                                                      (2, 6, 7, 35, 3, 3, 1, 1, "same", "reflect"),
+                                                      (3, 9, 8, 3, 3, 3, 1, 2, "same", "constant")]:
+        x = rng.random((c * h * w, F)).astype(np.float32)
+        oh, ow, _, _ = oracle.im2col_geometry(h, w, fh, fw, ys, xs, pad)
+        dy = rng.standard_normal((c * fh * fw, F * oh * ow)).astype(np.float32)
+        y, dx = oracle.ref_im2col(x, c, h, w, F, fh, fw, ys, xs, pad, border, dy=dy)
+        xb = synth.bernoulli_bits(rng, c * h * w, F)
+        yb, _ = oracle.ref_im2col(xb, c, h, w, F, fh, fw, ys, xs, pad, border, bit=True)
+        q = "i%d_" % k
+        cases.update({q + "geom": np.array([c, h, w, F, fh, fw, ys, xs, int(pad == "same"), oracle.BORDER_MODES[border]], np.int32),
+                      q + "x": x, q + "dy": dy, q + "y": y, q + "dx": dx, q + "xbits": xb, q + "ybits": mask_bits(yb, F * oh * ow)})
+        k += 1
+    cases["im2col_count"] = np.array([k], np.int32)
+    k = 0
+    for (c, h, w, F) in [(3, 4, 5, 6), (2, 1, 7, 33), (5, 3, 3, 64)]:
+        x = rng.random((c, F * h * w)).astype(np.float32)
+        dy = rng.standard_normal((c * h * w, F)).astype(np.float32)
+        y, dx = oracle.ref_col2im(x, c, h, w, F, dy=dy)
+        xb = synth.bernoulli_bits(rng, c, F * h * w)
+        yb, _ = oracle.ref_col2im(xb, c, h, w, F, bit=True)
+        q = "c%d_" % k
+        cases.update({q + "geom": np.array([c, h, w, F], np.int32), q + "x": x, q + "dy": dy, q + "y": y, q + "dx": dx,
+                      q + "xbits": xb, q + "ybits": mask_bits(yb, F)})
+        k += 1
+    cases["col2im_count"] = np.array([k], np.int32)
+    k = 0
+    for (c, h, w, F) in [(2, 4, 6, 5), (3, 5, 7, 9), (1, 1, 1, 3), (2, 30, 30, 16)]:
+        x = rng.random((c * h * w, F)).astype(np.float32)
+        dy = rng.standard_normal((c * ((h + 1) // 2) * ((w + 1) // 2), F)).astype(np.float32)
+        y, dx = oracle.ref_stochastic_maxpool2x2(x, c, h, w, F, dy=dy)
+        q = "p%d_" % k
+        cases.update({q + "geom": np.array([c, h, w, F], np.int32), q + "x": x, q + "dy": dy, q + "y": y, q + "dx": dx})
+        k += 1
+    cases["pool_count"] = np.array([k], np.int32)
+    np.savez_compressed(os.path.join(OUT, "conv.npz"), **cases)
+
+
 if __name__ == "__main__":
     assert oracle.have_ref(), "build oracle/_ref first (make -C oracle ref)"
-    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam"]
+    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam", "conv"]
     if "stochastic" in which: stochastic_cases()
     if "differentiable" in which: differentiable_cases()
     if "binary" in which: binary_cases()
     if "adam" in which: adam_cases()
+    if "conv" in which: conv_cases()
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)), "bytes")
