@@ -156,6 +156,62 @@ def bench_conv(args, lib):
     print(json.dumps(out))
 
 
+def bench_tail(args, lib):
+    """The tail of the MNIST-like classifier (secondary measurement): AverageLut 7 -> 1 over 70 -> 10 nodes, softmax cross
+    entropy and categorical accuracy over the 10 classes.  Measured at 65536 frames (streaming rate) and at the
+    configuration's own batch of 1024 frames (launch-bound).  Algorithmic bytes: every element of input and output once."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import ops, synth
+    n, I, O = 7, 70, 10
+    kernels = {}
+    totals = {}
+    for F in (65536, 1024):
+        g = torch.Generator(device="cuda"); g.manual_seed(0)
+        S = synth.frame_stride_fp32(F)
+        idx = torch.arange(I, dtype=torch.int32, device="cuda").reshape(O, n).contiguous()
+        x = torch.rand((I, S), device="cuda", generator=g)
+        dy = torch.rand((O, S), device="cuda", generator=g)
+        y = torch.rand((O, S), device="cuda", generator=g)
+        t = torch.zeros((O, S), device="cuda")
+        label = torch.randint(0, O, (F,), device="cuda", generator=g)
+        t[label, torch.arange(F, device="cuda")] = 1.0
+        e = 4
+        cases = [
+            ("average_lut_forward_kernel", lambda: ops.average_lut_forward(x, idx, F, False, False), e * F * (I + O)),
+            ("average_lut_backward_kernel (+ reverse wiring)", lambda: ops.average_lut_backward(dy, idx, I, F), e * F * (I + O)),
+            ("softmax_cross_entropy_kernel", lambda: ops.loss_softmax_cross_entropy(y, t, O, 1, F, t_sum=float(F)), e * F * 3 * O + 8 * F),
+            ("categorical_accuracy_kernel", lambda: ops.metrics_categorical_accuracy(y, t, O, 1, F), e * F * 2 * O + 8 * F),
+        ]
+        total_ms = 0.0
+        for name, fn, nbytes in cases:
+            for _ in range(args.warmup):
+                fn()
+            torch.cuda.synchronize()
+            ms = []
+            for _ in range(args.steps):
+                e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+                out = fn(); del out
+                torch.cuda.synchronize()
+                e0.record(); out = fn(); e1.record(); torch.cuda.synchronize()
+                ms.append(e0.elapsed_time(e1))
+            med = sorted(ms)[len(ms) // 2]
+            total_ms += med
+            if F == 65536:
+                kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
+        totals[F] = total_ms
+    dom = max(kernels, key=lambda k: kernels[k]["ms"])
+    out = {"metric": "classifier tail (AverageLut fwd+bwd, softmax cross entropy, accuracy), ms per pass over 65536 frames", "value": totals[65536],
+           "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": totals[65536], "higher_is_better": False,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "AverageLut 7->1 over 70->10 nodes + LossSoftmaxCrossEntropy + MetricsCategoricalAccuracy, 65536 frames",
+                      "ms_at_1024_frames": totals[1024]},
+           "roofline": {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},
+           "kernels": kernels}
+    print(json.dumps(out))
+
+
 def bench_binarylut6(args, lib):
     """BinaryLut6 packed inference: 8192 -> 16384 nodes, 262144 frames, 32 frames per word (secondary measurement)."""
     import numpy as np
@@ -227,7 +283,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "adam", "conv"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "adam", "conv", "tail"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -248,6 +304,8 @@ def main():
         return bench_adam(args, lib)
     if args.workload == "conv":
         return bench_conv(args, lib)
+    if args.workload == "tail":
+        return bench_tail(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)

@@ -52,6 +52,11 @@ _SIGNATURES = {
     "bbhip_fp32_Col2Im_Backward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_fp32_StochasticMaxPooling2x2_Forward": (C.c_int, [_vp, _vp] + [_i] * 7 + [_vp]),
     "bbhip_fp32_StochasticMaxPooling2x2_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 7 + [_vp]),
+    "bbhip_fp32_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_bit_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
+    "bbhip_fp32_AverageLut_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 5 + [_vp]),
+    "bbhip_fp32_LossSoftmaxCrossEntropy": (C.c_int, [_vp, _vp, _vp, _vp, _f] + [_i] * 4 + [_vp]),
+    "bbhip_fp32_MetricsCategoricalAccuracy": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "bbhip_bit_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),

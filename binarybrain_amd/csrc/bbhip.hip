@@ -16,6 +16,7 @@
 #include "lut_kernels.hpp"
 #include "vector_kernels.hpp"
 #include "conv_kernels.hpp"
+#include "tail_kernels.hpp"
 
 using namespace bbhip;
 
@@ -885,6 +886,123 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
 {
     PoolArgs a{dev_x_buf, dev_dy_buf, dev_dx_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
     return launch_pool(a, true, stream, __func__);
+}
+
+static int check_average_lut(void const *a, void const *b, int const *idx, int n, int node_size, int frame_size, int frame_stride, int row_items,
+                             char const *name)
+{
+    if (!(a && b && idx)) { return fail("%s: null buffer", name); }
+    if (!(n > 0 && node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (frame_stride < row_items) { return fail("%s: frame stride shorter than the frames", name); }
+    if ((long long)node_size * n > 0x7fffffffLL) { return fail("%s: connection table too large", name); }
+    return 0;
+}
+
+int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                  int frame_stride, int binarize_input, int binarize_output, void *stream)
+{
+    if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
+    int const f_blocks = ceil_div(frame_size, kTailBlock);
+    long long const blocks = (long long)node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipLaunchKernelGGL(average_lut_forward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_x_buf,
+                       dev_y_buf, dev_input_index, n, frame_size, frame_stride, binarize_input, binarize_output, f_blocks);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                 int frame_stride, void *stream)
+{
+    int const words = (frame_size > 0) ? ceil_div(frame_size, 32) : 0;
+    if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, words, __func__)) { return 1; }
+    int const w_blocks = ceil_div(words, kTailBlock);
+    long long const blocks = (long long)node_size * w_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    int planes = 1;
+    while ((1 << planes) <= n && planes < 31) { ++planes; }      // planes = bits of n: counts 0..n fit
+    dim3 const grid((unsigned)blocks), block(kTailBlock);
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+#define BBHIP_AVERAGE_BIT(P) hipLaunchKernelGGL(average_lut_forward_bit_kernel<P>, grid, block, 0, st, dev_x_buf, dev_y_buf, dev_input_index, n, words, frame_stride, w_blocks)
+    switch (planes) {
+    case 1: BBHIP_AVERAGE_BIT(1); break;
+    case 2: BBHIP_AVERAGE_BIT(2); break;
+    case 3: BBHIP_AVERAGE_BIT(3); break;
+    case 4: BBHIP_AVERAGE_BIT(4); break;
+    case 5: BBHIP_AVERAGE_BIT(5); break;
+    case 6: BBHIP_AVERAGE_BIT(6); break;
+    case 7: BBHIP_AVERAGE_BIT(7); break;
+    case 8: BBHIP_AVERAGE_BIT(8); break;
+    default:
+        hipLaunchKernelGGL(average_lut_forward_bit_wide_kernel, grid, block, 0, st, dev_x_buf, dev_y_buf, dev_input_index, n, words, frame_stride, w_blocks);
+    }
+#undef BBHIP_AVERAGE_BIT
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
+                                   int output_node_size, int frame_size, int frame_stride, void *stream)
+{
+    if (check_average_lut(dev_dy_buf, dev_dx_buf, dev_input_index, n, output_node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
+    if (input_node_size <= 0) { return fail("%s: sizes must be positive", __func__); }
+    int const total = output_node_size * n;
+    int const f_blocks = ceil_div(frame_stride, kTailBlock);
+    long long const blocks = (long long)input_node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    char *scratch = nullptr;
+    size_t const offsets_bytes = align256(sizeof(int) * ((size_t)input_node_size + 1));
+    if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch)) { return 1; }
+    int *offsets = reinterpret_cast<int *>(scratch), *list = reinterpret_cast<int *>(scratch + offsets_bytes);
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(average_lut_reverse_kernel, dim3((unsigned)ceil_div(input_node_size + 1, kTailBlock)), dim3(kTailBlock), 0, st,
+                       dev_input_index, total, n, input_node_size, offsets, list);
+    BBHIP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(average_lut_backward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_dy_buf, dev_dx_buf, offsets, list, n,
+                       frame_size, frame_stride, f_blocks);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, float t_sum,
+                                       int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
+{
+    if (!(dev_y_buf && dev_t_buf && dev_dy_buf && dev_loss_buf)) { return fail("%s: null buffer", __func__); }
+    if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    if ((long long)pix_size * ch_size > 0x7fffffffLL) { return fail("%s: node count too large", __func__); }
+    int const f_blocks = ceil_div(frame_size, kTailBlock);
+    long long const blocks = (long long)pix_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    double *partial = dev_loss_buf;
+    if (pix_size > 1) {
+        char *scratch = nullptr;
+        if (arena_get(sizeof(double) * (size_t)pix_size * (size_t)frame_size, &scratch)) { return 1; }
+        partial = reinterpret_cast<double *>(scratch);
+    }
+    hipLaunchKernelGGL(softmax_cross_entropy_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_y_buf, dev_t_buf, dev_dy_buf, partial,
+                       t_sum, pix_size, ch_size, frame_size, frame_stride, f_blocks);
+    BBHIP_LAUNCH_CHECK();
+    if (pix_size > 1) {
+        hipLaunchKernelGGL(loss_pixel_sum_kernel, dim3((unsigned)f_blocks), dim3(kTailBlock), 0, st, partial, dev_loss_buf, pix_size, frame_size);
+        BBHIP_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *dev_t_buf, int *dev_accuracy_buf, int *dev_category_buf,
+                                          int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
+{
+    if (!(dev_y_buf && dev_t_buf && dev_accuracy_buf && dev_category_buf)) { return fail("%s: null buffer", __func__); }
+    if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    if ((long long)pix_size * ch_size > 0x7fffffffLL) { return fail("%s: node count too large", __func__); }
+    hipLaunchKernelGGL(categorical_accuracy_kernel, dim3((unsigned)ceil_div(frame_size, kTailBlock)), dim3(kTailBlock), 0,
+                       static_cast<hipStream_t>(stream), dev_y_buf, dev_t_buf, dev_accuracy_buf, dev_category_buf, pix_size, ch_size, frame_size,
+                       frame_stride);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
 }
 
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,

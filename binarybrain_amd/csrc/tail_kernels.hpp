@@ -1,0 +1,195 @@
+// The tail of a LUT classifier: AverageLut (sum / vote over n wired inputs), softmax cross entropy and categorical accuracy.
+//
+// All of it is streaming work over node-major, frame-minor buffers: one lane per frame (or per 32-frame word), rows read
+// as contiguous runs.  Results follow the reference's host loops (include/bb/AverageLut.h:320-345, 386-406;
+// LossSoftmaxCrossEntropy.h:159-211; MetricsCategoricalAccuracy.h:144-173): AverageLut writes the SUM when the output is
+// not binarized, gradients are dy / n added node ascending then input ascending, each product that the host code rounds
+// on its own is rounded on its own here.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "vector_kernels.hpp"
+
+namespace bbhip {
+
+constexpr int kTailBlock = 256;
+
+// one thread per (output node, frame)
+__global__ __launch_bounds__(kTailBlock) void average_lut_forward_kernel(float const *x, float *y, int const *idx, int n, int frame_size,
+                                                                         int frame_stride, int binarize_input, int binarize_output, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const node = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    int const *row = idx + (size_t)node * n;
+    float sum = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        float v = x[(size_t)row[i] * frame_stride + f];
+        if (binarize_input) { v = (v > 0.0f) ? 1.0f : -1.0f; }
+        sum += v;
+    }
+    if (binarize_output) { sum = (sum > 0.0f) ? 1.0f : -1.0f; }
+    y[(size_t)node * frame_stride + f] = sum;
+}
+
+// Packed bits, one thread per (output node, 32-frame word): the n input words are added into P bit planes (plane p holds
+// bit p of each frame's count of ones) and the count is compared with floor(n / 2): ones > n / 2 is the strict majority
+// that the host loop computes as (ones - zeros) > 0.
+template <int P>
+__global__ __launch_bounds__(kTailBlock) void average_lut_forward_bit_kernel(int const *x, int *y, int const *idx, int n, int words,
+                                                                             int frame_stride, int w_blocks)
+{
+    int const w = (int)(blockIdx.x % w_blocks) * kTailBlock + threadIdx.x;
+    int const node = blockIdx.x / w_blocks;
+    if (w >= words) { return; }
+    int const *row = idx + (size_t)node * n;
+    uint32_t plane[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) { plane[p] = 0u; }
+    for (int i = 0; i < n; ++i) {
+        uint32_t carry = (uint32_t)x[(size_t)row[i] * frame_stride + w];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            uint32_t const t = plane[p] & carry;
+            plane[p] ^= carry;
+            carry = t;
+        }
+    }
+    uint32_t const threshold = (uint32_t)n >> 1;
+    uint32_t gt = 0u, eq = ~0u;
+#pragma unroll
+    for (int p = P - 1; p >= 0; --p) {
+        uint32_t const tb = ((threshold >> p) & 1u) ? ~0u : 0u;
+        gt |= eq & plane[p] & ~tb;
+        eq &= ~(plane[p] ^ tb);
+    }
+    y[(size_t)node * frame_stride + w] = (int)gt;
+}
+
+// any n: per frame bit, count the ones directly
+__global__ __launch_bounds__(kTailBlock) void average_lut_forward_bit_wide_kernel(int const *x, int *y, int const *idx, int n, int words,
+                                                                                  int frame_stride, int w_blocks)
+{
+    int const w = (int)(blockIdx.x % w_blocks) * kTailBlock + threadIdx.x;
+    int const node = blockIdx.x / w_blocks;
+    if (w >= words) { return; }
+    int const *row = idx + (size_t)node * n;
+    uint32_t out = 0u;
+    for (int base = 0; base < 32; base += 4) {               // four frame bits per sweep over the inputs
+        int ones[4] = {0, 0, 0, 0};
+        for (int i = 0; i < n; ++i) {
+            uint32_t const v = (uint32_t)x[(size_t)row[i] * frame_stride + w] >> base;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) { ones[b] += (int)((v >> b) & 1u); }
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) { out |= (2 * ones[b] > n) ? (1u << (base + b)) : 0u; }
+    }
+    y[(size_t)node * frame_stride + w] = (int)out;
+}
+
+// Reverse wiring for the backward pass, built on the device: for input node i, offsets[i] = number of table entries that
+// name a smaller input, and list[offsets[i] ...] = the output nodes wired to i in table order (node ascending, input
+// position ascending).  One thread per input node (plus one for the end offset) sweeps the whole table twice; the sweeps
+// read the same entry in every lane, so they run on the scalar unit.  Entries outside [0, input_node_size) match no thread.
+__global__ __launch_bounds__(kTailBlock) void average_lut_reverse_kernel(int const *__restrict__ idx, int total, int n, int input_node_size,
+                                                                         int *__restrict__ offsets, int *__restrict__ list)
+{
+    int const i = blockIdx.x * kTailBlock + threadIdx.x;
+    if (i > input_node_size) { return; }
+    int below = 0;
+    for (int e = 0; e < total; ++e) { below += ((uint32_t)idx[e] < (uint32_t)i) ? 1 : 0; }
+    offsets[i] = below;
+    if (i == input_node_size) { return; }
+    int at = below;
+    for (int e = 0; e < total; ++e) {
+        if (idx[e] == i) { list[at++] = e / n; }
+    }
+}
+
+// one thread per (input node, column of the row pitch): dx = sum over the wired output nodes, in table order, of dy / n
+__global__ __launch_bounds__(kTailBlock) void average_lut_backward_kernel(float const *dy, float *dx, int const *offsets, int const *list,
+                                                                          int n, int frame_size, int frame_stride, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const in = blockIdx.x / f_blocks;
+    if (f >= frame_stride) { return; }
+    if (f >= frame_size) { dx[(size_t)in * frame_stride + f] = 0.0f; return; }      // the row's padding reads as zero, as after the host's FillZero
+    int const begin = offsets[in], end = offsets[in + 1];
+    float const fn = (float)n;
+    float acc = 0.0f;
+    for (int k = begin; k < end; ++k) { acc += dy[(size_t)list[k] * frame_stride + f] / fn; }
+    dx[(size_t)in * frame_stride + f] = acc;
+}
+
+// Softmax cross entropy, one thread per (pixel, frame); node = ch * pix_size + pix.  partial[pix * frame_size + frame]
+// receives sum over the channels with t > 0 of log(softmax + eps) * t_max in double; with one pixel that is loss_buf itself.
+__global__ __launch_bounds__(kTailBlock) void softmax_cross_entropy_kernel(float const *y, float const *t, float *dy, double *partial,
+                                                                           float t_sum, int pix_size, int ch_size, int frame_size,
+                                                                           int frame_stride, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const pix = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    float const eps = 1.0e-7f;
+    size_t const node_step = (size_t)pix_size * frame_stride;
+    size_t const first = (size_t)pix * frame_stride + f;
+    float c = -3.402823466e+38f;
+    for (int ch = 0; ch < ch_size; ++ch) {
+        float const v = y[first + ch * node_step];
+        c = (c < v) ? v : c;
+    }
+    float y_sum = 0.0f, t_max = 0.0f;
+    for (int ch = 0; ch < ch_size; ++ch) {
+        y_sum += expf(y[first + ch * node_step] - c);
+        t_max += t[first + ch * node_step];
+    }
+    if (y_sum <= eps) { y_sum = eps; }
+    double loss = 0.0;
+    for (int ch = 0; ch < ch_size; ++ch) {
+        size_t const at = first + ch * node_step;
+        float const tv = t[at];
+        float const softmax = expf(y[at] - c) / y_sum;
+        if (tv > 0.0f) { loss += (double)rounded_mul(logf(softmax + eps), t_max); }
+        dy[at] = (rounded_mul(t_max, softmax) - tv) / t_sum;
+    }
+    partial[(size_t)pix * frame_size + f] = loss;
+}
+
+// loss_buf[frame] = sum over the pixels, ascending, of the per-pixel terms
+__global__ __launch_bounds__(kTailBlock) void loss_pixel_sum_kernel(double const *partial, double *loss_buf, int pix_size, int frame_size)
+{
+    int const f = blockIdx.x * kTailBlock + threadIdx.x;
+    if (f >= frame_size) { return; }
+    double loss = 0.0;
+    for (int pix = 0; pix < pix_size; ++pix) { loss += partial[(size_t)pix * frame_size + f]; }
+    loss_buf[f] = loss;
+}
+
+// Per frame: pixels with a positive target (category) and, of those, pixels whose first largest y sits on a channel with
+// a positive target (accuracy).  One thread per frame.
+__global__ __launch_bounds__(kTailBlock) void categorical_accuracy_kernel(float const *y, float const *t, int *accuracy_buf, int *category_buf,
+                                                                          int pix_size, int ch_size, int frame_size, int frame_stride)
+{
+    int const f = blockIdx.x * kTailBlock + threadIdx.x;
+    if (f >= frame_size) { return; }
+    size_t const node_step = (size_t)pix_size * frame_stride;
+    int accuracy = 0, category = 0;
+    for (int pix = 0; pix < pix_size; ++pix) {
+        size_t const first = (size_t)pix * frame_stride + f;
+        float max_y = -3.402823466e+38f, max_t = -3.402823466e+38f;
+        bool valid = false;
+        for (int ch = 0; ch < ch_size; ++ch) {
+            float const yv = y[first + ch * node_step], tv = t[first + ch * node_step];
+            valid = valid || (tv > 0.0f);
+            if (yv > max_y) { max_y = yv; max_t = tv; }
+        }
+        if (valid) { category += 1; accuracy += (max_t > 0.0f) ? 1 : 0; }
+    }
+    accuracy_buf[f] = accuracy;
+    category_buf[f] = category;
+}
+
+}  // namespace bbhip

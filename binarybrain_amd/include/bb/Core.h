@@ -21,6 +21,7 @@
 #define BB_TYPE_BIT     (0x0000 + 1)
 #define BB_TYPE_BINARY  (0x0000 + 2)
 #define BB_TYPE_FP32    (0x0100 + 32)
+#define BB_TYPE_FP64    (0x0100 + 64)
 #define BB_TYPE_INT32   (0x0200 + 32)
 #define BB_TYPE_UINT8   (0x0300 + 8)
 
@@ -57,6 +58,7 @@ public:
 
 template <typename T> struct DataType {};
 template <> struct DataType<float>        { static constexpr int type = BB_TYPE_FP32;  static constexpr int bits = 32; static std::string Name() { return "fp32"; } };
+template <> struct DataType<double>       { static constexpr int type = BB_TYPE_FP64;  static constexpr int bits = 64; static std::string Name() { return "fp64"; } };
 template <> struct DataType<std::int32_t> { static constexpr int type = BB_TYPE_INT32; static constexpr int bits = 32; static std::string Name() { return "int32"; } };
 template <> struct DataType<std::uint8_t> { static constexpr int type = BB_TYPE_UINT8; static constexpr int bits = 8;  static std::string Name() { return "uint8"; } };
 template <> struct DataType<Bit>          { static constexpr int type = BB_TYPE_BIT;   static constexpr int bits = 1;  static std::string Name() { return "bit"; } };
@@ -67,6 +69,7 @@ inline int DataType_GetBitSize(int type)
     case BB_TYPE_BIT:   return 1;
     case BB_TYPE_UINT8: return 8;
     case BB_TYPE_FP32:  return 32;
+    case BB_TYPE_FP64:  return 64;
     case BB_TYPE_INT32: return 32;
     }
     throw Exception("unsupported data type code " + std::to_string(type));

@@ -120,6 +120,24 @@ public:
     void  SetBit(index_t frame, index_t node, bool v)   { Lock<Bit>().Set(frame, node, Bit(v)); }
     bool  GetBit(index_t frame, index_t node) const     { return (bool)LockConst<Bit>().Get(frame, node); }
 
+    // sum of all elements in double, taken on the host (reference: Tensor_<T>::Sum, include/bb/Tensor.h:918-926)
+    double Sum(void) const
+    {
+        double sum = 0;
+        if (m_type == BB_TYPE_FP32) {
+            auto p = LockConst<float>();
+            for (index_t node = 0; node < m_node_size; ++node) { float const *row = p.GetAddr(node); for (index_t f = 0; f < m_frame_size; ++f) { sum += row[f]; } }
+        }
+        else if (m_type == BB_TYPE_INT32) {
+            auto p = LockConst<std::int32_t>();
+            for (index_t node = 0; node < m_node_size; ++node) { std::int32_t const *row = p.GetAddr(node); for (index_t f = 0; f < m_frame_size; ++f) { sum += row[f]; } }
+        }
+        else {
+            throw Exception("FrameBuffer::Sum: fp32 and int32 buffers only");
+        }
+        return sum;
+    }
+
     // packed bits -> fp32 0/1 on the device (reference: FrameBuffer::ConvertTo, include/bb/FrameBuffer.h:838-900)
     FrameBuffer ConvertBitToFP32(void) const
     {

@@ -186,6 +186,55 @@ def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
     return dx
 
 
+def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
+    """fp32 x [I, stride] -> y [O, stride]: sum of the n wired inputs (their votes when binarize_input), or its sign."""
+    _dev(x, idx)
+    O, n = idx.shape
+    y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_AverageLut_Forward(ptr(x), ptr(y), ptr(idx), n, O, frame_size, x.shape[1], int(binarize_input),
+                                              int(binarize_output), stream_ptr()))
+    return y
+
+
+def bit_average_lut_forward(xbits, idx, frame_size):
+    """packed x [I, words] -> packed y [O, words]: strict majority of the n wired inputs."""
+    _dev(xbits, idx)
+    O, n = idx.shape
+    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    check(lib().bbhip_bit_AverageLut_Forward(ptr(xbits), ptr(y), ptr(idx), n, O, frame_size, xbits.shape[1], stream_ptr()))
+    return y
+
+
+def average_lut_backward(dy, idx, input_nodes, frame_size):
+    _dev(dy, idx)
+    O, n = idx.shape
+    dx = torch.empty((input_nodes, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_AverageLut_Backward(ptr(dy), ptr(dx), ptr(idx), n, input_nodes, O, frame_size, dy.shape[1], stream_ptr()))
+    return dx
+
+
+def loss_softmax_cross_entropy(y, t, ch_size, pix_size, frame_size, t_sum=None):
+    """y, t [ch*pix, stride] -> (dy, loss_buf [frames] float64, t_sum).  t_sum defaults to the sum of the targets of the
+    frames in use, taken in float64 as the reference's device path does; the loss of the batch is -loss_buf.sum() / t_sum."""
+    _dev(y, t)
+    if t_sum is None:
+        t_sum = float(t[:, :frame_size].sum(dtype=torch.float64).item())
+    dy = torch.empty_like(y)
+    loss_buf = torch.empty((frame_size,), dtype=torch.float64, device=y.device)
+    check(lib().bbhip_fp32_LossSoftmaxCrossEntropy(ptr(y), ptr(t), ptr(dy), ptr(loss_buf), t_sum, pix_size, ch_size, frame_size, y.shape[1],
+                                                   stream_ptr()))
+    return dy, loss_buf, t_sum
+
+
+def metrics_categorical_accuracy(y, t, ch_size, pix_size, frame_size):
+    """-> (accuracy_buf, category_buf) int32 [frames]; the metric of the batch is the ratio of their sums."""
+    _dev(y, t)
+    acc = torch.empty((frame_size,), dtype=torch.int32, device=y.device)
+    cat = torch.empty((frame_size,), dtype=torch.int32, device=y.device)
+    check(lib().bbhip_fp32_MetricsCategoricalAccuracy(ptr(y), ptr(t), ptr(acc), ptr(cat), pix_size, ch_size, frame_size, y.shape[1], stream_ptr()))
+    return acc, cat
+
+
 def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
     _dev(xbits)
     y = torch.empty((xbits.shape[0], y_stride), dtype=torch.float32, device=xbits.device)

@@ -161,6 +161,34 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
                                                 int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
                                                 int frame_stride, void *stream);
 
+/* ---- AverageLut, softmax cross entropy, categorical accuracy (the tail of a LUT classifier) ---- */
+/* bbcu_AverageLut_Forward<float>, include/bbcu/bbcu.h:321-334.  y = sum over the n inputs dev_input_index[node*n + i] of x (each
+ * replaced by +1 / -1 on x > 0 when binarize_input), written as +1 / -1 on sum > 0 when binarize_output.  Without
+ * binarize_output the SUM is written, as by the reference's host loop (include/bb/AverageLut.h:331-343); its CUDA kernel
+ * writes sum / n (cuda/AverageLut.cu:46-54). */
+int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                  int frame_stride, int binarize_input, int binarize_output, void *stream);
+/* bbcu_bit_AverageLut_Forward, include/bbcu/bbcu.h:336-346: packed bits, y = strict majority of the n inputs (a tie of an even
+ * n gives 0); frame_stride in 32-bit words */
+int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                 int frame_stride, void *stream);
+/* bbcu_AverageLut_Backward<float>, include/bbcu/bbcu.h:348-361: dx[input] = sum of dy[node] / n over the table entries that name the
+ * input, in table order (the order of the host loop, include/bb/AverageLut.h:395-404); inputs that no node names, and
+ * the padding of every row, are written as 0.  Deterministic: the reverse wiring is built on the device in library scratch. */
+int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
+                                   int output_node_size, int frame_size, int frame_stride, void *stream);
+/* bbcu_LossSoftmaxCrossEntropy<float>, include/bbcu/bbcu.h:1506-1519.  Nodes are [ch][pix]; per frame and pixel softmax over the
+ * channels; dev_loss_buf[frame] = sum over pixels and channels with t > 0 of log(softmax + 1e-7) * t_max (t_max = sum of the pixel's
+ * targets), dy = (t_max * softmax - t) / t_sum.  The caller passes t_sum = sum of all targets and reports
+ * -sum(dev_loss_buf) / t_sum (include/bb/LossSoftmaxCrossEntropy.h:99-125, 159-219).  dy is divided by t_sum as on the host path;
+ * the CUDA kernel multiplies by its reciprocal. */
+int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, float t_sum,
+                                       int pix_size, int ch_size, int frame_size, int frame_stride, void *stream);
+/* bbcu_MetricsCategoricalAccuracy<float>, include/bbcu/bbcu.h:1540-1553: per frame, dev_category_buf = pixels with a positive target,
+ * dev_accuracy_buf = those of them whose first largest y sits on a channel with a positive target */
+int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *dev_t_buf, int *dev_accuracy_buf, int *dev_category_buf,
+                                          int pix_size, int ch_size, int frame_size, int frame_stride, void *stream);
+
 /* ---- StochasticLut ---- */
 /* bbcu_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:667-681 */
 int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,

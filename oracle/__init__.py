@@ -187,6 +187,63 @@ def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
     return dx
 
 
+def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
+    """fp32 x [I, stride] -> y [O, stride]: sum (or its sign) of the n wired inputs."""
+    x = _c(x, np.float32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    y = np.zeros((O, x.shape[1]), np.float32)
+    lib().oracle_fp32_AverageLut_Forward(_ptr(x), _ptr(y), _ptr(idx), C.c_int(n), C.c_int(O), C.c_int(frame_size), C.c_int(x.shape[1]),
+                                         C.c_int(int(binarize_input)), C.c_int(int(binarize_output)))
+    return y
+
+
+def bit_average_lut_forward(xbits, idx, frame_size):
+    """packed x [I, words] -> packed y [O, words]: strict majority of the n wired inputs."""
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    y = np.zeros((O, xbits.shape[1]), np.int32)
+    lib().oracle_bit_AverageLut_Forward(_ptr(xbits), _ptr(y), _ptr(idx), C.c_int(n), C.c_int(O), C.c_int(frame_size), C.c_int(xbits.shape[1]))
+    return y
+
+
+def average_lut_backward(dy, idx, input_node_size, frame_size):
+    dy = _c(dy, np.float32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    dx = np.zeros((input_node_size, dy.shape[1]), np.float32)
+    lib().oracle_fp32_AverageLut_Backward(_ptr(dy), _ptr(dx), _ptr(idx), C.c_int(n), C.c_int(input_node_size), C.c_int(O),
+                                          C.c_int(frame_size), C.c_int(dy.shape[1]))
+    return dx
+
+
+def loss_t_sum(t, frame_size):
+    t = _c(t, np.float32)
+    f = lib().oracle_fp32_LossSoftmaxCrossEntropy_TSum
+    f.restype = C.c_float
+    return float(f(_ptr(t), C.c_int(t.shape[0]), C.c_int(frame_size), C.c_int(t.shape[1])))
+
+
+def loss_softmax_cross_entropy(y, t, ch_size, pix_size, frame_size, t_sum=None):
+    """y, t [ch*pix, stride] -> (dy [ch*pix, stride], loss_buf [frames] float64, t_sum).  The loss of the batch is
+    -loss_buf.sum() / t_sum."""
+    y = _c(y, np.float32); t = _c(t, np.float32)
+    if t_sum is None:
+        t_sum = loss_t_sum(t, frame_size)
+    dy = np.zeros_like(y)
+    loss_buf = np.zeros(frame_size, np.float64)
+    lib().oracle_fp32_LossSoftmaxCrossEntropy(_ptr(y), _ptr(t), _ptr(dy), _ptr(loss_buf), C.c_float(t_sum), C.c_int(pix_size),
+                                              C.c_int(ch_size), C.c_int(frame_size), C.c_int(y.shape[1]))
+    return dy, loss_buf, t_sum
+
+
+def metrics_categorical_accuracy(y, t, ch_size, pix_size, frame_size):
+    """-> (accuracy_buf, category_buf) int32 [frames]; the metric of the batch is their sums' ratio."""
+    y = _c(y, np.float32); t = _c(t, np.float32)
+    acc = np.zeros(frame_size, np.int32); cat = np.zeros(frame_size, np.int32)
+    lib().oracle_fp32_MetricsCategoricalAccuracy(_ptr(y), _ptr(t), _ptr(acc), _ptr(cat), C.c_int(pix_size), C.c_int(ch_size),
+                                                 C.c_int(frame_size), C.c_int(y.shape[1]))
+    return acc, cat
+
+
 def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, simd=True):
     """fp32 x [I, stride] -> y [O, stride] (padding columns zero)."""
     x = _c(x, np.float32); idx = _c(idx, np.int32); W = _c(W, np.float32)
@@ -501,6 +558,32 @@ def ref_stochastic_maxpool2x2(x, c, h, w, frames, dy=None):
         dy = _c(dy, np.float32); dx = np.zeros((c * h * w, frames), np.float32)
     assert ref().bbref_StochasticMaxPooling2x2(C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(frames), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx)) == 0
     return y, dx
+
+
+def ref_average_lut(x, idx, input_node_size, frames, bit=False, binarize_input=False, binarize_output=True, dy=None):
+    """The reference's AverageLut host path on dense [nodes, frames] (or [nodes, words]) arrays -> (y, dx)."""
+    idx = _c(idx, np.int32)
+    O, n = idx.shape
+    if bit:
+        x = _c(x, np.int32); y = np.zeros((O, (frames + 31) // 32), np.int32)
+    else:
+        x = _c(x, np.float32); y = np.zeros((O, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((input_node_size, frames), np.float32)
+    assert ref().bbref_AverageLut(C.c_int(int(bit)), C.c_int(n), C.c_int(input_node_size), C.c_int(O), C.c_int(frames), _ptr(x), _ptr(idx),
+                                  C.c_int(int(binarize_input)), C.c_int(int(binarize_output)), _ptr(y), _ptr(dy), _ptr(dx)) == 0
+    return y, dx
+
+
+def ref_loss_and_accuracy(y, t, ch_size, pix_size, frames):
+    """The reference's LossSoftmaxCrossEntropy and MetricsCategoricalAccuracy host paths -> (dy, loss, metric)."""
+    y = _c(y, np.float32); t = _c(t, np.float32)
+    dy = np.zeros((ch_size * pix_size, frames), np.float32)
+    loss = C.c_double(0); metric = C.c_double(0)
+    assert ref().bbref_LossAndAccuracy(C.c_int(ch_size), C.c_int(pix_size), C.c_int(frames), _ptr(y), _ptr(t), _ptr(dy),
+                                       C.byref(loss), C.byref(metric)) == 0
+    return dy, loss.value, metric.value
 
 
 def time_stochastic_lut6(x, dy, idx, W, reps=3, use_ref=None):

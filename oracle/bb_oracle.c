@@ -917,3 +917,127 @@ void oracle_fp32_StochasticMaxPooling2x2_Backward(float const *x, float const *d
         }
     }
 }
+
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ * AverageLut, LossSoftmaxCrossEntropy, MetricsCategoricalAccuracy: the host loops of the reference.
+ *
+ * Pinned by: bit-exact agreement with the reference's own classes (oracle/_ref) and the vectors written from them
+ * (tests/golden/tail.npz); the NumPy known answers held by the reference's loss test
+ * (tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-92: loss 2.29783..., dy table, tolerances 1e-4 / 1e-6); closed forms
+ * (AverageLut of +-1 inputs = sign of the count; backward column sums = n * dy / n; softmax rows sum to 1 so each
+ * frame's dy sums to (t_max - sum t)/t_sum = 0 for one-hot targets; uniform logits give loss log(ch); accuracy of
+ * y = t is 1).
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+/* AverageLut.h:320-345 (host loop; the value written without binarize_output is the SUM, not the mean) */
+void oracle_fp32_AverageLut_Forward(float const *x, float *y, int32_t const *idx, int n, int node_size, int frame_size,
+                                    int frame_stride, int binarize_input, int binarize_output)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float sum = 0;
+            for (int i = 0; i < n; ++i) {
+                float val = x[(long long)idx[node * n + i] * frame_stride + f];
+                if (binarize_input) { val = (val > 0) ? 1.0f : -1.0f; }
+                sum += val;
+            }
+            if (binarize_output) { sum = (sum > 0) ? 1.0f : -1.0f; }
+            y[(long long)node * frame_stride + f] = sum;
+        }
+    }
+}
+
+/* The same loop on packed bits: a Bit reads as +1 / -1 (DataType.h:302-303) and is written as (sum > 0)
+ * (DataType.h:277-278), so the flags do not matter and the result is the strict majority of the n inputs. */
+void oracle_bit_AverageLut_Forward(int const *x, int *y, int32_t const *idx, int n, int node_size, int frame_size,
+                                   int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float sum = 0;
+            for (int i = 0; i < n; ++i) {
+                sum += get_bit(x + (long long)idx[node * n + i] * frame_stride, f) ? 1.0f : -1.0f;
+            }
+            set_bit(y + (long long)node * frame_stride, f, sum > 0);
+        }
+    }
+}
+
+/* AverageLut.h:386-406: dx = 0, then node ascending, input ascending: dx[input] += dy / n */
+void oracle_fp32_AverageLut_Backward(float const *dy, float *dx, int32_t const *idx, int n, int input_node_size,
+                                     int output_node_size, int frame_size, int frame_stride)
+{
+    memset(dx, 0, sizeof(float) * (size_t)input_node_size * (size_t)frame_stride);
+    for (int node = 0; node < output_node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float const g = dy[(long long)node * frame_stride + f] / n;
+            for (int i = 0; i < n; ++i) {
+                dx[(long long)idx[node * n + i] * frame_stride + f] += g;
+            }
+        }
+    }
+}
+
+/* LossSoftmaxCrossEntropy.h:150-156: the host path's sum of the targets, frame outer, node inner, in float */
+float oracle_fp32_LossSoftmaxCrossEntropy_TSum(float const *t, int node_size, int frame_size, int frame_stride)
+{
+    float t_sum = 0;
+    for (int f = 0; f < frame_size; ++f) {
+        for (int node = 0; node < node_size; ++node) { t_sum += t[(long long)node * frame_stride + f]; }
+    }
+    return t_sum;
+}
+
+/* LossSoftmaxCrossEntropy.h:159-211: node = ch * pix_size + pix; per frame loss_buf += log(softmax + eps) * t_max over
+ * the channels with t > 0; dy = (t_max * softmax - t) / t_sum.  The caller negates and sums loss_buf (:213-219). */
+void oracle_fp32_LossSoftmaxCrossEntropy(float const *y, float const *t, float *dy, double *loss_buf, float t_sum,
+                                         int pix_size, int ch_size, int frame_size, int frame_stride)
+{
+    float const eps = 1.0e-7f;
+    for (int f = 0; f < frame_size; ++f) {
+        loss_buf[f] = 0;
+        for (int pix = 0; pix < pix_size; ++pix) {
+            float c = -3.402823466e+38f;
+            for (int ch = 0; ch < ch_size; ++ch) {
+                float const v = y[(long long)(ch * pix_size + pix) * frame_stride + f];
+                c = (c < v) ? v : c;                                           /* std::max(c, v) */
+            }
+            float y_sum = 0, t_max = 0;
+            for (int ch = 0; ch < ch_size; ++ch) {
+                long long const at = (long long)(ch * pix_size + pix) * frame_stride + f;
+                y_sum += expf(y[at] - c);
+                t_max += t[at];
+            }
+            if (y_sum <= eps) { y_sum = eps; }
+            for (int ch = 0; ch < ch_size; ++ch) {
+                long long const at = (long long)(ch * pix_size + pix) * frame_stride + f;
+                float const softmax = expf(y[at] - c) / y_sum;
+                if (t[at] > 0) { loss_buf[f] += logf(softmax + eps) * t_max; }
+                dy[at] = (t_max * softmax - t[at]) / t_sum;
+            }
+        }
+    }
+}
+
+/* MetricsCategoricalAccuracy.h:144-173: per pixel the first channel holding the largest y decides; pixels whose targets
+ * are all <= 0 are not counted */
+void oracle_fp32_MetricsCategoricalAccuracy(float const *y, float const *t, int *accuracy_buf, int *category_buf,
+                                            int pix_size, int ch_size, int frame_size, int frame_stride)
+{
+    for (int f = 0; f < frame_size; ++f) {
+        int accuracy = 0, category = 0;
+        for (int pix = 0; pix < pix_size; ++pix) {
+            float max_y = -3.402823466e+38f, max_t = -3.402823466e+38f;
+            int valid = 0;
+            for (int ch = 0; ch < ch_size; ++ch) {
+                long long const at = (long long)(ch * pix_size + pix) * frame_stride + f;
+                if (t[at] > 0) { valid = 1; }
+                if (y[at] > max_y) { max_y = y[at]; max_t = t[at]; }
+            }
+            if (valid) { category += 1; if (max_t > 0) { accuracy += 1; } }
+        }
+        accuracy_buf[f] = accuracy;
+        category_buf[f] = category;
+    }
+}

@@ -26,6 +26,9 @@
 #include "bb/ConvolutionCol2Im.h"
 #include "bb/StochasticMaxPooling2x2.h"
 #include "bb/TensorOperator.h"
+#include "bb/AverageLut.h"
+#include "bb/LossSoftmaxCrossEntropy.h"
+#include "bb/MetricsCategoricalAccuracy.h"
 
 namespace {
 
@@ -425,4 +428,58 @@ extern "C" int bbref_StochasticMaxPooling2x2(int c, int h, int w, int frames, fl
     return 0;
 }
 
-  // extern "C"
+// AverageLut<BinType, float> (host path).  x: [I][frames] (fp32) or [I][words] (bits); y likewise for O nodes.
+namespace {
+template <typename BinType>
+int run_average_lut(int n, int I, int O, int F, void const *x, std::int32_t const *idx, int binarize_input, int binarize_output,
+                    void *y, float const *dy, float *dx)
+{
+    auto m = bb::AverageLut<BinType, float>::Create(n, bb::indices_t({(index_t)O}));
+    m->SendCommand("host_only true");
+    m->SendCommand("binarize_input " + onoff(binarize_input));
+    m->SendCommand("binarize_output " + onoff(binarize_output));
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)I}), xtype, true);
+    m->SetInputShape(xb.GetShape());
+    for (int o = 0; o < O; ++o) { for (int i = 0; i < n; ++i) { m->SetNodeConnectionIndex(o, i, idx[o * n + i]); } }
+    if (xtype == BB_TYPE_BIT) { put_bit(xb, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(xb, (float const *)x, I, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (xtype == BB_TYPE_BIT) { get_bit(yb, (std::int32_t *)y, O, (F + 31) / 32); }
+    else                      { get_fp32(yb, (float *)y, O, F); }
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, bb::indices_t({(index_t)O}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, O, F);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, I, F);
+    }
+    return 0;
+}
+}  // namespace
+
+extern "C" int bbref_AverageLut(int bit, int n, int I, int O, int F, void const *x, std::int32_t const *idx, int binarize_input,
+                                int binarize_output, void *y, float const *dy, float *dx)
+{
+    return bit ? run_average_lut<bb::Bit>(n, I, O, F, x, idx, binarize_input, binarize_output, y, dy, dx)
+               : run_average_lut<float>(n, I, O, F, x, idx, binarize_input, binarize_output, y, dy, dx);
+}
+
+// LossSoftmaxCrossEntropy<float> and MetricsCategoricalAccuracy<float> (host paths) on [ch][pix] nodes.
+// loss = GetLoss(), metric = GetMetrics() after one batch.
+extern "C" int bbref_LossAndAccuracy(int ch, int pix, int F, float const *y, float const *t, float *dy, double *loss, double *metric)
+{
+    bb::indices_t const shape({(index_t)ch, (index_t)pix});
+    bb::FrameBuffer yb((index_t)F, shape, BB_TYPE_FP32, true), tb((index_t)F, shape, BB_TYPE_FP32, true);
+    put_fp32(yb, y, (index_t)ch * pix, F);
+    put_fp32(tb, t, (index_t)ch * pix, F);
+    auto lossFunc = bb::LossSoftmaxCrossEntropy<float>::Create();
+    lossFunc->Clear();
+    bb::FrameBuffer dyb = lossFunc->CalculateLoss(yb, tb, (index_t)F);
+    get_fp32(dyb, dy, (index_t)ch * pix, F);
+    *loss = lossFunc->GetLoss();
+    auto metrics = bb::MetricsCategoricalAccuracy<float>::Create();
+    metrics->Clear();
+    metrics->CalculateMetrics(yb, tb);
+    *metric = metrics->GetMetrics();
+    return 0;
+}

@@ -14,8 +14,14 @@
 #include "bb/ConvolutionIm2Col.h"
 #include "bb/ConvolutionCol2Im.h"
 #include "bb/StochasticMaxPooling2x2.h"
+#include "bb/AverageLut.h"
+#include "bb/LossSoftmaxCrossEntropy.h"
+#include "bb/MetricsCategoricalAccuracy.h"
 
 extern "C" {
+void oracle_fp32_AverageLut_Forward(float const *x, float *y, std::int32_t const *idx, int n, int node_size, int frame_size, int frame_stride, int binarize_input, int binarize_output);
+void oracle_bit_AverageLut_Forward(int const *x, int *y, std::int32_t const *idx, int n, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_AverageLut_Backward(float const *dy, float *dx, std::int32_t const *idx, int n, int input_node_size, int output_node_size, int frame_size, int frame_stride);
 void oracle_fp32_Im2Col_Backward(float const *dy, float *dx, int x_stride, int y_stride, int x_offset, int y_offset, int input_frame_size,
                                  int input_frame_stride, int w, int h, int c, int ow, int oh, int output_frame_stride, int fw, int fh);
 void oracle_fp32_StochasticMaxPooling2x2_Forward(float const *x, float *y, int w, int h, int ow, int oh, int c, int frame_size, int frame_stride);
@@ -299,6 +305,90 @@ static void test_conv_plumbing(void)
     CHECK(bad == 0, "StochasticMaxPooling2x2 backward: %zu wrong", bad);
 }
 
+// The tail of a classifier through the host classes: AverageLut against the oracle, and the reference's own known-answer test
+// of the loss (tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-92, NumPy goldens: loss within 1e-4, dy within 1e-6).
+static void test_tail(void)
+{
+    int const n = 7, O = 10, I = 70, F = 100;
+    std::mt19937_64 mt(9);
+    std::uniform_real_distribution<float> uni(-1.0f, 1.0f);
+    std::vector<std::int32_t> idx((size_t)O * n);
+    for (auto &v : idx) { v = (std::int32_t)(mt() % (std::uint64_t)I); }
+    std::vector<float> x((size_t)I * F), dy((size_t)O * F), y_ref((size_t)O * F), dx_ref((size_t)I * F), got;
+    for (auto &v : x) { v = uni(mt); }
+    for (auto &v : dy) { v = uni(mt); }
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), dy_buf(F, {O}, BB_TYPE_FP32);
+    for (int i = 0; i < I; ++i) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, i, x[(size_t)i * F + f]); }
+    for (int o = 0; o < O; ++o) for (int f = 0; f < F; ++f) { dy_buf.SetFP32(f, o, dy[(size_t)o * F + f]); }
+    for (int binarize = 0; binarize < 2; ++binarize) {
+        auto avg = bb::AverageLut<>::Create(n, (bb::index_t)O, "", binarize != 0);
+        avg->SetInputShape({I});
+        for (int o = 0; o < O; ++o) for (int i = 0; i < n; ++i) { avg->SetNodeConnectionIndex(o, i, idx[(size_t)o * n + i]); }
+        bb::FrameBuffer y_buf = avg->Forward(x_buf);
+        oracle_fp32_AverageLut_Forward(x.data(), y_ref.data(), idx.data(), n, O, F, F, 0, binarize);
+        read_fp32(y_buf, got);
+        CHECK(got == y_ref, "AverageLut forward (binarize %d)", binarize);
+        bb::FrameBuffer dx_buf = avg->Backward(dy_buf);
+        oracle_fp32_AverageLut_Backward(dy.data(), dx_ref.data(), idx.data(), n, I, O, F, F);
+        read_fp32(dx_buf, got);
+        CHECK(got == dx_ref, "AverageLut backward");
+    }
+    {
+        auto avg = bb::AverageLut<bb::Bit>::Create(n, (bb::index_t)O);
+        avg->SetInputShape({I});
+        for (int o = 0; o < O; ++o) for (int i = 0; i < n; ++i) { avg->SetNodeConnectionIndex(o, i, idx[(size_t)o * n + i]); }
+        int const words = (F + 31) / 32;
+        std::vector<std::int32_t> xb((size_t)I * words, 0), yb_ref((size_t)O * words, 0);
+        bb::FrameBuffer xb_buf(F, {I}, BB_TYPE_BIT);
+        xb_buf.FillZero();
+        for (int i = 0; i < I; ++i) for (int f = 0; f < F; ++f) {
+            bool const v = x[(size_t)i * F + f] > 0;
+            if (v) { xb[(size_t)i * words + (f >> 5)] |= (std::int32_t)(1u << (f & 31)); }
+            xb_buf.SetBit(f, i, v);
+        }
+        bb::FrameBuffer yb_buf = avg->Forward(xb_buf);
+        oracle_bit_AverageLut_Forward(xb.data(), yb_ref.data(), idx.data(), n, O, F, words);
+        size_t bad = 0;
+        for (int o = 0; o < O; ++o) for (int f = 0; f < F; ++f) { bad += (yb_buf.GetBit(f, o) != (((yb_ref[(size_t)o * words + (f >> 5)] >> (f & 31)) & 1) != 0)); }
+        CHECK(bad == 0, "AverageLut bit forward: %zu wrong", bad);
+        CHECK(avg->GetLutTable(0, 0x0f) && !avg->GetLutTable(0, 0x07), "AverageLut table view: majority of 7 index bits");
+    }
+
+    float const x_table[5][10] = {
+        {0.03682449f, 0.7174495f, 0.9130372f, 0.6275032f, 0.11995261f, 0.25850186f, 0.9942376f, 0.23910977f, 0.75574166f, 0.38816985f},
+        {0.59729785f, 0.7654758f, 0.35820892f, 0.0122047f, 0.05050702f, 0.323845f, 0.6889169f, 0.16161442f, 0.06116614f, 0.769033f},
+        {0.94036084f, 0.25700864f, 0.73131865f, 0.58721095f, 0.78960747f, 0.29338115f, 0.36369365f, 0.5750651f, 0.81494033f, 0.05262487f},
+        {0.98256797f, 0.15146895f, 0.51034707f, 0.38718516f, 0.18072742f, 0.7927627f, 0.13334593f, 0.03729849f, 0.20618507f, 0.9241972f},
+        {0.713539f, 0.48547512f, 0.27168426f, 0.54288715f, 0.6140953f, 0.67773014f, 0.03847398f, 0.7239832f, 0.64887875f, 0.42749837f}};
+    int const x_label[5] = {2, 5, 6, 3, 4};
+    float const dx_table[5][10] = {
+        {0.01189111f, 0.02348626f, -0.17144011f, 0.02146598f, 0.01292184f, 0.0148421f, 0.03097572f, 0.01455706f, 0.02440304f, 0.016897f},
+        {0.02385998f, 0.02822986f, 0.01878603f, 0.01329129f, 0.01381026f, -0.18184856f, 0.02614928f, 0.01543317f, 0.01395825f, 0.02833046f},
+        {0.02876907f, 0.01452612f, 0.0233421f, 0.02020946f, 0.02474312f, 0.0150642f, -0.18383847f, 0.01996549f, 0.02537794f, 0.01184096f},
+        {0.03275547f, 0.01426731f, 0.02042683f, -0.18194023f, 0.01469092f, 0.02709271f, 0.01401107f, 0.01272795f, 0.01506971f, 0.03089824f},
+        {0.02392219f, 0.01904382f, 0.01537821f, 0.02016916f, -0.17834225f, 0.02308072f, 0.01217935f, 0.02417335f, 0.02242433f, 0.01797112f}};
+    bb::FrameBuffer y_buf(5, {10}, BB_TYPE_FP32), t_buf(5, {10}, BB_TYPE_FP32);
+    for (int i = 0; i < 5; ++i) for (int j = 0; j < 10; ++j) {
+        y_buf.SetFP32(i, j, x_table[i][j]);
+        t_buf.SetFP32(i, j, (j == x_label[i]) ? 1.0f : 0.0f);
+    }
+    auto lossFunc = bb::LossSoftmaxCrossEntropy<float>::Create();
+    lossFunc->Clear();
+    bb::FrameBuffer dyb = lossFunc->CalculateLoss(y_buf, t_buf, y_buf.GetFrameSize());
+    CHECK(std::fabs(lossFunc->GetLoss() - 2.297830009460449) < 0.0001, "loss %.9f, expected 2.297830009", lossFunc->GetLoss());
+    double worst = 0;
+    for (int i = 0; i < 5; ++i) for (int j = 0; j < 10; ++j) { worst = std::max(worst, (double)std::fabs(dyb.GetFP32(i, j) - dx_table[i][j])); }
+    CHECK(worst < 0.000001, "loss gradient off by %.3g", worst);
+    auto metrics = bb::MetricsCategoricalAccuracy<float>::Create();
+    metrics->CalculateMetrics(t_buf, t_buf);
+    CHECK(metrics->GetMetrics() == 1.0, "accuracy of the targets themselves: %f", metrics->GetMetrics());
+    metrics->Clear();
+    metrics->CalculateMetrics(y_buf, t_buf);
+    int hits = 0;
+    for (int i = 0; i < 5; ++i) { int best = 0; for (int j = 1; j < 10; ++j) { if (x_table[i][j] > x_table[i][best]) { best = j; } } hits += (best == x_label[i]); }
+    CHECK(metrics->GetMetrics() == hits / 5.0, "accuracy %f, expected %f", metrics->GetMetrics(), hits / 5.0);
+}
+
 int main(void)
 {
     if (!bb::Manager::IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
@@ -325,6 +415,7 @@ int main(void)
         test_import_layer();
         test_adam();
         test_conv_plumbing();
+        test_tail();
     }
     catch (std::exception const &e) {
         std::printf("exception: %s\n", e.what());

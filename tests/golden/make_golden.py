@@ -187,14 +187,62 @@ def conv_cases():
     np.savez_compressed(os.path.join(OUT, "conv.npz"), **cases)
 
 
+def tail_cases():
+    """AverageLut, LossSoftmaxCrossEntropy and MetricsCategoricalAccuracy of the reference (host paths)."""
+    rng = np.random.default_rng(20240611)
+    cases = {}
+    k = 0
+    # AverageLut::Backward runs `#pragma omp parallel for` over output nodes around an unsynchronised dx += (AverageLut.h:395-404):
+    # with several threads, nodes that share an input lose updates.  One thread gives the loop its serial meaning.
+    import ctypes
+    gomp = ctypes.CDLL("libgomp.so.1")
+    threads = gomp.omp_get_max_threads()
+    gomp.omp_set_num_threads(1)
+    for (n, I, O, F, bin_in, bin_out) in [(7, 70, 10, 37, False, True), (7, 70, 10, 37, False, False), (4, 9, 5, 64, True, True),
+                                          (6, 12, 16, 33, True, False), (1, 3, 3, 5, False, False), (8, 8, 2, 100, False, True)]:
+        idx = rng.integers(0, I, (O, n)).astype(np.int32)              # repeats allowed: AverageLut wiring need not be distinct
+        x = (rng.random((I, F)) * 2 - 1).astype(np.float32)
+        x[rng.random((I, F)) < 0.1] = 0.0                               # exact zeros sit on the binarize threshold
+        dy = rng.standard_normal((O, F)).astype(np.float32)
+        y, dx = oracle.ref_average_lut(x, idx, I, F, binarize_input=bin_in, binarize_output=bin_out, dy=dy)
+        xb = synth.bernoulli_bits(rng, I, F)
+        yb, _ = oracle.ref_average_lut(xb, idx, I, F, bit=True, binarize_input=bin_in, binarize_output=bin_out)
+        q = "a%d_" % k
+        cases.update({q + "geom": np.array([n, I, O, F, int(bin_in), int(bin_out)], np.int32), q + "idx": idx, q + "x": x, q + "dy": dy,
+                      q + "y": y, q + "dx": dx, q + "xbits": xb, q + "ybits": mask_bits(yb, F)})
+        k += 1
+    cases["average_count"] = np.array([k], np.int32)
+    gomp.omp_set_num_threads(threads)
+    k = 0
+    for (ch, pix, F, kind) in [(10, 1, 33, "onehot"), (10, 1, 64, "sharp"), (4, 6, 17, "onehot"), (3, 5, 20, "weighted"), (7, 1, 9, "ties")]:
+        y = (rng.standard_normal((ch * pix, F)) * (30.0 if kind == "sharp" else 1.0)).astype(np.float32)
+        t = np.zeros((ch * pix, F), np.float32)
+        for f in range(F):
+            for p in range(pix):
+                if kind == "weighted" and rng.random() < 0.3:
+                    continue                                            # an unlabeled pixel
+                c = int(rng.integers(0, ch))
+                t[c * pix + p, f] = 1.0 if kind != "weighted" else np.float32(rng.integers(1, 4) * 0.5)
+        if kind == "ties":
+            y = np.round(y)                                             # repeated maxima: the first channel decides
+        dy, loss, metric = oracle.ref_loss_and_accuracy(y, t, ch, pix, F)
+        q = "l%d_" % k
+        cases.update({q + "geom": np.array([ch, pix, F], np.int32), q + "y": y, q + "t": t, q + "dy": dy,
+                      q + "loss": np.array([loss], np.float64), q + "metric": np.array([metric], np.float64)})
+        k += 1
+    cases["loss_count"] = np.array([k], np.int32)
+    np.savez_compressed(os.path.join(OUT, "tail.npz"), **cases)
+
+
 if __name__ == "__main__":
     assert oracle.have_ref(), "build oracle/_ref first (make -C oracle ref)"
-    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam", "conv"]
+    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam", "conv", "tail"]
     if "stochastic" in which: stochastic_cases()
     if "differentiable" in which: differentiable_cases()
     if "binary" in which: binary_cases()
     if "adam" in which: adam_cases()
     if "conv" in which: conv_cases()
+    if "tail" in which: tail_cases()
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)), "bytes")

@@ -1,0 +1,182 @@
+"""GPU parity of AverageLut, LossSoftmaxCrossEntropy and MetricsCategoricalAccuracy (through the C ABI) against the CPU
+oracle.  AverageLut and the accuracy counts are sums in a fixed order, votes and integers: bit-exact.  The loss goes
+through exp and log, whose device and host library versions may differ in the last place: tolerances are written at
+the assertions."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from binarybrain_amd import synth
+from util import dev, host
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "tail.npz"))
+LOSS_RTOL = 1e-5      # batch loss, relative
+DY_ATOL = 2e-6        # dy * t_sum / t_max (softmax minus target, values in [-1, 1]), absolute
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from binarybrain_amd import ops as o
+    return o
+
+
+def _pad(a, stride):
+    out = np.zeros((a.shape[0], stride), a.dtype)
+    out[:, :a.shape[1]] = a
+    return out
+
+
+AVERAGE_SHAPES = [
+    # n, I, O, frames
+    (7, 70, 10, 1024),          # the tail of the MNIST classifier
+    (7, 70, 10, 37),
+    (4, 9, 5, 64),
+    (1, 3, 3, 5),
+    (8, 8, 2, 100),
+    (15, 200, 33, 300),
+    (16, 64, 7, 257),
+    (300, 40, 3, 70),           # more inputs than the bit-plane counter covers
+    (6, 6144, 1024, 130),
+]
+
+
+@pytest.mark.parametrize("shape", AVERAGE_SHAPES)
+def test_average_lut(ops, shape):
+    n, I, O, F = shape
+    rng = np.random.default_rng(sum(shape))
+    idx = rng.integers(0, I, (O, n)).astype(np.int32)
+    stride = synth.frame_stride_fp32(F)
+    x = _pad((rng.random((I, F)) * 2 - 1).astype(F32), stride)
+    x[rng.random(x.shape) < 0.05] = 0.0
+    dy = _pad(rng.standard_normal((O, F)).astype(F32), stride)
+    for bin_in in (False, True):
+        for bin_out in (False, True):
+            y = host(ops.average_lut_forward(dev(x), dev(idx), F, bin_in, bin_out))
+            assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, bin_in, bin_out)[:, :F]), (bin_in, bin_out)
+    dx = host(ops.average_lut_backward(dev(dy), dev(idx), I, F))
+    assert np.array_equal(dx, oracle.average_lut_backward(dy, idx, I, F))          # padding columns included: zero
+    xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))
+    yb = host(ops.bit_average_lut_forward(dev(xb), dev(idx), F))
+    assert np.array_equal(synth.unpack_bits(yb, F), synth.unpack_bits(oracle.bit_average_lut_forward(xb, idx, F), F))
+
+
+def test_average_lut_reference_vectors(ops):
+    for k in range(int(GOLD["average_count"][0])):
+        n, I, O, F, bin_in, bin_out = [int(v) for v in GOLD["a%d_geom" % k]]; q = "a%d_" % k
+        idx = GOLD[q + "idx"]
+        y = host(ops.average_lut_forward(dev(GOLD[q + "x"]), dev(idx), F, bool(bin_in), bool(bin_out)))
+        assert np.array_equal(y, GOLD[q + "y"]), k
+        dx = host(ops.average_lut_backward(dev(GOLD[q + "dy"]), dev(idx), I, F))
+        assert np.array_equal(dx, GOLD[q + "dx"]), k
+        yb = host(ops.bit_average_lut_forward(dev(GOLD[q + "xbits"]), dev(idx), F))
+        assert np.array_equal(synth.unpack_bits(yb, F), synth.unpack_bits(GOLD[q + "ybits"], F)), k
+
+
+def test_average_lut_serial_wiring_and_unused_inputs(ops):
+    # inputs [o*n, (o+1)*n) feed node o; the inputs after the last node feed nothing and receive a zero gradient
+    n, O, F = 7, 10, 200
+    I = n * O + 5
+    idx = np.arange(n * O, dtype=np.int32).reshape(O, n)
+    rng = np.random.default_rng(3)
+    stride = synth.frame_stride_fp32(F)
+    dy = _pad(rng.standard_normal((O, F)).astype(F32), stride)
+    dx = host(ops.average_lut_backward(dev(dy), dev(idx), I, F))
+    assert np.array_equal(dx[:n * O, :F], np.repeat(dy[:, :F] / F32(n), n, axis=0))
+    assert not dx[n * O:].any() and not dx[:, F:].any()
+
+
+def _targets(rng, ch, pix, F, weighted=False):
+    t = np.zeros((ch * pix, F), F32)
+    for f in range(F):
+        for p in range(pix):
+            if weighted and rng.random() < 0.3:
+                continue
+            t[int(rng.integers(0, ch)) * pix + p, f] = F32(rng.integers(1, 4) * 0.5) if weighted else 1.0
+    return t
+
+
+def _check_loss(ops, y, t, ch, pix, F, stride):
+    ys, ts = _pad(y, stride), _pad(t, stride)
+    dy_ref, lb_ref, t_sum = oracle.loss_softmax_cross_entropy(ys, ts, ch, pix, F)
+    dy, lb, t_sum_dev = ops.loss_softmax_cross_entropy(dev(ys), dev(ts), ch, pix, F)
+    assert t_sum_dev == t_sum
+    dy, lb = host(dy), host(lb)
+    t_max = max(float(t.reshape(ch, pix, F).sum(axis=0).max()), 1e-30)
+    assert np.abs(dy[:, :F] - dy_ref[:, :F]).max() * t_sum / t_max <= DY_ATOL
+    loss, loss_ref = -lb.sum() / t_sum, -lb_ref.sum() / t_sum
+    assert abs(loss - loss_ref) <= LOSS_RTOL * abs(loss_ref)
+    assert np.allclose(lb, lb_ref, rtol=LOSS_RTOL, atol=1e-6 * t_max)
+    acc, cat = ops.metrics_categorical_accuracy(dev(ys), dev(ts), ch, pix, F)
+    acc_ref, cat_ref = oracle.metrics_categorical_accuracy(ys, ts, ch, pix, F)
+    assert np.array_equal(host(acc), acc_ref) and np.array_equal(host(cat), cat_ref)
+    return loss, dy
+
+
+@pytest.mark.parametrize("shape", [(10, 1, 1024), (10, 1, 33), (4, 6, 17), (3, 5, 300), (2, 1, 1), (21, 64, 70), (1000, 1, 65)])
+@pytest.mark.parametrize("kind", ["onehot", "sharp", "weighted", "ties"])
+def test_loss_and_accuracy(ops, shape, kind):
+    ch, pix, F = shape
+    rng = np.random.default_rng(ch * 1000 + pix * 10 + F)
+    y = (rng.standard_normal((ch * pix, F)) * (30.0 if kind == "sharp" else 1.0)).astype(F32)
+    if kind == "ties":
+        y = np.round(y)
+    t = _targets(rng, ch, pix, F, weighted=(kind == "weighted"))
+    if not t.any():
+        t[0, 0] = 1
+    _check_loss(ops, y, t, ch, pix, F, synth.frame_stride_fp32(F))
+
+
+def test_loss_known_answers_of_the_reference_test(ops):
+    # tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-92: NumPy goldens, loss within 1e-4, dy within 1e-6
+    from test_oracle_tail import DX_TABLE, KNOWN_LOSS, known_answer_buffers
+    y, t = known_answer_buffers()
+    loss, dy = _check_loss(ops, y, t, 10, 1, 5, synth.frame_stride_fp32(5))
+    assert abs(loss - KNOWN_LOSS) < 1e-4
+    assert np.abs(dy[:, :5].T - DX_TABLE).max() < 1e-6
+
+
+def test_loss_and_accuracy_reference_vectors(ops):
+    for k in range(int(GOLD["loss_count"][0])):
+        ch, pix, F = [int(v) for v in GOLD["l%d_geom" % k]]; q = "l%d_" % k
+        loss, dy = _check_loss(ops, GOLD[q + "y"], GOLD[q + "t"], ch, pix, F, synth.frame_stride_fp32(F))
+        assert abs(loss - GOLD[q + "loss"][0]) <= LOSS_RTOL * abs(GOLD[q + "loss"][0])
+        t_sum = float(GOLD[q + "t"].sum(dtype=np.float64))
+        t_max = float(GOLD[q + "t"].reshape(ch, pix, F).sum(axis=0).max())
+        assert np.abs(dy[:, :F] - GOLD[q + "dy"]).max() * t_sum / t_max <= DY_ATOL
+        acc, cat = ops.metrics_categorical_accuracy(dev(GOLD[q + "y"]), dev(GOLD[q + "t"]), ch, pix, F)
+        assert int(host(acc).sum()) / int(host(cat).sum()) == GOLD[q + "metric"][0]
+
+
+def test_loss_size_independent_properties(ops):
+    # a batch as large as the benchmark's frames: one-hot dy sums to zero per pixel, equal logits give log(ch)
+    ch, pix, F = 10, 1, 8192
+    rng = np.random.default_rng(11)
+    stride = synth.frame_stride_fp32(F)
+    t = _pad(_targets(rng, ch, pix, F), stride)
+    y = _pad(rng.standard_normal((ch, F)).astype(F32), stride)
+    dy, lb, t_sum = ops.loss_softmax_cross_entropy(dev(y), dev(t), ch, pix, F)
+    assert t_sum == F
+    assert np.abs(host(dy)[:, :F].astype(np.float64).sum(axis=0)).max() * t_sum < 1e-6
+    dy0, lb0, _ = ops.loss_softmax_cross_entropy(dev(np.zeros_like(y)), dev(t), ch, pix, F)
+    assert abs(-host(lb0).sum() / t_sum - np.log(ch)) < 1e-5
+    acc, cat = ops.metrics_categorical_accuracy(dev(t), dev(t), ch, pix, F)
+    assert int(host(acc).sum()) == F and int(host(cat).sum()) == F
+
+
+def test_rejected_arguments(ops):
+    import torch
+    x = torch.zeros((4, 64), device="cuda"); idx = torch.zeros((2, 3), dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.average_lut_forward(x, idx, 0)                       # no frames
+    with pytest.raises(RuntimeError):
+        ops.average_lut_forward(x, idx, 65)                      # frames beyond the row pitch
+    with pytest.raises(RuntimeError):
+        ops.average_lut_backward(x[:2], idx, 0, 64)              # no input nodes
+    with pytest.raises(RuntimeError):
+        ops.loss_softmax_cross_entropy(x, x, 4, 1, 100, t_sum=1.0)
+    with pytest.raises(RuntimeError):
+        ops.metrics_categorical_accuracy(x, x, 4, 1, 0)

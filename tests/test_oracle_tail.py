@@ -1,0 +1,192 @@
+"""The oracle's AverageLut, LossSoftmaxCrossEntropy and MetricsCategoricalAccuracy, pinned without a GPU: vectors written by
+the reference's own host classes (tests/golden/tail.npz), the compiled reference where oracle/_ref is present, the NumPy
+known answers of the reference's loss test (tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-92) and closed forms."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from binarybrain_amd import synth
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "tail.npz"))
+F32 = np.float32
+
+
+def average_gold(k):
+    n, I, O, F, bin_in, bin_out = [int(v) for v in GOLD["a%d_geom" % k]]
+    return n, I, O, F, bool(bin_in), bool(bin_out)
+
+
+def test_average_lut_reference_vectors():
+    for k in range(int(GOLD["average_count"][0])):
+        n, I, O, F, bin_in, bin_out = average_gold(k); q = "a%d_" % k
+        idx = GOLD[q + "idx"]
+        assert np.array_equal(oracle.average_lut_forward(GOLD[q + "x"], idx, F, bin_in, bin_out), GOLD[q + "y"]), k
+        assert np.array_equal(oracle.average_lut_backward(GOLD[q + "dy"], idx, I, F), GOLD[q + "dx"]), k
+        yb = oracle.bit_average_lut_forward(GOLD[q + "xbits"], idx, F)
+        assert np.array_equal(synth.unpack_bits(yb, F), synth.unpack_bits(GOLD[q + "ybits"], F)), k
+
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref not built")
+def test_average_lut_against_compiled_reference():
+    rng = np.random.default_rng(5)
+    gomp = ctypes.CDLL("libgomp.so.1")
+    threads = gomp.omp_get_max_threads()
+    for (n, I, O, F) in [(7, 70, 10, 130), (3, 40, 33, 65), (9, 20, 4, 31)]:
+        idx = rng.integers(0, I, (O, n)).astype(np.int32)
+        x = (rng.random((I, F)) * 2 - 1).astype(F32)
+        dy = rng.standard_normal((O, F)).astype(F32)
+        for bin_in in (False, True):
+            for bin_out in (False, True):
+                # the reference's backward loses updates when its OpenMP threads share an input node: one thread
+                gomp.omp_set_num_threads(1)
+                y, dx = oracle.ref_average_lut(x, idx, I, F, binarize_input=bin_in, binarize_output=bin_out, dy=dy)
+                gomp.omp_set_num_threads(threads)
+                assert np.array_equal(oracle.average_lut_forward(x, idx, F, bin_in, bin_out), y)
+                assert np.array_equal(oracle.average_lut_backward(dy, idx, I, F), dx)
+        xb = synth.bernoulli_bits(rng, I, F)
+        yb, _ = oracle.ref_average_lut(xb, idx, I, F, bit=True)
+        assert np.array_equal(synth.unpack_bits(oracle.bit_average_lut_forward(xb, idx, F), F), synth.unpack_bits(yb, F))
+
+
+def test_average_lut_closed_forms():
+    rng = np.random.default_rng(6)
+    n, I, O, F = 5, 30, 12, 77
+    idx = np.stack([rng.choice(I, n, replace=False) for _ in range(O)]).astype(np.int32)
+    x = (rng.random((I, F)) * 2 - 1).astype(F32)
+    # plain sum in input order (float32, left to right); its sign; the vote of the signs
+    acc = np.zeros((O, F), F32)
+    for i in range(n):
+        acc = acc + x[idx[:, i]]
+    assert np.array_equal(oracle.average_lut_forward(x, idx, F, False, False), acc)
+    assert np.array_equal(oracle.average_lut_forward(x, idx, F, False, True), np.where(acc > 0, 1, -1).astype(F32))
+    votes = np.where(x > 0, 1, -1)[idx].sum(axis=1)
+    assert np.array_equal(oracle.average_lut_forward(x, idx, F, True, True), np.where(votes > 0, 1, -1).astype(F32))
+    assert np.array_equal(oracle.average_lut_forward(x, idx, F, True, False), votes.astype(F32))
+    # packed bits: strict majority, so a tie of an even n reads 0
+    xb = synth.bernoulli_bits(rng, I, F)
+    bits = synth.unpack_bits(xb, F).astype(np.int32)
+    for nn in (4, 5):
+        got = synth.unpack_bits(oracle.bit_average_lut_forward(xb, idx[:, :nn].copy(), F), F)
+        assert np.array_equal(got, (2 * bits[idx[:, :nn]].sum(axis=1) > nn))
+    # backward: every wired input receives dy / n; distinct wiring -> a column's total is dy itself (n * dy / n up to rounding)
+    dy = rng.standard_normal((O, F)).astype(F32)
+    dx = oracle.average_lut_backward(dy, idx, I, F)
+    want = np.zeros((I, F), np.float64)
+    for o in range(O):
+        for i in range(n):
+            want[idx[o, i]] += (dy[o] / F32(n)).astype(np.float64)
+    assert np.allclose(dx, want, rtol=1e-6, atol=1e-7)
+    assert np.allclose(dx.sum(axis=0), dy.sum(axis=0), rtol=1e-4, atol=1e-5)
+    one = np.zeros((O, F), F32); one[3] = 1
+    dx1 = oracle.average_lut_backward(one, idx, I, F)
+    assert np.array_equal(np.flatnonzero(dx1[:, 0]), np.sort(idx[3])) and np.all(dx1[idx[3]] == F32(1) / F32(n))
+
+
+# the reference's known-answer test: NumPy goldens held in tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-49
+X_TABLE = np.array([
+    [0.03682449, 0.7174495, 0.9130372, 0.6275032, 0.11995261, 0.25850186, 0.9942376, 0.23910977, 0.75574166, 0.38816985],
+    [0.59729785, 0.7654758, 0.35820892, 0.0122047, 0.05050702, 0.323845, 0.6889169, 0.16161442, 0.06116614, 0.769033],
+    [0.94036084, 0.25700864, 0.73131865, 0.58721095, 0.78960747, 0.29338115, 0.36369365, 0.5750651, 0.81494033, 0.05262487],
+    [0.98256797, 0.15146895, 0.51034707, 0.38718516, 0.18072742, 0.7927627, 0.13334593, 0.03729849, 0.20618507, 0.9241972],
+    [0.713539, 0.48547512, 0.27168426, 0.54288715, 0.6140953, 0.67773014, 0.03847398, 0.7239832, 0.64887875, 0.42749837]], F32)
+X_LABEL = [2, 5, 6, 3, 4]
+DX_TABLE = np.array([
+    [0.01189111, 0.02348626, -0.17144011, 0.02146598, 0.01292184, 0.0148421, 0.03097572, 0.01455706, 0.02440304, 0.016897],
+    [0.02385998, 0.02822986, 0.01878603, 0.01329129, 0.01381026, -0.18184856, 0.02614928, 0.01543317, 0.01395825, 0.02833046],
+    [0.02876907, 0.01452612, 0.0233421, 0.02020946, 0.02474312, 0.0150642, -0.18383847, 0.01996549, 0.02537794, 0.01184096],
+    [0.03275547, 0.01426731, 0.02042683, -0.18194023, 0.01469092, 0.02709271, 0.01401107, 0.01272795, 0.01506971, 0.03089824],
+    [0.02392219, 0.01904382, 0.01537821, 0.02016916, -0.17834225, 0.02308072, 0.01217935, 0.02417335, 0.02242433, 0.01797112]], F32)
+KNOWN_LOSS = 2.297830009460449
+
+
+def known_answer_buffers():
+    y = np.ascontiguousarray(X_TABLE.T)                     # [10 nodes][5 frames]
+    t = np.zeros_like(y)
+    for f, c in enumerate(X_LABEL):
+        t[c, f] = 1
+    return y, t
+
+
+def test_loss_known_answers_of_the_reference_test():
+    y, t = known_answer_buffers()
+    dy, loss_buf, t_sum = oracle.loss_softmax_cross_entropy(y, t, 10, 1, 5)
+    assert t_sum == 5.0
+    assert abs(-loss_buf.sum() / t_sum - KNOWN_LOSS) < 1e-4         # LossSoftmaxCrossEntropyTest.cpp:83
+    assert np.abs(dy.T - DX_TABLE).max() < 1e-6                      # :88
+    acc, cat = oracle.metrics_categorical_accuracy(y, t, 10, 1, 5)
+    want = [int(np.argmax(y[:, f]) == X_LABEL[f]) for f in range(5)]
+    assert acc.tolist() == want and cat.tolist() == [1] * 5
+
+
+def loss_gold(k):
+    ch, pix, F = [int(v) for v in GOLD["l%d_geom" % k]]
+    return ch, pix, F
+
+
+def test_loss_and_accuracy_reference_vectors():
+    for k in range(int(GOLD["loss_count"][0])):
+        ch, pix, F = loss_gold(k); q = "l%d_" % k
+        y, t = GOLD[q + "y"], GOLD[q + "t"]
+        dy, loss_buf, t_sum = oracle.loss_softmax_cross_entropy(y, t, ch, pix, F)
+        # a few ulp: the reference's build may fuse t_max * softmax - t, the oracle keeps the two roundings apart
+        assert np.allclose(dy, GOLD[q + "dy"], rtol=0, atol=4 * np.finfo(F32).eps * np.abs(GOLD[q + "dy"]).max()), k
+        assert abs(-loss_buf.sum() / t_sum - GOLD[q + "loss"][0]) <= 1e-12 * abs(GOLD[q + "loss"][0]), k
+        acc, cat = oracle.metrics_categorical_accuracy(y, t, ch, pix, F)
+        assert acc.sum() / cat.sum() == GOLD[q + "metric"][0], k
+
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref not built")
+def test_loss_and_accuracy_against_compiled_reference():
+    rng = np.random.default_rng(8)
+    for (ch, pix, F) in [(10, 1, 200), (5, 7, 33), (2, 1, 64)]:
+        y = rng.standard_normal((ch * pix, F)).astype(F32) * 3
+        t = np.zeros_like(y)
+        for f in range(F):
+            for p in range(pix):
+                t[int(rng.integers(0, ch)) * pix + p, f] = 1
+        dyr, lossr, metricr = oracle.ref_loss_and_accuracy(y, t, ch, pix, F)
+        dy, loss_buf, t_sum = oracle.loss_softmax_cross_entropy(y, t, ch, pix, F)
+        assert np.allclose(dy, dyr, rtol=0, atol=4 * np.finfo(F32).eps * np.abs(dyr).max())
+        assert abs(-loss_buf.sum() / t_sum - lossr) <= 1e-12 * abs(lossr)
+        acc, cat = oracle.metrics_categorical_accuracy(y, t, ch, pix, F)
+        assert acc.sum() / cat.sum() == metricr
+
+
+def test_loss_closed_forms():
+    rng = np.random.default_rng(9)
+    ch, pix, F = 6, 3, 40
+    y = rng.standard_normal((ch * pix, F)).astype(F32) * 2
+    label = rng.integers(0, ch, (pix, F))
+    t = np.zeros_like(y)
+    for f in range(F):
+        for p in range(pix):
+            t[label[p, f] * pix + p, f] = 1
+    dy, loss_buf, t_sum = oracle.loss_softmax_cross_entropy(y, t, ch, pix, F)
+    assert t_sum == pix * F
+    # float64 softmax cross entropy
+    y3 = y.astype(np.float64).reshape(ch, pix, F)
+    sm = np.exp(y3 - y3.max(axis=0)); sm /= sm.sum(axis=0)
+    t3 = t.astype(np.float64).reshape(ch, pix, F)
+    assert np.allclose(dy.reshape(ch, pix, F), (sm - t3) / t_sum, rtol=1e-5, atol=1e-8)
+    assert np.allclose(loss_buf, (np.log(sm + 1e-7) * t3).sum(axis=(0, 1)), rtol=1e-5, atol=1e-6)
+    # one-hot targets: each pixel's dy sums to zero over the channels
+    assert np.abs(dy.reshape(ch, pix, F).sum(axis=0)).max() < 1e-7
+    # equal logits: loss = log(ch), whatever the shift
+    for shift in (0.0, -50.0, 1e4):
+        dyu, lb, ts = oracle.loss_softmax_cross_entropy(np.full_like(y, shift), t, ch, pix, F)
+        assert abs(-lb.sum() / ts - np.log(ch)) < 1e-5
+    # y = t: every labeled pixel is predicted; an unlabeled pixel is not counted; ties go to the first channel
+    acc, cat = oracle.metrics_categorical_accuracy(t, t, ch, pix, F)
+    assert np.all(acc == pix) and np.all(cat == pix)
+    t2 = t.copy(); t2[:, 0] = 0
+    acc, cat = oracle.metrics_categorical_accuracy(y, t2, ch, pix, F)
+    assert cat[0] == 0 and acc[0] == 0
+    yt = np.zeros((3, 2), F32); tt = np.array([[1, 0], [0, 1], [0, 0]], F32)
+    acc, cat = oracle.metrics_categorical_accuracy(yt, tt, 3, 1, 2)
+    assert acc.tolist() == [1, 0] and cat.tolist() == [1, 1]
+    # weights: t_sum follows the weights and the host sum runs frame-major in float
+    tw = t * F32(0.3)
+    assert oracle.loss_t_sum(tw, F) == np.cumsum(np.full(pix * F, F32(0.3), F32), dtype=F32)[-1]
