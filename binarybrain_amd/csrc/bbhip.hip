@@ -60,7 +60,7 @@ int  g_dx_mode   = 0;
 // ------------------------------------------------------------------------------------------------
 //  optional kernel timer: HIP events around the dominant kernel of each entry point, on the launch stream
 // ------------------------------------------------------------------------------------------------
-enum TimedKernel : int { kTimeForward = 0, kTimeBackward = 1, kTimeBinary = 2, kTimeDx = 3, kTimedKinds = 4 };
+enum TimedKernel : int { kTimeForward = 0, kTimeBackward = 1, kTimeBinary = 2, kTimeDx = 3, kTimeOther = 4, kTimedKinds = 5 };
 struct TimedLaunch { hipEvent_t start, stop; int which; };
 bool g_timer_on = false;
 std::vector<TimedLaunch> g_timed;
@@ -583,6 +583,7 @@ int vector_op(float *dst, float const *src0, float const *src1, float a, float b
     int const aligned = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src0) |
                           (vec_binary<OP>() ? reinterpret_cast<uintptr_t>(src1) : 0)) & 15) == 0;
     size_t const blocks = ((size_t)size + kVecBlock * 4 - 1) / (kVecBlock * 4);
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(vector_op_kernel<OP>, dim3((unsigned)blocks), dim3(kVecBlock), 0, static_cast<hipStream_t>(stream),
                        dst, src0, src1, a, b, c, d, (size_t)size, aligned);
     BBHIP_LAUNCH_CHECK();
@@ -742,6 +743,7 @@ int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *
     BBHIP_REQUIRE(dev_size_table != nullptr && dev_params_buf_table != nullptr && dev_grads_buf_table != nullptr &&
                   dev_m_buf_table != nullptr && dev_v_buf_table != nullptr);
     // the element counts live on the device: a fixed number of blocks per tensor strides over its elements
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(adam_kernel, dim3(kAdamBlocksPerTensor, (unsigned)size), dim3(kVecBlock), 0, static_cast<hipStream_t>(stream),
                        dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table,
                        lr_t, 1.0f - beta1, 1.0f - beta2);
@@ -762,6 +764,7 @@ int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_st
     a.f_tiles  = ceil_div(a.input_frame_size, kTile);
     long long const blocks = (long long)a.c * a.fh * a.fw * a.oh * a.ox_tiles * a.f_tiles;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(im2col_forward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a);
     BBHIP_LAUNCH_CHECK();
     return 0;
@@ -781,6 +784,7 @@ int bbhip_bit_Im2Col_Forward(int const *dev_x_buf, int *dev_y_buf, int x_stride,
     long long const total = (long long)a.c * a.fh * a.fw * words;
     long long const blocks = (total + kConvBlock - 1) / kConvBlock;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(im2col_forward_bit_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, words, total);
     BBHIP_LAUNCH_CHECK();
     return 0;
@@ -799,6 +803,7 @@ int bbhip_fp32_Im2Col_Backward(float const *dev_dy_buf, float *dev_dx_buf, int x
     a.f_tiles = ceil_div(a.input_frame_size, kTile);
     long long const blocks = (long long)a.c * a.h * x_tiles * a.f_tiles;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(im2col_backward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, x_tiles);
     BBHIP_LAUNCH_CHECK();
     return 0;
@@ -824,6 +829,7 @@ int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_si
     int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
     long long const blocks = (long long)c_size * xy_tiles * f_tiles;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(col2im_kernel<true>, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream),
                        dev_x_buf, dev_y_buf, hw, c_size, input_frame_stride, output_frame_size, output_frame_stride, xy_tiles, f_tiles);
     BBHIP_LAUNCH_CHECK();
@@ -837,6 +843,7 @@ int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w
     int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
     long long const blocks = (long long)c_size * xy_tiles * f_tiles;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(col2im_kernel<false>, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream),
                        dev_dy_buf, dev_dx_buf, hw, c_size, input_frame_stride, output_frame_size, output_frame_stride, xy_tiles, f_tiles);
     BBHIP_LAUNCH_CHECK();
@@ -851,6 +858,7 @@ int bbhip_bit_Col2Im_Forward(int const *dev_x_buf, int *dev_y_buf, int w_size, i
     long long const total = (long long)c_size * hw * words;
     long long const blocks = (total + kConvBlock - 1) / kConvBlock;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(col2im_forward_bit_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream),
                        reinterpret_cast<uint32_t const *>(dev_x_buf), reinterpret_cast<uint32_t *>(dev_y_buf), hw, input_frame_stride,
                        output_frame_size, output_frame_stride, words, total);
@@ -867,6 +875,7 @@ static int launch_pool(PoolArgs const &a, bool backward, void *stream, char cons
     int const f_blocks = ceil_div(a.frame_size, kConvBlock);
     long long const blocks = (long long)a.c * a.oh * a.ow * f_blocks;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     if (backward) { hipLaunchKernelGGL(stochastic_maxpool2x2_backward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, f_blocks); }
     else          { hipLaunchKernelGGL(stochastic_maxpool2x2_forward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, f_blocks); }
     BBHIP_LAUNCH_CHECK();
@@ -905,6 +914,7 @@ int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int 
     int const f_blocks = ceil_div(frame_size, kTailBlock);
     long long const blocks = (long long)node_size * f_blocks;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(average_lut_forward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_x_buf,
                        dev_y_buf, dev_input_index, n, frame_size, frame_stride, binarize_input, binarize_output, f_blocks);
     BBHIP_LAUNCH_CHECK();
@@ -923,6 +933,7 @@ int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     while ((1 << planes) <= n && planes < 31) { ++planes; }      // planes = bits of n: counts 0..n fit
     dim3 const grid((unsigned)blocks), block(kTailBlock);
     hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
 #define BBHIP_AVERAGE_BIT(P) hipLaunchKernelGGL(average_lut_forward_bit_kernel<P>, grid, block, 0, st, dev_x_buf, dev_y_buf, dev_input_index, n, words, frame_stride, w_blocks)
     switch (planes) {
     case 1: BBHIP_AVERAGE_BIT(1); break;
@@ -955,6 +966,7 @@ int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
     if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch)) { return 1; }
     int *offsets = reinterpret_cast<int *>(scratch), *list = reinterpret_cast<int *>(scratch + offsets_bytes);
     hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(average_lut_reverse_kernel, dim3((unsigned)ceil_div(input_node_size + 1, kTailBlock)), dim3(kTailBlock), 0, st,
                        dev_input_index, total, n, input_node_size, offsets, list);
     BBHIP_LAUNCH_CHECK();
@@ -981,6 +993,7 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
         if (arena_get(sizeof(double) * (size_t)pix_size * (size_t)frame_size, &scratch)) { return 1; }
         partial = reinterpret_cast<double *>(scratch);
     }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(softmax_cross_entropy_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_y_buf, dev_t_buf, dev_dy_buf, partial,
                        t_sum, pix_size, ch_size, frame_size, frame_stride, f_blocks);
     BBHIP_LAUNCH_CHECK();
@@ -998,6 +1011,7 @@ int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *d
     if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
     if ((long long)pix_size * ch_size > 0x7fffffffLL) { return fail("%s: node count too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(categorical_accuracy_kernel, dim3((unsigned)ceil_div(frame_size, kTailBlock)), dim3(kTailBlock), 0,
                        static_cast<hipStream_t>(stream), dev_y_buf, dev_t_buf, dev_accuracy_buf, dev_category_buf, pix_size, ch_size, frame_size,
                        frame_stride);

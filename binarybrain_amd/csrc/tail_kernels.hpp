@@ -92,20 +92,53 @@ __global__ __launch_bounds__(kTailBlock) void average_lut_forward_bit_wide_kerne
 
 // Reverse wiring for the backward pass, built on the device: for input node i, offsets[i] = number of table entries that
 // name a smaller input, and list[offsets[i] ...] = the output nodes wired to i in table order (node ascending, input
-// position ascending).  One thread per input node (plus one for the end offset) sweeps the whole table twice; the sweeps
-// read the same entry in every lane, so they run on the scalar unit.  Entries outside [0, input_node_size) match no thread.
+// position ascending).  One thread per input node (plus one for the end offset) sweeps the whole table twice; the block
+// stages the table through LDS in pieces, so a sweep is one coalesced load per piece and broadcast LDS reads.
+// Entries outside [0, input_node_size) match no thread.
+constexpr int kReversePiece = 2048;
+
+// copy `count` table entries into LDS and fill up to the next multiple of four with -1, which matches no input node
+__device__ __forceinline__ void stage_piece(int *piece, int const *__restrict__ src, int count)
+{
+    int const padded = (count + 3) & ~3;
+    for (int k = threadIdx.x; k < padded; k += kTailBlock) { piece[k] = (k < count) ? src[k] : -1; }
+}
+
 __global__ __launch_bounds__(kTailBlock) void average_lut_reverse_kernel(int const *__restrict__ idx, int total, int n, int input_node_size,
                                                                          int *__restrict__ offsets, int *__restrict__ list)
 {
+    __shared__ __attribute__((aligned(16))) int piece[kReversePiece];
     int const i = blockIdx.x * kTailBlock + threadIdx.x;
-    if (i > input_node_size) { return; }
+    bool const live = (i <= input_node_size);
     int below = 0;
-    for (int e = 0; e < total; ++e) { below += ((uint32_t)idx[e] < (uint32_t)i) ? 1 : 0; }
-    offsets[i] = below;
-    if (i == input_node_size) { return; }
+    for (int base = 0; base < total; base += kReversePiece) {
+        int const count = min(kReversePiece, total - base);
+        __syncthreads();
+        stage_piece(piece, idx + base, count);
+        __syncthreads();
+#pragma unroll 2
+        for (int k = 0; k < count; k += 4) {
+            int4 const e = *reinterpret_cast<int4 const *>(&piece[k]);
+            below += ((uint32_t)e.x < (uint32_t)i) + ((uint32_t)e.y < (uint32_t)i) + ((uint32_t)e.z < (uint32_t)i) + ((uint32_t)e.w < (uint32_t)i);
+        }
+    }
+    if (live) { offsets[i] = below; }
     int at = below;
-    for (int e = 0; e < total; ++e) {
-        if (idx[e] == i) { list[at++] = e / n; }
+    for (int base = 0; base < total; base += kReversePiece) {
+        int const count = min(kReversePiece, total - base);
+        __syncthreads();
+        stage_piece(piece, idx + base, count);
+        __syncthreads();
+        if (live && i < input_node_size) {
+#pragma unroll 2
+            for (int k = 0; k < count; k += 4) {
+                int4 const e = *reinterpret_cast<int4 const *>(&piece[k]);
+                if (e.x == i) { list[at++] = (base + k) / n; }
+                if (e.y == i) { list[at++] = (base + k + 1) / n; }
+                if (e.z == i) { list[at++] = (base + k + 2) / n; }
+                if (e.w == i) { list[at++] = (base + k + 3) / n; }
+            }
+        }
     }
 }
 

@@ -71,7 +71,8 @@ int  bbhip_GetDxMode(void);
 
 /* ---- kernel timer (instrumentation; no counterpart in the reference) ----
  * While enabled, every call brackets its dominant kernel (which: 0 = LUT forward kernel, 1 = LUT backward kernel,
- * 2 = BinaryLut6 kernel, 3 = input-centric dx kernel) with HIP events on the launch stream.  Read waits for the recorded launches of one kind,
+ * 2 = BinaryLut6 kernel, 3 = input-centric dx kernel, 4 = the kernels of any other entry: vector operations, Adam, Im2Col,
+ * Col2Im, pooling, AverageLut, loss, accuracy) with HIP events on the launch stream.  Read waits for the recorded launches of one kind,
  * returns their summed duration and count, and forgets them. */
 void bbhip_KernelTimer_Enable(int enable);
 int  bbhip_KernelTimer_Read(int which, float *total_ms, int *launches);
