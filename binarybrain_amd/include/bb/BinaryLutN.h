@@ -18,6 +18,7 @@ class BinaryLutN : public Model {
 
 protected:
     bool        m_host_only = false;
+    bool        m_host_simd = true;             // carried through serialization only: there is no host path here
     std::string m_connection;
     indices_t   m_input_shape, m_output_shape;
     Tensor_<std::int32_t> m_table;          // [output nodes][2]
@@ -49,9 +50,44 @@ protected:
         m_table = 0;
     }
 
+    // the reference's object layout (include/bb/BinaryLutN.h:481-519): version, Model part, flags, connection policy, shapes,
+    // truth table object, input index object
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        Model::DumpObjectData(os);
+        SaveValue(os, m_host_only);
+        SaveValue(os, m_host_simd);
+        SaveValue(os, m_connection);
+        SaveValue(os, m_input_shape);
+        SaveValue(os, m_output_shape);
+        m_table.DumpObject(os);
+        m_input_index.DumpObject(os);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = 0;
+        LoadValue(is, ver); BB_ASSERT(ver == 1);
+        Model::LoadObjectData(is);
+        LoadValue(is, m_host_only);
+        LoadValue(is, m_host_simd);
+        LoadValue(is, m_connection);
+        LoadValue(is, m_input_shape);
+        LoadValue(is, m_output_shape);
+        m_table.LoadObject(is);
+        m_input_index.LoadObject(is);
+        index_t const O = CalcShapeSize(m_output_shape), I = CalcShapeSize(m_input_shape);
+        BB_ASSERT(m_table.GetShape() == indices_t({O, (index_t)kTableUnit}) && m_input_index.GetShape() == indices_t({O, (index_t)N}));
+        // wiring read from a file is checked before any kernel follows it
+        auto idx = m_input_index.LockConst();
+        for (index_t i = 0; i < O * N; ++i) { BB_ASSERT(idx[i] >= 0 && idx[i] < I); }
+    }
+
 public:
     static std::string ModelName(void) { return "BinaryLut" + std::to_string(N); }
+    static std::string ObjectName(void) { return ModelName() + "_" + DataType<FT>::Name() + "_" + DataType<BT>::Name(); }
     std::string GetModelName(void) const override { return ModelName(); }
+    std::string GetObjectName(void) const override { return ObjectName(); }
 
     static std::shared_ptr<BinaryLutN> Create(create_t const &create) { return std::shared_ptr<BinaryLutN>(new BinaryLutN(create)); }
     static std::shared_ptr<BinaryLutN> Create(indices_t const &output_shape, std::uint64_t seed = 1)

@@ -82,9 +82,64 @@ protected:
         m_dW = std::make_shared<Tensor>();
     }
 
+    // the reference's object layout (include/bb/DifferentiableLutN.h:266-334): version, Model part, flags, shapes, connection
+    // table object, W object, bias, momentum, gamma, beta, running mean and variance objects
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        Model::DumpObjectData(os);
+        SaveValue(os, m_host_only);
+        SaveValue(os, m_lut_binarize);
+        SaveValue(os, m_binary_mode);
+        SaveValue(os, m_batch_norm);
+        SaveValue(os, m_flagClamp);
+        SaveValue(os, m_input_shape);
+        SaveValue(os, m_output_shape);
+        m_connection_table.DumpObject(os);
+        m_W->DumpObject(os);
+        SaveValue(os, m_unbinarize_bias);
+        SaveValue(os, m_momentum);
+        SaveValue(os, m_gamma);
+        SaveValue(os, m_beta);
+        m_running_mean.DumpObject(os);
+        m_running_var.DumpObject(os);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = 0;
+        LoadValue(is, ver); BB_ASSERT(ver == 1);
+        Model::LoadObjectData(is);
+        LoadValue(is, m_host_only);
+        LoadValue(is, m_lut_binarize);
+        LoadValue(is, m_binary_mode);
+        LoadValue(is, m_batch_norm);
+        LoadValue(is, m_flagClamp);
+        LoadValue(is, m_input_shape);
+        LoadValue(is, m_output_shape);
+        m_connection_table.LoadObject(is);
+        m_W->LoadObject(is);
+        LoadValue(is, m_unbinarize_bias);
+        LoadValue(is, m_momentum);
+        LoadValue(is, m_gamma);
+        LoadValue(is, m_beta);
+        m_running_mean.LoadObject(is);
+        m_running_var.LoadObject(is);
+        index_t const O = CalcShapeSize(m_output_shape);
+        BB_ASSERT(m_connection_table.GetOutputNodeSize() == O && m_connection_table.GetInputNodeSize() == CalcShapeSize(m_input_shape));
+        BB_ASSERT(m_W->GetType() == DataType<RealType>::type && m_W->GetShape() == indices_t({O, (index_t)NN}));
+        BB_ASSERT(m_running_mean.GetSize() == O && m_running_var.GetSize() == O);
+        if (kBitType) { m_binary_mode = true; }
+        m_dW->Resize(m_W->GetShape(), DataType<RealType>::type);
+        m_dW->FillZero();
+        m_mean.Resize(m_output_shape);
+        m_rstd.Resize(m_output_shape);
+    }
+
 public:
     static std::string ModelName(void) { return "DifferentiableLut" + std::to_string(N); }
+    static std::string ObjectName(void) { return ModelName() + "_" + DataType<BinType>::Name() + "_" + DataType<RealType>::Name(); }
     std::string GetModelName(void) const override { return ModelName(); }
+    std::string GetObjectName(void) const override { return ObjectName(); }
 
     static std::shared_ptr<DifferentiableLutN> Create(create_t const &create) { return std::shared_ptr<DifferentiableLutN>(new DifferentiableLutN(create)); }
     static std::shared_ptr<DifferentiableLutN> Create(indices_t const &output_shape, bool batch_norm = true, std::string connection = "")

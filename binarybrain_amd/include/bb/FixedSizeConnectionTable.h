@@ -15,7 +15,7 @@
 namespace bb {
 
 template <int N, typename IndexType = std::int32_t>
-class FixedSizeConnectionTable {
+class FixedSizeConnectionTable : public Object {
     indices_t           m_input_shape, m_output_shape;
     index_t             m_input_node_size = 0, m_output_node_size = 0;
     Tensor_<IndexType>  m_input_table;
@@ -93,7 +93,36 @@ public:
     auto LockDeviceMemConst_ReverseTable(void) { BuildReverseTable(); return m_reverse_table.LockDeviceMemoryConst(); }
     index_t GetReverseTableStride(void)        { BuildReverseTable(); return m_reverse_table.GetShape()[1]; }
 
+    std::string GetObjectName(void) const override { return "FixedSizeConnectionTable" + std::to_string(N) + "_" + DataType<IndexType>::Name(); }
+
 protected:
+    // version | ConnectionTable part: version, Object version 0, input shape, output shape | input table object
+    // (reference: include/bb/FixedSizeConnectionTable.h:50-82, ConnectionTable.h:47-74)
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        SaveValue(os, (std::int64_t)1);
+        SaveValue(os, (std::int64_t)0);
+        SaveIndices(os, m_input_shape);
+        SaveIndices(os, m_output_shape);
+        m_input_table.DumpObject(os);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = 0, parent = 0, base = -1;
+        LoadValue(is, ver);    BB_ASSERT(ver == 1);
+        LoadValue(is, parent); BB_ASSERT(parent == 1);
+        LoadValue(is, base);   BB_ASSERT(base == 0);
+        indices_t const input_shape = LoadIndices(is), output_shape = LoadIndices(is);
+        SetShape(input_shape, output_shape);
+        m_input_table.LoadObject(is);
+        BB_ASSERT(m_input_table.GetShape() == indices_t({m_output_node_size, (index_t)N}));
+        // wiring read from a file is checked before any kernel follows it
+        auto tbl = m_input_table.LockConst();
+        for (index_t i = 0; i < m_output_node_size * N; ++i) { BB_ASSERT(tbl[i] >= 0 && tbl[i] < m_input_node_size); }
+        m_reverse_table_dirty = true;
+    }
+
     void BuildReverseTable(void)
     {
         if (!m_reverse_table_dirty) { return; }

@@ -10,7 +10,7 @@
 
 namespace bb {
 
-class Model {
+class Model : public Object {
 protected:
     std::string             m_name;
     bool                    m_parameter_lock = false;
@@ -31,10 +31,34 @@ protected:
         return buf;
     }
 
+    // version 1 | int64 length of the name | name (reference: include/bb/Model.h:392-426; a version 0 record carries no name)
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        SaveValue(os, (std::int64_t)m_name.size());
+        os.write(m_name.data(), (std::streamsize)m_name.size());
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = -1;
+        LoadValue(is, ver);
+        BB_ASSERT(ver == 0 || ver == 1);
+        if (ver == 1) {
+            std::int64_t size = -1;
+            LoadValue(is, size);
+            BB_ASSERT(is.good() && size >= 0 && size < (1ll << 20));
+            std::string name((std::size_t)size, '\0');
+            if (size > 0) { is.read(&name[0], (std::streamsize)size); }
+            if (m_name.empty()) { m_name = name; }          // a name given before loading is kept
+        }
+    }
+
 public:
     virtual ~Model() {}
 
     virtual std::string GetModelName(void) const = 0;
+    // serialized type name; layers with element types append them (e.g. "StochasticLut6_fp32_fp32")
+    std::string GetObjectName(void) const override { return GetModelName(); }
     virtual void        SetName(std::string const &name) { m_name = name; }
     virtual std::string GetName(void) const { return m_name.empty() ? GetModelName() : m_name; }
 

@@ -1,0 +1,57 @@
+// Reconstruct a serialized object from its recorded type name (reference: include/bb/ObjectLoader.h:407-447
+// `Object_Load` / `Object_LoadFromFile`).  Known here: the LUT layers of widths 2..6 on fp32 or packed-bit frames,
+// BinaryLut6, and tensors.  An unknown name yields an empty pointer, as in the reference.
+#pragma once
+
+#include "bb/StochasticLutN.h"
+#include "bb/DifferentiableLutN.h"
+#include "bb/BinaryLutN.h"
+
+namespace bb {
+
+namespace detail {
+
+template <int N>
+inline std::shared_ptr<Object> CreateLutByName(std::string const &name)
+{
+    if (name == StochasticLutN<N, float, float>::ObjectName())     { return StochasticLutN<N, float, float>::Create((index_t)1); }
+    if (name == StochasticLutN<N, Bit, float>::ObjectName())       { return StochasticLutN<N, Bit, float>::Create((index_t)1); }
+    if (name == DifferentiableLutN<N, float, float>::ObjectName()) { return DifferentiableLutN<N, float, float>::Create((index_t)1); }
+    if (name == DifferentiableLutN<N, Bit, float>::ObjectName())   { return DifferentiableLutN<N, Bit, float>::Create((index_t)1); }
+    return std::shared_ptr<Object>();
+}
+
+inline std::shared_ptr<Object> CreateByName(std::string const &name)
+{
+    if (name == "Tensor")       { return std::make_shared<Tensor>(); }
+    if (name == "Tensor_fp32")  { return std::make_shared<Tensor_<float>>(); }
+    if (name == "Tensor_fp64")  { return std::make_shared<Tensor_<double>>(); }
+    if (name == "Tensor_int32") { return std::make_shared<Tensor_<std::int32_t>>(); }
+    if (name == BinaryLutN<6, Bit, float>::ObjectName()) { return BinaryLutN<6, Bit, float>::Create((index_t)1); }
+    std::shared_ptr<Object> obj;
+    if ((obj = CreateLutByName<6>(name))) { return obj; }
+    if ((obj = CreateLutByName<5>(name))) { return obj; }
+    if ((obj = CreateLutByName<4>(name))) { return obj; }
+    if ((obj = CreateLutByName<3>(name))) { return obj; }
+    if ((obj = CreateLutByName<2>(name))) { return obj; }
+    return obj;
+}
+
+}  // namespace detail
+
+inline std::shared_ptr<Object> Object_Load(std::istream &is)
+{
+    std::string const name = Object::ReadHeader(is);
+    std::shared_ptr<Object> obj = detail::CreateByName(name);
+    if (obj) { obj->LoadObjectData(is); }
+    return obj;
+}
+
+inline std::shared_ptr<Object> Object_LoadFromFile(std::string filename)
+{
+    std::ifstream ifs(filename, std::ios::binary);
+    if (!ifs.is_open()) { return std::shared_ptr<Object>(); }
+    return Object_Load(ifs);
+}
+
+}  // namespace bb

@@ -21,6 +21,8 @@ class StochasticLutN : public Model {
 
 protected:
     bool        m_host_only = false;
+    bool        m_host_simd = true;                 // carried through serialization only: there is no host path here
+    bool        m_y_binarize = false;               // likewise
     bool        m_binary_mode = kBitInput;
     bool        m_lut_binarize = true;              // class default of the reference (StochasticLutN.h:45)
     RealType    m_unbinarize_bias = (RealType)0.25;
@@ -65,9 +67,55 @@ protected:
         m_dW = std::make_shared<Tensor>();
     }
 
+    // the reference's object layout (include/bb/StochasticLutN.h:170-223): version, Model part, flags, tmp size, connection
+    // policy, bias, shapes, connection table object, W object
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        Model::DumpObjectData(os);
+        SaveValue(os, m_host_only);
+        SaveValue(os, m_host_simd);
+        SaveValue(os, m_binary_mode);
+        SaveValue(os, m_lut_binarize);
+        SaveValue(os, m_y_binarize);
+        SaveValue(os, (std::int64_t)m_max_tmp_mem_size);
+        SaveValue(os, m_connection);
+        SaveValue(os, m_unbinarize_bias);
+        SaveValue(os, m_input_shape);
+        SaveValue(os, m_output_shape);
+        m_connection_table.DumpObject(os);
+        m_W->DumpObject(os);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = 0, tmp = 0;
+        LoadValue(is, ver); BB_ASSERT(ver == 1);
+        Model::LoadObjectData(is);
+        LoadValue(is, m_host_only);
+        LoadValue(is, m_host_simd);
+        LoadValue(is, m_binary_mode);
+        LoadValue(is, m_lut_binarize);
+        LoadValue(is, m_y_binarize);
+        LoadValue(is, tmp); m_max_tmp_mem_size = (index_t)tmp;
+        LoadValue(is, m_connection);
+        LoadValue(is, m_unbinarize_bias);
+        LoadValue(is, m_input_shape);
+        LoadValue(is, m_output_shape);
+        m_connection_table.LoadObject(is);
+        m_W->LoadObject(is);
+        index_t const O = CalcShapeSize(m_output_shape);
+        BB_ASSERT(m_connection_table.GetOutputNodeSize() == O && m_connection_table.GetInputNodeSize() == CalcShapeSize(m_input_shape));
+        BB_ASSERT(m_W->GetType() == DataType<RealType>::type && m_W->GetShape() == indices_t({O, (index_t)NN}));
+        if (kBitInput) { m_binary_mode = true; }
+        m_dW->Resize({O, (index_t)NN}, DataType<RealType>::type);
+        m_dW->FillZero();
+    }
+
 public:
     static std::string ModelName(void) { return "StochasticLut" + std::to_string(N); }
+    static std::string ObjectName(void) { return ModelName() + "_" + DataType<BinType>::Name() + "_" + DataType<RealType>::Name(); }
     std::string GetModelName(void) const override { return ModelName(); }
+    std::string GetObjectName(void) const override { return ObjectName(); }
 
     static std::shared_ptr<StochasticLutN> Create(create_t const &create) { return std::shared_ptr<StochasticLutN>(new StochasticLutN(create)); }
     static std::shared_ptr<StochasticLutN> Create(indices_t const &output_shape, std::string connection = "", std::uint64_t seed = 1)

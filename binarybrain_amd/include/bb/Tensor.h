@@ -8,6 +8,7 @@
 #include <random>
 
 #include "bb/Core.h"
+#include "bb/Object.h"
 
 namespace bb {
 
@@ -42,7 +43,7 @@ public:
 };
 
 
-class Tensor {
+class Tensor : public Object {
 protected:
     int                     m_type = BB_TYPE_FP32;
     indices_t               m_shape;
@@ -62,6 +63,57 @@ public:
         m_mem   = Memory::Create((std::size_t)m_size * (std::size_t)(DataType_GetBitSize(type) / 8), m_host_only);
     }
 
+    std::string GetObjectName(void) const override { return "Tensor"; }
+
+protected:
+    // the layout of the reference's typed tensor (include/bb/Tensor.h:614-651): version, parent version, element offset,
+    // element count, shape, row-major strides, elements
+    void DumpTypedData(std::ostream &os) const
+    {
+        SaveValue(os, (std::int64_t)1);
+        SaveValue(os, (std::int64_t)0);
+        SaveValue(os, (std::int64_t)0);
+        SaveValue(os, (std::int64_t)m_size);
+        SaveIndices(os, m_shape);
+        indices_t stride(m_shape.size());
+        index_t total = 1;
+        for (std::size_t i = m_shape.size(); i-- > 0;) { stride[i] = total; total *= m_shape[i]; }
+        SaveIndices(os, stride);
+        if (m_size > 0) { os.write(static_cast<char const *>(m_mem->LockConst()), (std::streamsize)(m_size * (DataType_GetBitSize(m_type) / 8))); }
+    }
+    void LoadTypedData(std::istream &is, int type)
+    {
+        std::int64_t ver = 0, parent = -1, offset = -1, size = -1;
+        LoadValue(is, ver);    BB_ASSERT(ver == 1);
+        LoadValue(is, parent); BB_ASSERT(parent == 0);
+        LoadValue(is, offset); BB_ASSERT(offset == 0);
+        LoadValue(is, size);
+        indices_t const shape = LoadIndices(is);
+        BB_ASSERT(is.good() && size == CalcShapeSize(shape));
+        Resize(shape, type);
+        (void)LoadIndices(is);
+        if (m_size > 0) { is.read(static_cast<char *>(m_mem->Lock(true)), (std::streamsize)(m_size * (DataType_GetBitSize(type) / 8))); }
+    }
+    // untyped tensor: version, parent version, element type code, then the typed layout (include/bb/Tensor.h:2159-2211)
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        SaveValue(os, (std::int64_t)0);
+        SaveValue(os, (std::int32_t)m_type);
+        DumpTypedData(os);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = 0, parent = -1;
+        std::int32_t type = 0;
+        LoadValue(is, ver);    BB_ASSERT(ver == 1);
+        LoadValue(is, parent); BB_ASSERT(parent == 0);
+        LoadValue(is, type);
+        (void)DataType_GetBitSize(type);        // throws on a type code this library does not hold
+        LoadTypedData(is, type);
+    }
+
+public:
     int       GetType(void) const  { return m_type; }
     indices_t GetShape(void) const { return m_shape; }
     index_t   GetSize(void) const  { return m_size; }
@@ -123,6 +175,11 @@ public:
     void Resize(index_t i0, index_t i1) { Resize(indices_t({i0, i1})); }
     auto Lock(bool discard = false) { return Tensor::Lock<T>(discard); }
     auto LockConst(void) const { return Tensor::LockConst<T>(); }
+    std::string GetObjectName(void) const override { return "Tensor_" + DataType<T>::Name(); }
+protected:
+    void DumpObjectData(std::ostream &os) const override { DumpTypedData(os); }
+    void LoadObjectData(std::istream &is) override { LoadTypedData(is, DataType<T>::type); }
+public:
     Tensor_ &operator=(T value)
     {
         auto p = Lock(true);

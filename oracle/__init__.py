@@ -586,6 +586,41 @@ def ref_loss_and_accuracy(y, t, ch_size, pix_size, frames):
     return dy, loss.value, metric.value
 
 
+LUT_OBJECT_KINDS = {"stochastic": 0, "differentiable": 1, "binary": 2}
+
+
+def ref_dump_lut_object(kind, bit, input_nodes, idx, params, mean=None, var=None, flags=0, scalars=(0.9, 0.3, 0.5), name=""):
+    """Bytes of a 6-input LUT layer serialized by the reference's own DumpObject.  params: W [O, 64] float32, or the truth
+    table [O, 2] int32 for kind "binary".  flags: 1 = binary, 2 = lut_binarize, 4 = batch_norm."""
+    idx = _c(idx, np.int32)
+    params = _c(params, np.int32 if kind == "binary" else np.float32)
+    O = idx.shape[0]
+    mean = _c(mean if mean is not None else np.zeros(O), np.float32)
+    var = _c(var if var is not None else np.ones(O), np.float32)
+    sc = _c(scalars, np.float32)
+    cap = 4096 + 64 * idx.nbytes + 2 * params.nbytes
+    out = np.zeros(cap, np.uint8)
+    f = ref().bbref_DumpLutObject
+    f.restype = C.c_long
+    n = f(C.c_int(LUT_OBJECT_KINDS[kind]), C.c_int(int(bit)), C.c_int(input_nodes), C.c_int(O), _ptr(idx), _ptr(params), _ptr(mean), _ptr(var),
+          C.c_int(flags), _ptr(sc), C.c_char_p(name.encode()), _ptr(out), C.c_long(cap))
+    assert n > 0, n
+    return out[:n].tobytes()
+
+
+def ref_load_lut_object(kind, bit, data, output_nodes):
+    """A serialized layer read by the reference's own LoadObject -> dict(input_nodes, idx, params, mean, var, name)."""
+    buf = np.frombuffer(data, np.uint8).copy()
+    idx = np.zeros((output_nodes, 6), np.int32)
+    params = np.zeros((output_nodes, 2), np.int32) if kind == "binary" else np.zeros((output_nodes, 64), np.float32)
+    mean = np.zeros(output_nodes, np.float32); var = np.zeros(output_nodes, np.float32)
+    name = C.create_string_buffer(256)
+    I = ref().bbref_LoadLutObject(C.c_int(LUT_OBJECT_KINDS[kind]), C.c_int(int(bit)), _ptr(buf), C.c_long(buf.size), C.c_int(output_nodes),
+                                  _ptr(idx), _ptr(params), _ptr(mean), _ptr(var), name, C.c_int(256))
+    assert I >= 0, I
+    return dict(input_nodes=I, idx=idx, params=params, mean=mean, var=var, name=name.value.decode())
+
+
 def time_stochastic_lut6(x, dy, idx, W, reps=3, use_ref=None):
     """Seconds per StochasticLut6 forward+backward on the host, one value per repetition (after one warm-up).
     use_ref=True times the reference's own AVX2/OpenMP path, False the C restatement; None picks the reference when built."""

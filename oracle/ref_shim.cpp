@@ -16,6 +16,7 @@
 #include <cstdint>
 #include <vector>
 #include <string>
+#include <sstream>
 
 #include "bb/StochasticLutN.h"
 #include "bb/DifferentiableLutN.h"
@@ -482,4 +483,132 @@ extern "C" int bbref_LossAndAccuracy(int ch, int pix, int F, float const *y, flo
     metrics->CalculateMetrics(yb, tb);
     *metric = metrics->GetMetrics();
     return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Object serialization of the three LUT layers (Object::DumpObject / LoadObject): a layer with the given wiring and
+// parameters is built through the reference's API and written to bytes, or read back from bytes and taken apart.
+// kind 0 = StochasticLutN<6>, 1 = DifferentiableLutN<6>, 2 = BinaryLutN<6, Bit, float>; bit selects BinType = Bit for
+// kinds 0 and 1.  flags: bit 0 = binary, bit 1 = lut_binarize, bit 2 = batch_norm.  scalars = {momentum, gamma, beta}.
+// params: W [O][64] fp32 (kinds 0, 1) or the truth table [O][2] int32 (kind 2).
+// ---------------------------------------------------------------------------------------------------------------------
+namespace {
+
+template <class M>
+void put_wiring(M &m, int O, std::int32_t const *idx)
+{
+    for (int o = 0; o < O; ++o) { for (int i = 0; i < 6; ++i) { m.SetNodeConnectionIndex(o, i, idx[o * 6 + i]); } }
+}
+template <class M>
+void get_wiring(M const &m, int O, std::int32_t *idx)
+{
+    for (int o = 0; o < O; ++o) { for (int i = 0; i < 6; ++i) { idx[o * 6 + i] = (std::int32_t)m.GetNodeConnectionIndex(o, i); } }
+}
+long emit(bb::Object const &obj, unsigned char *out, long cap)
+{
+    std::ostringstream os(std::ios::binary);
+    obj.DumpObject(os);
+    std::string const bytes = os.str();
+    if ((long)bytes.size() > cap) { return -(long)bytes.size(); }
+    std::memcpy(out, bytes.data(), bytes.size());
+    return (long)bytes.size();
+}
+
+template <typename BinType>
+long dump_stochastic(int I, int O, std::int32_t const *idx, float const *W, int flags, char const *name, unsigned char *out, long cap)
+{
+    auto m = bb::StochasticLutN<6, BinType, float>::Create((index_t)O);
+    if (name && *name) { m->SetName(name); }
+    m->SetInputShape({(index_t)I});
+    put_wiring(*m, O, idx);
+    { auto Wp = m->lock_W(); for (int i = 0; i < O * 64; ++i) { Wp(i / 64, i % 64) = W[i]; } }
+    m->SendCommand("binary " + onoff(flags & 1));
+    m->SendCommand("lut_binarize " + onoff(flags & 2));
+    return emit(*m, out, cap);
+}
+template <typename BinType>
+int load_stochastic(unsigned char const *bytes, long size, int O, std::int32_t *idx, float *W, char *name, int name_cap)
+{
+    auto m = bb::StochasticLutN<6, BinType, float>::Create((index_t)O);
+    std::istringstream is(std::string((char const *)bytes, (size_t)size), std::ios::binary);
+    m->LoadObject(is);
+    if ((int)m->GetOutputNodeSize() != O) { return -1; }
+    get_wiring(*m, O, idx);
+    { auto Wp = m->lock_W_const(); for (int i = 0; i < O * 64; ++i) { W[i] = Wp(i / 64, i % 64); } }
+    std::snprintf(name, (size_t)name_cap, "%s", m->GetName().c_str());
+    return (int)m->GetInputNodeSize();
+}
+
+template <typename BinType>
+long dump_differentiable(int I, int O, std::int32_t const *idx, float const *W, float const *mean, float const *var, int flags,
+                         float const *scalars, char const *name, unsigned char *out, long cap)
+{
+    typename bb::DifferentiableLutN<6, BinType, float>::create_t c;
+    c.output_shape = {(index_t)O};
+    c.batch_norm = (flags & 4) != 0;
+    c.binary = (flags & 1) != 0;
+    c.momentum = scalars[0]; c.gamma = scalars[1]; c.beta = scalars[2];
+    auto m = bb::DifferentiableLutN<6, BinType, float>::Create(c);
+    if (name && *name) { m->SetName(name); }
+    m->SetInputShape({(index_t)I});
+    put_wiring(*m, O, idx);
+    { auto Wp = m->lock_W(); for (int i = 0; i < O * 64; ++i) { Wp(i / 64, i % 64) = W[i]; } }
+    { auto p = m->lock_mean(); for (int o = 0; o < O; ++o) { p[o] = mean[o]; } }
+    { auto p = m->lock_var();  for (int o = 0; o < O; ++o) { p[o] = var[o]; } }
+    m->SendCommand("lut_binarize " + onoff(flags & 2));
+    return emit(*m, out, cap);
+}
+template <typename BinType>
+int load_differentiable(unsigned char const *bytes, long size, int O, std::int32_t *idx, float *W, float *mean, float *var, char *name, int name_cap)
+{
+    auto m = bb::DifferentiableLutN<6, BinType, float>::Create((index_t)O);
+    std::istringstream is(std::string((char const *)bytes, (size_t)size), std::ios::binary);
+    m->LoadObject(is);
+    if ((int)m->GetOutputNodeSize() != O) { return -1; }
+    get_wiring(*m, O, idx);
+    { auto Wp = m->lock_W_const(); for (int i = 0; i < O * 64; ++i) { W[i] = Wp(i / 64, i % 64); } }
+    { auto p = m->lock_mean_const(); for (int o = 0; o < O; ++o) { mean[o] = p[o]; } }
+    { auto p = m->lock_var_const();  for (int o = 0; o < O; ++o) { var[o] = p[o]; } }
+    std::snprintf(name, (size_t)name_cap, "%s", m->GetName().c_str());
+    return (int)m->GetInputNodeSize();
+}
+
+}  // namespace
+
+extern "C" long bbref_DumpLutObject(int kind, int bit, int I, int O, std::int32_t const *idx, void const *params, float const *mean,
+                                    float const *var, int flags, float const *scalars, char const *name, unsigned char *out, long cap)
+{
+    if (kind == 0) { return bit ? dump_stochastic<bb::Bit>(I, O, idx, (float const *)params, flags, name, out, cap)
+                                : dump_stochastic<float>(I, O, idx, (float const *)params, flags, name, out, cap); }
+    if (kind == 1) { return bit ? dump_differentiable<bb::Bit>(I, O, idx, (float const *)params, mean, var, flags, scalars, name, out, cap)
+                                : dump_differentiable<float>(I, O, idx, (float const *)params, mean, var, flags, scalars, name, out, cap); }
+    auto m = bb::BinaryLutN<6, bb::Bit, float>::Create((index_t)O);
+    if (name && *name) { m->SetName(name); }
+    m->SetInputShape({(index_t)I});
+    put_wiring(*m, O, idx);
+    std::int32_t const *table = (std::int32_t const *)params;
+    for (int o = 0; o < O; ++o) { for (int b = 0; b < 64; ++b) { m->SetLutTable(o, b, ((table[o * 2 + b / 32] >> (b % 32)) & 1) != 0); } }
+    return emit(*m, out, cap);
+}
+
+// returns the input node count of the loaded layer (negative on a mismatch)
+extern "C" int bbref_LoadLutObject(int kind, int bit, unsigned char const *bytes, long size, int O, std::int32_t *idx, void *params,
+                                   float *mean, float *var, char *name, int name_cap)
+{
+    if (kind == 0) { return bit ? load_stochastic<bb::Bit>(bytes, size, O, idx, (float *)params, name, name_cap)
+                                : load_stochastic<float>(bytes, size, O, idx, (float *)params, name, name_cap); }
+    if (kind == 1) { return bit ? load_differentiable<bb::Bit>(bytes, size, O, idx, (float *)params, mean, var, name, name_cap)
+                                : load_differentiable<float>(bytes, size, O, idx, (float *)params, mean, var, name, name_cap); }
+    auto m = bb::BinaryLutN<6, bb::Bit, float>::Create((index_t)O);
+    std::istringstream is(std::string((char const *)bytes, (size_t)size), std::ios::binary);
+    m->LoadObject(is);
+    if ((int)m->GetOutputNodeSize() != O) { return -1; }
+    get_wiring(*m, O, idx);
+    std::int32_t *table = (std::int32_t *)params;
+    for (int o = 0; o < O; ++o) {
+        table[o * 2] = table[o * 2 + 1] = 0;
+        for (int b = 0; b < 64; ++b) { if (m->GetLutTable(o, b)) { table[o * 2 + b / 32] |= (std::int32_t)(1u << (b % 32)); } }
+    }
+    std::snprintf(name, (size_t)name_cap, "%s", m->GetName().c_str());
+    return (int)m->GetInputNodeSize();
 }

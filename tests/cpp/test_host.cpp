@@ -3,11 +3,13 @@
 #include <cstdio>
 #include <map>
 #include <set>
+#include <sstream>
 #include <vector>
 
 #include "bb/StochasticLutN.h"
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
+#include "bb/ObjectLoader.h"
 #include "../../binarybrain_amd/csrc/tile_divisor.hpp"
 
 extern "C" int oracle_ReverseTable(int n, std::int32_t const *idx, int input_node_size, int output_node_size, std::int32_t *rev, int rev_cap);
@@ -132,6 +134,58 @@ int main(void)
         for (int i = 0; i < 6; ++i) { seen.insert(bl->GetNodeConnectionIndex(4, i)); }
         CHECK(seen.size() == 6);
         CHECK(bl->Backward(bb::FrameBuffer(8, {5}, BB_TYPE_FP32, true)).GetNodeSize() == 9);
+    }
+    // serialization, in the shape of the reference's tests (tests/gtest/DifferentiableLutTest.cpp:10-53: dump, load into a
+    // fresh layer, compare; tests/gtest/ObjectTest.cpp:191-216: reconstruct by the recorded name)
+    {
+        auto lut0 = bb::DifferentiableLutN<6, float>::Create(16);
+        lut0->SetInputShape({16});
+        { auto W = lut0->lock_W(); W(5, 9) = 0.125f; }
+        { auto v = lut0->lock_var(); v[3] = 2.5f; }
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        lut0->DumpObject(ss);
+        auto lut1 = bb::DifferentiableLutN<6, float>::Create(16);
+        lut1->LoadObject(ss);
+        CHECK(lut0->GetGamma() == lut1->GetGamma() && lut0->GetBeta() == lut1->GetBeta());
+        CHECK(lut0->GetOutputShape() == lut1->GetOutputShape() && lut0->GetInputShape() == lut1->GetInputShape());
+        bool same = true;
+        for (bb::index_t o = 0; o < lut0->GetOutputNodeSize(); ++o) {
+            for (bb::index_t i = 0; i < lut0->GetNodeConnectionSize(o); ++i) { same = same && (lut0->GetNodeConnectionIndex(o, i) == lut1->GetNodeConnectionIndex(o, i)); }
+        }
+        CHECK(same);
+        { auto a = lut0->lock_W_const(); auto b = lut1->lock_W_const(); for (int k = 0; k < 16 * 64; ++k) { same = same && (a[k] == b[k]); } }
+        { auto v = lut1->lock_var_const(); same = same && (v[3] == 2.5f) && (v[4] == 1.0f); }
+        CHECK(same);
+        CHECK(lut1->GetGradients().GetSize() == 1 && lut1->dW().GetShape() == bb::indices_t({16, 64}));
+
+        auto model = bb::DifferentiableLutN<6, bb::Bit, float>::Create(bb::indices_t({1, 2, 3}));
+        model->SetInputShape({32, 8});
+        CHECK(model->GetObjectName() == "DifferentiableLut6_bit_fp32");
+        std::stringstream s2(std::ios::in | std::ios::out | std::ios::binary);
+        model->DumpObject(s2);
+        auto obj = std::dynamic_pointer_cast<bb::DifferentiableLutN<6, bb::Bit, float>>(bb::Object_Load(s2));
+        CHECK((bool)obj);
+        if (obj) {
+            CHECK(obj->GetObjectName() == model->GetObjectName());
+            CHECK(obj->GetInputShape() == bb::indices_t({32, 8}) && obj->GetOutputShape() == bb::indices_t({1, 2, 3}));
+        }
+        // a layer of another class or width does not load into this one, and a name nobody knows reconstructs to nothing
+        std::stringstream s3(std::ios::in | std::ios::out | std::ios::binary);
+        model->DumpObject(s3);
+        bool threw = false;
+        try { bb::StochasticLutN<6, bb::Bit>::Create(6)->LoadObject(s3); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);
+        std::stringstream s4(std::ios::in | std::ios::out | std::ios::binary);
+        s4.write("BB_OBJ", 6); bb::SaveValue(s4, (std::int64_t)1); bb::SaveValue(s4, std::string("NoSuchLayer"));
+        CHECK(!bb::Object_Load(s4));
+        // tensors on their own
+        bb::Tensor_<std::int32_t> t(bb::indices_t({2, 3}), true);
+        { auto p = t.Lock(); for (int k = 0; k < 6; ++k) { p[k] = k + 1; } }
+        std::stringstream s5(std::ios::in | std::ios::out | std::ios::binary);
+        t.DumpObject(s5);
+        auto t2 = std::dynamic_pointer_cast<bb::Tensor_<std::int32_t>>(bb::Object_Load(s5));
+        CHECK(t2 && t2->GetShape() == bb::indices_t({2, 3}));
+        if (t2) { auto p = t2->LockConst(); CHECK(p(1, 1) == 5 && p(1, 2) == 6); }          // ObjectTest.cpp:185-186
     }
     // workgroup index -> (frame chunk, node tile) without an integer division: exact for every index below 2^31
     {

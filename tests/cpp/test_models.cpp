@@ -17,6 +17,7 @@
 #include "bb/AverageLut.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
+#include "bb/ObjectLoader.h"
 
 extern "C" {
 void oracle_fp32_AverageLut_Forward(float const *x, float *y, std::int32_t const *idx, int n, int node_size, int frame_size, int frame_stride, int binarize_input, int binarize_output);
@@ -389,6 +390,51 @@ static void test_tail(void)
     CHECK(metrics->GetMetrics() == hits / 5.0, "accuracy %f, expected %f", metrics->GetMetrics(), hits / 5.0);
 }
 
+// The trained-layer hand-off end to end through files: a DifferentiableLut6 on packed bits is written as a `.bb_net` object,
+// reconstructed from the file by its recorded name, gives the same inference output, is tabulated into a BinaryLut6
+// (ImportLayer), which is written and read back as well and reproduces those bits on the device.
+static void test_hand_off_through_files(void)
+{
+    int const I = 48, O = 40, F = 300;
+    std::mt19937_64 mt(17);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    auto src = bb::DifferentiableLutN<6, bb::Bit>::Create(O);
+    src->SetName("trained");
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_BIT);
+    src->SetInputShape(x_buf.GetShape());
+    { auto Wp = src->lock_W(); for (int k = 0; k < O * 64; ++k) { Wp[k] = uni(mt); } }
+    { auto m = src->lock_mean(); auto v = src->lock_var(); for (int o = 0; o < O; ++o) { m[o] = 0.35f + 0.3f * uni(mt); v[o] = 0.02f + 0.1f * uni(mt); } }
+    { auto xp = x_buf.Lock<bb::Bit>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { xp.Set(f, n, bb::Bit((mt() & 1) != 0)); } }
+    std::string const dir = "/tmp/";
+    CHECK(src->DumpToFile(dir + "bbhip_hand_off_layer.bb_net"), "DumpToFile");
+    auto loaded = std::dynamic_pointer_cast<bb::DifferentiableLutN<6, bb::Bit>>(bb::Object_LoadFromFile(dir + "bbhip_hand_off_layer.bb_net"));
+    CHECK((bool)loaded, "Object_LoadFromFile did not reconstruct a DifferentiableLut6_bit_fp32");
+    if (!loaded) { return; }
+    CHECK(loaded->GetName() == "trained", "name %s", loaded->GetName().c_str());
+    auto y_src = src->Forward(x_buf, false);
+    auto y_loaded = loaded->Forward(x_buf, false);
+    auto dst = bb::BinaryLutN<6, bb::Bit>::Create(O);
+    dst->SetInputShape(x_buf.GetShape());
+    dst->ImportLayer(loaded);
+    CHECK(dst->DumpToFile(dir + "bbhip_hand_off_table.bb_net"), "DumpToFile");
+    auto table = std::dynamic_pointer_cast<bb::BinaryLutN<6, bb::Bit>>(bb::Object_LoadFromFile(dir + "bbhip_hand_off_table.bb_net"));
+    CHECK((bool)table, "Object_LoadFromFile did not reconstruct a BinaryLut6_bit_fp32");
+    if (!table) { return; }
+    auto y_table = table->Forward(x_buf);
+    auto a = y_src.LockConst<bb::Bit>(); auto b = y_loaded.LockConst<bb::Bit>(); auto c = y_table.LockConst<bb::Bit>();
+    size_t reload = 0, tabulated = 0, ones = 0;
+    for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) {
+        reload += ((bool)a.Get(f, n) != (bool)b.Get(f, n));
+        tabulated += ((bool)a.Get(f, n) != (bool)c.Get(f, n));
+        ones += (bool)a.Get(f, n);
+    }
+    CHECK(reload == 0, "reloaded layer: %zu mismatching bits", reload);
+    CHECK(tabulated == 0, "tabulated layer: %zu mismatching bits", tabulated);
+    CHECK(ones > (size_t)O * F / 10 && ones < (size_t)O * F * 9 / 10, "degenerate outputs (%zu ones)", ones);
+    std::remove((dir + "bbhip_hand_off_layer.bb_net").c_str());
+    std::remove((dir + "bbhip_hand_off_table.bb_net").c_str());
+}
+
 int main(void)
 {
     if (!bb::Manager::IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
@@ -416,6 +462,7 @@ int main(void)
         test_adam();
         test_conv_plumbing();
         test_tail();
+        test_hand_off_through_files();
     }
     catch (std::exception const &e) {
         std::printf("exception: %s\n", e.what());

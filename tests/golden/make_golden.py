@@ -234,15 +234,36 @@ def tail_cases():
     np.savez_compressed(os.path.join(OUT, "tail.npz"), **cases)
 
 
+def object_cases():
+    """6-input LUT layers serialized by the reference's own Object::DumpObject (`.bb_net` object bytes)."""
+    rng = np.random.default_rng(20240617)
+    cases = {}
+    k = 0
+    for (kind, bit, I, O, flags, name) in [("stochastic", 0, 20, 7, 2, ""), ("stochastic", 1, 9, 3, 3, "lut_a"),
+                                            ("differentiable", 0, 16, 5, 5, "layer0"), ("differentiable", 1, 12, 4, 7, ""),
+                                            ("differentiable", 0, 8, 2, 0, "plain"), ("binary", 1, 33, 11, 0, "packed")]:
+        idx = np.stack([rng.choice(I, 6, replace=False) for _ in range(O)]).astype(np.int32)
+        params = rng.integers(-2**31, 2**31, (O, 2)).astype(np.int32) if kind == "binary" else rng.random((O, 64)).astype(np.float32)
+        mean = rng.random(O).astype(np.float32); var = (rng.random(O) + 0.5).astype(np.float32)
+        data = oracle.ref_dump_lut_object(kind, bit, I, idx, params, mean, var, flags, (0.75, 0.4, 0.6), name)
+        q = "o%d_" % k
+        cases.update({q + "desc": np.array([oracle.LUT_OBJECT_KINDS[kind], bit, I, O, flags], np.int32), q + "name": np.frombuffer(name.encode(), np.uint8),
+                      q + "idx": idx, q + "params": params, q + "mean": mean, q + "var": var, q + "bytes": np.frombuffer(data, np.uint8)})
+        k += 1
+    cases["object_count"] = np.array([k], np.int32)
+    np.savez_compressed(os.path.join(OUT, "objects.npz"), **cases)
+
+
 if __name__ == "__main__":
     assert oracle.have_ref(), "build oracle/_ref first (make -C oracle ref)"
-    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam", "conv", "tail"]
+    which = sys.argv[1:] or ["stochastic", "differentiable", "binary", "adam", "conv", "tail", "objects"]
     if "stochastic" in which: stochastic_cases()
     if "differentiable" in which: differentiable_cases()
     if "binary" in which: binary_cases()
     if "adam" in which: adam_cases()
     if "conv" in which: conv_cases()
     if "tail" in which: tail_cases()
+    if "objects" in which: object_cases()
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)), "bytes")
