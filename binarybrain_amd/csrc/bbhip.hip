@@ -760,9 +760,10 @@ int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_st
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  border_mode, border_value, 0, 0};
     if (check_im2col(a, false, __func__)) { return 1; }
-    a.ox_tiles = ceil_div(a.ow, kTile);
+    if ((long long)a.oh * a.ow > 0x7fffffffLL) { return fail("%s: output plane too large", __func__); }
+    a.q_tiles = ceil_div(a.oh * a.ow, kTile);
     a.f_tiles  = ceil_div(a.input_frame_size, kTile);
-    long long const blocks = (long long)a.c * a.fh * a.fw * a.oh * a.ox_tiles * a.f_tiles;
+    long long const blocks = (long long)a.c * a.fh * a.fw * a.q_tiles * a.f_tiles;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(im2col_forward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a);
@@ -799,12 +800,16 @@ int bbhip_fp32_Im2Col_Backward(float const *dev_dy_buf, float *dev_dx_buf, int x
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  0, 0.0f, 0, 0};
     if (check_im2col(a, false, __func__)) { return 1; }
-    int const x_tiles = ceil_div(a.w, kTile);
-    a.f_tiles = ceil_div(a.input_frame_size, kTile);
-    long long const blocks = (long long)a.c * a.h * x_tiles * a.f_tiles;
+    if ((long long)a.h * a.w > 0x7fffffffLL) { return fail("%s: image too large", __func__); }
+    int const p_tiles = ceil_div(a.h * a.w, kTile);
+    // 64 frames per block, or 16 when that leaves fewer than eight blocks per compute unit
+    int const tf = ((long long)a.c * p_tiles * ceil_div(a.input_frame_size, 64) >= 2048) ? 64 : 16;
+    a.f_tiles = ceil_div(a.input_frame_size, tf);
+    long long const blocks = (long long)a.c * p_tiles * a.f_tiles;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
-    hipLaunchKernelGGL(im2col_backward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, x_tiles);
+    if (tf == 64) { hipLaunchKernelGGL(im2col_backward_kernel<64>, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, p_tiles); }
+    else          { hipLaunchKernelGGL(im2col_backward_kernel<16>, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, p_tiles); }
     BBHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -27,7 +27,7 @@ struct Im2ColArgs {
     int w, h, c, ow, oh, output_frame_stride, fw, fh;
     int border_mode;
     float border_value;
-    int ox_tiles, f_tiles;
+    int q_tiles, f_tiles;      // q_tiles: 64-position tiles of the flattened output plane (forward)
 };
 
 // include/bb/ConvolutionIm2Col.h:251-286
@@ -51,24 +51,26 @@ __device__ __forceinline__ bool im2col_source(Im2ColArgs const &a, int oy, int o
     return im2col_border(a.border_mode, ix, iy, a.w, a.h);
 }
 
-// block = (output node, oy, 64 window columns, 64 input frames)
+// block = (output node, 64 window positions of the flattened (oy, ox) plane, 64 input frames): rows of the input are read
+// along the frames, the tile is written along the window positions, which are contiguous in the output
 __global__ __launch_bounds__(kConvBlock) void im2col_forward_kernel(Im2ColArgs a)
 {
-    __shared__ float tile[kTile][kTile + 1];                 // [ox][frame]
+    __shared__ float tile[kTile][kTile + 1];                 // [window position][frame]
     int b = blockIdx.x;
     int const ft = b % a.f_tiles;  b /= a.f_tiles;
-    int const xt = b % a.ox_tiles; b /= a.ox_tiles;
-    int const oy = b % a.oh;       b /= a.oh;
+    int const qt = b % a.q_tiles;  b /= a.q_tiles;
     int const node = b;                                      // (c*fh + fy)*fw + fx
     int const fx = node % a.fw, fy = (node / a.fw) % a.fh, c = node / (a.fw * a.fh);
     int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int const f0 = ft * kTile, ox0 = xt * kTile;
+    int const f0 = ft * kTile, q0 = qt * kTile;
+    int const plane = a.oh * a.ow;
     float const *x = static_cast<float const *>(a.x);
     float *y = static_cast<float *>(a.y);
 
     for (int i = wave; i < kTile; i += kConvBlock / 64) {
-        int const ox = ox0 + i;
-        if (ox >= a.ow) { break; }
+        int const q = q0 + i;
+        if (q >= plane) { break; }
+        int const oy = q / a.ow, ox = q - oy * a.ow;
         int iy, ix;
         bool const have = im2col_source(a, oy, ox, fy, fx, iy, ix);      // wave-uniform
         float v = a.border_value;
@@ -78,11 +80,10 @@ __global__ __launch_bounds__(kConvBlock) void im2col_forward_kernel(Im2ColArgs a
         tile[i][lane] = v;
     }
     __syncthreads();
-    size_t const plane = (size_t)a.oh * a.ow;
     for (int f = wave; f < kTile; f += kConvBlock / 64) {
         if (f0 + f >= a.input_frame_size) { break; }
-        if (ox0 + lane < a.ow) {
-            y[(size_t)node * a.output_frame_stride + (size_t)(f0 + f) * plane + (size_t)oy * a.ow + ox0 + lane] = tile[lane][f];
+        if (q0 + lane < plane) {
+            y[(size_t)node * a.output_frame_stride + (size_t)(f0 + f) * plane + q0 + lane] = tile[lane][f];
         }
     }
 }
@@ -114,29 +115,34 @@ __global__ __launch_bounds__(kConvBlock) void im2col_forward_bit_kernel(Im2ColAr
 }
 
 // dx[(c, y, x)][f] = sum over the taps (fy, fx) whose window holds (y, x), in (fy, fx) order, of dy[(c, fy, fx)][(f, oy, ox)]
-// (include/bb/ConvolutionIm2Col.h:411-452: border replicas carry no gradient).  block = (c, y, 64 columns, 64 frames);
-// the sums are formed with one lane per column (runs along ox are contiguous in dy) and transposed through LDS.
-__global__ __launch_bounds__(kConvBlock) void im2col_backward_kernel(Im2ColArgs a, int x_tiles)
+// (include/bb/ConvolutionIm2Col.h:411-452: border replicas carry no gradient).  block = (c, 64 pixels of the flattened
+// image, 64 frames): one lane per pixel forms the sums (pixels of one image row are contiguous along ox in dy), which are
+// then transposed through LDS so that the stores run along the frames.  Flattening keeps the lanes busy for images
+// narrower than a wavefront; TF (frames per block) is 64, or 16 when the batch is too small to fill the device otherwise.
+template <int TF>
+__global__ __launch_bounds__(kConvBlock) void im2col_backward_kernel(Im2ColArgs a, int p_tiles)
 {
-    __shared__ float tile[kTile][kTile + 1];                 // [x][frame]
+    __shared__ float tile[kTile][TF + 1];                    // [pixel][frame]
     int b = blockIdx.x;
     int const ft = b % a.f_tiles; b /= a.f_tiles;
-    int const xt = b % x_tiles;   b /= x_tiles;
-    int const y  = b % a.h;       b /= a.h;
+    int const pt = b % p_tiles;   b /= p_tiles;
     int const c  = b;
     int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int const f0 = ft * kTile, x0 = xt * kTile;
-    int const x = x0 + lane;
+    int const f0 = ft * TF, p0 = pt * kTile;
+    int const hw = a.h * a.w;
+    int const p = p0 + lane;
     float const *dy = static_cast<float const *>(a.x);       // the gradient buffer comes in through the first slot
     float *dx = static_cast<float *>(a.y);
-    constexpr int kPer = kTile / (kConvBlock / 64);          // frames per thread
+    constexpr int kWaves = kConvBlock / 64;
+    constexpr int kPer = TF / kWaves;                        // frames per thread
     float acc[kPer];
 #pragma unroll
     for (int j = 0; j < kPer; ++j) { acc[j] = 0.0f; }
 
     int const iy_limit = (a.oh - 1) * a.y_stride, ix_limit = (a.ow - 1) * a.x_stride;
     size_t const plane = (size_t)a.oh * a.ow;
-    if (x < a.w) {
+    if (p < hw) {
+        int const y = p / a.w, x = p - y * a.w;
         int const x_align = x % a.x_stride, y_align = y % a.y_stride;
         for (int fy = y_align; fy < a.fh; fy += a.y_stride) {
             int const iy = y - fy + a.y_offset;
@@ -148,19 +154,21 @@ __global__ __launch_bounds__(kConvBlock) void im2col_backward_kernel(Im2ColArgs 
                                       + (size_t)(iy / a.y_stride) * a.ow + (ix / a.x_stride);
 #pragma unroll
                 for (int j = 0; j < kPer; ++j) {
-                    int const f = f0 + wave + j * (kConvBlock / 64);
+                    int const f = f0 + wave + j * kWaves;
                     if (f < a.input_frame_size) { acc[j] += row[(size_t)f * plane]; }
                 }
             }
         }
     }
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) { tile[lane][wave + j * (kConvBlock / 64)] = acc[j]; }
+    for (int j = 0; j < kPer; ++j) { tile[lane][wave + j * kWaves] = acc[j]; }
     __syncthreads();
-    for (int i = wave; i < kTile; i += kConvBlock / 64) {
-        if (x0 + i >= a.w) { break; }
-        if (f0 + lane < a.input_frame_size) {
-            dx[((size_t)(c * a.h + y) * a.w + x0 + i) * a.input_frame_stride + f0 + lane] = tile[i][lane];
+    // TF consecutive threads store the TF frames of one pixel
+    constexpr int kPixelsPerPass = kConvBlock / TF;
+    int const fl = threadIdx.x % TF, pl = threadIdx.x / TF;
+    for (int i = pl; i < kTile; i += kPixelsPerPass) {
+        if (p0 + i < hw && f0 + fl < a.input_frame_size) {
+            dx[((size_t)c * hw + p0 + i) * a.input_frame_stride + f0 + fl] = tile[i][fl];
         }
     }
 }

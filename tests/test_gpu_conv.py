@@ -38,6 +38,7 @@ IM2COL_SHAPES = [
     (2, 6, 7, 35, 3, 3, 1, 1, "same", "reflect"),
     (3, 9, 8, 3, 3, 3, 1, 2, "same", "constant"),
     (1, 1, 1, 1, 1, 1, 1, 1, "valid", "constant"),
+    (32, 8, 8, 4096, 2, 1, 1, 1, "valid", "constant"),         # enough blocks for the backward kernel's 64-frame tiles
 ]
 
 
