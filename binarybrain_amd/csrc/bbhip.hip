@@ -178,7 +178,7 @@ int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, hipStream
 template <int N>
 int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStream_t st)
 {
-    dim3 const grid(a.slab_count * a.tiles.count), block(kBlock);
+    dim3 const grid(a.tt.blocks + a.slab_count * a.tiles.count), block(kBlock);
 #define BBHIP_BWD_CASE(X, K, M) if (xmode == X && kind == K && dxmode == M) { hipLaunchKernelGGL((lut_backward_kernel<N, X, K, M>), grid, block, 0, st, a); return 0; }
     BBHIP_BWD_CASE(kXClamp,  0, kDxAtomic) BBHIP_BWD_CASE(kXClamp,  0, kDxTmp)
     BBHIP_BWD_CASE(kXBinary, 0, kDxAtomic) BBHIP_BWD_CASE(kXBinary, 0, kDxTmp)
@@ -199,7 +199,7 @@ int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStre
 template <int N, int U>
 int dispatch_dx_u(int xmode, DxArgs const &a, hipStream_t st)
 {
-    dim3 const grid(a.chunk_count * a.tiles.count), block(kBlock);
+    dim3 const grid(a.fin_blocks + a.chunk_count * a.tiles.count), block(kBlock);
     switch (xmode) {
     case kXClamp:  hipLaunchKernelGGL((lut_dx_kernel<N, kXClamp, U>),  grid, block, 0, st, a); return 0;
     case kXBinary: hipLaunchKernelGGL((lut_dx_kernel<N, kXBinary, U>), grid, block, 0, st, a); return 0;
@@ -383,28 +383,32 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     size_t const stat_bytes = c.bn ? align256((size_t)slab_total * c.output_node_size * 2 * sizeof(float)) : 0;
     size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;
     size_t const dtab_bytes = align256(term_count * sizeof(int));
-    size_t const otab_bytes = (dxmode == kDxNone) ? c_bytes : 0;        // plain-basis coefficients for the dx kernel
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes + dyh_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes, &base)) { return 1; }
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
     int   *term = reinterpret_cast<int *>(base + c_bytes + part_bytes + stat_bytes);
-    float *P    = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
-    float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + otab_bytes);
+    float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
 
-    launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
-    BBHIP_LAUNCH_CHECK();
+    // centred coefficients: needed where the LUT output is recomputed (batch-norm) or per-connection gradients are formed
+    if (c.bn || dxmode != kDxNone) {
+        launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
+        BBHIP_LAUNCH_CHECK();
+    }
+    // the term table of the dx kernel is built by extra workgroups at the front of the table-gradient launch
+    TermArgs tt{};
     if (dxmode == kDxNone && term_count > 0) {
-        launch_table_prep<N, true>(c.W, P, c.output_node_size, c.lut_binarize, st);
-        BBHIP_LAUNCH_CHECK();
-        size_t const blocks = (term_count + kBlock - 1) / kBlock;
-        if (blocks > 0x7fffffffULL) { return fail("backward: reverse table too large"); }
-        hipLaunchKernelGGL(term_table_kernel<N>, dim3((unsigned)blocks), dim3(kBlock), 0, st, P, c.idx, c.rev, c.rev_stride, c.input_node_size,
-                           (unsigned long long)(uintptr_t)c.x, (unsigned long long)c.x_stride * 4ULL,
-                           (unsigned long long)(uintptr_t)(c.bn ? (void const *)dyh : (void const *)c.dy), (unsigned long long)c.frame_stride * 4ULL, term);
-        BBHIP_LAUNCH_CHECK();
+        size_t const records = (size_t)c.input_node_size * (size_t)(c.rev_stride - 1);
+        size_t const blocks = (((records + kWavesPerBlk - 1) / kWavesPerBlk) + 7) & ~(size_t)7;      // whole rounds over the XCDs
+        if (blocks + (size_t)slab_total * tile_count > 0x7fffffffULL) { return fail("backward: grid too large"); }
+        tt.W = c.W; tt.idx = c.idx; tt.rev = c.rev; tt.term = term;
+        tt.x_base = (unsigned long long)(uintptr_t)c.x; tt.x_row_pitch_bytes = (unsigned long long)c.x_stride * 4ULL;
+        tt.dy_base = (unsigned long long)(uintptr_t)(c.bn ? (void const *)dyh : (void const *)c.dy);
+        tt.dy_row_pitch_bytes = (unsigned long long)c.frame_stride * 4ULL;
+        tt.lut_binarize = c.lut_binarize; tt.rev_stride = c.rev_stride; tt.input_node_size = c.input_node_size;
+        tt.blocks = (int)blocks;
     }
 
     BwdArgs a{};
@@ -421,6 +425,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         a.f_base = 0; a.f_limit = c.frame_size; a.slab_first = 0;
         a.slab_count = ceil_div(c.frame_size, slab);
         a.dx = nullptr; a.dx_stride = 0;
+        a.tt = TermArgs{};
         if (dispatch_backward<N>(c.xmode, 2, kDxTmp, a, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
         hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, kBlock)), dim3(kBlock), 0, st,
@@ -443,6 +448,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         if (dxmode == kDxAtomic)    { a.dx = c.dx;     a.dx_stride = c.frame_stride; }
         else if (dxmode == kDxTmp)  { a.dx = c.dx_tmp; a.dx_stride = c.tmp_frame_stride; }
         else                        { a.dx = dyh;      a.dx_stride = c.frame_stride; }
+        a.tt = (r == 0) ? tt : TermArgs{};
         {
             ScopedTimer tm(kTimeBackward, st);
             if (dispatch_backward<N>(c.xmode, c.bn ? 1 : 0, dxmode, a, st)) { return 1; }
@@ -469,11 +475,16 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
         d.chunk = chunk; d.chunk_count = chunk_count; d.tiles = make_tile_divisor(in_tiles);
         d.bias = c.bias;
+        // folding the slab sums into dW rides at the front of this launch
+        d.fin_partial = part; d.fin_dW = c.dW; d.fin_node_size = c.output_node_size; d.fin_slab_count = slab_total;
+        d.fin_blocks = (ceil_div(c.output_node_size * NN, kBlock) + 7) & ~7;
+        if ((long long)d.fin_blocks + (long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
         {
             ScopedTimer tm(kTimeDx, st);
             if (dispatch_dx<N>(c.xmode, steps, d, st)) { return 1; }
         }
         BBHIP_LAUNCH_CHECK();
+        return 0;
     }
 
     int const total = c.output_node_size * NN;

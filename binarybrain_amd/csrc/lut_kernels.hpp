@@ -65,11 +65,10 @@ __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restr
 
 // dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order)
 template <int N>
-__global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__restrict__ partial, float *__restrict__ dW,
-                                                            int node_size, int slab_count)
+__device__ __forceinline__ void dw_finalize_block(float const *__restrict__ partial, float *__restrict__ dW, int node_size, int slab_count, int block)
 {
     constexpr int NN = 1 << N;
-    int const t = blockIdx.x * kBlock + threadIdx.x;
+    int const t = block * kBlock + threadIdx.x;
     int const total = node_size * NN;
     float v = 0.0f;
     if (t < total) {
@@ -82,6 +81,13 @@ __global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__rest
         v = ((i >> j) & 1) ? (o * 0.5f + v) : (v * 0.5f - o);
     }
     if (t < total) { dW[t] += v; }
+}
+
+template <int N>
+__global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__restrict__ partial, float *__restrict__ dW,
+                                                            int node_size, int slab_count)
+{
+    dw_finalize_block<N>(partial, dW, node_size, slab_count, blockIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -256,6 +262,74 @@ __global__ __launch_bounds__(kBlock) void rsqrt_kernel(float const *__restrict__
     if (i < size) { rstd[i] = 1.0f / sqrtf(var[i]); }
 }
 
+// Term table for the input-centric dx kernel: for input node `in` and its t-th consumer connection (t-th entry of
+// the reverse-table row, e = node*N + k) one record of kTermHead + 2^(N-1) dwords at
+// ((in * max_fan + t) * record):  dwords [2j, 2j+1], j < N-1: the 64-bit device address of the row of the consumer's
+// other input j (ascending connection order, k skipped); dwords [2(N-1), 2(N-1)+1]: the address of the consumer's dy
+// row; rest of the head unused; then the 2^(N-1) coefficients Dk (entries of the consumer's plain-basis table P).  The addresses
+// are final, so the dx kernel spends no scalar arithmetic on them.  All records of one input node are contiguous, so a
+// wavefront reads its whole work list from one base address with scalar loads.
+constexpr int kTermHead = 12;
+
+struct TermArgs {
+    float const *W;             // [O][2^N]
+    int const   *idx;           // [O][N]
+    int const   *rev;           // reverse table [I][rev_stride]
+    int         *term;          // the records
+    unsigned long long x_base, x_row_pitch_bytes, dy_base, dy_row_pitch_bytes;
+    int lut_binarize, rev_stride, input_node_size;
+    int blocks;                 // workgroups that build records (kWavesPerBlk records each); 0 = nothing to build
+};
+
+// one wavefront per record: lane i holds entry i of the consumer's table while it is brought into the plain basis.
+// Slots beyond an input's fan-out are never read by the dx kernel and are left alone.
+template <int N>
+__device__ __forceinline__ void term_table_block(TermArgs const &a, int block)
+{
+    static_assert(2 * N <= kTermHead && kTermHead <= kWave, "head size");
+    constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN;
+    int const max_fan = a.rev_stride - 1;
+    long long const rec = (long long)block * kWavesPerBlk + (int)(threadIdx.x / kWave);
+    if (rec >= (long long)a.input_node_size * max_fan) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+    int const in   = (int)(rec / max_fan);
+    int const slot = (int)(rec - (long long)in * max_fan);
+    int const *r = a.rev + (size_t)in * a.rev_stride;
+    int const cnt  = r[0];
+    int const e    = r[1 + slot];                  // inside the row for every slot: both loads go out together
+    if (slot >= cnt) { return; }
+    int const k    = e % N;
+    int const node = e / N;
+    int *out = a.term + rec * REC;
+
+    if (lane < kTermHead) {
+        int v = 0;
+        if (lane < 2 * N) {
+            int const j = lane >> 1;
+            unsigned long long const addr = (j < N - 1) ? a.x_base + (unsigned long long)a.idx[node * N + ((j < k) ? j : j + 1)] * a.x_row_pitch_bytes
+                                                        : a.dy_base + (unsigned long long)node * a.dy_row_pitch_bytes;
+            v = (lane & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
+        }
+        out[lane] = v;
+    }
+
+    // P = plain-basis coefficients of W' (W' = lut_binarize ? W > 0.5 : W): the butterfly (a, b) -> (a, b - a) per index bit
+    float v = 0.0f;
+    if (lane < NN) {
+        v = a.W[(size_t)node * NN + lane];
+        if (a.lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float const o = __shfl_xor(v, 1 << j, 64);
+        v = ((lane >> j) & 1) ? (v - o) : v;
+    }
+    if (lane < NN && ((lane >> k) & 1)) {
+        int const sidx = (lane & ((1 << k) - 1)) | ((lane >> (k + 1)) << k);      // the entry's index with bit k taken out
+        out[kTermHead + sidx] = __float_as_int(v);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 //  backward
 // ------------------------------------------------------------------------------------------------
@@ -280,6 +354,7 @@ struct BwdArgs {
     int   slab_count;
     TileDivisor tiles;
     float bias, gamma, beta, inv_frames;
+    TermArgs tt;                // kDxNone: the first tt.blocks workgroups of the launch build the dx kernel's term table
 };
 
 enum DxMode : int { kDxAtomic = 0, kDxTmp = 1, kDxNone = 2 };
@@ -292,8 +367,15 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     using D = LutDims<N>;
     __shared__ float red[kWavesPerBlk][16][kWave + 1];
 
+    // The term table of the dx kernel that follows depends on nothing this kernel computes: its workgroups ride at the
+    // front of this launch instead of taking a launch of their own.
+    int bid = blockIdx.x;
+    if (DXMODE == kDxNone && BWD_KIND != 2) {
+        if (bid < a.tt.blocks) { term_table_block<N>(a.tt, bid); return; }
+        bid -= a.tt.blocks;
+    }
     int const B    = a.slab_count * a.tiles.count;
-    int const lid  = xcd_remap(blockIdx.x, B);
+    int const lid  = xcd_remap(bid, B);
     int sl, tile;
     split_tile(lid, a.tiles, sl, tile);
     int const wv   = threadIdx.x / kWave;
@@ -301,9 +383,13 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
+    // the table itself enters only the batch-norm kinds (the LUT output is recomputed) and the per-connection gradients
+    constexpr bool kNeedTable = (BWD_KIND != 0) || (DXMODE != kDxNone);
     float C[D::NN], cv[D::H];
-    LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
-    LutEval<N>::pin_constants(C, cv);
+    if (kNeedTable) {
+        LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
+        LutEval<N>::pin_constants(C, cv);
+    }
     void const *rows[N];
     int ins[N];
 #pragma unroll
@@ -356,7 +442,7 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
             float l[D::L], h[D::H], q[D::H];
             monomials<D::NL>(zl, l);
             monomials<D::NH>(zh, h);
-            if (BWD_KIND != 0 || DXMODE != kDxNone) { LutEval<N>::partial_q(C, cv, l, q); }
+            if (kNeedTable) { LutEval<N>::partial_q(C, cv, l, q); }
 
             if (BWD_KIND != 0) {
                 // hard-tanh window on the batch-norm output (reference: DifferentiableLutN.h:1206-1211, 1241-1246)
@@ -457,67 +543,21 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     }
 }
 
-// Term table for the input-centric dx kernel: for input node `in` and its t-th consumer connection (t-th entry of
-// the reverse-table row, e = node*N + k) one record of kTermHead + 2^(N-1) dwords at
-// ((in * max_fan + t) * record):  dwords [2j, 2j+1], j < N-1: the 64-bit device address of the row of the consumer's
-// other input j (ascending connection order, k skipped); dwords [2(N-1), 2(N-1)+1]: the address of the consumer's dy
-// row; rest of the head unused; then the 2^(N-1) coefficients Dk (taken from the plain-basis table P).  The addresses
-// are final, so the dx kernel spends no scalar arithmetic on them.  All records of one input node are contiguous, so a
-// wavefront reads its whole work list from one base address with scalar loads.
-constexpr int kTermHead = 12;
-
-template <int N>
-__global__ __launch_bounds__(kBlock) void term_table_kernel(float const *__restrict__ P, int const *__restrict__ idx,
-                                                           int const *__restrict__ rev, int rev_stride, int input_node_size,
-                                                           unsigned long long x_base, unsigned long long x_row_pitch_bytes,
-                                                           unsigned long long dy_base, unsigned long long dy_row_pitch_bytes,
-                                                           int *__restrict__ term)
-{
-    static_assert(2 * N <= kTermHead, "head too small");
-    constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN;
-    int const max_fan = rev_stride - 1;
-    long long const t = (long long)blockIdx.x * kBlock + threadIdx.x;
-    long long const total = (long long)input_node_size * max_fan * REC;
-    if (t >= total) { return; }
-    int const w    = (int)(t % REC);
-    long long const rec = t / REC;
-    int const slot = (int)(rec % max_fan);
-    int const in   = (int)(rec / max_fan);
-    int const *r = rev + (size_t)in * rev_stride;
-    bool const live = slot < r[0];
-    int const e    = live ? r[1 + slot] : 0;
-    int const k    = e % N;
-    int const node = e / N;
-    int v = 0;
-    if (w < 2 * N) {
-        int const j = w >> 1;
-        unsigned long long addr = (j < N - 1) ? x_base : dy_base;          // unused slots point at valid memory
-        if (live) {
-            addr = (j < N - 1) ? x_base + (unsigned long long)idx[node * N + ((j < k) ? j : j + 1)] * x_row_pitch_bytes
-                               : dy_base + (unsigned long long)node * dy_row_pitch_bytes;
-        }
-        v = (w & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
-    }
-    else if (w >= kTermHead && live) {
-        int const sidx = w - kTermHead;
-        int const lo = sidx & ((1 << k) - 1);
-        int const hi = sidx >> k;
-        v = __float_as_int(P[(size_t)node * NN + ((hi << (k + 1)) | (1 << k) | lo)]);
-    }
-    term[t] = v;
-}
-
 struct DxArgs {
     void const  *x;
     float const *dy;            // dL/d(LUT output) [O][dy_stride]
     float       *dx;            // [I][dx_stride]
     int const   *rev;           // reverse table [I][rev_stride]: count, then connection ids node*N + k
-    int const   *term;          // term table, see term_table_kernel
+    int const   *term;          // term table, see term_table_block
     int   rev_stride, input_node_size, frame_size;
     int   x_stride, dy_stride, dx_stride;
     int   chunk, chunk_count;
     TileDivisor tiles;
     float bias;
+    // the first fin_blocks workgroups of the launch fold the table-gradient partial sums into dW (dw_finalize_block)
+    float const *fin_partial;
+    float       *fin_dW;
+    int   fin_node_size, fin_slab_count, fin_blocks;
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -634,8 +674,13 @@ template <int N, int XMODE, int U>
 __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 {
     using T = DxTerm<N, XMODE, U>;
+    // the table-gradient partial sums are complete before this launch and independent of it: folding them into dW rides at
+    // the front of this launch instead of taking a launch of its own
+    int bid = blockIdx.x;
+    if (bid < a.fin_blocks) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid); return; }
+    bid -= a.fin_blocks;
     int const B    = a.chunk_count * a.tiles.count;
-    int const lid  = xcd_remap(blockIdx.x, B);
+    int const lid  = xcd_remap(bid, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
     int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
