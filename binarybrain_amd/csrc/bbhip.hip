@@ -397,7 +397,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
         BBHIP_LAUNCH_CHECK();
     }
-    // the term table of the dx kernel is built by extra workgroups at the front of the table-gradient launch
+    // the term table of the dx kernel is built by extra workgroups at the end of the table-gradient launch
     TermArgs tt{};
     if (dxmode == kDxNone && term_count > 0) {
         size_t const records = (size_t)c.input_node_size * (size_t)(c.rev_stride - 1);
@@ -475,7 +475,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
         d.chunk = chunk; d.chunk_count = chunk_count; d.tiles = make_tile_divisor(in_tiles);
         d.bias = c.bias;
-        // folding the slab sums into dW rides at the front of this launch
+        // folding the slab sums into dW rides at the end of this launch
         d.fin_partial = part; d.fin_dW = c.dW; d.fin_node_size = c.output_node_size; d.fin_slab_count = slab_total;
         d.fin_blocks = (ceil_div(c.output_node_size * NN, kBlock) + 7) & ~7;
         if ((long long)d.fin_blocks + (long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }

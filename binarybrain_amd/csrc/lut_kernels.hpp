@@ -354,7 +354,7 @@ struct BwdArgs {
     int   slab_count;
     TileDivisor tiles;
     float bias, gamma, beta, inv_frames;
-    TermArgs tt;                // kDxNone: the first tt.blocks workgroups of the launch build the dx kernel's term table
+    TermArgs tt;                // kDxNone: the last tt.blocks workgroups of the launch build the dx kernel's term table
 };
 
 enum DxMode : int { kDxAtomic = 0, kDxTmp = 1, kDxNone = 2 };
@@ -368,13 +368,12 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     __shared__ float red[kWavesPerBlk][16][kWave + 1];
 
     // The term table of the dx kernel that follows depends on nothing this kernel computes: its workgroups ride at the
-    // front of this launch instead of taking a launch of their own.
-    int bid = blockIdx.x;
+    // end of this launch, where they fill the device while the last slabs drain, instead of taking a launch of their own.
+    int const bid = blockIdx.x;
+    int const B   = a.slab_count * a.tiles.count;
     if (DXMODE == kDxNone && BWD_KIND != 2) {
-        if (bid < a.tt.blocks) { term_table_block<N>(a.tt, bid); return; }
-        bid -= a.tt.blocks;
+        if (bid >= B) { term_table_block<N>(a.tt, bid - B); return; }
     }
-    int const B    = a.slab_count * a.tiles.count;
     int const lid  = xcd_remap(bid, B);
     int sl, tile;
     split_tile(lid, a.tiles, sl, tile);
@@ -554,7 +553,7 @@ struct DxArgs {
     int   chunk, chunk_count;
     TileDivisor tiles;
     float bias;
-    // the first fin_blocks workgroups of the launch fold the table-gradient partial sums into dW (dw_finalize_block)
+    // the last fin_blocks workgroups of the launch fold the table-gradient partial sums into dW (dw_finalize_block)
     float const *fin_partial;
     float       *fin_dW;
     int   fin_node_size, fin_slab_count, fin_blocks;
@@ -675,11 +674,10 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 {
     using T = DxTerm<N, XMODE, U>;
     // the table-gradient partial sums are complete before this launch and independent of it: folding them into dW rides at
-    // the front of this launch instead of taking a launch of its own
-    int bid = blockIdx.x;
-    if (bid < a.fin_blocks) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid); return; }
-    bid -= a.fin_blocks;
-    int const B    = a.chunk_count * a.tiles.count;
+    // the end of this launch instead of taking a launch of its own
+    int const bid = blockIdx.x;
+    int const B   = a.chunk_count * a.tiles.count;
+    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B); return; }
     int const lid  = xcd_remap(bid, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
