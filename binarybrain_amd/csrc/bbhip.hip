@@ -92,7 +92,7 @@ int env_int(char const *name, int def)
 
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 256); return ((v + 63) / 64) * 64; }
-int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 1024);  return ((v + 63) / 64) * 64; }
+int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  return ((v + 63) / 64) * 64; }       // 0: chosen per call
 int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
 int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 2); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
 int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
@@ -142,11 +142,11 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
     default: return fail("LUT width n=%d not in 2..6", n); \
     }
 
-template <int N, bool PLAIN = false>
+template <int N>
 void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st)
 {
     int const total = node_size * (1 << N);
-    hipLaunchKernelGGL((table_prep_kernel<N, PLAIN>), dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize);
+    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize);
 }
 
 template <int N, int XMODE, int YMODE, int KIND>
@@ -363,8 +363,14 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     int const range      = (dxmode == kDxTmp) ? (c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size) : c.frame_size;
     int const range_count = ceil_div(c.frame_size, range);
 
-    // slab length: a wavefront multiple; long enough that the per-slab partial tables stay below 256 MiB
+    // slab length: a wavefront multiple.  Long slabs amortise the cross-lane reduction that ends each of them (4096 frames
+    // unless that leaves fewer than eight workgroups per compute unit), and long enough that the per-slab partial tables
+    // stay below 256 MiB
     int slab = bwd_slab_frames();
+    if (slab == 0) {
+        slab = 4096;
+        while (slab > 256 && (long long)tile_count * range_count * ceil_div(range, slab) < 2048) { slab /= 2; }
+    }
     for (;;) {
         long long slabs = (long long)range_count * ceil_div(range, slab);
         if (slabs * c.output_node_size * NN * (long long)sizeof(float) <= (256LL << 20) || slab >= range) { break; }

@@ -38,10 +38,10 @@ __device__ __forceinline__ float wave_sum(float v)
 
 // ------------------------------------------------------------------------------------------------
 //  table preparation from W' (W' = lut_binarize ? W > 0.5 : W):
-//    PLAIN = false: C = coefficients in the centred monomial basis,  y = sum_S C[S] prod_{j in S} (x_j - 1/2)
-//    PLAIN = true : P = coefficients in the plain monomial basis,    y = sum_S P[S] prod_{j in S} x_j
+//    C = coefficients in the centred monomial basis,  y = sum_S C[S] prod_{j in S} (x_j - 1/2)
+//  (the plain-basis coefficients P,  y = sum_S P[S] prod_{j in S} x_j,  are formed inside term_table_block)
 // ------------------------------------------------------------------------------------------------
-template <int N, bool PLAIN>
+template <int N>
 __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
                                                            int node_size, int lut_binarize)
 {
@@ -57,8 +57,7 @@ __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restr
 #pragma unroll
     for (int j = 0; j < N; ++j) {
         float const o = __shfl_xor(v, 1 << j, 64);
-        if (PLAIN) { v = ((i >> j) & 1) ? (v - o) : v; }
-        else       { v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f; }
+        v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f;
     }
     if (t < total) { C[t] = v; }
 }
