@@ -855,27 +855,30 @@ __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
         asm("v_mov_b32 %0, %1" : "=v"(m_lo[k]) : "s"(lo));
     }
 
-    uint32_t const *rows[6];
+    // rows are addressed through buffer descriptors that end with the last word of the row: lanes beyond it read 0 and
+    // their stores are dropped, so the loop carries neither index clamps nor lane masks
+    uint32_t const row_bytes = (uint32_t)a.word_count * 4u;
+    __amdgpu_buffer_rsrc_t rows[6];
 #pragma unroll
-    for (int k = 0; k < 6; ++k) { rows[k] = a.x + (size_t)a.idx[node * 6 + k] * a.stride; }
-    uint32_t *yr = a.y + (size_t)node * a.stride;
+    for (int k = 0; k < 6; ++k) { rows[k] = row_descriptor(a.x, a.idx[node * 6 + k], a.stride, row_bytes); }
+    __amdgpu_buffer_rsrc_t const yr = row_descriptor(a.y, node, a.stride, row_bytes);
 
     int const w_begin = ck * a.chunk;
-    int const w_end   = min(w_begin + a.chunk, a.word_count);
+    int const w_end   = min(w_begin + a.chunk, a.word_count);       // a.chunk is a multiple of the words per step
     int const w_last  = a.word_count - 1;
     uint32_t const tail_mask = (a.frame_size & 31) ? ((1u << (a.frame_size & 31)) - 1u) : 0xffffffffu;
 
-    for (int w0 = w_begin; w0 < w_end; w0 += kWave * WPL) {
+    uint32_t off = (uint32_t)(w_begin + lane) * 4u;
+    for (int w0 = w_begin; w0 < w_end; w0 += kWave * WPL, off += kWave * WPL * 4u) {
         uint32_t xv[WPL][6];
 #pragma unroll
         for (int u = 0; u < WPL; ++u) {
-            uint32_t const off = (uint32_t)min(w0 + u * kWave + lane, w_last) * 4u;
 #pragma unroll
-            for (int k = 0; k < 6; ++k) { xv[u][k] = *reinterpret_cast<uint32_t const *>(reinterpret_cast<char const *>(rows[k]) + off); }
+            for (int k = 0; k < 6; ++k) { xv[u][k] = __builtin_amdgcn_raw_buffer_load_b32(rows[k], off + u * (kWave * 4u), 0, 0); }
         }
+        bool const has_tail = (w0 + kWave * WPL > w_last);          // wave-uniform: only the last step of a row
 #pragma unroll
         for (int u = 0; u < WPL; ++u) {
-            int const w = w0 + u * kWave + lane;
             uint32_t t[32];
 #pragma unroll
             for (int k = 0; k < 32; ++k) { t[k] = bfi_vsv(xv[u][0], m_hi[k], m_lo[k]); }
@@ -885,8 +888,9 @@ __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
                 for (int k = 0; k < (32 >> lv); ++k) { t[k] = bfi_vvv(xv[u][lv], t[2 * k + 1], t[2 * k]); }
             }
             uint32_t r = t[0];
-            if (w == w_last) { r &= tail_mask; }
-            if (w < w_end) { __builtin_nontemporal_store(r, yr + w); }     // streamed once: keep it from displacing x rows in L2
+            if (has_tail && (w0 + u * kWave + lane == w_last)) { r &= tail_mask; }
+            // streamed once (non-temporal): keep it from displacing x rows in L2
+            __builtin_amdgcn_raw_buffer_store_b32(r, yr, off + u * (kWave * 4u), 0, 2);
         }
     }
 }
