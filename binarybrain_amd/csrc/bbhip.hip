@@ -91,6 +91,7 @@ int env_int(char const *name, int def)
 }
 
 // frames per unit; both are rounded to wavefront multiples where used
+int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); return v >= 2 ? 2 : 1; }
 int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 256); return ((v + 63) / 64) * 64; }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  return ((v + 63) / 64) * 64; }       // 0: chosen per call
 int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
@@ -150,16 +151,18 @@ void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize
 }
 
 template <int N, int XMODE, int YMODE, int KIND>
-void launch_forward(FwdArgs const &a, hipStream_t st)
+void launch_forward(FwdArgs const &a, int npw, hipStream_t st)
 {
-    hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND>), dim3(a.chunk_count * a.tiles.count), dim3(kBlock), 0, st, a);
+    dim3 const grid(a.chunk_count * a.tiles.count), block(kBlock);
+    if (npw == 2) { hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND, 2>), grid, block, 0, st, a); }
+    else          { hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND, 1>), grid, block, 0, st, a); }
 }
 
 // xmode / ymode / kind are runtime values here; the combinations that exist are enumerated explicitly
 template <int N>
-int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, hipStream_t st)
+int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, int npw, hipStream_t st)
 {
-#define BBHIP_FWD_CASE(X, Y, K) if (xmode == X && ymode == Y && kind == K) { launch_forward<N, X, Y, K>(a, st); return 0; }
+#define BBHIP_FWD_CASE(X, Y, K) if (xmode == X && ymode == Y && kind == K) { launch_forward<N, X, Y, K>(a, npw, st); return 0; }
     BBHIP_FWD_CASE(kXClamp,  kYClamp,    0)
     BBHIP_FWD_CASE(kXBinary, kYClamp,    0)
     BBHIP_FWD_CASE(kXBit,    kYClamp,    0)
@@ -255,9 +258,10 @@ template <int N>
 int run_forward(ForwardCall const &c, hipStream_t st)
 {
     constexpr int NN = 1 << N;
+    int const npw         = fwd_nodes_per_wave();
     int const chunk       = fwd_chunk_frames();
     int const chunk_count = ceil_div(c.frame_size, chunk);
-    int const tile_count  = ceil_div(c.node_size, kWavesPerBlk);
+    int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
     if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("forward: grid too large"); }
 
     size_t const c_bytes    = align256((size_t)c.node_size * NN * sizeof(float));
@@ -282,7 +286,7 @@ int run_forward(ForwardCall const &c, hipStream_t st)
     int kind = 0;
     if (c.bn == 1) {
         a.stat_partial = stat;
-        if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, st)) { return 1; }
+        if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
         hipLaunchKernelGGL(bn_forward_finalize_kernel, dim3(ceil_div(c.node_size, kBlock)), dim3(kBlock), 0, st,
                            stat, C, NN, c.mean, c.rstd, c.running_mean, c.running_var, c.momentum,
@@ -300,7 +304,7 @@ int run_forward(ForwardCall const &c, hipStream_t st)
     }
     {
         ScopedTimer tm(kTimeForward, st);
-        if (dispatch_forward<N>(c.xmode, c.ymode, kind, a, st)) { return 1; }
+        if (dispatch_forward<N>(c.xmode, c.ymode, kind, a, npw, st)) { return 1; }
     }
     BBHIP_LAUNCH_CHECK();
     return 0;

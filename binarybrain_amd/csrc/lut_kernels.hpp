@@ -134,7 +134,10 @@ struct FwdArgs {
 };
 
 // FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only
-template <int N, int XMODE, int YMODE, int FWD_KIND>
+// NPW: nodes per wavefront.  A wavefront issues the loads of NPW nodes x U steps together (NPW x U = 4); with two nodes the
+// set-up of a wavefront (index and table loads, two memory latencies before the first gather can go out) is shared by twice
+// the work.
+template <int N, int XMODE, int YMODE, int FWD_KIND, int NPW>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void lut_forward_kernel(FwdArgs a)
 {
     using D = LutDims<N>;
@@ -142,44 +145,55 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     int const lid  = xcd_remap(blockIdx.x, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
-    int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
-    if (node >= a.node_size) { return; }
+    int const node0 = __builtin_amdgcn_readfirstlane((tile * kWavesPerBlk + (int)(threadIdx.x / kWave)) * NPW);
+    if (node0 >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
     constexpr bool kMatrix = LutMatrixQ<N>::kUsable;
-    float C[kMatrix ? 1 : D::NN], cv[D::H];
-    LutMatrixQ<N> mq;
-    if constexpr (kMatrix) {
-        mq.load(a.C + (size_t)node * D::NN, lane);
-        C[0] = a.C[(size_t)node * D::NN];
-    }
-    else {
-        LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
-        LutEval<N>::pin_constants(C, cv);
-    }
-    void const *rows[N];
+    float C[NPW][kMatrix ? 1 : D::NN], cv[NPW][D::H];
+    LutMatrixQ<N> mq[NPW];
+    void const *rows[NPW][N];
+    float mean[NPW], rstd[NPW], c0[NPW];
+    int node[NPW];
+    bool live[NPW];
 #pragma unroll
-    for (int k = 0; k < N; ++k) {
-        int const in = a.idx[node * N + k];
-        rows[k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
-                                   : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
+    for (int p = 0; p < NPW; ++p) {
+        live[p] = (node0 + p < a.node_size);
+        node[p] = live[p] ? node0 + p : node0;              // a wavefront past the last node repeats its first one and stores nothing
+        if constexpr (kMatrix) {
+            mq[p].load(a.C + (size_t)node[p] * D::NN, lane);
+            C[p][0] = a.C[(size_t)node[p] * D::NN];
+        }
+        else {
+            LutEval<N>::load_table(a.C + (size_t)node[p] * D::NN, C[p]);
+            LutEval<N>::pin_constants(C[p], cv[p]);
+        }
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            int const in = a.idx[node[p] * N + k];
+            rows[p][k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
+                                          : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
+        }
+        mean[p] = 0.0f; rstd[p] = 1.0f;
+        if (FWD_KIND == 1) { mean[p] = a.mean[node[p]]; rstd[p] = a.rstd[node[p]]; }
+        c0[p] = C[p][0];
     }
-    float mean = 0.0f, rstd = 1.0f;
-    if (FWD_KIND == 1) { mean = a.mean[node]; rstd = a.rstd[node]; }
-    float const c0 = C[0];
 
     int const f_begin = ck * a.chunk;
     int const f_end   = min(f_begin + a.chunk, a.frame_size);
-    float s1 = 0.0f, s2 = 0.0f;
+    float s1[NPW], s2[NPW];
+#pragma unroll
+    for (int p = 0; p < NPW; ++p) { s1[p] = 0.0f; s2[p] = 0.0f; }
 
-    constexpr int U = 4;                         // wavefront-steps whose loads are issued together
+    constexpr int U = 4 / NPW;                   // wavefront-steps whose loads are issued together
     int const f_last = a.frame_size - 1;
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
-        uint32_t raw[U][N];
+        uint32_t raw[NPW][U][N];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
-                Gather<N, XMODE>::load_raw(rows, min(fb + u * kWave + lane, f_last), raw[u]);
+#pragma unroll
+                for (int p = 0; p < NPW; ++p) { Gather<N, XMODE>::load_raw(rows[p], min(fb + u * kWave + lane, f_last), raw[p][u]); }
             }
         }
 #pragma unroll
@@ -188,43 +202,49 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
             if (f0 >= f_end) { break; }
             int const  f  = f0 + lane;
             bool const ok = f < f_end;
-            float z[N];
-            Gather<N, XMODE>::centre_all(raw[u], min(f, f_last), a.bias, z);
-            float v;
-            if constexpr (kMatrix) { v = mq.forward(z); }
-            else                   { v = LutEval<N>::forward(C, cv, z); }
+#pragma unroll
+            for (int p = 0; p < NPW; ++p) {
+                float z[N];
+                Gather<N, XMODE>::centre_all(raw[p][u], min(f, f_last), a.bias, z);
+                float v;
+                if constexpr (kMatrix) { v = mq[p].forward(z); }
+                else                   { v = LutEval<N>::forward(C[p], cv[p], z); }
 
-            if (FWD_KIND == 2) {
-                float const d = ok ? (v - c0) : 0.0f;
-                s1 += d;
-                s2 = __builtin_fmaf(d, d, s2);
-                continue;
-            }
-            if (FWD_KIND == 1) {
-                v = (v - mean) * rstd;
-                v = v * a.gamma + a.beta;
-            }
-            if (YMODE == kYBit) {
-                uint64_t const m = __ballot(ok && (v > 0.5f));
-                uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
-                if (lane == 0)                          { yr[0] = (uint32_t)m; }
-                if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
-            }
-            else {
-                if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
-                else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
-                if (ok) { __builtin_nontemporal_store(v, reinterpret_cast<float *>(a.y) + (size_t)node * a.y_stride + f); }
+                if (FWD_KIND == 2) {
+                    float const d = ok ? (v - c0[p]) : 0.0f;
+                    s1[p] += d;
+                    s2[p] = __builtin_fmaf(d, d, s2[p]);
+                    continue;
+                }
+                if (FWD_KIND == 1) {
+                    v = (v - mean[p]) * rstd[p];
+                    v = v * a.gamma + a.beta;
+                }
+                if (!live[p]) { continue; }
+                if (YMODE == kYBit) {
+                    uint64_t const m = __ballot(ok && (v > 0.5f));
+                    uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node[p] * a.y_stride + (f0 >> 5);
+                    if (lane == 0)                          { yr[0] = (uint32_t)m; }
+                    if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
+                }
+                else {
+                    if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+                    else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+                    if (ok) { __builtin_nontemporal_store(v, reinterpret_cast<float *>(a.y) + (size_t)node[p] * a.y_stride + f); }
+                }
             }
         }
     }
 
     if (FWD_KIND == 2) {
-        s1 = wave_sum(s1);
-        s2 = wave_sum(s2);
-        if (lane == 0) {
-            float *p = a.stat_partial + ((size_t)ck * a.node_size + node) * 2;
-            p[0] = s1;
-            p[1] = s2;
+#pragma unroll
+        for (int p = 0; p < NPW; ++p) {
+            float const t1 = wave_sum(s1[p]), t2 = wave_sum(s2[p]);
+            if (lane == 0 && live[p]) {
+                float *q = a.stat_partial + ((size_t)ck * a.node_size + node[p]) * 2;
+                q[0] = t1;
+                q[1] = t2;
+            }
         }
     }
 }
