@@ -52,9 +52,30 @@ def cpu_baseline(I, O, frames, threads, reps=9):
     dy = synth.normal_frames(rng, O, frames, frames)
     secs, kind = oracle.time_stochastic_lut6(x, dy, idx, W, reps)
     med = float(np.median(secs))
-    return {"value": O * frames / med / 1e9, "unit": "G node-evals/s", "cores": threads, "kind": kind,
-            "sample": "StochasticLut6 fwd+bwd (AVX2+OpenMP host path), %d->%d nodes, %d frames, 1 warm-up + median of %d"
-                      % (I, O, frames, reps)}
+    out = {"value": O * frames / med / 1e9, "unit": "G node-evals/s", "cores": threads, "kind": kind,
+           "sample": "StochasticLut6 fwd+bwd (AVX2+OpenMP host path), %d->%d nodes, %d frames, 1 warm-up + median of %d"
+                     % (I, O, frames, reps)}
+    # the same code on one thread, on an eighth of the frames (the OpenMP thread count is switched through the runtime the
+    # libraries share; the environment variable was read when it was loaded)
+    try:
+        import ctypes
+        gomp = ctypes.CDLL("libgomp.so.1")
+        gomp.omp_set_num_threads(1)
+        f1 = max(64, frames // 8)
+        secs1, _ = oracle.time_stochastic_lut6(np.ascontiguousarray(x[:, :f1]), np.ascontiguousarray(dy[:, :f1]), idx, W, 3)
+        gomp.omp_set_num_threads(threads)
+        out["value_1_thread"] = O * f1 / float(np.median(secs1)) / 1e9
+        out["sample_1_thread"] = "%d frames, 1 warm-up + median of 3" % f1
+    except OSError:
+        pass
+    try:
+        with open("/proc/cpuinfo") as f:
+            models = [l.split(":", 1)[1].strip() for l in f if l.startswith("model name")]
+        out["cpu_model"] = models[0] if models else None
+        out["host_logical_cpus"] = len(models)
+    except OSError:
+        pass
+    return out
 
 
 def bench_adam(args, lib):

@@ -140,3 +140,22 @@ def test_against_compiled_reference():
     yr, dxr = oracle.ref_stochastic_maxpool2x2(x, 3, 7, 5, 6, dy=dy)
     assert np.array_equal(oracle.stochastic_maxpool2x2_forward(x, 3, 7, 5, 6), yr)
     assert np.array_equal(oracle.stochastic_maxpool2x2_backward(x, dy, 3, 7, 5, 6), dxr)
+
+
+def test_col2im_known_answers_of_the_reference_test():
+    # testConvolutionCol2ImTest (tests/gtest/ConvolutionCol2ImTest.cpp:9-90): 2 channels, 2 frames of 3 x 4 pixels,
+    # value 1000 f + 100 c + 10 y + x at frame (f*3 + y)*4 + x of channel c goes to pixel (c, y, x) of frame f
+    c, h, w, F = 2, 3, 4, 2
+    x = np.zeros((c, F * h * w), F32)
+    for f in range(F):
+        for yy in range(h):
+            for xx in range(w):
+                for cc in range(c):
+                    x[cc, (f * h + yy) * w + xx] = 1000 * f + 100 * cc + 10 * yy + xx
+    y = oracle.col2im_forward(x, c, h, w, F)
+    for f in range(F):
+        for cc in range(c):
+            for yy in range(h):
+                for xx in range(w):
+                    assert y[(cc * h + yy) * w + xx, f] == 1000 * f + 100 * cc + 10 * yy + xx
+    assert np.array_equal(oracle.col2im_backward(y, c, h, w, F), x)
