@@ -234,6 +234,55 @@ def bench_tail(args, lib):
     print(json.dumps(out))
 
 
+def bench_differentiablelut6(args, lib):
+    """DifferentiableLut6 training step (secondary measurement): the LUT fused with per-node batch normalisation in binary
+    mode (the class defaults), forward (statistics pass, normalising pass) and backward (statistics pass, table-gradient
+    pass, input-centric dx) at the shape of the headline workload."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import ops, synth
+    I = O = 4096
+    F = 8192
+    rng = np.random.default_rng(0)
+    idx = torch.from_numpy(synth.wiring(rng, I, O)).cuda()
+    W = torch.from_numpy(synth.lut_tables(rng, O)).cuda()
+    S = synth.frame_stride_fp32(F)
+    x = torch.from_numpy(synth.uniform_frames(rng, I, F, S)).cuda()
+    dy = torch.from_numpy(synth.normal_frames(rng, O, F, S)).cuda()
+    dW = torch.zeros((O, 64), device="cuda")
+    rm = torch.zeros(O, device="cuda"); rv = torch.ones(O, device="cuda")
+    ops.set_dx_mode(0)
+    rev = ops.reverse_table(idx, I)
+
+    def step():
+        ops.vector_clamp_(W)
+        y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv)
+        ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev)
+
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < args.ramp_seconds:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    # every tensor once per pass: forward x, y, tables; backward x, dy, dx, tables, per-node statistics
+    nbytes = 4 * F * (I + O) + 4 * F * (2 * I + O) + 4 * 280 * O + 32 * O
+    out = {"metric": "G node-evals/s DifferentiableLut6 fp32 fwd+bwd with batch-norm, binary mode (8192 frames x 4096 nodes)",
+           "value": O * F / dt / 1e9, "unit": "G node-evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "DifferentiableLut6 training fwd+bwd fp32 (batch_norm, binary), 4096 in x 4096 out x 8192 frames"},
+           "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+    print(json.dumps(out))
+
+
 def bench_binarylut6(args, lib):
     """BinaryLut6 packed inference: 8192 -> 16384 nodes, 262144 frames, 32 frames per word (secondary measurement)."""
     import numpy as np
@@ -309,7 +358,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "adam", "conv", "tail"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "adam", "conv", "tail"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -332,6 +381,8 @@ def main():
         return bench_conv(args, lib)
     if args.workload == "tail":
         return bench_tail(args, lib)
+    if args.workload == "differentiablelut6":
+        return bench_differentiablelut6(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)

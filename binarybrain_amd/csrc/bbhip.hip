@@ -174,6 +174,9 @@ int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, int npw, 
     BBHIP_FWD_CASE(kXClamp,  kYClamp,    2)
     BBHIP_FWD_CASE(kXBinary, kYClamp,    2)
     BBHIP_FWD_CASE(kXBit,    kYClamp,    2)
+    BBHIP_FWD_CASE(kXClamp,  kYClamp,    3)
+    BBHIP_FWD_CASE(kXBinary, kYClamp,    3)
+    BBHIP_FWD_CASE(kXBit,    kYClamp,    3)
 #undef BBHIP_FWD_CASE
     return fail("forward variant (x=%d, y=%d, kind=%d) not built", xmode, ymode, kind);
 }
@@ -192,9 +195,6 @@ int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStre
     BBHIP_BWD_CASE(kXClamp,  0, kDxNone) BBHIP_BWD_CASE(kXClamp,  1, kDxNone)
     BBHIP_BWD_CASE(kXBinary, 0, kDxNone) BBHIP_BWD_CASE(kXBinary, 1, kDxNone)
     BBHIP_BWD_CASE(kXBit,    0, kDxNone) BBHIP_BWD_CASE(kXBit,    1, kDxNone)
-    BBHIP_BWD_CASE(kXClamp,  2, kDxTmp)
-    BBHIP_BWD_CASE(kXBinary, 2, kDxTmp)
-    BBHIP_BWD_CASE(kXBit,    2, kDxTmp)
 #undef BBHIP_BWD_CASE
     return fail("backward variant (x=%d, kind=%d, dx=%d) not built", xmode, kind, dxmode);
 }
@@ -390,7 +390,10 @@ int run_backward(BackwardCall const &c, hipStream_t st)
 
     size_t const c_bytes    = align256((size_t)c.output_node_size * NN * sizeof(float));
     size_t const part_bytes = align256((size_t)slab_total * c.output_node_size * NN * sizeof(float));
-    size_t const stat_bytes = c.bn ? align256((size_t)slab_total * c.output_node_size * 2 * sizeof(float)) : 0;
+    // batch-norm statistics pass: the forward kernel's unit structure (frame chunks, see below)
+    int const stat_chunk       = fwd_chunk_frames();
+    int const stat_chunk_count = ceil_div(c.frame_size, stat_chunk);
+    size_t const stat_bytes = c.bn ? align256((size_t)stat_chunk_count * c.output_node_size * 2 * sizeof(float)) : 0;
     size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;
     size_t const dtab_bytes = align256(term_count * sizeof(int));
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
@@ -423,7 +426,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
 
     BwdArgs a{};
     a.x = c.x; a.dy = c.dy; a.idx = c.idx; a.C = C;
-    a.dw_partial = part; a.stat_partial = stat;
+    a.dw_partial = part;
     a.mean = c.mean; a.rstd = c.rstd; a.dmean = c.dmean_tmp; a.dvar = c.dvar_tmp;
     a.node_size = c.output_node_size; a.frame_size = c.frame_size;
     a.x_stride = c.x_stride; a.dy_stride = c.frame_stride;
@@ -431,15 +434,21 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     a.bias = c.bias; a.gamma = c.gamma; a.beta = c.beta; a.inv_frames = 1.0f / (float)c.frame_size;
 
     if (c.bn) {
-        // phase 0: per-node sums over ALL frames, then dmean / dvar
-        a.f_base = 0; a.f_limit = c.frame_size; a.slab_first = 0;
-        a.slab_count = ceil_div(c.frame_size, slab);
-        a.dx = nullptr; a.dx_stride = 0;
-        a.tt = TermArgs{};
-        if (dispatch_backward<N>(c.xmode, 2, kDxTmp, a, st)) { return 1; }
+        // phase 0: per-node sums over ALL frames, then dmean / dvar.  It only recomputes the LUT output, so it runs in the
+        // forward kernel (kind 3): frame chunks that keep the gathered rows in L2, partial sums from the matrix unit
+        int const npw = fwd_nodes_per_wave();
+        int const stat_tiles = ceil_div(c.output_node_size, kWavesPerBlk * npw);
+        if ((long long)stat_chunk_count * stat_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
+        FwdArgs f{};
+        f.x = c.x; f.idx = c.idx; f.C = C; f.mean = c.mean; f.rstd = c.rstd; f.stat_partial = stat;
+        f.dy = c.dy; f.dy_stride = c.frame_stride;
+        f.node_size = c.output_node_size; f.frame_size = c.frame_size; f.x_stride = c.x_stride;
+        f.chunk = stat_chunk; f.chunk_count = stat_chunk_count; f.tiles = make_tile_divisor(stat_tiles);
+        f.bias = c.bias; f.gamma = c.gamma; f.beta = c.beta;
+        if (dispatch_forward<N>(c.xmode, kYClamp, 3, f, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
         hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, kBlock)), dim3(kBlock), 0, st,
-                           stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, a.slab_count, c.frame_size);
+                           stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, stat_chunk_count, c.frame_size);
         BBHIP_LAUNCH_CHECK();
     }
 

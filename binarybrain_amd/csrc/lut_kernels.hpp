@@ -71,6 +71,7 @@ __device__ __forceinline__ void dw_finalize_block(float const *__restrict__ part
     int const total = node_size * NN;
     float v = 0.0f;
     if (t < total) {
+#pragma unroll 8
         for (int s = 0; s < slab_count; ++s) { v += partial[(size_t)s * total + t]; }
     }
     int const i = t & (NN - 1);
@@ -124,7 +125,9 @@ struct FwdArgs {
     float const *C;             // [O][2^N] centred coefficients
     float const *mean;          // BN: per node (nullptr otherwise)
     float const *rstd;
-    float       *stat_partial;  // STATS: [chunk][O][2] partial sums of (v - C0), (v - C0)^2
+    float       *stat_partial;  // STATS: [chunk][O][2] partial sums of (v - C0), (v - C0)^2;  kind 3: of g, g (v - mean)
+    float const *dy;            // kind 3: [O][dy_stride]
+    int   dy_stride;
     int   node_size, frame_size;
     int   x_stride, y_stride;   // elements per node row (floats or words)
     int   chunk;                // frames per unit, multiple of 64
@@ -133,7 +136,9 @@ struct FwdArgs {
     float bias, gamma, beta;
 };
 
-// FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only
+// FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only,
+//           3 = statistics of the backward pass through batch-norm: per node the sums of g and g (v - mean), where g = dy gated by
+//               the hard-tanh window 0 < t < 1 of the batch-norm output t (reference: DifferentiableLutN.h:1206-1222)
 // NPW: nodes per wavefront.  A wavefront issues the loads of NPW nodes x U steps together (NPW x U = 4); with two nodes the
 // set-up of a wavefront (index and table loads, two memory latencies before the first gather can go out) is shared by twice
 // the work.
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
                                           : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
         }
         mean[p] = 0.0f; rstd[p] = 1.0f;
-        if (FWD_KIND == 1) { mean[p] = a.mean[node[p]]; rstd[p] = a.rstd[node[p]]; }
+        if (FWD_KIND == 1 || FWD_KIND == 3) { mean[p] = a.mean[node[p]]; rstd[p] = a.rstd[node[p]]; }
         c0[p] = C[p][0];
     }
 
@@ -189,11 +194,16 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     int const f_last = a.frame_size - 1;
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
         uint32_t raw[NPW][U][N];
+        float dyv[NPW][U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
 #pragma unroll
-                for (int p = 0; p < NPW; ++p) { Gather<N, XMODE>::load_raw(rows[p], min(fb + u * kWave + lane, f_last), raw[p][u]); }
+                for (int p = 0; p < NPW; ++p) {
+                    int const fs = min(fb + u * kWave + lane, f_last);
+                    Gather<N, XMODE>::load_raw(rows[p], fs, raw[p][u]);
+                    if (FWD_KIND == 3) { dyv[p][u] = a.dy[(size_t)node[p] * a.dy_stride + fs]; }
+                }
             }
         }
 #pragma unroll
@@ -216,6 +226,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
                     s2[p] = __builtin_fmaf(d, d, s2[p]);
                     continue;
                 }
+                if (FWD_KIND == 3) {
+                    float const t = ((v - mean[p]) * rstd[p]) * a.gamma + a.beta;
+                    float d = ok ? dyv[p][u] : 0.0f;
+                    if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
+                    s1[p] += d;
+                    s2[p] = __builtin_fmaf(d, v - mean[p], s2[p]);
+                    continue;
+                }
                 if (FWD_KIND == 1) {
                     v = (v - mean[p]) * rstd[p];
                     v = v * a.gamma + a.beta;
@@ -236,7 +254,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         }
     }
 
-    if (FWD_KIND == 2) {
+    if (FWD_KIND == 2 || FWD_KIND == 3) {
 #pragma unroll
         for (int p = 0; p < NPW; ++p) {
             float const t1 = wave_sum(s1[p]), t2 = wave_sum(s2[p]);
@@ -258,6 +276,7 @@ __global__ __launch_bounds__(kBlock) void bn_forward_finalize_kernel(float const
     int const node = blockIdx.x * kBlock + threadIdx.x;
     if (node >= node_size) { return; }
     float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll 8
     for (int c = 0; c < chunk_count; ++c) {
         float const *p = stat_partial + ((size_t)c * node_size + node) * 2;
         s1 += p[0];
@@ -364,7 +383,6 @@ struct BwdArgs {
     float const *rstd;
     float const *dmean;         // BN phase 1
     float const *dvar;
-    float       *stat_partial;  // BN phase 0: [slab][O][2]
     int   node_size, frame_size;
     int   x_stride, dy_stride, dx_stride;
     int   f_base, f_limit;      // frame range handled by this launch
@@ -378,7 +396,7 @@ struct BwdArgs {
 
 enum DxMode : int { kDxAtomic = 0, kDxTmp = 1, kDxNone = 2 };
 
-// BWD_KIND: 0 = plain LUT backward, 1 = backward through batch-norm (phase 1), 2 = batch-norm statistics (phase 0)
+// BWD_KIND: 0 = plain LUT backward, 1 = backward through batch-norm (its statistics pass is kind 3 of the forward kernel)
 // DXMODE  : how (whether) the per-connection input gradients leave the kernel
 template <int N, int XMODE, int BWD_KIND, int DXMODE>
 __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
@@ -390,7 +408,7 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     // end of this launch, where they fill the device while the last slabs drain, instead of taking a launch of their own.
     int const bid = blockIdx.x;
     int const B   = a.slab_count * a.tiles.count;
-    if (DXMODE == kDxNone && BWD_KIND != 2) {
+    if (DXMODE == kDxNone) {
         if (bid >= B) { term_table_block<N>(a.tt, bid - B); return; }
     }
     int const lid  = xcd_remap(bid, B);
@@ -403,6 +421,9 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 
     // the table itself enters only the batch-norm kinds (the LUT output is recomputed) and the per-connection gradients
     constexpr bool kNeedTable = (BWD_KIND != 0) || (DXMODE != kDxNone);
+    // (the partial sums stay on the vector ALU here: the matrix unit's operand registers would cost this kernel a wavefront of
+    // occupancy, which measured slower; the batch-norm statistics pass, which only recomputes the LUT output, runs in the
+    // forward kernel instead)
     float C[D::NN], cv[D::H];
     if (kNeedTable) {
         LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
@@ -430,7 +451,6 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     float acc[D::NN];
 #pragma unroll
     for (int i = 0; i < D::NN; ++i) { acc[i] = 0.0f; }
-    float s0 = 0.0f, s1 = 0.0f;
 
     constexpr int U = 2;                         // wavefront-steps whose loads are issued together
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
@@ -467,11 +487,6 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
                 float const v = LutEval<N>::combine(h, q);
                 float const t = ((v - mean) * rstd) * a.gamma + a.beta;
                 if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
-                if (BWD_KIND == 2) {
-                    s0 += d;
-                    s1 = __builtin_fmaf(d, v - mean, s1);
-                    continue;
-                }
                 // dL/d(LUT output) (reference: DifferentiableLutN.h:1248-1250)
                 d = ok ? (__builtin_fmaf(d, grs, dmean) + v * dvarf) : 0.0f;
                 if (DXMODE == kDxNone && ok) { a.dx[(size_t)node * a.dx_stride + f] = d; }
@@ -520,17 +535,6 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
                 }
             }
         }
-    }
-
-    if (BWD_KIND == 2) {
-        s0 = wave_sum(s0);
-        s1 = wave_sum(s1);
-        if (lane == 0) {
-            float *pp = a.stat_partial + ((size_t)(a.slab_first + sl) * a.node_size + node) * 2;
-            pp[0] = s0;
-            pp[1] = s1;
-        }
-        return;
     }
 
     // frame reduction of the 2^N per-lane accumulators through LDS, 16 at a time:
@@ -751,6 +755,7 @@ __global__ __launch_bounds__(kBlock) void bn_backward_finalize_kernel(float cons
     int const node = blockIdx.x * kBlock + threadIdx.x;
     if (node >= node_size) { return; }
     float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll 8
     for (int s = 0; s < slab_count; ++s) {
         float const *p = stat_partial + ((size_t)s * node_size + node) * 2;
         s0 += p[0];
