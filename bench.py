@@ -253,11 +253,18 @@ def bench_differentiablelut6(args, lib):
     rm = torch.zeros(O, device="cuda"); rv = torch.ones(O, device="cuda")
     ops.set_dx_mode(0)
     rev = ops.reverse_table(idx, I)
+    bits = args.workload.endswith("_bit")
+    if bits:
+        xb = torch.from_numpy(synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))).cuda()
 
     def step():
         ops.vector_clamp_(W)
-        y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv)
-        ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev)
+        if bits:
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv)
+            ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev)
+        else:
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv)
+            ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev)
 
     t_ramp = time.perf_counter()
     while time.perf_counter() - t_ramp < args.ramp_seconds:
@@ -274,10 +281,13 @@ def bench_differentiablelut6(args, lib):
     dt = (time.perf_counter() - t0) / args.steps
     # every tensor once per pass: forward x, y, tables; backward x, dy, dx, tables, per-node statistics
     nbytes = 4 * F * (I + O) + 4 * F * (2 * I + O) + 4 * 280 * O + 32 * O
-    out = {"metric": "G node-evals/s DifferentiableLut6 fp32 fwd+bwd with batch-norm, binary mode (8192 frames x 4096 nodes)",
+    if bits:      # packed x and y (1 bit per element), fp32 dy and dx
+        nbytes = (F // 8) * (I + O) + (F // 8) * I + 4 * F * (I + O) + 4 * 280 * O + 32 * O
+    out = {"metric": "G node-evals/s DifferentiableLut6 %s fwd+bwd with batch-norm, binary mode (8192 frames x 4096 nodes)" % ("packed-bit" if bits else "fp32"),
            "value": O * F / dt / 1e9, "unit": "G node-evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "DifferentiableLut6 training fwd+bwd fp32 (batch_norm, binary), 4096 in x 4096 out x 8192 frames"},
+           "config": {"workload": "DifferentiableLut6 training fwd+bwd %s (batch_norm, binary), 4096 in x 4096 out x 8192 frames"
+                                  % ("packed-bit activations, fp32 gradients" if bits else "fp32")},
            "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
     print(json.dumps(out))
@@ -358,7 +368,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "adam", "conv", "tail"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "adam", "conv", "tail"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -381,7 +391,7 @@ def main():
         return bench_conv(args, lib)
     if args.workload == "tail":
         return bench_tail(args, lib)
-    if args.workload == "differentiablelut6":
+    if args.workload in ("differentiablelut6", "differentiablelut6_bit"):
         return bench_differentiablelut6(args, lib)
     I = O = 4096
     F = 8192
