@@ -92,7 +92,17 @@ int env_int(char const *name, int def)
 
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); return v >= 2 ? 2 : 1; }
-int fwd_chunk_frames(void) { static int v = env_int("BBHIP_FWD_CHUNK", 256); return ((v + 63) / 64) * 64; }
+// Frames per forward unit.  fp32 rows are gathered through L2, and a 256-frame piece of every input row is what one XCD's L2
+// holds; packed-bit rows are 32 times smaller, so their units are longer and a unit's set-up (wiring, table) weighs less.
+// Longer units are halved while they would leave the launch with fewer than 2048 workgroups.
+int fwd_chunk_frames(int xmode, int frame_size, int tile_count)
+{
+    static int env = env_int("BBHIP_FWD_CHUNK", 0);
+    if (env > 0) { return ((env + 63) / 64) * 64; }
+    int chunk = (xmode == kXBit) ? 1024 : 256;
+    while (chunk > 256 && (long long)((frame_size + chunk - 1) / chunk) * tile_count < 2048) { chunk /= 2; }
+    return chunk;
+}
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  return ((v + 63) / 64) * 64; }       // 0: chosen per call
 int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
 int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 2); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
@@ -259,9 +269,9 @@ int run_forward(ForwardCall const &c, hipStream_t st)
 {
     constexpr int NN = 1 << N;
     int const npw         = fwd_nodes_per_wave();
-    int const chunk       = fwd_chunk_frames();
-    int const chunk_count = ceil_div(c.frame_size, chunk);
     int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
+    int const chunk       = fwd_chunk_frames(c.xmode, c.frame_size, tile_count);
+    int const chunk_count = ceil_div(c.frame_size, chunk);
     if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("forward: grid too large"); }
 
     size_t const c_bytes    = align256((size_t)c.node_size * NN * sizeof(float));
@@ -391,7 +401,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     size_t const c_bytes    = align256((size_t)c.output_node_size * NN * sizeof(float));
     size_t const part_bytes = align256((size_t)slab_total * c.output_node_size * NN * sizeof(float));
     // batch-norm statistics pass: the forward kernel's unit structure (frame chunks, see below)
-    int const stat_chunk       = fwd_chunk_frames();
+    int const stat_chunk       = fwd_chunk_frames(c.xmode, c.frame_size, ceil_div(c.output_node_size, kWavesPerBlk * fwd_nodes_per_wave()));
     int const stat_chunk_count = ceil_div(c.frame_size, stat_chunk);
     size_t const stat_bytes = c.bn ? align256((size_t)stat_chunk_count * c.output_node_size * 2 * sizeof(float)) : 0;
     size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;

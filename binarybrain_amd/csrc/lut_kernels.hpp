@@ -95,26 +95,57 @@ __global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__rest
 // ------------------------------------------------------------------------------------------------
 template <int N, int XMODE>
 struct Gather {
-    // rows[k]: wave-uniform pointer to the input row of connection k (float rows, or packed words for kXBit).
-    // fs is a frame index already clamped into the buffer, so every lane loads unconditionally and the N loads
-    // are issued back to back.
+    using Raw = uint32_t;
+
+    // rows[k]: wave-uniform pointer to the input row of connection k.  f0 is the wavefront step's first frame; the
+    // frame index of a lane is clamped into the buffer, so every lane loads unconditionally and the N loads are
+    // issued back to back.
     // The element offset is an unsigned 32-bit byte offset from the wave-uniform row pointer, which lets the load use the
     // scalar-base + vector-offset addressing form (no per-load 64-bit vector add).
-    __device__ __forceinline__ static void load_raw(void const *(&rows)[N], int fs, uint32_t (&raw)[N])
+    __device__ __forceinline__ static void load_raw(void const *(&rows)[N], int f0, int lane, int f_last, Raw (&raw)[N])
     {
-        uint32_t const off = ((XMODE == kXBit) ? (uint32_t)(fs >> 5) : (uint32_t)fs) * 4u;
+        uint32_t const off = (uint32_t)min(f0 + lane, f_last) * 4u;
 #pragma unroll
         for (int k = 0; k < N; ++k) {
             raw[k] = *reinterpret_cast<uint32_t const *>(reinterpret_cast<char const *>(rows[k]) + off);
         }
     }
 
-    __device__ __forceinline__ static void centre_all(uint32_t const (&raw)[N], int fs, float bias, float (&z)[N])
+    __device__ __forceinline__ static void centre_all(Raw const (&raw)[N], float bias, float (&z)[N])
     {
 #pragma unroll
+        for (int k = 0; k < N; ++k) { z[k] = centre<XMODE>(__uint_as_float(raw[k]), bias); }
+    }
+};
+
+// Packed bits: the 64 frames of a wavefront step (f0 a multiple of 64) are the two words f0 / 32 and f0 / 32 + 1 of the
+// row, the same for every lane, and bit l of the pair belongs to lane l.  They are fetched with scalar loads through the
+// constant address space (the input is not written by the kernels that gather) and used directly as the lane mask of a
+// select between -bias and +bias: no vector memory instruction and one vector ALU instruction per input.
+// Where the second word would hold no frame of the buffer the first is loaded in its place: lanes beyond the last frame
+// get bits of the row's padding or of other frames, and their results are discarded by the callers.
+template <int N>
+struct Gather<N, kXBit> {
+    using Raw = uint64_t;
+    typedef __attribute__((address_space(4))) uint32_t const const_u32;
+
+    __device__ __forceinline__ static void load_raw(void const *(&rows)[N], int f0, int, int f_last, Raw (&raw)[N])
+    {
+        int const  w0     = min(f0, f_last) >> 5;
+        bool const second = ((w0 + 1) << 5) <= f_last;
+#pragma unroll
         for (int k = 0; k < N; ++k) {
-            z[k] = (XMODE == kXBit) ? centre_bit(raw[k], fs & 31, bias) : centre<XMODE>(__uint_as_float(raw[k]), bias);
+            const_u32 *p = (const_u32 *)rows[k] + w0;
+            uint32_t const lo = p[0];
+            uint32_t const hi = p[second ? 1 : 0];          // always a word of the row
+            raw[k] = (uint64_t)lo | ((uint64_t)hi << 32);
         }
+    }
+
+    __device__ __forceinline__ static void centre_all(Raw const (&raw)[N], float bias, float (&z)[N])
+    {
+#pragma unroll
+        for (int k = 0; k < N; ++k) { z[k] = __builtin_amdgcn_inverse_ballot_w64(raw[k]) ? bias : -bias; }
     }
 };
 
@@ -190,10 +221,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
     for (int p = 0; p < NPW; ++p) { s1[p] = 0.0f; s2[p] = 0.0f; }
 
-    constexpr int U = 4 / NPW;                   // wavefront-steps whose loads are issued together
+    // wavefront-steps whose loads are issued together; packed-bit inputs arrive as scalar lane masks, two registers each
+    constexpr int U = (XMODE == kXBit) ? 2 / NPW : 4 / NPW;
     int const f_last = a.frame_size - 1;
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
-        uint32_t raw[NPW][U][N];
+        typename Gather<N, XMODE>::Raw raw[NPW][U][N];
         float dyv[NPW][U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -201,7 +233,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
                 for (int p = 0; p < NPW; ++p) {
                     int const fs = min(fb + u * kWave + lane, f_last);
-                    Gather<N, XMODE>::load_raw(rows[p], fs, raw[p][u]);
+                    Gather<N, XMODE>::load_raw(rows[p], fb + u * kWave, lane, f_last, raw[p][u]);
                     if (FWD_KIND == 3) { dyv[p][u] = a.dy[(size_t)node[p] * a.dy_stride + fs]; }
                 }
             }
@@ -215,7 +247,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
             for (int p = 0; p < NPW; ++p) {
                 float z[N];
-                Gather<N, XMODE>::centre_all(raw[p][u], min(f, f_last), a.bias, z);
+                Gather<N, XMODE>::centre_all(raw[p][u], a.bias, z);
                 float v;
                 if constexpr (kMatrix) { v = mq[p].forward(z); }
                 else                   { v = LutEval<N>::forward(C[p], cv[p], z); }
@@ -453,13 +485,15 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     for (int i = 0; i < D::NN; ++i) { acc[i] = 0.0f; }
 
     constexpr int U = 2;                         // wavefront-steps whose loads are issued together
+    // packed-bit inputs are scalar lane masks: where the table already fills the scalar registers they are fetched step by step
+    constexpr bool kLateGather = (XMODE == kXBit) && kNeedTable;
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
-        uint32_t raw[U][N];
+        typename Gather<N, XMODE>::Raw raw[U][N];
         float dyv[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             int const fs = min(fb + u * kWave + lane, f_last);
-            Gather<N, XMODE>::load_raw(rows, fs, raw[u]);
+            if (!kLateGather) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
             dyv[u] = *reinterpret_cast<float const *>(reinterpret_cast<char const *>(dyr) + (uint32_t)fs * 4u);
         }
 #pragma unroll
@@ -469,7 +503,8 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
             int const  f  = f0 + lane;
             bool const ok = f < f_end;
             float z[N];
-            Gather<N, XMODE>::centre_all(raw[u], min(f, f_last), a.bias, z);
+            if (kLateGather) { Gather<N, XMODE>::load_raw(rows, f0, lane, f_last, raw[u]); }
+            Gather<N, XMODE>::centre_all(raw[u], a.bias, z);
             float d = ok ? dyv[u] : 0.0f;
 
             float zl[D::NL], zh[D::NH];
