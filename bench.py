@@ -293,6 +293,111 @@ def bench_differentiablelut6(args, lib):
     print(json.dumps(out))
 
 
+def bench_mnist_step(args, lib):
+    """One training step of the MNIST-like LUT classifier (secondary measurement; launch- and latency-bound): DifferentiableLut6
+    784 -> 6144 -> 1024 -> 70 with batch-norm in binary mode, AverageLut 7 -> 1 (10 classes), softmax cross entropy,
+    accuracy, Adam, 1024 frames.  Timed twice: every entry point called from the host per step, and the forward + backward
+    part of the step replayed as one HIP graph (captured from the same calls on a torch capture stream; Adam stays a
+    launch of its own because its bias-corrected rate is a host scalar that changes per step)."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import ops, synth
+    sizes = [784, 6144, 1024, 70]
+    CLASSES, N_AVG, F = 10, 7, 1024
+    rng = np.random.default_rng(0)
+    S = synth.frame_stride_fp32(F)
+    layers = []
+    for I, O in zip(sizes[:-1], sizes[1:]):
+        idx = torch.from_numpy(synth.wiring(rng, I, O)).cuda()
+        W = torch.from_numpy((0.5 + 0.01 * rng.standard_normal((O, 64))).astype(np.float32)).cuda()
+        layers.append(dict(I=I, O=O, idx=idx, W=W, dW=torch.zeros_like(W), rm=torch.zeros(O, device="cuda"), rv=torch.ones(O, device="cuda"),
+                           rev=ops.reverse_table(idx, I)))
+    idx_avg = torch.arange(sizes[-1], dtype=torch.int32, device="cuda").reshape(CLASSES, N_AVG).contiguous()
+    x = torch.from_numpy(synth.uniform_frames(rng, sizes[0], F, S)).cuda()
+    t = torch.zeros((CLASSES, S), device="cuda")
+    label = torch.from_numpy(rng.integers(0, CLASSES, F)).cuda()
+    t[label, torch.arange(F, device="cuda")] = 1.0
+    adam = ops.AdamState([l["W"] for l in layers], [l["dW"] for l in layers], learning_rate=0.001)
+    ops.set_dx_mode(0)
+    keep = {}
+
+    def forward_backward():
+        a = x
+        acts = []
+        for l in layers:
+            ops.vector_clamp_(l["W"])
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"])
+            acts.append((a, mean, rstd)); a = y
+        out = ops.average_lut_forward(a, idx_avg, F, False, False)
+        dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
+        acc, cat = ops.metrics_categorical_accuracy(out, t, CLASSES, 1, F)
+        dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
+        for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
+            l["dW"].zero_()
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"])
+        keep["loss_buf"], keep["acc"] = loss_buf, acc
+
+    def timed(fn):
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < args.ramp_seconds:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    def eager_step():
+        forward_backward(); adam.step()
+
+    dt_eager = timed(eager_step)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        forward_backward()
+
+    def graph_step():
+        graph.replay(); adam.step()
+
+    dt_graph = timed(graph_step)
+    loss = -float(keep["loss_buf"].sum().item()) / F
+    node_evals = sum(sizes[1:]) * F
+    # every activation, gradient and table once per pass over the three LUT layers
+    nbytes = sum(4 * F * (3 * l["I"] + 2 * l["O"]) + 4 * 280 * l["O"] * 2 for l in layers)
+    dt = min(dt_eager, dt_graph)
+    out = {"metric": "training steps/s, MNIST-like DifferentiableLut6 classifier 784-6144-1024-70, 1024 frames", "value": 1.0 / dt,
+           "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "DifferentiableLut6 784->6144->1024->70 (batch_norm, binary) + AverageLut 7->1 + softmax CE + accuracy + Adam, 1024 frames",
+                      "ms_per_step_host_launched": dt_eager * 1e3, "ms_per_step_graph_replay": dt_graph * 1e3,
+                      "G_node_evals_per_s": node_evals / dt / 1e9, "loss_after_run": loss},
+           "roofline": {"bound": "hbm", "kernel": "whole step (launch-bound)", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+    if not args.no_cpu:
+        import oracle
+        xs = x.cpu().numpy(); ts = t.cpu().numpy()
+        Ws = [l["W"].cpu().numpy() for l in layers]; idxs = [l["idx"].cpu().numpy() for l in layers]
+        t0 = time.perf_counter()
+        a = xs; acts = []
+        for l, W, idx in zip(layers, Ws, idxs):
+            y, mean, rstd, _, _ = oracle.differentiable_lut_forward_training(6, a, idx, W, F, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))
+            acts.append((a, mean, rstd)); a = y
+        o = oracle.average_lut_forward(a, idx_avg.cpu().numpy(), F, False, False)
+        dy, _, _ = oracle.loss_softmax_cross_entropy(o, ts, CLASSES, 1, F)
+        dy = oracle.average_lut_backward(dy, idx_avg.cpu().numpy(), sizes[-1], F)
+        for l, W, idx, (a_in, mean, rstd) in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(acts)):
+            dy, _ = oracle.differentiable_lut_backward(6, a_in, dy, idx, W, F, mean, rstd)
+        cpu_dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": 1.0 / cpu_dt, "unit": "steps/s", "cores": 1, "kind": "port",
+                               "sample": "one forward + backward of the same network through the C restatement of the reference's generic "
+                                         "DifferentiableLut path (its batch-norm backward is single-threaded in the reference too), Adam not included"}
+    print(json.dumps(out))
+
+
 def bench_binarylut6(args, lib):
     """BinaryLut6 packed inference: 8192 -> 16384 nodes, 262144 frames, 32 frames per word (secondary measurement)."""
     import numpy as np
@@ -368,7 +473,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "adam", "conv", "tail"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "adam", "conv", "tail"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -393,6 +498,8 @@ def main():
         return bench_tail(args, lib)
     if args.workload in ("differentiablelut6", "differentiablelut6_bit"):
         return bench_differentiablelut6(args, lib)
+    if args.workload == "mnist_step":
+        return bench_mnist_step(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)
