@@ -293,6 +293,100 @@ def bench_differentiablelut6(args, lib):
     print(json.dumps(out))
 
 
+def conv_block_layers(rng, synth, ops, torch, np):
+    """wiring and tables of the two per-pixel LUT layers of the conv block (27 -> 216 -> 36)"""
+    layers = []
+    for I, O in ((27, 216), (216, 36)):
+        idx = torch.from_numpy(synth.wiring(rng, I, O)).cuda()
+        W = torch.from_numpy((0.5 + 0.1 * rng.standard_normal((O, 64))).astype(np.float32)).cuda()
+        layers.append(dict(I=I, O=O, idx=idx, W=W, dW=torch.zeros_like(W), rm=torch.zeros(O, device="cuda"), rv=torch.ones(O, device="cuda"),
+                           rev=ops.reverse_table(idx, I)))
+    return layers
+
+
+def bench_conv_block(args, lib):
+    """Forward + backward of the convolutional LUT block (secondary measurement): 256 images of 3 x 32 x 32, Im2Col 3 x 3 valid
+    (27 taps, 230400 window frames), DifferentiableLut6 27 -> 216 -> 36 per pixel with batch-norm in binary mode, Col2Im to
+    36 x 30 x 30, StochasticMaxPooling2x2 to 36 x 15 x 15, and the backward pass of all of it down to the image gradient."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import ops, synth
+    F, C, H, W_, FH, FW, CO = 256, 3, 32, 32, 3, 3, 36
+    OH, OW = H - FH + 1, W_ - FW + 1
+    FW_FRAMES = F * OH * OW
+    rng = np.random.default_rng(0)
+    layers = conv_block_layers(rng, synth, ops, torch, np)
+    g = torch.Generator(device="cuda"); g.manual_seed(0)
+    img = torch.rand((C * H * W_, synth.frame_stride_fp32(F)), device="cuda", generator=g)
+    dpooled = torch.randn((CO * (OH // 2) * (OW // 2), synth.frame_stride_fp32(F)), device="cuda", generator=g)
+    ops.set_dx_mode(0)
+
+    def step():
+        cols = ops.im2col_forward(img, C, H, W_, F, FH, FW)
+        a = cols; acts = []
+        for l in layers:
+            ops.vector_clamp_(l["W"])
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"])
+            acts.append((a, mean, rstd)); a = y
+        maps = ops.col2im_forward(a, CO, OH, OW, F)
+        pooled = ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F)
+        dmaps = ops.stochastic_maxpool2x2_backward(maps, dpooled, CO, OH, OW, F)
+        dy = ops.col2im_backward(dmaps, CO, OH, OW, F)
+        for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
+            l["dW"].zero_()
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"])
+        return ops.im2col_backward(dy, C, H, W_, F, FH, FW), pooled
+
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < args.ramp_seconds:
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    node_evals = sum(l["O"] for l in layers) * FW_FRAMES
+    e = 4
+    # every activation and gradient once per pass: image, window columns, both LUT layers, maps, pooled maps
+    nbytes = (e * F * (C * H * W_ + 27 * OH * OW) * 2 + sum(e * FW_FRAMES * (3 * l["I"] + 2 * l["O"]) for l in layers)
+              + 2 * e * F * CO * OH * OW * 2 + e * F * CO * (OH * OW * 3 + 2 * (OH // 2) * (OW // 2)))
+    out = {"metric": "G node-evals/s, convolutional DifferentiableLut6 block 27->216->36 per pixel, 256 images of 3x32x32, fwd+bwd",
+           "value": node_evals / dt / 1e9, "unit": "G node-evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "Im2Col 3x3 -> DifferentiableLut6 27->216->36 (batch_norm, binary) -> Col2Im 36x30x30 -> StochasticMaxPooling2x2, "
+                                  "256 images of 3x32x32, forward + backward", "images_per_s": F / dt},
+           "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+    if not args.no_cpu:
+        import oracle
+        Fs = 4                                                # images in the CPU sample
+        S = synth.frame_stride_fp32(Fs); FWs = Fs * OH * OW
+        xs = np.zeros((C * H * W_, S), np.float32); xs[:, :Fs] = img[:, :Fs].cpu().numpy()
+        Ws = [l["W"].cpu().numpy() for l in layers]; idxs = [l["idx"].cpu().numpy() for l in layers]
+        dps = np.ascontiguousarray(dpooled[:, :Fs].cpu().numpy())          # the oracle's conv functions work on dense rows
+        t0 = time.perf_counter()
+        a = oracle.im2col_forward(xs, C, H, W_, Fs, FH, FW); acts = []
+        for l, Wt, idx in zip(layers, Ws, idxs):
+            y, mean, rstd, _, _ = oracle.differentiable_lut_forward_training(6, a, idx, Wt, FWs, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))
+            acts.append((a, mean, rstd)); a = y
+        maps = oracle.col2im_forward(a, CO, OH, OW, Fs)
+        oracle.stochastic_maxpool2x2_forward(maps, CO, OH, OW, Fs)
+        dy = oracle.col2im_backward(oracle.stochastic_maxpool2x2_backward(maps, dps, CO, OH, OW, Fs), CO, OH, OW, Fs)
+        for l, Wt, idx, (a_in, mean, rstd) in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(acts)):
+            dy, _ = oracle.differentiable_lut_backward(6, a_in, dy, idx, Wt, FWs, mean, rstd)
+        oracle.im2col_backward(dy, C, H, W_, Fs, FH, FW)
+        cpu_dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": sum(l["O"] for l in layers) * FWs / cpu_dt / 1e9, "unit": "G node-evals/s", "cores": 1, "kind": "port",
+                               "sample": "the same block on %d images through the C restatement of the reference's host path (generic DifferentiableLut "
+                                         "algorithm, whose batch-norm backward is single-threaded in the reference too)" % Fs}
+    print(json.dumps(out))
+
+
 def bench_mnist_step(args, lib):
     """One training step of the MNIST-like LUT classifier (secondary measurement; launch- and latency-bound): DifferentiableLut6
     784 -> 6144 -> 1024 -> 70 with batch-norm in binary mode, AverageLut 7 -> 1 (10 classes), softmax cross entropy,
@@ -473,7 +567,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "adam", "conv", "tail"],
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
     args = ap.parse_args()
@@ -500,6 +594,8 @@ def main():
         return bench_differentiablelut6(args, lib)
     if args.workload == "mnist_step":
         return bench_mnist_step(args, lib)
+    if args.workload == "conv_block":
+        return bench_conv_block(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)

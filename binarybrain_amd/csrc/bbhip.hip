@@ -264,6 +264,10 @@ int check_forward(ForwardCall const &c)
     return 0;
 }
 
+// nodes per workgroup of the batch-norm finalize kernels: the more units there are to add per node, the more of the
+// workgroup's threads share one node
+int stat_nodes_per_block(int unit_count) { return unit_count >= 512 ? 4 : unit_count >= 64 ? 16 : 64; }
+
 template <int N>
 int run_forward(ForwardCall const &c, hipStream_t st)
 {
@@ -298,9 +302,10 @@ int run_forward(ForwardCall const &c, hipStream_t st)
         a.stat_partial = stat;
         if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
-        hipLaunchKernelGGL(bn_forward_finalize_kernel, dim3(ceil_div(c.node_size, kBlock)), dim3(kBlock), 0, st,
+        int const npb = stat_nodes_per_block(chunk_count);
+        hipLaunchKernelGGL(bn_forward_finalize_kernel, dim3(ceil_div(c.node_size, npb)), dim3(kBlock), 0, st,
                            stat, C, NN, c.mean, c.rstd, c.running_mean, c.running_var, c.momentum,
-                           c.node_size, chunk_count, c.frame_size);
+                           c.node_size, chunk_count, c.frame_size, npb);
         BBHIP_LAUNCH_CHECK();
         a.mean = c.mean; a.rstd = c.rstd;
         kind = 1;
@@ -457,8 +462,9 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         f.bias = c.bias; f.gamma = c.gamma; f.beta = c.beta;
         if (dispatch_forward<N>(c.xmode, kYClamp, 3, f, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
-        hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, kBlock)), dim3(kBlock), 0, st,
-                           stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, stat_chunk_count, c.frame_size);
+        int const npb = stat_nodes_per_block(stat_chunk_count);
+        hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, npb)), dim3(kBlock), 0, st,
+                           stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, stat_chunk_count, c.frame_size, npb);
         BBHIP_LAUNCH_CHECK();
     }
 

@@ -299,21 +299,48 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     }
 }
 
+// Sum of the per-unit partial sums [count][node_size][2] of one node.  A workgroup owns nodes_per_block consecutive nodes
+// (a power of two up to kBlock) and splits the units over its kBlock / nodes_per_block thread groups: group g adds units
+// g, g + G, ... in ascending order and the groups are added in ascending order through LDS — a fixed order, so the result
+// does not depend on the launch.  Consecutive threads of a group read consecutive nodes (8 bytes each).  Returns true in
+// the one thread per node that holds the sums.
+__device__ __forceinline__ bool sum_stat_partials(float const *__restrict__ stat_partial, int node_size, int count,
+                                                  int nodes_per_block, int &node, float &s1, float &s2)
+{
+    __shared__ float2 red[kBlock];
+    int const n_local = threadIdx.x % nodes_per_block, g = threadIdx.x / nodes_per_block, groups = kBlock / nodes_per_block;
+    node = blockIdx.x * nodes_per_block + n_local;
+    float a = 0.0f, b = 0.0f;
+    if (node < node_size) {
+#pragma unroll 4
+        for (int c = g; c < count; c += groups) {
+            float2 const v = *reinterpret_cast<float2 const *>(stat_partial + ((size_t)c * node_size + node) * 2);
+            a += v.x;
+            b += v.y;
+        }
+    }
+    red[threadIdx.x] = make_float2(a, b);                  // index = g * nodes_per_block + n_local
+    __syncthreads();
+    if (g != 0 || node >= node_size) { return false; }
+    s1 = 0.0f; s2 = 0.0f;
+    for (int k = 0; k < groups; ++k) {
+        float2 const v = red[k * nodes_per_block + n_local];
+        s1 += v.x;
+        s2 += v.y;
+    }
+    return true;
+}
+
 // per node: mean, var (>= 1e-5), rstd, running statistics (reference: include/bb/DifferentiableLutN.h:804-812)
 __global__ __launch_bounds__(kBlock) void bn_forward_finalize_kernel(float const *__restrict__ stat_partial, float const *__restrict__ C, int nn,
                                                                     float *__restrict__ mean, float *__restrict__ rstd,
                                                                     float *__restrict__ running_mean, float *__restrict__ running_var,
-                                                                    float momentum, int node_size, int chunk_count, int frame_size)
+                                                                    float momentum, int node_size, int chunk_count, int frame_size,
+                                                                    int nodes_per_block)
 {
-    int const node = blockIdx.x * kBlock + threadIdx.x;
-    if (node >= node_size) { return; }
-    float s1 = 0.0f, s2 = 0.0f;
-#pragma unroll 8
-    for (int c = 0; c < chunk_count; ++c) {
-        float const *p = stat_partial + ((size_t)c * node_size + node) * 2;
-        s1 += p[0];
-        s2 += p[1];
-    }
+    int node;
+    float s1, s2;
+    if (!sum_stat_partials(stat_partial, node_size, chunk_count, nodes_per_block, node, s1, s2)) { return; }
     float const r  = 1.0f / (float)frame_size;
     float const m0 = s1 * r;                                  // mean of (v - C0)
     float const m  = C[(size_t)node * nn] + m0;
@@ -785,17 +812,12 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 __global__ __launch_bounds__(kBlock) void bn_backward_finalize_kernel(float const *__restrict__ stat_partial,
                                                                      float const *__restrict__ mean, float const *__restrict__ rstd,
                                                                      float *__restrict__ dmean, float *__restrict__ dvar,
-                                                                     float gamma, int node_size, int slab_count, int frame_size)
+                                                                     float gamma, int node_size, int slab_count, int frame_size,
+                                                                     int nodes_per_block)
 {
-    int const node = blockIdx.x * kBlock + threadIdx.x;
-    if (node >= node_size) { return; }
-    float s0 = 0.0f, s1 = 0.0f;
-#pragma unroll 8
-    for (int s = 0; s < slab_count; ++s) {
-        float const *p = stat_partial + ((size_t)s * node_size + node) * 2;
-        s0 += p[0];
-        s1 += p[1];
-    }
+    int node;
+    float s0, s1;
+    if (!sum_stat_partials(stat_partial, node_size, slab_count, nodes_per_block, node, s0, s1)) { return; }
     float const rs = rstd[node];
     float const dstd   = -(gamma * s1) * (rs * rs);
     float const dmeanx = -(gamma * s0) * rs;
