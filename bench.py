@@ -26,7 +26,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("lut_dx_kernel<6>", 0):       (686295.3 * 2.0 + 132096.0) * 1024,
     ("lut_forward_kernel<6>", 0):  (132275.3 * 2.0 + 131072.0) * 1024,
     ("lut_backward_kernel<6>", 0): (352923.2 * 2.0 + 6352.6) * 1024,
-    ("binary_lut6_kernel", 0):     (1020878.0 * 2.0 + 524288.0) * 1024,
+    ("binary_lut6_kernel", 0):     (649069.0 * 2.0 + 524288.0) * 1024,
     ("adam_kernel", 0):            (527931.3 * 2.0 + 791860.5) * 1024,
 }
 

@@ -106,7 +106,11 @@ int fwd_chunk_frames(int xmode, int frame_size, int tile_count)
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  return ((v + 63) / 64) * 64; }       // 0: chosen per call
 int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
 int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 2); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
-int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 256); return ((v + 63) / 64) * 64; }
+// BinaryLut6 units of 192 words: 8192 input rows x 768 bytes is what stays in an XCD's L2 next to the output stream
+// (256-word units fetch 2.3 GB per launch at the benchmark shape, 192-word units 1.9 GB; 128-word units fetch less still
+// but leave a wavefront too little work per set-up)
+int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 192); return ((v + 63) / 64) * 64; }
+int bin_nodes_per_wave(void) { static int v = env_int("BBHIP_BIN_NODES", 0); return v >= 4 ? 4 : v >= 2 ? 2 : v == 1 ? 1 : 0; }     // 0: chosen per call
 
 // ------------------------------------------------------------------------------------------------
 //  scratch arena: one growing device buffer per device, reused by every call
@@ -1281,25 +1285,30 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     BBHIP_REQUIRE(node_size > 0 && node_size <= (0x7fffffff >> 6) && frame_size > 0);
     BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    char *base = nullptr;
-    if (arena_get(align256((size_t)node_size * 64 * sizeof(uint32_t)), &base)) { return 1; }
-    uint32_t *mask = reinterpret_cast<uint32_t *>(base);
-    hipLaunchKernelGGL(binary_mask_kernel, dim3(ceil_div(node_size * 64, kBlock)), dim3(kBlock), 0, st, dev_table, mask, node_size);
-    BBHIP_LAUNCH_CHECK();
     BinArgs a{};
     a.x = reinterpret_cast<uint32_t const *>(dev_x_buf);
     a.y = reinterpret_cast<uint32_t *>(dev_y_buf);
-    a.idx = dev_input_index; a.mask = mask;
+    a.idx = dev_input_index; a.table = dev_table;
     a.node_size = node_size; a.frame_size = frame_size; a.stride = frame_stride;
     a.word_count = (frame_size + 31) / 32;
     a.chunk = bin_chunk_words();
     a.chunk_count = ceil_div(a.word_count, a.chunk);
-    a.tiles = make_tile_divisor(ceil_div(node_size, kWavesPerBlk));
+    // nodes per wavefront: four share a unit's set-up where that still leaves the launch 2048 workgroups
+    int npw = bin_nodes_per_wave();
+    if (npw == 0) {
+        npw = 4;
+        while (npw > 1 && (long long)a.chunk_count * ceil_div(node_size, kWavesPerBlk * npw) < 2048) { npw /= 2; }
+    }
+    a.tiles = make_tile_divisor(ceil_div(node_size, kWavesPerBlk * npw));
     BBHIP_REQUIRE((long long)a.chunk_count * a.tiles.count <= 0x7fffffffLL);
     {
         ScopedTimer tm(kTimeBinary, st);
-        if (a.chunk % 128 == 0) { hipLaunchKernelGGL(binary_lut6_kernel<2>, dim3(a.chunk_count * a.tiles.count), dim3(kBlock), 0, st, a); }
-        else                    { hipLaunchKernelGGL(binary_lut6_kernel<1>, dim3(a.chunk_count * a.tiles.count), dim3(kBlock), 0, st, a); }
+        dim3 const grid(a.chunk_count * a.tiles.count), block(kBlock);
+        switch (npw) {
+        case 1: hipLaunchKernelGGL(binary_lut6_kernel<1>, grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL(binary_lut6_kernel<2>, grid, block, 0, st, a); break;
+        default: hipLaunchKernelGGL(binary_lut6_kernel<4>, grid, block, 0, st, a); break;
+        }
     }
     BBHIP_LAUNCH_CHECK();
     return 0;

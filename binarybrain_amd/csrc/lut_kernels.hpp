@@ -875,31 +875,15 @@ __global__ __launch_bounds__(kBlock) void conv_bit_to_real_kernel(uint32_t const
 }
 
 // ------------------------------------------------------------------------------------------------
-//  BinaryLut6: y = table[x5 x4 x3 x2 x1 x0] on 32 frames per word, as a 6-level multiplexer tree of bit-selects
-//  (reference semantics: include/bb/BinaryLutN.h:436-463 — input k is index bit k, entries 0-31 in table word 0)
+//  BinaryLut6: y = table[x5 x4 x3 x2 x1 x0] on 32 frames per word
+//  (reference semantics: include/bb/BinaryLutN.h:436-463 — input k is index bit k, entries 0-31 in table word 0).
+//  Evaluated as a 6-level multiplexer tree whose first two levels are replaced by a register lookup: they turn each
+//  group of four table entries into one of the 16 Boolean functions of (x0, x1), and which one is the group's table
+//  nibble, the same for every frame.  Per word the kernel forms all 16 functions once (12 three-input bit operations),
+//  picks the group values out of that register array with the nibbles as wave-uniform register indices while
+//  multiplexing by x2 (16 instructions), and finishes with the last three levels (7 bit-selects): 35 vector
+//  instructions per word where the plain tree takes 63, and the table stays packed in two scalar registers per node.
 // ------------------------------------------------------------------------------------------------
-struct BinArgs {
-    uint32_t const *x;
-    uint32_t       *y;
-    int const      *idx;
-    uint32_t const *mask;       // [O][64]: table bit k expanded to 0 / 0xffffffff (binary_mask_kernel)
-    int node_size, frame_size, stride;   // stride in words
-    int word_count;             // (frame_size + 31) / 32
-    int chunk;                  // words per unit, multiple of 64
-    int chunk_count;
-    TileDivisor tiles;
-};
-
-// table [O][2] (entries 0-31 in word 0) -> mask [O][64]
-__global__ __launch_bounds__(kBlock) void binary_mask_kernel(int const *__restrict__ table, uint32_t *__restrict__ mask, int node_size)
-{
-    int const t = blockIdx.x * kBlock + threadIdx.x;
-    if (t >= node_size * 64) { return; }
-    int const node = t >> 6, k = t & 63;
-    uint32_t const w = (uint32_t)table[node * 2 + (k >> 5)];
-    mask[t] = ((w >> (k & 31)) & 1u) ? 0xffffffffu : 0u;
-}
-
 // bit-select d = (s & hi) | (~s & lo): one instruction per multiplexer of the tree
 __device__ __forceinline__ uint32_t bfi_vvv(uint32_t s, uint32_t hi, uint32_t lo)
 {
@@ -907,72 +891,139 @@ __device__ __forceinline__ uint32_t bfi_vvv(uint32_t s, uint32_t hi, uint32_t lo
     asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "v"(s), "v"(hi), "v"(lo));
     return d;
 }
-// same with the "hi" operand wave-uniform (scalar register)
-__device__ __forceinline__ uint32_t bfi_vsv(uint32_t s, uint32_t hi, uint32_t lo)
+
+struct BinArgs {
+    uint32_t const *x;
+    uint32_t       *y;
+    int const      *idx;
+    int const      *table;      // [O][2]: entries 0-31 in word 0
+    int node_size, frame_size, word_count, stride;
+    int chunk;                  // words per unit, multiple of 64
+    int chunk_count;
+    TileDivisor tiles;
+};
+
+typedef uint32_t bin_u32x16 __attribute__((ext_vector_type(16)));
+
+// value of a two-input function as x1 varies, for fixed x0: (at x1 = 0, at x1 = 1) -> one of 0, ~0, x1, ~x1
+__device__ __forceinline__ uint32_t bin_pick(int at0, int at1, uint32_t x1, uint32_t nx1)
 {
-    uint32_t d;
-    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "v"(s), "s"(hi), "v"(lo));
-    return d;
+    return at0 ? (at1 ? 0xffffffffu : nx1) : (at1 ? x1 : 0u);
 }
 
-template <int WPL>   // words per lane per step
+// Four level-2 multiplexers t_j = x2 ? fn[nibble 2j+1] : fn[nibble 2j] of one 32-bit table word (eight groups of four
+// entries).  The function values sit in fixed registers v48..v63 and are picked with the vector-register index mode:
+// while it is on for source 0, source 0 of a vector instruction names register v48 + index.  One move fetches the x2 = 0
+// value, one three-input bit operation (truth table 0xe2: source 1 selects between source 0 and source 2) fetches the
+// x2 = 1 value and multiplexes.  The mode stays on across the block; only the index changes, each nibble extracted by
+// the scalar unit right before it is used (the table stays packed: two scalar registers per node).
+__device__ __forceinline__ void bin_select_level2(bin_u32x16 const &fn, uint32_t table_word, uint32_t x2,
+                                                  uint32_t &t0, uint32_t &t1, uint32_t &t2, uint32_t &t3)
+{
+    uint32_t tmp, idx;
+    asm volatile(
+        "s_bfe_u32 %[i], %[tw], 0x40000\n\t"
+        "s_set_gpr_idx_on %[i], gpr_idx(SRC0)\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x40004\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_bitop3_b32 %[t0], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x40008\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x4000c\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_bitop3_b32 %[t1], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x40010\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x40014\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_bitop3_b32 %[t2], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x40018\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_bfe_u32 %[i], %[tw], 0x4001c\n\t"
+        "s_set_gpr_idx_idx %[i]\n\t"
+        "v_bitop3_b32 %[t3], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_set_gpr_idx_off"
+        : [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [tmp] "=&v"(tmp), [i] "=&s"(idx)
+        : [tw] "s"(table_word), [x2] "v"(x2),
+          "{v48}"(fn[0]), "{v49}"(fn[1]), "{v50}"(fn[2]), "{v51}"(fn[3]), "{v52}"(fn[4]), "{v53}"(fn[5]), "{v54}"(fn[6]), "{v55}"(fn[7]),
+          "{v56}"(fn[8]), "{v57}"(fn[9]), "{v58}"(fn[10]), "{v59}"(fn[11]), "{v60}"(fn[12]), "{v61}"(fn[13]), "{v62}"(fn[14]), "{v63}"(fn[15])
+        : "m0", "scc");
+}
+
+template <int NPW>   // nodes per wavefront
 __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
 {
     int const B    = a.chunk_count * a.tiles.count;
     int const lid  = xcd_remap(blockIdx.x, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
-    int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
-    if (node >= a.node_size) { return; }
+    int const node0 = __builtin_amdgcn_readfirstlane((tile * kWavesPerBlk + (int)(threadIdx.x / kWave)) * NPW);
+    if (node0 >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
-    // level-0 multiplexers select between two table entries: entry 2k+1 stays in a scalar register, entry 2k is
-    // copied once per unit into a vector register (an instruction may read one scalar register only)
-    uint32_t const *__restrict__ mg = a.mask + (size_t)node * 64;
-    uint32_t m_hi[32], m_lo[32];
+    uint32_t const row_bytes = (uint32_t)a.word_count * 4u;
+    uint32_t tw[NPW][2];
+    char const *rows[NPW][6];               // wave-uniform row bases: loads take a scalar base and a 32-bit lane offset
+    __amdgpu_buffer_rsrc_t yr[NPW];
+    bool live[NPW];
 #pragma unroll
-    for (int k = 0; k < 32; ++k) {
-        m_hi[k] = mg[2 * k + 1];
-        uint32_t const lo = mg[2 * k];
-        asm("v_mov_b32 %0, %1" : "=v"(m_lo[k]) : "s"(lo));
+    for (int p = 0; p < NPW; ++p) {
+        live[p] = node0 + p < a.node_size;
+        int const node = live[p] ? node0 + p : node0;       // a wavefront past the last node repeats its first one and stores nothing
+        tw[p][0] = (uint32_t)__builtin_amdgcn_readfirstlane(a.table[node * 2]);
+        tw[p][1] = (uint32_t)__builtin_amdgcn_readfirstlane(a.table[node * 2 + 1]);
+#pragma unroll
+        for (int k = 0; k < 6; ++k) {
+            rows[p][k] = reinterpret_cast<char const *>(a.x) + (size_t)a.idx[node * 6 + k] * (size_t)a.stride * 4u;
+        }
+        // outputs go through a buffer descriptor that ends with the row: stores of lanes beyond it are dropped
+        // (an empty range drops every store)
+        yr[p] = row_descriptor(a.y, node, a.stride, live[p] ? row_bytes : 0u);
     }
 
-    // rows are addressed through buffer descriptors that end with the last word of the row: lanes beyond it read 0 and
-    // their stores are dropped, so the loop carries neither index clamps nor lane masks
-    uint32_t const row_bytes = (uint32_t)a.word_count * 4u;
-    __amdgpu_buffer_rsrc_t rows[6];
-#pragma unroll
-    for (int k = 0; k < 6; ++k) { rows[k] = row_descriptor(a.x, a.idx[node * 6 + k], a.stride, row_bytes); }
-    __amdgpu_buffer_rsrc_t const yr = row_descriptor(a.y, node, a.stride, row_bytes);
-
     int const w_begin = ck * a.chunk;
-    int const w_end   = min(w_begin + a.chunk, a.word_count);       // a.chunk is a multiple of the words per step
+    int const w_end   = min(w_begin + a.chunk, a.word_count);
     int const w_last  = a.word_count - 1;
     uint32_t const tail_mask = (a.frame_size & 31) ? ((1u << (a.frame_size & 31)) - 1u) : 0xffffffffu;
 
+    uint32_t const last_off = (uint32_t)w_last * 4u;        // lanes beyond the row re-read its last word; their stores are dropped
     uint32_t off = (uint32_t)(w_begin + lane) * 4u;
-    for (int w0 = w_begin; w0 < w_end; w0 += kWave * WPL, off += kWave * WPL * 4u) {
-        uint32_t xv[WPL][6];
+    for (int w0 = w_begin; w0 < w_end; w0 += kWave, off += kWave * 4u) {
+        uint32_t xv[NPW][6];
+        uint32_t const at = min(off, last_off);
 #pragma unroll
-        for (int u = 0; u < WPL; ++u) {
+        for (int p = 0; p < NPW; ++p) {
 #pragma unroll
-            for (int k = 0; k < 6; ++k) { xv[u][k] = __builtin_amdgcn_raw_buffer_load_b32(rows[k], off + u * (kWave * 4u), 0, 0); }
+            for (int k = 0; k < 6; ++k) { xv[p][k] = *reinterpret_cast<uint32_t const *>(rows[p][k] + at); }
         }
-        bool const has_tail = (w0 + kWave * WPL > w_last);          // wave-uniform: only the last step of a row
+        bool const has_tail = (w0 + kWave > w_last);            // wave-uniform: only the last step of a row
 #pragma unroll
-        for (int u = 0; u < WPL; ++u) {
-            uint32_t t[32];
+        for (int p = 0; p < NPW; ++p) {
+            uint32_t const x0 = xv[p][0], x1 = xv[p][1], nx1 = ~x1;
+            bin_u32x16 fn;
 #pragma unroll
-            for (int k = 0; k < 32; ++k) { t[k] = bfi_vsv(xv[u][0], m_hi[k], m_lo[k]); }
+            for (int c = 0; c < 16; ++c) {
+                // table position q = x0 + 2 * x1: bit q of c is the function's value there
+                uint32_t const g0 = bin_pick(c & 1, (c >> 2) & 1, x1, nx1);          // x0 = 0
+                uint32_t const g1 = bin_pick((c >> 1) & 1, (c >> 3) & 1, x1, nx1);   // x0 = 1
+                fn[c] = (x0 & g1) | (~x0 & g0);
+            }
+            uint32_t t[8];
+            bin_select_level2(fn, tw[p][0], xv[p][2], t[0], t[1], t[2], t[3]);
+            bin_select_level2(fn, tw[p][1], xv[p][2], t[4], t[5], t[6], t[7]);
 #pragma unroll
-            for (int lv = 1; lv < 6; ++lv) {
+            for (int lv = 3; lv < 6; ++lv) {
 #pragma unroll
-                for (int k = 0; k < (32 >> lv); ++k) { t[k] = bfi_vvv(xv[u][lv], t[2 * k + 1], t[2 * k]); }
+                for (int k = 0; k < (32 >> lv); ++k) { t[k] = bfi_vvv(xv[p][lv], t[2 * k + 1], t[2 * k]); }
             }
             uint32_t r = t[0];
-            if (has_tail && (w0 + u * kWave + lane == w_last)) { r &= tail_mask; }
+            if (has_tail && (w0 + lane == w_last)) { r &= tail_mask; }
             // streamed once (non-temporal): keep it from displacing x rows in L2
-            __builtin_amdgcn_raw_buffer_store_b32(r, yr, off + u * (kWave * 4u), 0, 2);
+            __builtin_amdgcn_raw_buffer_store_b32(r, yr[p], off, 0, 2);
         }
     }
 }
