@@ -951,7 +951,7 @@ __device__ __forceinline__ void bin_select_level2(bin_u32x16 const &fn, uint32_t
         : [tw] "s"(table_word), [x2] "v"(x2),
           "{v48}"(fn[0]), "{v49}"(fn[1]), "{v50}"(fn[2]), "{v51}"(fn[3]), "{v52}"(fn[4]), "{v53}"(fn[5]), "{v54}"(fn[6]), "{v55}"(fn[7]),
           "{v56}"(fn[8]), "{v57}"(fn[9]), "{v58}"(fn[10]), "{v59}"(fn[11]), "{v60}"(fn[12]), "{v61}"(fn[13]), "{v62}"(fn[14]), "{v63}"(fn[15])
-        : "m0", "scc");
+        : "scc");                // (M0 is changed too; the compiler keeps nothing there across statements)
 }
 
 template <int NPW>   // nodes per wavefront
