@@ -158,16 +158,30 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
     }
 
 template <int N>
-void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st)
+void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st, float *V = nullptr, float bias = 0.0f)
 {
     int const total = node_size * (1 << N);
-    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize);
+    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize, V, bias);
 }
 
 template <int N, int XMODE, int YMODE, int KIND>
 void launch_forward(FwdArgs const &a, int npw, hipStream_t st)
 {
     dim3 const grid(a.chunk_count * a.tiles.count), block(kBlock);
+    if constexpr (XMODE == kXBit || XMODE == kXBinary) {
+        // two-valued inputs: the corner-value kernel wherever the caller prepared the values (one node per wavefront)
+        if (a.V != nullptr) {
+            if constexpr (XMODE == kXBit) {
+                // 32-byte scalar loads where they stay inside the row pitch and never straddle a unit
+                if (a.x_stride % 8 == 0 && a.chunk % 256 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 3u) == 0) {
+                    hipLaunchKernelGGL((lut_forward_corner_kernel<N, XMODE, YMODE, KIND, true>), grid, block, 0, st, a);
+                    return;
+                }
+            }
+            hipLaunchKernelGGL((lut_forward_corner_kernel<N, XMODE, YMODE, KIND>), grid, block, 0, st, a);
+            return;
+        }
+    }
     if (npw == 2) { hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND, 2>), grid, block, 0, st, a); }
     else          { hipLaunchKernelGGL((lut_forward_kernel<N, XMODE, YMODE, KIND, 1>), grid, block, 0, st, a); }
 }
@@ -272,30 +286,40 @@ int check_forward(ForwardCall const &c)
 // workgroup's threads share one node
 int stat_nodes_per_block(int unit_count) { return unit_count >= 512 ? 4 : unit_count >= 64 ? 16 : 64; }
 
+// two-valued inputs (packed bits, fp32 binarized at 0.5): the kernels that look the LUT output up among the node's corner values
+bool use_corner_values(int xmode)
+{
+    static int const on = env_int("BBHIP_CORNER", 1);
+    return on == 1 && (xmode == kXBit || xmode == kXBinary);
+}
+
 template <int N>
 int run_forward(ForwardCall const &c, hipStream_t st)
 {
     constexpr int NN = 1 << N;
-    int const npw         = fwd_nodes_per_wave();
+    bool const corner     = use_corner_values(c.xmode);
+    int const npw         = corner ? 1 : fwd_nodes_per_wave();
     int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
     int const chunk       = fwd_chunk_frames(c.xmode, c.frame_size, tile_count);
     int const chunk_count = ceil_div(c.frame_size, chunk);
     if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("forward: grid too large"); }
 
     size_t const c_bytes    = align256((size_t)c.node_size * NN * sizeof(float));
+    size_t const v_bytes    = corner ? c_bytes : 0;
     size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
     size_t const rstd_bytes = (c.bn == 2) ? align256((size_t)c.node_size * sizeof(float)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + stat_bytes + rstd_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + v_bytes + stat_bytes + rstd_bytes, &base)) { return 1; }
     float *C        = reinterpret_cast<float *>(base);
-    float *stat     = reinterpret_cast<float *>(base + c_bytes);
-    float *rstd_tmp = reinterpret_cast<float *>(base + c_bytes + stat_bytes);
+    float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
+    float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
+    float *rstd_tmp = reinterpret_cast<float *>(base + c_bytes + v_bytes + stat_bytes);
 
-    launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st);
+    launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias);
     BBHIP_LAUNCH_CHECK();
 
     FwdArgs a{};
-    a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C;
+    a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C; a.V = V;
     a.node_size = c.node_size; a.frame_size = c.frame_size;
     a.x_stride = c.x_stride; a.y_stride = c.y_stride;
     a.chunk = chunk; a.chunk_count = chunk_count; a.tiles = make_tile_divisor(tile_count);
@@ -410,14 +434,18 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     size_t const c_bytes    = align256((size_t)c.output_node_size * NN * sizeof(float));
     size_t const part_bytes = align256((size_t)slab_total * c.output_node_size * NN * sizeof(float));
     // batch-norm statistics pass: the forward kernel's unit structure (frame chunks, see below)
-    int const stat_chunk       = fwd_chunk_frames(c.xmode, c.frame_size, ceil_div(c.output_node_size, kWavesPerBlk * fwd_nodes_per_wave()));
+    bool const corner = c.bn && use_corner_values(c.xmode);     // the statistics pass looks the LUT output up among corner values
+    int const stat_npw = corner ? 1 : fwd_nodes_per_wave();
+    int const stat_chunk       = fwd_chunk_frames(c.xmode, c.frame_size, ceil_div(c.output_node_size, kWavesPerBlk * stat_npw));
     int const stat_chunk_count = ceil_div(c.frame_size, stat_chunk);
     size_t const stat_bytes = c.bn ? align256((size_t)stat_chunk_count * c.output_node_size * 2 * sizeof(float)) : 0;
     size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;
     size_t const dtab_bytes = align256(term_count * sizeof(int));
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
+    size_t const v_bytes = corner ? c_bytes : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes, &base)) { return 1; }
+    float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
@@ -426,7 +454,7 @@ int run_backward(BackwardCall const &c, hipStream_t st)
 
     // centred coefficients: needed where the LUT output is recomputed (batch-norm) or per-connection gradients are formed
     if (c.bn || dxmode != kDxNone) {
-        launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st);
+        launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st, V, c.bias);
         BBHIP_LAUNCH_CHECK();
     }
     // the term table of the dx kernel is built by extra workgroups at the end of the table-gradient launch
@@ -455,11 +483,11 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     if (c.bn) {
         // phase 0: per-node sums over ALL frames, then dmean / dvar.  It only recomputes the LUT output, so it runs in the
         // forward kernel (kind 3): frame chunks that keep the gathered rows in L2, partial sums from the matrix unit
-        int const npw = fwd_nodes_per_wave();
+        int const npw = stat_npw;
         int const stat_tiles = ceil_div(c.output_node_size, kWavesPerBlk * npw);
         if ((long long)stat_chunk_count * stat_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
         FwdArgs f{};
-        f.x = c.x; f.idx = c.idx; f.C = C; f.mean = c.mean; f.rstd = c.rstd; f.stat_partial = stat;
+        f.x = c.x; f.idx = c.idx; f.C = C; f.V = V; f.mean = c.mean; f.rstd = c.rstd; f.stat_partial = stat;
         f.dy = c.dy; f.dy_stride = c.frame_stride;
         f.node_size = c.output_node_size; f.frame_size = c.frame_size; f.x_stride = c.x_stride;
         f.chunk = stat_chunk; f.chunk_count = stat_chunk_count; f.tiles = make_tile_divisor(stat_tiles);

@@ -41,9 +41,12 @@ __device__ __forceinline__ float wave_sum(float v)
 //    C = coefficients in the centred monomial basis,  y = sum_S C[S] prod_{j in S} (x_j - 1/2)
 //  (the plain-basis coefficients P,  y = sum_S P[S] prod_{j in S} x_j,  are formed inside term_table_block)
 // ------------------------------------------------------------------------------------------------
+//  For two-valued inputs (x_j = 1/2 -+ bias) the layer is a table of 2^N values, V[p] = y at the corner whose bit j says
+//  which value input j takes: one more butterfly over C, (a, b) -> (a - bias b, a + bias b) per variable.
 template <int N>
 __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
-                                                           int node_size, int lut_binarize)
+                                                           int node_size, int lut_binarize,
+                                                           float *__restrict__ V = nullptr, float bias = 0.0f)
 {
     constexpr int NN = 1 << N;
     int const t = blockIdx.x * kBlock + threadIdx.x;
@@ -60,6 +63,13 @@ __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restr
         v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f;
     }
     if (t < total) { C[t] = v; }
+    if (V == nullptr) { return; }           // same for every thread of the launch
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float const o = __shfl_xor(v, 1 << j, 64);
+        v = ((i >> j) & 1) ? __builtin_fmaf(bias, v, o) : __builtin_fmaf(-bias, o, v);
+    }
+    if (t < total) { V[t] = v; }
 }
 
 // dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order)
@@ -154,6 +164,7 @@ struct FwdArgs {
     void        *y;
     int const   *idx;
     float const *C;             // [O][2^N] centred coefficients
+    float const *V;             // [O][2^N] corner values (two-valued inputs: lut_forward_corner_kernel)
     float const *mean;          // BN: per node (nullptr otherwise)
     float const *rstd;
     float       *stat_partial;  // STATS: [chunk][O][2] partial sums of (v - C0), (v - C0)^2;  kind 3: of g, g (v - mean)
@@ -166,6 +177,55 @@ struct FwdArgs {
     TileDivisor tiles;
     float bias, gamma, beta;
 };
+
+// What a forward kernel does with the LUT output v of (node, frame f = f0 + lane): accumulate statistics (kinds 2, 3) or
+// apply the batch-norm output stage (kind 1) and store.  ok: the frame belongs to the unit; live: the node exists.
+template <int YMODE, int FWD_KIND>
+__device__ __forceinline__ void forward_stage(FwdArgs const &a, float v, bool ok, bool live, int lane, int node, int f0, int f, int f_end,
+                                              float mean, float rstd, float c0, float dyv, float &s1, float &s2)
+{
+    if (FWD_KIND == 2) {
+        float const d = ok ? (v - c0) : 0.0f;
+        s1 += d;
+        s2 = __builtin_fmaf(d, d, s2);
+        return;
+    }
+    if (FWD_KIND == 3) {
+        float const t = ((v - mean) * rstd) * a.gamma + a.beta;
+        float d = ok ? dyv : 0.0f;
+        if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
+        s1 += d;
+        s2 = __builtin_fmaf(d, v - mean, s2);
+        return;
+    }
+    if (FWD_KIND == 1) {
+        v = (v - mean) * rstd;
+        v = v * a.gamma + a.beta;
+    }
+    if (!live) { return; }
+    if (YMODE == kYBit) {
+        uint64_t const m = __ballot(ok && (v > 0.5f));
+        uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
+        if (lane == 0)                          { yr[0] = (uint32_t)m; }
+        if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
+    }
+    else {
+        if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+        else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+        if (ok) { __builtin_nontemporal_store(v, reinterpret_cast<float *>(a.y) + (size_t)node * a.y_stride + f); }
+    }
+}
+
+// per (unit, node) partial sums of the statistics kinds
+__device__ __forceinline__ void forward_store_stats(FwdArgs const &a, int ck, int node, bool live, int lane, float s1, float s2)
+{
+    float const t1 = wave_sum(s1), t2 = wave_sum(s2);
+    if (lane == 0 && live) {
+        float *q = a.stat_partial + ((size_t)ck * a.node_size + node) * 2;
+        q[0] = t1;
+        q[1] = t2;
+    }
+}
 
 // FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only,
 //           3 = statistics of the backward pass through batch-norm: per node the sums of g and g (v - mean), where g = dy gated by
@@ -252,51 +312,100 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
                 if constexpr (kMatrix) { v = mq[p].forward(z); }
                 else                   { v = LutEval<N>::forward(C[p], cv[p], z); }
 
-                if (FWD_KIND == 2) {
-                    float const d = ok ? (v - c0[p]) : 0.0f;
-                    s1[p] += d;
-                    s2[p] = __builtin_fmaf(d, d, s2[p]);
-                    continue;
-                }
-                if (FWD_KIND == 3) {
-                    float const t = ((v - mean[p]) * rstd[p]) * a.gamma + a.beta;
-                    float d = ok ? dyv[p][u] : 0.0f;
-                    if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
-                    s1[p] += d;
-                    s2[p] = __builtin_fmaf(d, v - mean[p], s2[p]);
-                    continue;
-                }
-                if (FWD_KIND == 1) {
-                    v = (v - mean[p]) * rstd[p];
-                    v = v * a.gamma + a.beta;
-                }
-                if (!live[p]) { continue; }
-                if (YMODE == kYBit) {
-                    uint64_t const m = __ballot(ok && (v > 0.5f));
-                    uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node[p] * a.y_stride + (f0 >> 5);
-                    if (lane == 0)                          { yr[0] = (uint32_t)m; }
-                    if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
-                }
-                else {
-                    if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
-                    else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
-                    if (ok) { __builtin_nontemporal_store(v, reinterpret_cast<float *>(a.y) + (size_t)node[p] * a.y_stride + f); }
-                }
+                forward_stage<YMODE, FWD_KIND>(a, v, ok, live[p], lane, node[p], f0, f, f_end, mean[p], rstd[p], c0[p],
+                                               (FWD_KIND == 3) ? dyv[p][u] : 0.0f, s1[p], s2[p]);
             }
         }
     }
 
     if (FWD_KIND == 2 || FWD_KIND == 3) {
 #pragma unroll
-        for (int p = 0; p < NPW; ++p) {
-            float const t1 = wave_sum(s1[p]), t2 = wave_sum(s2[p]);
-            if (lane == 0 && live[p]) {
-                float *q = a.stat_partial + ((size_t)ck * a.node_size + node[p]) * 2;
-                q[0] = t1;
-                q[1] = t2;
+        for (int p = 0; p < NPW; ++p) { forward_store_stats(a, ck, node[p], live[p], lane, s1[p], s2[p]); }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  Forward for two-valued inputs (packed bits, or fp32 frames binarized at 0.5): the LUT output is one of the 2^N corner
+//  values V of the node.  A lane builds the corner index of its frame from the N input bits (one add-with-carry per input:
+//  index = 2 index + bit, the bit arriving as a lane mask in a scalar register pair) and fetches V[index] from the lane
+//  that holds it (ds_bpermute): N + 2 instructions per (node, 64 frames) instead of the polynomial's 45.
+//  One wavefront = one node x one unit of frames; kinds and output modes as in lut_forward_kernel.
+// ------------------------------------------------------------------------------------------------
+//  WIDE (packed bits, row pitch a multiple of 8 words, units a multiple of 256 frames): the bits of 256 frames of an input
+//  are one 32-byte scalar load, so a unit costs N scalar loads per four steps instead of 2 N per step.
+template <int N, int XMODE, int YMODE, int FWD_KIND, bool WIDE = false>
+__global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
+{
+    static_assert(XMODE == kXBit || XMODE == kXBinary, "corner values need two-valued inputs");
+    static_assert(!WIDE || XMODE == kXBit, "wide loads are for packed bits");
+    constexpr int NN = 1 << N;
+    int const B    = a.chunk_count * a.tiles.count;
+    int const lid  = xcd_remap(blockIdx.x, B);
+    int ck, tile;
+    split_tile(lid, a.tiles, ck, tile);
+    int const node = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
+    if (node >= a.node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    int const corner = __float_as_int(a.V[(size_t)node * NN + (lane & (NN - 1))]);      // lane p holds V[p]
+    void const *rows[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        int const in = a.idx[node * N + k];
+        rows[k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
+                                   : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
+    }
+    float mean = 0.0f, rstd = 1.0f, c0 = 0.0f;
+    if (FWD_KIND == 1 || FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
+    if (FWD_KIND == 2) { c0 = a.C[(size_t)node * NN]; }
+
+    int const f_begin = ck * a.chunk;
+    int const f_end   = min(f_begin + a.chunk, a.frame_size);
+    int const f_last  = a.frame_size - 1;
+    float s1 = 0.0f, s2 = 0.0f;
+
+    constexpr int U = (XMODE == kXBit && !WIDE) ? 2 : 4;  // wavefront-steps whose loads are issued together
+    for (int fb = f_begin; fb < f_end; fb += kWave * U) {
+        typename Gather<N, XMODE>::Raw raw[U][N];
+        float dyv[U];
+        if constexpr (WIDE) {
+            typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+            typedef __attribute__((address_space(4))) u32x8 const const_u32x8;
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                u32x8 const w = *(const_u32x8 *)(reinterpret_cast<uint32_t const *>(rows[k]) + (fb >> 5));     // fb is a multiple of 256
+#pragma unroll
+                for (int u = 0; u < U; ++u) { raw[u][k] = (uint64_t)w[2 * u] | ((uint64_t)w[2 * u + 1] << 32); }
             }
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
+                if constexpr (!WIDE) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
+                if (FWD_KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int const f0 = fb + u * kWave;
+            if (f0 >= f_end) { break; }
+            int const  f  = f0 + lane;
+            bool const ok = f < f_end;
+            // corner index, most significant input first: index = 2 index + bit
+            uint32_t index = 0;
+#pragma unroll
+            for (int k = N - 1; k >= 0; --k) {
+                uint64_t mask, carry;
+                if constexpr (XMODE == kXBit) { mask = raw[u][k]; }
+                else                          { mask = __ballot(__uint_as_float(raw[u][k]) > 0.5f); }
+                asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(index), "=s"(carry) : "v"(index), "s"(mask));
+            }
+            float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), corner));
+            forward_stage<YMODE, FWD_KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
+                                           (FWD_KIND == 3) ? dyv[u] : 0.0f, s1, s2);
+        }
     }
+    if (FWD_KIND == 2 || FWD_KIND == 3) { forward_store_stats(a, ck, node, true, lane, s1, s2); }
 }
 
 // Sum of the per-unit partial sums [count][node_size][2] of one node.  A workgroup owns nodes_per_block consecutive nodes

@@ -102,6 +102,25 @@ def test_bit_input(ops, n):
     ops.set_dx_mode(0)
 
 
+@pytest.mark.parametrize("extra_words", [1, 3, 8])
+def test_bit_input_row_pitches(ops, extra_words):
+    """packed rows whose pitch is not a multiple of 8 words take the per-step loads, others the 32-byte loads: same results"""
+    rng = np.random.default_rng(300 + extra_words)
+    I, O, F = 40, 24, 1000
+    idx = synth.wiring(rng, I, O, 6); W = synth.lut_tables(rng, O, 6)
+    xs = (F + 31) // 32 + extra_words; ys = synth.frame_stride_fp32(F)
+    xb = synth.bernoulli_bits(rng, I, F, xs); dy = synth.normal_frames(rng, O, F, ys)
+    y_ref = oracle.bit_stochastic_lut_forward(6, xb, idx, W, F, ys, 0)
+    y = ops.bit_stochastic_lut_forward(6, dev(xb), dev(idx), dev(W), F, ys, 0)
+    assert_fwd(host(y)[:, :F], y_ref[:, :F])
+    yb = ops.bit_bit_stochastic_lut_forward(6, dev(xb), dev(idx), dev(W), F, 0)
+    assert np.array_equal(synth.unpack_bits(host(yb), F), synth.unpack_bits(oracle.bit_bit_stochastic_lut_forward(6, xb, idx, W, F, 0), F))
+    dx_ref, dW_ref = oracle.bit_stochastic_lut_backward(6, xb, dy, idx, W, F, None, 0)
+    dW = dev(np.zeros((O, 64), np.float32))
+    dx = ops.bit_stochastic_lut_backward(6, dev(xb), dev(dy), dev(idx), dev(W), dW, F, ops.reverse_table(dev(idx), I), 0)
+    assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
+
+
 def test_golden_vectors_on_gpu(ops):
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "stochastic_lut.npz"))
     for k in range(int(g["count"][0])):
