@@ -90,6 +90,13 @@ int env_int(char const *name, int def)
     return v > 0 ? v : def;
 }
 
+// two-valued inputs (packed bits, fp32 binarized at 0.5): the kernels that look the LUT output up among the node's corner values
+bool use_corner_values(int xmode)
+{
+    static int const on = env_int("BBHIP_CORNER", 1);
+    return on == 1 && (xmode == kXBit || xmode == kXBinary);
+}
+
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); return v >= 2 ? 2 : 1; }
 // Frames per forward unit.  fp32 rows are gathered through L2, and a 256-frame piece of every input row is what one XCD's L2
@@ -104,8 +111,11 @@ int fwd_chunk_frames(int xmode, int frame_size, int tile_count)
     return chunk;
 }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  return ((v + 63) / 64) * 64; }       // 0: chosen per call
-int dx_chunk_frames(void)  { static int v = env_int("BBHIP_DX_CHUNK", 128); return ((v + 63) / 64) * 64; }
-int dx_pass_steps(void)    { static int v = env_int("BBHIP_DX_STEPS", 2); return (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
+// dx units: frames per unit and wavefront-steps per pass over the work list.  128 frames in passes of two steps where the
+// gathered rows are fp32 (what L2 holds); packed-bit rows leave room for 256 frames in passes of four, which halves the
+// per-term set-up per frame.  0: not set in the environment.
+int dx_chunk_frames_env(void) { static int v = env_int("BBHIP_DX_CHUNK", 0); return ((v + 63) / 64) * 64; }
+int dx_pass_steps_env(void)   { static int v = env_int("BBHIP_DX_STEPS", 0); return (v <= 0) ? 0 : (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
 // BinaryLut6 units of 192 words: 8192 input rows x 768 bytes is what stays in an XCD's L2 next to the output stream
 // (256-word units fetch 2.3 GB per launch at the benchmark shape, 192-word units 1.9 GB; 128-word units fetch less still
 // but leave a wavefront too little work per set-up)
@@ -231,6 +241,11 @@ template <int N, int U>
 int dispatch_dx_u(int xmode, DxArgs const &a, hipStream_t st)
 {
     dim3 const grid(a.fin_blocks + a.chunk_count * a.tiles.count), block(kBlock);
+    if (use_corner_values(xmode)) {         // the term table then holds corner values
+        if (xmode == kXBit) { hipLaunchKernelGGL((lut_dx_corner_kernel<N, kXBit, U>),    grid, block, 0, st, a); }
+        else                { hipLaunchKernelGGL((lut_dx_corner_kernel<N, kXBinary, U>), grid, block, 0, st, a); }
+        return 0;
+    }
     switch (xmode) {
     case kXClamp:  hipLaunchKernelGGL((lut_dx_kernel<N, kXClamp, U>),  grid, block, 0, st, a); return 0;
     case kXBinary: hipLaunchKernelGGL((lut_dx_kernel<N, kXBinary, U>), grid, block, 0, st, a); return 0;
@@ -285,13 +300,6 @@ int check_forward(ForwardCall const &c)
 // nodes per workgroup of the batch-norm finalize kernels: the more units there are to add per node, the more of the
 // workgroup's threads share one node
 int stat_nodes_per_block(int unit_count) { return unit_count >= 512 ? 4 : unit_count >= 64 ? 16 : 64; }
-
-// two-valued inputs (packed bits, fp32 binarized at 0.5): the kernels that look the LUT output up among the node's corner values
-bool use_corner_values(int xmode)
-{
-    static int const on = env_int("BBHIP_CORNER", 1);
-    return on == 1 && (xmode == kXBit || xmode == kXBinary);
-}
 
 template <int N>
 int run_forward(ForwardCall const &c, hipStream_t st)
@@ -469,6 +477,8 @@ int run_backward(BackwardCall const &c, hipStream_t st)
         tt.dy_row_pitch_bytes = (unsigned long long)c.frame_stride * 4ULL;
         tt.lut_binarize = c.lut_binarize; tt.rev_stride = c.rev_stride; tt.input_node_size = c.input_node_size;
         tt.blocks = (int)blocks;
+        tt.corner = use_corner_values(c.xmode) ? 1 : 0;
+        tt.lo = 0.5f - c.bias; tt.hi = 0.5f + c.bias;
     }
 
     BwdArgs a{};
@@ -531,8 +541,10 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     }
 
     if (dxmode == kDxNone) {
-        int const steps = dx_pass_steps();              // wavefront-steps per pass: {1, 2, 4}
-        int const chunk = ((dx_chunk_frames() + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
+        bool const bit_corner = (c.xmode == kXBit) && use_corner_values(c.xmode);
+        int const steps  = dx_pass_steps_env() ? dx_pass_steps_env() : (bit_corner ? 4 : 2);        // wavefront-steps per pass: {1, 2, 4}
+        int const frames = dx_chunk_frames_env() ? dx_chunk_frames_env() : (bit_corner ? 256 : 128);
+        int const chunk  = ((frames + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
         int const chunk_count = ceil_div(c.frame_size, chunk);
         int const in_tiles    = ceil_div(c.input_node_size, kWavesPerBlk);
         if ((long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }

@@ -485,6 +485,8 @@ struct TermArgs {
     unsigned long long x_base, x_row_pitch_bytes, dy_base, dy_row_pitch_bytes;
     int lut_binarize, rev_stride, input_node_size;
     int blocks;                 // workgroups that build records (kWavesPerBlk records each); 0 = nothing to build
+    int corner;                 // 1: records hold the derivative's corner values for two-valued inputs (lut_dx_corner_kernel)
+    float lo, hi;               //    the two input values, 1/2 -+ bias
 };
 
 // one wavefront per record: lane i holds entry i of the consumer's table while it is brought into the plain basis.
@@ -519,7 +521,10 @@ __device__ __forceinline__ void term_table_block(TermArgs const &a, int block)
         out[lane] = v;
     }
 
-    // P = plain-basis coefficients of W' (W' = lut_binarize ? W > 0.5 : W): the butterfly (a, b) -> (a, b - a) per index bit
+    // P = plain-basis coefficients of W' (W' = lut_binarize ? W > 0.5 : W): the butterfly (a, b) -> (a, b - a) per index bit.
+    // For two-valued inputs the record holds values instead of coefficients: dy/dx_k at the corner where every other
+    // input j takes lo or hi.  W' is the table of y at x in {0, 1}^N and y is linear in each input, so input j != k
+    // interpolates, (a, b) -> (a + lo (b - a), a + hi (b - a)), and input k differentiates, (a, b) -> (., b - a).
     float v = 0.0f;
     if (lane < NN) {
         v = a.W[(size_t)node * NN + lane];
@@ -527,8 +532,15 @@ __device__ __forceinline__ void term_table_block(TermArgs const &a, int block)
     }
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-        float const o = __shfl_xor(v, 1 << j, 64);
-        v = ((lane >> j) & 1) ? (v - o) : v;
+        float const o   = __shfl_xor(v, 1 << j, 64);
+        bool const  up  = (lane >> j) & 1;
+        if (a.corner && j != k) {
+            float const lower = up ? o : v, step = up ? (v - o) : (o - v);
+            v = __builtin_fmaf(up ? a.hi : a.lo, step, lower);
+        }
+        else {
+            v = up ? (v - o) : v;
+        }
     }
     if (lane < NN && ((lane >> k) & 1)) {
         int const sidx = (lane & ((1 << k) - 1)) | ((lane >> (k + 1)) << k);      // the entry's index with bit k taken out
@@ -907,6 +919,77 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
             T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
             T::load_coefficients(rec + (size_t)t * T::REC, Dk);
             T::accumulate(st, Dk, bit, lo, hi, acc);
+        }
+
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int const f = f_begin + u * kWave + lane;
+            if (f < a.frame_size) { __builtin_nontemporal_store(acc[u], a.dx + (size_t)in * a.dx_stride + f); }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  Input-centric dx for two-valued inputs (packed bits, fp32 binarized at 0.5).  A term's dy/dx_k is one of 2^(N-1)
+//  values, chosen by the other inputs' bits: the term record holds that table (term_table_block with corner = 1), lane p
+//  keeps entry p, and a lane fetches the entry of its frame with ds_bpermute.  The index is assembled two instructions
+//  per input (the input's bit rotated into place, then merged): 2 (N - 1) + 2 vector instructions per term and step instead
+//  of the polynomial's 43.  Units, work list, loads and the dW rider are those of lut_dx_kernel.
+// ------------------------------------------------------------------------------------------------
+template <int N, int XMODE, int U>
+__global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
+{
+    static_assert(XMODE == kXBit || XMODE == kXBinary, "corner values need two-valued inputs");
+    using T = DxTerm<N, XMODE, U>;
+    int const bid = blockIdx.x;
+    int const B   = a.chunk_count * a.tiles.count;
+    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B); return; }
+    int const lid  = xcd_remap(bid, B);
+    int ck, tile;
+    split_tile(lid, a.tiles, ck, tile);
+    int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
+    if (in >= a.input_node_size) { return; }
+    int const lane = threadIdx.x & (kWave - 1);
+
+    int const cnt = a.rev[(size_t)in * a.rev_stride];
+    typedef __attribute__((address_space(4))) int const const_int;
+    const_int *rec = (const_int *)(a.term + (size_t)in * (a.rev_stride - 1) * T::REC);
+    int const *rec_v = a.term + (size_t)in * (a.rev_stride - 1) * T::REC + kTermHead + (lane & (T::HN - 1));
+    uint32_t const y_row_bytes = (uint32_t)a.frame_size * 4u;
+    uint32_t const x_row_bytes = (XMODE == kXBit) ? (uint32_t)((a.frame_size + 31) >> 5) * 4u : y_row_bytes;
+    // rotation that brings the lane's frame bit of a packed word to bit j + 2 of the byte index
+    uint32_t rot[T::M];
+#pragma unroll
+    for (int j = 0; j < T::M; ++j) { rot[j] = (uint32_t)((lane & 31) - (j + 2)) & 31u; }
+
+    for (int f_begin = ck * a.chunk; f_begin < min((ck + 1) * a.chunk, a.frame_size); f_begin += kWave * U) {
+        uint32_t const f0   = (uint32_t)(f_begin + lane);
+        uint32_t const yoff = f0 * 4u;
+        uint32_t const xoff = (XMODE == kXBit) ? (f0 >> 5) * 4u : yoff;
+        float acc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
+
+        for (int t = 0; t < cnt; ++t) {
+            int const values = rec_v[(size_t)t * T::REC];          // lane p: the term's value at corner p
+            typename T::Stage st;
+            T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                uint32_t index = 0;
+#pragma unroll
+                for (int j = 0; j < T::M; ++j) {
+                    if constexpr (XMODE == kXBit) {
+                        uint32_t const r = __builtin_amdgcn_alignbit(st.raw[u][j], st.raw[u][j], rot[j]);
+                        index = (r & (4u << j)) | index;
+                    }
+                    else {
+                        index |= (__uint_as_float(st.raw[u][j]) > 0.5f) ? (4u << j) : 0u;
+                    }
+                }
+                float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index, values));
+                acc[u] = __builtin_fmaf(st.dyv[u], d, acc[u]);
+            }
         }
 
 #pragma unroll
