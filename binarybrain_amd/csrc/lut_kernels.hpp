@@ -325,6 +325,39 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 }
 
 // ------------------------------------------------------------------------------------------------
+//  helpers of the kernels for two-valued inputs
+// ------------------------------------------------------------------------------------------------
+// lane masks of four wavefront-steps (256 frames from fb, a multiple of 256) of N packed rows: one 32-byte scalar load per row
+template <int N>
+__device__ __forceinline__ void corner_masks_wide(void const *(&rows)[N], int fb, uint64_t (&raw)[4][N])
+{
+    typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(4))) u32x8 const const_u32x8;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        u32x8 const w = *(const_u32x8 *)(reinterpret_cast<uint32_t const *>(rows[k]) + (fb >> 5));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { raw[u][k] = (uint64_t)w[2 * u] | ((uint64_t)w[2 * u + 1] << 32); }
+    }
+}
+
+// corner index of the lane's frame, most significant input first: index = 2 index + bit, one add-with-carry per input
+// with the input's lane mask as the carry
+template <int N, int XMODE, typename Raw>
+__device__ __forceinline__ uint32_t corner_index(Raw const (&raw)[N])
+{
+    uint32_t index = 0;
+#pragma unroll
+    for (int k = N - 1; k >= 0; --k) {
+        uint64_t mask, carry;
+        if constexpr (XMODE == kXBit) { mask = raw[k]; }
+        else                          { mask = __ballot(__uint_as_float(raw[k]) > 0.5f); }
+        asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(index), "=s"(carry) : "v"(index), "s"(mask));
+    }
+    return index;
+}
+
+// ------------------------------------------------------------------------------------------------
 //  Forward for two-valued inputs (packed bits, or fp32 frames binarized at 0.5): the LUT output is one of the 2^N corner
 //  values V of the node.  A lane builds the corner index of its frame from the N input bits (one add-with-carry per input:
 //  index = 2 index + bit, the bit arriving as a lane mask in a scalar register pair) and fetches V[index] from the lane
@@ -368,16 +401,7 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
         typename Gather<N, XMODE>::Raw raw[U][N];
         float dyv[U];
-        if constexpr (WIDE) {
-            typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
-            typedef __attribute__((address_space(4))) u32x8 const const_u32x8;
-#pragma unroll
-            for (int k = 0; k < N; ++k) {
-                u32x8 const w = *(const_u32x8 *)(reinterpret_cast<uint32_t const *>(rows[k]) + (fb >> 5));     // fb is a multiple of 256
-#pragma unroll
-                for (int u = 0; u < U; ++u) { raw[u][k] = (uint64_t)w[2 * u] | ((uint64_t)w[2 * u + 1] << 32); }
-            }
-        }
+        if constexpr (WIDE) { corner_masks_wide<N>(rows, fb, raw); }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
@@ -391,15 +415,7 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
             if (f0 >= f_end) { break; }
             int const  f  = f0 + lane;
             bool const ok = f < f_end;
-            // corner index, most significant input first: index = 2 index + bit
-            uint32_t index = 0;
-#pragma unroll
-            for (int k = N - 1; k >= 0; --k) {
-                uint64_t mask, carry;
-                if constexpr (XMODE == kXBit) { mask = raw[u][k]; }
-                else                          { mask = __ballot(__uint_as_float(raw[u][k]) > 0.5f); }
-                asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(index), "=s"(carry) : "v"(index), "s"(mask));
-            }
+            uint32_t const index = corner_index<N, XMODE>(raw[u]);
             float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), corner));
             forward_stage<YMODE, FWD_KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
                                            (FWD_KIND == 3) ? dyv[u] : 0.0f, s1, s2);
