@@ -97,6 +97,8 @@ bool use_corner_values(int xmode)
     return on == 1 && (xmode == kXBit || xmode == kXBinary);
 }
 
+bool pack_binarized_input(void) { static int const on = env_int("BBHIP_PACK", 1); return on == 1; }
+
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); return v >= 2 ? 2 : 1; }
 // Frames per forward unit.  fp32 rows are gathered through L2, and a 256-frame piece of every input row is what one XCD's L2
@@ -408,11 +410,21 @@ int check_backward(BackwardCall const &c, int dxmode)
 }
 
 template <int N>
-int run_backward(BackwardCall const &c, hipStream_t st)
+int run_backward(BackwardCall const &call, hipStream_t st)
 {
     constexpr int NN = 1 << N;
     int const dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
-    if (check_backward(c, dxmode)) { return 1; }
+    if (check_backward(call, dxmode)) { return 1; }
+
+    // fp32 frames that the layer binarizes at 0.5 are packed to bits once (reading them once costs less than the three
+    // kernels of this pass gain from packed rows); from here on the call is a packed-bit call
+    BackwardCall c = call;
+    bool const pack = (c.xmode == kXBinary) && dxmode == kDxNone && use_corner_values(kXBinary) && pack_binarized_input();
+    if (pack) {
+        int pack_stride = (((c.frame_size + 31) / 32) + 7) & ~7;
+        if ((pack_stride * 4) % 2048 == 0) { pack_stride += 96; }      // keep the row pitch off the multiples of 2 KiB
+        c.xmode = kXBit; c.x_stride = pack_stride; c.x = nullptr;      // the packed rows get their place in the arena below
+    }
 
     int const tile_count = ceil_div(c.output_node_size, kWavesPerBlk);
     int const range      = (dxmode == kDxTmp) ? (c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size) : c.frame_size;
@@ -451,9 +463,21 @@ int run_backward(BackwardCall const &c, hipStream_t st)
     size_t const dtab_bytes = align256(term_count * sizeof(int));
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     size_t const v_bytes = corner ? c_bytes : 0;
+    size_t const bits_bytes = pack ? align256((size_t)c.input_node_size * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes, &base)) { return 1; }
     float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
+    if (pack) {
+        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes);
+        for (int n0 = 0; n0 < c.input_node_size; n0 += 65535) {        // grid.y is limited to 65535 rows per launch
+            int const rows = (c.input_node_size - n0 < 65535) ? c.input_node_size - n0 : 65535;
+            hipLaunchKernelGGL(binarize_pack_kernel, dim3(ceil_div(c.x_stride * 32, kBlock), rows), dim3(kBlock), 0, st,
+                               reinterpret_cast<float const *>(call.x) + (size_t)n0 * call.x_stride, bits + (size_t)n0 * c.x_stride,
+                               c.frame_size, call.x_stride, c.x_stride);
+        }
+        BBHIP_LAUNCH_CHECK();
+        c.x = bits;
+    }
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);

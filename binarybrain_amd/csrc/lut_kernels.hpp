@@ -1071,6 +1071,21 @@ __global__ __launch_bounds__(kBlock) void clamp_kernel(float *__restrict__ dst, 
     if (i < size) { dst[i] = fminf(hi, fmaxf(lo, src[i])); }
 }
 
+// fp32 frames -> packed bits, bit = x > 0.5 (the binarization of binary mode, include/bb/StochasticLutN.h:539): one lane per
+// frame, a wavefront writes two words.  Rows of `bits` are y_stride words long; bits beyond the last frame are 0.
+__global__ __launch_bounds__(kBlock) void binarize_pack_kernel(float const *__restrict__ x, uint32_t *__restrict__ bits,
+                                                               int frame_size, int x_stride, int y_stride)
+{
+    int const f    = blockIdx.x * kBlock + threadIdx.x;
+    int const node = blockIdx.y;
+    bool const on  = (f < frame_size) && (x[(size_t)node * x_stride + (f < frame_size ? f : 0)] > 0.5f);
+    uint64_t const m = __ballot(on);
+    int const lane = threadIdx.x & (kWave - 1);
+    int const w = (f & ~(kWave - 1)) >> 5;                 // first word of the wavefront's 64 frames
+    if (lane == 0  && w     < y_stride) { bits[(size_t)node * y_stride + w]     = (uint32_t)m; }
+    if (lane == 32 && w + 1 < y_stride) { bits[(size_t)node * y_stride + w + 1] = (uint32_t)(m >> 32); }
+}
+
 // packed bits -> fp32 values (reference: cuda/ConvBitToReal.cu, include/bb/FrameBuffer.h:850-866)
 __global__ __launch_bounds__(kBlock) void conv_bit_to_real_kernel(uint32_t const *__restrict__ x, float *__restrict__ y, float v0, float v1,
                                                                  int frame_size, int x_stride, int y_stride)
