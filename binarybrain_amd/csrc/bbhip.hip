@@ -471,9 +471,16 @@ int run_backward(BackwardCall const &call, hipStream_t st)
         uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes);
         for (int n0 = 0; n0 < c.input_node_size; n0 += 65535) {        // grid.y is limited to 65535 rows per launch
             int const rows = (c.input_node_size - n0 < 65535) ? c.input_node_size - n0 : 65535;
-            hipLaunchKernelGGL(binarize_pack_kernel, dim3(ceil_div(c.x_stride * 32, kBlock), rows), dim3(kBlock), 0, st,
-                               reinterpret_cast<float const *>(call.x) + (size_t)n0 * call.x_stride, bits + (size_t)n0 * c.x_stride,
-                               c.frame_size, call.x_stride, c.x_stride);
+            float const *src = reinterpret_cast<float const *>(call.x) + (size_t)n0 * call.x_stride;
+            uint32_t *dst = bits + (size_t)n0 * c.x_stride;
+            if (call.x_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(call.x) & 15u) == 0) {
+                hipLaunchKernelGGL(binarize_pack4_kernel, dim3(ceil_div(c.x_stride * 8, kBlock), rows), dim3(kBlock), 0, st,
+                                   src, dst, c.frame_size, call.x_stride, c.x_stride);
+            }
+            else {
+                hipLaunchKernelGGL(binarize_pack_kernel, dim3(ceil_div(c.x_stride * 32, kBlock), rows), dim3(kBlock), 0, st,
+                                   src, dst, c.frame_size, call.x_stride, c.x_stride);
+            }
         }
         BBHIP_LAUNCH_CHECK();
         c.x = bits;

@@ -1086,6 +1086,28 @@ __global__ __launch_bounds__(kBlock) void binarize_pack_kernel(float const *__re
     if (lane == 32 && w + 1 < y_stride) { bits[(size_t)node * y_stride + w + 1] = (uint32_t)(m >> 32); }
 }
 
+// the same with four frames per lane (16-byte loads; rows 16-byte aligned, x_stride a multiple of 4): a lane's four bits
+// are shifted to their place in the word that eight neighbouring lanes share and the eight are combined by three exchanges
+__global__ __launch_bounds__(kBlock) void binarize_pack4_kernel(float const *__restrict__ x, uint32_t *__restrict__ bits,
+                                                                int frame_size, int x_stride, int y_stride)
+{
+    int const q    = blockIdx.x * kBlock + threadIdx.x;     // group of four frames
+    int const node = blockIdx.y;
+    int const f    = q * 4;
+    uint32_t v = 0;
+    if (f < frame_size) {
+        float4 const t = *reinterpret_cast<float4 const *>(x + (size_t)node * x_stride + f);
+        v = (t.x > 0.5f ? 1u : 0u) | ((f + 1 < frame_size && t.y > 0.5f) ? 2u : 0u) |
+            ((f + 2 < frame_size && t.z > 0.5f) ? 4u : 0u) | ((f + 3 < frame_size && t.w > 0.5f) ? 8u : 0u);
+    }
+    v <<= 4 * (threadIdx.x & 7);
+    v |= __shfl_xor(v, 1, 64);
+    v |= __shfl_xor(v, 2, 64);
+    v |= __shfl_xor(v, 4, 64);
+    int const w = q >> 3;
+    if ((threadIdx.x & 7) == 0 && w < y_stride) { bits[(size_t)node * y_stride + w] = v; }
+}
+
 // packed bits -> fp32 values (reference: cuda/ConvBitToReal.cu, include/bb/FrameBuffer.h:850-866)
 __global__ __launch_bounds__(kBlock) void conv_bit_to_real_kernel(uint32_t const *__restrict__ x, float *__restrict__ y, float v0, float v1,
                                                                  int frame_size, int x_stride, int y_stride)

@@ -121,6 +121,23 @@ def test_bit_input_row_pitches(ops, extra_words):
     assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
 
 
+@pytest.mark.parametrize("stride", [1001, 1002, 1004])
+def test_binarized_input_row_pitches(ops, stride):
+    """binary mode on fp32 frames: the backward pass packs the binarized input, four frames per lane where the row pitch
+    allows 16-byte loads and frame by frame elsewhere: same results"""
+    rng = np.random.default_rng(400 + stride)
+    I, O, F = 40, 24, 1000
+    idx = synth.wiring(rng, I, O, 6); W = synth.lut_tables(rng, O, 6)
+    x = synth.uniform_frames(rng, I, F, stride); dy = synth.normal_frames(rng, O, F, stride)
+    y_ref = oracle.stochastic_lut_forward(6, x, idx, W, F, 1, 0, 0.25, False)
+    dx_ref, dW_ref = oracle.stochastic_lut_backward(6, x, dy, idx, W, F, None, 1, 0, 0.25, False)
+    y = ops.stochastic_lut_forward(6, dev(x), dev(idx), dev(W), F, True, False)
+    assert_fwd(host(y)[:, :F], y_ref[:, :F])
+    dW = dev(np.zeros((O, 64), np.float32))
+    dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, ops.reverse_table(dev(idx), I), True, False)
+    assert_bwd(host(dx)[:, :F], dx_ref[:, :F]); assert_bwd(host(dW), dW_ref)
+
+
 def test_golden_vectors_on_gpu(ops):
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "stochastic_lut.npz"))
     for k in range(int(g["count"][0])):
