@@ -1,0 +1,20 @@
+"""The kernels behind the environment switches.  The library reads its switches once per process, so each setting runs the
+same parity case (tests/two_valued_case.py) in one child process: the default (lookup kernels for two-valued inputs,
+packed backward pass) and the polynomial kernels for the same inputs."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.mark.parametrize("env", [{}, {"BBHIP_CORNER": "2", "BBHIP_PACK": "2"}, {"BBHIP_PACK": "2"}, {"BBHIP_FWD_NODES": "1", "BBHIP_BWD_SLAB": "256"}])
+def test_two_valued_inputs_under_switches(env):
+    child_env = dict(os.environ)
+    child_env.update(env)
+    child_env["PYTHONPATH"] = os.pathsep.join([os.path.dirname(HERE), HERE, child_env.get("PYTHONPATH", "")])
+    p = subprocess.run([sys.executable, os.path.join(HERE, "two_valued_case.py")], env=child_env, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0 and "two-valued case ok" in p.stdout, (env, p.stdout[-2000:], p.stderr[-2000:])
