@@ -243,6 +243,43 @@ def test_full_size_properties(ops):
     assert_bwd(host(dxb)[:, :fs], dx_ref)
 
 
+def test_full_size_properties_packed_bits(ops):
+    """4096 -> 4096 nodes, 8192 frames of packed bits (the lookup kernels for two-valued inputs at their full shape): a slice of
+    nodes and a slice of frames against the oracle, the fp32 entry point on the unpacked 0/1 frames in binary mode, linearity"""
+    import torch
+    rng = np.random.default_rng(43)
+    I = O = 4096; F = 8192
+    idx = synth.wiring(rng, I, O); W = synth.lut_tables(rng, O)
+    xs = synth.frame_stride_bit(F); ys = synth.frame_stride_fp32(F)
+    xb = synth.bernoulli_bits(rng, I, F, xs); dy = synth.normal_frames(rng, O, F, ys)
+    xd, dyd, idxd, Wd = dev(xb), dev(dy), dev(idx), dev(W)
+    ops.set_dx_mode(0)
+    y = ops.bit_stochastic_lut_forward(6, xd, idxd, Wd, F, ys, 0)
+    sel = np.arange(0, O, 64)
+    assert_fwd(host(y)[sel][:, :F], oracle.bit_stochastic_lut_forward(6, xb, idx[sel], W[sel], F, ys, 0)[:, :F])
+    rev = ops.reverse_table(idxd, I)
+    dW = torch.zeros((O, 64), device="cuda")
+    dx = ops.bit_stochastic_lut_backward(6, xd, dyd, idxd, Wd, dW, F, rev, 0)
+    s = dy[:, :F].astype(np.float64).sum(1)
+    assert np.abs(host(dW).astype(np.float64).sum(1) - s).max() <= 1e-4 * np.abs(s).max()
+    _, dW_ref = oracle.bit_stochastic_lut_backward(6, xb, dy[sel], idx[sel], W[sel], F, None, 0)
+    assert_bwd(host(dW)[sel], dW_ref)
+    # the same frames as fp32 0 / 1 values through the fp32 entry points in binary mode
+    xf = np.zeros((I, ys), np.float32); xf[:, :F] = synth.unpack_bits(xb, F)
+    yf = ops.stochastic_lut_forward(6, dev(xf), idxd, Wd, F, True, False)
+    assert rel_err(host(yf)[:, :F], host(y)[:, :F]) <= 1e-6
+    dWf = torch.zeros((O, 64), device="cuda")
+    dxf = ops.stochastic_lut_backward(6, dev(xf), dyd, idxd, Wd, dWf, F, rev, True, False)
+    assert rel_err(host(dxf)[:, :F], host(dx)[:, :F]) <= 1e-6 and rel_err(host(dWf), host(dW)) <= 1e-6
+    # linear in dy, and a slice of frames against the oracle
+    dWc = torch.zeros((O, 64), device="cuda")
+    dxc = ops.bit_stochastic_lut_backward(6, xd, (dyd * 2.0).contiguous(), idxd, Wd, dWc, F, rev, 0)
+    assert rel_err(host(dxc), 2.0 * host(dx)) <= 1e-6
+    fs = 256
+    dx_ref, _ = oracle.bit_stochastic_lut_backward(6, np.ascontiguousarray(xb[:, :fs // 32]), np.ascontiguousarray(dy[:, :fs]), idx, W, fs, None, 0)
+    assert_bwd(host(dx)[:, :fs], dx_ref)
+
+
 def _adversarial_tables(n):
     """Tables whose monomial coefficients are as large as a [0,1] table allows: parity, AND, OR, single spikes."""
     nn = 1 << n
