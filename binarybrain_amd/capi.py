@@ -31,6 +31,7 @@ _SIGNATURES = {
     "bbhip_KernelTimer_Enable": (None, [_i]),
     "bbhip_KernelTimer_Read": (C.c_int, [_i, C.POINTER(C.c_float), C.POINTER(C.c_int)]),
     "bbhip_SetDxMode": (None, [_i]),
+    "bbhip_HintInputNodeSize": (None, [_i]),
     "bbhip_GetDxMode": (C.c_int, []),
     "bbhip_fp32_Vector_set": (C.c_int, [_vp, _f, _i, _vp]),
     "bbhip_fp32_Vector_clamp": (C.c_int, [_vp, _vp, _f, _f, _i, _vp]),

@@ -56,6 +56,7 @@ int fail(char const *fmt, ...)
 // ------------------------------------------------------------------------------------------------
 bool g_host_only = false;
 int  g_dx_mode   = 0;
+thread_local int g_input_node_hint = 0;      // bbhip_HintInputNodeSize: rows of the next forward call's input, 0 = unknown
 
 // ------------------------------------------------------------------------------------------------
 //  optional kernel timer: HIP events around the dominant kernel of each entry point, on the launch stream
@@ -211,6 +212,8 @@ int dispatch_forward(int xmode, int ymode, int kind, FwdArgs const &a, int npw, 
     BBHIP_FWD_CASE(kXClamp,  kYClamp,    1)
     BBHIP_FWD_CASE(kXBinary, kYBinarize, 1)
     BBHIP_FWD_CASE(kXBit,    kYBit,      1)
+    BBHIP_FWD_CASE(kXBit,    kYBinarize, 0)         // fp32 frames of binary mode, packed by the library
+    BBHIP_FWD_CASE(kXBit,    kYBinarize, 1)
     BBHIP_FWD_CASE(kXClamp,  kYClamp,    2)
     BBHIP_FWD_CASE(kXBinary, kYClamp,    2)
     BBHIP_FWD_CASE(kXBit,    kYClamp,    2)
@@ -303,10 +306,44 @@ int check_forward(ForwardCall const &c)
 // workgroup's threads share one node
 int stat_nodes_per_block(int unit_count) { return unit_count >= 512 ? 4 : unit_count >= 64 ? 16 : 64; }
 
+// row pitch (words) of the library's packed copy of `frame_size` binarized frames
+int packed_row_words(int frame_size)
+{
+    int words = (((frame_size + 31) / 32) + 7) & ~7;
+    if ((words * 4) % 2048 == 0) { words += 96; }          // keep the row pitch off the multiples of 2 KiB
+    return words;
+}
+
+// fp32 frames -> packed bits (bit = x > 0.5) for `node_size` rows
+int launch_binarize_pack(float const *x, int x_stride, uint32_t *bits, int bit_stride, int node_size, int frame_size, hipStream_t st)
+{
+    for (int n0 = 0; n0 < node_size; n0 += 65535) {        // grid.y is limited to 65535 rows per launch
+        int const rows = (node_size - n0 < 65535) ? node_size - n0 : 65535;
+        float const *src = x + (size_t)n0 * x_stride;
+        uint32_t *dst = bits + (size_t)n0 * bit_stride;
+        if (x_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+            hipLaunchKernelGGL(binarize_pack4_kernel, dim3(ceil_div(bit_stride * 8, kBlock), rows), dim3(kBlock), 0, st,
+                               src, dst, frame_size, x_stride, bit_stride);
+        }
+        else {
+            hipLaunchKernelGGL(binarize_pack_kernel, dim3(ceil_div(bit_stride * 32, kBlock), rows), dim3(kBlock), 0, st,
+                               src, dst, frame_size, x_stride, bit_stride);
+        }
+    }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 template <int N>
-int run_forward(ForwardCall const &c, hipStream_t st)
+int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
 {
     constexpr int NN = 1 << N;
+    // input_rows: what the caller said about the input's row count (bbhip_HintInputNodeSize), 0 = nothing.
+    // fp32 frames that the layer binarizes at 0.5 are packed to bits once where the row count is known; from here on the
+    // call is a packed-bit call (same outputs)
+    ForwardCall c = call;
+    bool const pack = (c.xmode == kXBinary) && input_rows > 0 && use_corner_values(kXBinary) && pack_binarized_input();
+    if (pack) { c.xmode = kXBit; c.x_stride = packed_row_words(c.frame_size); c.x = nullptr; }
     bool const corner     = use_corner_values(c.xmode);
     int const npw         = corner ? 1 : fwd_nodes_per_wave();
     int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
@@ -318,8 +355,14 @@ int run_forward(ForwardCall const &c, hipStream_t st)
     size_t const v_bytes    = corner ? c_bytes : 0;
     size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
     size_t const rstd_bytes = (c.bn == 2) ? align256((size_t)c.node_size * sizeof(float)) : 0;
+    size_t const bits_bytes = pack ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + v_bytes + stat_bytes + rstd_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + v_bytes + stat_bytes + rstd_bytes + bits_bytes, &base)) { return 1; }
+    if (pack) {
+        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes + rstd_bytes);
+        if (launch_binarize_pack(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size, st)) { return 1; }
+        c.x = bits;
+    }
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
@@ -365,9 +408,11 @@ int run_forward(ForwardCall const &c, hipStream_t st)
 
 int forward_entry(ForwardCall const &c, void *stream)
 {
+    int const input_rows = g_input_node_hint;       // the hint is spent by this call, whatever becomes of it
+    g_input_node_hint = 0;
     if (check_forward(c)) { return 1; }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, st));
+    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st));
     return 0;
 }
 
@@ -420,11 +465,7 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     // kernels of this pass gain from packed rows); from here on the call is a packed-bit call
     BackwardCall c = call;
     bool const pack = (c.xmode == kXBinary) && dxmode == kDxNone && use_corner_values(kXBinary) && pack_binarized_input();
-    if (pack) {
-        int pack_stride = (((c.frame_size + 31) / 32) + 7) & ~7;
-        if ((pack_stride * 4) % 2048 == 0) { pack_stride += 96; }      // keep the row pitch off the multiples of 2 KiB
-        c.xmode = kXBit; c.x_stride = pack_stride; c.x = nullptr;      // the packed rows get their place in the arena below
-    }
+    if (pack) { c.xmode = kXBit; c.x_stride = packed_row_words(c.frame_size); c.x = nullptr; }      // the packed rows get their place in the arena below
 
     int const tile_count = ceil_div(c.output_node_size, kWavesPerBlk);
     int const range      = (dxmode == kDxTmp) ? (c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size) : c.frame_size;
@@ -469,20 +510,7 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
     if (pack) {
         uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes);
-        for (int n0 = 0; n0 < c.input_node_size; n0 += 65535) {        // grid.y is limited to 65535 rows per launch
-            int const rows = (c.input_node_size - n0 < 65535) ? c.input_node_size - n0 : 65535;
-            float const *src = reinterpret_cast<float const *>(call.x) + (size_t)n0 * call.x_stride;
-            uint32_t *dst = bits + (size_t)n0 * c.x_stride;
-            if (call.x_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(call.x) & 15u) == 0) {
-                hipLaunchKernelGGL(binarize_pack4_kernel, dim3(ceil_div(c.x_stride * 8, kBlock), rows), dim3(kBlock), 0, st,
-                                   src, dst, c.frame_size, call.x_stride, c.x_stride);
-            }
-            else {
-                hipLaunchKernelGGL(binarize_pack_kernel, dim3(ceil_div(c.x_stride * 32, kBlock), rows), dim3(kBlock), 0, st,
-                                   src, dst, c.frame_size, call.x_stride, c.x_stride);
-            }
-        }
-        BBHIP_LAUNCH_CHECK();
+        if (launch_binarize_pack(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, c.input_node_size, c.frame_size, st)) { return 1; }
         c.x = bits;
     }
     float *C    = reinterpret_cast<float *>(base);
@@ -817,6 +845,7 @@ int bbhip_KernelTimer_Read(int which, float *total_ms, int *launches)
 }
 
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
+void bbhip_HintInputNodeSize(int input_node_size) { g_input_node_hint = input_node_size > 0 ? input_node_size : 0; }
 int  bbhip_GetDxMode(void) { return g_dx_mode; }
 
 int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)

@@ -252,6 +252,7 @@ public:
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTraining");
             }
             else {
+                bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTraining(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
                                 (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
@@ -268,6 +269,7 @@ public:
                             "bbhip_bit_fp32_DifferentiableLutN_ForwardInference");
             }
             else {
+                bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardInference(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float const *)rm_ptr.GetAddr(), (float const *)rv_ptr.GetAddr(),
                                 m_gamma, m_beta, m_unbinarize_bias, O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr),
@@ -280,6 +282,7 @@ public:
                             m_lut_binarize ? 1 : 0, m_unbinarize_bias, nullptr), "bbhip_bit_bit_fp32_StochasticLut_Forward");
         }
         else {
+            bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
             CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardNoBn(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                             (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), m_unbinarize_bias, O, F, y_stride,
                             m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_ForwardNoBn");

@@ -204,6 +204,7 @@ public:
         }
         else {
             BB_ASSERT(x_buf.GetFrameStride() == y_buf.GetFrameStride());
+            bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
             CheckDevice(bbhip_fp32_StochasticLut_Forward(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                             (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(),
                             (int)y_buf.GetNodeSize(), (int)y_buf.GetFrameSize(), (int)(y_buf.GetFrameStride() / sizeof(float)),

@@ -247,6 +247,7 @@ def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_bin
     _dev(x, idx, W, out)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
+    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
     check(lib().bbhip_fp32_StochasticLut_Forward(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, frame_size, x.shape[1],
                                                  int(input_binary), int(lut_binarize), bias, stream_ptr()))
     return y
@@ -326,6 +327,7 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
     mean = torch.empty(O, dtype=torch.float32, device=x.device)
     rstd = torch.empty(O, dtype=torch.float32, device=x.device)
+    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardTraining(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                               ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
                                                               O, frame_size, x.shape[1], int(lut_binarize), int(binary_mode),
@@ -351,6 +353,7 @@ def differentiable_lut_forward_inference(n, x, idx, W, frame_size, running_mean,
     _dev(x, idx, W, running_mean, running_var)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardInference(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(running_mean),
                                                                ptr(running_var), gamma, beta, bias, O, frame_size, x.shape[1],
                                                                int(lut_binarize), int(binary_mode), stream_ptr()))
@@ -372,6 +375,7 @@ def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_bin
     _dev(x, idx, W)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardNoBn(n, ptr(x), ptr(y), ptr(idx), ptr(W), bias, O, frame_size, x.shape[1],
                                                           int(lut_binarize), int(binary_mode), stream_ptr()))
     return y

@@ -69,6 +69,15 @@ int bbhip_DeviceSynchronize(void);
 void bbhip_SetDxMode(int mode);
 int  bbhip_GetDxMode(void);
 
+/* ---- number of input node rows for the next forward call (no counterpart in the reference) ----
+ * The forward entry points keep the reference's signatures, which do not say how many rows the input buffer has
+ * (input_index names them).  A caller that knows may say so right before a forward call of the same thread: in binary
+ * mode on fp32 frames the library then packs the binarized input to bits once (it has to know how many rows to pack)
+ * and runs the packed-bit kernels, as the backward entry points — which are told input_node_size — always do.
+ * The hint holds for one forward call and is cleared by it; 0 clears it.  The rows [0, input_node_size) of the input
+ * buffer must exist: the value is trusted like the sizes of any entry point.  Results do not depend on the hint. */
+void bbhip_HintInputNodeSize(int input_node_size);
+
 /* ---- kernel timer (instrumentation; no counterpart in the reference) ----
  * While enabled, every call brackets its dominant kernel (which: 0 = LUT forward kernel, 1 = LUT backward kernel,
  * 2 = BinaryLut6 kernel, 3 = input-centric dx kernel, 4 = the kernels of any other entry: vector operations, Adam, Im2Col,
