@@ -948,9 +948,9 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 // ------------------------------------------------------------------------------------------------
 //  Input-centric dx for two-valued inputs (packed bits, fp32 binarized at 0.5).  A term's dy/dx_k is one of 2^(N-1)
 //  values, chosen by the other inputs' bits: the term record holds that table (term_table_block with corner = 1), lane p
-//  keeps entry p, and a lane fetches the entry of its frame with ds_bpermute.  The index is assembled two instructions
-//  per input (the input's bit rotated into place, then merged): 2 (N - 1) + 2 vector instructions per term and step instead
-//  of the polynomial's 43.  Units, work list, loads and the dW rider are those of lut_dx_kernel.
+//  keeps entry p, and a lane fetches the entry of its frame with ds_bpermute: about a dozen vector instructions per term
+//  and step instead of the polynomial's 43.  Units, work list and the dW rider are those of lut_dx_kernel; fp32 rows are
+//  loaded as there and compared with 0.5, packed rows take one load per row and pass (see below).
 // ------------------------------------------------------------------------------------------------
 template <int N, int XMODE, int U>
 __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
@@ -973,36 +973,56 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
     int const *rec_v = a.term + (size_t)in * (a.rev_stride - 1) * T::REC + kTermHead + (lane & (T::HN - 1));
     uint32_t const y_row_bytes = (uint32_t)a.frame_size * 4u;
     uint32_t const x_row_bytes = (XMODE == kXBit) ? (uint32_t)((a.frame_size + 31) >> 5) * 4u : y_row_bytes;
-    // rotation that brings the lane's frame bit of a packed word to bit j + 2 of the byte index
-    uint32_t rot[T::M];
-#pragma unroll
-    for (int j = 0; j < T::M; ++j) { rot[j] = (uint32_t)((lane & 31) - (j + 2)) & 31u; }
 
     for (int f_begin = ck * a.chunk; f_begin < min((ck + 1) * a.chunk, a.frame_size); f_begin += kWave * U) {
         uint32_t const f0   = (uint32_t)(f_begin + lane);
         uint32_t const yoff = f0 * 4u;
         uint32_t const xoff = (XMODE == kXBit) ? (f0 >> 5) * 4u : yoff;
+        uint32_t const wordoff = ((uint32_t)(f_begin >> 5) + (uint32_t)(lane & (2 * U - 1))) * 4u;      // packed rows: word (lane mod 2 U) of the pass
         float acc[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
 
         for (int t = 0; t < cnt; ++t) {
             int const values = rec_v[(size_t)t * T::REC];          // lane p: the term's value at corner p
+            if constexpr (XMODE == kXBit) {
+                // The 64 U frames of a pass are 2 U words of a packed row, the same for every lane: one load per row
+                // brings them in (lane i holds word i of the pass), each step's two words are read back as a lane mask,
+                // and the index costs one add-with-carry per input.  Per term and pass: M + U + 1 vector memory
+                // instructions instead of (M + 1) U + 1.
+                const_int *r = rec + (size_t)t * T::REC;
+                uint32_t w[T::M];
+#pragma unroll
+                for (int j = 0; j < T::M; ++j) {
+                    __amdgpu_buffer_rsrc_t const d = address_descriptor((uint32_t)r[2 * j], (uint32_t)r[2 * j + 1], x_row_bytes);
+                    w[j] = __builtin_amdgcn_raw_buffer_load_b32(d, wordoff, 0, 0);
+                }
+                __amdgpu_buffer_rsrc_t const dyr = address_descriptor((uint32_t)r[2 * T::M], (uint32_t)r[2 * T::M + 1], y_row_bytes);
+                float dyv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) { dyv[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0)); }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t index = 0;                            // most significant input first: index = 2 index + bit
+#pragma unroll
+                    for (int j = T::M - 1; j >= 0; --j) {
+                        uint64_t const mask = (uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)w[j], 2 * u) |
+                                              ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)w[j], 2 * u + 1) << 32);
+                        uint64_t carry;
+                        asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(index), "=s"(carry) : "v"(index), "s"(mask));
+                    }
+                    float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), values));
+                    acc[u] = __builtin_fmaf(dyv[u], d, acc[u]);
+                }
+                continue;
+            }
             typename T::Stage st;
             T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 uint32_t index = 0;
 #pragma unroll
-                for (int j = 0; j < T::M; ++j) {
-                    if constexpr (XMODE == kXBit) {
-                        uint32_t const r = __builtin_amdgcn_alignbit(st.raw[u][j], st.raw[u][j], rot[j]);
-                        index = (r & (4u << j)) | index;
-                    }
-                    else {
-                        index |= (__uint_as_float(st.raw[u][j]) > 0.5f) ? (4u << j) : 0u;
-                    }
-                }
+                for (int j = 0; j < T::M; ++j) { index |= (__uint_as_float(st.raw[u][j]) > 0.5f) ? (4u << j) : 0u; }
                 float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index, values));
                 acc[u] = __builtin_fmaf(st.dyv[u], d, acc[u]);
             }
