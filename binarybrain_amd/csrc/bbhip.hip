@@ -228,6 +228,10 @@ template <int N>
 int dispatch_backward(int xmode, int kind, int dxmode, BwdArgs const &a, hipStream_t st)
 {
     dim3 const grid(a.tt.blocks + a.slab_count * a.tiles.count), block(kBlock);
+    if (xmode == kXBit && kind == 1 && dxmode == kDxNone && a.V != nullptr) {       // batch-norm window from the corner values
+        hipLaunchKernelGGL((lut_backward_kernel<N, kXBit, 1, kDxNone, true>), grid, block, 0, st, a);
+        return 0;
+    }
 #define BBHIP_BWD_CASE(X, K, M) if (xmode == X && kind == K && dxmode == M) { hipLaunchKernelGGL((lut_backward_kernel<N, X, K, M>), grid, block, 0, st, a); return 0; }
     BBHIP_BWD_CASE(kXClamp,  0, kDxAtomic) BBHIP_BWD_CASE(kXClamp,  0, kDxTmp)
     BBHIP_BWD_CASE(kXBinary, 0, kDxAtomic) BBHIP_BWD_CASE(kXBinary, 0, kDxTmp)
@@ -541,7 +545,7 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     }
 
     BwdArgs a{};
-    a.x = c.x; a.dy = c.dy; a.idx = c.idx; a.C = C;
+    a.x = c.x; a.dy = c.dy; a.idx = c.idx; a.C = C; a.V = V;
     a.dw_partial = part;
     a.mean = c.mean; a.rstd = c.rstd; a.dmean = c.dmean_tmp; a.dvar = c.dvar_tmp;
     a.node_size = c.output_node_size; a.frame_size = c.frame_size;

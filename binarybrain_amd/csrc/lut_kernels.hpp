@@ -588,13 +588,17 @@ struct BwdArgs {
     TileDivisor tiles;
     float bias, gamma, beta, inv_frames;
     TermArgs tt;                // kDxNone: the last tt.blocks workgroups of the launch build the dx kernel's term table
+    float const *V;             // [O][2^N] corner values (CORNER variant)
 };
 
 enum DxMode : int { kDxAtomic = 0, kDxTmp = 1, kDxNone = 2 };
 
 // BWD_KIND: 0 = plain LUT backward, 1 = backward through batch-norm (its statistics pass is kind 3 of the forward kernel)
 // DXMODE  : how (whether) the per-connection input gradients leave the kernel
-template <int N, int XMODE, int BWD_KIND, int DXMODE>
+// CORNER (packed bits, batch-norm, dx left to the dx kernel): the LUT output that the batch-norm window needs comes from
+// the node's corner values (index by add-with-carry from the lane masks, ds_bpermute) instead of the 64-term polynomial,
+// and the table leaves the scalar registers.
+template <int N, int XMODE, int BWD_KIND, int DXMODE, bool CORNER = false>
 __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 {
     using D = LutDims<N>;
@@ -616,7 +620,8 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     int const lane = threadIdx.x & (kWave - 1);
 
     // the table itself enters only the batch-norm kinds (the LUT output is recomputed) and the per-connection gradients
-    constexpr bool kNeedTable = (BWD_KIND != 0) || (DXMODE != kDxNone);
+    static_assert(!CORNER || (XMODE == kXBit && BWD_KIND != 0 && DXMODE == kDxNone), "corner values: packed bits, batch-norm, no dx here");
+    constexpr bool kNeedTable = ((BWD_KIND != 0) || (DXMODE != kDxNone)) && !CORNER;
     // (the partial sums stay on the vector ALU here: the matrix unit's operand registers would cost this kernel a wavefront of
     // occupancy, which measured slower; the batch-norm statistics pass, which only recomputes the LUT output, runs in the
     // forward kernel instead)
@@ -625,6 +630,8 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
         LutEval<N>::load_table(a.C + (size_t)node * D::NN, C);
         LutEval<N>::pin_constants(C, cv);
     }
+    int corner = 0;
+    if (CORNER) { corner = __float_as_int(a.V[(size_t)node * D::NN + (lane & (D::NN - 1))]); }      // lane p holds V[p]
     void const *rows[N];
     int ins[N];
 #pragma unroll
@@ -683,7 +690,9 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 
             if (BWD_KIND != 0) {
                 // hard-tanh window on the batch-norm output (reference: DifferentiableLutN.h:1206-1211, 1241-1246)
-                float const v = LutEval<N>::combine(h, q);
+                float v;
+                if constexpr (CORNER) { v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(corner_index<N, XMODE>(raw[u]) << 2), corner)); }
+                else                  { v = LutEval<N>::combine(h, q); }
                 float const t = ((v - mean) * rstd) * a.gamma + a.beta;
                 if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
                 // dL/d(LUT output) (reference: DifferentiableLutN.h:1248-1250)
