@@ -338,6 +338,28 @@ int launch_binarize_pack(float const *x, int x_stride, uint32_t *bits, int bit_s
     return 0;
 }
 
+// packing and table preparation; one launch for both where the packing takes the 16-byte path
+template <int N>
+int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_stride, int rows, int frame_size,
+                         float const *W, float *C, float *V, int node_size, int lut_binarize, float bias, hipStream_t st)
+{
+    int const row_blocks = ceil_div(bit_stride * 8, kBlock);
+    long long const pack_blocks = (long long)rows * row_blocks, prep_blocks = ceil_div(node_size * (1 << N), kBlock);
+    if (x_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && pack_blocks + prep_blocks <= 0x7fffffffLL) {
+        PackPrepArgs a{};
+        a.x = x; a.bits = bits; a.frame_size = frame_size; a.x_stride = x_stride; a.y_stride = bit_stride;
+        a.row_blocks = make_tile_divisor(row_blocks); a.pack_blocks = (int)pack_blocks;
+        a.W = W; a.C = C; a.V = V; a.node_size = node_size; a.lut_binarize = lut_binarize; a.bias = bias;
+        hipLaunchKernelGGL(binarize_pack4_prep_kernel<N>, dim3((unsigned)(pack_blocks + prep_blocks)), dim3(kBlock), 0, st, a);
+        BBHIP_LAUNCH_CHECK();
+        return 0;
+    }
+    if (launch_binarize_pack(x, x_stride, bits, bit_stride, rows, frame_size, st)) { return 1; }
+    launch_table_prep<N>(W, C, node_size, lut_binarize, st, V, bias);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 template <int N>
 int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
 {
@@ -362,18 +384,20 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
     size_t const bits_bytes = pack ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
     if (arena_get(c_bytes + v_bytes + stat_bytes + rstd_bytes + bits_bytes, &base)) { return 1; }
-    if (pack) {
-        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes + rstd_bytes);
-        if (launch_binarize_pack(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size, st)) { return 1; }
-        c.x = bits;
-    }
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
     float *rstd_tmp = reinterpret_cast<float *>(base + c_bytes + v_bytes + stat_bytes);
-
-    launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias);
-    BBHIP_LAUNCH_CHECK();
+    if (pack) {
+        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes + rstd_bytes);
+        if (launch_pack_and_prep<N>(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size,
+                                    c.W, C, V, c.node_size, c.lut_binarize, c.bias, st)) { return 1; }
+        c.x = bits;
+    }
+    else {
+        launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias);
+        BBHIP_LAUNCH_CHECK();
+    }
 
     FwdArgs a{};
     a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C; a.V = V;
@@ -512,11 +536,6 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     char *base = nullptr;
     if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes, &base)) { return 1; }
     float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
-    if (pack) {
-        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes);
-        if (launch_binarize_pack(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, c.input_node_size, c.frame_size, st)) { return 1; }
-        c.x = bits;
-    }
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
     float *stat = reinterpret_cast<float *>(base + c_bytes + part_bytes);
@@ -524,7 +543,18 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
 
     // centred coefficients: needed where the LUT output is recomputed (batch-norm) or per-connection gradients are formed
-    if (c.bn || dxmode != kDxNone) {
+    bool const prep = c.bn || dxmode != kDxNone;
+    if (pack) {
+        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes);
+        float const *src = reinterpret_cast<float const *>(call.x);
+        if (prep) {
+            if (launch_pack_and_prep<N>(src, call.x_stride, bits, c.x_stride, c.input_node_size, c.frame_size,
+                                        c.W, C, V, c.output_node_size, c.lut_binarize, c.bias, st)) { return 1; }
+        }
+        else if (launch_binarize_pack(src, call.x_stride, bits, c.x_stride, c.input_node_size, c.frame_size, st)) { return 1; }
+        c.x = bits;
+    }
+    else if (prep) {
         launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st, V, c.bias);
         BBHIP_LAUNCH_CHECK();
     }

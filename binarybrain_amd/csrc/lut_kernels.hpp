@@ -44,12 +44,11 @@ __device__ __forceinline__ float wave_sum(float v)
 //  For two-valued inputs (x_j = 1/2 -+ bias) the layer is a table of 2^N values, V[p] = y at the corner whose bit j says
 //  which value input j takes: one more butterfly over C, (a, b) -> (a - bias b, a + bias b) per variable.
 template <int N>
-__global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
-                                                           int node_size, int lut_binarize,
-                                                           float *__restrict__ V = nullptr, float bias = 0.0f)
+__device__ __forceinline__ void table_prep_block(float const *__restrict__ W, float *__restrict__ C, int node_size, int lut_binarize,
+                                                 float *__restrict__ V, float bias, int block)
 {
     constexpr int NN = 1 << N;
-    int const t = blockIdx.x * kBlock + threadIdx.x;
+    int const t = block * kBlock + threadIdx.x;
     int const total = node_size * NN;
     float v = 0.0f;
     if (t < total) {
@@ -70,6 +69,14 @@ __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restr
         v = ((i >> j) & 1) ? __builtin_fmaf(bias, v, o) : __builtin_fmaf(-bias, o, v);
     }
     if (t < total) { V[t] = v; }
+}
+
+template <int N>
+__global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
+                                                           int node_size, int lut_binarize,
+                                                           float *__restrict__ V = nullptr, float bias = 0.0f)
+{
+    table_prep_block<N>(W, C, node_size, lut_binarize, V, bias, blockIdx.x);
 }
 
 // dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order)
@@ -1117,11 +1124,10 @@ __global__ __launch_bounds__(kBlock) void binarize_pack_kernel(float const *__re
 
 // the same with four frames per lane (16-byte loads; rows 16-byte aligned, x_stride a multiple of 4): a lane's four bits
 // are shifted to their place in the word that eight neighbouring lanes share and the eight are combined by three exchanges
-__global__ __launch_bounds__(kBlock) void binarize_pack4_kernel(float const *__restrict__ x, uint32_t *__restrict__ bits,
-                                                                int frame_size, int x_stride, int y_stride)
+__device__ __forceinline__ void binarize_pack4_block(float const *__restrict__ x, uint32_t *__restrict__ bits,
+                                                     int frame_size, int x_stride, int y_stride, int node, int block)
 {
-    int const q    = blockIdx.x * kBlock + threadIdx.x;     // group of four frames
-    int const node = blockIdx.y;
+    int const q    = block * kBlock + threadIdx.x;          // group of four frames
     int const f    = q * 4;
     uint32_t v = 0;
     if (f < frame_size) {
@@ -1135,6 +1141,34 @@ __global__ __launch_bounds__(kBlock) void binarize_pack4_kernel(float const *__r
     v |= __shfl_xor(v, 4, 64);
     int const w = q >> 3;
     if ((threadIdx.x & 7) == 0 && w < y_stride) { bits[(size_t)node * y_stride + w] = v; }
+}
+
+__global__ __launch_bounds__(kBlock) void binarize_pack4_kernel(float const *__restrict__ x, uint32_t *__restrict__ bits,
+                                                                int frame_size, int x_stride, int y_stride)
+{
+    binarize_pack4_block(x, bits, frame_size, x_stride, y_stride, blockIdx.y, blockIdx.x);
+}
+
+// Packing and table preparation in one launch: they are independent, and a launch of its own costs each of them more than
+// its work.  Workgroups [0, rows * row_blocks.count) pack, the rest prepare the tables.
+struct PackPrepArgs {
+    float const *x;  uint32_t *bits;  int frame_size, x_stride, y_stride;
+    TileDivisor row_blocks;     // workgroups per packed row
+    int pack_blocks;            // rows * row_blocks.count
+    float const *W;  float *C;  float *V;  int node_size, lut_binarize;  float bias;
+};
+
+template <int N>
+__global__ __launch_bounds__(kBlock) void binarize_pack4_prep_kernel(PackPrepArgs a)
+{
+    int const bid = blockIdx.x;
+    if (bid < a.pack_blocks) {
+        int row, block;
+        split_tile(bid, a.row_blocks, row, block);
+        binarize_pack4_block(a.x, a.bits, a.frame_size, a.x_stride, a.y_stride, row, block);
+        return;
+    }
+    table_prep_block<N>(a.W, a.C, a.node_size, a.lut_binarize, a.V, a.bias, bid - a.pack_blocks);
 }
 
 // packed bits -> fp32 values (reference: cuda/ConvBitToReal.cu, include/bb/FrameBuffer.h:850-866)
