@@ -11,7 +11,9 @@ pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-@pytest.mark.parametrize("env", [{}, {"BBHIP_CORNER": "2", "BBHIP_PACK": "2"}, {"BBHIP_PACK": "2"}, {"BBHIP_FWD_NODES": "1", "BBHIP_BWD_SLAB": "256"}])
+@pytest.mark.parametrize("env", [{}, {"BBHIP_CORNER": "2", "BBHIP_PACK": "2"}, {"BBHIP_PACK": "2"}, {"BBHIP_FWD_NODES": "1", "BBHIP_BWD_SLAB": "256"},
+                                 {"BBHIP_DX_STEPS": "1", "BBHIP_DX_CHUNK": "64", "BBHIP_BIN_NODES": "1", "BBHIP_BIN_CHUNK": "64"},
+                                 {"BBHIP_DX_STEPS": "4", "BBHIP_DX_CHUNK": "512", "BBHIP_FWD_CHUNK": "512", "BBHIP_BIN_NODES": "2", "BBHIP_BIN_CHUNK": "256"}])
 def test_two_valued_inputs_under_switches(env):
     child_env = dict(os.environ)
     child_env.update(env)

@@ -1,5 +1,5 @@
 """One parity case on two-valued inputs (packed bits, and fp32 frames in binary mode), forward and backward, StochasticLut and
-DifferentiableLut, against the CPU oracle.  Run as a script by test_gpu_tunables.py in a process of its own, because the
+DifferentiableLut, plus continuous fp32 frames and BinaryLut6, against the CPU oracle.  Run as a script by test_gpu_tunables.py in a process of its own, because the
 library reads its environment switches once: with BBHIP_CORNER=2 BBHIP_PACK=2 the polynomial kernels serve these inputs."""
 import sys
 
@@ -40,6 +40,20 @@ def main():
     dW = dev(np.zeros((O, 64), np.float32))
     dx = ops.differentiable_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, dev(m_ref), dev(r_ref), rev)
     assert_bwd(host(dx)[:, :F], dx_ref[:, :F], "binary dx"); assert_bwd(host(dW), dW_ref, "binary dW")
+    # continuous fp32 frames (the polynomial kernels under whatever unit sizes the environment sets)
+    xc = synth.uniform_frames(rng, I, F, ys, -0.1, 1.1)
+    assert_fwd(host(ops.stochastic_lut_forward(6, dev(xc), dev(idx), dev(W), F))[:, :F], oracle.stochastic_lut_forward(6, xc, idx, W, F, 0, 0, 0.25, False)[:, :F], "fp32")
+    dx_ref, dW_ref = oracle.stochastic_lut_backward(6, xc, dy, idx, W, F, None, 0, 0, 0.25, False)
+    dW = dev(np.zeros((O, 64), np.float32))
+    dx = ops.stochastic_lut_backward(6, dev(xc), dev(dy), dev(idx), dev(W), dW, F, rev)
+    assert_bwd(host(dx)[:, :F], dx_ref[:, :F], "fp32 dx"); assert_bwd(host(dW), dW_ref, "fp32 dW")
+
+    # BinaryLut6
+    T = rng.integers(-2**31, 2**31, (O, 2)).astype(np.int32)
+    Fb = 70000
+    xbb = synth.bernoulli_bits(rng, I, Fb, synth.frame_stride_bit(Fb))
+    yb = ops.binary_lut6_forward(dev(xbb), dev(idx), dev(T), Fb)
+    assert np.array_equal(host(yb), oracle.binary_lut6_forward(xbb, idx, T, Fb))
     print("two-valued case ok")
 
 
