@@ -999,14 +999,31 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
 
+        // packed rows: the head (row addresses) and the value table of the next term are requested while the current term
+        // is evaluated — this path is bound by the round trips of a term, not by its instructions
+        int head_next[2 * T::M + 2], values_next = 0;
+        if constexpr (XMODE == kXBit) {
+            if (cnt > 0) {
+#pragma unroll
+                for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[i]; }
+                values_next = rec_v[0];
+            }
+        }
         for (int t = 0; t < cnt; ++t) {
-            int const values = rec_v[(size_t)t * T::REC];          // lane p: the term's value at corner p
             if constexpr (XMODE == kXBit) {
+                int r[2 * T::M + 2];
+#pragma unroll
+                for (int i = 0; i < 2 * T::M + 2; ++i) { r[i] = head_next[i]; }
+                int const values = values_next;                    // lane p: the term's value at corner p
+                if (t + 1 < cnt) {
+#pragma unroll
+                    for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[(size_t)(t + 1) * T::REC + i]; }
+                    values_next = rec_v[(size_t)(t + 1) * T::REC];
+                }
                 // The 64 U frames of a pass are 2 U words of a packed row, the same for every lane: one load per row
                 // brings them in (lane i holds word i of the pass), each step's two words are read back as a lane mask,
                 // and the index costs one add-with-carry per input.  Per term and pass: M + U + 1 vector memory
                 // instructions instead of (M + 1) U + 1.
-                const_int *r = rec + (size_t)t * T::REC;
                 uint32_t w[T::M];
 #pragma unroll
                 for (int j = 0; j < T::M; ++j) {
@@ -1032,6 +1049,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
                 }
                 continue;
             }
+            int const values = rec_v[(size_t)t * T::REC];          // lane p: the term's value at corner p
             typename T::Stage st;
             T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
 #pragma unroll
