@@ -945,10 +945,25 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
 
+        // the head (row addresses) of the next term is requested while the current term is evaluated, so that a term's
+        // loads do not wait for a scalar-memory round trip first
+        constexpr int HEAD = 2 * T::M + 2;
+        int head_next[HEAD];
+        if (cnt > 0) {
+#pragma unroll
+            for (int i = 0; i < HEAD; ++i) { head_next[i] = rec[i]; }
+        }
         for (int t = 0; t < cnt; ++t) {
             typename T::Stage st;
             float Dk[T::HN];
-            T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
+            int head[HEAD];
+#pragma unroll
+            for (int i = 0; i < HEAD; ++i) { head[i] = head_next[i]; }
+            if (t + 1 < cnt) {
+#pragma unroll
+                for (int i = 0; i < HEAD; ++i) { head_next[i] = rec[(size_t)(t + 1) * T::REC + i]; }
+            }
+            T::issue(head, xoff, yoff, x_row_bytes, y_row_bytes, st);
             T::load_coefficients(rec + (size_t)t * T::REC, Dk);
             T::accumulate(st, Dk, bit, lo, hi, acc);
         }
