@@ -23,10 +23,10 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # the same profiler run.  The counter tables and the commands are in profiles/*.md.  A kernel or workload that is not
 # listed reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("lut_dx_kernel<6>", 0):       (686295.3 * 2.0 + 132096.0) * 1024,
-    ("lut_forward_kernel<6>", 0):  (132275.3 * 2.0 + 131072.0) * 1024,
-    ("lut_backward_kernel<6>", 0): (352923.2 * 2.0 + 6352.6) * 1024,
-    ("binary_lut6_kernel", 0):     (649069.0 * 2.0 + 524288.0) * 1024,
+    ("lut_dx_kernel<6>", 0):       (652361.0 * 2.0 + 132096.0) * 1024,
+    ("lut_forward_kernel<6>", 0):  (133352.3 * 2.0 + 131072.0) * 1024,
+    ("lut_backward_kernel<6>", 0): (354315.3 * 2.0 + 6372.5) * 1024,
+    ("binary_lut6_kernel", 0):     (651698.0 * 2.0 + 524288.0) * 1024,
     ("adam_kernel", 0):            (527931.3 * 2.0 + 791860.5) * 1024,
 }
 
