@@ -121,6 +121,115 @@ def test_larger_layer(ops, n):
         assert_bwd(host(dx), dx_ref); assert_bwd(host(dW), dW_ref)
 
 
+def _backward_fp64(x, dy, idx, W, mean, rstd, gamma, beta, binary_mode):
+    """fp64 evaluation of DifferentiableLut6's backward with batch-norm (include/bb/DifferentiableLutN.h:1157-1266) for
+    the table gradient: the gradient behind the hard-tanh window, the batch-norm backward from the stored statistics,
+    then dW[i] = sum_f d * prod_j(x_j or 1 - x_j).  Also returns the batch-norm output t [O, F], which decides the window."""
+    F = x.shape[1]
+    dW = np.zeros((idx.shape[0], 64)); t_all = np.zeros((idx.shape[0], F))
+    for o in range(idx.shape[0]):
+        xs = x[idx[o]].astype(np.float64)
+        xs = np.where(xs > 0.5, 0.75, 0.25) if binary_mode else np.clip(xs, 0.0, 1.0)
+        p = np.ones((64, F))
+        for i in range(64):
+            for j in range(6):
+                p[i] *= xs[j] if (i >> j) & 1 else 1.0 - xs[j]
+        v = W[o].astype(np.float64) @ p
+        m, r = float(mean[o]), float(rstd[o])
+        t = ((v - m) * r) * gamma + beta
+        g = np.where((t > 0.0) & (t < 1.0), dy[o].astype(np.float64), 0.0) * gamma
+        dstd = -(g * (v - m) * r * r).sum(); dmeanx = -(g * r).sum()
+        dvar = dstd * r; dmean = (dmeanx - m * dvar) / F
+        dW[o] = p @ (g * r + dmean + v * dvar / F)
+        t_all[o] = t
+    return dW, t_all
+
+
+def _layer_at_full_shape(ops, I, O, F, binary_mode, slice_nodes):
+    """A layer at a shape of the reference's configurations.  Nodes are independent in everything but dx, and batch-norm
+    couples all frames of a node, so the oracle (whose backward is a single-threaded loop, as the reference's) checks a
+    layer made of a slice of the nodes over all frames: y, statistics, dW and the slice's dx.  The full layer is
+    checked against that slice, and its dx through rules that hold at any size: exactly linear in dy under a factor of
+    two, the same in all three accumulation modes."""
+    import torch
+    rng = np.random.default_rng(I * O + binary_mode)
+    stride = synth.frame_stride_fp32(F)
+    idx = synth.wiring(rng, I, O); W = synth.lut_tables(rng, O)
+    x = synth.uniform_frames(rng, I, F, stride); dy = synth.normal_frames(rng, O, F, stride)
+    sel = np.linspace(0, O - 1, slice_nodes).astype(np.int64)
+    seld = torch.from_numpy(sel).cuda()
+    xd, dyd, idxd, Wd = dev(x), dev(dy), dev(idx), dev(W)
+    rm = np.zeros(O, np.float32); rv = np.ones(O, np.float32)
+    y_ref, mean_ref, rstd_ref, rm_ref, rv_ref = oracle.differentiable_lut_forward_training(6, x, idx[sel], W[sel], F, rm[sel], rv[sel],
+                                                                                           binary_mode=binary_mode)
+    rmd, rvd = dev(rm), dev(rv)
+    y, mean, rstd = ops.differentiable_lut_forward_training(6, xd, idxd, Wd, F, rmd, rvd, binary_mode=binary_mode)
+    assert rel_err(host(mean)[sel], mean_ref) <= 1e-5 and rel_err(host(rstd)[sel], rstd_ref) <= 1e-4
+    assert rel_err(host(rmd)[sel], rm_ref) <= 1e-5 and rel_err(host(rvd)[sel], rv_ref) <= 1e-5
+    if binary_mode:
+        assert (host(y)[sel][:, :F] != y_ref[:, :F]).mean() <= 1e-4
+    else:
+        assert (np.abs(host(y)[sel][:, :F] - y_ref[:, :F]) <= 1e-5 * np.maximum(1.0, 0.3 * rstd_ref)[:, None]).all()
+    # The gradient passes a frame only where the batch-norm output t lies inside (0, 1).  Among a million (node, frame)
+    # pairs a few have t within rounding of an edge, and which side fp32 puts them on is not part of the contract: dy is
+    # zeroed for those pairs of the checked nodes, so that both sides pass nothing there.
+    _, t64 = _backward_fp64(x[:, :F], dy[sel][:, :F], idx[sel], W[sel], mean_ref, rstd_ref, 0.3, 0.5, binary_mode)
+    near = (np.abs(t64) < 1e-5) | (np.abs(t64 - 1.0) < 1e-5)
+    assert near.sum() <= 1e-3 * near.size
+    for k, o in enumerate(sel):
+        dy[o, :F][near[k]] = 0.0
+    dyd = dev(dy)
+    # the slice as a layer of its own: dx and dW against the oracle over all frames
+    dx_ref, dW_ref = oracle.differentiable_lut_backward(6, x, dy[sel], idx[sel], W[sel], F, mean_ref, rstd_ref, binary_mode=binary_mode)
+    ops.set_dx_mode(0)
+    rev_sel = ops.reverse_table(dev(idx[sel]), I)
+    dW_sel = torch.zeros((len(sel), 64), device="cuda")
+    dx_sel = ops.differentiable_lut_backward(6, xd, dev(dy[sel]), dev(idx[sel]), dev(W[sel]), dW_sel, F, dev(mean_ref), dev(rstd_ref),
+                                             rev_sel, binary_mode=binary_mode)
+    assert_bwd(host(dx_sel)[:, :F], dx_ref[:, :F], "dx of the slice")
+    if F <= 65536:
+        assert_bwd(host(dW_sel), dW_ref, "dW of the slice")
+    else:
+        # The oracle adds the F terms of a table gradient, and of the two batch-norm sums behind every one of them, in
+        # one fp32 accumulator each, as the reference does; beyond some 10^5 frames its own rounding reaches the
+        # tolerance.  An fp64 evaluation of the same formulas is the arbiter: the device within the tolerance, the
+        # oracle within ten times that.
+        dW64, _ = _backward_fp64(x[:, :F], dy[sel][:, :F], idx[sel], W[sel], mean_ref, rstd_ref, 0.3, 0.5, binary_mode)
+        assert_bwd(host(dW_sel), dW64, "dW of the slice against fp64")
+        assert rel_err(dW_ref, dW64) <= 1e-3
+    # the full layer, from the device's own statistics; the slice again from the same statistics
+    rev = ops.reverse_table(idxd, I)
+    dW = torch.zeros((O, 64), device="cuda")
+    dx = ops.differentiable_lut_backward(6, xd, dyd, idxd, Wd, dW, F, mean, rstd, rev, binary_mode=binary_mode)
+    dW_own = torch.zeros((len(sel), 64), device="cuda")
+    ops.differentiable_lut_backward(6, xd, dev(dy[sel]), dev(idx[sel]), dev(W[sel]), dW_own, F, mean[seld].contiguous(),
+                                    rstd[seld].contiguous(), rev_sel, binary_mode=binary_mode)
+    assert rel_err(host(dW)[sel], host(dW_own)) <= 1e-5            # the two launches divide the frames differently
+    dW2 = torch.zeros((O, 64), device="cuda")
+    dx2 = ops.differentiable_lut_backward(6, xd, (dyd * 2.0).contiguous(), idxd, Wd, dW2, F, mean, rstd, rev, binary_mode=binary_mode)
+    assert torch.equal(dx2[:, :F], 2.0 * dx[:, :F]) and torch.equal(dW2, 2.0 * dW)
+    for mode in (1, 2):
+        ops.set_dx_mode(mode)
+        dWm = torch.zeros((O, 64), device="cuda")
+        dxm = ops.differentiable_lut_backward(6, xd, dyd, idxd, Wd, dWm, F, mean, rstd, rev, binary_mode=binary_mode)
+        assert rel_err(host(dxm)[:, :F], host(dx)[:, :F]) <= 1e-5 and rel_err(host(dWm), host(dW)) <= 1e-5
+    ops.set_dx_mode(0)
+
+
+@pytest.mark.parametrize("shape", [(784, 6144, 256), (6144, 1024, 256), (1024, 70, 70)])
+def test_classifier_layers_at_full_shape(ops, shape):
+    """the three layers of the MNIST-like classifier at its batch of 1024 frames (binary mode, the class default)"""
+    I, O, slice_nodes = shape
+    _layer_at_full_shape(ops, I, O, 1024, 1, slice_nodes)
+
+
+@pytest.mark.parametrize("shape", [(27, 216, 1), (216, 36, 1), (216, 36, 0)])
+def test_conv_block_layers_at_full_shape(ops, shape):
+    """the two per-pixel layers of the convolutional configuration at their 230 400 frames (256 images of 30 x 30 pixels)"""
+    I, O, binary_mode = shape
+    _layer_at_full_shape(ops, I, O, 230400, binary_mode, 4)
+
+
 @pytest.mark.parametrize("n", [6, 4])
 def test_bit_variants(ops, n):
     rng = np.random.default_rng(300 + n)
