@@ -380,16 +380,14 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
     size_t const c_bytes    = align256((size_t)c.node_size * NN * sizeof(float));
     size_t const v_bytes    = corner ? c_bytes : 0;
     size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
-    size_t const rstd_bytes = (c.bn == 2) ? align256((size_t)c.node_size * sizeof(float)) : 0;
     size_t const bits_bytes = pack ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + v_bytes + stat_bytes + rstd_bytes + bits_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + v_bytes + stat_bytes + bits_bytes, &base)) { return 1; }
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
-    float *rstd_tmp = reinterpret_cast<float *>(base + c_bytes + v_bytes + stat_bytes);
     if (pack) {
-        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes + rstd_bytes);
+        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes);
         if (launch_pack_and_prep<N>(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size,
                                     c.W, C, V, c.node_size, c.lut_binarize, c.bias, st)) { return 1; }
         c.x = bits;
@@ -411,19 +409,24 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
         a.stat_partial = stat;
         if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
-        int const npb = stat_nodes_per_block(chunk_count);
-        hipLaunchKernelGGL(bn_forward_finalize_kernel, dim3(ceil_div(c.node_size, npb)), dim3(kBlock), 0, st,
-                           stat, C, NN, c.mean, c.rstd, c.running_mean, c.running_var, c.momentum,
-                           c.node_size, chunk_count, c.frame_size, npb);
-        BBHIP_LAUNCH_CHECK();
-        a.mean = c.mean; a.rstd = c.rstd;
+        if (chunk_count <= kInlineStatUnits) {
+            // few units: every wavefront of the output pass adds up the partial sums of its node itself, and the wavefront of a
+            // node's first unit stores the statistics; a launch that does it once per node would cost more than that
+            a.stat_mode = kStatPartial; a.momentum = c.momentum;
+            a.mean_out = c.mean; a.rstd_out = c.rstd; a.running_mean = c.running_mean; a.running_var = c.running_var;
+        }
+        else {
+            int const npb = stat_nodes_per_block(chunk_count);
+            hipLaunchKernelGGL(bn_forward_finalize_kernel, dim3(ceil_div(c.node_size, npb)), dim3(kBlock), 0, st,
+                               stat, C, NN, c.mean, c.rstd, c.running_mean, c.running_var, c.momentum,
+                               c.node_size, chunk_count, c.frame_size, npb);
+            BBHIP_LAUNCH_CHECK();
+            a.mean = c.mean; a.rstd = c.rstd;
+        }
         kind = 1;
     }
     else if (c.bn == 2) {
-        hipLaunchKernelGGL(rsqrt_kernel, dim3(ceil_div(c.node_size, kBlock)), dim3(kBlock), 0, st,
-                           c.running_var, rstd_tmp, c.node_size);
-        BBHIP_LAUNCH_CHECK();
-        a.mean = c.running_mean; a.rstd = rstd_tmp;
+        a.stat_mode = kStatRunning; a.mean = c.running_mean; a.rstd = c.running_var;       // rstd = 1 / sqrt(var) in the kernel
         kind = 1;
     }
     {
@@ -597,10 +600,15 @@ int run_backward(BackwardCall const &call, hipStream_t st)
         f.bias = c.bias; f.gamma = c.gamma; f.beta = c.beta;
         if (dispatch_forward<N>(c.xmode, kYClamp, 3, f, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
-        int const npb = stat_nodes_per_block(stat_chunk_count);
-        hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, npb)), dim3(kBlock), 0, st,
-                           stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, stat_chunk_count, c.frame_size, npb);
-        BBHIP_LAUNCH_CHECK();
+        if (stat_chunk_count <= kInlineStatUnits) {
+            a.stat_partial = stat; a.stat_count = stat_chunk_count;     // few units: the table-gradient wavefronts add them up themselves
+        }
+        else {
+            int const npb = stat_nodes_per_block(stat_chunk_count);
+            hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3(ceil_div(c.output_node_size, npb)), dim3(kBlock), 0, st,
+                               stat, c.mean, c.rstd, c.dmean_tmp, c.dvar_tmp, c.gamma, c.output_node_size, stat_chunk_count, c.frame_size, npb);
+            BBHIP_LAUNCH_CHECK();
+        }
     }
 
     if (dxmode == kDxAtomic) {

@@ -183,7 +183,15 @@ struct FwdArgs {
     int   chunk_count;
     TileDivisor tiles;
     float bias, gamma, beta;
+    // where kind 1 takes the batch-norm statistics of a node from (see forward_statistics)
+    int   stat_mode;            // kStatGiven: mean / rstd;  kStatRunning: mean = running mean, rstd holds the running variance;
+                                // kStatPartial: from the partial sums that a kind 2 launch of the same shape left in stat_partial
+    float momentum;             // kStatPartial: the wavefront of a node's first unit also stores the statistics:
+    float *mean_out, *rstd_out, *running_mean, *running_var;
 };
+
+enum StatMode : int { kStatGiven = 0, kStatRunning = 1, kStatPartial = 2 };
+constexpr int kInlineStatUnits = kWave;     // most units whose partial sums a wavefront adds up itself: one load per lane
 
 // What a forward kernel does with the LUT output v of (node, frame f = f0 + lane): accumulate statistics (kinds 2, 3) or
 // apply the batch-norm output stage (kind 1) and store.  ok: the frame belongs to the unit; live: the node exists.
@@ -234,6 +242,69 @@ __device__ __forceinline__ void forward_store_stats(FwdArgs const &a, int ck, in
     }
 }
 
+// Sum of the per-unit partial sums [count][node_size][2] of one node by one wavefront, count <= kInlineStatUnits: lane l
+// holds unit l and wave_sum adds the lanes, a fixed order: every wavefront that sums a node gets the same bits.  With few
+// units this costs a wavefront one load and a dozen cross-lane steps, less than the launch that would do it once per node.
+__device__ __forceinline__ void wave_stat_sums(float const *__restrict__ stat_partial, int node_size, int count, int node, int lane,
+                                               float &s1, float &s2)
+{
+    float2 v = make_float2(0.0f, 0.0f);
+    if (lane < count) { v = *reinterpret_cast<float2 const *>(stat_partial + ((size_t)lane * node_size + node) * 2); }
+    s1 = wave_sum(v.x);
+    s2 = wave_sum(v.y);
+}
+
+// mean, var (>= 1e-5) and rstd of a node from the sums of (v - C0) and (v - C0)^2 over the frames
+// (reference: include/bb/DifferentiableLutN.h:804-806)
+__device__ __forceinline__ void batch_statistics(float s1, float s2, float c0, int frame_size, float &mean, float &var, float &rstd)
+{
+    float const r  = 1.0f / (float)frame_size;
+    float const m0 = s1 * r;                                  // mean of (v - C0)
+    mean = c0 + m0;
+    var  = fmaxf(1.0e-5f, s2 * r - m0 * m0);
+    rstd = 1.0f / sqrtf(var);
+}
+
+// running statistics and the stored mean / rstd of a training pass (reference: DifferentiableLutN.h:809-812)
+__device__ __forceinline__ void store_statistics(float *__restrict__ mean_out, float *__restrict__ rstd_out,
+                                                 float *__restrict__ running_mean, float *__restrict__ running_var,
+                                                 int node, float mean, float var, float rstd, float momentum)
+{
+    running_mean[node] = running_mean[node] * momentum + mean * (1.0f - momentum);
+    running_var[node]  = running_var[node]  * momentum + var  * (1.0f - momentum);
+    mean_out[node] = mean;
+    rstd_out[node] = rstd;
+}
+
+// batch-norm statistics of a node for the output stage (kind 1), by the mode of the call; var only with kStatPartial
+__device__ __forceinline__ void forward_statistics(FwdArgs const &a, int node, int lane, float c0, float &mean, float &var, float &rstd)
+{
+    var = 0.0f;
+    if (a.stat_mode == kStatPartial) {
+        float s1, s2;
+        wave_stat_sums(a.stat_partial, a.node_size, a.chunk_count, node, lane, s1, s2);
+        batch_statistics(s1, s2, c0, a.frame_size, mean, var, rstd);
+    }
+    else {
+        mean = a.mean[node];
+        rstd = a.rstd[node];
+        if (a.stat_mode == kStatRunning) { rstd = 1.0f / sqrtf(rstd); }       // reference: DifferentiableLutN.h:866-868
+    }
+    // the same in every lane: kept in scalar registers, as when they are read from memory
+    mean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mean)));
+    var  = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(var)));
+    rstd = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(rstd)));
+}
+
+// kStatPartial: the wavefront of a node's first unit stores the statistics.  Called at the end of the kernel: a store ahead
+// of the wave-uniform loads of the set-up would take them off the scalar path.
+__device__ __forceinline__ void forward_store_statistics(FwdArgs const &a, int node, bool live, int ck, int lane, float mean, float var, float rstd)
+{
+    if (a.stat_mode == kStatPartial && ck == 0 && lane == 0 && live) {
+        store_statistics(a.mean_out, a.rstd_out, a.running_mean, a.running_var, node, mean, var, rstd, a.momentum);
+    }
+}
+
 // FWD_KIND: 0 = plain LUT output, 1 = LUT + batch-norm (mean/rstd/gamma/beta) output, 2 = statistics only,
 //           3 = statistics of the backward pass through batch-norm: per node the sums of g and g (v - mean), where g = dy gated by
 //               the hard-tanh window 0 < t < 1 of the batch-norm output t (reference: DifferentiableLutN.h:1206-1222)
@@ -256,13 +327,21 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     float C[NPW][kMatrix ? 1 : D::NN], cv[NPW][D::H];
     LutMatrixQ<N> mq[NPW];
     void const *rows[NPW][N];
-    float mean[NPW], rstd[NPW], c0[NPW];
+    float mean[NPW], rstd[NPW], var[NPW], c0[NPW];
     int node[NPW];
     bool live[NPW];
+    // (the statistics first: what they need in registers is gone before the tables arrive)
 #pragma unroll
     for (int p = 0; p < NPW; ++p) {
         live[p] = (node0 + p < a.node_size);
         node[p] = live[p] ? node0 + p : node0;              // a wavefront past the last node repeats its first one and stores nothing
+        mean[p] = 0.0f; rstd[p] = 1.0f; var[p] = 0.0f;
+        c0[p] = a.C[(size_t)node[p] * D::NN];
+        if (FWD_KIND == 1) { forward_statistics(a, node[p], lane, c0[p], mean[p], var[p], rstd[p]); }
+        if (FWD_KIND == 3) { mean[p] = a.mean[node[p]]; rstd[p] = a.rstd[node[p]]; }
+    }
+#pragma unroll
+    for (int p = 0; p < NPW; ++p) {
         if constexpr (kMatrix) {
             mq[p].load(a.C + (size_t)node[p] * D::NN, lane);
             C[p][0] = a.C[(size_t)node[p] * D::NN];
@@ -277,9 +356,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
             rows[p][k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
                                           : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
         }
-        mean[p] = 0.0f; rstd[p] = 1.0f;
-        if (FWD_KIND == 1 || FWD_KIND == 3) { mean[p] = a.mean[node[p]]; rstd[p] = a.rstd[node[p]]; }
-        c0[p] = C[p][0];
     }
 
     int const f_begin = ck * a.chunk;
@@ -328,6 +404,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     if (FWD_KIND == 2 || FWD_KIND == 3) {
 #pragma unroll
         for (int p = 0; p < NPW; ++p) { forward_store_stats(a, ck, node[p], live[p], lane, s1[p], s2[p]); }
+    }
+    if (FWD_KIND == 1) {
+#pragma unroll
+        for (int p = 0; p < NPW; ++p) { forward_store_statistics(a, node[p], live[p], ck, lane, mean[p], var[p], rstd[p]); }
     }
 }
 
@@ -396,8 +476,10 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
                                    : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
     }
     float mean = 0.0f, rstd = 1.0f, c0 = 0.0f;
-    if (FWD_KIND == 1 || FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
-    if (FWD_KIND == 2) { c0 = a.C[(size_t)node * NN]; }
+    if (FWD_KIND == 2 || (FWD_KIND == 1 && a.stat_mode == kStatPartial)) { c0 = a.C[(size_t)node * NN]; }
+    float var = 0.0f;
+    if (FWD_KIND == 1) { forward_statistics(a, node, lane, c0, mean, var, rstd); }
+    if (FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
 
     int const f_begin = ck * a.chunk;
     int const f_end   = min(f_begin + a.chunk, a.frame_size);
@@ -429,6 +511,7 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
         }
     }
     if (FWD_KIND == 2 || FWD_KIND == 3) { forward_store_stats(a, ck, node, true, lane, s1, s2); }
+    if (FWD_KIND == 1) { forward_store_statistics(a, node, true, ck, lane, mean, var, rstd); }
 }
 
 // Sum of the per-unit partial sums [count][node_size][2] of one node.  A workgroup owns nodes_per_block consecutive nodes
@@ -473,22 +556,9 @@ __global__ __launch_bounds__(kBlock) void bn_forward_finalize_kernel(float const
     int node;
     float s1, s2;
     if (!sum_stat_partials(stat_partial, node_size, chunk_count, nodes_per_block, node, s1, s2)) { return; }
-    float const r  = 1.0f / (float)frame_size;
-    float const m0 = s1 * r;                                  // mean of (v - C0)
-    float const m  = C[(size_t)node * nn] + m0;
-    float const var = fmaxf(1.0e-5f, s2 * r - m0 * m0);
-    float const rs  = 1.0f / sqrtf(var);
-    running_mean[node] = running_mean[node] * momentum + m   * (1.0f - momentum);
-    running_var[node]  = running_var[node]  * momentum + var * (1.0f - momentum);
-    mean[node] = m;
-    rstd[node] = rs;
-}
-
-// rstd = 1/sqrt(var) for inference (reference: DifferentiableLutN.h:866-868)
-__global__ __launch_bounds__(kBlock) void rsqrt_kernel(float const *__restrict__ var, float *__restrict__ rstd, int size)
-{
-    int const i = blockIdx.x * kBlock + threadIdx.x;
-    if (i < size) { rstd[i] = 1.0f / sqrtf(var[i]); }
+    float m, var, rs;
+    batch_statistics(s1, s2, C[(size_t)node * nn], frame_size, m, var, rs);
+    store_statistics(mean, rstd, running_mean, running_var, node, m, var, rs, momentum);
 }
 
 // Term table for the input-centric dx kernel: for input node `in` and its t-th consumer connection (t-th entry of
@@ -596,7 +666,19 @@ struct BwdArgs {
     float bias, gamma, beta, inv_frames;
     TermArgs tt;                // kDxNone: the last tt.blocks workgroups of the launch build the dx kernel's term table
     float const *V;             // [O][2^N] corner values (CORNER variant)
+    float const *stat_partial;  // BN, not null: dmean / dvar come from the stat_count (<= kInlineStatUnits) partial sums
+    int   stat_count;           //     [unit][O][2] that the kind 3 launch left, added up by every wavefront for its node
 };
+
+// dvar and dmean of a node from the sums of g and g (v - mean) over the frames (reference: DifferentiableLutN.h:1218-1222)
+__device__ __forceinline__ void batch_gradient_statistics(float s0, float s1, float mean, float rstd, float gamma, int frame_size,
+                                                          float &dmean, float &dvar)
+{
+    float const dstd   = -(gamma * s1) * (rstd * rstd);
+    float const dmeanx = -(gamma * s0) * rstd;
+    dvar  = dstd * rstd;
+    dmean = (dmeanx - mean * dvar) * (1.0f / (float)frame_size);
+}
 
 enum DxMode : int { kDxAtomic = 0, kDxTmp = 1, kDxNone = 2 };
 
@@ -651,7 +733,17 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
 
     float mean = 0.0f, rstd = 1.0f, dmean = 0.0f, dvarf = 0.0f;
     if (BWD_KIND != 0) { mean = a.mean[node]; rstd = a.rstd[node]; }
-    if (BWD_KIND == 1) { dmean = a.dmean[node]; dvarf = a.dvar[node] * a.inv_frames; }
+    if (BWD_KIND == 1) {
+        if (a.stat_partial) {
+            float s0, s1, dv;
+            wave_stat_sums(a.stat_partial, a.node_size, a.stat_count, node, lane, s0, s1);
+            batch_gradient_statistics(s0, s1, mean, rstd, a.gamma, a.frame_size, dmean, dv);
+            dvarf = dv * a.inv_frames;
+        }
+        else { dmean = a.dmean[node]; dvarf = a.dvar[node] * a.inv_frames; }
+        dmean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(dmean)));       // the same in every lane
+        dvarf = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(dvarf)));
+    }
     float const grs = a.gamma * rstd;
 
     int const f_begin = a.f_base + sl * a.slab;
@@ -1095,12 +1187,10 @@ __global__ __launch_bounds__(kBlock) void bn_backward_finalize_kernel(float cons
     int node;
     float s0, s1;
     if (!sum_stat_partials(stat_partial, node_size, slab_count, nodes_per_block, node, s0, s1)) { return; }
-    float const rs = rstd[node];
-    float const dstd   = -(gamma * s1) * (rs * rs);
-    float const dmeanx = -(gamma * s0) * rs;
-    float const dv = dstd * rs;
+    float dm, dv;
+    batch_gradient_statistics(s0, s1, mean[node], rstd[node], gamma, frame_size, dm, dv);
     dvar[node]  = dv;
-    dmean[node] = (dmeanx - mean[node] * dv) * (1.0f / (float)frame_size);
+    dmean[node] = dm;
 }
 
 // dx[in][f] = sum_k tmp[rev[in][k]][f - base], k = 1 .. rev[in][0]  (the reference's reverse-table order,
