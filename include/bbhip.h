@@ -75,7 +75,8 @@ int  bbhip_GetDxMode(void);
  * mode on fp32 frames the library then packs the binarized input to bits once (it has to know how many rows to pack)
  * and runs the packed-bit kernels, as the backward entry points — which are told input_node_size — always do.
  * The hint holds for one forward call and is cleared by it; 0 clears it.  The rows [0, input_node_size) of the input
- * buffer must exist: the value is trusted like the sizes of any entry point.  Results do not depend on the hint. */
+ * buffer must exist and input_index must name no row beyond them (only the named rows are read without the hint, all
+ * of them with it): the value is trusted like the sizes of any entry point.  Results do not depend on the hint. */
 void bbhip_HintInputNodeSize(int input_node_size);
 
 /* ---- kernel timer (instrumentation; no counterpart in the reference) ----
