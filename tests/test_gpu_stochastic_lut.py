@@ -274,7 +274,7 @@ def test_full_size_properties_packed_bits(ops):
     # linear in dy, and a slice of frames against the oracle
     dWc = torch.zeros((O, 64), device="cuda")
     dxc = ops.bit_stochastic_lut_backward(6, xd, (dyd * 2.0).contiguous(), idxd, Wd, dWc, F, rev, 0)
-    assert rel_err(host(dxc), 2.0 * host(dx)) <= 1e-6
+    assert rel_err(host(dxc)[:, :F], 2.0 * host(dx)[:, :F]) <= 1e-6          # (the padding of a row is not written)
     fs = 256
     dx_ref, _ = oracle.bit_stochastic_lut_backward(6, np.ascontiguousarray(xb[:, :fs // 32]), np.ascontiguousarray(dy[:, :fs]), idx, W, fs, None, 0)
     assert_bwd(host(dx)[:, :fs], dx_ref)
