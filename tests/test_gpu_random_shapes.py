@@ -1,0 +1,122 @@
+"""GPU parity on random shapes: LUT width, node and frame counts, row pitches, input kind (fp32, fp32 binarized, packed
+bits), table binarization, batch-norm or not, and the dx mode are drawn from a seeded generator; every case goes through
+the C ABI and is compared with the CPU oracle at the tolerances of the other GPU tests.  What the draws hit that fixed
+cases rarely do, and how the comparison deals with it:
+  * a table that is constant after binarization has dx = 0 exactly, and batch-norm can cancel a whole table gradient: the
+    oracle then holds rounding noise, so dx and dW are measured against max(|reference|, |dy|);
+  * the oracle's var = E[y^2] - E[y]^2 (the reference's formula) loses digits when var is small against mean^2 (narrow
+    LUTs on two-valued inputs): rstd gets 1e-7 / var on top of its 1e-4;
+  * frames whose batch-norm output is within 1e-5 of the binarization threshold or of an edge of the hard-tanh window may
+    fall on either side (sometimes for a whole class of frames, when a corner value of a binarized table equals the
+    mean): outputs are compared away from the threshold, and dy is zeroed at the window's edges."""
+import numpy as np
+import pytest
+
+import oracle
+from binarybrain_amd import synth
+from test_gpu_differentiable_lut import _pre_activation
+from util import dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(a, b, floor=0.0):
+    a = np.asarray(a, np.float64); b = np.asarray(b, np.float64)
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), floor, 1e-30))
+
+
+def stride_fp32(rng, F):
+    return int(rng.choice([F, ((F + 63) // 64) * 64, synth.frame_stride_fp32(F), F + int(rng.integers(0, 70))]))
+
+
+def run_case(ops, torch, seed):
+    rng = np.random.default_rng(seed)
+    n = int(rng.choice([2, 3, 4, 5, 6], p=[0.1, 0.1, 0.15, 0.15, 0.5]))
+    I = int(rng.integers(n, 300)); O = int(rng.integers(1, 200))
+    F = int(rng.choice([int(rng.integers(1, 70)), int(rng.integers(64, 700)), int(rng.integers(700, 5000))]))
+    kind = str(rng.choice(["st_fp32", "st_bin", "st_bit", "dl_fp32", "dl_bit"]))
+    lut_binarize = int(rng.integers(0, 2)); mode = int(rng.integers(0, 3))
+    print("seed %d: %s n=%d I=%d O=%d F=%d lut_binarize=%d dx mode %d" % (seed, kind, n, I, O, F, lut_binarize, mode), flush=True)
+    idx = synth.wiring(rng, I, O, n); W = synth.lut_tables(rng, O, n)
+    ys = stride_fp32(rng, F)
+    dy = synth.normal_frames(rng, O, F, ys)
+    ops.set_dx_mode(mode)
+    rev = ops.reverse_table(dev(idx), I)
+    dW = torch.zeros((O, 1 << n), device="cuda")
+    if kind in ("st_fp32", "st_bin"):
+        binary = kind == "st_bin"
+        x = synth.uniform_frames(rng, I, F, ys, -0.1, 1.1)
+        y = ops.stochastic_lut_forward(n, dev(x), dev(idx), dev(W), F, binary, bool(lut_binarize))
+        y_ref = oracle.stochastic_lut_forward(n, x, idx, W, F, binary, bool(lut_binarize))
+        dx = ops.stochastic_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, binary, bool(lut_binarize))
+        dx_ref, dW_ref = oracle.stochastic_lut_backward(n, x, dy, idx, W, F, None, binary, bool(lut_binarize))
+        assert np.abs(host(y)[:, :F] - y_ref[:, :F]).max() <= 1e-5
+        assert rel_err(host(dx)[:, :F], dx_ref[:, :F], float(np.abs(dy).max())) <= 1e-4 and rel_err(host(dW), dW_ref, float(np.abs(dy).max())) <= 1e-4
+    elif kind == "st_bit":
+        xs = int(rng.choice([synth.frame_stride_bit(F), (F + 31) // 32, (F + 31) // 32 + int(rng.integers(0, 9))]))
+        xb = synth.bernoulli_bits(rng, I, F, xs)
+        y = ops.bit_stochastic_lut_forward(n, dev(xb), dev(idx), dev(W), F, ys, lut_binarize)
+        y_ref = oracle.bit_stochastic_lut_forward(n, xb, idx, W, F, ys, lut_binarize)
+        dx = ops.bit_stochastic_lut_backward(n, dev(xb), dev(dy), dev(idx), dev(W), dW, F, rev, lut_binarize)
+        dx_ref, dW_ref = oracle.bit_stochastic_lut_backward(n, xb, dy, idx, W, F, None, lut_binarize)
+        assert np.abs(host(y)[:, :F] - y_ref[:, :F]).max() <= 1e-5
+        assert rel_err(host(dx)[:, :F], dx_ref[:, :F], float(np.abs(dy).max())) <= 1e-4 and rel_err(host(dW), dW_ref, float(np.abs(dy).max())) <= 1e-4
+    else:
+        if F < 8:
+            return
+        binary_mode = 1 if kind == "dl_bit" else int(rng.integers(0, 2))
+        rm = rng.random(O).astype(np.float32); rv = (rng.random(O) + 0.5).astype(np.float32)
+        Wb = (W > 0.5).astype(np.float32) if lut_binarize else W
+        # statistics from the oracle first: they say where the batch-norm output t sits; dy is zeroed where t is within
+        # rounding of an edge of the hard-tanh window (either side is right there)
+        if kind == "dl_fp32":
+            x = synth.uniform_frames(rng, I, F, ys, -0.1, 1.1)
+            xc = (np.where(x > 0.5, 0.75, 0.25) if binary_mode else np.clip(x, 0, 1))[:, :F]
+            _, mean0, rstd0, _, _ = oracle.differentiable_lut_forward_training(n, x, idx, W, F, rm, rv, 0.3, 0.5, 0.9, 0.25, lut_binarize, binary_mode)
+        else:
+            xs = synth.frame_stride_bit(F)
+            xb = synth.bernoulli_bits(rng, I, F, xs)
+            dy = synth.normal_frames(rng, O, F, synth.frame_stride_fp32(F))
+            xc = np.where(synth.unpack_bits(xb, F) > 0, 0.75, 0.25)
+            _, mean0, rstd0, _, _ = oracle.bit_differentiable_lut_forward_training(n, xb, idx, W, F, rm, rv, lut_binarize=lut_binarize)
+        pre = _pre_activation(n, xc, idx, Wb, mean0.astype(np.float64), rstd0.astype(np.float64), 0.3, 0.5)
+        edge = (np.abs(pre) < 1e-5) | (np.abs(pre - 1.0) < 1e-5)
+        dy[:, :F][edge] = 0.0
+        if kind == "dl_fp32":
+            y_ref, mean_ref, rstd_ref, rm_ref, rv_ref = oracle.differentiable_lut_forward_training(n, x, idx, W, F, rm, rv, 0.3, 0.5, 0.9, 0.25, lut_binarize, binary_mode)
+            rmd, rvd = dev(rm), dev(rv)
+            y, mean, rstd = ops.differentiable_lut_forward_training(n, dev(x), dev(idx), dev(W), F, rmd, rvd, 0.3, 0.5, 0.9, 0.25, lut_binarize, binary_mode)
+            yg, yr = host(y)[:, :F], y_ref[:, :F]
+            dx_ref, dW_ref = oracle.differentiable_lut_backward(n, x, dy, idx, W, F, mean_ref, rstd_ref, None, 0.3, 0.5, 0.25, lut_binarize, binary_mode)
+            dx = ops.differentiable_lut_backward(n, dev(x), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev, 0.3, 0.5, 0.25, lut_binarize, binary_mode)
+        else:
+            y_ref, mean_ref, rstd_ref, rm_ref, rv_ref = oracle.bit_differentiable_lut_forward_training(n, xb, idx, W, F, rm, rv, lut_binarize=lut_binarize)
+            rmd, rvd = dev(rm), dev(rv)
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(n, dev(xb), dev(idx), dev(W), F, rmd, rvd, lut_binarize=lut_binarize)
+            yg, yr = synth.unpack_bits(host(y), F), synth.unpack_bits(y_ref, F)
+            dx_ref, dW_ref = oracle.bit_differentiable_lut_backward(n, xb, dy, idx, W, F, mean_ref, rstd_ref, lut_binarize=lut_binarize)
+            dx = ops.bit_differentiable_lut_backward(n, dev(xb), dev(dy), dev(idx), dev(W), dW, F, dev(mean_ref), dev(rstd_ref), rev, lut_binarize=lut_binarize)
+        # the oracle's var = E[y^2] - E[y]^2 (the reference's formula) loses digits when var is small against mean^2
+        rtol = 1e-4 + 1e-7 / np.minimum(1.0, 1.0 / rstd_ref.astype(np.float64) ** 2)
+        assert rel_err(host(mean), mean_ref) <= 1e-5 and (np.abs(host(rstd) - rstd_ref) <= rtol * rstd_ref).all()
+        assert rel_err(host(rmd), rm_ref) <= 1e-5 and rel_err(host(rvd), rv_ref) <= 1e-4
+        if binary_mode:
+            diff = (yg != yr); near = np.abs(pre - 0.5) < 1e-5
+            assert not (diff & ~near).any()
+        else:
+            tol = 1e-5 * np.maximum(1.0, 0.3 * rstd_ref)[:, None]
+            assert (np.abs(yg - yr) <= tol).all()
+        if np.abs(dx_ref).max() > 0:
+            e1, e2 = rel_err(host(dx)[:, :F], dx_ref[:, :F], float(np.abs(dy).max())), rel_err(host(dW), dW_ref, float(np.abs(dy).max()))
+            assert e1 <= 1e-4 and e2 <= 1e-4, (e1, e2)
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_shapes(block):
+    import torch
+    from binarybrain_amd import ops
+    try:
+        for seed in range(7000 + 40 * block, 7000 + 40 * (block + 1)):
+            run_case(ops, torch, seed)
+    finally:
+        ops.set_dx_mode(0)
