@@ -1,6 +1,7 @@
 """GPU parity on random shapes: LUT width, node and frame counts, row pitches, input kind (fp32, fp32 binarized, packed
 bits), table binarization, batch-norm or not, and the dx mode are drawn from a seeded generator; every case goes through
-the C ABI and is compared with the CPU oracle at the tolerances of the other GPU tests.  What the draws hit that fixed
+the C ABI and is compared with the CPU oracle at the tolerances of the other GPU tests (BinaryLut6, the bit-to-bit forward,
+Im2Col, Col2Im and pooling, drawn the same way, bit for bit).  What the draws hit that fixed
 cases rarely do, and how the comparison deals with it:
   * a table that is constant after binarization has dx = 0 exactly, and batch-norm can cancel a whole table gradient: the
     oracle then holds rounding noise, so dx and dW are measured against max(|reference|, |dy|);
@@ -120,3 +121,86 @@ def test_random_shapes(block):
             run_case(ops, torch, seed)
     finally:
         ops.set_dx_mode(0)
+
+
+def pad(a, stride):
+    out = np.zeros((a.shape[0], stride), a.dtype); out[:, :a.shape[1]] = a
+    return out
+
+
+def run_exact_case(ops, seed):
+    """the rows whose results are integers, bits or permutations: equal to the oracle bit for bit"""
+    F32 = np.float32
+    rng = np.random.default_rng(seed)
+    kind = str(rng.choice(["binary", "bitbit", "im2col", "col2im", "pool"]))
+    if kind == "binary":
+        I = int(rng.integers(6, 600)); O = int(rng.integers(1, 400))
+        F = int(rng.choice([int(rng.integers(1, 100)), int(rng.integers(100, 3000)), int(rng.integers(3000, 40000))]))
+        print("seed %d: binary I=%d O=%d F=%d" % (seed, I, O, F), flush=True)
+        words = (F + 31) // 32
+        stride = int(rng.choice([synth.frame_stride_bit(F), words, words + int(rng.integers(0, 9))]))
+        idx = synth.wiring(rng, I, O); T = synth.truth_tables(rng, O)
+        xb = synth.bernoulli_bits(rng, I, F, stride)
+        y = ops.binary_lut6_forward(dev(xb), dev(idx), dev(T), F)
+        assert np.array_equal(synth.unpack_bits(host(y), F), synth.unpack_bits(oracle.binary_lut6_forward(xb, idx, T, F), F))
+    elif kind == "bitbit":
+        n = int(rng.integers(2, 7)); I = int(rng.integers(n, 300)); O = int(rng.integers(1, 200)); F = int(rng.integers(1, 6000))
+        lb = int(rng.integers(0, 2))
+        print("seed %d: bitbit n=%d I=%d O=%d F=%d lb=%d" % (seed, n, I, O, F, lb), flush=True)
+        idx = synth.wiring(rng, I, O, n)
+        W = synth.lut_tables(rng, O, n)
+        xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))
+        y = ops.bit_bit_stochastic_lut_forward(n, dev(xb), dev(idx), dev(W), F, lb)
+        y_ref = oracle.bit_bit_stochastic_lut_forward(n, xb, idx, W, F, lb)
+        yf = oracle.bit_stochastic_lut_forward(n, xb, idx, W, F, synth.frame_stride_fp32(F), lb)[:, :F]
+        diff = synth.unpack_bits(host(y), F) != synth.unpack_bits(y_ref, F)
+        assert not (diff & (np.abs(yf - 0.5) > 1e-6)).any()          # an output bit may differ only where the fp32 output sits on the threshold
+    elif kind == "im2col":
+        c = int(rng.integers(1, 5)); h = int(rng.integers(1, 20)); w = int(rng.integers(1, 80)); F = int(rng.integers(1, 200))
+        fh = int(rng.integers(1, min(h, 4) + 1)); fw = int(rng.integers(1, min(w, 5) + 1))
+        ys = int(rng.integers(1, 3)); xs = int(rng.integers(1, 3))
+        padm = str(rng.choice(["valid", "same"])); border = str(rng.choice(["reflect_101", "replicate", "constant", "wrap", "reflect"]))
+        if padm == "same" and border in ("reflect_101", "reflect") and (h < fh or w < fw or h < 2 or w < 2):
+            return
+        print("seed %d: im2col c=%d h=%d w=%d F=%d f=%dx%d s=%d,%d %s %s" % (seed, c, h, w, F, fh, fw, ys, xs, padm, border), flush=True)
+        x = rng.random((c * h * w, F)).astype(F32)
+        y_ref = oracle.im2col_forward(x, c, h, w, F, fh, fw, ys, xs, padm, border, 0.25)
+        of = y_ref.shape[1]
+        y = host(ops.im2col_forward(dev(pad(x, synth.frame_stride_fp32(F))), c, h, w, F, fh, fw, ys, xs, padm, border, 0.25))
+        assert np.array_equal(y[:, :of], y_ref)
+        dy = rng.standard_normal((c * fh * fw, of)).astype(F32)
+        dx_ref = oracle.im2col_backward(dy, c, h, w, F, fh, fw, ys, xs, padm)
+        dx = host(ops.im2col_backward(dev(pad(dy, synth.frame_stride_fp32(of))), c, h, w, F, fh, fw, ys, xs, padm))
+        assert np.array_equal(dx[:, :F], dx_ref)
+        xb = synth.bernoulli_bits(rng, c * h * w, F, synth.frame_stride_bit(F))
+        yb_ref = oracle.im2col_forward(xb, c, h, w, F, fh, fw, ys, xs, padm, border, bit=True)
+        yb = host(ops.im2col_forward(dev(xb), c, h, w, F, fh, fw, ys, xs, padm, border))
+        assert np.array_equal(synth.unpack_bits(yb, of), synth.unpack_bits(yb_ref, of))
+    elif kind == "col2im":
+        c = int(rng.integers(1, 40)); h = int(rng.integers(1, 20)); w = int(rng.integers(1, 20)); F = int(rng.integers(1, 40))
+        print("seed %d: col2im c=%d h=%d w=%d F=%d" % (seed, c, h, w, F), flush=True)
+        x = rng.random((c, F * h * w)).astype(F32)
+        y_ref = oracle.col2im_forward(x, c, h, w, F)
+        y = host(ops.col2im_forward(dev(pad(x, synth.frame_stride_fp32(F * h * w))), c, h, w, F))
+        assert np.array_equal(y[:, :F], y_ref[:, :F])
+        dy = rng.standard_normal((c * h * w, F)).astype(F32)
+        dx_ref = oracle.col2im_backward(dy, c, h, w, F)
+        dx = host(ops.col2im_backward(dev(pad(dy, synth.frame_stride_fp32(F))), c, h, w, F))
+        assert np.array_equal(dx[:, :F * h * w], dx_ref[:, :F * h * w])
+    else:
+        c = int(rng.integers(1, 20)); h = int(rng.integers(1, 24)); w = int(rng.integers(1, 24)); F = int(rng.integers(1, 300))
+        print("seed %d: pool c=%d h=%d w=%d F=%d" % (seed, c, h, w, F), flush=True)
+        x = rng.random((c * h * w, F)).astype(F32)
+        y_ref = oracle.stochastic_maxpool2x2_forward(x, c, h, w, F)
+        xd = dev(pad(x, synth.frame_stride_fp32(F)))
+        y = host(ops.stochastic_maxpool2x2_forward(xd, c, h, w, F))
+        assert np.array_equal(y[:, :F], y_ref[:, :F])
+        dy = rng.standard_normal((y_ref.shape[0], F)).astype(F32)
+        dx_ref = oracle.stochastic_maxpool2x2_backward(x, dy, c, h, w, F)
+        dx = host(ops.stochastic_maxpool2x2_backward(xd, dev(pad(dy, synth.frame_stride_fp32(F))), c, h, w, F))
+        assert np.array_equal(dx[:, :F], dx_ref[:, :F])
+
+def test_random_shapes_of_the_exact_rows():
+    from binarybrain_amd import ops
+    for seed in range(9000, 9400):
+        run_exact_case(ops, seed)
