@@ -1,7 +1,7 @@
 """GPU parity on random shapes: LUT width, node and frame counts, row pitches, input kind (fp32, fp32 binarized, packed
 bits), table binarization, batch-norm or not, and the dx mode are drawn from a seeded generator; every case goes through
 the C ABI and is compared with the CPU oracle at the tolerances of the other GPU tests (BinaryLut6, the bit-to-bit forward,
-Im2Col, Col2Im and pooling, drawn the same way, bit for bit).  What the draws hit that fixed
+Im2Col, Col2Im and pooling, drawn the same way, bit for bit; AverageLut, the loss, accuracy and Adam at their own tests' bars).  What the draws hit that fixed
 cases rarely do, and how the comparison deals with it:
   * a table that is constant after binarization has dx = 0 exactly, and batch-norm can cancel a whole table gradient: the
     oracle then holds rounding noise, so dx and dW are measured against max(|reference|, |dy|);
@@ -204,3 +204,64 @@ def test_random_shapes_of_the_exact_rows():
     from binarybrain_amd import ops
     for seed in range(9000, 9400):
         run_exact_case(ops, seed)
+
+
+def run_tail_case(ops, torch, seed):
+    """AverageLut and accuracy bit-exact, the loss at the tolerances of tests/test_gpu_tail.py, Adam bit-exact"""
+    import test_gpu_tail as tail
+    F32 = np.float32
+    rng = np.random.default_rng(seed)
+    kind = str(rng.choice(["average", "loss", "adam"]))
+    if kind == "average":
+        n = int(rng.choice([int(rng.integers(1, 17)), int(rng.integers(17, 400))])); I = int(rng.integers(1, 400)); O = int(rng.integers(1, 120))
+        F = int(rng.integers(1, 1500))
+        print("seed %d: average n=%d I=%d O=%d F=%d" % (seed, n, I, O, F), flush=True)
+        idx = rng.integers(0, I, (O, n)).astype(np.int32)
+        stride = synth.frame_stride_fp32(F)
+        x = tail._pad((rng.random((I, F)) * 2 - 1).astype(F32), stride)
+        x[rng.random(x.shape) < 0.05] = 0.0
+        dy = tail._pad(rng.standard_normal((O, F)).astype(F32), stride)
+        for bin_in in (False, True):
+            for bin_out in (False, True):
+                y = host(ops.average_lut_forward(dev(x), dev(idx), F, bin_in, bin_out))
+                assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, bin_in, bin_out)[:, :F]), (bin_in, bin_out)
+        dx = host(ops.average_lut_backward(dev(dy), dev(idx), I, F))
+        assert np.array_equal(dx, oracle.average_lut_backward(dy, idx, I, F))
+        xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))
+        yb = host(ops.bit_average_lut_forward(dev(xb), dev(idx), F))
+        assert np.array_equal(synth.unpack_bits(yb, F), synth.unpack_bits(oracle.bit_average_lut_forward(xb, idx, F), F))
+    elif kind == "loss":
+        ch = int(rng.choice([int(rng.integers(1, 12)), int(rng.integers(12, 300))])); pix = int(rng.choice([1, int(rng.integers(1, 40))]))
+        F = int(rng.integers(1, 600))
+        sharp = bool(rng.integers(0, 2)); weighted = bool(rng.integers(0, 2))
+        print("seed %d: loss ch=%d pix=%d F=%d sharp=%d weighted=%d" % (seed, ch, pix, F, sharp, weighted), flush=True)
+        y = (rng.standard_normal((ch * pix, F)) * (30.0 if sharp else 1.0)).astype(F32)
+        t = tail._targets(rng, ch, pix, F, weighted=weighted)
+        if not t.any():
+            t[0, 0] = 1
+        tail._check_loss(ops, y, t, ch, pix, F, synth.frame_stride_fp32(F))
+    else:
+        k = int(rng.integers(1, 6))
+        shapes = [(int(rng.integers(1, 3000)),) if rng.integers(0, 2) else (int(rng.integers(1, 300)), 64) for _ in range(k)]
+        lr = float(rng.choice([0.001, 0.01, 0.1])); b1 = float(rng.choice([0.9, 0.5])); b2 = float(rng.choice([0.999, 0.9]))
+        steps = int(rng.integers(1, 5))
+        print("seed %d: adam %s lr=%g b=%g,%g steps=%d" % (seed, shapes, lr, b1, b2, steps), flush=True)
+        p0 = [rng.random(s).astype(F32) for s in shapes]
+        params = [dev(a.copy()) for a in p0]
+        grads = [torch.zeros_like(p) for p in params]
+        st = ops.AdamState(params, grads, lr, b1, b2)
+        gs = [[(rng.standard_normal(s) * 0.1).astype(F32) for s in shapes] for _ in range(steps)]
+        for step in gs:
+            for g, a in zip(grads, step):
+                g.copy_(dev(a))
+            st.step()
+        for i, s in enumerate(shapes):
+            ref, m, v = oracle.adam_steps(p0[i].ravel(), [step[i].ravel() for step in gs], lr, b1, b2)
+            assert np.array_equal(host(params[i]).ravel(), ref), s
+            assert np.array_equal(host(st.m[i]).ravel(), m) and np.array_equal(host(st.v[i]).ravel(), v)
+
+def test_random_shapes_of_the_classifier_tail_and_adam():
+    import torch
+    from binarybrain_amd import ops
+    for seed in range(11000, 11150):
+        run_tail_case(ops, torch, seed)
