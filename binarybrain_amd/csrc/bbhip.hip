@@ -64,6 +64,7 @@ thread_local int g_input_node_hint = 0;      // bbhip_HintInputNodeSize: rows of
 enum TimedKernel : int { kTimeForward = 0, kTimeBackward = 1, kTimeBinary = 2, kTimeDx = 3, kTimeOther = 4, kTimedKinds = 5 };
 struct TimedLaunch { hipEvent_t start, stop; int which; };
 bool g_timer_on = false;
+std::mutex g_timed_mtx;                      // guards g_timed: calls may come from several host threads
 std::vector<TimedLaunch> g_timed;
 
 struct ScopedTimer {
@@ -79,26 +80,37 @@ struct ScopedTimer {
     {
         if (!on) { return; }
         (void)hipEventRecord(t.stop, st);
+        std::lock_guard<std::mutex> lk(g_timed_mtx);
         g_timed.push_back(t);
     }
 };
 
+// integer tunable from the environment: unset, empty or negative = the default
 int env_int(char const *name, int def)
 {
     char const *s = getenv(name);
     if (!s || !*s) { return def; }
     int v = atoi(s);
-    return v > 0 ? v : def;
+    return v >= 0 ? v : def;
+}
+
+// on/off switch from the environment: 0 (or 2, the older spelling) = off, any other number = on, unset = the default
+bool env_switch(char const *name, bool def)
+{
+    char const *s = getenv(name);
+    if (!s || !*s) { return def; }
+    int v = atoi(s);
+    return !(v == 0 || v == 2);
 }
 
 // two-valued inputs (packed bits, fp32 binarized at 0.5): the kernels that look the LUT output up among the node's corner values
 bool use_corner_values(int xmode)
 {
-    static int const on = env_int("BBHIP_CORNER", 1);
-    return on == 1 && (xmode == kXBit || xmode == kXBinary);
+    static bool const on = env_switch("BBHIP_CORNER", true);
+    return on && (xmode == kXBit || xmode == kXBinary);
 }
 
-bool pack_binarized_input(void) { static int const on = env_int("BBHIP_PACK", 1); return on == 1; }
+bool pack_binarized_input(void) { static bool const on = env_switch("BBHIP_PACK", true); return on; }
 
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); return v >= 2 ? 2 : 1; }
@@ -122,31 +134,45 @@ int dx_pass_steps_env(void)   { static int v = env_int("BBHIP_DX_STEPS", 0); ret
 // BinaryLut6 units of 192 words: 8192 input rows x 768 bytes is what stays in an XCD's L2 next to the output stream
 // (256-word units fetch 2.3 GB per launch at the benchmark shape, 192-word units 1.9 GB; 128-word units fetch less still
 // but leave a wavefront too little work per set-up)
-int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 192); return ((v + 63) / 64) * 64; }
+int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 192); return (((v > 0 ? v : 192) + 63) / 64) * 64; }
 int bin_nodes_per_wave(void) { static int v = env_int("BBHIP_BIN_NODES", 0); return v >= 4 ? 4 : v >= 2 ? 2 : v == 1 ? 1 : 0; }     // 0: chosen per call
 
 // ------------------------------------------------------------------------------------------------
 //  scratch arena: one growing device buffer per device, reused by every call
 // ------------------------------------------------------------------------------------------------
 constexpr int kMaxDevices = 64;
-struct Arena { void *ptr = nullptr; size_t cap = 0; };
+// Blocks that a growing arena has left behind stay allocated: kernels already queued and HIP graphs captured earlier hold
+// their addresses.  bbhip_ReleaseScratch frees everything.
+struct Arena { void *ptr = nullptr; size_t cap = 0; std::vector<void *> retired; };
 Arena g_arena[kMaxDevices];
 
-int arena_get(size_t bytes, char **out)
+// Scratch for one call.  Either the library's arena (grown with hipMalloc where needed, never while the stream is being
+// captured) or, for the entry point that must not allocate, a fixed block handed in by the caller of run_forward.
+struct Scratch { char *fixed = nullptr; size_t fixed_cap = 0; };
+
+int arena_get(size_t bytes, char **out, hipStream_t st, Scratch const *fixed = nullptr)
 {
+    if (fixed && fixed->fixed) {
+        if (bytes > fixed->fixed_cap) { return fail("scratch of %zu bytes needed, the fixed block holds %zu", bytes, fixed->fixed_cap); }
+        *out = fixed->fixed;
+        return 0;
+    }
     int dev = 0;
     BBHIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) { return fail("device index %d out of range", dev); }
     Arena &a = g_arena[dev];
     if (a.cap < bytes) {
-        if (a.ptr) {
-            BBHIP_TRY(hipDeviceSynchronize());
-            BBHIP_TRY(hipFree(a.ptr));
-            a.ptr = nullptr;
-            a.cap = 0;
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) {
+            return fail("the scratch arena would have to grow from %zu to %zu bytes during stream capture: "
+                        "run the call once outside the capture, or bbhip_ReserveScratch first", a.cap, bytes);
         }
+        (void)hipGetLastError();
         size_t want = bytes + bytes / 2 + (1u << 20);
-        BBHIP_TRY(hipMalloc(&a.ptr, want));
+        void *p = nullptr;
+        BBHIP_TRY(hipMalloc(&p, want));
+        if (a.ptr) { a.retired.push_back(a.ptr); }
+        a.ptr = p;
         a.cap = want;
     }
     *out = static_cast<char *>(a.ptr);
@@ -361,7 +387,7 @@ int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_s
 }
 
 template <int N>
-int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
+int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch const *fixed = nullptr)
 {
     constexpr int NN = 1 << N;
     // input_rows: what the caller said about the input's row count (bbhip_HintInputNodeSize), 0 = nothing.
@@ -382,7 +408,7 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
     size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
     size_t const bits_bytes = pack ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + v_bytes + stat_bytes + bits_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + v_bytes + stat_bytes + bits_bytes, &base, st, fixed)) { return 1; }
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
@@ -437,13 +463,13 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st)
     return 0;
 }
 
-int forward_entry(ForwardCall const &c, void *stream)
+int forward_entry(ForwardCall const &c, void *stream, Scratch const *fixed = nullptr)
 {
-    int const input_rows = g_input_node_hint;       // the hint is spent by this call, whatever becomes of it
+    int const input_rows = fixed ? 0 : g_input_node_hint;       // the hint is spent by this call, whatever becomes of it
     g_input_node_hint = 0;
     if (check_forward(c)) { return 1; }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st));
+    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed));
     return 0;
 }
 
@@ -537,7 +563,7 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     size_t const v_bytes = corner ? c_bytes : 0;
     size_t const bits_bytes = pack ? align256((size_t)c.input_node_size * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes, &base)) { return 1; }
+    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes, &base, st)) { return 1; }
     float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
@@ -675,6 +701,7 @@ int run_backward(BackwardCall const &call, hipStream_t st)
 
 int backward_entry(BackwardCall const &c, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next forward call only
     hipStream_t st = static_cast<hipStream_t>(stream);
     BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st));
     return 0;
@@ -867,23 +894,68 @@ void bbhip_KernelTimer_Enable(int enable) { g_timer_on = enable != 0; }
 int bbhip_KernelTimer_Read(int which, float *total_ms, int *launches)
 {
     BBHIP_REQUIRE(which >= 0 && which < kTimedKinds && total_ms != nullptr && launches != nullptr);
+    // take the launches of this kind out of the list first; whatever happens below, none of them stays behind with
+    // destroyed events
+    std::vector<TimedLaunch> mine;
+    {
+        std::lock_guard<std::mutex> lk(g_timed_mtx);
+        std::vector<TimedLaunch> keep;
+        for (auto &t : g_timed) { (t.which == which ? mine : keep).push_back(t); }
+        g_timed.swap(keep);
+    }
     float total = 0.0f;
     int count = 0;
-    std::vector<TimedLaunch> keep;
-    for (auto &t : g_timed) {
-        if (t.which != which) { keep.push_back(t); continue; }
+    hipError_t first_error = hipSuccess;
+    for (auto &t : mine) {
         float ms = 0.0f;
-        BBHIP_TRY(hipEventSynchronize(t.stop));
-        BBHIP_TRY(hipEventElapsedTime(&ms, t.start, t.stop));
+        hipError_t e = hipEventSynchronize(t.stop);
+        if (e == hipSuccess) { e = hipEventElapsedTime(&ms, t.start, t.stop); }
         (void)hipEventDestroy(t.start);
         (void)hipEventDestroy(t.stop);
+        if (e != hipSuccess) { if (first_error == hipSuccess) { first_error = e; } continue; }
         total += ms;
         ++count;
     }
-    g_timed.swap(keep);
     *total_ms = total;
     *launches = count;
+    if (first_error != hipSuccess) { return fail("bbhip_KernelTimer_Read: %s", hipGetErrorString(first_error)); }
     return 0;
+}
+
+int bbhip_ReserveScratch(size_t bytes)
+{
+    char *p = nullptr;
+    return arena_get(bytes, &p, nullptr);
+}
+
+int bbhip_ReleaseScratch(void)
+{
+    int dev = 0;
+    BBHIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) { return fail("device index %d out of range", dev); }
+    BBHIP_TRY(hipDeviceSynchronize());
+    Arena &a = g_arena[dev];
+    for (void *p : a.retired) { (void)hipFree(p); }
+    a.retired.clear();
+    if (a.ptr) { (void)hipFree(a.ptr); }
+    a.ptr = nullptr;
+    a.cap = 0;
+    return 0;
+}
+
+size_t bbhip_GetScratchSize(void)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { (void)hipGetLastError(); return 0; }
+    return g_arena[dev].cap;
+}
+
+int bbhip_GetSwitch(char const *name)
+{
+    if (!name) { return -1; }
+    if (!strcmp(name, "corner")) { return use_corner_values(kXBit) ? 1 : 0; }
+    if (!strcmp(name, "pack"))   { return pack_binarized_input() ? 1 : 0; }
+    return -1;
 }
 
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
@@ -892,6 +964,7 @@ int  bbhip_GetDxMode(void) { return g_dx_mode; }
 
 int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_dst != nullptr && size >= 0);
     if (size == 0) { return 0; }
     hipLaunchKernelGGL(fill_kernel, dim3(ceil_div(size, kBlock * 4)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, a, (size_t)size);
@@ -901,6 +974,7 @@ int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)
 
 int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, float hi, int size, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_dst != nullptr && dev_src != nullptr && size >= 0);
     if (size == 0) { return 0; }
     hipLaunchKernelGGL(clamp_kernel, dim3(ceil_div(size, kBlock)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, dev_src, lo, hi, size);
@@ -909,27 +983,63 @@ int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, floa
 }
 
 int bbhip_fp32_Vector_add_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c, int size, void *stream)
-{ return vector_op<kVecAddEx>(dev_dst, dev_src0, dev_src1, a, b, c, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecAddEx>(dev_dst, dev_src0, dev_src1, a, b, c, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_mul_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, int size, void *stream)
-{ return vector_op<kVecMulEx>(dev_dst, dev_src0, dev_src1, a, b, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecMulEx>(dev_dst, dev_src0, dev_src1, a, b, 0.0f, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_div_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c, float d, int size, void *stream)
-{ return vector_op<kVecDivEx>(dev_dst, dev_src0, dev_src1, a, b, c, d, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecDivEx>(dev_dst, dev_src0, dev_src1, a, b, c, d, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_sqrt(float *dev_dst, float const *dev_src, int size, void *stream)
-{ return vector_op<kVecSqrt>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecSqrt>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_exp(float *dev_dst, float const *dev_src, int size, void *stream)
-{ return vector_op<kVecExp>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecExp>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_min(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream)
-{ return vector_op<kVecMin>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecMin>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_min_v(float *dev_dst, float const *dev_src, float a, int size, void *stream)
-{ return vector_op<kVecMinV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecMinV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_max(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream)
-{ return vector_op<kVecMax>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecMax>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
+}
+
 int bbhip_fp32_Vector_max_v(float *dev_dst, float const *dev_src, float a, int size, void *stream)
-{ return vector_op<kVecMaxV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__); }
+{
+    g_input_node_hint = 0;
+    return vector_op<kVecMaxV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__);
+}
 
 int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
                              float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(size >= 0 && size <= 65535);
     if (size == 0) { return 0; }
     BBHIP_REQUIRE(dev_size_table != nullptr && dev_params_buf_table != nullptr && dev_grads_buf_table != nullptr &&
@@ -948,6 +1058,7 @@ int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_st
                               int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
                               int border_mode, float border_value, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     Im2ColArgs a{dev_x_buf, dev_y_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  border_mode, border_value, 0, 0};
@@ -968,6 +1079,7 @@ int bbhip_bit_Im2Col_Forward(int const *dev_x_buf, int *dev_y_buf, int x_stride,
                              int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
                              int border_mode, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     Im2ColArgs a{dev_x_buf, dev_y_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  border_mode, 0.0f, 0, 0};
@@ -988,6 +1100,7 @@ int bbhip_fp32_Im2Col_Backward(float const *dev_dy_buf, float *dev_dx_buf, int x
                                int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
                                void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     Im2ColArgs a{dev_dy_buf, dev_dx_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  0, 0.0f, 0, 0};
@@ -1022,6 +1135,7 @@ static int check_col2im(void const *p, void const *q, int w, int h, int c, int n
 int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
                               int output_frame_size, int output_frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (check_col2im(dev_x_buf, dev_y_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, false, __func__)) { return 1; }
     int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
     long long const blocks = (long long)c_size * xy_tiles * f_tiles;
@@ -1036,6 +1150,7 @@ int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_si
 int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w_size, int h_size, int c_size, int input_frame_stride,
                                int output_frame_size, int output_frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (check_col2im(dev_dy_buf, dev_dx_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, false, __func__)) { return 1; }
     int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
     long long const blocks = (long long)c_size * xy_tiles * f_tiles;
@@ -1050,6 +1165,7 @@ int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w
 int bbhip_bit_Col2Im_Forward(int const *dev_x_buf, int *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
                              int output_frame_size, int output_frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (check_col2im(dev_x_buf, dev_y_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, true, __func__)) { return 1; }
     int const hw = h_size * w_size, words = (output_frame_size + 31) / 32;
     long long const total = (long long)c_size * hw * words;
@@ -1082,6 +1198,7 @@ static int launch_pool(PoolArgs const &a, bool backward, void *stream, char cons
 int bbhip_fp32_StochasticMaxPooling2x2_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size,
                                                int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     PoolArgs a{dev_x_buf, nullptr, dev_y_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
     return launch_pool(a, false, stream, __func__);
 }
@@ -1090,6 +1207,7 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
                                                 int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
                                                 int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     PoolArgs a{dev_x_buf, dev_dy_buf, dev_dx_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
     return launch_pool(a, true, stream, __func__);
 }
@@ -1107,6 +1225,7 @@ static int check_average_lut(void const *a, void const *b, int const *idx, int n
 int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                                   int frame_stride, int binarize_input, int binarize_output, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
     int const f_blocks = ceil_div(frame_size, kTailBlock);
     long long const blocks = (long long)node_size * f_blocks;
@@ -1121,6 +1240,7 @@ int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int 
 int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                                  int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     int const words = (frame_size > 0) ? ceil_div(frame_size, 32) : 0;
     if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, words, __func__)) { return 1; }
     int const w_blocks = ceil_div(words, kTailBlock);
@@ -1152,6 +1272,7 @@ int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const
 int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
                                    int output_node_size, int frame_size, int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (check_average_lut(dev_dy_buf, dev_dx_buf, dev_input_index, n, output_node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
     if (input_node_size <= 0) { return fail("%s: sizes must be positive", __func__); }
     int const total = output_node_size * n;
@@ -1160,7 +1281,7 @@ int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
     char *scratch = nullptr;
     size_t const offsets_bytes = align256(sizeof(int) * ((size_t)input_node_size + 1));
-    if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch)) { return 1; }
+    if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch, static_cast<hipStream_t>(stream))) { return 1; }
     int *offsets = reinterpret_cast<int *>(scratch), *list = reinterpret_cast<int *>(scratch + offsets_bytes);
     hipStream_t const st = static_cast<hipStream_t>(stream);
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
@@ -1176,6 +1297,7 @@ int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
 int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, float t_sum,
                                        int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (!(dev_y_buf && dev_t_buf && dev_dy_buf && dev_loss_buf)) { return fail("%s: null buffer", __func__); }
     if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -1187,7 +1309,7 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
     double *partial = dev_loss_buf;
     if (pix_size > 1) {
         char *scratch = nullptr;
-        if (arena_get(sizeof(double) * (size_t)pix_size * (size_t)frame_size, &scratch)) { return 1; }
+        if (arena_get(sizeof(double) * (size_t)pix_size * (size_t)frame_size, &scratch, st)) { return 1; }
         partial = reinterpret_cast<double *>(scratch);
     }
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
@@ -1204,6 +1326,7 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
 int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *dev_t_buf, int *dev_accuracy_buf, int *dev_category_buf,
                                           int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     if (!(dev_y_buf && dev_t_buf && dev_accuracy_buf && dev_category_buf)) { return fail("%s: null buffer", __func__); }
     if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -1219,6 +1342,7 @@ int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *d
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
                              int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr);
     BBHIP_REQUIRE(node_size > 0 && node_size <= 65535 * 1024 && frame_size > 0);
     BBHIP_REQUIRE(x_frame_stride >= (frame_size + 31) / 32 && y_frame_stride >= frame_size);
@@ -1423,6 +1547,7 @@ int bbhip_bit_fp32_DifferentiableLutN_Backward(int n, int const *dev_x_buf, floa
 int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
                                  int node_size, int frame_size, int frame_stride, void *stream)
 {
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr && dev_input_index != nullptr && dev_table != nullptr);
     BBHIP_REQUIRE(node_size > 0 && node_size <= (0x7fffffff >> 6) && frame_size > 0);
     BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);
