@@ -30,6 +30,10 @@ _SIGNATURES = {
     "bbhip_DeviceSynchronize": (C.c_int, []),
     "bbhip_KernelTimer_Enable": (None, [_i]),
     "bbhip_KernelTimer_Read": (C.c_int, [_i, C.POINTER(C.c_float), C.POINTER(C.c_int)]),
+    "bbhip_ReserveScratch": (C.c_int, [C.c_size_t]),
+    "bbhip_ReleaseScratch": (C.c_int, []),
+    "bbhip_GetScratchSize": (C.c_size_t, []),
+    "bbhip_GetSwitch": (C.c_int, [C.c_char_p]),
     "bbhip_SetDxMode": (None, [_i]),
     "bbhip_HintInputNodeSize": (None, [_i]),
     "bbhip_GetDxMode": (C.c_int, []),

@@ -20,6 +20,9 @@
  * Internal scratch (transformed tables, per-slab partial sums) comes from a library-owned arena that grows with
  * hipMalloc on demand and is reused by later calls; calls that overlap on one device (different host threads or
  * streams) race on it, exactly as the reference's allocator singleton is not thread-safe (cuda/LocalHeap.cu:174).
+ * A block that the arena outgrows stays allocated until bbhip_ReleaseScratch, so kernels already queued and HIP graphs
+ * captured earlier keep valid addresses; the arena never grows while the call's stream is being captured (the call fails
+ * with a message instead: run it once before the capture, or bbhip_ReserveScratch).
  */
 #ifndef BBHIP_H_
 #define BBHIP_H_
@@ -57,6 +60,21 @@ int bbhip_FreeHost(void *ptr);
 int bbhip_Memcpy(void *dst, void const *src, size_t size, int kind);
 int bbhip_Memset(void *dev_ptr, int value, size_t size);
 int bbhip_DeviceSynchronize(void);
+
+/* ---- scratch arena of the current device (no counterpart in the reference: its entry points take dx_tmp from the caller
+ * and allocate their other temporaries through the LocalHeap singleton) ----
+ * ReserveScratch grows the arena to at least `bytes` now, so that later calls (in particular captured ones) find it large
+ * enough.  ReleaseScratch waits for the device and frees the arena together with every block it has outgrown: HIP graphs
+ * captured before it must not be replayed afterwards.  GetScratchSize: bytes the arena holds at present. */
+int    bbhip_ReserveScratch(size_t bytes);
+int    bbhip_ReleaseScratch(void);
+size_t bbhip_GetScratchSize(void);
+
+/* ---- state of an environment switch as the library read it (instrumentation; no counterpart in the reference) ----
+ * name "corner" (BBHIP_CORNER: lookup kernels for two-valued inputs) or "pack" (BBHIP_PACK: binarized fp32 frames are
+ * packed to bits first): 1 on, 0 off, -1 unknown name.  A switch is off when its variable is 0 (or 2), on for any other
+ * number, and takes its default (on) when unset. */
+int bbhip_GetSwitch(char const *name);
 
 /* ---- how dx is accumulated over the fan-out of an input node (no counterpart in the reference) ----
  * 0 (default): deterministic, no scratch — one wavefront per (input node, frame chunk) walks reverse_index in the

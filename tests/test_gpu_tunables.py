@@ -11,7 +11,8 @@ pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-@pytest.mark.parametrize("env", [{}, {"BBHIP_CORNER": "2", "BBHIP_PACK": "2"}, {"BBHIP_PACK": "2"}, {"BBHIP_FWD_NODES": "1", "BBHIP_BWD_SLAB": "256"},
+@pytest.mark.parametrize("env", [{}, {"BBHIP_CORNER": "2", "BBHIP_PACK": "2"}, {"BBHIP_PACK": "2"}, {"BBHIP_CORNER": "0", "BBHIP_PACK": "0"},
+                                 {"BBHIP_CORNER": "0"}, {"BBHIP_FWD_NODES": "1", "BBHIP_BWD_SLAB": "256"},
                                  {"BBHIP_DX_STEPS": "1", "BBHIP_DX_CHUNK": "64", "BBHIP_BIN_NODES": "1", "BBHIP_BIN_CHUNK": "64"},
                                  {"BBHIP_DX_STEPS": "4", "BBHIP_DX_CHUNK": "512", "BBHIP_FWD_CHUNK": "512", "BBHIP_BIN_NODES": "2", "BBHIP_BIN_CHUNK": "256"}])
 def test_two_valued_inputs_under_switches(env):
@@ -20,3 +21,6 @@ def test_two_valued_inputs_under_switches(env):
     child_env["PYTHONPATH"] = os.pathsep.join([os.path.dirname(HERE), HERE, child_env.get("PYTHONPATH", "")])
     p = subprocess.run([sys.executable, os.path.join(HERE, "two_valued_case.py")], env=child_env, capture_output=True, text=True, timeout=300)
     assert p.returncode == 0 and "two-valued case ok" in p.stdout, (env, p.stdout[-2000:], p.stderr[-2000:])
+    # the switches took effect: 0 and 2 turn a path off, unset leaves it on
+    want = {name: 0 if env.get(var) in ("0", "2") else 1 for name, var in (("corner", "BBHIP_CORNER"), ("pack", "BBHIP_PACK"))}
+    assert "switches corner=%d pack=%d" % (want["corner"], want["pack"]) in p.stdout, (env, p.stdout[-500:])

@@ -54,6 +54,8 @@ def main():
     xbb = synth.bernoulli_bits(rng, I, Fb, synth.frame_stride_bit(Fb))
     yb = ops.binary_lut6_forward(dev(xbb), dev(idx), dev(T), Fb)
     assert np.array_equal(host(yb), oracle.binary_lut6_forward(xbb, idx, T, Fb))
+    from binarybrain_amd import capi
+    print("switches corner=%d pack=%d" % (capi.lib().bbhip_GetSwitch(b"corner"), capi.lib().bbhip_GetSwitch(b"pack")))
     print("two-valued case ok")
 
 
