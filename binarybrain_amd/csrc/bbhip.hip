@@ -20,6 +20,11 @@
 
 using namespace bbhip;
 
+// Scratch of bbhip_fp32_StochasticLut_Forward_NoAlloc: the transformed tables of one call (centred coefficients and, for
+// binarized inputs, corner values).  One copy per GPU, held until the process ends; every call on a GPU shares it.
+constexpr size_t kNoAllocScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
 namespace {
 
 // ------------------------------------------------------------------------------------------------
@@ -69,7 +74,7 @@ std::vector<TimedLaunch> g_timed;
 
 struct ScopedTimer {
     hipStream_t st; bool on; TimedLaunch t;
-    ScopedTimer(int which, hipStream_t s) : st(s), on(g_timer_on)
+    ScopedTimer(int which, hipStream_t s, bool allowed = true) : st(s), on(g_timer_on && allowed)
     {
         if (!on) { return; }
         t.which = which;
@@ -456,7 +461,7 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
         kind = 1;
     }
     {
-        ScopedTimer tm(kTimeForward, st);
+        ScopedTimer tm(kTimeForward, st, fixed == nullptr);     // (event creation may allocate: not on the path that must not)
         if (dispatch_forward<N>(c.xmode, c.ymode, kind, a, npw, st)) { return 1; }
     }
     BBHIP_LAUNCH_CHECK();
@@ -1369,6 +1374,46 @@ int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y
     c.xmode = input_binary ? kXBinary : kXClamp; c.ymode = kYClamp;
     c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
     return forward_entry(c, stream);
+}
+
+int bbhip_fp32_StochasticLut_Forward_NoAlloc(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                             float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                             int input_binary, int lut_binarize, float unbinarize_bias, void *stream)
+{
+    // device address of the file-scope scratch array, looked up once per device with that device current (the array's
+    // name is only a host-side handle; each GPU holds its own copy at its own address)
+    static void      *scratch_ptr[kMaxDevices] = {};
+    static std::mutex scratch_mtx;
+    int dev = 0;
+    BBHIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) { return fail("device index %d out of range", dev); }
+    void *base = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(scratch_mtx);
+        if (!scratch_ptr[dev]) {
+            void *p = nullptr;
+            BBHIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            scratch_ptr[dev] = p;
+        }
+        base = scratch_ptr[dev];
+    }
+    if (n < 2 || n > 6) { return fail("LUT width n=%d not in 2..6", n); }
+    // both tables of a call must fit: [node_size][2^n] floats each, rounded to 256 bytes
+    size_t const table = align256((size_t)(node_size > 0 ? node_size : 0) * ((size_t)1 << n) * sizeof(float));
+    size_t const need  = table * (input_binary ? 2 : 1);
+    if (need > kNoAllocScratchBytes) {
+        return fail("bbhip_fp32_StochasticLut_Forward_NoAlloc: node_size=%d at n=%d needs %zu bytes of scratch, the fixed block holds %zu "
+                    "(use bbhip_fp32_StochasticLut_Forward)", node_size, n, need, (size_t)kNoAllocScratchBytes);
+    }
+    Scratch fixed;
+    fixed.fixed = static_cast<char *>(base);
+    fixed.fixed_cap = kNoAllocScratchBytes;
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = input_binary ? kXBinary : kXClamp; c.ymode = kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return forward_entry(c, stream, &fixed);
 }
 
 int bbhip_bit_fp32_StochasticLut_Forward(int n, int const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,

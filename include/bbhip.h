@@ -223,6 +223,16 @@ int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *d
 int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
                                      float const *dev_W, int node_size, int frame_size, int frame_stride,
                                      int input_binary, int lut_binarize, float unbinarize_bias, void *stream);
+/* No counterpart in the reference.  bbhip_fp32_StochasticLut_Forward for callers that cannot allocate device memory — code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc: same arguments and results, but the
+ * tables that the kernels read come from a fixed 8 MiB block inside the library (one per GPU, held until the process
+ * ends) instead of the growing arena, and the call never calls hipMalloc, hipFree or any allocating routine.  Limit:
+ * node_size * 2^n * 4 bytes (twice that with input_binary) must fit the block — 32768 nodes (16384 with input_binary)
+ * at n = 6; larger layers are rejected with a message.  bbhip_HintInputNodeSize is ignored and the kernel timer does not
+ * record this entry.  All calls on a GPU share the block: calls that overlap on one GPU (two streams, two threads) race. */
+int bbhip_fp32_StochasticLut_Forward_NoAlloc(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                             float const *dev_W, int node_size, int frame_size, int frame_stride,
+                                             int input_binary, int lut_binarize, float unbinarize_bias, void *stream);
 /* bbcu_bit_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:683-697 */
 int bbhip_bit_fp32_StochasticLut_Forward(int n, int const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
                                          float const *dev_W, int node_size, int frame_size, int frame_stride,
