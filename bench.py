@@ -120,10 +120,10 @@ def bench_adam(args, lib):
         oracle.adam_steps(p, [gr] * reps)
         out["cpu_baseline"] = {"value": n * reps / (time.perf_counter() - t) / 1e9, "unit": "G updates/s", "cores": 1, "kind": "port",
                                "sample": "C restatement of the reference's host update, one tensor of %d elements, %d steps" % (n, reps)}
-    print(json.dumps(out))
+    return out
 
 
-def library_timed_ms(lib, fn, steps, warmup):
+def library_timed_ms(lib, fn, steps, warmup, which=4):
     """Mean duration (ms) of the kernels one call of fn launches, from the HIP events that the library records around
     them on the launch stream (kind 4: the entries outside the LUT layers).  Events recorded by the caller would span
     the Python call as well, which is longer than these kernels."""
@@ -139,7 +139,7 @@ def library_timed_ms(lib, fn, steps, warmup):
     torch.cuda.synchronize()
     lib.bbhip_KernelTimer_Enable(0)
     ms = C.c_float(0); cnt = C.c_int(0)
-    capi.check(lib.bbhip_KernelTimer_Read(4, C.byref(ms), C.byref(cnt)))
+    capi.check(lib.bbhip_KernelTimer_Read(which, C.byref(ms), C.byref(cnt)))
     assert cnt.value == steps, (cnt.value, steps)
     return ms.value / cnt.value
 
@@ -185,7 +185,7 @@ def bench_conv(args, lib):
            "roofline": {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},
            "kernels": kernels}
-    print(json.dumps(out))
+    return out
 
 
 def bench_tail(args, lib):
@@ -231,7 +231,7 @@ def bench_tail(args, lib):
            "roofline": {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},
            "kernels": kernels}
-    print(json.dumps(out))
+    return out
 
 
 def bench_differentiablelut6(args, lib):
@@ -290,7 +290,7 @@ def bench_differentiablelut6(args, lib):
                                   % ("packed-bit activations, fp32 gradients" if bits else "fp32")},
            "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
-    print(json.dumps(out))
+    return out
 
 
 def conv_block_layers(rng, synth, ops, torch, np):
@@ -384,7 +384,7 @@ def bench_conv_block(args, lib):
         out["cpu_baseline"] = {"value": sum(l["O"] for l in layers) * FWs / cpu_dt / 1e9, "unit": "G node-evals/s", "cores": 1, "kind": "port",
                                "sample": "the same block on %d images through the C restatement of the reference's host path (generic DifferentiableLut "
                                          "algorithm, whose batch-norm backward is single-threaded in the reference too)" % Fs}
-    print(json.dumps(out))
+    return out
 
 
 def bench_mnist_step(args, lib):
@@ -489,7 +489,7 @@ def bench_mnist_step(args, lib):
         out["cpu_baseline"] = {"value": 1.0 / cpu_dt, "unit": "steps/s", "cores": 1, "kind": "port",
                                "sample": "one forward + backward of the same network through the C restatement of the reference's generic "
                                          "DifferentiableLut path (its batch-norm backward is single-threaded in the reference too), Adam not included"}
-    print(json.dumps(out))
+    return out
 
 
 def bench_binarylut6(args, lib):
@@ -504,6 +504,11 @@ def bench_binarylut6(args, lib):
     T = torch.from_numpy(synth.truth_tables(rng, O)).cuda()
     x = torch.from_numpy(synth.bernoulli_bits(rng, I, F, SW)).cuda()
     y = torch.zeros((O, SW), dtype=torch.int32, device="cuda")
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < args.ramp_seconds:      # untimed: the device reaches its sustained clock under load
+        for _ in range(10):
+            ops.binary_lut6_forward(x, idx, T, F, out=y)
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         ops.binary_lut6_forward(x, idx, T, F, out=y)
     torch.cuda.synchronize()
@@ -550,52 +555,14 @@ def bench_binarylut6(args, lib):
         out["cpu_baseline"] = {"value": O * fs / best / 1e12, "unit": "T node-evals/s", "cores": min(os.cpu_count() or 1, 16),
                                "kind": "reference" if oracle.have_ref() else "port",
                                "sample": "BinaryLut6 forward (AVX2+OpenMP host path incl. harness copies), 8192 -> 16384 nodes, 8192 of the 262144 frames, best of 3"}
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=100,
-                    help="untimed steps first; the device needs a few dozen steps of load to reach its sustained clock")
-    ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "0")),
-                    help="0: deterministic input-centric dx; 1: fp32 atomics; 2: dx_tmp + reverse table")
-    ap.add_argument("--ramp-seconds", type=float, default=0.3,
-                    help="before the warm-up steps, keep the device under the same load for this long (untimed): from idle it "
-                         "takes a few dozen steps to reach its sustained clock, whatever --warmup says")
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--profile-copy", action="store_true",
-                    help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail"],
-                    help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
-    ap.add_argument("--cpu-frames", type=int, default=8192)
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path would shard over the "
-              "frame axis; no multi-GPU code is built)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-
+def bench_stochasticlut6(args, lib):
+    """The headline workload: W clamp + StochasticLut6 forward + backward (dW, dx), fp32, 4096 -> 4096 nodes, 8192 frames."""
     import numpy as np
     import torch
     from binarybrain_amd import capi, ops, synth
-
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    lib = capi.lib()
-    if args.workload == "binarylut6":
-        return bench_binarylut6(args, lib)
-    if args.workload == "adam":
-        return bench_adam(args, lib)
-    if args.workload == "conv":
-        return bench_conv(args, lib)
-    if args.workload == "tail":
-        return bench_tail(args, lib)
-    if args.workload in ("differentiablelut6", "differentiablelut6_bit"):
-        return bench_differentiablelut6(args, lib)
-    if args.workload == "mnist_step":
-        return bench_mnist_step(args, lib)
-    if args.workload == "conv_block":
-        return bench_conv_block(args, lib)
     I = O = 4096
     F = 8192
     rng = np.random.default_rng(0)
@@ -622,10 +589,13 @@ def main():
         ops.stochastic_lut_backward(6, x, dy, idx, W, dW, F, rev, dx_tmp=dx_tmp, tmp_frame_size=tmp_frames, out=dx)
 
     t_ramp = time.perf_counter()
+    ramp_steps = 0
     while time.perf_counter() - t_ramp < args.ramp_seconds:
         for _ in range(10):
             step()
+        ramp_steps += 10
         torch.cuda.synchronize()
+    ramp_done = time.perf_counter() - t_ramp
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -677,6 +647,10 @@ def main():
         "unit": "G node-evals/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "ms_per_step_with_kernel_events": dt_events / args.steps * 1e3,
+        # the per-kernel times below come from the second pass, whose event records (about 3 us each on the device) make it
+        # this much slower than the timed region: kernel times sum to slightly more than ms_per_step
+        "event_pass_inflation": dt_events / dt,
+        "ramp_seconds": ramp_done, "ramp_steps": ramp_steps,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "StochasticLut6 fwd+bwd fp32, 4096 in x 4096 out x 8192 frames, uniform random 6-of-4096 wiring",
                    "dx_mode": ["deterministic (input-centric, reverse table)", "atomic", "dx_tmp + reverse table"][args.dx_mode],
@@ -694,7 +668,148 @@ def main():
         out["profile_copy_bytes"] = int(x.numel() * 4)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(I, O, args.cpu_frames, os.cpu_count() if (os.cpu_count() or 1) <= 16 else 16)
-    print(json.dumps(out))
+    return out
+
+
+def bench_forward_small(args, lib):
+    """BASELINE configuration 1: StochasticLut6 forward only, 784 -> 1024 nodes, 64 frames (the case the reference's CPU path
+    runs as is).  Two launches (table preparation, forward) of a few microseconds: the figure is launch latency."""
+    import numpy as np
+    import torch
+    from binarybrain_amd import ops, synth
+    I, O, F = 784, 1024, 64
+    rng = np.random.default_rng(0)
+    S = synth.frame_stride_fp32(F)
+    idx_h = synth.wiring(rng, I, O); W_h = synth.lut_tables(rng, O); x_h = synth.uniform_frames(rng, I, F, S)
+    idx = torch.from_numpy(idx_h).cuda(); W = torch.from_numpy(W_h).cuda(); x = torch.from_numpy(x_h).cuda()
+    y = torch.empty((O, S), device="cuda")
+
+    def step():
+        ops.stochastic_lut_forward(6, x, idx, W, F, out=y)
+
+    for _ in range(max(args.warmup, 20)):
+        step()
+    torch.cuda.synchronize()
+    steps = max(args.steps, 200)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    kernel_ms = library_timed_ms(lib, step, steps, 5, which=0)
+    nbytes = 4 * F * (I + O) + 280 * O
+    out = {"metric": "G node-evals/s StochasticLut6 fp32 forward (784 -> 1024 nodes, 64 frames)", "value": O * F / dt / 1e9,
+           "unit": "G node-evals/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 20), "ms_per_step": dt * 1e3,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "StochasticLut6 forward fp32, 784 in x 1024 out x 64 frames (launch-bound: two launches per call)"},
+           "roofline": {"bound": "hbm", "kernel": "lut_forward_kernel<6>", "achieved": nbytes / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                        "unit": "GB/s", "frac": nbytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "kernel_ms": kernel_ms}}
+    if not args.no_cpu:
+        import oracle
+        best = None
+        for _ in range(20):
+            t1 = time.perf_counter()
+            if oracle.have_ref():
+                oracle.ref_stochastic_lut(6, x_h, idx_h, W_h)
+            else:
+                oracle.stochastic_lut_forward(6, x_h, idx_h, W_h, F)
+            d = time.perf_counter() - t1
+            best = d if best is None else min(best, d)
+        out["cpu_baseline"] = {"value": O * F / best / 1e9, "unit": "G node-evals/s", "cores": min(os.cpu_count() or 1, 16),
+                               "kind": "reference" if oracle.have_ref() else "port",
+                               "sample": "the whole configuration (AVX2+OpenMP host Forward incl. the harness's buffer copies), best of 20"}
+    return out
+
+
+def bench_gather_ceiling(args, lib):
+    """What the GPU sustains on the dx kernel's access pattern alone (instrumentation): per (input row, 128-frame window) 36
+    pseudo-randomly chosen rows' 512-byte segments are read and discarded — 6 consumers x (5 rows + dy) as in the headline
+    shape.  Reported as a rate through L1; the dx kernel moves the same bytes and does its arithmetic on top."""
+    import torch
+    from binarybrain_amd import capi, synth
+    from binarybrain_amd.capi import ptr, stream_ptr
+    I, F = 4096, 8192
+    S = synth.frame_stride_fp32(F)
+    x = torch.rand((I, S), device="cuda")
+    sink = torch.zeros(1, device="cuda")
+    loads = 36
+
+    def step():
+        capi.check(lib.bbhip_Probe_RowGather(ptr(x), ptr(sink), I, F, S, loads, stream_ptr()))
+
+    kernel_ms = library_timed_ms(lib, step, max(args.steps, 20), max(args.warmup, 20))
+    nbytes = I * (F // 128) * loads * 512
+    return {"metric": "TB/s of gathered 512-byte row segments through L1 (access pattern of the dx kernel, no arithmetic)",
+            "value": nbytes / (kernel_ms * 1e-3) / 1e12, "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 20),
+            "ms_per_step": kernel_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "row gather probe, 4096 rows x 8192 frames, 36 row segments per (row, 128 frames)", "bytes_per_launch": nbytes}}
+
+
+def other_configs(args, lib):
+    """The other BASELINE configurations, measured after the headline workload in the same process: configuration 1 (forward
+    784 -> 1024 x 64), 3 (classifier training step), 4 (BinaryLut6 inference), 5 (convolutional block), and the gather
+    ceiling that the dx kernel is judged against.  Each entry keeps its own roofline and CPU baseline."""
+    import copy
+    sub = copy.copy(args)
+    sub.ramp_seconds = min(args.ramp_seconds, 0.15)
+    sub.profile_copy = False
+    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "dtype", "config", "roofline", "cpu_baseline")
+    out = {}
+    for name, fn, workload in (("cfg1_forward_784x1024x64", bench_forward_small, "forward_784x1024x64"),
+                               ("cfg3_mnist_step", bench_mnist_step, "mnist_step"),
+                               ("cfg4_binarylut6", bench_binarylut6, "binarylut6"),
+                               ("cfg5_conv_block", bench_conv_block, "conv_block"),
+                               ("dx_gather_ceiling", bench_gather_ceiling, "gather_ceiling")):
+        sub.workload = workload
+        r = fn(sub, lib)
+        out[name] = {k: r[k] for k in keep if k in r}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed steps first; the device needs a few dozen steps of load to reach its sustained clock")
+    ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "0")),
+                    help="0: deterministic input-centric dx; 1: fp32 atomics; 2: dx_tmp + reverse table")
+    ap.add_argument("--ramp-seconds", type=float, default=0.3,
+                    help="before the warm-up steps, keep the device under the same load for this long (untimed): from idle it "
+                         "takes a few dozen steps to reach its sustained clock, whatever --warmup says")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="headline workload only: skip the other BASELINE configurations that the default run reports under `configs`")
+    ap.add_argument("--profile-copy", action="store_true",
+                    help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail",
+                             "forward_784x1024x64", "gather_ceiling"],
+                    help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
+    ap.add_argument("--cpu-frames", type=int, default=8192)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path would shard over the "
+              "frame axis; no multi-GPU code is built)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from binarybrain_amd import capi, ops, synth
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    lib = capi.lib()
+    secondary = {"binarylut6": bench_binarylut6, "adam": bench_adam, "conv": bench_conv, "tail": bench_tail,
+                 "differentiablelut6": bench_differentiablelut6, "differentiablelut6_bit": bench_differentiablelut6,
+                 "mnist_step": bench_mnist_step, "conv_block": bench_conv_block, "forward_784x1024x64": bench_forward_small,
+                 "gather_ceiling": bench_gather_ceiling}
+    if args.workload in secondary:
+        print(json.dumps(secondary[args.workload](args, lib)))
+        return
+    res = bench_stochasticlut6(args, lib)
+    if not args.no_configs:
+        res["configs"] = other_configs(args, lib)
+    print(json.dumps(res))
 
 
 if __name__ == "__main__":

@@ -963,6 +963,19 @@ int bbhip_GetSwitch(char const *name)
     return -1;
 }
 
+int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit, void *stream)
+{
+    BBHIP_REQUIRE(dev_x != nullptr && dev_sink != nullptr && row_count > 0 && frame_size > 0 && frame_stride >= frame_size && loads_per_unit > 0);
+    int const chunk_count = ceil_div(frame_size, 128), tile_count = ceil_div(row_count, kWavesPerBlk);
+    BBHIP_REQUIRE((long long)chunk_count * tile_count <= 0x7fffffffLL);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    hipLaunchKernelGGL(row_gather_probe_kernel, dim3(chunk_count * tile_count), dim3(kBlock), 0, st, dev_x, dev_sink, row_count, frame_stride,
+                       frame_size, chunk_count, make_tile_divisor(tile_count), loads_per_unit);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
 void bbhip_HintInputNodeSize(int input_node_size) { g_input_node_hint = input_node_size > 0 ? input_node_size : 0; }
 int  bbhip_GetDxMode(void) { return g_dx_mode; }

@@ -1211,6 +1211,42 @@ __global__ __launch_bounds__(kBlock) void dx_gather_kernel(float const *__restri
 }
 
 // ------------------------------------------------------------------------------------------------
+//  Instrumentation: the gather pattern of lut_dx_kernel without its arithmetic.  One wavefront per (row, 128-frame unit),
+//  units dealt to the XCDs as everywhere; it reads `loads` pseudo-randomly chosen rows' 512-byte segments of its frame window,
+//  twelve 256-byte loads in flight at a time like a dx term, and adds them up.  What this kernel sustains is the rate at
+//  which this GPU delivers gathered row segments from L2 to the compute units — the practical ceiling of any kernel with
+//  the dx kernel's access pattern.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void row_gather_probe_kernel(float const *__restrict__ x, float *__restrict__ sink, int rows, int stride,
+                                                                  int frame_size, int chunk_count, TileDivisor tiles, int loads)
+{
+    int const B   = chunk_count * tiles.count;
+    int const lid = xcd_remap(blockIdx.x, B);
+    int ck, tile;
+    split_tile(lid, tiles, ck, tile);
+    int const lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (tile * kWavesPerBlk + wave >= rows) { return; }
+    uint32_t s = (uint32_t)(lid * kWavesPerBlk + wave) * 2654435761u + 12345u;
+    int const f_last = frame_size - 1;
+    uint32_t const o0 = (uint32_t)min(ck * 128 + lane, f_last) * 4u, o1 = (uint32_t)min(ck * 128 + kWave + lane, f_last) * 4u;
+    float acc = 0.0f;
+    for (int r = 0; r < loads; r += 6) {
+        float v[6][2];
+#pragma unroll
+        for (int j = 0; j < 6; ++j) {
+            s = s * 1664525u + 1013904223u;
+            int const row = __builtin_amdgcn_readfirstlane((int)((s >> 8) % (uint32_t)rows));
+            char const *p = reinterpret_cast<char const *>(x + (size_t)row * stride);
+            v[j][0] = *reinterpret_cast<float const *>(p + o0);
+            v[j][1] = *reinterpret_cast<float const *>(p + o1);
+        }
+#pragma unroll
+        for (int j = 0; j < 6; ++j) { acc += v[j][0] + v[j][1]; }
+    }
+    if (acc == 123.456f) { sink[0] = acc; }                 // (never true for the buffers it is run on; keeps the loads alive)
+}
+
+// ------------------------------------------------------------------------------------------------
 //  elementwise helpers
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void fill_kernel(float *__restrict__ dst, float v, size_t size)

@@ -183,43 +183,66 @@ struct LutEval {
 //  v_mfma_f32_4x4x1_16b_f32 performs, for each of the 16 lane quads b of a wavefront, the rank-1 update
 //      D_b[r][c] += A_b[r] * B_b[c],      A_b[r] = srcA of lane 4b + r,   B_b[c] = srcB of lane 4b + c,
 //  and returns D_b[r][c] in result register r of lane 4b + c.  With srcB = l[i] of the lane's own frame and
-//  srcA = C[(4g + r)*L + i] (the same in every quad), L - 1 such updates starting from the constant terms leave
-//  q[4g + r] of the lane's own frame in result register r: 4 coefficients per lane and instruction instead of 1,
-//  with the frames staying one per lane and no data movement between lanes.
+//  srcA = C[(4g + r)*L + i] (the same for every quad), L such updates (l[0] = 1) leave q[4g + r] of the lane's own
+//  frame in result register r: 4 coefficients per lane and instruction instead of 1, with the frames staying one per
+//  lane and no data movement between lanes.  The instruction's broadcast control (cbsz = 4, abid = s) makes all 16
+//  quads take their A values from quad s of the source register, so the coefficients of 16 updates sit in one register.
 // ------------------------------------------------------------------------------------------------
 typedef float mfma_f4 __attribute__((ext_vector_type(4)));
 
+// One update with the A operand broadcast from lane quad SLOT to all 16 quads (cbsz = 4, abid = SLOT):
+//     D[r] (own lane) += A(lane 4 SLOT + r) * B(own lane)
+// A single vector register then carries 16 updates' worth of coefficients: a whole 64-entry table.
+template <int SLOT>
+__device__ __forceinline__ mfma_f4 mfma_broadcast(float a, float b, mfma_f4 d)
+{
+    static_assert(SLOT >= 0 && SLOT < 16, "a register holds 16 quads");
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, d, 4, SLOT, 0);
+}
+
+// sum over i < COUNT of A(quad BASE + i) * b[i], four results per lane (the quad index must be a compile-time constant)
+template <int BASE, int COUNT, int I = 0>
+__device__ __forceinline__ mfma_f4 mfma_broadcast_chain(float a, float const (&b)[COUNT], mfma_f4 d)
+{
+    d = mfma_broadcast<BASE + I>(a, b[I], d);
+    if constexpr (I + 1 < COUNT) { return mfma_broadcast_chain<BASE, COUNT, I + 1>(a, b, d); }
+    else                         { return d; }
+}
+
+// out[4 g + v] = sum_i A(quad g * COUNT + i)[v] * b[i] for g < GROUPS
+template <int GROUPS, int COUNT, int G = 0>
+__device__ __forceinline__ void mfma_broadcast_matvec(float a, float const (&b)[COUNT], float (&out)[GROUPS * 4])
+{
+    mfma_f4 const d = mfma_broadcast_chain<G * COUNT, COUNT>(a, b, mfma_f4{0.0f, 0.0f, 0.0f, 0.0f});
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { out[4 * G + v] = d[v]; }
+    if constexpr (G + 1 < GROUPS) { mfma_broadcast_matvec<GROUPS, COUNT, G + 1>(a, b, out); }
+}
+
+// The node's whole table in ONE vector register: lane 4 s + r holds C[(4 g + r) * L + i] for update s = g * L + i, and each
+// update takes its A operand from quad s of that register (the loads of a wavefront cover the table's 2^N consecutive
+// floats once, in permuted order).
 template <int N>
 struct LutMatrixQ {
     using D = LutDims<N>;
-    static constexpr bool kUsable = (D::H % 4 == 0) && (D::L >= 4);
+    static constexpr bool kUsable = (D::H % 4 == 0) && (D::L >= 4) && ((D::H / 4) * D::L <= 16);
     static constexpr int  G = (D::H >= 4) ? D::H / 4 : 1;     // groups of 4 partial sums
 
-    float   a[G][D::L];      // a[g][i]: coefficient C[(4g + lane%4)*L + i]   (i >= 1 used)
-    mfma_f4 c0[G];           // c0[g][r]: constant term C[(4g + r)*L], identical in all lanes
+    float t;
 
-    __device__ __forceinline__ void load(float const *__restrict__ Cg, int lane)
+    __device__ __forceinline__ static int table_index(int lane)
     {
-        int const r = lane & 3;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-#pragma unroll
-            for (int i = 1; i < D::L; ++i) { a[g][i] = Cg[(4 * g + r) * D::L + i]; }
-#pragma unroll
-            for (int v = 0; v < 4; ++v) { c0[g][v] = Cg[(4 * g + v) * D::L]; }
-        }
+        int const s = lane >> 2, r = lane & 3;
+        int const g = s / D::L, i = s % D::L;
+        int const e = (4 * g + r) * D::L + i;
+        return e < D::NN ? e : D::NN - 1;                      // (lanes beyond the updates of a narrow table: any entry)
     }
+
+    __device__ __forceinline__ void load(float const *__restrict__ Cg, int lane) { t = Cg[table_index(lane)]; }
 
     __device__ __forceinline__ void partial_q(float const (&l)[D::L], float (&q)[D::H]) const
     {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            mfma_f4 acc = c0[g];
-#pragma unroll
-            for (int i = 1; i < D::L; ++i) { acc = __builtin_amdgcn_mfma_f32_4x4x1f32(a[g][i], l[i], acc, 0, 0, 0); }
-#pragma unroll
-            for (int v = 0; v < 4; ++v) { q[4 * g + v] = acc[v]; }
-        }
+        mfma_broadcast_matvec<G, D::L>(t, l, q);
     }
 
     // y for one frame from the centred inputs z[0..N-1]

@@ -105,6 +105,15 @@ void bbhip_HintInputNodeSize(int input_node_size);
 void bbhip_KernelTimer_Enable(int enable);
 int  bbhip_KernelTimer_Read(int which, float *total_ms, int *launches);
 
+/* ---- gather probe (instrumentation; no counterpart in the reference) ----
+ * Runs the memory access pattern of the input-centric dx kernel without its arithmetic: one wavefront per (row, 128-frame
+ * window) reads `loads_per_unit` (rounded up to a multiple of 6) pseudo-randomly chosen rows' 512-byte segments of that
+ * window from dev_x [row_count][frame_stride] and discards them.  Bytes moved per launch:
+ * row_count * ceil(frame_size / 128) * loads_per_unit * 512.  Timed by the kernel timer as kind 4.  Used by bench.py to put
+ * a measured ceiling next to the dx kernel's rate.  dev_sink: one float that is never written in practice. */
+int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
+                          void *stream);
+
 /* ---- elementwise helpers ---- */
 /* bbcu_fp32_Vector_set, include/bbcu/bbcu.h:89-94 */
 int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream);
