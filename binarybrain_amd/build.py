@@ -34,10 +34,10 @@ def build_library(verbose=False):
 
 
 def build_cpp_tests(verbose=False):
-    """tests/cpp/test_host and object_tool (CPU) and tests/cpp/test_models (GPU): plain host C++ over the C ABI; the oracle
-    library is linked as the checker."""
+    """tests/cpp/test_host, object_tool and test_binding (CPU; test_binding --gpu runs on the device) and tests/cpp/test_models
+    (GPU): plain host C++ over the C ABI; the oracle library is linked as the checker."""
     out = []
-    for name in ("test_host", "test_models", "object_tool"):
+    for name in ("test_host", "test_models", "object_tool", "test_binding"):
         exe = os.path.join(ROOT, "tests", "cpp", name)
         _run(["g++", "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "include"),
               os.path.join(ROOT, "tests", "cpp", name + ".cpp"), "-o", exe,

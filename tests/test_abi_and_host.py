@@ -62,3 +62,15 @@ def test_host_side_cpp():
         build_cpp_tests()
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert res.returncode == 0, res.stdout
+
+
+def test_binding_header_signatures():
+    """include/bbcu_hip_binding.h gives every entry the reference's name and parameter list: tests/cpp/test_binding.cpp holds
+    the reference's declarations (include/bbcu/bbcu.h) as function-pointer types and static_asserts each one, for the LUT
+    widths 2..6; compiling it is the test, running it prints the count."""
+    exe = os.path.join(ROOT, "tests", "cpp", "test_binding")
+    if not os.path.exists(exe):
+        from binarybrain_amd.build import build_cpp_tests
+        build_cpp_tests()
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode == 0 and "signatures equal the reference's declarations" in res.stdout, res.stdout

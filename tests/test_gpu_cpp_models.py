@@ -16,3 +16,13 @@ def test_cpp_model_classes():
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
     print(res.stdout)
     assert res.returncode == 0, res.stdout
+
+
+def test_layer_through_the_reference_named_binding():
+    """One StochasticLut6 forward + backward called through the templates of include/bbcu_hip_binding.h (the reference's
+    names, default width and default stream) equals the same calls on the C ABI bit for bit; a rejected call throws."""
+    exe = os.path.join(ROOT, "tests", "cpp", "test_binding")
+    assert os.path.exists(exe), "tests/cpp/test_binding is missing: run __graft_entry__.build()"
+    res = subprocess.run([exe, "--gpu"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    print(res.stdout)
+    assert res.returncode == 0, res.stdout
