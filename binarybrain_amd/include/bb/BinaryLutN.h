@@ -6,6 +6,7 @@
 
 #include <random>
 
+#include "bb/ConnectionPolicy.h"
 #include "bb/Model.h"
 
 namespace bb {
@@ -131,24 +132,27 @@ public:
         m_input_shape = shape;
         index_t const I = CalcShapeSize(shape), O = this->GetOutputNodeSize();
         BB_ASSERT(I >= N);
-        // seeded default wiring (distinct inputs per node) and random tables (reference: BinaryLutN.h:201-218)
+        // seeded wiring by policy, then random tables: one draw of the layer's generator seeds each, and the table bits come
+        // from a generator of their own, entry by entry (reference: BinaryLutN.h:201-218, SparseModel.h:97-233,
+        // BinaryLutModel.h:45-59)
         {
             auto idx = m_input_index.Lock(true);
-            std::uniform_int_distribution<index_t> pick(0, I - 1);
-            for (index_t o = 0; o < O; ++o) {
-                for (int i = 0; i < N; ++i) {
-                    for (;;) {
-                        std::int32_t const c = (std::int32_t)pick(m_mt);
-                        bool dup = false;
-                        for (int j = 0; j < i; ++j) { dup = dup || (idx(o, j) == c); }
-                        if (!dup) { idx(o, i) = c; break; }
-                    }
-                }
-            }
+            connection_policy::Initialize(m_mt(), m_connection, m_input_shape, m_output_shape, N, connection_policy::Layout::kChannelLast,
+                                          [&](index_t node, int i, index_t input) {
+                                              BB_ASSERT(input >= 0 && input < I);
+                                              idx(node, (index_t)i) = (std::int32_t)input;
+                                          });
         }
         {
+            std::mt19937_64 mt(m_mt());
+            std::uniform_int_distribution<int> coin(0, 1);
             auto tbl = m_table.Lock(true);
-            for (index_t o = 0; o < O; ++o) { for (int u = 0; u < kTableUnit; ++u) { tbl(o, u) = (std::int32_t)(std::uint32_t)m_mt(); } }
+            for (index_t o = 0; o < O; ++o) {
+                for (int u = 0; u < kTableUnit; ++u) { tbl(o, u) = 0; }
+                for (int i = 0; i < kTableSize; ++i) {
+                    if (coin(mt) != 0) { tbl(o, i / 32) = (std::int32_t)((std::uint32_t)tbl(o, i / 32) | (1u << (i % 32))); }
+                }
+            }
         }
         return m_output_shape;
     }

@@ -6,9 +6,8 @@
 #pragma once
 
 #include <algorithm>
-#include <numeric>
-#include <random>
 
+#include "bb/ConnectionPolicy.h"
 #include "bb/Core.h"
 #include "bb/Tensor.h"
 
@@ -49,39 +48,18 @@ public:
         m_reverse_table_dirty = true;
     }
 
-    // Seeded wiring.  "serial": node o reads inputs (o*N + i) mod I.  Anything else ("", "random"): inputs are dealt from
-    // reshuffled decks of all input nodes so that every input is used about equally often and the N inputs of a
-    // node are distinct (the balance property of the reference's random policy, include/bb/ShuffleSet.h:62-102;
-    // the exact permutation is a property of the random-number library and is not part of the contract —
-    // inject wiring with SetInputConnection where it has to match another implementation).
+    // Seeded wiring by policy ("" or "random", "serial", "pointwise", "depthwise", "gauss": bb/ConnectionPolicy.h; reference:
+    // include/bb/ConnectionTable.h:150-284).  An unknown policy string throws.
     void InitializeConnection(std::uint64_t seed, std::string const &connection = "")
     {
-        BB_ASSERT(m_input_node_size >= N);
+        BB_ASSERT(m_input_node_size >= 1);
         auto tbl = m_input_table.Lock(true);
-        if (connection == "serial") {
-            for (index_t o = 0; o < m_output_node_size; ++o) {
-                for (int i = 0; i < N; ++i) { tbl(o, i) = (IndexType)((o * N + i) % m_input_node_size); }
-            }
-        }
-        else {
-            std::mt19937_64 mt(seed);
-            std::vector<IndexType> deck((std::size_t)m_input_node_size);
-            std::iota(deck.begin(), deck.end(), (IndexType)0);
-            std::size_t pos = deck.size();
-            for (index_t o = 0; o < m_output_node_size; ++o) {
-                IndexType pick[N];
-                for (int i = 0; i < N; ++i) {
-                    for (;;) {
-                        if (pos >= deck.size()) { std::shuffle(deck.begin(), deck.end(), mt); pos = 0; }
-                        IndexType const c = deck[pos++];
-                        bool dup = false;
-                        for (int j = 0; j < i; ++j) { dup = dup || (pick[j] == c); }
-                        if (!dup) { pick[i] = c; break; }
-                    }
-                }
-                for (int i = 0; i < N; ++i) { tbl(o, i) = pick[i]; }
-            }
-        }
+        index_t const inputs = m_input_node_size;
+        connection_policy::Initialize(seed, connection, m_input_shape, m_output_shape, N, connection_policy::Layout::kChannelFirst,
+                                      [&](index_t node, int i, index_t input) {
+                                          BB_ASSERT(input >= 0 && input < inputs);
+                                          tbl(node, (index_t)i) = (IndexType)input;
+                                      });
         m_reverse_table_dirty = true;
     }
 

@@ -483,6 +483,19 @@ def ref_binary_lut6(xbits, idx, table, frame_size, host_simd=True):
     return y
 
 
+def ref_wiring6(kind, input_shape, output_shape, seed, policy):
+    """Wiring that the reference gives a 6-input layer from a seed and a policy string.  kind 0: the connection table of
+    StochasticLutN / DifferentiableLutN; kind 1: BinaryLutN (also returns its random truth tables [O][2])."""
+    ins = np.asarray(input_shape, np.int64); outs = np.asarray(output_shape, np.int64)
+    O = int(np.prod(outs))
+    idx = np.zeros((O, 6), np.int32); table = np.zeros((O, 2), np.int32)
+    f = ref().bbref_Wiring6
+    f.restype = C.c_int
+    rc = f(C.c_int(kind), C.c_int(len(ins)), _ptr(ins), _ptr(outs), C.c_uint64(seed), C.c_char_p(policy.encode()), _ptr(idx), _ptr(table))
+    assert rc == 0
+    return (idx, table) if kind == 1 else idx
+
+
 def ref_reverse_table6(idx, input_node_size):
     idx = _c(idx, np.int32)
     O = idx.shape[0]

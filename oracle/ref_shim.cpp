@@ -297,6 +297,40 @@ int bbref_DefaultWiring6(int I, int O, std::uint64_t seed, std::int32_t *idx)
 }
 
 
+// Seeded wiring by policy.  kind 0: FixedSizeConnectionTable<6>::InitializeConnection(seed, policy) (the table behind
+// StochasticLutN / DifferentiableLutN, include/bb/ConnectionTable.h:150-284); kind 1: BinaryLutN<6, Bit> created with
+// (output_shape, policy, seed) and given its input shape, which draws the wiring seed and then the table seed from the
+// layer's generator (include/bb/BinaryLutN.h:201-218, SparseModel.h:97-233, BinaryLutModel.h:45-59) — `table` then
+// receives the layer's random truth tables, int32 [O][2].  Shapes have `dims` entries.  idx: int32 [O][6].
+int bbref_Wiring6(int kind, int dims, long long const *in_shape, long long const *out_shape, std::uint64_t seed, char const *policy,
+                  std::int32_t *idx, std::int32_t *table)
+{
+    bb::indices_t in((size_t)dims), out((size_t)dims);
+    for (int i = 0; i < dims; ++i) { in[(size_t)i] = (index_t)in_shape[i]; out[(size_t)i] = (index_t)out_shape[i]; }
+    index_t const O = bb::CalcShapeSize(out);
+    if (kind == 0) {
+        bb::FixedSizeConnectionTable<6> tbl;
+        tbl.SetShape(in, out);
+        tbl.InitializeConnection(seed, policy);
+        for (index_t nd = 0; nd < O; ++nd) for (int i = 0; i < 6; ++i) { idx[nd * 6 + i] = (std::int32_t)tbl.GetInputConnection(nd, i); }
+        return 0;
+    }
+    typename bb::BinaryLutN<6, bb::Bit>::create_t create;
+    create.output_shape = out;
+    create.connection   = policy;
+    create.seed         = seed;
+    auto lut = bb::BinaryLutN<6, bb::Bit>::Create(create);
+    lut->SetInputShape(in);
+    for (index_t nd = 0; nd < O; ++nd) {
+        for (int i = 0; i < 6; ++i) { idx[nd * 6 + i] = (std::int32_t)lut->GetNodeConnectionIndex(nd, i); }
+        std::uint32_t w[2] = {0, 0};
+        for (int b = 0; b < 64; ++b) { if (lut->GetLutTable(nd, b)) { w[b / 32] |= (1u << (b % 32)); } }
+        table[nd * 2] = (std::int32_t)w[0]; table[nd * 2 + 1] = (std::int32_t)w[1];
+    }
+    return 0;
+}
+
+
 // bb::OptimizerAdam<float> (host path, include/bb/OptimizerAdam.h:142-180): `steps` updates of one fp32 tensor of
 // `size` elements; grads is [steps][size]; param is updated in place.
 int bbref_OptimizerAdam(int size, int steps, float *param, float const *grads, float learning_rate, float beta1, float beta2)

@@ -5,6 +5,9 @@
 //   object_tool make      <kind> <bit> <I> <O> <flags> <name|-> <prefix> <out.bb_net>
 //   object_tool roundtrip <kind> <bit> <in.bb_net> <out.bb_net>
 //   object_tool describe  <kind> <bit> <in.bb_net> <prefix>          prints "I O name" on one line
+//   object_tool wiring    <kind> <seed> <policy|-> <dims> <input shape ...> <output shape ...> <prefix>
+//                         seeded wiring of a fresh layer (kind 0: the connection table of StochasticLutN / DifferentiableLutN,
+//                         2: BinaryLutN created with that seed, 3: StochasticLutN created with that seed): writes <prefix>.idx and, for BinaryLutN, <prefix>.params
 //
 // kind 0 = StochasticLutN<6>, 1 = DifferentiableLutN<6>, 2 = BinaryLutN<6, Bit>; bit selects BinType = Bit for kinds 0, 1.
 // flags: bit 0 = binary, bit 1 = lut_binarize, bit 2 = batch_norm.  DifferentiableLut scalars are fixed: momentum 0.75,
@@ -151,11 +154,56 @@ static int run(std::string const &cmd, char **a, MakeModel make_model)
     return 1;
 }
 
+// object_tool wiring <kind> <seed> <policy|-> <dims> <input shape ...> <output shape ...> <prefix>
+static int wiring(int argc, char **argv)
+{
+    if (argc < 6) { std::fprintf(stderr, "usage: object_tool wiring <kind> <seed> <policy|-> <dims> <shapes ...> <prefix>\n"); return 1; }
+    int const kind = std::atoi(argv[2]);
+    std::uint64_t const seed = std::strtoull(argv[3], nullptr, 10);
+    std::string const policy = std::string(argv[4]) == "-" ? "" : argv[4];
+    int const dims = std::atoi(argv[5]);
+    if (dims < 1 || argc != 6 + 2 * dims + 1) { std::fprintf(stderr, "wiring: %d shape entries and a prefix expected\n", 2 * dims); return 1; }
+    bb::indices_t in((size_t)dims), out((size_t)dims);
+    for (int i = 0; i < dims; ++i) { in[(size_t)i] = std::atoll(argv[6 + i]); out[(size_t)i] = std::atoll(argv[6 + dims + i]); }
+    std::string const prefix = argv[6 + 2 * dims];
+    bb::index_t const O = bb::CalcShapeSize(out);
+    std::vector<std::int32_t> idx((size_t)O * 6);
+    if (kind == 0) {
+        bb::FixedSizeConnectionTable<6> tbl;
+        tbl.SetShape(in, out);
+        tbl.InitializeConnection(seed, policy);
+        for (bb::index_t o = 0; o < O; ++o) { for (int i = 0; i < 6; ++i) { idx[(size_t)o * 6 + i] = (std::int32_t)tbl.GetInputConnection(o, i); } }
+    }
+    else if (kind == 3) {           // a whole StochasticLutN created with the seed: its generator's first draw seeds the table
+        auto lut = bb::StochasticLutN<6, float, float>::Create(out, policy, seed);
+        lut->SetInputShape(in);
+        idx = get_wiring(*lut);
+    }
+    else {
+        bb::BinaryLutN<6, bb::Bit>::create_t create;
+        create.output_shape = out; create.connection = policy; create.seed = seed;
+        auto lut = bb::BinaryLutN<6, bb::Bit>::Create(create);
+        lut->SetInputShape(in);
+        idx = get_wiring(*lut);
+        std::vector<std::int32_t> table((size_t)O * 2, 0);
+        for (bb::index_t o = 0; o < O; ++o) {
+            for (int b = 0; b < 64; ++b) { if (lut->GetLutTable(o, b)) { table[(size_t)o * 2 + b / 32] = (std::int32_t)((std::uint32_t)table[(size_t)o * 2 + b / 32] | (1u << (b % 32))); } }
+        }
+        write_raw(prefix + ".params", table);
+    }
+    write_raw(prefix + ".idx", idx);
+    return 0;
+}
+
 int main(int argc, char **argv)
 {
-    if (argc < 6) { std::fprintf(stderr, "usage: object_tool make|roundtrip|describe <kind> <bit> ...\n"); return 1; }
+    if (argc < 6) { std::fprintf(stderr, "usage: object_tool make|roundtrip|describe|wiring <kind> ...\n"); return 1; }
     bb::Manager::SetHostOnly(true);             // serialization is host work; no device is touched
     std::string const cmd = argv[1];
+    if (cmd == "wiring") {
+        try { return wiring(argc, argv); }
+        catch (std::exception const &e) { std::fprintf(stderr, "rejected: %s\n", e.what()); return 1; }
+    }
     int const kind = std::atoi(argv[2]), bit = std::atoi(argv[3]);
     char **rest = argv + 4;
     try {
