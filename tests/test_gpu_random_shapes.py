@@ -265,3 +265,25 @@ def test_random_shapes_of_the_classifier_tail_and_adam():
     from binarybrain_amd import ops
     for seed in range(11000, 11150):
         run_tail_case(ops, torch, seed)
+
+
+def test_extended_random_run():
+    """The same three generators over further seeds, for a longer run on the device: set BBHIP_EXTENDED_CASES=N (N cases of each
+    generator, at most 200 000; seeds continue after the ones above).  Stops at the first failing case, whose seed the case
+    prints.  Without the variable the test is skipped, so the default suite stays short:
+        BBHIP_EXTENDED_CASES=10000 python -u -m pytest tests/test_gpu_random_shapes.py -k extended -x -s"""
+    import os
+    count = int(os.environ.get("BBHIP_EXTENDED_CASES", "0") or 0)
+    if count <= 0:
+        pytest.skip("BBHIP_EXTENDED_CASES is not set")
+    count = min(count, 200000)
+    import torch
+    from binarybrain_amd import ops
+    try:
+        for k in range(count):
+            run_case(ops, torch, 100000 + k)
+            run_exact_case(ops, 400000 + k)
+            run_tail_case(ops, torch, 700000 + k)
+    finally:
+        ops.set_dx_mode(0)
+    print("extended run: %d cases of each generator, no mismatch" % count)
