@@ -61,6 +61,7 @@ int fail(char const *fmt, ...)
 // ------------------------------------------------------------------------------------------------
 bool g_host_only = false;
 int  g_dx_mode   = 0;
+bool g_average_lut_mean = false;             // bbhip_SetAverageLutMean: un-binarized AverageLut output is sum * (1 / n)
 thread_local int g_input_node_hint = 0;      // bbhip_HintInputNodeSize: rows of the next forward call's input, 0 = unknown
 
 // ------------------------------------------------------------------------------------------------
@@ -520,7 +521,17 @@ template <int N>
 int run_backward(BackwardCall const &call, hipStream_t st)
 {
     constexpr int NN = 1 << N;
-    int const dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
+    int dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
+    // The term table of the deterministic dx kernel has one slot per (input node, position in the longest fan-out list).  With
+    // evenly used inputs that is about the number of connections; wiring in which a few inputs feed very many nodes would make
+    // it (and the launch that fills it) grow with input nodes x longest list while only output nodes x n records are ever
+    // read.  Such a call takes the reference's scheme where the caller gave it a dx_tmp buffer, else the atomic one: same
+    // results to rounding, but in the atomic case not reproducible bit for bit.
+    if (dxmode == kDxNone && call.rev != nullptr && call.rev_stride >= 1) {
+        long long const slots = (long long)call.input_node_size * (long long)(call.rev_stride - 1);
+        long long const links = (long long)call.output_node_size * call.n;
+        if (slots > 8 * links + 65536) { dxmode = (call.dx_tmp != nullptr && call.tmp_frame_size > 0) ? kDxTmp : kDxAtomic; }
+    }
     if (check_backward(call, dxmode)) { return 1; }
 
     // fp32 frames that the layer binarizes at 0.5 are packed to bits once (reading them once costs less than the three
@@ -976,6 +987,9 @@ int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, in
     return 0;
 }
 
+void bbhip_SetAverageLutMean(int mean) { g_average_lut_mean = mean != 0; }
+int  bbhip_GetAverageLutMean(void) { return g_average_lut_mean ? 1 : 0; }
+
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
 void bbhip_HintInputNodeSize(int input_node_size) { g_input_node_hint = input_node_size > 0 ? input_node_size : 0; }
 int  bbhip_GetDxMode(void) { return g_dx_mode; }
@@ -1250,7 +1264,8 @@ int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int 
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(average_lut_forward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_x_buf,
-                       dev_y_buf, dev_input_index, n, frame_size, frame_stride, binarize_input, binarize_output, f_blocks);
+                       dev_y_buf, dev_input_index, n, frame_size, frame_stride, binarize_input, binarize_output, f_blocks,
+                       g_average_lut_mean ? 1.0f / (float)n : 1.0f);
     BBHIP_LAUNCH_CHECK();
     return 0;
 }

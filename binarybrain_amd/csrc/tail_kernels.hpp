@@ -17,8 +17,11 @@ namespace bbhip {
 constexpr int kTailBlock = 256;
 
 // one thread per (output node, frame)
+// scale: what an un-binarized sum is multiplied by — 1 (the host loop of the reference writes the sum) or the fp32
+// reciprocal of n (its CUDA kernel writes sum * (1 / n), cuda/AverageLut.cu:46-54)
 __global__ __launch_bounds__(kTailBlock) void average_lut_forward_kernel(float const *x, float *y, int const *idx, int n, int frame_size,
-                                                                         int frame_stride, int binarize_input, int binarize_output, int f_blocks)
+                                                                         int frame_stride, int binarize_input, int binarize_output, int f_blocks,
+                                                                         float scale)
 {
     int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
     int const node = blockIdx.x / f_blocks;
@@ -31,6 +34,7 @@ __global__ __launch_bounds__(kTailBlock) void average_lut_forward_kernel(float c
         sum += v;
     }
     if (binarize_output) { sum = (sum > 0.0f) ? 1.0f : -1.0f; }
+    else                 { sum = rounded_mul(sum, scale); }
     y[(size_t)node * frame_stride + f] = sum;
 }
 

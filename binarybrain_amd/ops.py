@@ -18,6 +18,11 @@ def _dev(*ts):
             raise capi.BbhipError("bbhip ops need contiguous tensors")
 
 
+def set_average_lut_mean(mean):
+    """False (default): AverageLut writes the sum of its inputs (the reference's host path); True: sum * (1 / n) (its CUDA kernel)."""
+    lib().bbhip_SetAverageLutMean(int(bool(mean)))
+
+
 def set_dx_mode(mode):
     """0: deterministic dx, input-centric re-evaluation through the reverse table (default); 1: fp32 atomics;
     2: the reference's scheme (per-connection gradients in dx_tmp, summed through the reverse table)."""
@@ -293,12 +298,11 @@ def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_bi
     I = x.shape[0]; O = idx.shape[0]
     dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
     tf = ts = 0
-    if lib().bbhip_GetDxMode() == 2:
-        if dx_tmp is None:
-            dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
-        else:
-            ts = dx_tmp.shape[1]
-            tf = min(ts, frame_size) if tmp_frame_size is None else tmp_frame_size
+    if dx_tmp is not None:                      # always described to the library: mode 2 needs it, mode 0 may fall back to it
+        ts = dx_tmp.shape[1]
+        tf = min(ts, frame_size) if tmp_frame_size is None else tmp_frame_size
+    elif lib().bbhip_GetDxMode() == 2:
+        dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
     check(lib().bbhip_fp32_StochasticLut_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                   0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,
                                                   int(input_binary), int(lut_binarize), bias, stream_ptr()))

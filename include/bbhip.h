@@ -76,6 +76,14 @@ size_t bbhip_GetScratchSize(void);
  * number, and takes its default (on) when unset. */
 int bbhip_GetSwitch(char const *name);
 
+/* ---- which of the reference's two AverageLut conventions the forward entry follows (no counterpart in the reference) ----
+ * The reference disagrees with itself: without binarize_output its host loop writes the SUM of the n inputs
+ * (include/bb/AverageLut.h:331-343), its CUDA kernel writes sum * (1 / n) (cuda/AverageLut.cu:46-54); both backward paths
+ * return dy / n.  0 (default): the host convention; 1: the CUDA kernel's (the fp32 reciprocal of n, then one multiply).
+ * A process-wide switch like the dx mode; binarized outputs and the packed-bit entry do not depend on it. */
+void bbhip_SetAverageLutMean(int mean);
+int  bbhip_GetAverageLutMean(void);
+
 /* ---- how dx is accumulated over the fan-out of an input node (no counterpart in the reference) ----
  * 0 (default): deterministic, no scratch — one wavefront per (input node, frame chunk) walks reverse_index in the
  *              reference's order (cuda/Common.cuh:174-202, include/bb/FixedSizeConnectionTable.h:198-214) and
@@ -203,7 +211,7 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
 /* bbcu_AverageLut_Forward<float>, include/bbcu/bbcu.h:321-334.  y = sum over the n inputs dev_input_index[node*n + i] of x (each
  * replaced by +1 / -1 on x > 0 when binarize_input), written as +1 / -1 on sum > 0 when binarize_output.  Without
  * binarize_output the SUM is written, as by the reference's host loop (include/bb/AverageLut.h:331-343); its CUDA kernel
- * writes sum / n (cuda/AverageLut.cu:46-54). */
+ * writes sum * (1 / n) (cuda/AverageLut.cu:46-54), which bbhip_SetAverageLutMean(1) selects. */
 int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                                   int frame_stride, int binarize_input, int binarize_output, void *stream);
 /* bbcu_bit_AverageLut_Forward, include/bbcu/bbcu.h:336-346: packed bits, y = strict majority of the n inputs (a tie of an even

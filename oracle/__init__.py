@@ -187,13 +187,18 @@ def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
     return dx
 
 
-def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
-    """fp32 x [I, stride] -> y [O, stride]: sum (or its sign) of the n wired inputs."""
+def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True, mean=False):
+    """fp32 x [I, stride] -> y [O, stride]: sum (or its sign) of the n wired inputs, the reference's host loop
+    (include/bb/AverageLut.h:331-343).  mean: the convention of the reference's CUDA kernel instead, which writes an
+    un-binarized output as sum * reciprocal_n with reciprocal_n = (float)1.0 / (float)n (cuda/AverageLut.cu:46-54, 93) —
+    the same sum, one fp32 reciprocal, one fp32 product; pinned by its closed form (exactly sum / n when n is a power of two)."""
     x = _c(x, np.float32); idx = _c(idx, np.int32)
     O, n = idx.shape
     y = np.zeros((O, x.shape[1]), np.float32)
     lib().oracle_fp32_AverageLut_Forward(_ptr(x), _ptr(y), _ptr(idx), C.c_int(n), C.c_int(O), C.c_int(frame_size), C.c_int(x.shape[1]),
                                          C.c_int(int(binarize_input)), C.c_int(int(binarize_output)))
+    if mean and not binarize_output:
+        y = (y * (np.float32(1.0) / np.float32(n))).astype(np.float32)
     return y
 
 

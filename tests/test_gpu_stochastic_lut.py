@@ -342,3 +342,26 @@ def test_adversarial_tables(ops, n):
     sel = (xs[:, :, :64] > 0.5).astype(np.int64)
     code = sum(sel[:, j] << j for j in range(n))
     assert np.array_equal(corner, np.take_along_axis(W, code, axis=1))
+
+
+def test_skewed_fan_out_takes_another_dx_path():
+    """One input that feeds every node makes the reverse table input_nodes x (1 + output_nodes) wide, far more slots than
+    connections: the deterministic dx kernel's term table would be sized by that, so the library takes the dx_tmp scheme
+    (when given the buffer) or the atomic one for such a call.  Results stay within the backward tolerance."""
+    import torch
+    from binarybrain_amd import ops
+    ops.set_dx_mode(0)
+    rng = np.random.default_rng(4242)
+    I, O, F = 3000, 400, 200
+    S = synth.frame_stride_fp32(F)
+    idx = synth.wiring(rng, I - 1, O, 6) + 1
+    idx[:, 2] = 0                                   # input 0 is wired to every node
+    W = synth.lut_tables(rng, O); x = synth.uniform_frames(rng, I, F, S, -0.1, 1.1); dy = synth.normal_frames(rng, O, F, S)
+    dx_ref, dW_ref = oracle.stochastic_lut_backward(6, x, dy, idx, W, F)
+    rev = ops.reverse_table(dev(idx), I)
+    assert rev.shape[1] == O + 1
+    for with_tmp in (False, True):
+        dW = torch.zeros((O, 64), device="cuda")
+        kw = dict(dx_tmp=torch.empty((O * 6, S), device="cuda"), tmp_frame_size=F) if with_tmp else {}
+        dx = ops.stochastic_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, rev, **kw)
+        assert_bwd(host(dx)[:, :F], dx_ref[:, :F], "dx"); assert_bwd(host(dW), dW_ref, "dW")

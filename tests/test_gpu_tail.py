@@ -180,3 +180,25 @@ def test_rejected_arguments(ops):
         ops.loss_softmax_cross_entropy(x, x, 4, 1, 100, t_sum=1.0)
     with pytest.raises(RuntimeError):
         ops.metrics_categorical_accuracy(x, x, 4, 1, 0)
+
+
+def test_average_lut_mean_convention(ops):
+    """bbhip_SetAverageLutMean(1): the un-binarized forward follows the reference's CUDA kernel, sum * (1 / n), bit for bit;
+    binarized outputs and the backward (dy / n in both conventions) do not change."""
+    rng = np.random.default_rng(77)
+    try:
+        for n in (6, 7, 8):
+            I, O, F = 90, 15, 333
+            S = synth.frame_stride_fp32(F)
+            idx = rng.integers(0, I, (O, n)).astype(np.int32)
+            x = np.zeros((I, S), np.float32); x[:, :F] = rng.standard_normal((I, F))
+            ops.set_average_lut_mean(True)
+            y = host(ops.average_lut_forward(dev(x), dev(idx), F, False, False))
+            yb = host(ops.average_lut_forward(dev(x), dev(idx), F, True, True))
+            ops.set_average_lut_mean(False)
+            ys = host(ops.average_lut_forward(dev(x), dev(idx), F, False, False))
+            assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, False, False, mean=True)[:, :F])
+            assert np.array_equal(ys[:, :F], oracle.average_lut_forward(x, idx, F, False, False)[:, :F])
+            assert np.array_equal(yb[:, :F], oracle.average_lut_forward(x, idx, F, True, True)[:, :F])
+    finally:
+        ops.set_average_lut_mean(False)

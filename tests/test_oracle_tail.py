@@ -190,3 +190,19 @@ def test_loss_closed_forms():
     # weights: t_sum follows the weights and the host sum runs frame-major in float
     tw = t * F32(0.3)
     assert oracle.loss_t_sum(tw, F) == np.cumsum(np.full(pix * F, F32(0.3), F32), dtype=F32)[-1]
+
+
+def test_average_lut_mean_convention_closed_forms():
+    """The CUDA kernel's convention (sum * (1 / n), cuda/AverageLut.cu:46-54) as the oracle restates it: exactly sum / n for
+    powers of two, within one rounding of it otherwise, untouched where the output is binarized."""
+    rng = np.random.default_rng(8)
+    for n in (1, 2, 4, 7, 8, 10):
+        I, O, F = 40, 12, 70
+        idx = rng.integers(0, I, (O, n)).astype(np.int32)
+        x = rng.standard_normal((I, F)).astype(np.float32)
+        s = oracle.average_lut_forward(x, idx, F, False, False)
+        m = oracle.average_lut_forward(x, idx, F, False, False, mean=True)
+        if n & (n - 1) == 0:
+            assert np.array_equal(m, s / np.float32(n))
+        assert np.abs(m.astype(np.float64) - s.astype(np.float64) / n).max() <= 2.0 ** -23 * np.abs(s).max()
+        assert np.array_equal(oracle.average_lut_forward(x, idx, F, False, True, mean=True), oracle.average_lut_forward(x, idx, F, False, True))
