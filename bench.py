@@ -23,10 +23,10 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # the same profiler run.  The counter tables and the commands are in profiles/*.md.  A kernel or workload that is not
 # listed reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("lut_dx_kernel<6>", 0):       (652361.0 * 2.0 + 132096.0) * 1024,
-    ("lut_forward_kernel<6>", 0):  (133352.3 * 2.0 + 131072.0) * 1024,
-    ("lut_backward_kernel<6>", 0): (354315.3 * 2.0 + 6372.5) * 1024,
-    ("binary_lut6_kernel", 0):     (651698.0 * 2.0 + 524288.0) * 1024,
+    ("lut_dx_kernel<6>", 0):       (651995.4 * 2.0 + 132096.0) * 1024,
+    ("lut_forward_kernel<6>", 0):  (129936.7 * 2.0 + 131072.0) * 1024,
+    ("lut_backward_kernel<6>", 0): (354707.1 * 2.0 + 6372.0) * 1024,
+    ("binary_lut6_kernel", 0):     (348316.2 * 2.0 + 524288.0) * 1024,
     ("adam_kernel", 0):            (527931.3 * 2.0 + 791860.5) * 1024,
 }
 
@@ -580,7 +580,7 @@ def bench_stochasticlut6(args, lib):
     dx_tmp = None
     tmp_frames = None
     if args.dx_mode == 2:
-        tmp_frames = ops._tmp_frames(O, 6, F)
+        tmp_frames = ops._tmp_frames(O, 6, F, args.tmp_mb << 20)
         dx_tmp = torch.empty((O * 6, ((tmp_frames + 63) // 64) * 64), device="cuda")
 
     def step():
@@ -775,6 +775,8 @@ def main():
                     help="untimed steps first; the device needs a few dozen steps of load to reach its sustained clock")
     ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "0")),
                     help="0: deterministic input-centric dx; 1: fp32 atomics; 2: dx_tmp + reverse table")
+    ap.add_argument("--tmp-mb", type=int, default=256,
+                    help="dx mode 2: size of the dx_tmp scratch in MiB (the reference caps it at 256; a smaller one takes more passes over shorter frame ranges)")
     ap.add_argument("--ramp-seconds", type=float, default=0.3,
                     help="before the warm-up steps, keep the device under the same load for this long (untimed): from idle it "
                          "takes a few dozen steps to reach its sustained clock, whatever --warmup says")

@@ -137,10 +137,10 @@ int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  retur
 // per-term set-up per frame.  0: not set in the environment.
 int dx_chunk_frames_env(void) { static int v = env_int("BBHIP_DX_CHUNK", 0); return ((v + 63) / 64) * 64; }
 int dx_pass_steps_env(void)   { static int v = env_int("BBHIP_DX_STEPS", 0); return (v <= 0) ? 0 : (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
-// BinaryLut6 units of 192 words: 8192 input rows x 768 bytes is what stays in an XCD's L2 next to the output stream
-// (256-word units fetch 2.3 GB per launch at the benchmark shape, 192-word units 1.9 GB; 128-word units fetch less still
-// but leave a wavefront too little work per set-up)
-int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 192); return (((v > 0 ? v : 192) + 63) / 64) * 64; }
+// BinaryLut6 units of 128 words: 8192 input rows x 512 bytes is what an XCD's 4 MiB L2 holds (1.2 GB fetched per launch at
+// the benchmark shape; 192-word units fetch 1.9 GB, 256-word units 2.3 GB).  With the per-wavefront set-up at its
+// present cost the shorter units are also the fastest (201 us; 192 words 206 us, 256 words 250 us, 64 words 251 us).
+int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 128); return (((v > 0 ? v : 128) + 63) / 64) * 64; }
 int bin_nodes_per_wave(void) { static int v = env_int("BBHIP_BIN_NODES", 0); return v >= 4 ? 4 : v >= 2 ? 2 : v == 1 ? 1 : 0; }     // 0: chosen per call
 
 // ------------------------------------------------------------------------------------------------
@@ -1624,6 +1624,7 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr && dev_input_index != nullptr && dev_table != nullptr);
     BBHIP_REQUIRE(node_size > 0 && node_size <= (0x7fffffff >> 6) && frame_size > 0);
     BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);
+    BBHIP_REQUIRE(frame_stride <= 0x07ffffff);          // row pitch in bytes, times the four nodes of a wavefront, stays a 32-bit extent
     hipStream_t st = static_cast<hipStream_t>(stream);
     BinArgs a{};
     a.x = reinterpret_cast<uint32_t const *>(dev_x_buf);
@@ -1644,10 +1645,15 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     {
         ScopedTimer tm(kTimeBinary, st);
         dim3 const grid(a.chunk_count * a.tiles.count), block(kBlock);
+        bool const exact = (node_size % npw) == 0;
         switch (npw) {
-        case 1: hipLaunchKernelGGL(binary_lut6_kernel<1>, grid, block, 0, st, a); break;
-        case 2: hipLaunchKernelGGL(binary_lut6_kernel<2>, grid, block, 0, st, a); break;
-        default: hipLaunchKernelGGL(binary_lut6_kernel<4>, grid, block, 0, st, a); break;
+        case 1: hipLaunchKernelGGL((binary_lut6_kernel<1, true>), grid, block, 0, st, a); break;
+        case 2: if (exact) { hipLaunchKernelGGL((binary_lut6_kernel<2, true>), grid, block, 0, st, a); }
+                else       { hipLaunchKernelGGL((binary_lut6_kernel<2, false>), grid, block, 0, st, a); }
+                break;
+        default: if (exact) { hipLaunchKernelGGL((binary_lut6_kernel<4, true>), grid, block, 0, st, a); }
+                 else       { hipLaunchKernelGGL((binary_lut6_kernel<4, false>), grid, block, 0, st, a); }
+                 break;
         }
     }
     BBHIP_LAUNCH_CHECK();

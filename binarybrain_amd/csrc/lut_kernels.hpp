@@ -24,9 +24,10 @@ constexpr int kXcd          = 8;
 // logical workgroup index for hardware workgroup id b of a grid of B: XCD x (= b % 8) owns a contiguous range
 __device__ __forceinline__ int xcd_remap(int b, int B)
 {
-    int const q = B / kXcd, r = B % kXcd;
-    int const x = b % kXcd, k = b / kXcd;
-    return x * q + (x < r ? x : r) + k;
+    // (unsigned: the shifts and masks of a division by 8 without the sign fix-ups, which cost the scalar unit a dozen instructions)
+    uint32_t const q = (uint32_t)B / kXcd, r = (uint32_t)B % kXcd;
+    uint32_t const x = (uint32_t)b % kXcd, k = (uint32_t)b / kXcd;
+    return (int)(x * q + (x < r ? x : r) + k);
 }
 
 __device__ __forceinline__ float wave_sum(float v)
@@ -1349,7 +1350,8 @@ __global__ __launch_bounds__(kBlock) void conv_bit_to_real_kernel(uint32_t const
 //  nibble, the same for every frame.  Per word the kernel forms all 16 functions once (12 three-input bit operations),
 //  picks the group values out of that register array with the nibbles as wave-uniform register indices while
 //  multiplexing by x2 (16 instructions), and finishes with the last three levels (7 bit-selects): 35 vector
-//  instructions per word where the plain tree takes 63, and the table stays packed in two scalar registers per node.
+//  instructions per word where the plain tree takes 63; the table is held as eight scalar registers per node, one 16-bit
+//  index field per nibble.
 // ------------------------------------------------------------------------------------------------
 // bit-select d = (s & hi) | (~s & lo): one instruction per multiplexer of the tree
 __device__ __forceinline__ uint32_t bfi_vvv(uint32_t s, uint32_t hi, uint32_t lo)
@@ -1378,50 +1380,74 @@ __device__ __forceinline__ uint32_t bin_pick(int at0, int at1, uint32_t x1, uint
     return at0 ? (at1 ? 0xffffffffu : nx1) : (at1 ? x1 : 0u);
 }
 
-// Four level-2 multiplexers t_j = x2 ? fn[nibble 2j+1] : fn[nibble 2j] of one 32-bit table word (eight groups of four
+// The eight level-2 multiplexers t_j = x2 ? fn[nibble 2j+1] : fn[nibble 2j] of a node (sixteen groups of four table
 // entries).  The function values sit in fixed registers v48..v63 and are picked with the vector-register index mode:
-// while it is on for source 0, source 0 of a vector instruction names register v48 + index.  One move fetches the x2 = 0
-// value, one three-input bit operation (truth table 0xe2: source 1 selects between source 0 and source 2) fetches the
-// x2 = 1 value and multiplexes.  The mode stays on across the block; only the index changes, each nibble extracted by
-// the scalar unit right before it is used (the table stays packed: two scalar registers per node).
-__device__ __forceinline__ void bin_select_level2(bin_u32x16 const &fn, uint32_t table_word, uint32_t x2,
-                                                  uint32_t &t0, uint32_t &t1, uint32_t &t2, uint32_t &t3)
+// while it is on for source 0, source 0 of a vector instruction names register v48 + M0[7:0].  One move fetches the
+// x2 = 0 value, one three-input bit operation (truth table 0xe2: source 1 selects between source 0 and source 2)
+// fetches the x2 = 1 value and multiplexes.  The mode stays on across the block and M0 is written whole for every pick:
+// the node's table is kept as eight scalar registers of two 16-bit fields 0x1000 | nibble (bits 15:12 = index source 0,
+// bits 7:0 = the index; bin_index_words), so that a pick costs one scalar instruction (and / shift into M0) where
+// extracting the nibble from the packed table and setting the index took two.
+__device__ __forceinline__ void bin_select_level2(bin_u32x16 const &fn, uint32_t const (&iw)[8], uint32_t x2, uint32_t (&t)[8])
 {
-    uint32_t tmp, idx;
+    uint32_t tmp;
     asm volatile(
-        "s_bfe_u32 %[i], %[tw], 0x40000\n\t"
-        "s_set_gpr_idx_on %[i], gpr_idx(SRC0)\n\t"
+        "s_set_gpr_idx_on %[w0], gpr_idx(SRC0)\n\t"
         "v_mov_b32 %[tmp], v48\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x40004\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_lshr_b32 m0, %[w0], 16\n\t"
         "v_bitop3_b32 %[t0], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x40008\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_and_b32 m0, %[w1], 0xffff\n\t"
         "v_mov_b32 %[tmp], v48\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x4000c\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_lshr_b32 m0, %[w1], 16\n\t"
         "v_bitop3_b32 %[t1], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x40010\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_and_b32 m0, %[w2], 0xffff\n\t"
         "v_mov_b32 %[tmp], v48\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x40014\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_lshr_b32 m0, %[w2], 16\n\t"
         "v_bitop3_b32 %[t2], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x40018\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_and_b32 m0, %[w3], 0xffff\n\t"
         "v_mov_b32 %[tmp], v48\n\t"
-        "s_bfe_u32 %[i], %[tw], 0x4001c\n\t"
-        "s_set_gpr_idx_idx %[i]\n\t"
+        "s_lshr_b32 m0, %[w3], 16\n\t"
         "v_bitop3_b32 %[t3], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_and_b32 m0, %[w4], 0xffff\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_lshr_b32 m0, %[w4], 16\n\t"
+        "v_bitop3_b32 %[t4], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_and_b32 m0, %[w5], 0xffff\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_lshr_b32 m0, %[w5], 16\n\t"
+        "v_bitop3_b32 %[t5], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_and_b32 m0, %[w6], 0xffff\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_lshr_b32 m0, %[w6], 16\n\t"
+        "v_bitop3_b32 %[t6], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
+        "s_and_b32 m0, %[w7], 0xffff\n\t"
+        "v_mov_b32 %[tmp], v48\n\t"
+        "s_lshr_b32 m0, %[w7], 16\n\t"
+        "v_bitop3_b32 %[t7], v48, %[x2], %[tmp] bitop3:0xe2\n\t"
         "s_set_gpr_idx_off"
-        : [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [tmp] "=&v"(tmp), [i] "=&s"(idx)
-        : [tw] "s"(table_word), [x2] "v"(x2),
+        : [t0] "=&v"(t[0]), [t1] "=&v"(t[1]), [t2] "=&v"(t[2]), [t3] "=&v"(t[3]),
+          [t4] "=&v"(t[4]), [t5] "=&v"(t[5]), [t6] "=&v"(t[6]), [t7] "=&v"(t[7]), [tmp] "=&v"(tmp)
+        : [w0] "s"(iw[0]), [w1] "s"(iw[1]), [w2] "s"(iw[2]), [w3] "s"(iw[3]), [w4] "s"(iw[4]), [w5] "s"(iw[5]), [w6] "s"(iw[6]), [w7] "s"(iw[7]),
+          [x2] "v"(x2),
           "{v48}"(fn[0]), "{v49}"(fn[1]), "{v50}"(fn[2]), "{v51}"(fn[3]), "{v52}"(fn[4]), "{v53}"(fn[5]), "{v54}"(fn[6]), "{v55}"(fn[7]),
           "{v56}"(fn[8]), "{v57}"(fn[9]), "{v58}"(fn[10]), "{v59}"(fn[11]), "{v60}"(fn[12]), "{v61}"(fn[13]), "{v62}"(fn[14]), "{v63}"(fn[15])
-        : "scc");                // (M0 is changed too; the compiler keeps nothing there across statements)
+        : "scc");                // (M0 is written too: it is reserved, the compiler keeps nothing there across statements)
 }
 
-template <int NPW>   // nodes per wavefront
+// The index words of a node's table for bin_select_level2: word j holds 0x1000 | nibble 2j in its low half and
+// 0x1000 | nibble 2j+1 in its high half (nibble k = table entries 4k .. 4k+3).  Lane j < 8 forms word j with a few vector
+// instructions and the eight words are read back into scalar registers: the vector unit has the room, the scalar unit
+// does not.
+__device__ __forceinline__ void bin_index_words(uint32_t table_lo, uint32_t table_hi, int lane, uint32_t (&iw)[8])
+{
+    uint32_t const w    = (lane & 4) ? table_hi : table_lo;
+    uint32_t const byte = (w >> ((lane & 3) * 8)) & 0xffu;
+    uint32_t const v    = 0x10001000u | (byte & 15u) | ((byte >> 4) << 16);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { iw[j] = (uint32_t)__builtin_amdgcn_readlane((int)v, j); }
+}
+
+template <int NPW, bool EXACT>   // nodes per wavefront; EXACT: the node count is a multiple of NPW, no wavefront has nodes to skip
 __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
 {
     int const B    = a.chunk_count * a.tiles.count;
@@ -1432,32 +1458,39 @@ __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
     if (node0 >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
-    uint32_t const row_bytes = (uint32_t)a.word_count * 4u;
-    uint32_t tw[NPW][2];
+    uint32_t const row_bytes    = (uint32_t)a.word_count * 4u;
+    uint32_t const stride_bytes = (uint32_t)a.stride * 4u;
+    // wiring and tables are read through the constant address space: wave-uniform scalar loads wherever the compiler
+    // places them relative to the stores of this kernel (neither is written here)
+    typedef __attribute__((address_space(4))) int const const_int;
+    const_int *idxc = (const_int *)a.idx + (size_t)node0 * 6;
+    const_int *tabc = (const_int *)a.table + (size_t)node0 * 2;
+    uint32_t iw[NPW][8];                    // the node's table as index words (bin_index_words)
     char const *rows[NPW][6];               // wave-uniform row bases: loads take a scalar base and a 32-bit lane offset
-    __amdgpu_buffer_rsrc_t yr[NPW];
     bool live[NPW];
 #pragma unroll
     for (int p = 0; p < NPW; ++p) {
-        live[p] = node0 + p < a.node_size;
-        int const node = live[p] ? node0 + p : node0;       // a wavefront past the last node repeats its first one and stores nothing
-        tw[p][0] = (uint32_t)__builtin_amdgcn_readfirstlane(a.table[node * 2]);
-        tw[p][1] = (uint32_t)__builtin_amdgcn_readfirstlane(a.table[node * 2 + 1]);
+        live[p] = EXACT || (node0 + p < a.node_size);
+        int const rel = live[p] ? p : 0;                    // a wavefront past the last node repeats its first one and stores nothing
+        bin_index_words((uint32_t)tabc[rel * 2], (uint32_t)tabc[rel * 2 + 1], lane, iw[p]);
 #pragma unroll
         for (int k = 0; k < 6; ++k) {
-            rows[p][k] = reinterpret_cast<char const *>(a.x) + (size_t)a.idx[node * 6 + k] * (size_t)a.stride * 4u;
+            // unsigned 32 x 32 -> 64 bit: two scalar multiplies and an add with carry per row (the wiring is validated
+            // as non-negative by whoever builds it; a signed 64-bit product costs the scalar unit three times as much)
+            rows[p][k] = reinterpret_cast<char const *>(a.x) + (uint64_t)(uint32_t)idxc[rel * 6 + k] * (uint64_t)stride_bytes;
         }
-        // outputs go through a buffer descriptor that ends with the row: stores of lanes beyond it are dropped
-        // (an empty range drops every store)
-        yr[p] = row_descriptor(a.y, node, a.stride, live[p] ? row_bytes : 0u);
     }
+    // Outputs of the wavefront's nodes go through one buffer descriptor over their NPW rows, the node's row added as the
+    // scalar offset of the store (the range check covers that offset too, so the extent cannot end with a row: lanes
+    // beyond the end of a row are masked in the one step of a row that has them).
+    __amdgpu_buffer_rsrc_t const yr = row_descriptor(a.y, node0, a.stride, (uint32_t)NPW * stride_bytes);
 
     int const w_begin = ck * a.chunk;
     int const w_end   = min(w_begin + a.chunk, a.word_count);
     int const w_last  = a.word_count - 1;
     uint32_t const tail_mask = (a.frame_size & 31) ? ((1u << (a.frame_size & 31)) - 1u) : 0xffffffffu;
 
-    uint32_t const last_off = (uint32_t)w_last * 4u;        // lanes beyond the row re-read its last word; their stores are dropped
+    uint32_t const last_off = (uint32_t)w_last * 4u;        // lanes beyond the row re-read its last word and store nothing
     uint32_t off = (uint32_t)(w_begin + lane) * 4u;
     for (int w0 = w_begin; w0 < w_end; w0 += kWave, off += kWave * 4u) {
         uint32_t xv[NPW][6];
@@ -1480,17 +1513,24 @@ __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
                 fn[c] = (x0 & g1) | (~x0 & g0);
             }
             uint32_t t[8];
-            bin_select_level2(fn, tw[p][0], xv[p][2], t[0], t[1], t[2], t[3]);
-            bin_select_level2(fn, tw[p][1], xv[p][2], t[4], t[5], t[6], t[7]);
+            bin_select_level2(fn, iw[p], xv[p][2], t);
+            // the next node's functions are formed after this point, straight into the fixed registers that are free
+            // again now (formed earlier, they would have to be moved there: fifteen moves per node)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int lv = 3; lv < 6; ++lv) {
 #pragma unroll
                 for (int k = 0; k < (32 >> lv); ++k) { t[k] = bfi_vvv(xv[p][lv], t[2 * k + 1], t[2 * k]); }
             }
             uint32_t r = t[0];
-            if (has_tail && (w0 + lane == w_last)) { r &= tail_mask; }
             // streamed once (non-temporal): keep it from displacing x rows in L2
-            __builtin_amdgcn_raw_buffer_store_b32(r, yr[p], off, 0, 2);
+            if (live[p]) {
+                if (!has_tail) { __builtin_amdgcn_raw_buffer_store_b32(r, yr, off, (uint32_t)p * stride_bytes, 2); }
+                else {
+                    if (w0 + lane == w_last) { r &= tail_mask; }
+                    if (w0 + lane <= w_last) { __builtin_amdgcn_raw_buffer_store_b32(r, yr, off, (uint32_t)p * stride_bytes, 2); }
+                }
+            }
         }
     }
 }
