@@ -584,8 +584,12 @@ def bench_stochasticlut6(args, lib):
         dx_tmp = torch.empty((O * 6, ((tmp_frames + 63) // 64) * 64), device="cuda")
 
     def step():
-        ops.vector_clamp_(W)                                    # StochasticLutN::Forward clamps W first
-        ops.stochastic_lut_forward(6, x, idx, W, F, out=y)
+        # StochasticLutN::Forward clamps W to [0, 1] in place first: the forward entry does that in its table-preparation launch
+        if args.separate_clamp:
+            ops.vector_clamp_(W)
+            ops.stochastic_lut_forward(6, x, idx, W, F, out=y)
+        else:
+            ops.stochastic_lut_forward(6, x, idx, W, F, out=y, clamp_w=(0.0, 1.0))
         ops.stochastic_lut_backward(6, x, dy, idx, W, dW, F, rev, dx_tmp=dx_tmp, tmp_frame_size=tmp_frames, out=dx)
 
     t_ramp = time.perf_counter()
@@ -775,6 +779,8 @@ def main():
                     help="untimed steps first; the device needs a few dozen steps of load to reach its sustained clock")
     ap.add_argument("--dx-mode", type=int, default=int(os.environ.get("BBHIP_BENCH_DX_MODE", "0")),
                     help="0: deterministic input-centric dx; 1: fp32 atomics; 2: dx_tmp + reverse table")
+    ap.add_argument("--separate-clamp", action="store_true",
+                    help="headline step: clamp W with a launch of its own (bbhip_fp32_Vector_clamp, then the forward entry) instead of inside the forward entry's table preparation")
     ap.add_argument("--tmp-mb", type=int, default=256,
                     help="dx mode 2: size of the dx_tmp scratch in MiB (the reference caps it at 256; a smaller one takes more passes over shorter frame ranges)")
     ap.add_argument("--ramp-seconds", type=float, default=0.3,

@@ -203,10 +203,11 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
     }
 
 template <int N>
-void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st, float *V = nullptr, float bias = 0.0f)
+void launch_table_prep(float const *W, float *C, int node_size, int lut_binarize, hipStream_t st, float *V = nullptr, float bias = 0.0f,
+                       float *clamp_W = nullptr, float clamp_lo = 0.0f, float clamp_hi = 0.0f)
 {
     int const total = node_size * (1 << N);
-    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize, V, bias);
+    hipLaunchKernelGGL(table_prep_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, W, C, node_size, lut_binarize, V, bias, clamp_W, clamp_lo, clamp_hi);
 }
 
 template <int N, int XMODE, int YMODE, int KIND>
@@ -319,6 +320,8 @@ struct ForwardCall {
     int bn;                      // 0 none, 1 training, 2 inference
     float *mean, *rstd, *running_mean, *running_var;
     float gamma, beta, momentum;
+    // non-null: W (the same buffer) is clamped in place to [clamp_lo, clamp_hi] by the table-preparation launch
+    float *clamp_W; float clamp_lo, clamp_hi;
 };
 
 // the kernels address a frame inside its node row with a 32-bit byte offset
@@ -373,7 +376,8 @@ int launch_binarize_pack(float const *x, int x_stride, uint32_t *bits, int bit_s
 // packing and table preparation; one launch for both where the packing takes the 16-byte path
 template <int N>
 int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_stride, int rows, int frame_size,
-                         float const *W, float *C, float *V, int node_size, int lut_binarize, float bias, hipStream_t st)
+                         float const *W, float *C, float *V, int node_size, int lut_binarize, float bias, hipStream_t st,
+                         float *clamp_W = nullptr, float clamp_lo = 0.0f, float clamp_hi = 0.0f)
 {
     int const row_blocks = ceil_div(bit_stride * 8, kBlock);
     long long const pack_blocks = (long long)rows * row_blocks, prep_blocks = ceil_div(node_size * (1 << N), kBlock);
@@ -382,12 +386,13 @@ int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_s
         a.x = x; a.bits = bits; a.frame_size = frame_size; a.x_stride = x_stride; a.y_stride = bit_stride;
         a.row_blocks = make_tile_divisor(row_blocks); a.pack_blocks = (int)pack_blocks;
         a.W = W; a.C = C; a.V = V; a.node_size = node_size; a.lut_binarize = lut_binarize; a.bias = bias;
+        a.clamp_W = clamp_W; a.clamp_lo = clamp_lo; a.clamp_hi = clamp_hi;
         hipLaunchKernelGGL(binarize_pack4_prep_kernel<N>, dim3((unsigned)(pack_blocks + prep_blocks)), dim3(kBlock), 0, st, a);
         BBHIP_LAUNCH_CHECK();
         return 0;
     }
     if (launch_binarize_pack(x, x_stride, bits, bit_stride, rows, frame_size, st)) { return 1; }
-    launch_table_prep<N>(W, C, node_size, lut_binarize, st, V, bias);
+    launch_table_prep<N>(W, C, node_size, lut_binarize, st, V, bias, clamp_W, clamp_lo, clamp_hi);
     BBHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -421,11 +426,11 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     if (pack) {
         uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes);
         if (launch_pack_and_prep<N>(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size,
-                                    c.W, C, V, c.node_size, c.lut_binarize, c.bias, st)) { return 1; }
+                                    c.W, C, V, c.node_size, c.lut_binarize, c.bias, st, c.clamp_W, c.clamp_lo, c.clamp_hi)) { return 1; }
         c.x = bits;
     }
     else {
-        launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias);
+        launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias, c.clamp_W, c.clamp_lo, c.clamp_hi);
         BBHIP_LAUNCH_CHECK();
     }
 
@@ -1401,6 +1406,21 @@ int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y
     c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
     c.xmode = input_binary ? kXBinary : kXClamp; c.ymode = kYClamp;
     c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    return forward_entry(c, stream);
+}
+
+int bbhip_fp32_StochasticLut_ForwardClampW(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                           float *dev_W, int node_size, int frame_size, int frame_stride,
+                                           int input_binary, int lut_binarize, float unbinarize_bias,
+                                           float w_lo, float w_hi, void *stream)
+{
+    BBHIP_REQUIRE(w_lo <= w_hi);
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = input_binary ? kXBinary : kXClamp; c.ymode = kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.clamp_W = dev_W; c.clamp_lo = w_lo; c.clamp_hi = w_hi;
     return forward_entry(c, stream);
 }
 

@@ -44,9 +44,13 @@ __device__ __forceinline__ float wave_sum(float v)
 // ------------------------------------------------------------------------------------------------
 //  For two-valued inputs (x_j = 1/2 -+ bias) the layer is a table of 2^N values, V[p] = y at the corner whose bit j says
 //  which value input j takes: one more butterfly over C, (a, b) -> (a - bias b, a + bias b) per variable.
+//  clamp_W != nullptr: the table is first clamped to [clamp_lo, clamp_hi] and written back there (the model classes clamp
+//  their table in place before every forward pass, include/bb/StochasticLutN.h:451; folded in here the clamp costs no
+//  launch of its own).  clamp_W is W itself, so neither pointer is declared unaliased.
 template <int N>
-__device__ __forceinline__ void table_prep_block(float const *__restrict__ W, float *__restrict__ C, int node_size, int lut_binarize,
-                                                 float *__restrict__ V, float bias, int block)
+__device__ __forceinline__ void table_prep_block(float const *W, float *__restrict__ C, int node_size, int lut_binarize,
+                                                 float *__restrict__ V, float bias, int block,
+                                                 float *clamp_W = nullptr, float clamp_lo = 0.0f, float clamp_hi = 0.0f)
 {
     constexpr int NN = 1 << N;
     int const t = block * kBlock + threadIdx.x;
@@ -54,6 +58,11 @@ __device__ __forceinline__ void table_prep_block(float const *__restrict__ W, fl
     float v = 0.0f;
     if (t < total) {
         v = W[t];
+        if (clamp_W != nullptr) {
+            float const w = fminf(clamp_hi, fmaxf(clamp_lo, v));        // as clamp_kernel
+            if (w != v) { clamp_W[t] = w; }
+            v = w;
+        }
         if (lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
     }
     int const i = t & (NN - 1);
@@ -73,11 +82,12 @@ __device__ __forceinline__ void table_prep_block(float const *__restrict__ W, fl
 }
 
 template <int N>
-__global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *__restrict__ W, float *__restrict__ C,
+__global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *W, float *__restrict__ C,
                                                            int node_size, int lut_binarize,
-                                                           float *__restrict__ V = nullptr, float bias = 0.0f)
+                                                           float *__restrict__ V = nullptr, float bias = 0.0f,
+                                                           float *clamp_W = nullptr, float clamp_lo = 0.0f, float clamp_hi = 0.0f)
 {
-    table_prep_block<N>(W, C, node_size, lut_binarize, V, bias, blockIdx.x);
+    table_prep_block<N>(W, C, node_size, lut_binarize, V, bias, blockIdx.x, clamp_W, clamp_lo, clamp_hi);
 }
 
 // dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order)
@@ -1316,6 +1326,7 @@ struct PackPrepArgs {
     TileDivisor row_blocks;     // workgroups per packed row
     int pack_blocks;            // rows * row_blocks.count
     float const *W;  float *C;  float *V;  int node_size, lut_binarize;  float bias;
+    float *clamp_W;  float clamp_lo, clamp_hi;      // see table_prep_block
 };
 
 template <int N>
@@ -1328,7 +1339,7 @@ __global__ __launch_bounds__(kBlock) void binarize_pack4_prep_kernel(PackPrepArg
         binarize_pack4_block(a.x, a.bits, a.frame_size, a.x_stride, a.y_stride, row, block);
         return;
     }
-    table_prep_block<N>(a.W, a.C, a.node_size, a.lut_binarize, a.V, a.bias, bid - a.pack_blocks);
+    table_prep_block<N>(a.W, a.C, a.node_size, a.lut_binarize, a.V, a.bias, bid - a.pack_blocks, a.clamp_W, a.clamp_lo, a.clamp_hi);
 }
 
 // packed bits -> fp32 values (reference: cuda/ConvBitToReal.cu, include/bb/FrameBuffer.h:850-866)

@@ -189,13 +189,14 @@ public:
         FrameBuffer y_buf(x_buf.GetFrameSize(), m_output_shape, DataType<RealType>::type);
         if (train) { m_x_buf = x_buf; }
 
-        m_W->Clamp_inplace(0.0f, 1.0f);                                      // reference: StochasticLutN.h:451
-
+        // The table is clamped to [0, 1] in place before every forward pass (reference: StochasticLutN.h:451): for fp32 frames
+        // by the forward entry itself, in its table-preparation launch; for packed frames by a call of its own.
         auto x_ptr   = x_buf.LockDeviceMemoryConst();
         auto y_ptr   = y_buf.LockDeviceMemory(true);
         auto idx_ptr = m_connection_table.LockDeviceMemConst_InputTable();
-        auto W_ptr   = m_W->LockDeviceMemoryConst();
         if (kBitInput) {
+            m_W->Clamp_inplace(0.0f, 1.0f);
+            auto W_ptr = m_W->LockDeviceMemoryConst();
             CheckDevice(bbhip_bit_fp32_StochasticLut_Forward(N, (int const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                             (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(),
                             (int)y_buf.GetNodeSize(), (int)y_buf.GetFrameSize(), (int)(y_buf.GetFrameStride() / sizeof(float)),
@@ -204,12 +205,13 @@ public:
         }
         else {
             BB_ASSERT(x_buf.GetFrameStride() == y_buf.GetFrameStride());
+            auto W_ptr = m_W->LockDeviceMemory();
             bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
-            CheckDevice(bbhip_fp32_StochasticLut_Forward(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
-                            (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(),
+            CheckDevice(bbhip_fp32_StochasticLut_ForwardClampW(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
+                            (int const *)idx_ptr.GetAddr(), (float *)W_ptr.GetAddr(),
                             (int)y_buf.GetNodeSize(), (int)y_buf.GetFrameSize(), (int)(y_buf.GetFrameStride() / sizeof(float)),
-                            m_binary_mode ? 1 : 0, m_lut_binarize ? 1 : 0, (float)m_unbinarize_bias, nullptr),
-                        "bbhip_fp32_StochasticLut_Forward");
+                            m_binary_mode ? 1 : 0, m_lut_binarize ? 1 : 0, (float)m_unbinarize_bias, 0.0f, 1.0f, nullptr),
+                        "bbhip_fp32_StochasticLut_ForwardClampW");
         }
         return y_buf;
     }

@@ -248,11 +248,17 @@ def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
     return y
 
 
-def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None):
+def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None, clamp_w=None):
+    """clamp_w = (lo, hi): W is clamped in place first, as StochasticLutN::Forward does (include/bb/StochasticLutN.h:451),
+    by the same launch that prepares the tables."""
     _dev(x, idx, W, out)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
     lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+    if clamp_w is not None:
+        check(lib().bbhip_fp32_StochasticLut_ForwardClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, frame_size, x.shape[1],
+                                                           int(input_binary), int(lut_binarize), bias, float(clamp_w[0]), float(clamp_w[1]), stream_ptr()))
+        return y
     check(lib().bbhip_fp32_StochasticLut_Forward(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, frame_size, x.shape[1],
                                                  int(input_binary), int(lut_binarize), bias, stream_ptr()))
     return y

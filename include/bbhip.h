@@ -240,6 +240,15 @@ int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *d
 int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
                                      float const *dev_W, int node_size, int frame_size, int frame_stride,
                                      int input_binary, int lut_binarize, float unbinarize_bias, void *stream);
+/* No single counterpart in the reference: its model class clamps the table in place and then calls the forward entry
+ * (m_W->Clamp_inplace(0, 1), include/bb/StochasticLutN.h:451, i.e. bbcu_fp32_Vector_clamp followed by
+ * bbcu_fp32_StochasticLut_Forward<N>).  This entry does both — dev_W is clamped to [w_lo, w_hi] in place by the launch that
+ * prepares the tables, then the forward pass runs on the clamped table: the same results as
+ * bbhip_fp32_Vector_clamp(dev_W, dev_W, w_lo, w_hi, node_size << n) + bbhip_fp32_StochasticLut_Forward, one launch fewer. */
+int bbhip_fp32_StochasticLut_ForwardClampW(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,
+                                           float *dev_W, int node_size, int frame_size, int frame_stride,
+                                           int input_binary, int lut_binarize, float unbinarize_bias,
+                                           float w_lo, float w_hi, void *stream);
 /* No counterpart in the reference.  bbhip_fp32_StochasticLut_Forward for callers that cannot allocate device memory — code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc: same arguments and results, but the
  * tables that the kernels read come from a fixed 8 MiB block inside the library (one per GPU, held until the process

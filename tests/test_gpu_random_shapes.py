@@ -284,6 +284,8 @@ def test_extended_random_run():
             run_case(ops, torch, 100000 + k)
             run_exact_case(ops, 400000 + k)
             run_tail_case(ops, torch, 700000 + k)
+            if (k + 1) % 500 == 0:
+                print("extended run: %d of %d" % (k + 1, count), flush=True)
     finally:
         ops.set_dx_mode(0)
     print("extended run: %d cases of each generator, no mismatch" % count)

@@ -57,6 +57,32 @@ def test_lut6_forward_backward(ops, shape, lut_binarize, input_binary):
     ops.set_dx_mode(0)
 
 
+@pytest.mark.parametrize("n,input_binary,lut_binarize", [(6, 0, 0), (6, 1, 0), (6, 0, 1), (4, 0, 0), (2, 1, 1)])
+def test_forward_that_clamps_the_table_in_place(ops, n, input_binary, lut_binarize):
+    """bbhip_fp32_StochasticLut_ForwardClampW = bbhip_fp32_Vector_clamp on W + bbhip_fp32_StochasticLut_Forward, bit for bit
+    (what StochasticLutN::Forward does before every pass, include/bb/StochasticLutN.h:451): W afterwards equals the oracle's
+    clamp, y equals the forward pass on the clamped table; a table already inside the range is left untouched."""
+    rng = np.random.default_rng(77 + n)
+    I, O, F = 40, 37, 700
+    stride = synth.frame_stride_fp32(F)
+    idx = synth.wiring(rng, I, O, n)
+    W0 = synth.lut_tables(rng, O, n, -0.3, 1.3)
+    x = synth.uniform_frames(rng, I, F, stride, -0.1, 1.1)
+    for lo, hi in ((0.0, 1.0), (0.25, 0.5)):
+        W = dev(W0.copy())
+        y = ops.stochastic_lut_forward(n, dev(x), dev(idx), W, F, input_binary, lut_binarize, clamp_w=(lo, hi))
+        Wc = oracle.vector_clamp(W0, lo, hi)
+        assert np.array_equal(host(W), Wc)
+        y2 = ops.stochastic_lut_forward(n, dev(x), dev(idx), dev(Wc), F, input_binary, lut_binarize)
+        assert np.array_equal(host(y)[:, :F], host(y2)[:, :F])
+        assert_fwd(host(y)[:, :F], oracle.stochastic_lut_forward(n, x, idx, Wc, F, input_binary, lut_binarize, 0.25, False)[:, :F], "y")
+        # a second call finds nothing to clamp and writes nothing back
+        y3 = ops.stochastic_lut_forward(n, dev(x), dev(idx), W, F, input_binary, lut_binarize, clamp_w=(lo, hi))
+        assert np.array_equal(host(W), Wc) and np.array_equal(host(y3)[:, :F], host(y)[:, :F])
+    with pytest.raises(RuntimeError):
+        ops.stochastic_lut_forward(n, dev(x), dev(idx), dev(W0.copy()), F, input_binary, lut_binarize, clamp_w=(1.0, 0.0))
+
+
 @pytest.mark.parametrize("n", [2, 3, 4, 5])
 def test_other_widths(ops, n):
     rng = np.random.default_rng(100 + n)
