@@ -258,12 +258,12 @@ def bench_differentiablelut6(args, lib):
         xb = torch.from_numpy(synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))).cuda()
 
     def step():
-        ops.vector_clamp_(W)
+        # (the table is clamped to [0, 1] in place by the forward entry's table launch, as the model class does before a forward pass)
         if bits:
-            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv)
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=(0.0, 1.0))
             ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev)
         else:
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=(0.0, 1.0))
             ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev)
 
     t_ramp = time.perf_counter()
@@ -325,8 +325,8 @@ def bench_conv_block(args, lib):
         cols = ops.im2col_forward(img, C, H, W_, F, FH, FW)
         a = cols; acts = []
         for l in layers:
-            ops.vector_clamp_(l["W"])
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"])
+            # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=(0.0, 1.0))
             acts.append((a, mean, rstd)); a = y
         maps = ops.col2im_forward(a, CO, OH, OW, F)
         pooled = ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F)
@@ -419,15 +419,15 @@ def bench_mnist_step(args, lib):
         a = x
         acts = []
         for l in layers:
-            ops.vector_clamp_(l["W"])
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"])
+            # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0))
             acts.append((a, mean, rstd)); a = y
         out = ops.average_lut_forward(a, idx_avg, F, False, False)
         dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
         acc, cat = ops.metrics_categorical_accuracy(out, t, CLASSES, 1, F)
         dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
         for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
-            l["dW"].zero_()
+            # dW accumulates; it is zero here because the optimizer's Update() zeroed it after the previous step (Optimizer.h:31-35)
             dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"])
         keep["loss_buf"], keep["acc"] = loss_buf, acc
 
@@ -447,7 +447,7 @@ def bench_mnist_step(args, lib):
         return (time.perf_counter() - t0) / args.steps
 
     def eager_step():
-        forward_backward(); adam.step()
+        forward_backward(); adam.update()
 
     dt_eager = timed(eager_step)
     graph = torch.cuda.CUDAGraph()
@@ -455,7 +455,7 @@ def bench_mnist_step(args, lib):
         forward_backward()
 
     def graph_step():
-        graph.replay(); adam.step()
+        graph.replay(); adam.update()
 
     dt_graph = timed(graph_step)
     loss = -float(keep["loss_buf"].sum().item()) / F

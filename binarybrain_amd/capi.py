@@ -52,6 +52,7 @@ _SIGNATURES = {
     "bbhip_fp32_Vector_max": (C.c_int, [_vp, _vp, _vp, _i, _vp]),
     "bbhip_fp32_Vector_max_v": (C.c_int, [_vp, _vp, _f, _i, _vp]),
     "bbhip_fp32_OptimizerAdam": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _vp]),
+    "bbhip_fp32_OptimizerAdam_Update": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _vp]),
     "bbhip_fp32_Im2Col_Forward": (C.c_int, [_vp, _vp] + [_i] * 15 + [_f, _vp]),
     "bbhip_bit_Im2Col_Forward": (C.c_int, [_vp, _vp] + [_i] * 15 + [_vp]),
     "bbhip_fp32_Im2Col_Backward": (C.c_int, [_vp, _vp] + [_i] * 14 + [_vp]),
@@ -75,6 +76,8 @@ _SIGNATURES = {
     "bbhip_bit_fp32_StochasticLut_Backward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 9 + [_f, _vp]),
     "bbhip_fp32_DifferentiableLutN_ForwardTraining": (C.c_int, [_i] + [_vp] * 8 + [_f] * 4 + [_i] * 5 + [_vp]),
     "bbhip_bit_fp32_DifferentiableLutN_ForwardTraining": (C.c_int, [_i] + [_vp] * 8 + [_f] * 4 + [_i] * 4 + [_vp]),
+    "bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW": (C.c_int, [_i] + [_vp] * 8 + [_f] * 4 + [_i] * 5 + [_f, _f, _vp]),
+    "bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW": (C.c_int, [_i] + [_vp] * 8 + [_f] * 4 + [_i] * 4 + [_f, _f, _vp]),
     "bbhip_fp32_DifferentiableLutN_ForwardInference": (C.c_int, [_i] + [_vp] * 6 + [_f] * 3 + [_i] * 5 + [_vp]),
     "bbhip_bit_fp32_DifferentiableLutN_ForwardInference": (C.c_int, [_i] + [_vp] * 6 + [_f] * 3 + [_i] * 4 + [_vp]),
     "bbhip_fp32_DifferentiableLutN_Backward": (C.c_int, [_i] + [_vp] * 12 + [_f] * 3 + [_i] * 9 + [_vp]),

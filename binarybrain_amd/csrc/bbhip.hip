@@ -1073,8 +1073,9 @@ int bbhip_fp32_Vector_max_v(float *dev_dst, float const *dev_src, float a, int s
     return vector_op<kVecMaxV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
-int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
-                             float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
+namespace {
+int adam_entry(bool zero_grads, int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
+               float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
 {
     g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(size >= 0 && size <= 65535);
@@ -1083,11 +1084,32 @@ int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *
                   dev_m_buf_table != nullptr && dev_v_buf_table != nullptr);
     // the element counts live on the device: a fixed number of blocks per tensor strides over its elements
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
-    hipLaunchKernelGGL(adam_kernel, dim3(kAdamBlocksPerTensor, (unsigned)size), dim3(kVecBlock), 0, static_cast<hipStream_t>(stream),
-                       dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table,
-                       lr_t, 1.0f - beta1, 1.0f - beta2);
+    dim3 const grid(kAdamBlocksPerTensor, (unsigned)size), block(kVecBlock);
+    if (zero_grads) {
+        hipLaunchKernelGGL(adam_kernel<true>, grid, block, 0, static_cast<hipStream_t>(stream),
+                           dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table,
+                           lr_t, 1.0f - beta1, 1.0f - beta2);
+    }
+    else {
+        hipLaunchKernelGGL(adam_kernel<false>, grid, block, 0, static_cast<hipStream_t>(stream),
+                           dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table,
+                           lr_t, 1.0f - beta1, 1.0f - beta2);
+    }
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+}  // namespace
+
+int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
+                             float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
+{
+    return adam_entry(false, size, dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table, lr_t, beta1, beta2, stream);
+}
+
+int bbhip_fp32_OptimizerAdam_Update(int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
+                                    float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
+{
+    return adam_entry(true, size, dev_size_table, dev_params_buf_table, dev_grads_buf_table, dev_m_buf_table, dev_v_buf_table, lr_t, beta1, beta2, stream);
 }
 
 int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
@@ -1564,6 +1586,42 @@ int bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(int n, int const *dev_x_bu
     c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
     c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.running_mean = dev_running_mean_buf; c.running_var = dev_running_var_buf;
     c.gamma = gamma; c.beta = beta; c.momentum = momentum;
+    return forward_entry(c, stream);
+}
+
+int bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode,
+        float w_lo, float w_hi, void *stream)
+{
+    BBHIP_REQUIRE(w_lo <= w_hi);
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = binary_mode ? kXBinary : kXClamp; c.ymode = binary_mode ? kYBinarize : kYClamp;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.running_mean = dev_running_mean_buf; c.running_var = dev_running_var_buf;
+    c.gamma = gamma; c.beta = beta; c.momentum = momentum;
+    c.clamp_W = dev_W; c.clamp_lo = w_lo; c.clamp_hi = w_hi;
+    return forward_entry(c, stream);
+}
+
+int bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW(int n, int const *dev_x_buf, int *dev_y_buf,
+        int const *dev_input_index, float *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize,
+        float w_lo, float w_hi, void *stream)
+{
+    BBHIP_REQUIRE(w_lo <= w_hi);
+    ForwardCall c{};
+    c.n = n; c.x = dev_x_buf; c.y = dev_y_buf; c.idx = dev_input_index; c.W = dev_W;
+    c.node_size = node_size; c.frame_size = frame_size; c.x_stride = frame_stride; c.y_stride = frame_stride;
+    c.xmode = kXBit; c.ymode = kYBit;
+    c.lut_binarize = lut_binarize; c.bias = unbinarize_bias;
+    c.bn = 1; c.mean = dev_mean_buf; c.rstd = dev_rstd_buf; c.running_mean = dev_running_mean_buf; c.running_var = dev_running_var_buf;
+    c.gamma = gamma; c.beta = beta; c.momentum = momentum;
+    c.clamp_W = dev_W; c.clamp_lo = w_lo; c.clamp_hi = w_hi;
     return forward_entry(c, stream);
 }
 

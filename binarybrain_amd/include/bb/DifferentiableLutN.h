@@ -228,7 +228,11 @@ public:
         if (x_buf.GetShape() != m_input_shape) { SetInputShape(x_buf.GetShape()); }
         FrameBuffer y_buf(x_buf.GetFrameSize(), m_output_shape, DataType<BinType>::type);
         if (train) { this->PushFrameBuffer(x_buf); }
-        if (m_flagClamp) { m_W->Clamp_inplace(0.0f, 1.0f); m_flagClamp = false; }
+        // The table is clamped to [0, 1] once after each backward pass (reference :605-608): by the training-forward entry
+        // itself, in its table-preparation launch, on the batch-norm training path; by a call of its own otherwise.
+        bool const clamp_in_entry = m_flagClamp && m_batch_norm && train;
+        if (m_flagClamp && !clamp_in_entry) { m_W->Clamp_inplace(0.0f, 1.0f); }
+        m_flagClamp = false;
         if (!kBitType && x_buf.GetType() == BB_TYPE_BIT) { x_buf = x_buf.ConvertBitToFP32(); }      // reference :610-613
         BB_ASSERT(x_buf.GetType() == DataType<BinType>::type);
 
@@ -238,6 +242,28 @@ public:
         auto x_ptr   = x_buf.LockDeviceMemoryConst();
         auto y_ptr   = y_buf.LockDeviceMemory(true);
         auto idx_ptr = m_connection_table.LockDeviceMemConst_InputTable();
+        if (clamp_in_entry) {
+            auto W_mut    = m_W->LockDeviceMemory();
+            auto mean_ptr = m_mean.LockDeviceMemory(true);
+            auto rstd_ptr = m_rstd.LockDeviceMemory(true);
+            auto rm_ptr   = m_running_mean.LockDeviceMemory();
+            auto rv_ptr   = m_running_var.LockDeviceMemory();
+            if (kBitType) {
+                CheckDevice(bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(),
+                                (int const *)idx_ptr.GetAddr(), (float *)W_mut.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
+                                (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
+                                O, F, y_stride, m_lut_binarize ? 1 : 0, 0.0f, 1.0f, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW");
+            }
+            else {
+                bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
+                CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
+                                (int const *)idx_ptr.GetAddr(), (float *)W_mut.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
+                                (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
+                                O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, 0.0f, 1.0f, nullptr),
+                            "bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW");
+            }
+            return y_buf;
+        }
         auto W_ptr   = m_W->LockDeviceMemoryConst();
 
         if (m_batch_norm && train) {

@@ -96,7 +96,14 @@ public:
 
     void ZeroGrad(void) override { m_grads.FillZero(); }
 
-    void Step(void) override
+    void Step(void) override { Apply(false); }
+
+    // Step() followed by ZeroGrad() (reference: Optimizer.h:31-35), as one launch: the update kernel zeroes each gradient
+    // element once it has used it.
+    void Update(void) override { Apply(true); }
+
+private:
+    void Apply(bool zero_grads)
     {
         index_t const n = m_params.GetSize();
         if (n == 0) { return; }
@@ -104,15 +111,16 @@ public:
         // make the device copies current (a host-side edit of a parameter or gradient marks them stale)
         for (index_t i = 0; i < n; ++i) {
             m_params[i].LockDeviceMemory();
-            m_grads[i].LockDeviceMemoryConst();
+            if (zero_grads) { m_grads[i].LockDeviceMemory(); } else { m_grads[i].LockDeviceMemoryConst(); }
             m_m[(std::size_t)i]->LockDeviceMemory();
             m_v[(std::size_t)i]->LockDeviceMemory();
         }
         T const lr_t = m_learning_rate * std::sqrt((T)1.0 - m_b2) / ((T)1.0 - m_b1);        // OptimizerAdam.h:171
-        CheckDevice(bbhip_fp32_OptimizerAdam((int)n, (int const *)m_size_table->LockDeviceConst(),
-                                             (float *const *)m_param_table->LockDeviceConst(), (float *const *)m_grad_table->LockDeviceConst(),
-                                             (float *const *)m_m_table->LockDeviceConst(), (float *const *)m_v_table->LockDeviceConst(),
-                                             lr_t, m_beta1, m_beta2, nullptr), "bbhip_fp32_OptimizerAdam");
+        auto const entry = zero_grads ? bbhip_fp32_OptimizerAdam_Update : bbhip_fp32_OptimizerAdam;
+        CheckDevice(entry((int)n, (int const *)m_size_table->LockDeviceConst(),
+                          (float *const *)m_param_table->LockDeviceConst(), (float *const *)m_grad_table->LockDeviceConst(),
+                          (float *const *)m_m_table->LockDeviceConst(), (float *const *)m_v_table->LockDeviceConst(),
+                          lr_t, m_beta1, m_beta2, nullptr), zero_grads ? "bbhip_fp32_OptimizerAdam_Update" : "bbhip_fp32_OptimizerAdam");
         m_b1 *= m_beta1;
         m_b2 *= m_beta2;
     }

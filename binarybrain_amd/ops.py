@@ -115,6 +115,14 @@ class AdamState:
         self.b1 = self.b1 * self.beta1
         self.b2 = self.b2 * self.beta2
 
+    def update(self):
+        """Optimizer::Update of the reference = step, then the gradients set to zero (include/bb/Optimizer.h:31-35), in one launch."""
+        check(lib().bbhip_fp32_OptimizerAdam_Update(len(self.params), ptr(self.t_size), ptr(self.t_params), ptr(self.t_grads),
+                                                    ptr(self.t_m), ptr(self.t_v), float(self.lr_t()), float(self.beta1),
+                                                    float(self.beta2), stream_ptr()))
+        self.b1 = self.b1 * self.beta1
+        self.b2 = self.b2 * self.beta2
+
 
 BORDER_MODES = {"constant": 0, "reflect": 1, "reflect_101": 2, "replicate": 3, "wrap": 4}
 
@@ -330,14 +338,22 @@ def bit_stochastic_lut_backward(n, xbits, dy, idx, W, dW, frame_size, rev=None, 
 
 
 def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True):
-    """fp32 frames. running_mean / running_var are updated in place. returns (y, mean, rstd)."""
+                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None):
+    """fp32 frames. running_mean / running_var are updated in place. returns (y, mean, rstd).
+    clamp_w = (lo, hi): W is clamped in place first, by the launch that prepares the tables (the model class's clamp before the
+    first forward pass after a backward pass, include/bb/DifferentiableLutN.h:605-608)."""
     _dev(x, idx, W, running_mean, running_var)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
     mean = torch.empty(O, dtype=torch.float32, device=x.device)
     rstd = torch.empty(O, dtype=torch.float32, device=x.device)
     lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+    if clamp_w is not None:
+        check(lib().bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
+                                                                        ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
+                                                                        O, frame_size, x.shape[1], int(lut_binarize), int(binary_mode),
+                                                                        float(clamp_w[0]), float(clamp_w[1]), stream_ptr()))
+        return y, mean, rstd
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardTraining(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                               ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
                                                               O, frame_size, x.shape[1], int(lut_binarize), int(binary_mode),
@@ -346,12 +362,18 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
 
 
 def bit_differentiable_lut_forward_training(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                            momentum=0.9, bias=0.25, lut_binarize=False):
+                                            momentum=0.9, bias=0.25, lut_binarize=False, clamp_w=None):
     _dev(xbits, idx, W, running_mean, running_var)
     O = idx.shape[0]
     y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
     mean = torch.empty(O, dtype=torch.float32, device=xbits.device)
     rstd = torch.empty(O, dtype=torch.float32, device=xbits.device)
+    if clamp_w is not None:
+        check(lib().bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
+                                                                            ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
+                                                                            O, frame_size, xbits.shape[1], int(lut_binarize),
+                                                                            float(clamp_w[0]), float(clamp_w[1]), stream_ptr()))
+        return y, mean, rstd
     check(lib().bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                                   ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
                                                                   O, frame_size, xbits.shape[1], int(lut_binarize), stream_ptr()))

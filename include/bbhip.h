@@ -160,6 +160,12 @@ int bbhip_fp32_Vector_max_v(float *dev_dst, float const *dev_src, float a, int s
 int bbhip_fp32_OptimizerAdam(int size, int const *dev_size_table, float *const *dev_params_buf_table,
                              float *const *dev_grads_buf_table, float *const *dev_m_buf_table,
                              float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream);
+/* No single counterpart in the reference: Optimizer::Update() is Step() followed by ZeroGrad() (include/bb/Optimizer.h:31-35,
+ * include/bb/OptimizerAdam.h:132-139), i.e. bbcu_fp32_OptimizerAdam and then one fill per gradient tensor.  This entry does
+ * both: the same update as bbhip_fp32_OptimizerAdam, and every gradient element is set to 0 once it has been used. */
+int bbhip_fp32_OptimizerAdam_Update(int size, int const *dev_size_table, float *const *dev_params_buf_table,
+                                    float *const *dev_grads_buf_table, float *const *dev_m_buf_table,
+                                    float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream);
 
 /* bbcu_ConvBitToReal<float>, include/bbcu/bbcu.h:246-258 */
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
@@ -294,6 +300,20 @@ int bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(int n, int const *dev_x_bu
         int const *dev_input_index, float const *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
         float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
         float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, void *stream);
+/* No single counterpart in the reference: its model class clamps the table in place before the first forward pass after a
+ * backward pass (m_W->Clamp_inplace(0, 1), include/bb/DifferentiableLutN.h:605-608) and then calls the forward entry.  These two
+ * do both, like bbhip_fp32_StochasticLut_ForwardClampW: dev_W is clamped to [w_lo, w_hi] in place by the launch that prepares
+ * the tables, and the pass runs on the clamped table; all other arguments and results as in the entries above. */
+int bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(int n, float const *dev_x_buf, float *dev_y_buf,
+        int const *dev_input_index, float *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode,
+        float w_lo, float w_hi, void *stream);
+int bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW(int n, int const *dev_x_buf, int *dev_y_buf,
+        int const *dev_input_index, float *dev_W, float *dev_mean_buf, float *dev_rstd_buf,
+        float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        float unbinarize_bias, int node_size, int frame_size, int frame_stride, int lut_binarize,
+        float w_lo, float w_hi, void *stream);
 /* bbcu_fp32_DifferentiableLutN_ForwardInference<N>, include/bbcu/bbcu.h:563-581
  * (rstd = 1/sqrt(running_var) and the hard-tanh clip follow the reference's CPU path, include/bb/DifferentiableLutN.h:866-897) */
 int bbhip_fp32_DifferentiableLutN_ForwardInference(int n, float const *dev_x_buf, float *dev_y_buf,

@@ -266,6 +266,35 @@ def test_bit_variants(ops, n):
             ops.set_dx_mode(0)
 
 
+@pytest.mark.parametrize("n", [6, 3])
+def test_training_forward_that_clamps_the_table_in_place(ops, n):
+    """The ...ForwardTrainingClampW entries = bbhip_fp32_Vector_clamp on W + the ForwardTraining entry, bit for bit (the model
+    class clamps its table before the first forward pass after a backward pass, include/bb/DifferentiableLutN.h:605-608):
+    W afterwards equals the oracle's clamp; outputs, statistics and running statistics equal those of the two-call form."""
+    rng = np.random.default_rng(900 + n)
+    I, O, F = 48, 41, 1100
+    idx = synth.wiring(rng, I, O, n)
+    W0 = synth.lut_tables(rng, O, n, -0.3, 1.3)
+    Wc = oracle.vector_clamp(W0, 0.0, 1.0)
+    ys = synth.frame_stride_fp32(F)
+    x = synth.uniform_frames(rng, I, F, ys)
+    xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))
+    rm = rng.random(O).astype(np.float32); rv = (rng.random(O) + 0.5).astype(np.float32)
+    for binary_mode in (True, False):
+        W = dev(W0.copy()); rm1, rv1 = dev(rm), dev(rv); rm2, rv2 = dev(rm), dev(rv)
+        y1, m1, r1 = ops.differentiable_lut_forward_training(n, dev(x), dev(idx), W, F, rm1, rv1, binary_mode=binary_mode, clamp_w=(0.0, 1.0))
+        y2, m2, r2 = ops.differentiable_lut_forward_training(n, dev(x), dev(idx), dev(Wc), F, rm2, rv2, binary_mode=binary_mode)
+        assert np.array_equal(host(W), Wc)
+        for a, b in ((y1[:, :F], y2[:, :F]), (m1, m2), (r1, r2), (rm1, rm2), (rv1, rv2)):
+            assert np.array_equal(host(a), host(b))
+    W = dev(W0.copy()); rm1, rv1 = dev(rm), dev(rv); rm2, rv2 = dev(rm), dev(rv)
+    y1, m1, r1 = ops.bit_differentiable_lut_forward_training(n, dev(xb), dev(idx), W, F, rm1, rv1, clamp_w=(0.0, 1.0))
+    y2, m2, r2 = ops.bit_differentiable_lut_forward_training(n, dev(xb), dev(idx), dev(Wc), F, rm2, rv2)
+    assert np.array_equal(host(W), Wc)
+    for a, b in ((y1, y2), (m1, m2), (r1, r2), (rm1, rm2), (rv1, rv2)):
+        assert np.array_equal(host(a), host(b))
+
+
 @pytest.mark.parametrize("n", [6, 4])
 def test_no_batchnorm_forward(ops, n):
     rng = np.random.default_rng(400 + n)
