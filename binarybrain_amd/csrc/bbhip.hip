@@ -139,7 +139,7 @@ int dx_chunk_frames_env(void) { static int v = env_int("BBHIP_DX_CHUNK", 0); ret
 int dx_pass_steps_env(void)   { static int v = env_int("BBHIP_DX_STEPS", 0); return (v <= 0) ? 0 : (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
 // BinaryLut6 units of 128 words: 8192 input rows x 512 bytes is what an XCD's 4 MiB L2 holds (1.2 GB fetched per launch at
 // the benchmark shape; 192-word units fetch 1.9 GB, 256-word units 2.3 GB).  With the per-wavefront set-up at its
-// present cost the shorter units are also the fastest (201 us; 192 words 206 us, 256 words 250 us, 64 words 251 us).
+// present cost the shorter units are also the fastest (241 us; 192 words 278 us, 256 words 332 us, 64 words 282 us).
 int bin_chunk_words(void)  { static int v = env_int("BBHIP_BIN_CHUNK", 128); return (((v > 0 ? v : 128) + 63) / 64) * 64; }
 int bin_nodes_per_wave(void) { static int v = env_int("BBHIP_BIN_NODES", 0); return v >= 4 ? 4 : v >= 2 ? 2 : v == 1 ? 1 : 0; }     // 0: chosen per call
 
