@@ -81,7 +81,9 @@ static void test_stochastic(int I, int O, int F, bool lut_binarize, bool binary)
     std::vector<std::int32_t> idx; wire<N>(mt, I, O, idx);
     for (int o = 0; o < O; ++o) for (int i = 0; i < N; ++i) { lut->SetNodeConnectionIndex(o, i, idx[(size_t)o * N + i]); }
     std::vector<float> W((size_t)O * NN), x((size_t)I * F), dy((size_t)O * F);
-    { auto Wp = lut->lock_W(); for (int o = 0; o < O; ++o) for (int i = 0; i < NN; ++i) { W[(size_t)o * NN + i] = std::min(1.0f, std::max(0.0f, uni(mt))); Wp(o, i) = W[(size_t)o * NN + i]; } }
+    // the layer gets table entries in [-0.1, 1.1]: Forward clamps them to [0, 1] in place first (reference: StochasticLutN.h:451),
+    // so the oracle works on the clamped table and the layer's own table must equal it afterwards
+    { auto Wp = lut->lock_W(); for (int o = 0; o < O; ++o) for (int i = 0; i < NN; ++i) { float const w = uni(mt); Wp(o, i) = w; W[(size_t)o * NN + i] = std::min(1.0f, std::max(0.0f, w)); } }
     { auto xp = x_buf.Lock<float>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x[(size_t)n * F + f] = uni(mt); xp.Set(f, n, x[(size_t)n * F + f]); } }
     bb::FrameBuffer dy_buf(F, {O}, BB_TYPE_FP32);
     { auto dp = dy_buf.Lock<float>(true); for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dy[(size_t)n * F + f] = nrm(mt); dp.Set(f, n, dy[(size_t)n * F + f]); } }
@@ -98,6 +100,12 @@ static void test_stochastic(int I, int O, int F, bool lut_binarize, bool binary)
         }
         std::vector<float> dW((size_t)O * NN);
         { auto p = lut->lock_dW_const(); for (int o = 0; o < O; ++o) for (int i = 0; i < NN; ++i) { dW[(size_t)o * NN + i] = p(o, i); } }
+        {
+            auto Wp = lut->lock_W_const();
+            size_t bad = 0;
+            for (int o = 0; o < O; ++o) for (int i = 0; i < NN; ++i) { bad += (Wp(o, i) != W[(size_t)o * NN + i]); }
+            CHECK(bad == 0, "StochasticLut%d: %zu table entries differ from the clamped table after Forward", N, bad);
+        }
         CHECK(max_diff(y, y_ref) <= 1e-5, "StochasticLut%d %dx%dx%d y err %g", N, I, O, F, max_diff(y, y_ref));
         CHECK(max_diff(dx, dx_ref) <= 1e-4 * max_abs(dx_ref), "StochasticLut%d dx err %g", N, max_diff(dx, dx_ref));
         CHECK(max_diff(dW, dW_ref) <= 1e-4 * max_abs(dW_ref), "StochasticLut%d dW err %g (loop %d)", N, max_diff(dW, dW_ref), loop);
