@@ -612,8 +612,10 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     TermArgs tt{};
     if (dxmode == kDxNone && term_count > 0) {
         size_t const records = (size_t)c.input_node_size * (size_t)(c.rev_stride - 1);
-        size_t const blocks = (((records + kWavesPerBlk - 1) / kWavesPerBlk) + 7) & ~(size_t)7;      // whole rounds over the XCDs
-        if (blocks + (size_t)slab_total * tile_count > 0x7fffffffULL) { return fail("backward: grid too large"); }
+        size_t const per_block = (size_t)kWavesPerBlk * kTermRecordsPerWave;
+        size_t const blocks = (((records + per_block - 1) / per_block) + 7) & ~(size_t)7;            // whole rounds over the XCDs
+        if (records > 0x7fffffffULL || blocks + (size_t)slab_total * tile_count > 0x7fffffffULL) { return fail("backward: grid too large"); }
+        tt.fan = make_tile_divisor(c.rev_stride - 1);
         tt.W = c.W; tt.idx = c.idx; tt.rev = c.rev; tt.term = term;
         tt.x_base = (unsigned long long)(uintptr_t)c.x; tt.x_row_pitch_bytes = (unsigned long long)c.x_stride * 4ULL;
         tt.dy_base = (unsigned long long)(uintptr_t)(c.bn ? (void const *)dyh : (void const *)c.dy);

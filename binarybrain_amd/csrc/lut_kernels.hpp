@@ -588,67 +588,87 @@ struct TermArgs {
     int         *term;          // the records
     unsigned long long x_base, x_row_pitch_bytes, dy_base, dy_row_pitch_bytes;
     int lut_binarize, rev_stride, input_node_size;
-    int blocks;                 // workgroups that build records (kWavesPerBlk records each); 0 = nothing to build
+    TileDivisor fan;            // division by the slots per input, rev_stride - 1
+    int blocks;                 // workgroups that build records (kWavesPerBlk * kTermRecordsPerWave records each); 0 = nothing to build
     int corner;                 // 1: records hold the derivative's corner values for two-valued inputs (lut_dx_corner_kernel)
     float lo, hi;               //    the two input values, 1/2 -+ bias
 };
 
-// one wavefront per record: lane i holds entry i of the consumer's table while it is brought into the plain basis.
+// A wavefront builds kTermRecordsPerWave consecutive records: lane i holds entry i of a consumer's table while it is
+// brought into the plain basis.  The records' loads go out together — reverse-table entries, then wiring and tables — so a
+// wavefront pays the two memory round trips of a record once for all of them (one record per wavefront made the builder
+// the longest part of the table-gradient launch of a layer with few nodes and many connections per input).
 // Slots beyond an input's fan-out are never read by the dx kernel and are left alone.
+constexpr int kTermRecordsPerWave = 4;
+
 template <int N>
 __device__ __forceinline__ void term_table_block(TermArgs const &a, int block)
 {
     static_assert(2 * N <= kTermHead && kTermHead <= kWave, "head size");
-    constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN;
-    int const max_fan = a.rev_stride - 1;
-    long long const rec = (long long)block * kWavesPerBlk + (int)(threadIdx.x / kWave);
-    if (rec >= (long long)a.input_node_size * max_fan) { return; }
+    constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN, R = kTermRecordsPerWave;
+    int const total = a.fan.count * a.input_node_size;          // records, below 2^31 (checked on the host)
+    int const rec0  = __builtin_amdgcn_readfirstlane((block * kWavesPerBlk + (int)(threadIdx.x / kWave)) * R);
+    if (rec0 >= total) { return; }
     int const lane = threadIdx.x & (kWave - 1);
-    int const in   = (int)(rec / max_fan);
-    int const slot = (int)(rec - (long long)in * max_fan);
-    int const *r = a.rev + (size_t)in * a.rev_stride;
-    int const cnt  = r[0];
-    int const e    = r[1 + slot];                  // inside the row for every slot: both loads go out together
-    if (slot >= cnt) { return; }
-    int const k    = e % N;
-    int const node = e / N;
-    int *out = a.term + rec * REC;
+    // wave-uniform loads of tables that no kernel of the call writes: scalar loads through the constant address space
+    typedef __attribute__((address_space(4))) int const const_int;
+    const_int *rev = (const_int *)a.rev;
 
-    if (lane < kTermHead) {
-        int v = 0;
+    int in[R], slot[R], cnt[R], e[R];
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+        int const rec = min(rec0 + q, total - 1);               // (a wavefront past the last record repeats it and stores nothing)
+        split_tile(rec, a.fan, in[q], slot[q]);                 // rec = in * max_fan + slot
+        const_int *r = rev + (size_t)in[q] * a.rev_stride;
+        cnt[q] = r[0];
+        e[q]   = r[1 + slot[q]];                                // inside the row for every slot
+    }
+    bool  live[R];
+    int   k[R], node[R], head[R];
+    float v[R];
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+        live[q] = (rec0 + q < total) && (slot[q] < cnt[q]);
+        int const eq = live[q] ? e[q] : 0;                      // (whatever an unused slot holds is not followed)
+        k[q]    = eq % N;
+        node[q] = eq / N;
+        head[q] = 0;
         if (lane < 2 * N) {
             int const j = lane >> 1;
-            unsigned long long const addr = (j < N - 1) ? a.x_base + (unsigned long long)a.idx[node * N + ((j < k) ? j : j + 1)] * a.x_row_pitch_bytes
-                                                        : a.dy_base + (unsigned long long)node * a.dy_row_pitch_bytes;
-            v = (lane & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
+            unsigned long long const addr = (j < N - 1) ? a.x_base + (unsigned long long)(unsigned)a.idx[node[q] * N + ((j < k[q]) ? j : j + 1)] * a.x_row_pitch_bytes
+                                                        : a.dy_base + (unsigned long long)(unsigned)node[q] * a.dy_row_pitch_bytes;
+            head[q] = (lane & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
         }
-        out[lane] = v;
-    }
-
-    // P = plain-basis coefficients of W' (W' = lut_binarize ? W > 0.5 : W): the butterfly (a, b) -> (a, b - a) per index bit.
-    // For two-valued inputs the record holds values instead of coefficients: dy/dx_k at the corner where every other
-    // input j takes lo or hi.  W' is the table of y at x in {0, 1}^N and y is linear in each input, so input j != k
-    // interpolates, (a, b) -> (a + lo (b - a), a + hi (b - a)), and input k differentiates, (a, b) -> (., b - a).
-    float v = 0.0f;
-    if (lane < NN) {
-        v = a.W[(size_t)node * NN + lane];
-        if (a.lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+        v[q] = 0.0f;
+        if (lane < NN) { v[q] = a.W[(size_t)node[q] * NN + lane]; }
     }
 #pragma unroll
-    for (int j = 0; j < N; ++j) {
-        float const o   = __shfl_xor(v, 1 << j, 64);
-        bool const  up  = (lane >> j) & 1;
-        if (a.corner && j != k) {
-            float const lower = up ? o : v, step = up ? (v - o) : (o - v);
-            v = __builtin_fmaf(up ? a.hi : a.lo, step, lower);
+    for (int q = 0; q < R; ++q) {
+        if (!live[q]) { continue; }                             // wave-uniform
+        int *out = a.term + (size_t)(rec0 + q) * REC;
+        if (lane < kTermHead) { out[lane] = head[q]; }
+        // P = plain-basis coefficients of W' (W' = lut_binarize ? W > 0.5 : W): the butterfly (a, b) -> (a, b - a) per index bit.
+        // For two-valued inputs the record holds values instead of coefficients: dy/dx_k at the corner where every other
+        // input j takes lo or hi.  W' is the table of y at x in {0, 1}^N and y is linear in each input, so input j != k
+        // interpolates, (a, b) -> (a + lo (b - a), a + hi (b - a)), and input k differentiates, (a, b) -> (., b - a).
+        float w = v[q];
+        if (a.lut_binarize) { w = (w > 0.5f) ? 1.0f : 0.0f; }
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            float const o   = __shfl_xor(w, 1 << j, 64);
+            bool const  up  = (lane >> j) & 1;
+            if (a.corner && j != k[q]) {
+                float const lower = up ? o : w, step = up ? (w - o) : (o - w);
+                w = __builtin_fmaf(up ? a.hi : a.lo, step, lower);
+            }
+            else {
+                w = up ? (w - o) : w;
+            }
         }
-        else {
-            v = up ? (v - o) : v;
+        if (lane < NN && ((lane >> k[q]) & 1)) {
+            int const sidx = (lane & ((1 << k[q]) - 1)) | ((lane >> (k[q] + 1)) << k[q]);      // the entry's index with bit k taken out
+            out[kTermHead + sidx] = __float_as_int(w);
         }
-    }
-    if (lane < NN && ((lane >> k) & 1)) {
-        int const sidx = (lane & ((1 << k) - 1)) | ((lane >> (k + 1)) << k);      // the entry's index with bit k taken out
-        out[kTermHead + sidx] = __float_as_int(v);
     }
 }
 
