@@ -137,6 +137,14 @@ int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  retur
 // per-term set-up per frame.  0: not set in the environment.
 int dx_chunk_frames_env(void) { static int v = env_int("BBHIP_DX_CHUNK", 0); return ((v + 63) / 64) * 64; }
 int dx_pass_steps_env(void)   { static int v = env_int("BBHIP_DX_STEPS", 0); return (v <= 0) ? 0 : (v <= 1) ? 1 : (v <= 2) ? 2 : 4; }
+// dx work lists split over the four wavefronts of a workgroup (DxArgs::split): where one wavefront per (input node, unit) would
+// leave the launch with fewer than 4096 workgroups and the lists are long enough to share.  BBHIP_DX_SPLIT = 0 / 1 forces it.
+bool dx_split_lists(int max_fan, long long workgroups)
+{
+    static int const env = env_int("BBHIP_DX_SPLIT", 2);
+    if (env == 0 || env == 1) { return env == 1; }
+    return max_fan >= 16 && workgroups < 4096;
+}
 // BinaryLut6 units of 128 words: 8192 input rows x 512 bytes is what an XCD's 4 MiB L2 holds (1.2 GB fetched per launch at
 // the benchmark shape; 192-word units fetch 1.9 GB, 256-word units 2.3 GB).  With the per-wavefront set-up at its
 // present cost the shorter units are also the fastest (241 us; 192 words 278 us, 256 words 332 us, 64 words 282 us).
@@ -696,14 +704,16 @@ int run_backward(BackwardCall const &call, hipStream_t st)
         int const frames = dx_chunk_frames_env() ? dx_chunk_frames_env() : (bit_corner ? 256 : 128);
         int const chunk  = ((frames + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
         int const chunk_count = ceil_div(c.frame_size, chunk);
-        int const in_tiles    = ceil_div(c.input_node_size, kWavesPerBlk);
+        // few input nodes with long work lists: the four wavefronts of a workgroup share one input node (DxArgs::split)
+        bool const split   = dx_split_lists(c.rev_stride - 1, (long long)chunk_count * ceil_div(c.input_node_size, kWavesPerBlk));
+        int const in_tiles = split ? c.input_node_size : ceil_div(c.input_node_size, kWavesPerBlk);
         if ((long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
         DxArgs d{};
         d.x = c.x; d.dy = c.bn ? dyh : c.dy; d.dx = c.dx; d.rev = c.rev; d.term = term;
         d.rev_stride = c.rev_stride; d.input_node_size = c.input_node_size; d.frame_size = c.frame_size;
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
         d.chunk = chunk; d.chunk_count = chunk_count; d.tiles = make_tile_divisor(in_tiles);
-        d.bias = c.bias;
+        d.bias = c.bias; d.split = split ? 1 : 0;
         // folding the slab sums into dW rides at the end of this launch
         d.fin_partial = part; d.fin_dW = c.dW; d.fin_node_size = c.output_node_size; d.fin_slab_count = slab_total;
         d.fin_blocks = (ceil_div(c.output_node_size * NN, kBlock) + 7) & ~7;

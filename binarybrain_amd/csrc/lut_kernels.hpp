@@ -914,6 +914,11 @@ struct DxArgs {
     int   chunk, chunk_count;
     TileDivisor tiles;
     float bias;
+    // split != 0: the four wavefronts of a workgroup share ONE input node and a quarter of its work list each; their sums are
+    // added in wavefront order through LDS.  For layers with few input nodes and long lists (784 inputs feeding 6144 nodes:
+    // 47 consumers each), where one wavefront per (input, unit) leaves most of the device idle behind a long serial walk.
+    // tiles then counts input nodes, not groups of four.
+    int   split;
     // the last fin_blocks workgroups of the launch fold the table-gradient partial sums into dW (dw_finalize_block)
     float const *fin_partial;
     float       *fin_dW;
@@ -1030,6 +1035,51 @@ struct DxTerm {
     }
 };
 
+// The wavefront's share of an input node's work list (the whole list, or a quarter of it in split mode) ...
+__device__ __forceinline__ void dx_list_share(DxArgs const &a, int tile, int wave, int &in, int &t_scale)
+{
+    // (the wavefront's number within the workgroup is the same in all its lanes; saying so keeps everything derived from it —
+    // list bounds, record addresses — in scalar registers and on scalar loads)
+    int const w = __builtin_amdgcn_readfirstlane(wave);
+    in      = __builtin_amdgcn_readfirstlane(a.split ? tile : tile * kWavesPerBlk + w);
+    t_scale = a.split ? w : -1;
+}
+__device__ __forceinline__ void dx_list_range(int cnt, int share, int &t_begin, int &t_end)
+{
+    t_begin = (share < 0) ? 0   : (cnt * share) / kWavesPerBlk;
+    t_end   = (share < 0) ? cnt : (cnt * (share + 1)) / kWavesPerBlk;
+}
+
+// ... and the end of a pass: the lane's U sums go to dx — directly, or in split mode added over the workgroup's wavefronts
+// in wavefront order (a fixed order: results do not depend on timing) by the first of them.  Every wavefront of the
+// workgroup must come here (the barrier).
+template <int U>
+__device__ __forceinline__ void dx_store_pass(DxArgs const &a, float (&part)[kWavesPerBlk][U][kWave], int in, int wave, int lane,
+                                              int f_begin, float (&acc)[U])
+{
+    if (a.split) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) { part[wave][u][lane] = acc[u]; }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float sum = part[0][u][lane];
+#pragma unroll
+                for (int w = 1; w < kWavesPerBlk; ++w) { sum += part[w][u][lane]; }
+                acc[u] = sum;
+            }
+        }
+        __syncthreads();                    // the next pass writes part again
+        if (wave != 0) { return; }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        int const f = f_begin + u * kWave + lane;
+        if (f < a.frame_size) { __builtin_nontemporal_store(acc[u], a.dx + (size_t)in * a.dx_stride + f); }
+    }
+}
+
 template <int N, int XMODE, int U>
 __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 {
@@ -1042,11 +1092,16 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
     int const lid  = xcd_remap(bid, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
-    int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
-    if (in >= a.input_node_size) { return; }
+    __shared__ float part[kWavesPerBlk][U][kWave];
+    int const wave = threadIdx.x / kWave;
+    int in, share;
+    dx_list_share(a, tile, wave, in, share);
+    if (in >= a.input_node_size) { return; }            // (workgroup-uniform in split mode)
     int const lane = threadIdx.x & (kWave - 1);
 
     int const cnt = a.rev[(size_t)in * a.rev_stride];
+    int t_begin, t_end;
+    dx_list_range(cnt, share, t_begin, t_end);
     // The term table is read through the constant address space: its wave-uniform loads stay scalar loads wherever
     // they are placed relative to the stores of this kernel (the table is written by an earlier kernel).
     typedef __attribute__((address_space(4))) int const const_int;
@@ -1072,17 +1127,17 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
         // loads do not wait for a scalar-memory round trip first
         constexpr int HEAD = 2 * T::M + 2;
         int head_next[HEAD];
-        if (cnt > 0) {
+        if (t_begin < t_end) {
 #pragma unroll
-            for (int i = 0; i < HEAD; ++i) { head_next[i] = rec[i]; }
+            for (int i = 0; i < HEAD; ++i) { head_next[i] = rec[(size_t)t_begin * T::REC + i]; }
         }
-        for (int t = 0; t < cnt; ++t) {
+        for (int t = t_begin; t < t_end; ++t) {
             typename T::Stage st;
             float Dk[T::HN];
             int head[HEAD];
 #pragma unroll
             for (int i = 0; i < HEAD; ++i) { head[i] = head_next[i]; }
-            if (t + 1 < cnt) {
+            if (t + 1 < t_end) {
 #pragma unroll
                 for (int i = 0; i < HEAD; ++i) { head_next[i] = rec[(size_t)(t + 1) * T::REC + i]; }
             }
@@ -1090,12 +1145,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
             T::load_coefficients(rec + (size_t)t * T::REC, Dk);
             T::accumulate(st, Dk, bit, lo, hi, acc);
         }
-
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int const f = f_begin + u * kWave + lane;
-            if (f < a.frame_size) { __builtin_nontemporal_store(acc[u], a.dx + (size_t)in * a.dx_stride + f); }
-        }
+        dx_store_pass<U>(a, part, in, wave, lane, f_begin, acc);
     }
 }
 
@@ -1117,11 +1167,16 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
     int const lid  = xcd_remap(bid, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
-    int const in   = __builtin_amdgcn_readfirstlane(tile * kWavesPerBlk + (int)(threadIdx.x / kWave));
-    if (in >= a.input_node_size) { return; }
+    __shared__ float part[kWavesPerBlk][U][kWave];
+    int const wave = threadIdx.x / kWave;
+    int in, share;
+    dx_list_share(a, tile, wave, in, share);
+    if (in >= a.input_node_size) { return; }            // (workgroup-uniform in split mode)
     int const lane = threadIdx.x & (kWave - 1);
 
     int const cnt = a.rev[(size_t)in * a.rev_stride];
+    int t_begin, t_end;
+    dx_list_range(cnt, share, t_begin, t_end);
     typedef __attribute__((address_space(4))) int const const_int;
     const_int *rec = (const_int *)(a.term + (size_t)in * (a.rev_stride - 1) * T::REC);
     int const *rec_v = a.term + (size_t)in * (a.rev_stride - 1) * T::REC + kTermHead + (lane & (T::HN - 1));
@@ -1141,19 +1196,19 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
         // is evaluated — this path is bound by the round trips of a term, not by its instructions
         int head_next[2 * T::M + 2], values_next = 0;
         if constexpr (XMODE == kXBit) {
-            if (cnt > 0) {
+            if (t_begin < t_end) {
 #pragma unroll
-                for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[i]; }
-                values_next = rec_v[0];
+                for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[(size_t)t_begin * T::REC + i]; }
+                values_next = rec_v[(size_t)t_begin * T::REC];
             }
         }
-        for (int t = 0; t < cnt; ++t) {
+        for (int t = t_begin; t < t_end; ++t) {
             if constexpr (XMODE == kXBit) {
                 int r[2 * T::M + 2];
 #pragma unroll
                 for (int i = 0; i < 2 * T::M + 2; ++i) { r[i] = head_next[i]; }
                 int const values = values_next;                    // lane p: the term's value at corner p
-                if (t + 1 < cnt) {
+                if (t + 1 < t_end) {
 #pragma unroll
                     for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[(size_t)(t + 1) * T::REC + i]; }
                     values_next = rec_v[(size_t)(t + 1) * T::REC];
@@ -1199,12 +1254,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
                 acc[u] = __builtin_fmaf(st.dyv[u], d, acc[u]);
             }
         }
-
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int const f = f_begin + u * kWave + lane;
-            if (f < a.frame_size) { __builtin_nontemporal_store(acc[u], a.dx + (size_t)in * a.dx_stride + f); }
-        }
+        dx_store_pass<U>(a, part, in, wave, lane, f_begin, acc);
     }
 }
 
