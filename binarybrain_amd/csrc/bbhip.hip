@@ -123,10 +123,10 @@ int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); ret
 // Frames per forward unit.  fp32 rows are gathered through L2, and a 256-frame piece of every input row is what one XCD's L2
 // holds; packed-bit rows are 32 times smaller, so their units are longer and a unit's set-up (wiring, table) weighs less.
 // Longer units are halved while they would leave the launch with fewer than 2048 workgroups.
+int fwd_chunk_frames_env(void) { static int env = env_int("BBHIP_FWD_CHUNK", 0); return env > 0 ? ((env + 63) / 64) * 64 : 0; }
 int fwd_chunk_frames(int xmode, int frame_size, int tile_count)
 {
-    static int env = env_int("BBHIP_FWD_CHUNK", 0);
-    if (env > 0) { return ((env + 63) / 64) * 64; }
+    if (fwd_chunk_frames_env() > 0) { return fwd_chunk_frames_env(); }
     int chunk = (xmode == kXBit) ? 1024 : 256;
     while (chunk > 256 && (long long)((frame_size + chunk - 1) / chunk) * tile_count < 2048) { chunk /= 2; }
     return chunk;
@@ -418,7 +418,11 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     bool const corner     = use_corner_values(c.xmode);
     int const npw         = corner ? 1 : fwd_nodes_per_wave();
     int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
-    int const chunk       = fwd_chunk_frames(c.xmode, c.frame_size, tile_count);
+    // Batch-norm training pass of a small batch on the corner-value kernel: one unit per node, so that the wavefront that writes a
+    // node's output can sum the node's statistics itself (kStatInline) and the statistics launch falls away — at up to 1024 frames
+    // a launch costs more than the second evaluation of the unit does.  BBHIP_FWD_CHUNK set in the environment keeps its say.
+    bool const one_unit   = (c.bn == 1) && corner && c.frame_size <= 1024 && fwd_chunk_frames_env() == 0;
+    int const chunk       = one_unit ? 1024 : fwd_chunk_frames(c.xmode, c.frame_size, tile_count);
     int const chunk_count = ceil_div(c.frame_size, chunk);
     if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("forward: grid too large"); }
 
@@ -450,7 +454,14 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     a.bias = c.bias; a.gamma = c.gamma; a.beta = c.beta;
 
     int kind = 0;
-    if (c.bn == 1) {
+    if (c.bn == 1 && corner && chunk_count == 1) {
+        // one unit per node and the cheap corner-value kernel: its wavefronts sum the statistics of their node themselves
+        // before they write its output, which saves the statistics launch (the evaluation it repeats costs less than that)
+        a.stat_mode = kStatInline; a.momentum = c.momentum;
+        a.mean_out = c.mean; a.rstd_out = c.rstd; a.running_mean = c.running_mean; a.running_var = c.running_var;
+        kind = 1;
+    }
+    else if (c.bn == 1) {
         a.stat_partial = stat;
         if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();

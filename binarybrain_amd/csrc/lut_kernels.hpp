@@ -201,7 +201,9 @@ struct FwdArgs {
     float *mean_out, *rstd_out, *running_mean, *running_var;
 };
 
-enum StatMode : int { kStatGiven = 0, kStatRunning = 1, kStatPartial = 2 };
+// kStatInline: the call has one unit per node, so the wavefront that writes a node's output first sums the node's statistics
+// itself (a pass of its own over the unit) instead of reading them from a statistics launch
+enum StatMode : int { kStatGiven = 0, kStatRunning = 1, kStatPartial = 2, kStatInline = 3 };
 constexpr int kInlineStatUnits = kWave;     // most units whose partial sums a wavefront adds up itself: one load per lane
 
 // What a forward kernel does with the LUT output v of (node, frame f = f0 + lane): accumulate statistics (kinds 2, 3) or
@@ -311,7 +313,7 @@ __device__ __forceinline__ void forward_statistics(FwdArgs const &a, int node, i
 // of the wave-uniform loads of the set-up would take them off the scalar path.
 __device__ __forceinline__ void forward_store_statistics(FwdArgs const &a, int node, bool live, int ck, int lane, float mean, float var, float rstd)
 {
-    if (a.stat_mode == kStatPartial && ck == 0 && lane == 0 && live) {
+    if ((a.stat_mode == kStatPartial || a.stat_mode == kStatInline) && ck == 0 && lane == 0 && live) {
         store_statistics(a.mean_out, a.rstd_out, a.running_mean, a.running_var, node, mean, var, rstd, a.momentum);
     }
 }
@@ -455,6 +457,38 @@ __device__ __forceinline__ uint32_t corner_index(Raw const (&raw)[N])
     return index;
 }
 
+// One pass of a corner-value wavefront over its unit (see lut_forward_corner_kernel): KIND says what is done with the LUT
+// output of a frame (forward_stage).
+template <int N, int XMODE, int YMODE, int KIND, bool WIDE>
+__device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(&rows)[N], int corner, int node, int lane,
+                                                 int f_begin, int f_end, int f_last, float mean, float rstd, float c0, float &s1, float &s2)
+{
+    constexpr int U = (XMODE == kXBit && !WIDE) ? 2 : 4;  // wavefront-steps whose loads are issued together
+    for (int fb = f_begin; fb < f_end; fb += kWave * U) {
+        typename Gather<N, XMODE>::Raw raw[U][N];
+        float dyv[U];
+        if constexpr (WIDE) { corner_masks_wide<N>(rows, fb, raw); }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
+                if constexpr (!WIDE) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
+                if (KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int const f0 = fb + u * kWave;
+            if (f0 >= f_end) { break; }
+            int const  f  = f0 + lane;
+            bool const ok = f < f_end;
+            uint32_t const index = corner_index<N, XMODE>(raw[u]);
+            float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), corner));
+            forward_stage<YMODE, KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
+                                       (KIND == 3) ? dyv[u] : 0.0f, s1, s2);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 //  Forward for two-valued inputs (packed bits, or fp32 frames binarized at 0.5): the LUT output is one of the 2^N corner
 //  values V of the node.  A lane builds the corner index of its frame from the N input bits (one add-with-carry per input:
@@ -487,40 +521,30 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
                                    : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
     }
     float mean = 0.0f, rstd = 1.0f, c0 = 0.0f;
-    if (FWD_KIND == 2 || (FWD_KIND == 1 && a.stat_mode == kStatPartial)) { c0 = a.C[(size_t)node * NN]; }
+    if (FWD_KIND == 2 || (FWD_KIND == 1 && (a.stat_mode == kStatPartial || a.stat_mode == kStatInline))) { c0 = a.C[(size_t)node * NN]; }
     float var = 0.0f;
-    if (FWD_KIND == 1) { forward_statistics(a, node, lane, c0, mean, var, rstd); }
-    if (FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
 
     int const f_begin = ck * a.chunk;
     int const f_end   = min(f_begin + a.chunk, a.frame_size);
     int const f_last  = a.frame_size - 1;
     float s1 = 0.0f, s2 = 0.0f;
 
-    constexpr int U = (XMODE == kXBit && !WIDE) ? 2 : 4;  // wavefront-steps whose loads are issued together
-    for (int fb = f_begin; fb < f_end; fb += kWave * U) {
-        typename Gather<N, XMODE>::Raw raw[U][N];
-        float dyv[U];
-        if constexpr (WIDE) { corner_masks_wide<N>(rows, fb, raw); }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
-                if constexpr (!WIDE) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
-                if (FWD_KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
-            }
+    if (FWD_KIND == 1) {
+        if (a.stat_mode == kStatInline) {
+            // one unit per node: the sums of the statistics kind, by the same steps in the same order, then what the
+            // statistics launch and the partial-sum read would have delivered (same bits)
+            corner_unit_pass<N, XMODE, YMODE, 2, WIDE>(a, rows, corner, node, lane, f_begin, f_end, f_last, 0.0f, 1.0f, c0, s1, s2);
+            batch_statistics(wave_sum(s1), wave_sum(s2), c0, a.frame_size, mean, var, rstd);
+            mean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mean)));
+            var  = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(var)));
+            rstd = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(rstd)));
+            s1 = 0.0f; s2 = 0.0f;
         }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int const f0 = fb + u * kWave;
-            if (f0 >= f_end) { break; }
-            int const  f  = f0 + lane;
-            bool const ok = f < f_end;
-            uint32_t const index = corner_index<N, XMODE>(raw[u]);
-            float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), corner));
-            forward_stage<YMODE, FWD_KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
-                                           (FWD_KIND == 3) ? dyv[u] : 0.0f, s1, s2);
-        }
+        else { forward_statistics(a, node, lane, c0, mean, var, rstd); }
     }
+    if (FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
+
+    corner_unit_pass<N, XMODE, YMODE, FWD_KIND, WIDE>(a, rows, corner, node, lane, f_begin, f_end, f_last, mean, rstd, c0, s1, s2);
     if (FWD_KIND == 2 || FWD_KIND == 3) { forward_store_stats(a, ck, node, true, lane, s1, s2); }
     if (FWD_KIND == 1) { forward_store_statistics(a, node, true, ck, lane, mean, var, rstd); }
 }
