@@ -441,12 +441,16 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
                                     c.W, C, V, c.node_size, c.lut_binarize, c.bias, st, c.clamp_W, c.clamp_lo, c.clamp_hi)) { return 1; }
         c.x = bits;
     }
-    else {
+    // plain output of a call with one unit per node on the polynomial kernel: the wavefronts prepare their node's table
+    // themselves (FwdArgs::W_inline) and the table launch falls away
+    bool const inline_table = (c.bn == 0) && !corner && chunk_count == 1 && LutMatrixQ<N>::kUsable && c.clamp_W == nullptr;
+    if (!pack && !inline_table) {
         launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias, c.clamp_W, c.clamp_lo, c.clamp_hi);
         BBHIP_LAUNCH_CHECK();
     }
 
     FwdArgs a{};
+    if (inline_table) { a.W_inline = c.W; a.lut_binarize = c.lut_binarize; }
     a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C; a.V = V;
     a.node_size = c.node_size; a.frame_size = c.frame_size;
     a.x_stride = c.x_stride; a.y_stride = c.y_stride;

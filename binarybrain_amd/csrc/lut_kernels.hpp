@@ -199,6 +199,11 @@ struct FwdArgs {
                                 // kStatPartial: from the partial sums that a kind 2 launch of the same shape left in stat_partial
     float momentum;             // kStatPartial: the wavefront of a node's first unit also stores the statistics:
     float *mean_out, *rstd_out, *running_mean, *running_var;
+    // Not null (plain output, one unit per node, widths whose table fits one vector register): no table-preparation launch has
+    // run; the wavefront brings its node's table W' into the centred basis itself — 2^N loads, one per lane, and the
+    // butterfly of table_prep_block over the lanes.  A call of a few hundred frames is two launches' worth of latency, not work.
+    float const *W_inline;
+    int   lut_binarize;
 };
 
 // kStatInline: the call has one unit per node, so the wavefront that writes a node's output first sums the node's statistics
@@ -349,15 +354,28 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         live[p] = (node0 + p < a.node_size);
         node[p] = live[p] ? node0 + p : node0;              // a wavefront past the last node repeats its first one and stores nothing
         mean[p] = 0.0f; rstd[p] = 1.0f; var[p] = 0.0f;
-        c0[p] = a.C[(size_t)node[p] * D::NN];
+        c0[p] = (FWD_KIND == 0) ? 0.0f : a.C[(size_t)node[p] * D::NN];      // (the plain output does not use it)
         if (FWD_KIND == 1) { forward_statistics(a, node[p], lane, c0[p], mean[p], var[p], rstd[p]); }
         if (FWD_KIND == 3) { mean[p] = a.mean[node[p]]; rstd[p] = a.rstd[node[p]]; }
     }
 #pragma unroll
     for (int p = 0; p < NPW; ++p) {
         if constexpr (kMatrix) {
-            mq[p].load(a.C + (size_t)node[p] * D::NN, lane);
-            C[p][0] = a.C[(size_t)node[p] * D::NN];
+            if (FWD_KIND == 0 && a.W_inline != nullptr) {
+                float v = a.W_inline[(size_t)node[p] * D::NN + (lane & (D::NN - 1))];
+                if (a.lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+#pragma unroll
+                for (int j = 0; j < N; ++j) {                 // as table_prep_block: (a, b) -> ((a + b) / 2, b - a) per index bit
+                    float const o = __shfl_xor(v, 1 << j, 64);
+                    v = ((lane >> j) & 1) ? (v - o) : (v + o) * 0.5f;
+                }
+                mq[p].take(v, lane);
+                C[p][0] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+            }
+            else {
+                mq[p].load(a.C + (size_t)node[p] * D::NN, lane);
+                C[p][0] = a.C[(size_t)node[p] * D::NN];
+            }
         }
         else {
             LutEval<N>::load_table(a.C + (size_t)node[p] * D::NN, C[p]);

@@ -239,6 +239,11 @@ struct LutMatrixQ {
     }
 
     __device__ __forceinline__ void load(float const *__restrict__ Cg, int lane) { t = Cg[table_index(lane)]; }
+    // the same from a table held one entry per lane (lane e: entry e)
+    __device__ __forceinline__ void take(float entry_of_lane, int lane)
+    {
+        t = __int_as_float(__builtin_amdgcn_ds_bpermute(table_index(lane) << 2, __float_as_int(entry_of_lane)));
+    }
 
     __device__ __forceinline__ void partial_q(float const (&l)[D::L], float (&q)[D::H]) const
     {
