@@ -23,9 +23,9 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # the same profiler run.  The counter tables and the commands are in profiles/*.md.  A kernel or workload that is not
 # listed reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("lut_dx_kernel<6>", 0):       (651995.4 * 2.0 + 132096.0) * 1024,
-    ("lut_forward_kernel<6>", 0):  (129936.7 * 2.0 + 131072.0) * 1024,
-    ("lut_backward_kernel<6>", 0): (354707.1 * 2.0 + 6372.0) * 1024,
+    ("lut_dx_kernel<6>", 0):       (651415.9 * 2.0 + 132096.0) * 1024,
+    ("lut_forward_kernel<6>", 0):  (128472.4 * 2.0 + 131072.0) * 1024,
+    ("lut_backward_kernel<6>", 0): (352168.3 * 2.0 + 6391.2) * 1024,
     ("binary_lut6_kernel", 0):     (348316.2 * 2.0 + 524288.0) * 1024,
     ("adam_kernel", 0):            (527931.3 * 2.0 + 791860.5) * 1024,
 }
