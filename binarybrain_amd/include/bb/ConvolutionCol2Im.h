@@ -29,9 +29,34 @@ public:
 protected:
     explicit ConvolutionCol2Im(create_t const &create) : m_h_size(create.h_size), m_w_size(create.w_size) {}
 
+    // version 1 | Model part | image height, width | input shape (reference: include/bb/ConvolutionCol2Im.h:334-367)
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        Model::DumpObjectData(os);
+        SaveValue(os, (std::int64_t)m_h_size);
+        SaveValue(os, (std::int64_t)m_w_size);
+        SaveIndices(os, m_input_shape);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = -1, h = 0, w = 0;
+        LoadValue(is, ver);
+        BB_ASSERT(ver == 1);
+        Model::LoadObjectData(is);
+        LoadValue(is, h);
+        LoadValue(is, w);
+        BB_ASSERT(is.good() && h >= 1 && w >= 1);
+        m_h_size = (index_t)h; m_w_size = (index_t)w;
+        m_input_shape = LoadIndices(is);
+        m_c_size = CalcShapeSize(m_input_shape);
+    }
+
 public:
-    static std::string ModelName(void) { return "ConvolutionCol2Im"; }
-    std::string GetModelName(void) const override { return ModelName(); }
+    static std::string ModelName(void)  { return "ConvolutionCol2Im"; }
+    static std::string ObjectName(void) { return ModelName() + "_" + DataType<FT>::Name() + "_" + DataType<BT>::Name(); }
+    std::string GetModelName(void) const override  { return ModelName(); }
+    std::string GetObjectName(void) const override { return ObjectName(); }
 
     static std::shared_ptr<ConvolutionCol2Im> Create(create_t const &create) { return std::shared_ptr<ConvolutionCol2Im>(new ConvolutionCol2Im(create)); }
     static std::shared_ptr<ConvolutionCol2Im> Create(index_t h_size = 1, index_t w_size = 1)

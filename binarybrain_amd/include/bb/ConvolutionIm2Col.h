@@ -68,9 +68,49 @@ protected:
         m_border_value = create.border_value;
     }
 
+    // version 1 | Model part | host_only, frame sizes of the last pass, input c/h/w, filter h/w, strides y/x, padding, border mode
+    // and value (reference: include/bb/ConvolutionIm2Col.h:492-563); the shapes are rebuilt from them
+    void DumpObjectData(std::ostream &os) const override
+    {
+        SaveValue(os, (std::int64_t)1);
+        Model::DumpObjectData(os);
+        SaveValue(os, m_host_only);
+        SaveValue(os, (std::int64_t)m_input_frame_size);  SaveValue(os, (std::int64_t)m_output_frame_size);
+        SaveValue(os, (std::int64_t)m_input_c_size);      SaveValue(os, (std::int64_t)m_input_h_size);  SaveValue(os, (std::int64_t)m_input_w_size);
+        SaveValue(os, (std::int64_t)m_filter_h_size);     SaveValue(os, (std::int64_t)m_filter_w_size);
+        SaveValue(os, (std::int64_t)m_y_stride);          SaveValue(os, (std::int64_t)m_x_stride);
+        SaveValue(os, m_padding);
+        SaveValue(os, (std::int32_t)m_border_mode);
+        SaveValue(os, m_border_value);
+    }
+    void LoadObjectData(std::istream &is) override
+    {
+        std::int64_t ver = -1;
+        LoadValue(is, ver);
+        BB_ASSERT(ver == 1);
+        Model::LoadObjectData(is);
+        auto load_index = [&is](index_t &v) { std::int64_t e = 0; LoadValue(is, e); v = (index_t)e; };
+        LoadValue(is, m_host_only);
+        load_index(m_input_frame_size); load_index(m_output_frame_size);
+        index_t c = 1, h = 1, w = 1;
+        load_index(c); load_index(h); load_index(w);
+        load_index(m_filter_h_size); load_index(m_filter_w_size);
+        load_index(m_y_stride); load_index(m_x_stride);
+        LoadValue(is, m_padding);
+        std::int32_t mode = 0;
+        LoadValue(is, mode);
+        LoadValue(is, m_border_value);
+        BB_ASSERT(is.good() && c >= 1 && h >= 1 && w >= 1 && m_filter_h_size >= 1 && m_filter_w_size >= 1 && m_y_stride >= 1 && m_x_stride >= 1);
+        BB_ASSERT(mode >= BB_BORDER_CONSTANT && mode <= BB_BORDER_WRAP);
+        m_border_mode = (int)mode;
+        SetInputShape(indices_t({c, h, w}));
+    }
+
 public:
-    static std::string ModelName(void) { return "ConvolutionIm2Col"; }
-    std::string GetModelName(void) const override { return ModelName(); }
+    static std::string ModelName(void)  { return "ConvolutionIm2Col"; }
+    static std::string ObjectName(void) { return ModelName() + "_" + DataType<FT>::Name() + "_" + DataType<BT>::Name(); }
+    std::string GetModelName(void) const override  { return ModelName(); }
+    std::string GetObjectName(void) const override { return ObjectName(); }
 
     static std::shared_ptr<ConvolutionIm2Col> Create(create_t const &create) { return std::shared_ptr<ConvolutionIm2Col>(new ConvolutionIm2Col(create)); }
     static std::shared_ptr<ConvolutionIm2Col> Create(index_t filter_h_size, index_t filter_w_size, index_t y_stride = 1, index_t x_stride = 1,

@@ -501,6 +501,29 @@ def ref_wiring6(kind, input_shape, output_shape, seed, policy):
     return (idx, table) if kind == 1 else idx
 
 
+def ref_dump_container_object(kind, c, h, w, fh, fw, ys=1, xs=1, same=False, border_mode="reflect_101", o1=16, o2=8, seed=1, name=""):
+    """Bytes of a container object as the reference writes it.  kind 0: Convolution2d over one DifferentiableLut6 (o2 nodes);
+    1: Convolution2d over a Sequential of two (o1, o2); 2: that Sequential alone; 3: ConvolutionIm2Col; 4: ConvolutionCol2Im
+    (image h x w, o2 channels)."""
+    f = ref().bbref_DumpContainerObject
+    f.restype = C.c_long
+    out = np.zeros(1 << 22, np.uint8)
+    n = f(C.c_int(kind), C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(fh), C.c_int(fw), C.c_int(ys), C.c_int(xs), C.c_int(int(same)),
+          C.c_char_p(border_mode.encode()), C.c_int(o1), C.c_int(o2), C.c_int(seed), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size))
+    assert n > 0, n
+    return out[:n].copy()
+
+
+def ref_reload_container_object(data):
+    """The reference loads the object (rebuilding it from the type names in the stream) and dumps it again; None if it cannot."""
+    data = _c(data, np.uint8)
+    f = ref().bbref_ReloadContainerObject
+    f.restype = C.c_long
+    out = np.zeros(max(1 << 22, 2 * data.size), np.uint8)
+    n = f(_ptr(data), C.c_long(data.size), _ptr(out), C.c_long(out.size))
+    return out[:n].copy() if n > 0 else None
+
+
 def ref_reverse_table6(idx, input_node_size):
     idx = _c(idx, np.int32)
     O = idx.shape[0]

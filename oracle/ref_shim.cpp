@@ -30,6 +30,8 @@
 #include "bb/AverageLut.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
+#include "bb/Convolution2d.h"
+#include "bb/Sequential.h"
 
 namespace {
 
@@ -645,4 +647,59 @@ extern "C" int bbref_LoadLutObject(int kind, int bit, unsigned char const *bytes
     }
     std::snprintf(name, (size_t)name_cap, "%s", m->GetName().c_str());
     return (int)m->GetInputNodeSize();
+}
+
+// ---- container objects: the convolution wrapper around one LUT layer or a list of two, the list alone, Im2Col, Col2Im ----
+// kind 0: Convolution2d over one DifferentiableLut6; 1: Convolution2d over a Sequential of two DifferentiableLut6 layers;
+// 2: that Sequential alone (input shape {c * fh * fw}); 3: ConvolutionIm2Col; 4: ConvolutionCol2Im (after SetInputShape({o2})).
+// The layers are wired and initialised by the reference with the given seed; their contents only have to survive.
+extern "C" long bbref_DumpContainerObject(int kind, int c, int h, int w, int fh, int fw, int ys, int xs, int same, char const *border_mode,
+                                          int o1, int o2, int seed, char const *name, unsigned char *out, long cap)
+{
+    std::string const padding = same ? "same" : "valid";
+    auto make_lut = [&](int o, int s) {
+        typename bb::DifferentiableLutN<6, float, float>::create_t cr;
+        cr.output_shape = {(index_t)o};
+        cr.seed = (std::uint64_t)s;
+        return bb::DifferentiableLutN<6, float, float>::Create(cr);
+    };
+    if (kind == 3) {
+        auto m = bb::ConvolutionIm2Col<float, float>::Create((index_t)fh, (index_t)fw, (index_t)ys, (index_t)xs, padding, border_mode);
+        if (name && *name) { m->SetName(name); }
+        m->SetInputShape({(index_t)c, (index_t)h, (index_t)w});
+        return emit(*m, out, cap);
+    }
+    if (kind == 4) {
+        auto m = bb::ConvolutionCol2Im<float, float>::Create((index_t)h, (index_t)w);
+        if (name && *name) { m->SetName(name); }
+        m->SetInputShape({(index_t)o2});
+        return emit(*m, out, cap);
+    }
+    std::shared_ptr<bb::Model> sub;
+    if (kind == 0) { sub = make_lut(o2, seed); }
+    else {
+        auto seq = bb::Sequential::Create();
+        seq->Add(make_lut(o1, seed));
+        seq->Add(make_lut(o2, seed + 1));
+        if (kind == 2 && name && *name) { seq->SetName(name); }
+        sub = seq;
+    }
+    if (kind == 2) {
+        sub->SetInputShape({(index_t)(c * fh * fw)});
+        return emit(*sub, out, cap);
+    }
+    auto m = bb::Convolution2d<float, float>::Create(sub, (index_t)fh, (index_t)fw, (index_t)ys, (index_t)xs, padding, border_mode);
+    if (name && *name) { m->SetName(name); }
+    m->SetInputShape({(index_t)c, (index_t)h, (index_t)w});
+    return emit(*m, out, cap);
+}
+
+// Loads a container object written elsewhere into the reference's own classes (rebuilt from the type names in the stream) and
+// dumps it again: returns the size of the re-dumped object, negative if the reference could not load it.
+extern "C" long bbref_ReloadContainerObject(unsigned char const *bytes, long size, unsigned char *out, long cap)
+{
+    std::istringstream is(std::string((char const *)bytes, (size_t)size), std::ios::binary);
+    auto obj = bb::Object_Load(is);
+    if (!obj) { return -1; }
+    return emit(*obj, out, cap);
 }

@@ -21,6 +21,7 @@
 #include "bb/StochasticLutN.h"
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
+#include "bb/ObjectLoader.h"
 
 template <typename T>
 static std::vector<T> read_raw(std::string const &path, size_t count)
@@ -197,9 +198,19 @@ static int wiring(int argc, char **argv)
 
 int main(int argc, char **argv)
 {
-    if (argc < 6) { std::fprintf(stderr, "usage: object_tool make|roundtrip|describe|wiring <kind> ...\n"); return 1; }
+    if (argc < 4) { std::fprintf(stderr, "usage: object_tool make|roundtrip|describe|wiring <kind> ... | reload <in> <out>\n"); return 1; }
     bb::Manager::SetHostOnly(true);             // serialization is host work; no device is touched
     std::string const cmd = argv[1];
+    if (cmd == "reload") {
+        // object_tool reload <in> <out>: any object this library knows, rebuilt from the type names in the file, written again
+        auto obj = bb::Object_LoadFromFile(argv[2]);
+        if (!obj) { std::fprintf(stderr, "cannot load %s\n", argv[2]); return 1; }
+        if (auto m = std::dynamic_pointer_cast<bb::Model>(obj)) {
+            std::printf("%s %s in %d out %d\n", m->GetObjectName().c_str(), m->GetName().c_str(), (int)m->GetInputNodeSize(), (int)m->GetOutputNodeSize());
+        }
+        return obj->DumpToFile(argv[3]) ? 0 : 1;
+    }
+    if (argc < 6) { std::fprintf(stderr, "usage: object_tool make|roundtrip|describe|wiring <kind> ...\n"); return 1; }
     if (cmd == "wiring") {
         try { return wiring(argc, argv); }
         catch (std::exception const &e) { std::fprintf(stderr, "rejected: %s\n", e.what()); return 1; }

@@ -4,7 +4,9 @@
 // checker only).  Exit status 0 = all checks passed.
 #include <cmath>
 #include <cstdio>
+#include <cstring>
 #include <random>
+#include <sstream>
 #include <vector>
 
 #include "bb/StochasticLutN.h"
@@ -17,6 +19,8 @@
 #include "bb/AverageLut.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
+#include "bb/Convolution2d.h"
+#include "bb/Sequential.h"
 #include "bb/ObjectLoader.h"
 
 extern "C" {
@@ -314,6 +318,79 @@ static void test_conv_plumbing(void)
     CHECK(bad == 0, "StochasticMaxPooling2x2 backward: %zu wrong", bad);
 }
 
+// The convolution wrapper (reference: include/bb/Convolution2d.h:278-309): Convolution2d over a list of two DifferentiableLut6
+// layers gives, bit for bit, what Im2Col -> layer -> layer -> Col2Im give when called one by one on copies of the same layers
+// (forward, backward down to the image gradient, table gradients); its shapes, parameter list and a trip through a stream.
+static bool same_bits(bb::FrameBuffer &a, bb::FrameBuffer &b)
+{
+    if (a.GetShape() != b.GetShape() || a.GetFrameSize() != b.GetFrameSize()) { return false; }
+    std::vector<float> va, vb;
+    read_fp32(a, va); read_fp32(b, vb);
+    return std::memcmp(va.data(), vb.data(), va.size() * sizeof(float)) == 0;
+}
+
+static void test_convolution2d(void)
+{
+    int const C = 3, H = 8, W = 9, F = 5, O1 = 24, O2 = 8, OH = 6, OW = 7;
+    auto lut1 = bb::DifferentiableLutN<6, float>::Create(O1);
+    auto lut2 = bb::DifferentiableLutN<6, float>::Create(O2);
+    auto body = bb::Sequential::Create();
+    body->Add(lut1); body->Add(lut2);
+    auto conv = bb::Convolution2d<>::Create(body, 3, 3);
+    bb::indices_t const out_shape = conv->SetInputShape({C, H, W});
+    CHECK(out_shape == bb::indices_t({O2, OH, OW}) && conv->GetOutputShape() == out_shape && conv->GetInputShape() == bb::indices_t({C, H, W}),
+          "Convolution2d shapes");
+    CHECK(lut1->GetInputShape() == bb::indices_t({C, 3, 3}) && lut2->GetInputNodeSize() == O1, "Convolution2d hands the shapes through");
+    CHECK(conv->GetParameters().GetSize() == lut1->GetParameters().GetSize() + lut2->GetParameters().GetSize() &&
+          conv->GetGradients().GetSize() == conv->GetParameters().GetSize(), "Convolution2d parameter list");
+
+    // copies of the two layers through their serialized form, and the plumbing by hand
+    auto copy_of = [](std::shared_ptr<bb::Model> const &m) {
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        m->DumpObject(ss);
+        return std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+    };
+    auto lut1b = copy_of(lut1), lut2b = copy_of(lut2);
+    auto im2col = bb::ConvolutionIm2Col<>::Create(3, 3);
+    auto col2im = bb::ConvolutionCol2Im<>::Create(OH, OW);
+
+    std::mt19937_64 mt(77);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    bb::FrameBuffer x(F, {C, H, W}, BB_TYPE_FP32), dy(F, {O2, OH, OW}, BB_TYPE_FP32);
+    for (int n = 0; n < C * H * W; ++n) for (int f = 0; f < F; ++f) { x.SetFP32(f, n, uni(mt)); }
+    for (int n = 0; n < O2 * OH * OW; ++n) for (int f = 0; f < F; ++f) { dy.SetFP32(f, n, uni(mt) - 0.5f); }
+
+    bb::FrameBuffer y = conv->Forward(x);
+    bb::FrameBuffer dx = conv->Backward(dy);
+    bb::FrameBuffer a = im2col->Forward(x);
+    col2im->SetInputShape(lut2b->SetInputShape(lut1b->SetInputShape(a.GetShape())));
+    bb::FrameBuffer y2 = col2im->Forward(lut2b->Forward(lut1b->Forward(a)));
+    bb::FrameBuffer dx2 = im2col->Backward(lut1b->Backward(lut2b->Backward(col2im->Backward(dy))));
+    CHECK(y.GetShape() == out_shape && y.GetFrameSize() == F, "Convolution2d output %d frames", (int)y.GetFrameSize());
+    CHECK(same_bits(y, y2), "Convolution2d forward differs from the layers called one by one");
+    CHECK(same_bits(dx, dx2), "Convolution2d backward differs from the layers called one by one");
+    {
+        auto g = conv->GetGradients(), gb1 = lut1b->GetGradients(), gb2 = lut2b->GetGradients();
+        auto p = g[0].LockConst<float>(); auto q = gb1[0].LockConst<float>();
+        size_t bad = 0;
+        for (bb::index_t i = 0; i < g[0].GetSize(); ++i) { bad += (p[i] != q[i]); }
+        auto p2 = g[g.GetSize() / 2].LockConst<float>(); auto q2 = gb2[0].LockConst<float>();
+        for (bb::index_t i = 0; i < gb2[0].GetSize(); ++i) { bad += (p2[i] != q2[i]); }
+        CHECK(bad == 0, "Convolution2d table gradients: %zu differ", bad);
+    }
+    // through a stream: the rebuilt wrapper (layers rebuilt from their type names) computes the same output
+    {
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        conv->DumpObject(ss);
+        auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)again && again->GetObjectName() == "Convolution2d_fp32_fp32", "Convolution2d reload");
+        if (again) {
+            bb::FrameBuffer y3 = again->Forward(x, false), y4 = conv->Forward(x, false);
+            CHECK(same_bits(y3, y4), "reloaded Convolution2d differs in inference");
+        }
+    }
+}
+
 // The tail of a classifier through the host classes: AverageLut against the oracle, and the reference's own known-answer test
 // of the loss (tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-92, NumPy goldens: loss within 1e-4, dy within 1e-6).
 static void test_tail(void)
@@ -469,6 +546,7 @@ int main(void)
         test_import_layer();
         test_adam();
         test_conv_plumbing();
+        test_convolution2d();
         test_tail();
         test_hand_off_through_files();
     }

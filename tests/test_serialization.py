@@ -138,3 +138,78 @@ def test_damaged_objects_are_rejected(tmp_path):
     assert rejected(bad)
     bad = bytearray(data); bad[at:at + 4] = struct.pack("<i", -1)
     assert rejected(bad)
+
+
+# ----------------------------------------------------------------------------------------------
+#  container objects: Convolution2d (include/bb/Convolution2d.h:355-409), Sequential (Sequential.h:239-288),
+#  ConvolutionIm2Col (:492-563), ConvolutionCol2Im (:334-367)
+# ----------------------------------------------------------------------------------------------
+CONTAINERS = np.load(os.path.join(HERE, "golden", "container_objects.npz"))
+CONTAINER_NAMES = {0: "Convolution2d_fp32_fp32", 1: "Convolution2d_fp32_fp32", 2: "Sequential", 3: "ConvolutionIm2Col_fp32_fp32",
+                   4: "ConvolutionCol2Im_fp32_fp32"}
+
+
+def container_shapes(kind, c, h, w, fh, fw, ys, xs, same, o1, o2):
+    """(input nodes, output nodes) that the loaded object must report"""
+    oh = (h + ys - 1) // ys if same else ((h - fh + 1) + (ys - 1)) // ys
+    ow = (w + xs - 1) // xs if same else ((w - fw + 1) + (xs - 1)) // xs
+    if kind in (0, 1):
+        return c * h * w, o2 * oh * ow
+    if kind == 2:
+        return c * fh * fw, o2
+    if kind == 3:
+        return c * h * w, c * fh * fw
+    return o2, o2 * h * w
+
+
+@pytest.mark.parametrize("k", range(int(CONTAINERS["count"][0])))
+def test_reference_container_objects_load_and_survive_a_round_trip(tmp_path, k):
+    """Bytes written by the reference are rebuilt here from the type names they carry (bb::Object_Load), report the shapes and the
+    name they were made with, and are written again unchanged — the layers inside (wiring, tables, statistics) included."""
+    p = "c%d_" % k
+    kind, c, h, w, fh, fw, ys, xs, same, o1, o2, seed = [int(v) for v in CONTAINERS[p + "args"]]
+    data = CONTAINERS[p + "bytes"].tobytes()
+    name = CONTAINERS[p + "name"].tobytes().decode()
+    src, dst = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    open(src, "wb").write(data)
+    out = tool("reload", src, dst).stdout.split()
+    assert out[0] == CONTAINER_NAMES[kind]
+    # (the convolution wrapper does not store a name of its own; the other objects do)
+    assert out[1] == (name if (name and kind in (2, 3, 4)) else CONTAINER_NAMES[kind].split("_")[0])
+    assert (int(out[3]), int(out[5])) == container_shapes(kind, c, h, w, fh, fw, ys, xs, same, o1, o2)
+    assert open(dst, "rb").read() == data
+
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref is not built")
+def test_container_objects_against_the_reference(tmp_path):
+    """Fresh objects from the reference (new geometry and seeds each): loaded and re-written here they keep their bytes, and the
+    reference loads what was written here — rebuilding it from the type names — and writes the same bytes again."""
+    rng = np.random.default_rng(2718)
+    borders = ["constant", "reflect", "reflect_101", "replicate", "wrap"]
+    for trial in range(12):
+        kind = trial % 5
+        c, fh, fw = int(rng.integers(1, 5)), int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        h, w = int(rng.integers(fh + 1, 12)), int(rng.integers(fw + 1, 12))
+        ys, xs, same = int(rng.integers(1, 3)), int(rng.integers(1, 3)), bool(rng.integers(0, 2))
+        o1, o2, seed = int(rng.integers(6, 40)), int(rng.integers(1, 20)), int(rng.integers(1, 1000))
+        data = oracle.ref_dump_container_object(kind, c, h, w, fh, fw, ys, xs, same, borders[trial % 5], o1, o2, seed, "n%d" % trial)
+        src, dst = str(tmp_path / ("in%d.bin" % trial)), str(tmp_path / ("out%d.bin" % trial))
+        open(src, "wb").write(data.tobytes())
+        tool("reload", src, dst)
+        mine = np.frombuffer(open(dst, "rb").read(), np.uint8)
+        assert np.array_equal(mine, data), (trial, kind)
+        back = oracle.ref_reload_container_object(mine)
+        assert back is not None and np.array_equal(back, data), (trial, kind)
+
+
+def test_damaged_container_objects_are_rejected(tmp_path):
+    data = bytearray(CONTAINERS["c2_bytes"].tobytes())          # a convolution over a list of two layers
+    for cut in (20, len(data) // 2, len(data) - 3):
+        p = str(tmp_path / ("cut%d.bin" % cut))
+        open(p, "wb").write(bytes(data[:cut]))
+        assert tool("reload", p, str(tmp_path / "x.bin"), check=False).returncode != 0
+    # a layer type that is not known here inside a known container
+    bad = bytes(data).replace(b"DifferentiableLut6_fp32_fp32", b"DifferentiableLut9_fp32_fp32")
+    p = str(tmp_path / "unknown.bin")
+    open(p, "wb").write(bad)
+    assert tool("reload", p, str(tmp_path / "x.bin"), check=False).returncode != 0
