@@ -188,6 +188,46 @@ def bench_conv(args, lib):
     return out
 
 
+def bench_stochastic_bn(args, lib):
+    """StochasticBatchNormalization (secondary measurement) at the size of a hidden layer of the headline configuration, 8192 nodes
+    x 4096 frames, and at the normalisation after a convolution, 32 channels x 50176 frames (few long rows: one workgroup per
+    row).  Algorithmic bytes: every element of each input and output once (training and inference 8 B, backward 12 B per element)."""
+    import torch
+    from binarybrain_amd import ops, synth
+    kernels = {}
+    totals = {}
+    for (nodes, F) in ((8192, 4096), (32, 50176)):
+        g = torch.Generator(device="cuda"); g.manual_seed(0)
+        S = synth.frame_stride_fp32(F)
+        x = torch.rand((nodes, S), device="cuda", generator=g)
+        dy = torch.randn((nodes, S), device="cuda", generator=g)
+        rm = torch.zeros(nodes, device="cuda"); rv = torch.ones(nodes, device="cuda")
+        _, mean, rstd = ops.stochastic_bn_forward_training(x, rm, rv, F)
+        e = 4 * nodes * F
+        cases = [
+            ("bn_forward_training_kernel", lambda: ops.stochastic_bn_forward_training(x, rm, rv, F), 2 * e),
+            ("bn_backward_kernel", lambda: ops.stochastic_bn_backward(x, dy, mean, rstd, F), 3 * e),
+            ("bn_apply_kernel (inference)", lambda: ops.stochastic_bn_forward_inference(x, rm, rv, F), 2 * e),
+        ]
+        total_ms = 0.0
+        for name, fn, nbytes in cases:
+            med = library_timed_ms(lib, fn, args.steps, args.warmup)
+            total_ms += med
+            kernels["%s %dx%d" % (name, nodes, F)] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
+        totals[(nodes, F)] = total_ms
+    big = {k: v for k, v in kernels.items() if k.endswith("8192x4096")}
+    dom = max(big, key=lambda k: big[k]["ms"])
+    ms = totals[(8192, 4096)]
+    out = {"metric": "StochasticBatchNormalization training fwd + bwd + inference, ms per pass over 8192 nodes x 4096 frames", "value": ms,
+           "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "StochasticBatchNormalization fp32, 8192 nodes x 4096 frames", "ms_at_32x50176": totals[(32, 50176)]},
+           "roofline": {"bound": "hbm", "kernel": dom, "achieved": big[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": big[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},
+           "kernels": kernels}
+    return out
+
+
 def bench_tail(args, lib):
     """The tail of the MNIST-like classifier (secondary measurement): AverageLut 7 -> 1 over 70 -> 10 nodes, softmax cross
     entropy and categorical accuracy over the 10 classes.  Measured at 65536 frames (streaming rate) and at the
@@ -791,7 +831,7 @@ def main():
                     help="headline workload only: skip the other BASELINE configurations that the default run reports under `configs`")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail",
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail", "stochastic_bn",
                              "forward_784x1024x64", "gather_ceiling"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
@@ -807,7 +847,7 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     lib = capi.lib()
-    secondary = {"binarylut6": bench_binarylut6, "adam": bench_adam, "conv": bench_conv, "tail": bench_tail,
+    secondary = {"binarylut6": bench_binarylut6, "adam": bench_adam, "conv": bench_conv, "tail": bench_tail, "stochastic_bn": bench_stochastic_bn,
                  "differentiablelut6": bench_differentiablelut6, "differentiablelut6_bit": bench_differentiablelut6,
                  "mnist_step": bench_mnist_step, "conv_block": bench_conv_block, "forward_784x1024x64": bench_forward_small,
                  "gather_ceiling": bench_gather_ceiling}

@@ -66,6 +66,10 @@ _SIGNATURES = {
     "bbhip_fp32_AverageLut_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 5 + [_vp]),
     "bbhip_fp32_LossSoftmaxCrossEntropy": (C.c_int, [_vp, _vp, _vp, _vp, _f] + [_i] * 4 + [_vp]),
     "bbhip_fp32_MetricsCategoricalAccuracy": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 4 + [_vp]),
+    "bbhip_fp32_StochasticBatchNormalization_ForwardTraining": (C.c_int, [_vp] * 6 + [_f, _f, _f, _i, _i, _i, _vp]),
+    "bbhip_fp32_StochasticBatchNormalization_ReForward": (C.c_int, [_vp] * 4 + [_f, _f, _i, _i, _i, _vp]),
+    "bbhip_fp32_StochasticBatchNormalization_ForwardInference": (C.c_int, [_vp] * 4 + [_f, _f, _i, _i, _i, _vp]),
+    "bbhip_fp32_StochasticBatchNormalization_Backward": (C.c_int, [_vp] * 5 + [_f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "bbhip_fp32_StochasticLut_Forward_NoAlloc": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),

@@ -17,6 +17,7 @@
 #include "vector_kernels.hpp"
 #include "conv_kernels.hpp"
 #include "tail_kernels.hpp"
+#include "bn_kernels.hpp"
 
 using namespace bbhip;
 
@@ -1424,6 +1425,122 @@ int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *d
                        frame_stride);
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+
+// ---- StochasticBatchNormalization ----
+// 128-bit accesses need rows that start on 16 bytes: both bases aligned and both strides a multiple of four floats
+static bool bn_rows_aligned(void const *p0, void const *p1, void const *p2, int stride0, int stride1)
+{
+    uintptr_t const bits = reinterpret_cast<uintptr_t>(p0) | reinterpret_cast<uintptr_t>(p1) | reinterpret_cast<uintptr_t>(p2);
+    return (bits & 15u) == 0 && (stride0 & 3) == 0 && (stride1 & 3) == 0;
+}
+
+static int check_bn(void const *x, void const *out, int node_size, int frame_size, int x_stride, int out_stride, char const *name)
+{
+    if (!(x && out)) { return fail("%s: null buffer", name); }
+    if (!(node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (x_stride < frame_size || out_stride < frame_size) { return fail("%s: frame stride shorter than the frames", name); }
+    return 0;
+}
+
+static int launch_bn_rows(BnArgs const &a, int node_size, bool backward, void *stream)
+{
+    bool const wide = bn_rows_aligned(a.x, backward ? a.dy : a.out, a.out, a.x_stride, a.out_stride);
+    bool const held = a.frame_size <= kBnBlock * kBnHeld * (wide ? 4 : 1);
+    dim3 const grid((unsigned)node_size), block(held ? kBnBlock : kBnLongBlock);
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+#define BBHIP_BN_ROWS(W, HELD)                                                                                  \
+    do {                                                                                                        \
+        if (backward) { hipLaunchKernelGGL((bn_backward_kernel<W, HELD>), grid, block, 0, st, a); }             \
+        else          { hipLaunchKernelGGL((bn_forward_training_kernel<W, HELD>), grid, block, 0, st, a); }     \
+    } while (0)
+    if (wide) { if (held) { BBHIP_BN_ROWS(4, true); } else { BBHIP_BN_ROWS(4, false); } }
+    else      { if (held) { BBHIP_BN_ROWS(1, true); } else { BBHIP_BN_ROWS(1, false); } }
+#undef BBHIP_BN_ROWS
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int launch_bn_apply(BnArgs const &a, int node_size, bool from_running, void *stream, char const *name)
+{
+    bool const wide = bn_rows_aligned(a.x, a.out, a.out, a.x_stride, a.out_stride);
+    int const f_blocks = ceil_div(a.frame_size, kBnBlock * (wide ? 4 : 1));
+    long long const blocks = (long long)node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    dim3 const grid((unsigned)blocks), block(kBnBlock);
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    if (wide) {
+        if (from_running) { hipLaunchKernelGGL((bn_apply_kernel<4, true>), grid, block, 0, st, a, f_blocks); }
+        else              { hipLaunchKernelGGL((bn_apply_kernel<4, false>), grid, block, 0, st, a, f_blocks); }
+    }
+    else {
+        if (from_running) { hipLaunchKernelGGL((bn_apply_kernel<1, true>), grid, block, 0, st, a, f_blocks); }
+        else              { hipLaunchKernelGGL((bn_apply_kernel<1, false>), grid, block, 0, st, a, f_blocks); }
+    }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_StochasticBatchNormalization_ForwardTraining(float const *dev_x_buf, float *dev_y_buf, float *dev_mean_buf, float *dev_rstd_buf,
+                                                            float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta,
+                                                            float momentum, int node_size, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_bn(dev_x_buf, dev_y_buf, node_size, frame_size, frame_stride, frame_stride, __func__)) { return 1; }
+    BBHIP_REQUIRE(dev_mean_buf != nullptr && dev_rstd_buf != nullptr && dev_running_mean_buf != nullptr && dev_running_var_buf != nullptr);
+    BnArgs a{};
+    a.x = dev_x_buf; a.out = dev_y_buf; a.mean = dev_mean_buf; a.rstd = dev_rstd_buf;
+    a.running_mean = dev_running_mean_buf; a.running_var = dev_running_var_buf;
+    a.gamma = gamma; a.beta = beta; a.momentum = momentum;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    return launch_bn_rows(a, node_size, false, stream);
+}
+
+int bbhip_fp32_StochasticBatchNormalization_ReForward(float const *dev_x_buf, float *dev_y_buf, float const *dev_mean_buf,
+                                                      float const *dev_rstd_buf, float gamma, float beta, int node_size, int frame_size,
+                                                      int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_bn(dev_x_buf, dev_y_buf, node_size, frame_size, frame_stride, frame_stride, __func__)) { return 1; }
+    BBHIP_REQUIRE(dev_mean_buf != nullptr && dev_rstd_buf != nullptr);
+    BnArgs a{};
+    a.x = dev_x_buf; a.out = dev_y_buf; a.mean = const_cast<float *>(dev_mean_buf); a.rstd = const_cast<float *>(dev_rstd_buf);
+    a.gamma = gamma; a.beta = beta;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    return launch_bn_apply(a, node_size, false, stream, __func__);
+}
+
+int bbhip_fp32_StochasticBatchNormalization_ForwardInference(float const *dev_x_buf, float *dev_y_buf, float const *dev_running_mean_buf,
+                                                             float const *dev_running_var_buf, float gamma, float beta, int node_size,
+                                                             int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_bn(dev_x_buf, dev_y_buf, node_size, frame_size, frame_stride, frame_stride, __func__)) { return 1; }
+    BBHIP_REQUIRE(dev_running_mean_buf != nullptr && dev_running_var_buf != nullptr);
+    BnArgs a{};
+    a.x = dev_x_buf; a.out = dev_y_buf;
+    a.running_mean = const_cast<float *>(dev_running_mean_buf); a.running_var = const_cast<float *>(dev_running_var_buf);
+    a.gamma = gamma; a.beta = beta;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    return launch_bn_apply(a, node_size, true, stream, __func__);
+}
+
+int bbhip_fp32_StochasticBatchNormalization_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+                                                     float const *dev_mean_buf, float const *dev_rstd_buf, float gamma,
+                                                     float reciprocal_frame_size, int node_size, int frame_size, int frame_stride,
+                                                     int x_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_bn(dev_x_buf, dev_dx_buf, node_size, frame_size, x_frame_stride, frame_stride, __func__)) { return 1; }
+    BBHIP_REQUIRE(dev_dy_buf != nullptr && dev_mean_buf != nullptr && dev_rstd_buf != nullptr);
+    BnArgs a{};
+    a.x = dev_x_buf; a.dy = dev_dy_buf; a.out = dev_dx_buf;
+    a.mean = const_cast<float *>(dev_mean_buf); a.rstd = const_cast<float *>(dev_rstd_buf);
+    a.gamma = gamma; a.reciprocal_frame_size = reciprocal_frame_size;
+    a.frame_size = frame_size; a.x_stride = x_frame_stride; a.out_stride = frame_stride;
+    return launch_bn_rows(a, node_size, true, stream);
 }
 
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,

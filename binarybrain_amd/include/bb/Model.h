@@ -78,6 +78,9 @@ public:
 
     virtual FrameBuffer Forward(FrameBuffer x_buf, bool train = true) = 0;
     virtual FrameBuffer Backward(FrameBuffer dy_buf) = 0;
+    // the training pass again on the same batch, with whatever the first pass fixed (batch statistics) kept
+    // (reference: include/bb/Model.h:312-315)
+    virtual FrameBuffer ReForward(FrameBuffer x_buf) { return Forward(x_buf, true); }
 
     // value of one output node for one vector of input values (used to tabulate a trained layer)
     virtual std::vector<double> ForwardNode(index_t, std::vector<double> input_value) const { return input_value; }

@@ -199,6 +199,44 @@ def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
     return dx
 
 
+def stochastic_bn_forward_training(x, running_mean, running_var, frame_size, gamma=0.2, beta=0.5, momentum=0.9):
+    """Per-node batch normalisation with scalar gamma / beta, training pass: x [nodes, stride] -> (y, mean, rstd); the running
+    statistics are updated in place."""
+    _dev(x, running_mean, running_var)
+    nodes = x.shape[0]
+    y = torch.empty_like(x)
+    mean = torch.empty(nodes, dtype=torch.float32, device=x.device)
+    rstd = torch.empty(nodes, dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_StochasticBatchNormalization_ForwardTraining(ptr(x), ptr(y), ptr(mean), ptr(rstd), ptr(running_mean),
+                                                                        ptr(running_var), gamma, beta, momentum, nodes, frame_size,
+                                                                        x.shape[1], stream_ptr()))
+    return y, mean, rstd
+
+
+def stochastic_bn_reforward(x, mean, rstd, frame_size, gamma=0.2, beta=0.5):
+    _dev(x, mean, rstd)
+    y = torch.empty_like(x)
+    check(lib().bbhip_fp32_StochasticBatchNormalization_ReForward(ptr(x), ptr(y), ptr(mean), ptr(rstd), gamma, beta, x.shape[0], frame_size,
+                                                                  x.shape[1], stream_ptr()))
+    return y
+
+
+def stochastic_bn_forward_inference(x, running_mean, running_var, frame_size, gamma=0.2, beta=0.5):
+    _dev(x, running_mean, running_var)
+    y = torch.empty_like(x)
+    check(lib().bbhip_fp32_StochasticBatchNormalization_ForwardInference(ptr(x), ptr(y), ptr(running_mean), ptr(running_var), gamma, beta,
+                                                                         x.shape[0], frame_size, x.shape[1], stream_ptr()))
+    return y
+
+
+def stochastic_bn_backward(x, dy, mean, rstd, frame_size, gamma=0.2):
+    _dev(x, dy, mean, rstd)
+    dx = torch.empty_like(dy)
+    check(lib().bbhip_fp32_StochasticBatchNormalization_Backward(ptr(x), ptr(dy), ptr(dx), ptr(mean), ptr(rstd), gamma, 1.0 / frame_size,
+                                                                 dy.shape[0], frame_size, dy.shape[1], x.shape[1], stream_ptr()))
+    return dx
+
+
 def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
     """fp32 x [I, stride] -> y [O, stride]: sum of the n wired inputs (their votes when binarize_input), or its sign."""
     _dev(x, idx)

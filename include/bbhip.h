@@ -241,6 +241,32 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
 int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *dev_t_buf, int *dev_accuracy_buf, int *dev_category_buf,
                                           int pix_size, int ch_size, int frame_size, int frame_stride, void *stream);
 
+/* ---- StochasticBatchNormalization ----
+ * Per node (a row of frames): mean and biased variance of the batch, rstd = 1 / (sqrt(var) + 1e-7),
+ * y = ((x - mean) * rstd) * gamma + beta with one scalar gamma and beta for the layer
+ * (include/bb/StochasticBatchNormalization.h:535-597).  Sums are taken in a fixed tree order: results are the same on every
+ * run and agree with the reference's frame-order sums to rounding. */
+/* bbcu_fp32_StochasticBatchNormalization_ForwardTraining, include/bbcu/bbcu.h:883-898: also writes the batch statistics and
+ * updates running = running * momentum + batch * (1 - momentum) */
+int bbhip_fp32_StochasticBatchNormalization_ForwardTraining(float const *dev_x_buf, float *dev_y_buf, float *dev_mean_buf, float *dev_rstd_buf,
+                                                            float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta,
+                                                            float momentum, int node_size, int frame_size, int frame_stride, void *stream);
+/* bbcu_fp32_StochasticBatchNormalization_ReForward, include/bbcu/bbcu.h:900-912: the output again from stored batch statistics */
+int bbhip_fp32_StochasticBatchNormalization_ReForward(float const *dev_x_buf, float *dev_y_buf, float const *dev_mean_buf,
+                                                      float const *dev_rstd_buf, float gamma, float beta, int node_size, int frame_size,
+                                                      int frame_stride, void *stream);
+/* bbcu_fp32_StochasticBatchNormalization_ForwardInference, include/bbcu/bbcu.h:914-926: mean = running mean,
+ * rstd = 1 / (sqrt(running var) + 1e-7) */
+int bbhip_fp32_StochasticBatchNormalization_ForwardInference(float const *dev_x_buf, float *dev_y_buf, float const *dev_running_mean_buf,
+                                                             float const *dev_running_var_buf, float gamma, float beta, int node_size,
+                                                             int frame_size, int frame_stride, void *stream);
+/* bbcu_fp32_StochasticBatchNormalization_Backward, include/bbcu/bbcu.h:928-942 (host loop: StochasticBatchNormalization.h:815-851);
+ * dev_x_buf rows are x_frame_stride apart, dy and dx rows frame_stride */
+int bbhip_fp32_StochasticBatchNormalization_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+                                                     float const *dev_mean_buf, float const *dev_rstd_buf, float gamma,
+                                                     float reciprocal_frame_size, int node_size, int frame_size, int frame_stride,
+                                                     int x_frame_stride, void *stream);
+
 /* ---- StochasticLut ---- */
 /* bbcu_fp32_StochasticLut_Forward<N>, include/bbcu/bbcu.h:667-681 */
 int bbhip_fp32_StochasticLut_Forward(int n, float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index,

@@ -187,6 +187,45 @@ def stochastic_maxpool2x2_backward(x, dy, c, h, w, frames):
     return dx
 
 
+def stochastic_bn_forward_training(x, running_mean, running_var, gamma, beta, momentum, frame_size):
+    """Per-node batch normalisation with scalar gamma / beta, training pass (the reference's generic host loop,
+    include/bb/StochasticBatchNormalization.h:535-597) -> (y, mean, rstd, running_mean', running_var')."""
+    x = _c(x, np.float32)
+    y = np.zeros_like(x)
+    nodes = x.shape[0]
+    mean = np.zeros(nodes, np.float32); rstd = np.zeros(nodes, np.float32)
+    rm = _c(running_mean, np.float32).copy(); rv = _c(running_var, np.float32).copy()
+    lib().oracle_fp32_StochasticBatchNormalization_ForwardTraining(_ptr(x), _ptr(y), _ptr(mean), _ptr(rstd), _ptr(rm), _ptr(rv),
+                                                                   C.c_float(gamma), C.c_float(beta), C.c_float(momentum), C.c_int(nodes),
+                                                                   C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y, mean, rstd, rm, rv
+
+
+def stochastic_bn_reforward(x, mean, rstd, gamma, beta, frame_size):
+    x = _c(x, np.float32); mean = _c(mean, np.float32); rstd = _c(rstd, np.float32)
+    y = np.zeros_like(x)
+    lib().oracle_fp32_StochasticBatchNormalization_ReForward(_ptr(x), _ptr(y), _ptr(mean), _ptr(rstd), C.c_float(gamma), C.c_float(beta),
+                                                             C.c_int(x.shape[0]), C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y
+
+
+def stochastic_bn_forward_inference(x, running_mean, running_var, gamma, beta, frame_size):
+    x = _c(x, np.float32); rm = _c(running_mean, np.float32); rv = _c(running_var, np.float32)
+    y = np.zeros_like(x)
+    lib().oracle_fp32_StochasticBatchNormalization_ForwardInference(_ptr(x), _ptr(y), _ptr(rm), _ptr(rv), C.c_float(gamma), C.c_float(beta),
+                                                                    C.c_int(x.shape[0]), C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y
+
+
+def stochastic_bn_backward(x, dy, mean, rstd, gamma, frame_size):
+    x = _c(x, np.float32); dy = _c(dy, np.float32); mean = _c(mean, np.float32); rstd = _c(rstd, np.float32)
+    dx = np.zeros_like(dy)
+    lib().oracle_fp32_StochasticBatchNormalization_Backward(_ptr(x), _ptr(dy), _ptr(dx), _ptr(mean), _ptr(rstd), C.c_float(gamma),
+                                                            C.c_int(dy.shape[0]), C.c_int(frame_size), C.c_int(dy.shape[1]),
+                                                            C.c_int(x.shape[1]))
+    return dx
+
+
 def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True, mean=False):
     """fp32 x [I, stride] -> y [O, stride]: sum (or its sign) of the n wired inputs, the reference's host loop
     (include/bb/AverageLut.h:331-343).  mean: the convention of the reference's CUDA kernel instead, which writes an
@@ -522,6 +561,27 @@ def ref_reload_container_object(data):
     out = np.zeros(max(1 << 22, 2 * data.size), np.uint8)
     n = f(_ptr(data), C.c_long(data.size), _ptr(out), C.c_long(out.size))
     return out[:n].copy() if n > 0 else None
+
+
+def ref_stochastic_bn(x, running_mean, running_var, gamma, beta, momentum, train=True, dy=None, name="", want_object=False):
+    """The reference's StochasticBatchNormalization<float> (generic host path) on dense [nodes, frames] arrays ->
+    dict(y, mean, rstd, running_mean, running_var, dx, object)."""
+    x = _c(x, np.float32)
+    nodes, frames = x.shape
+    y = np.zeros_like(x)
+    rm = _c(running_mean, np.float32).copy(); rv = _c(running_var, np.float32).copy()
+    mean = np.zeros(nodes, np.float32); rstd = np.zeros(nodes, np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros_like(x)
+    out = np.zeros((1 << 16) + 16 * nodes, np.uint8) if want_object else None
+    f = ref().bbref_StochasticBatchNormalization
+    f.restype = C.c_long
+    n = f(C.c_int(nodes), C.c_int(frames), C.c_float(momentum), C.c_float(gamma), C.c_float(beta), C.c_int(int(train)), _ptr(x), _ptr(rm),
+          _ptr(rv), _ptr(y), _ptr(mean), _ptr(rstd), _ptr(dy), _ptr(dx), C.c_char_p(name.encode()), _ptr(out),
+          C.c_long(out.size if want_object else 0))
+    assert n >= 0, n
+    return dict(y=y, mean=mean, rstd=rstd, running_mean=rm, running_var=rv, dx=dx, object=out[:n].copy() if want_object else None)
 
 
 def ref_reverse_table6(idx, input_node_size):

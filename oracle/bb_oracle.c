@@ -1041,3 +1041,95 @@ void oracle_fp32_MetricsCategoricalAccuracy(float const *y, float const *t, int 
         category_buf[f] = category;
     }
 }
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ *  StochasticBatchNormalization: per-node batch normalisation with scalar gamma / beta, the unfused twin of the
+ *  normalisation inside DifferentiableLutN (reference host path, include/bb/StochasticBatchNormalization.h: training forward
+ *  :535-597, re-forward :655-678, backward :815-851).  fp32 sums in frame order, as the reference's generic loops.
+ *  Pinned by tests/test_oracle_bn.py: the reference's own class where oracle/_ref is built, tests/golden/bn.npz elsewhere,
+ *  textbook mean / variance in fp64, the invariants sum_f dx = 0 and sum_f dx (x - mean) = 0.
+ *  Inference: y = ((x - running_mean) * rstd) * gamma + beta with rstd = 1 / (sqrt(running_var) + 1e-7), the form of the
+ *  reference's re-forward, its ForwardNode (:319-341) and its CUDA kernel.  The reference's generic host inference (:599-616)
+ *  folds the same into gain * x + offset but takes the mean of the LAST TRAINING BATCH for the offset where every other path
+ *  takes the running mean; that is not reproduced.
+ * ------------------------------------------------------------------------------------------------------------------- */
+void oracle_fp32_StochasticBatchNormalization_ForwardTraining(float const *x, float *y, float *mean_buf, float *rstd_buf,
+                                                              float *running_mean, float *running_var, float gamma, float beta,
+                                                              float momentum, int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        float const *xr = x + (size_t)node * frame_stride;
+        float *yr = y + (size_t)node * frame_stride;
+        float mean = 0.0f;
+        for (int f = 0; f < frame_size; ++f) { mean += xr[f]; }
+        mean /= (float)frame_size;
+        float var = 0.0f;
+        for (int f = 0; f < frame_size; ++f) { float const xc = xr[f] - mean; var += xc * xc; }
+        var /= (float)frame_size;
+        var = fmaxf(0.0f, var);
+        float const rstd = 1.0f / (sqrtf(var) + 1.0e-7f);
+        running_mean[node] = running_mean[node] * momentum + mean * (1.0f - momentum);
+        running_var[node]  = running_var[node]  * momentum + var  * (1.0f - momentum);
+        mean_buf[node] = mean;
+        rstd_buf[node] = rstd;
+        for (int f = 0; f < frame_size; ++f) {
+            float v = (xr[f] - mean) * rstd;
+            yr[f] = v * gamma + beta;
+        }
+    }
+}
+
+/* re-forward with stored statistics (:655-678) */
+void oracle_fp32_StochasticBatchNormalization_ReForward(float const *x, float *y, float const *mean_buf, float const *rstd_buf,
+                                                        float gamma, float beta, int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        float const mean = mean_buf[node], rstd = rstd_buf[node];
+        for (int f = 0; f < frame_size; ++f) {
+            float v = (x[(size_t)node * frame_stride + f] - mean) * rstd;
+            y[(size_t)node * frame_stride + f] = v * gamma + beta;
+        }
+    }
+}
+
+void oracle_fp32_StochasticBatchNormalization_ForwardInference(float const *x, float *y, float const *running_mean,
+                                                               float const *running_var, float gamma, float beta,
+                                                               int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        float const mean = running_mean[node];
+        float const rstd = 1.0f / (sqrtf(running_var[node]) + 1.0e-7f);
+        for (int f = 0; f < frame_size; ++f) {
+            float v = (x[(size_t)node * frame_stride + f] - mean) * rstd;
+            y[(size_t)node * frame_stride + f] = v * gamma + beta;
+        }
+    }
+}
+
+/* backward (:815-851): dstd = -sum dxn xc rstd^2, dmeanx = -sum dxn rstd with dxn = gamma dy;
+ * dvar = dstd rstd; dmean = (dmeanx - mean dvar) / F; dx = dxn rstd + dmean + x dvar / F */
+void oracle_fp32_StochasticBatchNormalization_Backward(float const *x, float const *dy, float *dx, float const *mean_buf,
+                                                       float const *rstd_buf, float gamma, int node_size, int frame_size,
+                                                       int frame_stride, int x_frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        float const *xr = x + (size_t)node * x_frame_stride;
+        float const *dyr = dy + (size_t)node * frame_stride;
+        float *dxr = dx + (size_t)node * frame_stride;
+        float const mean = mean_buf[node], rstd = rstd_buf[node];
+        float dmeanx = 0.0f, dstd = 0.0f;
+        for (int f = 0; f < frame_size; ++f) {
+            float const xc = xr[f] - mean;
+            float const dxn = gamma * dyr[f];
+            dstd   += -(dxn * xc * (rstd * rstd));
+            dmeanx += -(dxn * rstd);
+        }
+        float const dvar  = dstd * rstd;
+        float const dmean = (dmeanx - (mean * dvar)) / (float)frame_size;
+        for (int f = 0; f < frame_size; ++f) {
+            float const dxn = dyr[f] * gamma;
+            float const dxc = dxn * rstd;
+            dxr[f] = dxc + dmean + (xr[f] * dvar / (float)frame_size);
+        }
+    }
+}

@@ -32,6 +32,7 @@
 #include "bb/MetricsCategoricalAccuracy.h"
 #include "bb/Convolution2d.h"
 #include "bb/Sequential.h"
+#include "bb/StochasticBatchNormalization.h"
 
 namespace {
 
@@ -702,4 +703,46 @@ extern "C" long bbref_ReloadContainerObject(unsigned char const *bytes, long siz
     auto obj = bb::Object_Load(is);
     if (!obj) { return -1; }
     return emit(*obj, out, cap);
+}
+
+// StochasticBatchNormalization<float> (generic host path: host_only, no SIMD).  x, y, dy, dx: [nodes][frames].
+// The running statistics start at running_mean / running_var (in) and come back updated; mean / rstd are the batch statistics
+// kept for the backward pass.  train == 0 runs the inference formula; it takes its offset from the batch mean of the last
+// training pass, so a caller that wants the running mean there runs one training pass with momentum 0 on the same batch first.
+// object_out (may be null) receives the layer dumped after the passes; returns its size (0 without object_out), negative on error.
+extern "C" long bbref_StochasticBatchNormalization(int nodes, int frames, float momentum, float gamma, float beta, int train,
+                                                   float const *x, float *running_mean, float *running_var, float *y, float *mean,
+                                                   float *rstd, float const *dy, float *dx, char const *name,
+                                                   unsigned char *object_out, long cap)
+{
+    auto m = bb::StochasticBatchNormalization<float>::Create(momentum, gamma, beta);
+    m->SendCommand("host_only true");
+    if (name && *name) { m->SetName(name); }
+    m->SetInputShape({(index_t)nodes});
+    {
+        auto rm = m->lock_mean();
+        auto rv = m->lock_var();
+        for (int n = 0; n < nodes; ++n) { rm[n] = running_mean[n]; rv[n] = running_var[n]; }
+    }
+    bb::FrameBuffer xb((index_t)frames, bb::indices_t({(index_t)nodes}), BB_TYPE_FP32, true);
+    put_fp32(xb, x, nodes, frames);
+    bb::FrameBuffer yb = m->Forward(xb, train != 0);
+    get_fp32(yb, y, nodes, frames);
+    {
+        auto rm = m->lock_mean_const();
+        auto rv = m->lock_var_const();
+        for (int n = 0; n < nodes; ++n) { running_mean[n] = rm[n]; running_var[n] = rv[n]; }
+    }
+    if (train) {
+        auto bm = m->lock_tmp_mean_const();
+        auto br = m->lock_tmp_rstd_const();
+        for (int n = 0; n < nodes; ++n) { mean[n] = bm[n]; rstd[n] = br[n]; }
+    }
+    if (train && dy) {
+        bb::FrameBuffer dyb((index_t)frames, bb::indices_t({(index_t)nodes}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, nodes, frames);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, nodes, frames);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
 }

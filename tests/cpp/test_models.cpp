@@ -21,6 +21,7 @@
 #include "bb/MetricsCategoricalAccuracy.h"
 #include "bb/Convolution2d.h"
 #include "bb/Sequential.h"
+#include "bb/StochasticBatchNormalization.h"
 #include "bb/ObjectLoader.h"
 
 extern "C" {
@@ -36,6 +37,9 @@ void oracle_fp32_StochasticLut_Forward(int n, float const *x, float *y, std::int
 void oracle_fp32_StochasticLut_Backward(int n, float const *x, float const *dy, float *dx, std::int32_t const *idx, float const *W, float *dW, int input_node_size, int output_node_size, int frame_size, int frame_stride, int input_binary, int lut_binarize, float bias, int simd);
 void oracle_fp32_DifferentiableLutN_ForwardTraining(int n, float const *x, float *y, std::int32_t const *idx, float const *W, float *mean, float *rstd, float *running_mean, float *running_var, float gamma, float beta, float momentum, float bias, int node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode);
 void oracle_fp32_DifferentiableLutN_Backward(int n, float const *x, float const *dy, float *dx, std::int32_t const *idx, float const *W, float *dW, float const *mean, float const *rstd, float gamma, float beta, float bias, int input_node_size, int output_node_size, int frame_size, int frame_stride, int lut_binarize, int binary_mode);
+void oracle_fp32_StochasticBatchNormalization_ForwardTraining(float const *x, float *y, float *mean, float *rstd, float *running_mean, float *running_var, float gamma, float beta, float momentum, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_StochasticBatchNormalization_ForwardInference(float const *x, float *y, float const *running_mean, float const *running_var, float gamma, float beta, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_StochasticBatchNormalization_Backward(float const *x, float const *dy, float *dx, float const *mean, float const *rstd, float gamma, int node_size, int frame_size, int frame_stride, int x_frame_stride);
 void oracle_bit_BinaryLut6_Forward(std::int32_t const *x, std::int32_t *y, std::int32_t const *idx, std::int32_t const *table, int node_size, int frame_size, int frame_stride);
 }
 
@@ -393,6 +397,86 @@ static void test_convolution2d(void)
 
 // The tail of a classifier through the host classes: AverageLut against the oracle, and the reference's own known-answer test
 // of the loss (tests/gtest/LossSoftmaxCrossEntropyTest.cpp:8-92, NumPy goldens: loss within 1e-4, dy within 1e-6).
+// StochasticBatchNormalization: two training passes (the running statistics move twice), backward, the pass repeated from the
+// stored statistics, inference, the gain / offset form of inference, and a round trip through a stream
+static void test_stochastic_batch_normalization(void)
+{
+    int const C = 5, H = 3, W = 4, NODES = C * H * W, F = 200;
+    float const momentum = 0.8f, gamma = 0.25f, beta = 0.5f;
+    auto bn = bb::StochasticBatchNormalization<>::Create(momentum, gamma, beta);
+    CHECK(bn->SetInputShape({C, H, W}) == bb::indices_t({C, H, W}) && bn->GetOutputNodeSize() == NODES, "normalisation shapes");
+    CHECK(bn->GetParameters().GetSize() == 0 && bn->GetGradients().GetSize() == 0, "normalisation has no trained parameters");
+    std::mt19937_64 mt(5);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    std::vector<float> rm((size_t)NODES, 0.0f), rv((size_t)NODES, 1.0f), mean((size_t)NODES), rstd((size_t)NODES);
+    std::vector<float> x, y, dy, dx, y_ref((size_t)NODES * F), dx_ref((size_t)NODES * F);
+    bb::FrameBuffer x_buf(F, {C, H, W}, BB_TYPE_FP32), dy_buf(F, {C, H, W}, BB_TYPE_FP32);
+    for (int pass = 0; pass < 2; ++pass) {
+        for (int n = 0; n < NODES; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, uni(mt) * (0.2f + 0.1f * (float)(n % 7))); dy_buf.SetFP32(f, n, uni(mt) - 0.5f); }
+        read_fp32(x_buf, x); read_fp32(dy_buf, dy);
+        bb::FrameBuffer y_buf = bn->Forward(x_buf, true);
+        read_fp32(y_buf, y);
+        oracle_fp32_StochasticBatchNormalization_ForwardTraining(x.data(), y_ref.data(), mean.data(), rstd.data(), rm.data(), rv.data(), gamma, beta, momentum, NODES, F, F);
+        CHECK(max_diff(y, y_ref) <= 2e-6 * (1.0 + max_abs(y_ref)) * 4, "normalisation y err %g (pass %d)", max_diff(y, y_ref), pass);
+        {
+            auto pm = bn->lock_mean_const(); auto pv = bn->lock_var_const(); auto bm = bn->lock_tmp_mean_const(); auto br = bn->lock_tmp_rstd_const();
+            double e = 0;
+            for (int n = 0; n < NODES; ++n) {
+                e = std::max(e, (double)std::fabs(pm[n] - rm[n])); e = std::max(e, (double)std::fabs(pv[n] - rv[n]));
+                e = std::max(e, (double)std::fabs(bm[n] - mean[n])); e = std::max(e, (double)std::fabs(br[n] - rstd[n]) / rstd[n]);
+            }
+            CHECK(e <= 5e-6, "normalisation statistics err %g (pass %d)", e, pass);
+        }
+        // the pass again from the stored statistics pushes the input a second time: two backward passes follow
+        bb::FrameBuffer y2_buf = bn->ReForward(x_buf);
+        CHECK(same_bits(y_buf, y2_buf), "normalisation: the repeated pass differs");
+        bb::FrameBuffer dx_buf = bn->Backward(dy_buf);
+        bb::FrameBuffer dx2_buf = bn->Backward(dy_buf);
+        CHECK(same_bits(dx_buf, dx2_buf), "normalisation: the two backward passes differ");
+        read_fp32(dx_buf, dx);
+        {
+            std::vector<float> bmean((size_t)NODES), brstd((size_t)NODES);
+            auto bm = bn->lock_tmp_mean_const(); auto br = bn->lock_tmp_rstd_const();
+            for (int n = 0; n < NODES; ++n) { bmean[(size_t)n] = bm[n]; brstd[(size_t)n] = br[n]; }
+            oracle_fp32_StochasticBatchNormalization_Backward(x.data(), dy.data(), dx_ref.data(), bmean.data(), brstd.data(), gamma, NODES, F, F, F);
+        }
+        CHECK(max_diff(dx, dx_ref) <= 1e-5 * max_abs(dx_ref), "normalisation dx err %g of %g", max_diff(dx, dx_ref), max_abs(dx_ref));
+    }
+    // inference from the running statistics, also as gain * x + offset and node by node
+    bb::FrameBuffer yi_buf = bn->Forward(x_buf, false);
+    read_fp32(yi_buf, y);
+    oracle_fp32_StochasticBatchNormalization_ForwardInference(x.data(), y_ref.data(), rm.data(), rv.data(), gamma, beta, NODES, F, F);
+    CHECK(max_diff(y, y_ref) <= 1e-5, "normalisation inference err %g", max_diff(y, y_ref));
+    {
+        double e = 0;
+        for (int n = 0; n < NODES; n += 7) {
+            double const v = (double)x[(size_t)n * F + 3];
+            e = std::max(e, std::fabs((double)bn->GetNormalizeGain(n) * v + (double)bn->GetNormalizeOffset(n) - (double)y[(size_t)n * F + 3]));
+            e = std::max(e, std::fabs(bn->ForwardNode(n, {v})[0] - (double)y[(size_t)n * F + 3]));
+        }
+        CHECK(e <= 1e-5, "normalisation gain / offset / ForwardNode err %g", e);
+    }
+    // through a stream, rebuilt from the type name: the same inference output, bit for bit
+    {
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        bn->DumpObject(ss);
+        auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)again && again->GetObjectName() == "StochasticBatchNormalization_fp32" && again->GetInputShape() == bb::indices_t({C, H, W}), "normalisation reload");
+        if (again) {
+            bb::FrameBuffer y3 = again->Forward(x_buf, false);
+            CHECK(same_bits(y3, yi_buf), "reloaded normalisation differs in inference");
+        }
+    }
+    // commands: gamma and beta can be changed; host-only execution is refused, not emulated
+    bn->SendCommand("set_gamma 0.5");
+    bn->SendCommand("set_beta 0.25");
+    CHECK(bn->GetGamma() == 0.5f && bn->GetBeta() == 0.25f, "set_gamma / set_beta");
+    bn->SendCommand("host_only true");
+    bool threw = false;
+    try { bn->Forward(x_buf); } catch (std::exception const &) { threw = true; }
+    CHECK(threw, "host_only normalisation must throw");
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -547,6 +631,7 @@ int main(void)
         test_adam();
         test_conv_plumbing();
         test_convolution2d();
+        test_stochastic_batch_normalization();
         test_tail();
         test_hand_off_through_files();
     }

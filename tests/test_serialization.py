@@ -213,3 +213,45 @@ def test_damaged_container_objects_are_rejected(tmp_path):
     p = str(tmp_path / "unknown.bin")
     open(p, "wb").write(bad)
     assert tool("reload", p, str(tmp_path / "x.bin"), check=False).returncode != 0
+
+
+# ----------------------------------------------------------------------------------------------
+#  StochasticBatchNormalization (include/bb/StochasticBatchNormalization.h:143-183): the objects that the reference's class wrote
+#  after a training pass (tests/golden/bn.npz), running statistics included
+# ----------------------------------------------------------------------------------------------
+BN = np.load(os.path.join(HERE, "golden", "bn.npz"))
+
+
+@pytest.mark.parametrize("k", range(int(BN["count"][0])))
+def test_reference_normalisation_objects_load_and_survive_a_round_trip(tmp_path, k):
+    p = "b%d_" % k
+    data = BN[p + "object"].tobytes()
+    name = BN[p + "name"].tobytes().decode()
+    nodes = int(BN[p + "geom"][0])
+    src, dst = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    open(src, "wb").write(data)
+    out = tool("reload", src, dst).stdout.split()
+    assert out[0] == "StochasticBatchNormalization_fp32"
+    assert out[1] == (name if name else "StochasticBatchNormalization")
+    assert (int(out[3]), int(out[5])) == (nodes, nodes)
+    assert open(dst, "rb").read() == data
+    # the running statistics sit at the end of the object: two typed tensors of `nodes` floats each
+    tail = np.frombuffer(data[-4 * nodes:], np.float32)
+    assert np.array_equal(tail, BN[p + "running_var"])
+
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref is not built")
+def test_normalisation_objects_against_the_reference(tmp_path):
+    rng = np.random.default_rng(99)
+    for trial in range(4):
+        nodes, frames = int(rng.integers(1, 40)), int(rng.integers(2, 90))
+        x = rng.random((nodes, frames)).astype(np.float32)
+        r = oracle.ref_stochastic_bn(x, rng.standard_normal(nodes), rng.random(nodes) + 0.5, 0.1 + 0.1 * trial, 0.5, 0.8,
+                                     train=True, name="bn%d" % trial if trial % 2 else "", want_object=True)
+        src, dst = str(tmp_path / ("in%d.bin" % trial)), str(tmp_path / ("out%d.bin" % trial))
+        open(src, "wb").write(r["object"].tobytes())
+        tool("reload", src, dst)
+        mine = np.frombuffer(open(dst, "rb").read(), np.uint8)
+        assert np.array_equal(mine, r["object"]), trial
+        back = oracle.ref_reload_container_object(mine)
+        assert back is not None and np.array_equal(back, r["object"]), trial
