@@ -250,6 +250,40 @@ inline int bbcu_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, fl
     return 0;
 }
 
+/* ---- StochasticBatchNormalization, include/bbcu/bbcu.h:883-942 ---- */
+inline int bbcu_fp32_StochasticBatchNormalization_ForwardTraining(float const *dev_x_buf, float *dev_y_buf, float *dev_mean_buf,
+        float *dev_rstd_buf, float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta, float momentum,
+        int node_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_StochasticBatchNormalization_ForwardTraining(dev_x_buf, dev_y_buf, dev_mean_buf, dev_rstd_buf, dev_running_mean_buf,
+                                                                          dev_running_var_buf, gamma, beta, momentum, node_size, frame_size,
+                                                                          frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_StochasticBatchNormalization_ReForward(float const *dev_x_buf, float *dev_y_buf, float const *dev_mean_buf,
+        float const *dev_rstd_buf, float gamma, float beta, int node_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_StochasticBatchNormalization_ReForward(dev_x_buf, dev_y_buf, dev_mean_buf, dev_rstd_buf, gamma, beta, node_size,
+                                                                    frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_StochasticBatchNormalization_ForwardInference(float const *dev_x_buf, float *dev_y_buf, float const *dev_running_mean_buf,
+        float const *dev_running_var_buf, float gamma, float beta, int node_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_StochasticBatchNormalization_ForwardInference(dev_x_buf, dev_y_buf, dev_running_mean_buf, dev_running_var_buf, gamma,
+                                                                           beta, node_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_StochasticBatchNormalization_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf,
+        float const *dev_mean_buf, float const *dev_rstd_buf, float gamma, float reciprocal_frame_size, int node_size, int frame_size,
+        int frame_stride, int x_frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_StochasticBatchNormalization_Backward(dev_x_buf, dev_dy_buf, dev_dx_buf, dev_mean_buf, dev_rstd_buf, gamma,
+                                                                   reciprocal_frame_size, node_size, frame_size, frame_stride, x_frame_stride,
+                                                                   streamId));
+    return 0;
+}
+
 /* ---- Im2Col / Col2Im, include/bbcu/bbcu.h:1076-1186 ---- */
 inline int bbcu_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
         int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size, int output_w_size,

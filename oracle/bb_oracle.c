@@ -24,6 +24,10 @@
  *     contraction choices), textbook mean/variance, BN gradient invariants.
  *   - BinaryLut6, reverse table: bit-exact against oracle/_ref and golden
  *     vectors; BinaryLut6 also against StochasticLut with W,x in {0,1}.
+ *   - StochasticBatchNormalization *: the reference's class (oracle/_ref) and
+ *     vectors written from it (tests/golden/bn.npz) to 1e-6 of the terms that
+ *     cancel (contraction, as above; the batch mean bit-exact), fp64 textbook
+ *     statistics, the gradient's two vanishing sums and a finite difference.
  *
  * Array conventions (the reference's FrameBuffer layout, include/bb/FrameBuffer.h:28-46,
  * 927-939): node-major, frame-minor; element (node n, frame f) of an fp32
