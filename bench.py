@@ -229,8 +229,8 @@ def bench_stochastic_bn(args, lib):
 
 
 def bench_tail(args, lib):
-    """The tail of the MNIST-like classifier (secondary measurement): AverageLut 7 -> 1 over 70 -> 10 nodes, softmax cross
-    entropy and categorical accuracy over the 10 classes.  Measured at 65536 frames (streaming rate) and at the
+    """The tail of the MNIST-like classifier (secondary measurement): AverageLut 7 -> 1 over 70 -> 10 nodes (and MaxLut at the same
+    shape), softmax cross entropy and categorical accuracy over the 10 classes.  Measured at 65536 frames (streaming rate) and at the
     configuration's own batch of 1024 frames (launch-bound).  Algorithmic bytes: every element of input and output once."""
     import numpy as np
     import torch
@@ -252,21 +252,24 @@ def bench_tail(args, lib):
         cases = [
             ("average_lut_forward_kernel", lambda: ops.average_lut_forward(x, idx, F, False, False), e * F * (I + O)),
             ("average_lut_backward_kernel (+ reverse wiring)", lambda: ops.average_lut_backward(dy, idx, I, F), e * F * (I + O)),
+            ("max_lut_forward_kernel", lambda: ops.max_lut_forward(x, idx, F, False, False), e * F * (I + O)),
+            ("max_lut_backward_kernel (+ reverse wiring)", lambda: ops.max_lut_backward(x, dy, idx, F), e * F * (2 * I + O)),
             ("softmax_cross_entropy_kernel", lambda: ops.loss_softmax_cross_entropy(y, t, O, 1, F, t_sum=float(F)), e * F * 3 * O + 8 * F),
             ("categorical_accuracy_kernel", lambda: ops.metrics_categorical_accuracy(y, t, O, 1, F), e * F * 2 * O + 8 * F),
         ]
         total_ms = 0.0
         for name, fn, nbytes in cases:
             med = library_timed_ms(lib, fn, args.steps, args.warmup)
-            total_ms += med
+            if not name.startswith("max_lut"):          # the classifier's tail uses AverageLut; MaxLut is listed beside it, not added
+                total_ms += med
             if F == 65536:
                 kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
         totals[F] = total_ms
-    dom = max(kernels, key=lambda k: kernels[k]["ms"])
+    dom = max((k for k in kernels if not k.startswith("max_lut")), key=lambda k: kernels[k]["ms"])
     out = {"metric": "classifier tail (AverageLut fwd+bwd, softmax cross entropy, accuracy), ms per pass over 65536 frames", "value": totals[65536],
            "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": totals[65536], "higher_is_better": False,
            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "AverageLut 7->1 over 70->10 nodes + LossSoftmaxCrossEntropy + MetricsCategoricalAccuracy, 65536 frames",
+           "config": {"workload": "AverageLut 7->1 over 70->10 nodes + LossSoftmaxCrossEntropy + MetricsCategoricalAccuracy, 65536 frames (MaxLut at the same shape listed under kernels)",
                       "ms_at_1024_frames": totals[1024]},
            "roofline": {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},

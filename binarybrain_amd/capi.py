@@ -64,6 +64,10 @@ _SIGNATURES = {
     "bbhip_fp32_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_bit_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_AverageLut_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 5 + [_vp]),
+    "bbhip_fp32_MaxLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_bit_MaxLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
+    "bbhip_fp32_MaxLut_Backward": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_bit_fp32_MaxLut_Backward": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_fp32_LossSoftmaxCrossEntropy": (C.c_int, [_vp, _vp, _vp, _vp, _f] + [_i] * 4 + [_vp]),
     "bbhip_fp32_MetricsCategoricalAccuracy": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_StochasticBatchNormalization_ForwardTraining": (C.c_int, [_vp] * 6 + [_f, _f, _f, _i, _i, _i, _vp]),

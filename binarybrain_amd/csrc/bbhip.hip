@@ -1374,12 +1374,94 @@ int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
     hipStream_t const st = static_cast<hipStream_t>(stream);
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(average_lut_reverse_kernel, dim3((unsigned)ceil_div(input_node_size + 1, kTailBlock)), dim3(kTailBlock), 0, st,
-                       dev_input_index, total, n, input_node_size, offsets, list);
+                       dev_input_index, total, n, input_node_size, offsets, list, 0);
     BBHIP_LAUNCH_CHECK();
     hipLaunchKernelGGL(average_lut_backward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_dy_buf, dev_dx_buf, offsets, list, n,
                        frame_size, frame_stride, f_blocks);
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+
+int bbhip_fp32_MaxLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                              int frame_stride, int binarize_input, int binarize_output, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
+    int const f_blocks = ceil_div(frame_size, kTailBlock);
+    long long const blocks = (long long)node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
+    hipLaunchKernelGGL(max_lut_forward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_x_buf,
+                       dev_y_buf, dev_input_index, n, frame_size, frame_stride, binarize_input, binarize_output, f_blocks);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_bit_MaxLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                             int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    int const words = (frame_size > 0) ? ceil_div(frame_size, 32) : 0;
+    if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, words, __func__)) { return 1; }
+    int const w_blocks = ceil_div(words, kTailBlock);
+    long long const blocks = (long long)node_size * w_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
+    hipLaunchKernelGGL(max_lut_forward_bit_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_x_buf,
+                       dev_y_buf, dev_input_index, n, words, frame_stride, w_blocks);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+// x: fp32 rows (bits == false) or packed rows of x_stride words; dy and dx: fp32 rows of dy_stride
+static int launch_max_lut_backward(void const *x, bool bits, float const *dy, float *dx, int const *idx, int n, int input_node_size,
+                                   int output_node_size, int frame_size, int x_stride, int dy_stride, int binarize_input, void *stream,
+                                   char const *name)
+{
+    if (check_average_lut(dy, dx, idx, n, output_node_size, frame_size, dy_stride, frame_size, name)) { return 1; }
+    if (x == nullptr) { return fail("%s: null buffer", name); }
+    if (input_node_size <= 0) { return fail("%s: sizes must be positive", name); }
+    if (x_stride < (bits ? ceil_div(frame_size, 32) : frame_size)) { return fail("%s: frame stride shorter than the frames", name); }
+    int const total = output_node_size * n;
+    int const f_blocks = ceil_div(dy_stride, kTailBlock);
+    long long const blocks = (long long)input_node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    char *scratch = nullptr;
+    size_t const offsets_bytes = align256(sizeof(int) * ((size_t)input_node_size + 1));
+    if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch, st)) { return 1; }
+    int *offsets = reinterpret_cast<int *>(scratch), *list = reinterpret_cast<int *>(scratch + offsets_bytes);
+    ScopedTimer tm(kTimeOther, st);
+    hipLaunchKernelGGL(average_lut_reverse_kernel, dim3((unsigned)ceil_div(input_node_size + 1, kTailBlock)), dim3(kTailBlock), 0, st,
+                       idx, total, n, input_node_size, offsets, list, 1);
+    BBHIP_LAUNCH_CHECK();
+    if (bits) {
+        hipLaunchKernelGGL(max_lut_backward_kernel<true>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, x, dy, dx, idx, offsets, list, n,
+                           frame_size, x_stride, dy_stride, 0, f_blocks);
+    }
+    else {
+        hipLaunchKernelGGL(max_lut_backward_kernel<false>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, x, dy, dx, idx, offsets, list, n,
+                           frame_size, x_stride, dy_stride, binarize_input, f_blocks);
+    }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_MaxLut_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n,
+                               int input_node_size, int output_node_size, int frame_size, int frame_stride, int binarize_input, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_max_lut_backward(dev_x_buf, false, dev_dy_buf, dev_dx_buf, dev_input_index, n, input_node_size, output_node_size, frame_size,
+                                   frame_stride, frame_stride, binarize_input, stream, __func__);
+}
+
+int bbhip_bit_fp32_MaxLut_Backward(int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n,
+                                   int input_node_size, int output_node_size, int frame_size, int x_frame_stride, int dy_frame_stride,
+                                   void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_max_lut_backward(dev_x_buf, true, dev_dy_buf, dev_dx_buf, dev_input_index, n, input_node_size, output_node_size, frame_size,
+                                   x_frame_stride, dy_frame_stride, 0, stream, __func__);
 }
 
 int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, float t_sum,

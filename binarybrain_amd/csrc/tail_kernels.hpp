@@ -108,8 +108,9 @@ __device__ __forceinline__ void stage_piece(int *piece, int const *__restrict__ 
     for (int k = threadIdx.x; k < padded; k += kTailBlock) { piece[k] = (k < count) ? src[k] : -1; }
 }
 
+// entry_ids: the list holds table positions (node * n + input position) instead of output nodes
 __global__ __launch_bounds__(kTailBlock) void average_lut_reverse_kernel(int const *__restrict__ idx, int total, int n, int input_node_size,
-                                                                         int *__restrict__ offsets, int *__restrict__ list)
+                                                                         int *__restrict__ offsets, int *__restrict__ list, int entry_ids)
 {
     __shared__ __attribute__((aligned(16))) int piece[kReversePiece];
     int const i = blockIdx.x * kTailBlock + threadIdx.x;
@@ -137,10 +138,10 @@ __global__ __launch_bounds__(kTailBlock) void average_lut_reverse_kernel(int con
 #pragma unroll 2
             for (int k = 0; k < count; k += 4) {
                 int4 const e = *reinterpret_cast<int4 const *>(&piece[k]);
-                if (e.x == i) { list[at++] = (base + k) / n; }
-                if (e.y == i) { list[at++] = (base + k + 1) / n; }
-                if (e.z == i) { list[at++] = (base + k + 2) / n; }
-                if (e.w == i) { list[at++] = (base + k + 3) / n; }
+                if (e.x == i) { list[at++] = entry_ids ? (base + k)     : (base + k) / n; }
+                if (e.y == i) { list[at++] = entry_ids ? (base + k + 1) : (base + k + 1) / n; }
+                if (e.z == i) { list[at++] = entry_ids ? (base + k + 2) : (base + k + 2) / n; }
+                if (e.w == i) { list[at++] = entry_ids ? (base + k + 3) : (base + k + 3) / n; }
             }
         }
     }
@@ -159,6 +160,77 @@ __global__ __launch_bounds__(kTailBlock) void average_lut_backward_kernel(float 
     float acc = 0.0f;
     for (int k = begin; k < end; ++k) { acc += dy[(size_t)list[k] * frame_stride + f] / fn; }
     dx[(size_t)in * frame_stride + f] = acc;
+}
+
+// MaxLut: the largest of the n wired inputs, starting from -1 and replaced by strictly larger values only (reference host
+// loop: include/bb/MaxLut.h:293-318); binarize_input as in the reference's device kernel (cuda/MaxLut.cu:33-36).
+// One thread per (output node, frame).
+__global__ __launch_bounds__(kTailBlock) void max_lut_forward_kernel(float const *x, float *y, int const *idx, int n, int frame_size,
+                                                                     int frame_stride, int binarize_input, int binarize_output, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const node = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    int const *row = idx + (size_t)node * n;
+    float max_val = -1.0f;
+    for (int i = 0; i < n; ++i) {
+        float v = x[(size_t)row[i] * frame_stride + f];
+        if (binarize_input) { v = (v > 0.0f) ? 1.0f : -1.0f; }
+        if (v > max_val) { max_val = v; }
+    }
+    if (binarize_output) { max_val = (max_val > 0.0f) ? 1.0f : -1.0f; }
+    y[(size_t)node * frame_stride + f] = max_val;
+}
+
+// packed bits, one thread per (output node, 32-frame word): the OR of the n input words
+__global__ __launch_bounds__(kTailBlock) void max_lut_forward_bit_kernel(int const *x, int *y, int const *idx, int n, int words,
+                                                                         int frame_stride, int w_blocks)
+{
+    int const w = (int)(blockIdx.x % w_blocks) * kTailBlock + threadIdx.x;
+    int const node = blockIdx.x / w_blocks;
+    if (w >= words) { return; }
+    int const *row = idx + (size_t)node * n;
+    uint32_t any = 0u;
+    for (int i = 0; i < n; ++i) { any |= (uint32_t)x[(size_t)row[i] * frame_stride + w]; }
+    y[(size_t)node * frame_stride + w] = (int)any;
+}
+
+// One thread per (input node, column of the dx row pitch): over the table positions that name this input, in table order, add
+// the node's dy where this position holds the node's first largest input (include/bb/MaxLut.h:394-424).  BITS: x is packed, the
+// first largest input is the first one that is set (position 0 when none is).
+template <bool BITS>
+__global__ __launch_bounds__(kTailBlock) void max_lut_backward_kernel(void const *x_buf, float const *dy, float *dx, int const *idx,
+                                                                      int const *offsets, int const *list, int n, int frame_size,
+                                                                      int x_stride, int dy_stride, int binarize_input, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const in = blockIdx.x / f_blocks;
+    if (f >= dy_stride) { return; }
+    if (f >= frame_size) { dx[(size_t)in * dy_stride + f] = 0.0f; return; }         // the row's padding reads as zero, as after the host's FillZero
+    int const begin = offsets[in], end = offsets[in + 1];
+    float acc = 0.0f;
+    for (int k = begin; k < end; ++k) {
+        int const entry = list[k], node = entry / n, pos = entry - node * n;
+        int const *row = idx + (size_t)node * n;
+        int first = 0;
+        if (BITS) {
+            uint32_t const *xb = static_cast<uint32_t const *>(x_buf);
+            for (int i = 0; i < n; ++i) {
+                if ((xb[(size_t)row[i] * x_stride + (f >> 5)] >> (f & 31)) & 1u) { first = i; break; }
+            }
+        }
+        else {
+            float const *xf = static_cast<float const *>(x_buf);
+            float max_val = -1.0f;
+            for (int i = 0; i < n; ++i) {
+                float v = xf[(size_t)row[i] * x_stride + f];
+                if (binarize_input) { v = (v > 0.0f) ? 1.0f : -1.0f; }
+                if (v > max_val) { max_val = v; first = i; }
+            }
+        }
+        if (first == pos) { acc += dy[(size_t)node * dy_stride + f]; }
+    }
+    dx[(size_t)in * dy_stride + f] = acc;
 }
 
 // Softmax cross entropy, one thread per (pixel, frame); node = ch * pix_size + pix.  partial[pix * frame_size + frame]

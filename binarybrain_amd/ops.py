@@ -264,6 +264,46 @@ def average_lut_backward(dy, idx, input_nodes, frame_size):
     return dx
 
 
+def max_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
+    """fp32 x [I, stride] -> y [O, stride]: the largest of the n wired inputs (not below -1), or its sign."""
+    _dev(x, idx)
+    O, n = idx.shape
+    y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_MaxLut_Forward(ptr(x), ptr(y), ptr(idx), n, O, frame_size, x.shape[1], int(binarize_input), int(binarize_output),
+                                          stream_ptr()))
+    return y
+
+
+def bit_max_lut_forward(xbits, idx, frame_size):
+    """packed x [I, words] -> packed y [O, words]: the OR of the n wired inputs."""
+    _dev(xbits, idx)
+    O, n = idx.shape
+    y = torch.empty((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    check(lib().bbhip_bit_MaxLut_Forward(ptr(xbits), ptr(y), ptr(idx), n, O, frame_size, xbits.shape[1], stream_ptr()))
+    return y
+
+
+def max_lut_backward(x, dy, idx, frame_size, binarize_input=False):
+    """dx [I, stride]: each node's dy goes to its first largest input."""
+    _dev(x, dy, idx)
+    O, n = idx.shape
+    if x.shape[1] != dy.shape[1]:
+        raise capi.BbhipError("max_lut_backward: x and dy must have the same row pitch")
+    dx = torch.empty((x.shape[0], dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_MaxLut_Backward(ptr(x), ptr(dy), ptr(dx), ptr(idx), n, x.shape[0], O, frame_size, dy.shape[1], int(binarize_input),
+                                           stream_ptr()))
+    return dx
+
+
+def bit_max_lut_backward(xbits, dy, idx, frame_size):
+    _dev(xbits, dy, idx)
+    O, n = idx.shape
+    dx = torch.empty((xbits.shape[0], dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_bit_fp32_MaxLut_Backward(ptr(xbits), ptr(dy), ptr(dx), ptr(idx), n, xbits.shape[0], O, frame_size, xbits.shape[1],
+                                               dy.shape[1], stream_ptr()))
+    return dx
+
+
 def loss_softmax_cross_entropy(y, t, ch_size, pix_size, frame_size, t_sum=None):
     """y, t [ch*pix, stride] -> (dy, loss_buf [frames] float64, t_sum).  t_sum defaults to the sum of the targets of the
     frames in use, taken in float64 as the reference's device path does; the loss of the batch is -loss_buf.sum() / t_sum."""

@@ -234,6 +234,39 @@ int bbcu_bit_fp32_StochasticLut_Backward(int const *dev_x_buf, float const *dev_
     return 0;
 }
 
+/* ---- MaxLut, include/bbcu/bbcu.h:364-427 (T = float).  The running maximum starts at -1, as in the reference's host loop
+ * (include/bb/MaxLut.h:293-318), not at the lowest float of its device kernel: outputs are never below -1. ---- */
+template <typename T>
+int bbcu_MaxLut_Forward(T const *dev_x_buf, T *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                        int frame_stride, bool binarize_input, bool binarize_output, cudaStream_t streamId = 0)
+{
+    static_assert(std::is_same<T, float>::value, "the library holds the fp32 instantiation");
+    BBCU_HIP_CALL(bbhip_fp32_MaxLut_Forward(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride,
+                                            binarize_input ? 1 : 0, binarize_output ? 1 : 0, streamId));
+    return 0;
+}
+inline int bbcu_bit_MaxLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size,
+                                   int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{ BBCU_HIP_CALL(bbhip_bit_MaxLut_Forward(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, streamId)); return 0; }
+template <typename T>
+int bbcu_MaxLut_Backward(T const *dev_x_buf, T const *dev_dy_buf, T *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
+                         int output_node_size, int frame_size, int frame_stride, bool binarize_input, cudaStream_t streamId = 0)
+{
+    static_assert(std::is_same<T, float>::value, "the library holds the fp32 instantiation");
+    BBCU_HIP_CALL(bbhip_fp32_MaxLut_Backward(dev_x_buf, dev_dy_buf, dev_dx_buf, dev_input_index, n, input_node_size, output_node_size, frame_size,
+                                             frame_stride, binarize_input ? 1 : 0, streamId));
+    return 0;
+}
+template <typename T>
+int bbcu_bit_MaxLut_Backward(int const *dev_x_buf, T const *dev_dy_buf, T *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
+                             int output_node_size, int frame_size, int x_frame_stride, int dy_frame_stride, cudaStream_t streamId = 0)
+{
+    static_assert(std::is_same<T, float>::value, "the library holds the fp32 instantiation");
+    BBCU_HIP_CALL(bbhip_bit_fp32_MaxLut_Backward(dev_x_buf, dev_dy_buf, dev_dx_buf, dev_input_index, n, input_node_size, output_node_size,
+                                                 frame_size, x_frame_stride, dy_frame_stride, streamId));
+    return 0;
+}
+
 /* ---- StochasticMaxPooling2x2, include/bbcu/bbcu.h:768-796 ---- */
 inline int bbcu_fp32_StochasticMaxPooling2x2_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size,
         int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)

@@ -229,6 +229,26 @@ int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const
  * the padding of every row, are written as 0.  Deterministic: the reverse wiring is built on the device in library scratch. */
 int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
                                    int output_node_size, int frame_size, int frame_stride, void *stream);
+/* ---- MaxLut ----
+ * The largest of n wired inputs, as the reference's host loop computes it (include/bb/MaxLut.h:293-318, 394-424): the running
+ * maximum starts at -1 and is replaced by strictly larger values, so the output is never below -1 (the reference's device kernel
+ * starts from the lowest float, cuda/MaxLut.cu:29) and the gradient goes to the first largest input.  binarize_input (read by the
+ * device kernel only, cuda/MaxLut.cu:33-36): inputs count as +1 where positive, else -1.  Bit-exact; the backward passes add in
+ * table order and give the same bits on every run. */
+/* bbcu_MaxLut_Forward<float>, include/bbcu/bbcu.h:368-381 */
+int bbhip_fp32_MaxLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                              int frame_stride, int binarize_input, int binarize_output, void *stream);
+/* bbcu_bit_MaxLut_Forward, include/bbcu/bbcu.h:383-393: the OR of the inputs */
+int bbhip_bit_MaxLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                             int frame_stride, void *stream);
+/* bbcu_MaxLut_Backward<float>, include/bbcu/bbcu.h:395-410; dx is overwritten (padding columns included, with zeros) */
+int bbhip_fp32_MaxLut_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n,
+                               int input_node_size, int output_node_size, int frame_size, int frame_stride, int binarize_input, void *stream);
+/* bbcu_bit_MaxLut_Backward<float>, include/bbcu/bbcu.h:413-427: packed x (rows of x_frame_stride words), fp32 dy and dx */
+int bbhip_bit_fp32_MaxLut_Backward(int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n,
+                                   int input_node_size, int output_node_size, int frame_size, int x_frame_stride, int dy_frame_stride,
+                                   void *stream);
+
 /* bbcu_LossSoftmaxCrossEntropy<float>, include/bbcu/bbcu.h:1506-1519.  Nodes are [ch][pix]; per frame and pixel softmax over the
  * channels; dev_loss_buf[frame] = sum over pixels and channels with t > 0 of log(softmax + 1e-7) * t_max (t_max = sum of the pixel's
  * targets), dy = (t_max * softmax - t) / t_sum.  The caller passes t_sum = sum of all targets and reports

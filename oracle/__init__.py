@@ -259,6 +259,46 @@ def average_lut_backward(dy, idx, input_node_size, frame_size):
     return dx
 
 
+def max_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
+    """fp32 x [I, stride] -> y [O, stride]: the largest of the n wired inputs, not below -1 (or its sign), the reference's host loop
+    (include/bb/MaxLut.h:293-318)."""
+    x = _c(x, np.float32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    y = np.zeros((O, x.shape[1]), np.float32)
+    lib().oracle_fp32_MaxLut_Forward(_ptr(x), _ptr(y), _ptr(idx), C.c_int(n), C.c_int(O), C.c_int(frame_size), C.c_int(x.shape[1]),
+                                     C.c_int(int(binarize_input)), C.c_int(int(binarize_output)))
+    return y
+
+
+def bit_max_lut_forward(xbits, idx, frame_size):
+    """packed x [I, words] -> packed y [O, words]: the OR of the n wired inputs."""
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    y = np.zeros((O, xbits.shape[1]), np.int32)
+    lib().oracle_bit_MaxLut_Forward(_ptr(xbits), _ptr(y), _ptr(idx), C.c_int(n), C.c_int(O), C.c_int(frame_size), C.c_int(xbits.shape[1]))
+    return y
+
+
+def max_lut_backward(x, dy, idx, frame_size, binarize_input=False):
+    """dx [I, stride]: each node's dy goes to its first largest input (include/bb/MaxLut.h:394-424)."""
+    x = _c(x, np.float32); dy = _c(dy, np.float32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    dx = np.zeros((x.shape[0], dy.shape[1]), np.float32)
+    assert x.shape[1] == dy.shape[1]
+    lib().oracle_fp32_MaxLut_Backward(_ptr(x), _ptr(dy), _ptr(dx), _ptr(idx), C.c_int(n), C.c_int(x.shape[0]), C.c_int(O),
+                                      C.c_int(frame_size), C.c_int(dy.shape[1]), C.c_int(int(binarize_input)))
+    return dx
+
+
+def bit_max_lut_backward(xbits, dy, idx, frame_size):
+    xbits = _c(xbits, np.int32); dy = _c(dy, np.float32); idx = _c(idx, np.int32)
+    O, n = idx.shape
+    dx = np.zeros((xbits.shape[0], dy.shape[1]), np.float32)
+    lib().oracle_bit_MaxLut_Backward(_ptr(xbits), _ptr(dy), _ptr(dx), _ptr(idx), C.c_int(n), C.c_int(xbits.shape[0]), C.c_int(O),
+                                     C.c_int(frame_size), C.c_int(xbits.shape[1]), C.c_int(dy.shape[1]))
+    return dx
+
+
 def loss_t_sum(t, frame_size):
     t = _c(t, np.float32)
     f = lib().oracle_fp32_LossSoftmaxCrossEntropy_TSum
@@ -675,6 +715,27 @@ def ref_average_lut(x, idx, input_node_size, frames, bit=False, binarize_input=F
     assert ref().bbref_AverageLut(C.c_int(int(bit)), C.c_int(n), C.c_int(input_node_size), C.c_int(O), C.c_int(frames), _ptr(x), _ptr(idx),
                                   C.c_int(int(binarize_input)), C.c_int(int(binarize_output)), _ptr(y), _ptr(dy), _ptr(dx)) == 0
     return y, dx
+
+
+def ref_max_lut(x, idx, input_node_size, frames, bit=False, binarize_input=False, binarize_output=True, dy=None, name="", want_object=False):
+    """The reference's MaxLut host path on dense [nodes, frames] (or [nodes, words]) arrays -> (y, dx, object bytes)."""
+    idx = _c(idx, np.int32)
+    O, n = idx.shape
+    if bit:
+        x = _c(x, np.int32); y = np.zeros((O, (frames + 31) // 32), np.int32)
+    else:
+        x = _c(x, np.float32); y = np.zeros((O, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((input_node_size, frames), np.float32)
+    out = np.zeros((1 << 16) + 8 * idx.size, np.uint8) if want_object else None
+    f = ref().bbref_MaxLut
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(n), C.c_int(input_node_size), C.c_int(O), C.c_int(frames), _ptr(x), _ptr(idx),
+          C.c_int(int(binarize_input)), C.c_int(int(binarize_output)), _ptr(y), _ptr(dy), _ptr(dx), C.c_char_p(name.encode()), _ptr(out),
+          C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
 
 
 def ref_loss_and_accuracy(y, t, ch_size, pix_size, frames):

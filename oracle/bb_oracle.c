@@ -24,6 +24,9 @@
  *     contraction choices), textbook mean/variance, BN gradient invariants.
  *   - BinaryLut6, reverse table: bit-exact against oracle/_ref and golden
  *     vectors; BinaryLut6 also against StochasticLut with W,x in {0,1}.
+ *   - MaxLut *: bit-exact against the reference's class (oracle/_ref), vectors
+ *     written from it (tests/golden/maxlut.npz), the known answers of
+ *     tests/gtest/MaxLutTest.cpp and numpy max / argmax.
  *   - StochasticBatchNormalization *: the reference's class (oracle/_ref) and
  *     vectors written from it (tests/golden/bn.npz) to 1e-6 of the terms that
  *     cancel (contraction, as above; the batch mean bit-exact), fp64 textbook
@@ -1134,6 +1137,80 @@ void oracle_fp32_StochasticBatchNormalization_Backward(float const *x, float con
             float const dxn = dyr[f] * gamma;
             float const dxc = dxn * rstd;
             dxr[f] = dxc + dmean + (xr[f] * dvar / (float)frame_size);
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ *  MaxLut: the largest of n wired inputs (reference host path, include/bb/MaxLut.h: forward :293-318, backward :394-424).
+ *  The running maximum starts at BB_BINARY_LO = -1 (DataType.h:49) and is replaced by a strictly larger value, so the
+ *  output is never below -1 and the gradient goes to the FIRST largest input (to input 0 when none exceeds -1).
+ *  binarize_output: +1 where the maximum is positive, else -1.  The host loop does not look at binarize_input; the
+ *  reference's device kernel does (cuda/MaxLut.cu:33-36: x = x > 0 ? +1 : -1 before the comparison) and the flag is
+ *  restated here in that meaning — with the flag off this is the host loop.
+ *  Packed bits: a Bit is +1 / -1, so the maximum is the OR of the inputs and the gradient goes to the first input
+ *  that is set (input 0 when none is).
+ *  Pinned by tests/test_oracle_maxlut.py: the reference's class (oracle/_ref) and vectors written from it
+ *  (tests/golden/maxlut.npz), the known answers of tests/gtest/MaxLutTest.cpp:15-139, numpy max / argmax.
+ * ------------------------------------------------------------------------------------------------------------------- */
+void oracle_fp32_MaxLut_Forward(float const *x, float *y, int32_t const *idx, int n, int node_size, int frame_size,
+                                int frame_stride, int binarize_input, int binarize_output)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float max_val = -1.0f;
+            for (int i = 0; i < n; ++i) {
+                float val = x[(long long)idx[node * n + i] * frame_stride + f];
+                if (binarize_input) { val = (val > 0) ? 1.0f : -1.0f; }
+                if (val > max_val) { max_val = val; }
+            }
+            if (binarize_output) { max_val = (max_val > 0) ? 1.0f : -1.0f; }
+            y[(long long)node * frame_stride + f] = max_val;
+        }
+    }
+}
+
+void oracle_bit_MaxLut_Forward(int const *x, int *y, int32_t const *idx, int n, int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            int any = 0;
+            for (int i = 0; i < n; ++i) { any |= get_bit(x + (long long)idx[node * n + i] * frame_stride, f); }
+            set_bit(y + (long long)node * frame_stride, f, any);
+        }
+    }
+}
+
+/* dx = 0, then node ascending: dx[first largest input] += dy */
+void oracle_fp32_MaxLut_Backward(float const *x, float const *dy, float *dx, int32_t const *idx, int n, int input_node_size,
+                                 int output_node_size, int frame_size, int frame_stride, int binarize_input)
+{
+    memset(dx, 0, sizeof(float) * (size_t)input_node_size * (size_t)frame_stride);
+    for (int node = 0; node < output_node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float max_val = -1.0f;
+            int max_idx = 0;
+            for (int i = 0; i < n; ++i) {
+                float val = x[(long long)idx[node * n + i] * frame_stride + f];
+                if (binarize_input) { val = (val > 0) ? 1.0f : -1.0f; }
+                if (val > max_val) { max_val = val; max_idx = i; }
+            }
+            dx[(long long)idx[node * n + max_idx] * frame_stride + f] += dy[(long long)node * frame_stride + f];
+        }
+    }
+}
+
+void oracle_bit_MaxLut_Backward(int const *x, float const *dy, float *dx, int32_t const *idx, int n, int input_node_size,
+                                int output_node_size, int frame_size, int x_frame_stride, int dy_frame_stride)
+{
+    memset(dx, 0, sizeof(float) * (size_t)input_node_size * (size_t)dy_frame_stride);
+    for (int node = 0; node < output_node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            int max_idx = 0;
+            for (int i = 0; i < n; ++i) {
+                if (get_bit(x + (long long)idx[node * n + i] * x_frame_stride, f)) { max_idx = i; break; }
+            }
+            dx[(long long)idx[node * n + max_idx] * dy_frame_stride + f] += dy[(long long)node * dy_frame_stride + f];
         }
     }
 }

@@ -28,6 +28,7 @@
 #include "bb/StochasticMaxPooling2x2.h"
 #include "bb/TensorOperator.h"
 #include "bb/AverageLut.h"
+#include "bb/MaxLut.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
 #include "bb/Convolution2d.h"
@@ -745,4 +746,42 @@ extern "C" long bbref_StochasticBatchNormalization(int nodes, int frames, float 
         get_fp32(dxb, dx, nodes, frames);
     }
     return object_out ? emit(*m, object_out, cap) : 0;
+}
+
+// MaxLut<BinType, float> (host path).  x: [I][frames] (fp32) or [I][words] (bits); y likewise for O nodes; dx is fp32 either way.
+// object_out (may be null) receives the layer dumped after the passes; returns its size (0 without), negative on error.
+namespace {
+template <typename BinType>
+long run_max_lut(int n, int I, int O, int F, void const *x, std::int32_t const *idx, int binarize_input, int binarize_output,
+                 void *y, float const *dy, float *dx, char const *name, unsigned char *object_out, long cap)
+{
+    auto m = bb::MaxLut<BinType, float>::Create(n, bb::indices_t({(index_t)O}));
+    m->SendCommand("host_only true");
+    m->SendCommand("binarize_input " + onoff(binarize_input));
+    m->SendCommand("binarize_output " + onoff(binarize_output));
+    if (name && *name) { m->SetName(name); }
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)I}), xtype, true);
+    m->SetInputShape(xb.GetShape());
+    for (int o = 0; o < O; ++o) { for (int i = 0; i < n; ++i) { m->SetNodeConnectionIndex(o, i, idx[o * n + i]); } }
+    if (xtype == BB_TYPE_BIT) { put_bit(xb, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(xb, (float const *)x, I, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (xtype == BB_TYPE_BIT) { get_bit(yb, (std::int32_t *)y, O, (F + 31) / 32); }
+    else                      { get_fp32(yb, (float *)y, O, F); }
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, bb::indices_t({(index_t)O}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, O, F);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, I, F);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+}  // namespace
+
+extern "C" long bbref_MaxLut(int bit, int n, int I, int O, int F, void const *x, std::int32_t const *idx, int binarize_input,
+                             int binarize_output, void *y, float const *dy, float *dx, char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_max_lut<bb::Bit>(n, I, O, F, x, idx, binarize_input, binarize_output, y, dy, dx, name, object_out, cap)
+               : run_max_lut<float>(n, I, O, F, x, idx, binarize_input, binarize_output, y, dy, dx, name, object_out, cap);
 }

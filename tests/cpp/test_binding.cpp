@@ -45,6 +45,10 @@ SAME(&bbcu_bit_BinatyLut6_Forward, int (*)(int const *, int *, int const *, int 
 SAME(&bbcu_AverageLut_Forward<float>, int (*)(float const *, float *, int const *, int, int, int, int, bool, bool, S));
 SAME(&bbcu_bit_AverageLut_Forward, int (*)(int const *, int *, int const *, int, int, int, int, S));
 SAME(&bbcu_AverageLut_Backward<float>, int (*)(float const *, float *, int const *, int, int, int, int, int, S));
+SAME(&bbcu_MaxLut_Forward<float>, int (*)(float const *, float *, int const *, int, int, int, int, bool, bool, S));
+SAME(&bbcu_bit_MaxLut_Forward, int (*)(int const *, int *, int const *, int, int, int, int, S));
+SAME(&bbcu_MaxLut_Backward<float>, int (*)(float const *, float const *, float *, int const *, int, int, int, int, int, bool, S));
+SAME(&bbcu_bit_MaxLut_Backward<float>, int (*)(int const *, float const *, float *, int const *, int, int, int, int, int, int, S));
 
 // the LUT entries, bbcu.h:518-761: one block of checks per width, and the default width
 template <int N>
@@ -162,7 +166,7 @@ static int run_on_gpu(void)
 
 int main(int argc, char **argv)
 {
-    int const checks = 11 + 11 + 6 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 11;
+    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 11;
     if (argc > 1 && !std::strcmp(argv[1], "--gpu")) {
         if (!bbcu_IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
         int const bad = run_on_gpu();

@@ -17,6 +17,7 @@
 #include "bb/ConvolutionCol2Im.h"
 #include "bb/StochasticMaxPooling2x2.h"
 #include "bb/AverageLut.h"
+#include "bb/MaxLut.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
 #include "bb/Convolution2d.h"
@@ -40,6 +41,8 @@ void oracle_fp32_DifferentiableLutN_Backward(int n, float const *x, float const 
 void oracle_fp32_StochasticBatchNormalization_ForwardTraining(float const *x, float *y, float *mean, float *rstd, float *running_mean, float *running_var, float gamma, float beta, float momentum, int node_size, int frame_size, int frame_stride);
 void oracle_fp32_StochasticBatchNormalization_ForwardInference(float const *x, float *y, float const *running_mean, float const *running_var, float gamma, float beta, int node_size, int frame_size, int frame_stride);
 void oracle_fp32_StochasticBatchNormalization_Backward(float const *x, float const *dy, float *dx, float const *mean, float const *rstd, float gamma, int node_size, int frame_size, int frame_stride, int x_frame_stride);
+void oracle_fp32_MaxLut_Forward(float const *x, float *y, std::int32_t const *idx, int n, int node_size, int frame_size, int frame_stride, int binarize_input, int binarize_output);
+void oracle_fp32_MaxLut_Backward(float const *x, float const *dy, float *dx, std::int32_t const *idx, int n, int input_node_size, int output_node_size, int frame_size, int frame_stride, int binarize_input);
 void oracle_bit_BinaryLut6_Forward(std::int32_t const *x, std::int32_t *y, std::int32_t const *idx, std::int32_t const *table, int node_size, int frame_size, int frame_stride);
 }
 
@@ -477,6 +480,80 @@ static void test_stochastic_batch_normalization(void)
     CHECK(threw, "host_only normalisation must throw");
 }
 
+// MaxLut: the known answers of the reference's own test on packed bits (tests/gtest/MaxLutTest.cpp:15-139), then a wired fp32
+// layer against the oracle, bit for bit, and a trip through a stream
+static void test_max_lut(void)
+{
+    {
+        auto lut = bb::MaxLut<bb::Bit>::Create(6, bb::indices_t({2}), "serial");
+        bb::FrameBuffer x(3, {2, 6}, BB_TYPE_BIT);
+        lut->SetInputShape(x.GetShape());
+        for (int f = 0; f < 3; ++f) for (int n = 0; n < 12; ++n) { x.SetBit(f, n, false); }
+        x.SetBit(0, 2, true);
+        x.SetBit(1, 1, true); x.SetBit(1, 5, true); x.SetBit(1, 11, true);
+        x.SetBit(2, 6, true);
+        bb::FrameBuffer y = lut->Forward(x);
+        bool const want_y[2][3] = {{true, true, false}, {false, true, true}};
+        for (int n = 0; n < 2; ++n) for (int f = 0; f < 3; ++f) { CHECK(y.GetBit(f, n) == want_y[n][f], "MaxLut bits y(%d, %d)", f, n); }
+        bb::FrameBuffer dy(3, {2}, BB_TYPE_FP32);
+        float const g[2][3] = {{0.1f, 0.2f, 0.3f}, {0.4f, 0.5f, 0.6f}};
+        for (int n = 0; n < 2; ++n) for (int f = 0; f < 3; ++f) { dy.SetFP32(f, n, g[n][f]); }
+        bb::FrameBuffer dx = lut->Backward(dy);
+        int const winner[2][3] = {{2, 1, 0}, {6, 11, 6}};       // the set input, the first of two set inputs, input 0 of the node when none is set
+        for (int n = 0; n < 12; ++n) for (int f = 0; f < 3; ++f) {
+            float const want = (winner[n / 6][f] == n) ? g[n / 6][f] : 0.0f;
+            CHECK(dx.GetFP32(f, n) == want, "MaxLut bits dx(%d, %d) = %g, want %g", f, n, (double)dx.GetFP32(f, n), (double)want);
+        }
+    }
+    int const N = 5, I = 60, O = 24, F = 150;
+    auto lut = bb::MaxLut<float>::Create(N, bb::indices_t({O}), "random", false);
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), dy_buf(F, {O}, BB_TYPE_FP32);
+    lut->SetInputShape(x_buf.GetShape());
+    std::vector<std::int32_t> idx((size_t)O * N);
+    {
+        std::vector<int> uses((size_t)I, 0);
+        for (int o = 0; o < O; ++o) for (int i = 0; i < N; ++i) {
+            idx[(size_t)o * N + i] = (std::int32_t)lut->GetNodeConnectionIndex(o, i);
+            uses[(size_t)idx[(size_t)o * N + i]] += 1;
+        }
+        int lo = 1 << 30, hi = 0;
+        for (int u : uses) { lo = std::min(lo, u); hi = std::max(hi, u); }
+        CHECK(hi - lo <= 1, "MaxLut random wiring uses the inputs %d to %d times", lo, hi);      // dealt from shuffled decks
+    }
+    std::mt19937_64 mt(9);
+    std::uniform_real_distribution<float> uni(-2.0f, 1.0f);
+    for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, (f % 5 == 0) ? std::round(uni(mt)) : uni(mt)); }
+    for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dy_buf.SetFP32(f, n, uni(mt)); }
+    std::vector<float> x, dy, y, dx, y_ref((size_t)O * F), dx_ref((size_t)I * F);
+    read_fp32(x_buf, x); read_fp32(dy_buf, dy);
+    bb::FrameBuffer y_buf = lut->Forward(x_buf);
+    bb::FrameBuffer dx_buf = lut->Backward(dy_buf);
+    read_fp32(y_buf, y); read_fp32(dx_buf, dx);
+    oracle_fp32_MaxLut_Forward(x.data(), y_ref.data(), idx.data(), N, O, F, F, 0, 0);
+    oracle_fp32_MaxLut_Backward(x.data(), dy.data(), dx_ref.data(), idx.data(), N, I, O, F, F, 0);
+    CHECK(max_diff(y, y_ref) == 0.0, "MaxLut y differs by %g", max_diff(y, y_ref));
+    CHECK(max_diff(dx, dx_ref) == 0.0, "MaxLut dx differs by %g", max_diff(dx, dx_ref));
+    lut->SendCommand("binarize_output true");
+    bb::FrameBuffer yb_buf = lut->Forward(x_buf, false);
+    read_fp32(yb_buf, y);
+    oracle_fp32_MaxLut_Forward(x.data(), y_ref.data(), idx.data(), N, O, F, F, 0, 1);
+    CHECK(max_diff(y, y_ref) == 0.0, "MaxLut binarized y differs by %g", max_diff(y, y_ref));
+    {
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        lut->DumpObject(ss);
+        auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)again && again->GetObjectName() == "MaxLut_fp32_fp32" && again->GetOutputNodeSize() == O, "MaxLut reload");
+        if (again) {
+            bb::FrameBuffer y3 = again->Forward(x_buf, false);
+            CHECK(same_bits(y3, yb_buf), "reloaded MaxLut differs");
+        }
+    }
+    lut->SendCommand("host_only true");
+    bool threw = false;
+    try { lut->Forward(x_buf); } catch (bb::Exception const &) { threw = true; }
+    CHECK(threw, "host_only MaxLut must throw");
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -632,6 +709,7 @@ int main(void)
         test_conv_plumbing();
         test_convolution2d();
         test_stochastic_batch_normalization();
+        test_max_lut();
         test_tail();
         test_hand_off_through_files();
     }
