@@ -1,6 +1,6 @@
 // Reconstruct a serialized object from its recorded type name (reference: include/bb/ObjectLoader.h:407-447
 // `Object_Load` / `Object_LoadFromFile`).  Known here: the LUT layers of widths 2..6 on fp32 or packed-bit frames,
-// BinaryLut6, StochasticBatchNormalization, MaxLut, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
+// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
 #pragma once
 
 #include "bb/StochasticLutN.h"
@@ -12,6 +12,7 @@
 #include "bb/Sequential.h"
 #include "bb/StochasticBatchNormalization.h"
 #include "bb/MaxLut.h"
+#include "bb/AverageLut.h"
 
 namespace bb {
 
@@ -36,6 +37,8 @@ inline std::shared_ptr<Object> CreateByName(std::string const &name)
     if (name == BinaryLutN<6, Bit, float>::ObjectName()) { return BinaryLutN<6, Bit, float>::Create((index_t)1); }
     if (name == Sequential::ObjectName())                         { return Sequential::Create(); }
     if (name == StochasticBatchNormalization<float>::ObjectName()) { return StochasticBatchNormalization<float>::Create(); }
+    if (name == AverageLut<float, float>::ObjectName())           { return AverageLut<float, float>::Create(); }
+    if (name == AverageLut<Bit, float>::ObjectName())             { return AverageLut<Bit, float>::Create(); }
     if (name == MaxLut<float, float>::ObjectName())               { return MaxLut<float, float>::Create(); }
     if (name == MaxLut<Bit, float>::ObjectName())                 { return MaxLut<Bit, float>::Create(); }
     if (name == Convolution2d<float, float>::ObjectName())        { return Convolution2d<float, float>::Create(); }

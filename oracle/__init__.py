@@ -738,6 +738,19 @@ def ref_max_lut(x, idx, input_node_size, frames, bit=False, binarize_input=False
     return y, dx, (out[:r].copy() if want_object else None)
 
 
+def ref_average_lut_object(idx, input_node_size, bit=False, binarize_input=False, binarize_output=True, name=""):
+    """Bytes of an AverageLut layer with the given wiring as the reference's DumpObject writes it."""
+    idx = _c(idx, np.int32)
+    O, n = idx.shape
+    out = np.zeros((1 << 16) + 8 * idx.size, np.uint8)
+    f = ref().bbref_AverageLutObject
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(n), C.c_int(input_node_size), C.c_int(O), _ptr(idx), C.c_int(int(binarize_input)),
+          C.c_int(int(binarize_output)), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size))
+    assert r > 0, r
+    return out[:r].copy()
+
+
 def ref_loss_and_accuracy(y, t, ch_size, pix_size, frames):
     """The reference's LossSoftmaxCrossEntropy and MetricsCategoricalAccuracy host paths -> (dy, loss, metric)."""
     y = _c(y, np.float32); t = _c(t, np.float32)

@@ -785,3 +785,19 @@ extern "C" long bbref_MaxLut(int bit, int n, int I, int O, int F, void const *x,
     return bit ? run_max_lut<bb::Bit>(n, I, O, F, x, idx, binarize_input, binarize_output, y, dy, dx, name, object_out, cap)
                : run_max_lut<float>(n, I, O, F, x, idx, binarize_input, binarize_output, y, dy, dx, name, object_out, cap);
 }
+
+// An AverageLut<BinType, float> with the given wiring, dumped: returns the object's size, negative on error.
+extern "C" long bbref_AverageLutObject(int bit, int n, int I, int O, std::int32_t const *idx, int binarize_input, int binarize_output,
+                                       char const *name, unsigned char *out, long cap)
+{
+    auto fill = [&](auto m) {
+        m->SendCommand("binarize_input " + onoff(binarize_input));
+        m->SendCommand("binarize_output " + onoff(binarize_output));
+        if (name && *name) { m->SetName(name); }
+        m->SetInputShape(bb::indices_t({(index_t)I}));
+        for (int o = 0; o < O; ++o) { for (int i = 0; i < n; ++i) { m->SetNodeConnectionIndex(o, i, idx[o * n + i]); } }
+        return emit(*m, out, cap);
+    };
+    if (bit) { return fill(bb::AverageLut<bb::Bit, float>::Create(n, bb::indices_t({(index_t)O}))); }
+    return fill(bb::AverageLut<float, float>::Create(n, bb::indices_t({(index_t)O})));
+}

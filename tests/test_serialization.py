@@ -297,3 +297,25 @@ def test_max_lut_objects_against_the_reference(tmp_path):
         # (the reference's own loader does not know the type name MaxLut, include/bb/ObjectLoader.h, so there is no trip back
         # through it; equal bytes are what its LoadObject would read)
         assert oracle.ref_reload_container_object(mine) is None
+
+
+# ----------------------------------------------------------------------------------------------
+#  AverageLut (include/bb/AverageLut.h:412-458): the same layout as MaxLut (tests/golden/average_lut_objects.npz)
+# ----------------------------------------------------------------------------------------------
+AVERAGE = np.load(os.path.join(HERE, "golden", "average_lut_objects.npz"))
+
+
+@pytest.mark.parametrize("k", range(int(AVERAGE["count"][0])))
+def test_reference_average_lut_objects_load_and_survive_a_round_trip(tmp_path, k):
+    p = "a%d_" % k
+    n, I, O, bit, bin_in, bin_out = [int(v) for v in AVERAGE[p + "args"]]
+    name = AVERAGE[p + "name"].tobytes().decode()
+    data = AVERAGE[p + "bytes"].tobytes()
+    src, dst = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    open(src, "wb").write(data)
+    out = tool("reload", src, dst).stdout.split()
+    assert out[0] == ("AverageLut_bit_fp32" if bit else "AverageLut_fp32_fp32") and out[1] == (name if name else "AverageLut")
+    assert (int(out[3]), int(out[5])) == (I, O)
+    assert open(dst, "rb").read() == data
+    assert np.array_equal(np.frombuffer(data[-4 * O * n:], np.int32).reshape(O, n), AVERAGE[p + "idx"])
+    # (as for MaxLut, the reference's own loader does not list this type name: equal bytes are what its LoadObject would read)
