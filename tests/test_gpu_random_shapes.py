@@ -207,12 +207,54 @@ def test_random_shapes_of_the_exact_rows():
 
 
 def run_tail_case(ops, torch, seed):
-    """AverageLut and accuracy bit-exact, the loss at the tolerances of tests/test_gpu_tail.py, Adam bit-exact"""
+    """AverageLut, MaxLut and accuracy bit-exact, the loss at the tolerances of tests/test_gpu_tail.py, the normalisation at those of
+    tests/test_gpu_stochastic_bn.py, Adam bit-exact"""
     import test_gpu_tail as tail
     F32 = np.float32
     rng = np.random.default_rng(seed)
     kind = str(rng.choice(["average", "loss", "adam"]))
-    if kind == "average":
+    if seed >= 11150:           # the first 150 seeds keep the cases they always drew; later ones also draw the two newer kinds
+        kind = str(rng.choice([kind, "maxlut", "bn"], p=[0.4, 0.3, 0.3]))
+    if kind == "maxlut":
+        n = int(rng.choice([int(rng.integers(1, 17)), int(rng.integers(17, 200))])); I = int(rng.integers(1, 400)); O = int(rng.integers(1, 120))
+        F = int(rng.integers(1, 1500))
+        print("seed %d: maxlut n=%d I=%d O=%d F=%d" % (seed, n, I, O, F), flush=True)
+        idx = rng.integers(0, I, (O, n)).astype(np.int32)
+        stride = synth.frame_stride_fp32(F)
+        x = (rng.random((I, F)) * 3 - 2).astype(F32)
+        x[rng.random(x.shape) < 0.1] = 0.0
+        x[:, ::3] = np.round(x[:, ::3])
+        x = tail._pad(x, stride)
+        dy = tail._pad(rng.standard_normal((O, F)).astype(F32), stride)
+        for bin_in in (False, True):
+            for bin_out in (False, True):
+                y = host(ops.max_lut_forward(dev(x), dev(idx), F, bin_in, bin_out))
+                assert np.array_equal(y[:, :F], oracle.max_lut_forward(x, idx, F, bin_in, bin_out)[:, :F]), (bin_in, bin_out)
+            dx = host(ops.max_lut_backward(dev(x), dev(dy), dev(idx), F, bin_in))
+            assert np.array_equal(dx, oracle.max_lut_backward(x, dy, idx, F, bin_in)), bin_in
+        xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F), p=float(rng.choice([0.05, 0.3, 0.9])))
+        yb = host(ops.bit_max_lut_forward(dev(xb), dev(idx), F))
+        assert np.array_equal(synth.unpack_bits(yb, F), synth.unpack_bits(oracle.bit_max_lut_forward(xb, idx, F), F))
+        assert np.array_equal(host(ops.bit_max_lut_backward(dev(xb), dev(dy), dev(idx), F)), oracle.bit_max_lut_backward(xb, dy, idx, F))
+    elif kind == "bn":
+        import test_gpu_stochastic_bn as bn
+        nodes = int(rng.integers(1, 300)); F = int(rng.choice([int(rng.integers(2, 70)), int(rng.integers(64, 3000)), int(rng.integers(3000, 20000))]))
+        stride = int(rng.choice([synth.frame_stride_fp32(F), F, F + int(rng.integers(1, 9))]))
+        gamma = float(rng.choice([0.2, 0.3, 1.0])); beta = float(rng.choice([0.5, 0.0])); momentum = float(rng.choice([0.9, 0.0, 0.99]))
+        print("seed %d: bn nodes=%d F=%d stride=%d gamma=%g beta=%g momentum=%g" % (seed, nodes, F, stride, gamma, beta, momentum), flush=True)
+        x = bn._pad((rng.random((nodes, F)) * float(rng.choice([1.0, 0.05]))).astype(F32), stride)
+        dy = bn._pad(rng.standard_normal((nodes, F)).astype(F32), stride)
+        rm0 = rng.standard_normal(nodes).astype(F32); rv0 = (rng.random(nodes) + 0.5).astype(F32)
+        want = oracle.stochastic_bn_forward_training(x, rm0, rv0, gamma, beta, momentum, F)
+        rm = dev(rm0); rv = dev(rv0)
+        y, mean, rstd = ops.stochastic_bn_forward_training(dev(x), rm, rv, F, gamma, beta, momentum)
+        bn.check_forward(host(y), host(mean), host(rstd), host(rm), host(rv), want, x, gamma, F)
+        dx = host(ops.stochastic_bn_backward(dev(x), dev(dy), dev(want[1]), dev(want[2]), F, gamma))
+        bn.check_backward(dx, oracle.stochastic_bn_backward(x, dy, want[1], want[2], gamma, F), dy, want[2], gamma, x, F)
+        yi = host(ops.stochastic_bn_forward_inference(dev(x), dev(rm0), dev(rv0), F, gamma, beta))
+        wi = oracle.stochastic_bn_forward_inference(x, rm0, rv0, gamma, beta, F)
+        assert np.all(np.abs(yi[:, :F] - wi[:, :F]) <= 2e-6 * (np.abs(wi[:, :F]) + 1.0))
+    elif kind == "average":
         n = int(rng.choice([int(rng.integers(1, 17)), int(rng.integers(17, 400))])); I = int(rng.integers(1, 400)); O = int(rng.integers(1, 120))
         F = int(rng.integers(1, 1500))
         print("seed %d: average n=%d I=%d O=%d F=%d" % (seed, n, I, O, F), flush=True)
@@ -263,7 +305,7 @@ def run_tail_case(ops, torch, seed):
 def test_random_shapes_of_the_classifier_tail_and_adam():
     import torch
     from binarybrain_amd import ops
-    for seed in range(11000, 11150):
+    for seed in range(11000, 11300):
         run_tail_case(ops, torch, seed)
 
 
