@@ -68,6 +68,11 @@ _SIGNATURES = {
     "bbhip_bit_MaxLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_MaxLut_Backward": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_bit_fp32_MaxLut_Backward": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_fp32_Reduce_Forward": (C.c_int, [_vp, _vp] + [_i] * 4 + [_vp]),
+    "bbhip_bit_fp32_Reduce_Forward": (C.c_int, [_vp, _vp] + [_i] * 5 + [_vp]),
+    "bbhip_fp32_Reduce_Backward": (C.c_int, [_vp, _vp] + [_i] * 4 + [_vp]),
+    "bbhip_fp32_LossMeanSquaredError": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 4 + [_f, C.c_double, _vp]),
+    "bbhip_fp32_MetricsMeanSquaredError": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_LossSoftmaxCrossEntropy": (C.c_int, [_vp, _vp, _vp, _vp, _f] + [_i] * 4 + [_vp]),
     "bbhip_fp32_MetricsCategoricalAccuracy": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_StochasticBatchNormalization_ForwardTraining": (C.c_int, [_vp] * 6 + [_f, _f, _f, _i, _i, _i, _vp]),

@@ -1464,6 +1464,102 @@ int bbhip_bit_fp32_MaxLut_Backward(int const *dev_x_buf, float const *dev_dy_buf
                                    x_frame_stride, dy_frame_stride, 0, stream, __func__);
 }
 
+static int launch_reduce_forward(void const *x, bool bits, float *y, int input_node_size, int output_node_size, int frame_size,
+                                 int x_stride, int y_stride, void *stream, char const *name)
+{
+    if (!(x && y)) { return fail("%s: null buffer", name); }
+    if (!(input_node_size > 0 && output_node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (input_node_size % output_node_size != 0) { return fail("%s: the input nodes must be a multiple of the output nodes", name); }
+    if (x_stride < (bits ? ceil_div(frame_size, 32) : frame_size) || y_stride < frame_size) { return fail("%s: frame stride shorter than the frames", name); }
+    int const f_blocks = ceil_div(frame_size, kTailBlock);
+    long long const blocks = (long long)output_node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    int const mux = input_node_size / output_node_size;
+    ScopedTimer tm(kTimeOther, st);
+    if (bits) { hipLaunchKernelGGL(reduce_forward_kernel<true>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, x, y, mux, output_node_size, frame_size, x_stride, y_stride, f_blocks); }
+    else      { hipLaunchKernelGGL(reduce_forward_kernel<false>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, x, y, mux, output_node_size, frame_size, x_stride, y_stride, f_blocks); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_Reduce_Forward(float const *dev_x_buf, float *dev_y_buf, int input_node_size, int output_node_size, int frame_size,
+                              int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_reduce_forward(dev_x_buf, false, dev_y_buf, input_node_size, output_node_size, frame_size, frame_stride, frame_stride, stream, __func__);
+}
+
+int bbhip_bit_fp32_Reduce_Forward(int const *dev_x_buf, float *dev_y_buf, int input_node_size, int output_node_size, int frame_size,
+                                  int x_frame_stride, int y_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_reduce_forward(dev_x_buf, true, dev_y_buf, input_node_size, output_node_size, frame_size, x_frame_stride, y_frame_stride, stream, __func__);
+}
+
+int bbhip_fp32_Reduce_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_node_size, int output_node_size, int frame_size,
+                               int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (!(dev_dy_buf && dev_dx_buf)) { return fail("%s: null buffer", __func__); }
+    if (!(input_node_size > 0 && output_node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
+    if (input_node_size % output_node_size != 0) { return fail("%s: the input nodes must be a multiple of the output nodes", __func__); }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    int const f_blocks = ceil_div(frame_size, kTailBlock);
+    long long const blocks = (long long)input_node_size * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
+    hipLaunchKernelGGL(reduce_backward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_dy_buf, dev_dx_buf,
+                       input_node_size / output_node_size, output_node_size, frame_size, frame_stride, f_blocks);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int launch_mean_squared_error(float const *y, float const *t, float *dy, double *buf, int buf_size, int node_size, int frame_size,
+                                     int frame_stride, float grad_scale, double loss_scale, bool loss, void *stream, char const *name)
+{
+    if (!(y && t && buf && (dy || !loss))) { return fail("%s: null buffer", name); }
+    if (!(node_size > 0 && frame_size > 0 && buf_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", name); }
+    int const groups = ceil_div(node_size, kMseNodes), f_blocks = ceil_div(frame_size, kTailBlock);
+    long long const blocks = (long long)groups * f_blocks;
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    char *scratch = nullptr;
+    if (arena_get(sizeof(double) * (size_t)groups * (size_t)frame_size, &scratch, st)) { return 1; }
+    double *partial = reinterpret_cast<double *>(scratch);
+    ScopedTimer tm(kTimeOther, st);
+    if (loss) {
+        hipLaunchKernelGGL(mean_squared_error_kernel<true>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, y, t, dy, partial, grad_scale, loss_scale,
+                           node_size, frame_size, frame_stride, f_blocks);
+    }
+    else {
+        hipLaunchKernelGGL(mean_squared_error_kernel<false>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, y, t, dy, partial, grad_scale, loss_scale,
+                           node_size, frame_size, frame_stride, f_blocks);
+    }
+    BBHIP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(mean_squared_error_sum_kernel, dim3((unsigned)ceil_div(buf_size < frame_size ? buf_size : frame_size, kTailBlock)), dim3(kTailBlock),
+                       0, st, partial, buf, buf_size, groups, frame_size);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_LossMeanSquaredError(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, int loss_buf_size,
+                                    int node_size, int frame_size, int frame_stride, float grad_reduction, double loss_reduction, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_mean_squared_error(dev_y_buf, dev_t_buf, dev_dy_buf, dev_loss_buf, loss_buf_size, node_size, frame_size, frame_stride,
+                                     grad_reduction, loss_reduction, true, stream, __func__);
+}
+
+int bbhip_fp32_MetricsMeanSquaredError(float const *dev_y_buf, float const *dev_t_buf, double *dev_accuracy_buf, int accuracy_buf_size,
+                                       int node_size, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_mean_squared_error(dev_y_buf, dev_t_buf, nullptr, dev_accuracy_buf, accuracy_buf_size, node_size, frame_size, frame_stride,
+                                     0.0f, (double)node_size, false, stream, __func__);
+}
+
 int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, float t_sum,
                                        int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
 {

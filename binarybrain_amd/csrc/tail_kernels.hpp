@@ -233,6 +233,79 @@ __global__ __launch_bounds__(kTailBlock) void max_lut_backward_kernel(void const
     dx[(size_t)in * dy_stride + f] = acc;
 }
 
+// Reduce: output node o is the mean of the input nodes o, O + o, 2 O + o, ... (reference host loop: include/bb/Reduce.h:172-190;
+// the reference has no device code for this layer).  One thread per (output node, frame); BITS: packed input read as +1 / -1.
+template <bool BITS>
+__global__ __launch_bounds__(kTailBlock) void reduce_forward_kernel(void const *x_buf, float *y, int mux, int output_node_size, int frame_size,
+                                                                    int x_stride, int y_stride, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const o = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    float sum = 0.0f;
+    for (int i = 0; i < mux; ++i) {
+        size_t const row = (size_t)output_node_size * i + o;
+        if (BITS) { sum += ((static_cast<uint32_t const *>(x_buf)[row * x_stride + (f >> 5)] >> (f & 31)) & 1u) ? 1.0f : -1.0f; }
+        else      { sum += static_cast<float const *>(x_buf)[row * x_stride + f]; }
+    }
+    y[(size_t)o * y_stride + f] = sum / (float)mux;
+}
+
+// dx[input node] = dy[input node mod O] / mux (include/bb/Reduce.h:229-247); one thread per (input node, frame)
+__global__ __launch_bounds__(kTailBlock) void reduce_backward_kernel(float const *dy, float *dx, int mux, int output_node_size, int frame_size,
+                                                                     int frame_stride, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const in = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    dx[(size_t)in * frame_stride + f] = dy[(size_t)(in % output_node_size) * frame_stride + f] / (float)mux;
+}
+
+// Mean squared error.  One thread per (group of kMseNodes nodes, frame): dy = (y - t) * grad_scale, and the group's share of the
+// frame's loss, node ascending, in double: partial[group][frame] = sum of (float)(y - t)^2 * loss_scale (LOSS: NaN squares left
+// out, as the reference's loss does, include/bb/LossMeanSquaredError.h:150-169; else sum of (float)(t - y)^2 / node_size, as its
+// metric, MetricsMeanSquaredError.h:66-85).
+constexpr int kMseNodes = 64;
+
+template <bool LOSS>
+__global__ __launch_bounds__(kTailBlock) void mean_squared_error_kernel(float const *y, float const *t, float *dy, double *partial,
+                                                                        float grad_scale, double loss_scale, int node_size, int frame_size,
+                                                                        int frame_stride, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const group = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    int const first = group * kMseNodes, last = min(first + kMseNodes, node_size);
+    double acc = 0.0;
+    for (int node = first; node < last; ++node) {
+        size_t const at = (size_t)node * frame_stride + f;
+        if (LOSS) {
+            float const grad = y[at] - t[at];
+            float const error = rounded_mul(grad, grad);
+            dy[at] = rounded_mul(grad, grad_scale);
+            if (error == error) { acc += (double)error * loss_scale; }
+        }
+        else {
+            float const grad = t[at] - y[at];
+            acc += (double)rounded_mul(grad, grad) / loss_scale;
+        }
+    }
+    partial[(size_t)group * frame_size + f] = acc;
+}
+
+// buf[s] += the partial sums of the frames s, s + buf_size, s + 2 buf_size, ...: frames ascending, groups ascending within a frame
+__global__ __launch_bounds__(kTailBlock) void mean_squared_error_sum_kernel(double const *partial, double *buf, int buf_size, int groups,
+                                                                            int frame_size)
+{
+    int const s = blockIdx.x * kTailBlock + threadIdx.x;
+    if (s >= buf_size || s >= frame_size) { return; }
+    double acc = 0.0;
+    for (int f = s; f < frame_size; f += buf_size) {
+        for (int g = 0; g < groups; ++g) { acc += partial[(size_t)g * frame_size + f]; }
+    }
+    buf[s] += acc;
+}
+
 // Softmax cross entropy, one thread per (pixel, frame); node = ch * pix_size + pix.  partial[pix * frame_size + frame]
 // receives sum over the channels with t > 0 of log(softmax + eps) * t_max in double; with one pixel that is loss_buf itself.
 __global__ __launch_bounds__(kTailBlock) void softmax_cross_entropy_kernel(float const *y, float const *t, float *dy, double *partial,

@@ -1,6 +1,6 @@
 // Reconstruct a serialized object from its recorded type name (reference: include/bb/ObjectLoader.h:407-447
 // `Object_Load` / `Object_LoadFromFile`).  Known here: the LUT layers of widths 2..6 on fp32 or packed-bit frames,
-// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
+// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
 #pragma once
 
 #include "bb/StochasticLutN.h"
@@ -13,6 +13,7 @@
 #include "bb/StochasticBatchNormalization.h"
 #include "bb/MaxLut.h"
 #include "bb/AverageLut.h"
+#include "bb/Reduce.h"
 
 namespace bb {
 
@@ -40,6 +41,8 @@ inline std::shared_ptr<Object> CreateByName(std::string const &name)
     if (name == AverageLut<float, float>::ObjectName())           { return AverageLut<float, float>::Create(); }
     if (name == AverageLut<Bit, float>::ObjectName())             { return AverageLut<Bit, float>::Create(); }
     if (name == MaxLut<float, float>::ObjectName())               { return MaxLut<float, float>::Create(); }
+    if (name == Reduce<float, float>::ObjectName())               { return Reduce<float, float>::Create(); }
+    if (name == Reduce<Bit, float>::ObjectName())                 { return Reduce<Bit, float>::Create(); }
     if (name == MaxLut<Bit, float>::ObjectName())                 { return MaxLut<Bit, float>::Create(); }
     if (name == Convolution2d<float, float>::ObjectName())        { return Convolution2d<float, float>::Create(); }
     if (name == Convolution2d<Bit, float>::ObjectName())          { return Convolution2d<Bit, float>::Create(); }

@@ -304,6 +304,51 @@ def bit_max_lut_backward(xbits, dy, idx, frame_size):
     return dx
 
 
+def reduce_forward(x, output_nodes, frame_size):
+    """fp32 x [I, stride] -> y [O, stride]: node o is the mean of the inputs o, O + o, 2 O + o, ..."""
+    _dev(x)
+    y = torch.empty((output_nodes, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().bbhip_fp32_Reduce_Forward(ptr(x), ptr(y), x.shape[0], output_nodes, frame_size, x.shape[1], stream_ptr()))
+    return y
+
+
+def bit_reduce_forward(xbits, output_nodes, frame_size, y_stride):
+    """packed x [I, words] (bits read as +1 / -1) -> fp32 y [O, y_stride]"""
+    _dev(xbits)
+    y = torch.empty((output_nodes, y_stride), dtype=torch.float32, device=xbits.device)
+    check(lib().bbhip_bit_fp32_Reduce_Forward(ptr(xbits), ptr(y), xbits.shape[0], output_nodes, frame_size, xbits.shape[1], y_stride, stream_ptr()))
+    return y
+
+
+def reduce_backward(dy, input_nodes, frame_size):
+    _dev(dy)
+    dx = torch.empty((input_nodes, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_Reduce_Backward(ptr(dy), ptr(dx), input_nodes, dy.shape[0], frame_size, dy.shape[1], stream_ptr()))
+    return dx
+
+
+def loss_mean_squared_error(y, t, frame_size, loss_buf, batch_size=None, reduction_sum=False):
+    """-> dy; loss_buf (float64, device, any length >= 1) receives the batch's partial sums ON TOP of what it holds.  The layer's loss is
+    loss_buf.sum() / frames seen (the sum itself with reduction "sum")."""
+    _dev(y, t, loss_buf)
+    nodes = y.shape[0]
+    batch_size = frame_size if batch_size is None else batch_size
+    import numpy as np
+    grad_reduction = np.float32(1.0) if reduction_sum else np.float32(1.0) / np.float32(nodes * batch_size)
+    loss_reduction = 1.0 if reduction_sum else 1.0 / nodes
+    dy = torch.empty_like(y)
+    check(lib().bbhip_fp32_LossMeanSquaredError(ptr(y), ptr(t), ptr(dy), ptr(loss_buf), loss_buf.numel(), nodes, frame_size, y.shape[1],
+                                                float(np.float32(2) * grad_reduction), loss_reduction, stream_ptr()))
+    return dy
+
+
+def metrics_mean_squared_error(y, t, frame_size, accuracy_buf):
+    """accuracy_buf (float64, device) += the batch's partial sums of (t - y)^2 / nodes; the metric is accuracy_buf.sum() / frames seen."""
+    _dev(y, t, accuracy_buf)
+    check(lib().bbhip_fp32_MetricsMeanSquaredError(ptr(y), ptr(t), ptr(accuracy_buf), accuracy_buf.numel(), y.shape[0], frame_size, y.shape[1],
+                                                   stream_ptr()))
+
+
 def loss_softmax_cross_entropy(y, t, ch_size, pix_size, frame_size, t_sum=None):
     """y, t [ch*pix, stride] -> (dy, loss_buf [frames] float64, t_sum).  t_sum defaults to the sum of the targets of the
     frames in use, taken in float64 as the reference's device path does; the loss of the batch is -loss_buf.sum() / t_sum."""

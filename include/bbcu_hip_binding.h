@@ -267,6 +267,16 @@ int bbcu_bit_MaxLut_Backward(int const *dev_x_buf, T const *dev_dy_buf, T *dev_d
     return 0;
 }
 
+/* ---- LossMeanSquaredError, include/bbcu/bbcu.h:1487-1500 ---- */
+inline int bbcu_fp32_LossMeanSquaredError(const float *dev_y_buf, const float *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf,
+        int loss_buf_size, int node_size, int frame_size, int frame_stride, float grad_reduction, double loss_reduction,
+        cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_LossMeanSquaredError(dev_y_buf, dev_t_buf, dev_dy_buf, dev_loss_buf, loss_buf_size, node_size, frame_size,
+                                                  frame_stride, grad_reduction, loss_reduction, streamId));
+    return 0;
+}
+
 /* ---- StochasticMaxPooling2x2, include/bbcu/bbcu.h:768-796 ---- */
 inline int bbcu_fp32_StochasticMaxPooling2x2_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size,
         int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)

@@ -249,6 +249,32 @@ int bbhip_bit_fp32_MaxLut_Backward(int const *dev_x_buf, float const *dev_dy_buf
                                    int input_node_size, int output_node_size, int frame_size, int x_frame_stride, int dy_frame_stride,
                                    void *stream);
 
+/* ---- Reduce ----
+ * Output node o is the mean of the input nodes o, O + o, 2 O + o, ...; backward hands dy / mux to each of them
+ * (include/bb/Reduce.h:172-190, 229-247).  These three have no counterpart in include/bbcu/bbcu.h: the reference runs this layer
+ * on the host (its device calls are compiled out, Reduce.h:150-170, 207-227), which costs a device-resident pipeline a round trip
+ * through host memory.  Bit-exact with the host loops. */
+int bbhip_fp32_Reduce_Forward(float const *dev_x_buf, float *dev_y_buf, int input_node_size, int output_node_size, int frame_size,
+                              int frame_stride, void *stream);
+/* packed input (rows of x_frame_stride words) read as +1 / -1 */
+int bbhip_bit_fp32_Reduce_Forward(int const *dev_x_buf, float *dev_y_buf, int input_node_size, int output_node_size, int frame_size,
+                                  int x_frame_stride, int y_frame_stride, void *stream);
+int bbhip_fp32_Reduce_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_node_size, int output_node_size, int frame_size,
+                               int frame_stride, void *stream);
+
+/* ---- mean squared error ---- */
+/* bbcu_fp32_LossMeanSquaredError, include/bbcu/bbcu.h:1487-1500: dy = (y - t) * grad_reduction (the caller passes 2 / (nodes * batch)
+ * or 2); dev_loss_buf[s] += the sum over the frames s, s + loss_buf_size, ... and all nodes of (float)(y - t)^2 * loss_reduction in
+ * double, squares that are NaN left out as on the host path (include/bb/LossMeanSquaredError.h:150-169).  The caller adds the
+ * loss_buf_size entries up.  Sums are taken node ascending within groups of 64 nodes, then groups, then frames: the same bits on
+ * every run, and equal to the host's single running sum to rounding of doubles. */
+int bbhip_fp32_LossMeanSquaredError(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, int loss_buf_size,
+                                    int node_size, int frame_size, int frame_stride, float grad_reduction, double loss_reduction, void *stream);
+/* No counterpart in include/bbcu/bbcu.h (the reference computes this metric on the host, include/bb/MetricsMeanSquaredError.h:66-85):
+ * dev_accuracy_buf[s] += the sum over the frames s, s + accuracy_buf_size, ... and all nodes of (float)(t - y)^2 / node_size. */
+int bbhip_fp32_MetricsMeanSquaredError(float const *dev_y_buf, float const *dev_t_buf, double *dev_accuracy_buf, int accuracy_buf_size,
+                                       int node_size, int frame_size, int frame_stride, void *stream);
+
 /* bbcu_LossSoftmaxCrossEntropy<float>, include/bbcu/bbcu.h:1506-1519.  Nodes are [ch][pix]; per frame and pixel softmax over the
  * channels; dev_loss_buf[frame] = sum over pixels and channels with t > 0 of log(softmax + 1e-7) * t_max (t_max = sum of the pixel's
  * targets), dy = (t_max * softmax - t) / t_sum.  The caller passes t_sum = sum of all targets and reports

@@ -299,6 +299,52 @@ def bit_max_lut_backward(xbits, dy, idx, frame_size):
     return dx
 
 
+def reduce_forward(x, output_node_size, frame_size):
+    """fp32 x [I, stride] -> y [O, stride]: node o is the mean of the inputs o, O + o, 2 O + o, ... (include/bb/Reduce.h:172-190)."""
+    x = _c(x, np.float32)
+    y = np.zeros((output_node_size, x.shape[1]), np.float32)
+    lib().oracle_fp32_Reduce_Forward(_ptr(x), _ptr(y), C.c_int(x.shape[0]), C.c_int(output_node_size), C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y
+
+
+def bit_reduce_forward(xbits, output_node_size, frame_size, y_stride):
+    xbits = _c(xbits, np.int32)
+    y = np.zeros((output_node_size, y_stride), np.float32)
+    lib().oracle_bit_fp32_Reduce_Forward(_ptr(xbits), _ptr(y), C.c_int(xbits.shape[0]), C.c_int(output_node_size), C.c_int(frame_size),
+                                         C.c_int(xbits.shape[1]), C.c_int(y_stride))
+    return y
+
+
+def reduce_backward(dy, input_node_size, frame_size):
+    dy = _c(dy, np.float32)
+    dx = np.zeros((input_node_size, dy.shape[1]), np.float32)
+    lib().oracle_fp32_Reduce_Backward(_ptr(dy), _ptr(dx), C.c_int(input_node_size), C.c_int(dy.shape[0]), C.c_int(frame_size), C.c_int(dy.shape[1]))
+    return dx
+
+
+def loss_mean_squared_error(y, t, frame_size, batch_size=None, reduction_sum=False, loss=0.0):
+    """-> (dy, loss accumulator): the reference's host loop (include/bb/LossMeanSquaredError.h:121-169) for one batch; `loss` is the
+    accumulator before the batch.  The layer's loss is accumulator / frames seen (the accumulator itself with reduction "sum")."""
+    y = _c(y, np.float32); t = _c(t, np.float32)
+    nodes = y.shape[0]
+    batch_size = frame_size if batch_size is None else batch_size
+    grad_reduction = np.float32(1.0) if reduction_sum else np.float32(1.0) / np.float32(nodes * batch_size)
+    loss_reduction = 1.0 if reduction_sum else 1.0 / nodes
+    dy = np.zeros_like(y)
+    acc = C.c_double(loss)
+    lib().oracle_fp32_LossMeanSquaredError(_ptr(y), _ptr(t), _ptr(dy), C.byref(acc), C.c_int(nodes), C.c_int(frame_size), C.c_int(y.shape[1]),
+                                           C.c_float(grad_reduction), C.c_double(loss_reduction))
+    return dy, acc.value
+
+
+def metrics_mean_squared_error(y, t, frame_size, accuracy=0.0):
+    """-> the accumulator after the batch (include/bb/MetricsMeanSquaredError.h:66-85); the metric is accumulator / frames seen."""
+    y = _c(y, np.float32); t = _c(t, np.float32)
+    acc = C.c_double(accuracy)
+    lib().oracle_fp32_MetricsMeanSquaredError(_ptr(y), _ptr(t), C.byref(acc), C.c_int(y.shape[0]), C.c_int(frame_size), C.c_int(y.shape[1]))
+    return acc.value
+
+
 def loss_t_sum(t, frame_size):
     t = _c(t, np.float32)
     f = lib().oracle_fp32_LossSoftmaxCrossEntropy_TSum
@@ -749,6 +795,35 @@ def ref_average_lut_object(idx, input_node_size, bit=False, binarize_input=False
           C.c_int(int(binarize_output)), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size))
     assert r > 0, r
     return out[:r].copy()
+
+
+def ref_reduce(x, output_node_size, frames, bit=False, integration_size=0, dy=None, name="", want_object=False):
+    """The reference's Reduce host path on dense [nodes, frames] (or [nodes, words]) arrays -> (y, dx, object bytes)."""
+    x = _c(x, np.int32 if bit else np.float32)
+    I = x.shape[0]
+    y = np.zeros((output_node_size, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((I, frames), np.float32)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_Reduce
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(I), C.c_int(output_node_size), C.c_int(frames), C.c_int(integration_size), _ptr(x), _ptr(y), _ptr(dy),
+          _ptr(dx), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
+
+
+def ref_mean_squared_error(y, t, frames, batches=1, reduction_sum=False):
+    """The reference's LossMeanSquaredError and MetricsMeanSquaredError host paths over `batches` batches of `frames` frames held side
+    by side in y and t -> (dy, loss, metric)."""
+    y = _c(y, np.float32); t = _c(t, np.float32)
+    assert y.shape[1] == frames * batches
+    dy = np.zeros_like(y)
+    loss = C.c_double(0); metric = C.c_double(0)
+    assert ref().bbref_MeanSquaredError(C.c_int(y.shape[0]), C.c_int(frames), C.c_int(batches), C.c_int(int(reduction_sum)), _ptr(y), _ptr(t),
+                                        _ptr(dy), C.byref(loss), C.byref(metric)) == 0
+    return dy, loss.value, metric.value
 
 
 def ref_loss_and_accuracy(y, t, ch_size, pix_size, frames):

@@ -27,6 +27,9 @@
  *   - MaxLut *: bit-exact against the reference's class (oracle/_ref), vectors
  *     written from it (tests/golden/maxlut.npz), the known answers of
  *     tests/gtest/MaxLutTest.cpp and numpy max / argmax.
+ *   - Reduce *, LossMeanSquaredError, MetricsMeanSquaredError: bit-exact (double
+ *     accumulators included) against the reference's classes and vectors
+ *     written from them (tests/golden/reduce_mse.npz); numpy means in fp64.
  *   - StochasticBatchNormalization *: the reference's class (oracle/_ref) and
  *     vectors written from it (tests/golden/bn.npz) to 1e-6 of the terms that
  *     cancel (contraction, as above; the batch mean bit-exact), fp64 textbook
@@ -1211,6 +1214,76 @@ void oracle_bit_MaxLut_Backward(int const *x, float const *dy, float *dx, int32_
                 if (get_bit(x + (long long)idx[node * n + i] * x_frame_stride, f)) { max_idx = i; break; }
             }
             dx[(long long)idx[node * n + max_idx] * dy_frame_stride + f] += dy[(long long)node * dy_frame_stride + f];
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ *  Reduce: output node o is the mean of the input nodes o, O + o, 2 O + o, ... (reference host loop,
+ *  include/bb/Reduce.h:172-190; backward :229-247: every one of them receives dy / mux).  Packed bits read as +1 / -1
+ *  (DataType.h:302-303).  fp32 sums in input order, one division.
+ *  LossMeanSquaredError (include/bb/LossMeanSquaredError.h:150-169): frame outer, node inner; dy = 2 (y - t) * grad_reduction
+ *  in fp32; the loss accumulator (double) += (float)(y - t)^2 * loss_reduction unless that square is NaN.
+ *  MetricsMeanSquaredError (include/bb/MetricsMeanSquaredError.h:66-85): accumulator (double) += (float)(t - y)^2 / node_size.
+ *  Pinned by tests/test_oracle_reduce_mse.py: the reference's classes (oracle/_ref), vectors written from them
+ *  (tests/golden/reduce_mse.npz), numpy means in fp64.
+ * ------------------------------------------------------------------------------------------------------------------- */
+void oracle_fp32_Reduce_Forward(float const *x, float *y, int input_node_size, int output_node_size, int frame_size, int frame_stride)
+{
+    int const mux = input_node_size / output_node_size;
+    for (int o = 0; o < output_node_size; ++o) {
+        for (int f = 0; f < frame_size; ++f) {
+            float sum = 0;
+            for (int i = 0; i < mux; ++i) { sum += x[(long long)(output_node_size * i + o) * frame_stride + f]; }
+            y[(long long)o * frame_stride + f] = sum / (float)mux;
+        }
+    }
+}
+
+void oracle_bit_fp32_Reduce_Forward(int const *x, float *y, int input_node_size, int output_node_size, int frame_size,
+                                    int x_frame_stride, int y_frame_stride)
+{
+    int const mux = input_node_size / output_node_size;
+    for (int o = 0; o < output_node_size; ++o) {
+        for (int f = 0; f < frame_size; ++f) {
+            float sum = 0;
+            for (int i = 0; i < mux; ++i) { sum += get_bit(x + (long long)(output_node_size * i + o) * x_frame_stride, f) ? 1.0f : -1.0f; }
+            y[(long long)o * y_frame_stride + f] = sum / (float)mux;
+        }
+    }
+}
+
+void oracle_fp32_Reduce_Backward(float const *dy, float *dx, int input_node_size, int output_node_size, int frame_size, int frame_stride)
+{
+    int const mux = input_node_size / output_node_size;
+    for (int o = 0; o < output_node_size; ++o) {
+        for (int f = 0; f < frame_size; ++f) {
+            float const g = dy[(long long)o * frame_stride + f] / (float)mux;
+            for (int i = 0; i < mux; ++i) { dx[(long long)(output_node_size * i + o) * frame_stride + f] = g; }
+        }
+    }
+}
+
+void oracle_fp32_LossMeanSquaredError(float const *y, float const *t, float *dy, double *loss, int node_size, int frame_size,
+                                      int frame_stride, float grad_reduction, double loss_reduction)
+{
+    for (int f = 0; f < frame_size; ++f) {
+        for (int node = 0; node < node_size; ++node) {
+            float const grad = y[(long long)node * frame_stride + f] - t[(long long)node * frame_stride + f];
+            float const error = grad * grad;
+            dy[(long long)node * frame_stride + f] = 2 * grad * grad_reduction;
+            if (!isnan(error)) { *loss += error * loss_reduction; }
+        }
+    }
+}
+
+void oracle_fp32_MetricsMeanSquaredError(float const *y, float const *t, double *accuracy, int node_size, int frame_size, int frame_stride)
+{
+    for (int f = 0; f < frame_size; ++f) {
+        for (int node = 0; node < node_size; ++node) {
+            float const grad = t[(long long)node * frame_stride + f] - y[(long long)node * frame_stride + f];
+            float const error = grad * grad;
+            *accuracy += error / (double)node_size;
         }
     }
 }

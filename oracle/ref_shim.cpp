@@ -29,6 +29,9 @@
 #include "bb/TensorOperator.h"
 #include "bb/AverageLut.h"
 #include "bb/MaxLut.h"
+#include "bb/Reduce.h"
+#include "bb/LossMeanSquaredError.h"
+#include "bb/MetricsMeanSquaredError.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
 #include "bb/Convolution2d.h"
@@ -800,4 +803,66 @@ extern "C" long bbref_AverageLutObject(int bit, int n, int I, int O, std::int32_
     };
     if (bit) { return fill(bb::AverageLut<bb::Bit, float>::Create(n, bb::indices_t({(index_t)O}))); }
     return fill(bb::AverageLut<float, float>::Create(n, bb::indices_t({(index_t)O})));
+}
+
+// Reduce<BinType, float> (host path).  x: [I][frames] fp32 or [I][words] bits; y, dy: [O][frames]; dx: [I][frames].
+// integration_size 0: the output shape {O} is given; otherwise the layer derives it from the input shape {I}.
+namespace {
+template <typename BinType>
+long run_reduce(int I, int O, int F, int integration_size, void const *x, float *y, float const *dy, float *dx, char const *name,
+                unsigned char *object_out, long cap)
+{
+    auto m = bb::Reduce<BinType, float>::Create(bb::indices_t({(index_t)O}), (index_t)integration_size);
+    if (name && *name) { m->SetName(name); }
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)I}), xtype, true);
+    m->SetInputShape(xb.GetShape());
+    if (m->GetOutputNodeSize() != O) { return -2; }
+    if (xtype == BB_TYPE_BIT) { put_bit(xb, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(xb, (float const *)x, I, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    get_fp32(yb, y, O, F);
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, bb::indices_t({(index_t)O}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, O, F);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, I, F);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+}  // namespace
+
+extern "C" long bbref_Reduce(int bit, int I, int O, int F, int integration_size, void const *x, float *y, float const *dy, float *dx,
+                             char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_reduce<bb::Bit>(I, O, F, integration_size, x, y, dy, dx, name, object_out, cap)
+               : run_reduce<float>(I, O, F, integration_size, x, y, dy, dx, name, object_out, cap);
+}
+
+// LossMeanSquaredError<float> and MetricsMeanSquaredError<float> (host paths) over `batches` equal batches of F frames held one
+// after the other in y and t ([nodes][batches * F]); dy likewise.  loss = GetLoss(), metric = GetMetrics() after all of them.
+extern "C" int bbref_MeanSquaredError(int nodes, int F, int batches, int reduction_sum, float const *y, float const *t, float *dy,
+                                      double *loss, double *metric)
+{
+    auto lossFunc = bb::LossMeanSquaredError<float>::Create(reduction_sum ? "sum" : "");
+    auto metrics = bb::MetricsMeanSquaredError<float>::Create();
+    lossFunc->Clear();
+    metrics->Clear();
+    std::vector<float> ys((size_t)nodes * F), ts((size_t)nodes * F), ds((size_t)nodes * F);
+    for (int b = 0; b < batches; ++b) {
+        for (int n = 0; n < nodes; ++n) {
+            std::memcpy(&ys[(size_t)n * F], y + ((size_t)n * batches + b) * F, sizeof(float) * (size_t)F);
+            std::memcpy(&ts[(size_t)n * F], t + ((size_t)n * batches + b) * F, sizeof(float) * (size_t)F);
+        }
+        bb::FrameBuffer yb((index_t)F, bb::indices_t({(index_t)nodes}), BB_TYPE_FP32, true), tb((index_t)F, bb::indices_t({(index_t)nodes}), BB_TYPE_FP32, true);
+        put_fp32(yb, ys.data(), nodes, F);
+        put_fp32(tb, ts.data(), nodes, F);
+        bb::FrameBuffer dyb = lossFunc->CalculateLoss(yb, tb, (index_t)F);
+        get_fp32(dyb, ds.data(), nodes, F);
+        for (int n = 0; n < nodes; ++n) { std::memcpy(dy + ((size_t)n * batches + b) * F, &ds[(size_t)n * F], sizeof(float) * (size_t)F); }
+        metrics->CalculateMetrics(yb, tb);
+    }
+    *loss = lossFunc->GetLoss();
+    *metric = metrics->GetMetrics();
+    return 0;
 }

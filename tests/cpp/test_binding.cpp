@@ -92,6 +92,7 @@ SAME(&bbcu_fp32_DifferentiableLutN_Backward<>, decltype(&bbcu_fp32_Differentiabl
 // bbcu.h:768-796, 1076-1186, 1506-1572
 SAME(&bbcu_fp32_StochasticMaxPooling2x2_Forward, int (*)(float const *, float *, int, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_StochasticMaxPooling2x2_Backward, int (*)(float const *, float const *, float *, int, int, int, int, int, int, int, S));
+SAME(&bbcu_fp32_LossMeanSquaredError, int (*)(const float *, const float *, float *, double *, int, int, int, int, float, double, S));
 SAME(&bbcu_fp32_StochasticBatchNormalization_ForwardTraining, int (*)(float const *, float *, float *, float *, float *, float *, float, float, float, int, int, int, S));
 SAME(&bbcu_fp32_StochasticBatchNormalization_ReForward, int (*)(float const *, float *, float const *, float const *, float, float, int, int, int, S));
 SAME(&bbcu_fp32_StochasticBatchNormalization_ForwardInference, int (*)(float const *, float *, float const *, float const *, float, float, int, int, int, S));
@@ -166,7 +167,7 @@ static int run_on_gpu(void)
 
 int main(int argc, char **argv)
 {
-    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 11;
+    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11;
     if (argc > 1 && !std::strcmp(argv[1], "--gpu")) {
         if (!bbcu_IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
         int const bad = run_on_gpu();

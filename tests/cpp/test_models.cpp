@@ -18,6 +18,9 @@
 #include "bb/StochasticMaxPooling2x2.h"
 #include "bb/AverageLut.h"
 #include "bb/MaxLut.h"
+#include "bb/Reduce.h"
+#include "bb/LossMeanSquaredError.h"
+#include "bb/MetricsMeanSquaredError.h"
 #include "bb/LossSoftmaxCrossEntropy.h"
 #include "bb/MetricsCategoricalAccuracy.h"
 #include "bb/Convolution2d.h"
@@ -43,6 +46,10 @@ void oracle_fp32_StochasticBatchNormalization_ForwardInference(float const *x, f
 void oracle_fp32_StochasticBatchNormalization_Backward(float const *x, float const *dy, float *dx, float const *mean, float const *rstd, float gamma, int node_size, int frame_size, int frame_stride, int x_frame_stride);
 void oracle_fp32_MaxLut_Forward(float const *x, float *y, std::int32_t const *idx, int n, int node_size, int frame_size, int frame_stride, int binarize_input, int binarize_output);
 void oracle_fp32_MaxLut_Backward(float const *x, float const *dy, float *dx, std::int32_t const *idx, int n, int input_node_size, int output_node_size, int frame_size, int frame_stride, int binarize_input);
+void oracle_fp32_Reduce_Forward(float const *x, float *y, int input_node_size, int output_node_size, int frame_size, int frame_stride);
+void oracle_fp32_Reduce_Backward(float const *dy, float *dx, int input_node_size, int output_node_size, int frame_size, int frame_stride);
+void oracle_fp32_LossMeanSquaredError(float const *y, float const *t, float *dy, double *loss, int node_size, int frame_size, int frame_stride, float grad_reduction, double loss_reduction);
+void oracle_fp32_MetricsMeanSquaredError(float const *y, float const *t, double *accuracy, int node_size, int frame_size, int frame_stride);
 void oracle_bit_BinaryLut6_Forward(std::int32_t const *x, std::int32_t *y, std::int32_t const *idx, std::int32_t const *table, int node_size, int frame_size, int frame_stride);
 }
 
@@ -554,6 +561,58 @@ static void test_max_lut(void)
     CHECK(threw, "host_only MaxLut must throw");
 }
 
+// Reduce (output shape given, and derived from an integration size), then the mean-squared-error loss and metric over two batches
+static void test_reduce_and_mean_squared_error(void)
+{
+    int const I = 70, O = 10, F = 90;
+    std::mt19937_64 mt(17);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    auto fold = bb::Reduce<>::Create((bb::index_t)O);
+    auto fold7 = bb::Reduce<>::Create(bb::indices_t(), 7);
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), dy_buf(F, {O}, BB_TYPE_FP32), t_buf(F, {O}, BB_TYPE_FP32);
+    CHECK(fold->SetInputShape({I}) == bb::indices_t({O}) && fold7->SetInputShape({I}) == bb::indices_t({O}), "Reduce shapes");
+    auto loss = bb::LossMeanSquaredError<>::Create();
+    auto metric = bb::MetricsMeanSquaredError<>::Create();
+    double loss_ref = 0, metric_ref = 0;
+    std::vector<float> x, y, dy, dx, t, g, y_ref((size_t)O * F), dx_ref((size_t)I * F), g_ref((size_t)O * F);
+    for (int batch = 0; batch < 2; ++batch) {
+        for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, uni(mt)); }
+        for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dy_buf.SetFP32(f, n, uni(mt) - 0.5f); t_buf.SetFP32(f, n, (uni(mt) > 0.5f) ? 1.0f : 0.0f); }
+        read_fp32(x_buf, x); read_fp32(dy_buf, dy); read_fp32(t_buf, t);
+        bb::FrameBuffer y_buf = fold->Forward(x_buf);
+        bb::FrameBuffer y7_buf = fold7->Forward(x_buf);
+        bb::FrameBuffer dx_buf = fold->Backward(dy_buf);
+        read_fp32(y_buf, y); read_fp32(dx_buf, dx);
+        oracle_fp32_Reduce_Forward(x.data(), y_ref.data(), I, O, F, F);
+        oracle_fp32_Reduce_Backward(dy.data(), dx_ref.data(), I, O, F, F);
+        CHECK(max_diff(y, y_ref) == 0.0 && same_bits(y_buf, y7_buf), "Reduce forward differs by %g", max_diff(y, y_ref));
+        CHECK(max_diff(dx, dx_ref) == 0.0, "Reduce backward differs by %g", max_diff(dx, dx_ref));
+        bb::FrameBuffer g_buf = loss->CalculateLoss(y_buf, t_buf, F);
+        metric->CalculateMetrics(y_buf, t_buf);
+        read_fp32(g_buf, g);
+        oracle_fp32_LossMeanSquaredError(y.data(), t.data(), g_ref.data(), &loss_ref, O, F, F, 1.0f / (float)(O * F), 1.0 / O);
+        oracle_fp32_MetricsMeanSquaredError(y.data(), t.data(), &metric_ref, O, F, F);
+        CHECK(max_diff(g, g_ref) == 0.0, "mean squared error gradient differs by %g", max_diff(g, g_ref));
+    }
+    double const want_loss = loss_ref / (2.0 * F), want_metric = metric_ref / (2.0 * F);
+    CHECK(std::fabs(loss->GetLoss() - want_loss) <= 1e-12 * want_loss, "mean squared error loss %.17g vs %.17g", loss->GetLoss(), want_loss);
+    CHECK(std::fabs(metric->GetMetrics() - want_metric) <= 1e-12 * want_metric, "mean squared error metric %.17g vs %.17g", metric->GetMetrics(), want_metric);
+    loss->Clear(); metric->Clear();
+    auto sum_loss = bb::LossMeanSquaredError<>::Create("sum");
+    bb::FrameBuffer y_buf = fold->Forward(x_buf);
+    sum_loss->CalculateLoss(y_buf, t_buf, F);
+    double sum_ref = 0;
+    oracle_fp32_LossMeanSquaredError(y.data(), t.data(), g_ref.data(), &sum_ref, O, F, F, 1.0f, 1.0);
+    CHECK(std::fabs(sum_loss->GetLoss() - sum_ref) <= 1e-12 * sum_ref, "summed squared error %.17g vs %.17g", sum_loss->GetLoss(), sum_ref);
+    {
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        fold7->DumpObject(ss);
+        auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)again && again->GetObjectName() == "Reduce_fp32_fp32" && again->GetOutputNodeSize() == O, "Reduce reload");
+        if (again) { bb::FrameBuffer y3 = again->Forward(x_buf); CHECK(same_bits(y3, y_buf), "reloaded Reduce differs"); }
+    }
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -710,6 +769,7 @@ int main(void)
         test_convolution2d();
         test_stochastic_batch_normalization();
         test_max_lut();
+        test_reduce_and_mean_squared_error();
         test_tail();
         test_hand_off_through_files();
     }

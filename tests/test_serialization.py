@@ -319,3 +319,27 @@ def test_reference_average_lut_objects_load_and_survive_a_round_trip(tmp_path, k
     assert open(dst, "rb").read() == data
     assert np.array_equal(np.frombuffer(data[-4 * O * n:], np.int32).reshape(O, n), AVERAGE[p + "idx"])
     # (as for MaxLut, the reference's own loader does not list this type name: equal bytes are what its LoadObject would read)
+
+
+# ----------------------------------------------------------------------------------------------
+#  Reduce (include/bb/Reduce.h:287-317): objects written by the reference's class, fp32 and bit (tests/golden/reduce_mse.npz)
+# ----------------------------------------------------------------------------------------------
+REDUCE = np.load(os.path.join(HERE, "golden", "reduce_mse.npz"))
+
+
+@pytest.mark.parametrize("k", range(int(REDUCE["reduce_count"][0])))
+def test_reference_reduce_objects_load_and_survive_a_round_trip(tmp_path, k):
+    p = "r%d_" % k
+    I, O, F, integ = [int(v) for v in REDUCE[p + "geom"]]
+    name = REDUCE[p + "name"].tobytes().decode()
+    for key, type_name in (("object", "Reduce_fp32_fp32"), ("object_bit", "Reduce_bit_fp32")):
+        data = REDUCE[p + key].tobytes()
+        src, dst = str(tmp_path / (key + ".in")), str(tmp_path / (key + ".out"))
+        open(src, "wb").write(data)
+        out = tool("reload", src, dst).stdout.split()
+        assert out[0] == type_name and out[1] == (name if name else "Reduce")
+        assert (int(out[3]), int(out[5])) == (I, O)
+        assert open(dst, "rb").read() == data
+        if oracle.have_ref():                           # the reference's loader lists this type: it reads what was written here
+            back = oracle.ref_reload_container_object(np.frombuffer(open(dst, "rb").read(), np.uint8))
+            assert back is not None and back.tobytes() == data
