@@ -787,10 +787,19 @@ def bench_gather_ceiling(args, lib):
 
     kernel_ms = library_timed_ms(lib, step, max(args.steps, 20), max(args.warmup, 20))
     nbytes = I * (F // 128) * loads * 512
+    # the same bytes as longer or shorter row segments: the rate grows with the bytes per visited row until the window of all rows
+    # (4096 rows x segment) no longer fits the 4 MiB L2 of an XCD
+    by_segment = {}
+    for seg in (64, 128, 256, 512):
+        def seg_step(seg=seg):
+            capi.check(lib.bbhip_Probe_RowGatherSegments(ptr(x), ptr(sink), I, F, S, loads, seg, stream_ptr()))
+        ms = library_timed_ms(lib, seg_step, max(args.steps, 20), max(args.warmup, 20))
+        by_segment["%d B" % (seg * 4)] = round(I * (F // seg) * loads * seg * 4 / (ms * 1e-3) / 1e12, 2)
     return {"metric": "TB/s of gathered 512-byte row segments through L1 (access pattern of the dx kernel, no arithmetic)",
             "value": nbytes / (kernel_ms * 1e-3) / 1e12, "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 20),
             "ms_per_step": kernel_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": "row gather probe, 4096 rows x 8192 frames, 36 row segments per (row, 128 frames)", "bytes_per_launch": nbytes}}
+            "config": {"workload": "row gather probe, 4096 rows x 8192 frames, 36 row segments per (row, 128 frames)", "bytes_per_launch": nbytes,
+                       "TBps_by_segment_length": by_segment}}
 
 
 def other_configs(args, lib):

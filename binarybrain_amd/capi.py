@@ -35,6 +35,7 @@ _SIGNATURES = {
     "bbhip_GetScratchSize": (C.c_size_t, []),
     "bbhip_GetSwitch": (C.c_int, [C.c_char_p]),
     "bbhip_Probe_RowGather": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _vp]),
+    "bbhip_Probe_RowGatherSegments": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "bbhip_SetAverageLutMean": (None, [_i]),
     "bbhip_GetAverageLutMean": (C.c_int, []),
     "bbhip_SetDxMode": (None, [_i]),

@@ -1007,17 +1007,40 @@ int bbhip_GetSwitch(char const *name)
     return -1;
 }
 
-int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit, void *stream)
+static int launch_row_gather_probe(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
+                                   int segment_frames, void *stream, char const *name)
 {
-    BBHIP_REQUIRE(dev_x != nullptr && dev_sink != nullptr && row_count > 0 && frame_size > 0 && frame_stride >= frame_size && loads_per_unit > 0);
-    int const chunk_count = ceil_div(frame_size, 128), tile_count = ceil_div(row_count, kWavesPerBlk);
-    BBHIP_REQUIRE((long long)chunk_count * tile_count <= 0x7fffffffLL);
+    if (!(dev_x != nullptr && dev_sink != nullptr && row_count > 0 && frame_size > 0 && frame_stride >= frame_size && loads_per_unit > 0)) {
+        return fail("%s: rejected argument", name);
+    }
+    if (!(segment_frames == 64 || segment_frames == 128 || segment_frames == 256 || segment_frames == 512)) {
+        return fail("%s: segments are 64, 128, 256 or 512 frames long", name);
+    }
+    int const chunk_count = ceil_div(frame_size, segment_frames), tile_count = ceil_div(row_count, kWavesPerBlk);
+    if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("%s: grid too large", name); }
     hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 const grid((unsigned)(chunk_count * tile_count)), block(kBlock);
+    TileDivisor const tiles = make_tile_divisor(tile_count);
     ScopedTimer tm(kTimeOther, st);
-    hipLaunchKernelGGL(row_gather_probe_kernel, dim3(chunk_count * tile_count), dim3(kBlock), 0, st, dev_x, dev_sink, row_count, frame_stride,
-                       frame_size, chunk_count, make_tile_divisor(tile_count), loads_per_unit);
+    switch (segment_frames / kWave) {
+    case 1: hipLaunchKernelGGL(row_gather_probe_kernel<1>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
+    case 2: hipLaunchKernelGGL(row_gather_probe_kernel<2>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
+    case 4: hipLaunchKernelGGL(row_gather_probe_kernel<4>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
+    default: hipLaunchKernelGGL(row_gather_probe_kernel<8>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
+    }
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+
+int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit, void *stream)
+{
+    return launch_row_gather_probe(dev_x, dev_sink, row_count, frame_size, frame_stride, loads_per_unit, 128, stream, __func__);
+}
+
+int bbhip_Probe_RowGatherSegments(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
+                                  int segment_frames, void *stream)
+{
+    return launch_row_gather_probe(dev_x, dev_sink, row_count, frame_size, frame_stride, loads_per_unit, segment_frames, stream, __func__);
 }
 
 void bbhip_SetAverageLutMean(int mean) { g_average_lut_mean = mean != 0; }

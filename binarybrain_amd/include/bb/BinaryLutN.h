@@ -30,6 +30,7 @@ protected:
     {
         Model::CommandProc(args);
         if (args.size() == 2 && args[0] == "host_only") { m_host_only = EvalBool(args[1]); }
+        if (args.size() == 2 && args[0] == "host_simd") { m_host_simd = EvalBool(args[1]); }     // kept and serialized only
     }
 
 public:

@@ -318,7 +318,10 @@ public:
 
     FrameBuffer Backward(FrameBuffer dy_buf) override
     {
-        if (m_backward_break || dy_buf.Empty()) { return FrameBuffer(); }
+        if (m_backward_break || dy_buf.Empty()) {          // a frozen layer: no gradient of its own, none passed on (reference :1015-1018)
+            m_dW->FillZero();
+            return FrameBuffer();
+        }
         BB_ASSERT(dy_buf.GetType() == DataType<RealType>::type);
         RequireDevice("DifferentiableLutN::Backward");
         m_flagClamp = true;

@@ -40,6 +40,9 @@ protected:
         if (!kBitInput && args.size() == 2 && args[0] == "binary") { m_binary_mode = EvalBool(args[1]); }
         if (args.size() == 2 && args[0] == "lut_binarize")         { m_lut_binarize = EvalBool(args[1]); }
         if (args.size() == 2 && args[0] == "host_only")            { m_host_only = EvalBool(args[1]); }
+        // kept and serialized as in the reference (StochasticLutN.h:105-120), where no computation reads the first either
+        if (args.size() == 2 && args[0] == "y_binarize")           { m_y_binarize = EvalBool(args[1]); }
+        if (args.size() == 2 && args[0] == "host_simd")            { m_host_simd = EvalBool(args[1]); }
     }
 
     void RequireDevice(char const *what) const

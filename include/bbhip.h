@@ -121,6 +121,10 @@ int  bbhip_KernelTimer_Read(int which, float *total_ms, int *launches);
  * a measured ceiling next to the dx kernel's rate.  dev_sink: one float that is never written in practice. */
 int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
                           void *stream);
+/* The same with windows of segment_frames = 64, 128, 256 or 512 frames (row segments of 256 bytes to 2 KiB): how the rate that the
+ * GPU sustains depends on the bytes read per visited row, and where the window of all rows stops fitting an L2. */
+int bbhip_Probe_RowGatherSegments(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
+                                  int segment_frames, void *stream);
 
 /* ---- elementwise helpers ---- */
 /* bbcu_fp32_Vector_set, include/bbcu/bbcu.h:89-94 */

@@ -182,6 +182,12 @@ static void test_differentiable(int I, int O, int F, bool binary)
     CHECK(max_diff(rm_gpu, rm) <= 1e-5 && max_diff(rv_gpu, rv) <= 1e-5, "running statistics err %g %g", max_diff(rm_gpu, rm), max_diff(rv_gpu, rv));
     CHECK(max_diff(dx, dx_ref) <= 1e-4 * max_abs(dx_ref), "DifferentiableLut%d dx err %g of %g", N, max_diff(dx, dx_ref), max_abs(dx_ref));
     CHECK(max_diff(dW, dW_ref) <= 1e-4 * max_abs(dW_ref), "DifferentiableLut%d dW err %g of %g", N, max_diff(dW, dW_ref), max_abs(dW_ref));
+    // a frozen layer passes nothing back and holds no gradient of its own
+    lut->SendCommand("backward_break true");
+    lut->Forward(x_buf, true);
+    bb::FrameBuffer none = lut->Backward(dy_buf);
+    { auto p = lut->lock_dW_const(); for (size_t k = 0; k < dW.size(); ++k) { dW[k] = p[(bb::index_t)k]; } }
+    CHECK(none.Empty() && max_abs(dW) == 0.0, "backward_break: the layer must return an empty buffer and zero its table gradient");
 }
 
 static void test_binary(int I, int O, int F)
