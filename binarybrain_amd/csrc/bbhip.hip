@@ -1322,6 +1322,16 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
     return launch_pool(a, true, stream, __func__);
 }
 
+// The backward passes of AverageLut and MaxLut are input-centric.  A table that fits one LDS piece can be walked whole by every
+// wavefront (no reverse wiring, one launch instead of two); that costs table entries x wavefronts comparisons, so it is taken only
+// while that product stays below what the saved launch costs (the tail of a classifier at a training batch: 70 entries, 70 input
+// nodes, 1024 frames).  Both ways add in table order: the same bits.
+static bool walk_whole_table(int total, int input_node_size, int frame_size)
+{
+    if (total > kReversePiece) { return false; }
+    return (long long)total * input_node_size * ceil_div(frame_size, kWave) <= 131072LL;
+}
+
 static int check_average_lut(void const *a, void const *b, int const *idx, int n, int node_size, int frame_size, int frame_stride, int row_items,
                              char const *name)
 {
@@ -1390,11 +1400,18 @@ int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
     int const f_blocks = ceil_div(frame_stride, kTailBlock);
     long long const blocks = (long long)input_node_size * f_blocks;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    if (walk_whole_table(total, input_node_size, frame_size)) {
+        ScopedTimer tm(kTimeOther, st);
+        hipLaunchKernelGGL(average_lut_backward_small_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_dy_buf, dev_dx_buf, dev_input_index,
+                           total, n, frame_size, frame_stride, f_blocks);
+        BBHIP_LAUNCH_CHECK();
+        return 0;
+    }
     char *scratch = nullptr;
     size_t const offsets_bytes = align256(sizeof(int) * ((size_t)input_node_size + 1));
     if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch, static_cast<hipStream_t>(stream))) { return 1; }
     int *offsets = reinterpret_cast<int *>(scratch), *list = reinterpret_cast<int *>(scratch + offsets_bytes);
-    hipStream_t const st = static_cast<hipStream_t>(stream);
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(average_lut_reverse_kernel, dim3((unsigned)ceil_div(input_node_size + 1, kTailBlock)), dim3(kTailBlock), 0, st,
                        dev_input_index, total, n, input_node_size, offsets, list, 0);
@@ -1450,6 +1467,19 @@ static int launch_max_lut_backward(void const *x, bool bits, float const *dy, fl
     long long const blocks = (long long)input_node_size * f_blocks;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
     hipStream_t const st = static_cast<hipStream_t>(stream);
+    if (walk_whole_table(total, input_node_size, frame_size)) {
+        ScopedTimer tm(kTimeOther, st);
+        if (bits) {
+            hipLaunchKernelGGL(max_lut_backward_small_kernel<true>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, x, dy, dx, idx, total, n,
+                               frame_size, x_stride, dy_stride, 0, f_blocks);
+        }
+        else {
+            hipLaunchKernelGGL(max_lut_backward_small_kernel<false>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, x, dy, dx, idx, total, n,
+                               frame_size, x_stride, dy_stride, binarize_input, f_blocks);
+        }
+        BBHIP_LAUNCH_CHECK();
+        return 0;
+    }
     char *scratch = nullptr;
     size_t const offsets_bytes = align256(sizeof(int) * ((size_t)input_node_size + 1));
     if (arena_get(offsets_bytes + sizeof(int) * (size_t)total, &scratch, st)) { return 1; }
@@ -1602,8 +1632,14 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
         partial = reinterpret_cast<double *>(scratch);
     }
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
-    hipLaunchKernelGGL(softmax_cross_entropy_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_y_buf, dev_t_buf, dev_dy_buf, partial,
-                       t_sum, pix_size, ch_size, frame_size, frame_stride, f_blocks);
+    if (ch_size <= 16) {
+        hipLaunchKernelGGL(softmax_cross_entropy_few_kernel<16>, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_y_buf, dev_t_buf, dev_dy_buf,
+                           partial, t_sum, pix_size, ch_size, frame_size, frame_stride, f_blocks);
+    }
+    else {
+        hipLaunchKernelGGL(softmax_cross_entropy_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, st, dev_y_buf, dev_t_buf, dev_dy_buf, partial,
+                           t_sum, pix_size, ch_size, frame_size, frame_stride, f_blocks);
+    }
     BBHIP_LAUNCH_CHECK();
     if (pix_size > 1) {
         hipLaunchKernelGGL(loss_pixel_sum_kernel, dim3((unsigned)f_blocks), dim3(kTailBlock), 0, st, partial, dev_loss_buf, pix_size, frame_size);

@@ -162,6 +162,27 @@ __global__ __launch_bounds__(kTailBlock) void average_lut_backward_kernel(float 
     dx[(size_t)in * frame_stride + f] = acc;
 }
 
+// The same for a table of at most kReversePiece entries, without the reverse wiring: every workgroup (one input node, kTailBlock
+// columns) stages the whole table in LDS and walks it in table order; the comparison is the same for all its threads.  For the
+// tails of classifiers (tens of entries) this saves the launch that builds the reverse wiring, which costs more than the walk.
+__global__ __launch_bounds__(kTailBlock) void average_lut_backward_small_kernel(float const *dy, float *dx, int const *__restrict__ idx, int total,
+                                                                                int n, int frame_size, int frame_stride, int f_blocks)
+{
+    __shared__ __attribute__((aligned(16))) int piece[kReversePiece];
+    stage_piece(piece, idx, total);
+    __syncthreads();
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const in = blockIdx.x / f_blocks;
+    if (f >= frame_stride) { return; }
+    if (f >= frame_size) { dx[(size_t)in * frame_stride + f] = 0.0f; return; }
+    float const fn = (float)n;
+    float acc = 0.0f;
+    for (int k = 0; k < total; ++k) {
+        if (piece[k] == in) { acc += dy[(size_t)(k / n) * frame_stride + f] / fn; }
+    }
+    dx[(size_t)in * frame_stride + f] = acc;
+}
+
 // MaxLut: the largest of the n wired inputs, starting from -1 and replaced by strictly larger values only (reference host
 // loop: include/bb/MaxLut.h:293-318); binarize_input as in the reference's device kernel (cuda/MaxLut.cu:33-36).
 // One thread per (output node, frame).
@@ -198,6 +219,31 @@ __global__ __launch_bounds__(kTailBlock) void max_lut_forward_bit_kernel(int con
 // One thread per (input node, column of the dx row pitch): over the table positions that name this input, in table order, add
 // the node's dy where this position holds the node's first largest input (include/bb/MaxLut.h:394-424).  BITS: x is packed, the
 // first largest input is the first one that is set (position 0 when none is).
+// the position of a node's first largest input at frame f (BITS: the first input that is set; position 0 when none is)
+template <bool BITS>
+__device__ __forceinline__ int max_lut_winner(void const *x_buf, int const *row, int n, int f, int x_stride, int binarize_input)
+{
+    int first = 0;
+    if (BITS) {
+        uint32_t const *xb = static_cast<uint32_t const *>(x_buf);
+        for (int i = 0; i < n; ++i) {
+            if ((xb[(size_t)row[i] * x_stride + (f >> 5)] >> (f & 31)) & 1u) { first = i; break; }
+        }
+    }
+    else {
+        float const *xf = static_cast<float const *>(x_buf);
+        float max_val = -1.0f;
+        for (int i = 0; i < n; ++i) {
+            float v = xf[(size_t)row[i] * x_stride + f];
+            if (binarize_input) { v = (v > 0.0f) ? 1.0f : -1.0f; }
+            if (v > max_val) { max_val = v; first = i; }
+        }
+    }
+    return first;
+}
+
+// One thread per (input node, column of the dx row pitch): over the table positions that name this input, in table order, add
+// the node's dy where this position holds the node's first largest input (include/bb/MaxLut.h:394-424).
 template <bool BITS>
 __global__ __launch_bounds__(kTailBlock) void max_lut_backward_kernel(void const *x_buf, float const *dy, float *dx, int const *idx,
                                                                       int const *offsets, int const *list, int n, int frame_size,
@@ -211,24 +257,29 @@ __global__ __launch_bounds__(kTailBlock) void max_lut_backward_kernel(void const
     float acc = 0.0f;
     for (int k = begin; k < end; ++k) {
         int const entry = list[k], node = entry / n, pos = entry - node * n;
-        int const *row = idx + (size_t)node * n;
-        int first = 0;
-        if (BITS) {
-            uint32_t const *xb = static_cast<uint32_t const *>(x_buf);
-            for (int i = 0; i < n; ++i) {
-                if ((xb[(size_t)row[i] * x_stride + (f >> 5)] >> (f & 31)) & 1u) { first = i; break; }
-            }
-        }
-        else {
-            float const *xf = static_cast<float const *>(x_buf);
-            float max_val = -1.0f;
-            for (int i = 0; i < n; ++i) {
-                float v = xf[(size_t)row[i] * x_stride + f];
-                if (binarize_input) { v = (v > 0.0f) ? 1.0f : -1.0f; }
-                if (v > max_val) { max_val = v; first = i; }
-            }
-        }
-        if (first == pos) { acc += dy[(size_t)node * dy_stride + f]; }
+        if (max_lut_winner<BITS>(x_buf, idx + (size_t)node * n, n, f, x_stride, binarize_input) == pos) { acc += dy[(size_t)node * dy_stride + f]; }
+    }
+    dx[(size_t)in * dy_stride + f] = acc;
+}
+
+// the same for a table of at most kReversePiece entries, walked from LDS without the reverse wiring (see average_lut_backward_small_kernel)
+template <bool BITS>
+__global__ __launch_bounds__(kTailBlock) void max_lut_backward_small_kernel(void const *x_buf, float const *dy, float *dx, int const *__restrict__ idx,
+                                                                            int total, int n, int frame_size, int x_stride, int dy_stride,
+                                                                            int binarize_input, int f_blocks)
+{
+    __shared__ __attribute__((aligned(16))) int piece[kReversePiece];
+    stage_piece(piece, idx, total);
+    __syncthreads();
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const in = blockIdx.x / f_blocks;
+    if (f >= dy_stride) { return; }
+    if (f >= frame_size) { dx[(size_t)in * dy_stride + f] = 0.0f; return; }
+    float acc = 0.0f;
+    for (int k = 0; k < total; ++k) {
+        if (piece[k] != in) { continue; }
+        int const node = k / n, pos = k - node * n;
+        if (max_lut_winner<BITS>(x_buf, piece + node * n, n, f, x_stride, binarize_input) == pos) { acc += dy[(size_t)node * dy_stride + f]; }
     }
     dx[(size_t)in * dy_stride + f] = acc;
 }
@@ -336,6 +387,50 @@ __global__ __launch_bounds__(kTailBlock) void softmax_cross_entropy_kernel(float
         float const softmax = expf(y[at] - c) / y_sum;
         if (tv > 0.0f) { loss += (double)rounded_mul(logf(softmax + eps), t_max); }
         dy[at] = (rounded_mul(t_max, softmax) - tv) / t_sum;
+    }
+    partial[(size_t)pix * frame_size + f] = loss;
+}
+
+// The same arithmetic for at most CH channels with every y and t of the (pixel, frame) loaded first: the loads of the three passes
+// above depend on nothing, but issued one pass after the other their latencies add up, which is what a small batch pays for.
+template <int CH>
+__global__ __launch_bounds__(kTailBlock) void softmax_cross_entropy_few_kernel(float const *y, float const *t, float *dy, double *partial,
+                                                                               float t_sum, int pix_size, int ch_size, int frame_size,
+                                                                               int frame_stride, int f_blocks)
+{
+    int const f = (int)(blockIdx.x % f_blocks) * kTailBlock + threadIdx.x;
+    int const pix = blockIdx.x / f_blocks;
+    if (f >= frame_size) { return; }
+    float const eps = 1.0e-7f;
+    size_t const node_step = (size_t)pix_size * frame_stride;
+    size_t const first = (size_t)pix * frame_stride + f;
+    float yv[CH], tv[CH];
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+        yv[ch] = (ch < ch_size) ? y[first + ch * node_step] : 0.0f;
+        tv[ch] = (ch < ch_size) ? t[first + ch * node_step] : 0.0f;
+    }
+    float c = -3.402823466e+38f;
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) { if (ch < ch_size) { c = (c < yv[ch]) ? yv[ch] : c; } }
+    float y_sum = 0.0f, t_max = 0.0f;
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+        if (ch < ch_size) {
+            yv[ch] = expf(yv[ch] - c);
+            y_sum += yv[ch];
+            t_max += tv[ch];
+        }
+    }
+    if (y_sum <= eps) { y_sum = eps; }
+    double loss = 0.0;
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+        if (ch < ch_size) {
+            float const softmax = yv[ch] / y_sum;
+            if (tv[ch] > 0.0f) { loss += (double)rounded_mul(logf(softmax + eps), t_max); }
+            dy[first + ch * node_step] = (rounded_mul(t_max, softmax) - tv[ch]) / t_sum;
+        }
     }
     partial[(size_t)pix * frame_size + f] = loss;
 }
