@@ -1198,10 +1198,11 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
 //  and step instead of the polynomial's 43.  Units, work list and the dW rider are those of lut_dx_kernel; fp32 rows are
 //  loaded as there and compared with 0.5, packed rows take one load per row and pass (see below).
 // ------------------------------------------------------------------------------------------------
-template <int N, int XMODE, int U>
+template <int N, int XMODE, int U, bool WIDE = false>
 __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
 {
     static_assert(XMODE == kXBit || XMODE == kXBinary, "corner values need two-valued inputs");
+    static_assert(!WIDE || XMODE == kXBit, "scalar loads of whole passes are for packed rows");
     using T = DxTerm<N, XMODE, U>;
     int const bid = blockIdx.x;
     int const B   = a.chunk_count * a.tiles.count;
@@ -1234,41 +1235,105 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
 
-        // packed rows: the head (row addresses) and the value table of the next term are requested while the current term
-        // is evaluated — this path is bound by the round trips of a term, not by its instructions
-        int head_next[2 * T::M + 2], values_next = 0;
+        // Packed rows: a term is a round trip — its head (row addresses, scalar loads), then the rows' words and dy — and a few
+        // dozen instructions, so the walk is bound by latency.  Two terms are in flight: while term t is evaluated, the rows of
+        // term t + 1 have been requested and the head of term t + 2 is on its way.
         if constexpr (XMODE == kXBit) {
-            if (t_begin < t_end) {
+            // The 64 U frames of a pass are 2 U words of a packed row, the same for every lane: one load per row brings them
+            // in (lane i holds word i of the pass), each step's two words are read back as a lane mask, and the index costs
+            // one add-with-carry per input.  Per term and pass: M + U + 1 vector memory instructions instead of (M + 1) U + 1.
+            constexpr int HEAD = 2 * T::M + 2;
+            int head[HEAD];
+            uint32_t w_next[T::M];
+            float dy_next[U];
+            int values_next = 0;
+            auto load_head = [&](int t) {
 #pragma unroll
-                for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[(size_t)t_begin * T::REC + i]; }
-                values_next = rec_v[(size_t)t_begin * T::REC];
-            }
-        }
-        for (int t = t_begin; t < t_end; ++t) {
-            if constexpr (XMODE == kXBit) {
-                int r[2 * T::M + 2];
-#pragma unroll
-                for (int i = 0; i < 2 * T::M + 2; ++i) { r[i] = head_next[i]; }
-                int const values = values_next;                    // lane p: the term's value at corner p
-                if (t + 1 < t_end) {
-#pragma unroll
-                    for (int i = 0; i < 2 * T::M + 2; ++i) { head_next[i] = rec[(size_t)(t + 1) * T::REC + i]; }
-                    values_next = rec_v[(size_t)(t + 1) * T::REC];
-                }
-                // The 64 U frames of a pass are 2 U words of a packed row, the same for every lane: one load per row
-                // brings them in (lane i holds word i of the pass), each step's two words are read back as a lane mask,
-                // and the index costs one add-with-carry per input.  Per term and pass: M + U + 1 vector memory
-                // instructions instead of (M + 1) U + 1.
-                uint32_t w[T::M];
+                for (int i = 0; i < HEAD; ++i) { head[i] = rec[(size_t)t * T::REC + i]; }
+            };
+            auto request_rows = [&](int t) {                      // of the term whose head is in `head`
 #pragma unroll
                 for (int j = 0; j < T::M; ++j) {
-                    __amdgpu_buffer_rsrc_t const d = address_descriptor((uint32_t)r[2 * j], (uint32_t)r[2 * j + 1], x_row_bytes);
-                    w[j] = __builtin_amdgcn_raw_buffer_load_b32(d, wordoff, 0, 0);
+                    __amdgpu_buffer_rsrc_t const d = address_descriptor((uint32_t)head[2 * j], (uint32_t)head[2 * j + 1], x_row_bytes);
+                    w_next[j] = __builtin_amdgcn_raw_buffer_load_b32(d, wordoff, 0, 0);
                 }
-                __amdgpu_buffer_rsrc_t const dyr = address_descriptor((uint32_t)r[2 * T::M], (uint32_t)r[2 * T::M + 1], y_row_bytes);
+                __amdgpu_buffer_rsrc_t const dyr = address_descriptor((uint32_t)head[2 * T::M], (uint32_t)head[2 * T::M + 1], y_row_bytes);
+#pragma unroll
+                for (int u = 0; u < U; ++u) { dy_next[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0)); }
+                values_next = rec_v[(size_t)t * T::REC];        // lane p: the term's value at corner p
+            };
+            if constexpr (WIDE) {
+                // Row pitch a multiple of 2 U words: the 2 U words of a pass are ONE scalar load per row (32 bytes with U = 4), each
+                // step's lane mask is a register pair of it, and the 2 M U read-lanes of the form below go away (a third of this
+                // kernel's instructions).  A term's corner indices are formed one term ahead, as soon as its words are there,
+                // so only the head of term t + 2 and the words of term t + 1 sit in scalar registers.
+                typedef uint32_t u32x8 __attribute__((ext_vector_type(2 * U)));
+                typedef __attribute__((address_space(4))) u32x8 const const_u32x8;
+                uint32_t index_next[U];
+                auto request_wide = [&](int t) {                  // of the term whose head is in `head`: its indices, dy, values
+                    u32x8 wq[T::M];
+#pragma unroll
+                    for (int j = 0; j < T::M; ++j) {
+                        uint64_t const row = ((uint64_t)(uint32_t)head[2 * j + 1] << 32) | (uint32_t)head[2 * j];
+                        wq[j] = *(const_u32x8 *)(row + (uint64_t)(uint32_t)(f_begin >> 5) * 4u);
+                    }
+                    __amdgpu_buffer_rsrc_t const dyr = address_descriptor((uint32_t)head[2 * T::M], (uint32_t)head[2 * T::M + 1], y_row_bytes);
+#pragma unroll
+                    for (int u = 0; u < U; ++u) { dy_next[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0)); }
+                    values_next = rec_v[(size_t)t * T::REC];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        uint32_t index = 0;                        // most significant input first: index = 2 index + bit
+#pragma unroll
+                        for (int j = T::M - 1; j >= 0; --j) {
+                            uint64_t const mask = (uint64_t)wq[j][2 * u] | ((uint64_t)wq[j][2 * u + 1] << 32);
+                            uint64_t carry;
+                            asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(index), "=s"(carry) : "v"(index), "s"(mask));
+                        }
+                        index_next[u] = index << 2;
+                    }
+                };
+                if (t_begin < t_end) {
+                    load_head(t_begin);
+                    request_wide(t_begin);
+                    if (t_begin + 1 < t_end) { load_head(t_begin + 1); }
+                }
+                for (int t = t_begin; t < t_end; ++t) {
+                    uint32_t idx4[U];
+                    float dyv[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) { idx4[u] = index_next[u]; dyv[u] = dy_next[u]; }
+                    int const values = values_next;
+                    if (t + 1 < t_end) {
+                        request_wide(t + 1);
+                        if (t + 2 < t_end) { load_head(t + 2); }
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)idx4[u], values));
+                        acc[u] = __builtin_fmaf(dyv[u], d, acc[u]);
+                    }
+                }
+                dx_store_pass<U>(a, part, in, wave, lane, f_begin, acc);
+                continue;
+            }
+            if (t_begin < t_end) {
+                load_head(t_begin);
+                request_rows(t_begin);
+                if (t_begin + 1 < t_end) { load_head(t_begin + 1); }
+            }
+            for (int t = t_begin; t < t_end; ++t) {
+                uint32_t w[T::M];
                 float dyv[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u) { dyv[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0)); }
+                for (int j = 0; j < T::M; ++j) { w[j] = w_next[j]; }
+#pragma unroll
+                for (int u = 0; u < U; ++u) { dyv[u] = dy_next[u]; }
+                int const values = values_next;
+                if (t + 1 < t_end) {
+                    request_rows(t + 1);
+                    if (t + 2 < t_end) { load_head(t + 2); }
+                }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     uint32_t index = 0;                            // most significant input first: index = 2 index + bit
@@ -1282,8 +1347,11 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
                     float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), values));
                     acc[u] = __builtin_fmaf(dyv[u], d, acc[u]);
                 }
-                continue;
             }
+            dx_store_pass<U>(a, part, in, wave, lane, f_begin, acc);
+            continue;
+        }
+        for (int t = t_begin; t < t_end; ++t) {
             int const values = rec_v[(size_t)t * T::REC];          // lane p: the term's value at corner p
             typename T::Stage st;
             T::issue(rec + (size_t)t * T::REC, xoff, yoff, x_row_bytes, y_row_bytes, st);
