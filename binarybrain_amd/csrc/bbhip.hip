@@ -120,6 +120,7 @@ bool use_corner_values(int xmode)
 bool pack_binarized_input(void) { static bool const on = env_switch("BBHIP_PACK", true); return on; }
 // packed rows in the dx kernel read with one scalar load per row and pass where pitch and alignment allow (0 = vector loads + read-lanes)
 bool dx_wide_rows(void) { static bool const on = env_switch("BBHIP_DX_WIDE", true); return on; }
+int dx_wide_max_rows(void) { static int const v = env_int("BBHIP_DX_WIDE_ROWS", 1024); return v; }
 
 // frames per unit; both are rounded to wavefront multiples where used
 int fwd_nodes_per_wave(void) { static int v = env_int("BBHIP_FWD_NODES", 2); return v >= 2 ? 2 : 1; }
@@ -732,10 +733,11 @@ int run_backward(BackwardCall const &call, hipStream_t st)
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
         d.chunk = chunk; d.chunk_count = chunk_count; d.tiles = make_tile_divisor(in_tiles);
         d.bias = c.bias; d.split = split ? 1 : 0;
-        // Packed rows with few input nodes (the layers of a convolution: tens of channels, very many frames): the words of a pass are
-        // read with one scalar load per row — the rows then stay in the scalar cache; with thousands of rows they do not, and
-        // the vector loads are faster (4096 rows: 385 vs 319 us per step).
-        bool const wide = bit_corner && dx_wide_rows() && steps == 4 && c.input_node_size <= 256 && c.x_stride % 8 == 0 &&
+        // Packed rows with up to about a thousand input nodes (the layers of a convolution: tens to hundreds of channels x taps, very
+        // many frames): the words of a pass are read with one scalar load per row — the rows then stay in the scalar cache.  With
+        // more rows they do not, and the vector loads are faster (dx kernel at 324 / 512 / 1024 / 2048 rows: 94 / 107 / 138 / 141 us
+        // against 104 / 127 / 147 / 135 us; 4096 rows: 385 against 319 us per step).
+        bool const wide = bit_corner && dx_wide_rows() && steps == 4 && c.input_node_size <= dx_wide_max_rows() && c.x_stride % 8 == 0 &&
                           (reinterpret_cast<uintptr_t>(c.x) % 32u) == 0;
         // folding the slab sums into dW rides at the end of this launch
         d.fin_partial = part; d.fin_dW = c.dW; d.fin_node_size = c.output_node_size; d.fin_slab_count = slab_total;
