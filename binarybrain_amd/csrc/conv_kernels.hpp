@@ -67,22 +67,29 @@ __global__ __launch_bounds__(kConvBlock) void im2col_forward_kernel(Im2ColArgs a
     float const *x = static_cast<float const *>(a.x);
     float *y = static_cast<float *>(a.y);
 
-    for (int i = wave; i < kTile; i += kConvBlock / 64) {
-        int const q = q0 + i;
-        if (q >= plane) { break; }
-        int const oy = q / a.ow, ox = q - oy * a.ow;
-        int iy, ix;
-        bool const have = im2col_source(a, oy, ox, fy, fx, iy, ix);      // wave-uniform
-        float v = a.border_value;
-        if (have && f0 + lane < a.input_frame_size) {
-            v = x[((size_t)(c * a.h + iy) * a.w + ix) * a.input_frame_stride + f0 + lane];
+    // all loads of a wavefront's 16 rows are issued before the first of them is used (one round trip instead of sixteen)
+    constexpr int kRows = kTile / (kConvBlock / 64);
+    float v[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        int const q = q0 + wave + r * (kConvBlock / 64);
+        v[r] = a.border_value;
+        if (q < plane) {
+            int const oy = q / a.ow, ox = q - oy * a.ow;
+            int iy, ix;
+            bool const have = im2col_source(a, oy, ox, fy, fx, iy, ix);  // wave-uniform
+            if (have && f0 + lane < a.input_frame_size) {
+                v[r] = x[((size_t)(c * a.h + iy) * a.w + ix) * a.input_frame_stride + f0 + lane];
+            }
         }
-        tile[i][lane] = v;
     }
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) { tile[wave + r * (kConvBlock / 64)][lane] = v[r]; }
     __syncthreads();
-    for (int f = wave; f < kTile; f += kConvBlock / 64) {
-        if (f0 + f >= a.input_frame_size) { break; }
-        if (q0 + lane < plane) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        int const f = wave + r * (kConvBlock / 64);
+        if (f0 + f < a.input_frame_size && q0 + lane < plane) {
             y[(size_t)node * a.output_frame_stride + (size_t)(f0 + f) * plane + q0 + lane] = tile[lane][f];
         }
     }
@@ -186,22 +193,37 @@ __global__ __launch_bounds__(kConvBlock) void col2im_kernel(float const *__restr
     int const c = b;
     int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int const f0 = ft * kTile, xy0 = xt * kTile;
+    // all loads of a wavefront's 16 rows are issued before the first of them is used (one round trip instead of sixteen)
+    constexpr int kStep = kConvBlock / 64, kRows = kTile / kStep;
+    float v[kRows];
     if (FORWARD) {
-        for (int f = wave; f < kTile && f0 + f < frames; f += kConvBlock / 64) {          // lanes along xy: contiguous in src
-            if (xy0 + lane < hw) { tile[f][lane] = src[(size_t)c * narrow_stride + (size_t)(f0 + f) * hw + xy0 + lane]; }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {                                                  // lanes along xy: contiguous in src
+            int const f = wave + r * kStep;
+            v[r] = (f0 + f < frames && xy0 + lane < hw) ? src[(size_t)c * narrow_stride + (size_t)(f0 + f) * hw + xy0 + lane] : 0.0f;
         }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) { tile[wave + r * kStep][lane] = v[r]; }
         __syncthreads();
-        for (int i = wave; i < kTile && xy0 + i < hw; i += kConvBlock / 64) {             // lanes along frames: contiguous in dst
-            if (f0 + lane < frames) { dst[((size_t)c * hw + xy0 + i) * wide_stride + f0 + lane] = tile[lane][i]; }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {                                                  // lanes along frames: contiguous in dst
+            int const i = wave + r * kStep;
+            if (xy0 + i < hw && f0 + lane < frames) { dst[((size_t)c * hw + xy0 + i) * wide_stride + f0 + lane] = tile[lane][i]; }
         }
     }
     else {
-        for (int i = wave; i < kTile && xy0 + i < hw; i += kConvBlock / 64) {
-            if (f0 + lane < frames) { tile[i][lane] = src[((size_t)c * hw + xy0 + i) * wide_stride + f0 + lane]; }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+            int const i = wave + r * kStep;
+            v[r] = (xy0 + i < hw && f0 + lane < frames) ? src[((size_t)c * hw + xy0 + i) * wide_stride + f0 + lane] : 0.0f;
         }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) { tile[wave + r * kStep][lane] = v[r]; }
         __syncthreads();
-        for (int f = wave; f < kTile && f0 + f < frames; f += kConvBlock / 64) {
-            if (xy0 + lane < hw) { dst[(size_t)c * narrow_stride + (size_t)(f0 + f) * hw + xy0 + lane] = tile[lane][f]; }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+            int const f = wave + r * kStep;
+            if (f0 + f < frames && xy0 + lane < hw) { dst[(size_t)c * narrow_stride + (size_t)(f0 + f) * hw + xy0 + lane] = tile[lane][f]; }
         }
     }
 }
