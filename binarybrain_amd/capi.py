@@ -6,7 +6,7 @@ from .build import LIB_PATH
 
 _lib = None
 
-_vp, _i, _f = C.c_void_p, C.c_int, C.c_float
+_vp, _i, _f, _u = C.c_void_p, C.c_int, C.c_float, C.c_uint
 
 _SIGNATURES = {
     "bbhip_GetDeviceCount": (C.c_int, []),
@@ -80,6 +80,15 @@ _SIGNATURES = {
     "bbhip_fp32_StochasticBatchNormalization_ReForward": (C.c_int, [_vp] * 4 + [_f, _f, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticBatchNormalization_ForwardInference": (C.c_int, [_vp] * 4 + [_f, _f, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticBatchNormalization_Backward": (C.c_int, [_vp] * 5 + [_f, _f, _i, _i, _i, _i, _vp]),
+    "bbhip_fp32_RealToBinary_Forward": (C.c_int, [_vp, _vp, _u, _u, _f, _f] + [_u] * 5 + [_i, _vp]),
+    "bbhip_fp32_bit_RealToBinary_Forward": (C.c_int, [_vp, _vp, _u, _u, _f, _f] + [_u] * 5 + [_i, _vp]),
+    "bbhip_fp32_BinaryToReal_Forward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_bit_fp32_BinaryToReal_Forward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_fp32_BinaryToReal_Backward": (C.c_int, [_vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_fp32_Binarize_Forward": (C.c_int, [_vp, _vp, _f, _f, _f, _i, _i, _i, _vp]),
+    "bbhip_fp32_bit_Binarize_Forward": (C.c_int, [_vp, _vp, _f, _i, _i, _i, _i, _vp]),
+    "bbhip_fp32_HardTanh_Forward": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _vp]),
+    "bbhip_fp32_HardTanh_Backward": (C.c_int, [_vp, _vp, _vp, _f, _f, _i, _i, _i, _vp]),
     "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "bbhip_fp32_StochasticLut_Forward_NoAlloc": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),

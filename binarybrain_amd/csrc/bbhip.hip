@@ -18,6 +18,7 @@
 #include "conv_kernels.hpp"
 #include "tail_kernels.hpp"
 #include "bn_kernels.hpp"
+#include "modulation_kernels.hpp"
 
 using namespace bbhip;
 
@@ -1792,6 +1793,220 @@ int bbhip_fp32_StochasticBatchNormalization_Backward(float const *dev_x_buf, flo
     a.gamma = gamma; a.reciprocal_frame_size = reciprocal_frame_size;
     a.frame_size = frame_size; a.x_stride = x_frame_stride; a.out_stride = frame_stride;
     return launch_bn_rows(a, node_size, true, stream);
+}
+
+// ---- RealToBinary, BinaryToReal, Binarize, HardTanh ----
+// `wide`: four frames per thread with 128-bit accesses; f_blocks = workgroups per row
+static int modulation_grid(int rows, int frame_size, bool wide, TileDivisor &f_blocks, unsigned &blocks, char const *name)
+{
+    int const per_row = ceil_div(frame_size, kModBlock * (wide ? 4 : 1));
+    long long const total = (long long)rows * per_row;
+    if (total > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    f_blocks = make_tile_divisor(per_row);
+    blocks = (unsigned)total;
+    return 0;
+}
+
+static int launch_row_map(int op, float const *x, float const *dy, float *out, float p0, float p1, float p2, int node_size, int frame_size,
+                          int frame_stride, void *stream, char const *name)
+{
+    if (!(x && out && (dy || op != kMapHardTanhBackward))) { return fail("%s: null buffer", name); }
+    if (!(node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", name); }
+    RowMapArgs a{};
+    a.x = x; a.dy = dy; a.out = out; a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    a.p0 = p0; a.p1 = p1; a.p2 = p2;
+    bool const wide = bn_rows_aligned(x, dy ? dy : x, out, frame_stride, frame_stride);
+    unsigned blocks;
+    if (modulation_grid(node_size, frame_size, wide, a.f_blocks, blocks, name)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    dim3 const grid(blocks), block(kModBlock);
+#define BBHIP_ROW_MAP(OP)                                                                               \
+    do {                                                                                                \
+        if (wide) { hipLaunchKernelGGL((row_map_kernel<OP, 4>), grid, block, 0, st, a); }               \
+        else      { hipLaunchKernelGGL((row_map_kernel<OP, 1>), grid, block, 0, st, a); }               \
+    } while (0)
+    switch (op) {
+    case kMapBinarize:  BBHIP_ROW_MAP(kMapBinarize); break;
+    case kMapHardTanh:  BBHIP_ROW_MAP(kMapHardTanh); break;
+    default:            BBHIP_ROW_MAP(kMapHardTanhBackward); break;
+    }
+#undef BBHIP_ROW_MAP
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_Binarize_Forward(float const *dev_x_buf, float *dev_y_buf, float binary_th, float binary_low, float binary_high,
+                                int node_size, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_row_map(kMapBinarize, dev_x_buf, nullptr, dev_y_buf, binary_th, binary_low, binary_high, node_size, frame_size, frame_stride,
+                          stream, __func__);
+}
+
+int bbhip_fp32_bit_Binarize_Forward(float const *dev_x_buf, int *dev_y_buf, float binary_th, int node_size, int frame_size,
+                                    int x_frame_stride, int y_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (!(dev_x_buf && dev_y_buf)) { return fail("%s: null buffer", __func__); }
+    if (!(node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
+    if (x_frame_stride < frame_size || y_frame_stride < (frame_size + 31) / 32) { return fail("%s: frame stride shorter than the frames", __func__); }
+    bool const wide = bn_rows_aligned(dev_x_buf, dev_x_buf, dev_x_buf, x_frame_stride, x_frame_stride);
+    TileDivisor f_blocks;
+    unsigned blocks;
+    if (modulation_grid(node_size, frame_size, wide, f_blocks, blocks, __func__)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    uint32_t *const y = reinterpret_cast<uint32_t *>(dev_y_buf);
+    if (wide) { hipLaunchKernelGGL((binarize_bits_kernel<4>), dim3(blocks), dim3(kModBlock), 0, st, dev_x_buf, y, binary_th, frame_size, x_frame_stride, y_frame_stride, f_blocks); }
+    else      { hipLaunchKernelGGL((binarize_bits_kernel<1>), dim3(blocks), dim3(kModBlock), 0, st, dev_x_buf, y, binary_th, frame_size, x_frame_stride, y_frame_stride, f_blocks); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_HardTanh_Forward(float const *dev_x_buf, float *dev_y_buf, float limit_min, float limit_max, int node_size, int frame_size,
+                                int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_row_map(kMapHardTanh, dev_x_buf, nullptr, dev_y_buf, limit_min, limit_max, 0.0f, node_size, frame_size, frame_stride, stream, __func__);
+}
+
+int bbhip_fp32_HardTanh_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, float limit_min, float limit_max,
+                                 int node_size, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_row_map(kMapHardTanhBackward, dev_x_buf, dev_dy_buf, dev_dx_buf, limit_min, limit_max, 0.0f, node_size, frame_size, frame_stride,
+                          stream, __func__);
+}
+
+static int launch_real_to_binary(float const *x, void *y, bool bit, unsigned depth_modulation_size, unsigned frame_modulation_size,
+                                 float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size, unsigned x_frame_size,
+                                 unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream, char const *name)
+{
+    if (!(x && y)) { return fail("%s: null buffer", name); }
+    if (!(depth_modulation_size > 0 && frame_modulation_size > 0 && point_size > 0 && x_depth_size > 0 && x_frame_size > 0)) {
+        return fail("%s: sizes must be positive", name);
+    }
+    long long const y_frames = (long long)x_frame_size * frame_modulation_size;
+    long long const y_nodes = (long long)x_depth_size * depth_modulation_size * point_size;
+    if (y_frames > 0x7fffffffLL || y_nodes > 0x7fffffffLL) { return fail("%s: output too large", name); }
+    if (x_frame_stride < x_frame_size || (long long)y_frame_stride < (bit ? (y_frames + 31) / 32 : y_frames)) {
+        return fail("%s: frame stride shorter than the frames", name);
+    }
+    RealToBinaryArgs a{};
+    a.x = x; a.y = y;
+    a.x_frame_size = (int)x_frame_size; a.y_frame_size = (int)y_frames; a.x_stride = (int)x_frame_stride; a.y_stride = (int)y_frame_stride;
+    a.point_size = (int)point_size; a.depth_modulation_size = (int)depth_modulation_size;
+    a.lo = input_range_lo; a.x_scale = 1.0f / (input_range_hi - input_range_lo);
+    a.depth_step = 1.0f / (float)depth_modulation_size; a.depth_step_recip = (float)depth_modulation_size;
+    a.frame_step = 1.0f / (float)frame_modulation_size; a.frame_step_recip = (float)frame_modulation_size;
+    a.binarize = binarize; a.threshold = binarize ? 0.5f : 0.0f;
+    a.frame_modulation = make_tile_divisor((int)frame_modulation_size);
+    // packed rows are assembled from whole threads either way; fp32 rows need 16-byte rows for the wide stores
+    bool const wide = bit || ((reinterpret_cast<uintptr_t>(y) & 15u) == 0 && (y_frame_stride & 3u) == 0);
+    unsigned blocks;
+    if (modulation_grid((int)y_nodes, (int)y_frames, wide, a.f_blocks, blocks, name)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    dim3 const grid(blocks), block(kModBlock);
+    if (bit)       { hipLaunchKernelGGL((real_to_binary_kernel<true, 4>), grid, block, 0, st, a); }
+    else if (wide) { hipLaunchKernelGGL((real_to_binary_kernel<false, 4>), grid, block, 0, st, a); }
+    else           { hipLaunchKernelGGL((real_to_binary_kernel<false, 1>), grid, block, 0, st, a); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_RealToBinary_Forward(float const *dev_x_buf, float *dev_y_buf, unsigned depth_modulation_size, unsigned frame_modulation_size,
+                                    float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size,
+                                    unsigned x_frame_size, unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_real_to_binary(dev_x_buf, dev_y_buf, false, depth_modulation_size, frame_modulation_size, input_range_lo, input_range_hi,
+                                 point_size, x_depth_size, x_frame_size, x_frame_stride, y_frame_stride, binarize, stream, __func__);
+}
+
+int bbhip_fp32_bit_RealToBinary_Forward(float const *dev_x_buf, int *dev_y_buf, unsigned depth_modulation_size, unsigned frame_modulation_size,
+                                        float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size,
+                                        unsigned x_frame_size, unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_real_to_binary(dev_x_buf, dev_y_buf, true, depth_modulation_size, frame_modulation_size, input_range_lo, input_range_hi,
+                                 point_size, x_depth_size, x_frame_size, x_frame_stride, y_frame_stride, binarize, stream, __func__);
+}
+
+static int check_binary_to_real(void const *a, void const *b, int node_mux_size, int frame_mux_size, int y_node_size, long long x_stride_frames,
+                                int y_frame_size, int y_frame_stride, char const *name)
+{
+    if (!(a && b)) { return fail("%s: null buffer", name); }
+    if (!(node_mux_size > 0 && frame_mux_size > 0 && y_node_size > 0 && y_frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if ((long long)y_frame_size * frame_mux_size > 0x7fffffffLL || (long long)node_mux_size * y_node_size > 0x7fffffffLL) {
+        return fail("%s: input too large", name);
+    }
+    if ((long long)node_mux_size * frame_mux_size >= (1 << 24)) { return fail("%s: more than 2^24 inputs fold into an output", name); }
+    if (y_frame_stride < y_frame_size || x_stride_frames < (long long)y_frame_size * frame_mux_size) {
+        return fail("%s: frame stride shorter than the frames", name);
+    }
+    return 0;
+}
+
+static int launch_binary_to_real_forward(void const *x, bool bit, float *y, int node_mux_size, int frame_mux_size, int y_node_size,
+                                         int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream, char const *name)
+{
+    if (check_binary_to_real(x, y, node_mux_size, frame_mux_size, y_node_size, (long long)x_frame_stride * (bit ? 32 : 1), y_frame_size,
+                             y_frame_stride, name)) { return 1; }
+    BinaryToRealArgs a{};
+    a.x = x; a.out = y; a.node_mux_size = node_mux_size; a.frame_mux_size = frame_mux_size; a.y_node_size = y_node_size;
+    a.x_stride = x_frame_stride; a.y_frame_size = y_frame_size; a.y_stride = y_frame_stride;
+    a.denominator = (float)(node_mux_size * frame_mux_size);
+    unsigned blocks;
+    if (modulation_grid(y_node_size, y_frame_size, false, a.f_blocks, blocks, name)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    if (bit) { hipLaunchKernelGGL((binary_to_real_forward_kernel<true>), dim3(blocks), dim3(kModBlock), 0, st, a); }
+    else     { hipLaunchKernelGGL((binary_to_real_forward_kernel<false>), dim3(blocks), dim3(kModBlock), 0, st, a); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_BinaryToReal_Forward(float const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+                                    int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_binary_to_real_forward(dev_x_buf, false, dev_y_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size,
+                                         y_frame_stride, stream, __func__);
+}
+
+int bbhip_bit_fp32_BinaryToReal_Forward(int const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+                                        int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_binary_to_real_forward(dev_x_buf, true, dev_y_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size,
+                                         y_frame_stride, stream, __func__);
+}
+
+int bbhip_fp32_BinaryToReal_Backward(float const *dev_dy_buf, float *dev_dx_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+                                     int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_binary_to_real(dev_dy_buf, dev_dx_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size, y_frame_stride,
+                             __func__)) { return 1; }
+    BinaryToRealArgs a{};
+    a.dy = dev_dy_buf; a.out = dev_dx_buf; a.node_mux_size = node_mux_size; a.frame_mux_size = frame_mux_size; a.y_node_size = y_node_size;
+    a.x_stride = x_frame_stride; a.y_frame_size = y_frame_size; a.y_stride = y_frame_stride;
+    // the host loop's gain (include/bb/BinaryToReal.h:342): output nodes / (input nodes * frames folded), in fp32
+    a.gain = (float)y_node_size / ((float)(node_mux_size * y_node_size) * (float)frame_mux_size);
+    a.frame_mux = make_tile_divisor(frame_mux_size);
+    int const x_frame_size = y_frame_size * frame_mux_size;
+    bool const wide = (reinterpret_cast<uintptr_t>(dev_dx_buf) & 15u) == 0 && (x_frame_stride & 3) == 0;
+    unsigned blocks;
+    if (modulation_grid(node_mux_size * y_node_size, x_frame_size, wide, a.f_blocks, blocks, __func__)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    if (wide) { hipLaunchKernelGGL((binary_to_real_backward_kernel<4>), dim3(blocks), dim3(kModBlock), 0, st, a, x_frame_size); }
+    else      { hipLaunchKernelGGL((binary_to_real_backward_kernel<1>), dim3(blocks), dim3(kModBlock), 0, st, a, x_frame_size); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
 }
 
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,

@@ -327,6 +327,71 @@ def reduce_backward(dy, input_nodes, frame_size):
     return dx
 
 
+def real_to_binary_forward(x, depth, points, frame_size, frame_mod=1, depth_mod=1, lo=0.0, hi=1.0, binarize=True, bit=False, y_stride=None):
+    """fp32 x [depth * points, stride] -> y [depth * depth_mod * points, y_stride]: fp32, or rows of packed words with `bit`
+    (padding words of a packed row beyond the last frame's word are left as allocated: zero)."""
+    _dev(x)
+    out_frames = frame_size * frame_mod
+    if y_stride is None:
+        y_stride = (out_frames + 31) // 32 if bit else out_frames
+    nodes = depth * depth_mod * points
+    if bit:
+        y = torch.zeros((nodes, y_stride), dtype=torch.int32, device=x.device)
+        f = lib().bbhip_fp32_bit_RealToBinary_Forward
+    else:
+        y = torch.empty((nodes, y_stride), dtype=torch.float32, device=x.device)
+        f = lib().bbhip_fp32_RealToBinary_Forward
+    check(f(ptr(x), ptr(y), depth_mod, frame_mod, lo, hi, points, depth, frame_size, x.shape[1], y_stride, int(binarize), stream_ptr()))
+    return y
+
+
+def binary_to_real_forward(x, output_nodes, y_frame_size, frame_mux=1, y_stride=None):
+    """x [I, stride] fp32 (counted where > 0) or int32 packed bits, y_frame_size * frame_mux frames -> fp32 y [O, y_stride]"""
+    _dev(x)
+    y_stride = y_frame_size if y_stride is None else y_stride
+    y = torch.empty((output_nodes, y_stride), dtype=torch.float32, device=x.device)
+    f = lib().bbhip_bit_fp32_BinaryToReal_Forward if x.dtype == torch.int32 else lib().bbhip_fp32_BinaryToReal_Forward
+    check(f(ptr(x), ptr(y), x.shape[0] // output_nodes, frame_mux, output_nodes, x.shape[1], y_frame_size, y_stride, stream_ptr()))
+    return y
+
+
+def binary_to_real_backward(dy, input_nodes, y_frame_size, frame_mux=1, x_stride=None):
+    _dev(dy)
+    x_stride = y_frame_size * frame_mux if x_stride is None else x_stride
+    dx = torch.empty((input_nodes, x_stride), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_BinaryToReal_Backward(ptr(dy), ptr(dx), input_nodes // dy.shape[0], frame_mux, dy.shape[0], x_stride, y_frame_size,
+                                                 dy.shape[1], stream_ptr()))
+    return dx
+
+
+def binarize_forward(x, frame_size, th=0.0, low=-1.0, high=1.0, bit=False, y_stride=None):
+    """y = x > th ? high : low, or with `bit` the packed bits of x > th"""
+    _dev(x)
+    if bit:
+        y_stride = (frame_size + 31) // 32 if y_stride is None else y_stride
+        y = torch.zeros((x.shape[0], y_stride), dtype=torch.int32, device=x.device)
+        check(lib().bbhip_fp32_bit_Binarize_Forward(ptr(x), ptr(y), th, x.shape[0], frame_size, x.shape[1], y_stride, stream_ptr()))
+        return y
+    y = torch.empty_like(x)
+    check(lib().bbhip_fp32_Binarize_Forward(ptr(x), ptr(y), th, low, high, x.shape[0], frame_size, x.shape[1], stream_ptr()))
+    return y
+
+
+def hard_tanh_forward(x, frame_size, lo=-1.0, hi=1.0):
+    _dev(x)
+    y = torch.empty_like(x)
+    check(lib().bbhip_fp32_HardTanh_Forward(ptr(x), ptr(y), lo, hi, x.shape[0], frame_size, x.shape[1], stream_ptr()))
+    return y
+
+
+def hard_tanh_backward(x, dy, frame_size, lo=-1.0, hi=1.0):
+    """dx = dy inside the open window (lo, hi), 0 elsewhere; also the backward of Binarize"""
+    _dev(x, dy)
+    dx = torch.empty_like(dy)
+    check(lib().bbhip_fp32_HardTanh_Backward(ptr(x), ptr(dy), ptr(dx), lo, hi, x.shape[0], frame_size, x.shape[1], stream_ptr()))
+    return dx
+
+
 def loss_mean_squared_error(y, t, frame_size, loss_buf, batch_size=None, reduction_sum=False):
     """-> dy; loss_buf (float64, device, any length >= 1) receives the batch's partial sums ON TOP of what it holds.  The layer's loss is
     loss_buf.sum() / frames seen (the sum itself with reduction "sum")."""

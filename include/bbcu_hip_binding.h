@@ -327,6 +327,77 @@ inline int bbcu_fp32_StochasticBatchNormalization_Backward(float const *dev_x_bu
     return 0;
 }
 
+/* ---- RealToBinary / BinaryToReal, include/bbcu/bbcu.h:1337-1413 ---- */
+template <typename T = float>
+inline int bbcu_RealToBinary_Forward(T const *dev_x_buf, T *dev_y_buf, unsigned int depth_modulation_size, unsigned int frame_modulation_size,
+        T input_range_lo, T input_range_hi, unsigned int point_size, unsigned int x_depth_size, unsigned int x_frame_size,
+        unsigned int x_frame_stride, unsigned int y_frame_stride, bool binarize, cudaStream_t streamId = 0)
+{
+    static_assert(sizeof(T) == sizeof(float), "the reference instantiates this template for float only");
+    BBCU_HIP_CALL(bbhip_fp32_RealToBinary_Forward(dev_x_buf, dev_y_buf, depth_modulation_size, frame_modulation_size, input_range_lo, input_range_hi,
+                                                  point_size, x_depth_size, x_frame_size, x_frame_stride, y_frame_stride, binarize ? 1 : 0, streamId));
+    return 0;
+}
+/* the reference's device kernel takes the bit as value > 0.5 whatever the layer's mode: binarize = 1 */
+template <typename T = float>
+inline int bbcu_bit_RealToBinary_Forward(T const *dev_x_buf, int *dev_y_buf, unsigned int depth_modulation_size, unsigned int frame_modulation_size,
+        T input_range_lo, T input_range_hi, unsigned int point_size, unsigned int x_depth_size, unsigned int x_frame_size,
+        unsigned int x_frame_stride, unsigned int y_frame_stride, cudaStream_t streamId = 0)
+{
+    static_assert(sizeof(T) == sizeof(float), "the reference instantiates this template for float only");
+    BBCU_HIP_CALL(bbhip_fp32_bit_RealToBinary_Forward(dev_x_buf, dev_y_buf, depth_modulation_size, frame_modulation_size, input_range_lo,
+                                                      input_range_hi, point_size, x_depth_size, x_frame_size, x_frame_stride, y_frame_stride, 1,
+                                                      streamId));
+    return 0;
+}
+inline int bbcu_fp32_BinaryToReal_Forward(float const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+        int x_frame_stride, int y_frame_size, int y_frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_BinaryToReal_Forward(dev_x_buf, dev_y_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size,
+                                                  y_frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_bit_fp32_BinaryToReal_Forward(int const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+        int x_frame_stride, int y_frame_size, int y_frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_bit_fp32_BinaryToReal_Forward(dev_x_buf, dev_y_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride,
+                                                      y_frame_size, y_frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_BinaryToReal_Backward(float const *dev_dy_buf, float *dev_dx_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+        int x_frame_stride, int y_frame_size, int y_frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_BinaryToReal_Backward(dev_dy_buf, dev_dx_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride,
+                                                   y_frame_size, y_frame_stride, streamId));
+    return 0;
+}
+
+/* ---- Binarize / HardTanh, include/bbcu/bbcu.h:1223-1276 ---- */
+inline int bbcu_fp32_Binarize_Forward(const float *dev_x_buf, float *dev_y_buf, float binary_th, float binary_low, float binary_high,
+        int node_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_Binarize_Forward(dev_x_buf, dev_y_buf, binary_th, binary_low, binary_high, node_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_bit_Binarize_Forward(float const *dev_x_buf, int *dev_y_buf, float binary_th, int node_size, int frame_size,
+        int x_frame_stride, int y_frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_bit_Binarize_Forward(dev_x_buf, dev_y_buf, binary_th, node_size, frame_size, x_frame_stride, y_frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_HardTanh_Forward(float const *dev_x_buf, float *dev_y_buf, float limit_min, float limit_max, int node_size, int frame_size,
+        int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_HardTanh_Forward(dev_x_buf, dev_y_buf, limit_min, limit_max, node_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_HardTanh_Backward(const float *dev_x_buf, const float *dev_dy_buf, float *dev_dx_buf, float limit_min, float limit_max,
+        int node_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_HardTanh_Backward(dev_x_buf, dev_dy_buf, dev_dx_buf, limit_min, limit_max, node_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+
 /* ---- Im2Col / Col2Im, include/bbcu/bbcu.h:1076-1186 ---- */
 inline int bbcu_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
         int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size, int output_w_size,

@@ -266,6 +266,52 @@ int bbhip_bit_fp32_Reduce_Forward(int const *dev_x_buf, float *dev_y_buf, int in
 int bbhip_fp32_Reduce_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_node_size, int output_node_size, int frame_size,
                                int frame_stride, void *stream);
 
+/* ---- RealToBinary, BinaryToReal ----
+ * The converters at either end of a binary network (include/bb/BinaryModulation.h:44-46).  Results are the bits of the reference's
+ * host loops evaluated in fp32 without fused multiply-adds. */
+/* bbcu_RealToBinary_Forward<float>, include/bbcu/bbcu.h:1337-1352 (host loop include/bb/RealToBinary.h:300-344, no value generator):
+ * input node (depth c, point p) and frame g give output node (depth c * depth_modulation_size + d, point p), frame
+ * g * frame_modulation_size + f the value  clamp01((((x - lo) / (hi - lo)) - d / dm) * dm - f / fm) * fm), and +1 / -1 by > 0.5 when
+ * `binarize`.  A NaN input gives 1. */
+int bbhip_fp32_RealToBinary_Forward(float const *dev_x_buf, float *dev_y_buf, unsigned depth_modulation_size, unsigned frame_modulation_size,
+                                    float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size,
+                                    unsigned x_frame_size, unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream);
+/* bbcu_bit_RealToBinary_Forward<float>, include/bbcu/bbcu.h:1355-1370, packed output (rows of y_frame_stride words; bits past the
+ * last frame of a row's last word are written as 0).  `binarize` is not in the reference's signature: its device kernel always takes
+ * the bit as value > 0.5 (pass 1 for that), its host loop takes the bit of the clamped value, value > 0, when the layer is not in
+ * binary mode (pass 0). */
+int bbhip_fp32_bit_RealToBinary_Forward(float const *dev_x_buf, int *dev_y_buf, unsigned depth_modulation_size, unsigned frame_modulation_size,
+                                        float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size,
+                                        unsigned x_frame_size, unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream);
+/* bbcu_fp32_BinaryToReal_Forward, include/bbcu/bbcu.h:1376-1387: y[o][g] = the share of inputs > 0 among the input nodes o, O + o, ...
+ * (node_mux_size of them) and the frames g * frame_mux_size ... + frame_mux_size - 1, the count divided by their number as on the host
+ * (include/bb/BinaryToReal.h:262-290; the reference's device kernel multiplies by a reciprocal). */
+int bbhip_fp32_BinaryToReal_Forward(float const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+                                    int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream);
+/* bbcu_bit_fp32_BinaryToReal_Forward, include/bbcu/bbcu.h:1389-1400: packed input, rows of x_frame_stride words */
+int bbhip_bit_fp32_BinaryToReal_Forward(int const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+                                        int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream);
+/* bbcu_fp32_BinaryToReal_Backward, include/bbcu/bbcu.h:1402-1413: every input that folds into (o, g) receives
+ * dy[o][g] * (O / (I * frame_mux_size)) (include/bb/BinaryToReal.h:333-352) */
+int bbhip_fp32_BinaryToReal_Backward(float const *dev_dy_buf, float *dev_dx_buf, int node_mux_size, int frame_mux_size, int y_node_size,
+                                     int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream);
+
+/* ---- Binarize, HardTanh ---- */
+/* bbcu_fp32_Binarize_Forward, include/bbcu/bbcu.h:1223-1234: y = x > binary_th ? binary_high : binary_low (include/bb/Binarize.h:196-213) */
+int bbhip_fp32_Binarize_Forward(float const *dev_x_buf, float *dev_y_buf, float binary_th, float binary_low, float binary_high,
+                                int node_size, int frame_size, int frame_stride, void *stream);
+/* bbcu_fp32_bit_Binarize_Forward, include/bbcu/bbcu.h:1236-1246: the packed bits of x > binary_th (bits past the last frame written as 0) */
+int bbhip_fp32_bit_Binarize_Forward(float const *dev_x_buf, int *dev_y_buf, float binary_th, int node_size, int frame_size,
+                                    int x_frame_stride, int y_frame_stride, void *stream);
+/* bbcu_fp32_HardTanh_Forward, include/bbcu/bbcu.h:1253-1263: x <= limit_min -> limit_min, x >= limit_max -> limit_max
+ * (include/bb/HardTanh.h:176-193) */
+int bbhip_fp32_HardTanh_Forward(float const *dev_x_buf, float *dev_y_buf, float limit_min, float limit_max, int node_size, int frame_size,
+                                int frame_stride, void *stream);
+/* bbcu_fp32_HardTanh_Backward, include/bbcu/bbcu.h:1265-1276: dx = dy where limit_min < x < limit_max, else 0; also the backward of
+ * Binarize (include/bb/HardTanh.h:253-271, Binarize.h:268-285) */
+int bbhip_fp32_HardTanh_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, float limit_min, float limit_max,
+                                 int node_size, int frame_size, int frame_stride, void *stream);
+
 /* ---- mean squared error ---- */
 /* bbcu_fp32_LossMeanSquaredError, include/bbcu/bbcu.h:1487-1500: dy = (y - t) * grad_reduction (the caller passes 2 / (nodes * batch)
  * or 2); dev_loss_buf[s] += the sum over the frames s, s + loss_buf_size, ... and all nodes of (float)(y - t)^2 * loss_reduction in

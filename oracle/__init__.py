@@ -322,6 +322,72 @@ def reduce_backward(dy, input_node_size, frame_size):
     return dx
 
 
+def real_to_binary_forward(x, depth, points, frame_size, frame_mod=1, depth_mod=1, lo=0.0, hi=1.0, binarize=True, bit=False, y_stride=None):
+    """x [depth * points, stride] -> y [depth * depth_mod * points, y_stride] (fp32, or words of packed bits): RealToBinary without a
+    value generator (include/bb/RealToBinary.h:300-344)."""
+    x = _c(x, np.float32)
+    out_frames = frame_size * frame_mod
+    if y_stride is None:
+        y_stride = (out_frames + 31) // 32 if bit else out_frames
+    y = np.zeros((depth * depth_mod * points, y_stride), np.int32 if bit else np.float32)
+    f = lib().oracle_bit_RealToBinary_Forward if bit else lib().oracle_fp32_RealToBinary_Forward
+    f(_ptr(x), _ptr(y), C.c_int(depth_mod), C.c_int(frame_mod), C.c_float(lo), C.c_float(hi), C.c_int(points), C.c_int(depth),
+      C.c_int(frame_size), C.c_int(x.shape[1]), C.c_int(y_stride), C.c_int(int(binarize)))
+    return y
+
+
+def binary_to_real_forward(x, output_node_size, y_frame_size, frame_mux=1, bit=False, y_stride=None):
+    """x [I, stride] (fp32 or packed bits; y_frame_size * frame_mux frames) -> y [O, y_stride]: the share of inputs > 0 among the
+    I / O nodes and frame_mux frames that fold into an output element (include/bb/BinaryToReal.h:262-290)."""
+    x = _c(x, np.int32 if bit else np.float32)
+    y_stride = y_frame_size if y_stride is None else y_stride
+    y = np.zeros((output_node_size, y_stride), np.float32)
+    f = lib().oracle_bit_fp32_BinaryToReal_Forward if bit else lib().oracle_fp32_BinaryToReal_Forward
+    f(_ptr(x), _ptr(y), C.c_int(x.shape[0] // output_node_size), C.c_int(frame_mux), C.c_int(output_node_size), C.c_int(x.shape[1]),
+      C.c_int(y_frame_size), C.c_int(y_stride))
+    return y
+
+
+def binary_to_real_backward(dy, input_node_size, y_frame_size, frame_mux=1, x_stride=None):
+    dy = _c(dy, np.float32)
+    x_stride = y_frame_size * frame_mux if x_stride is None else x_stride
+    dx = np.zeros((input_node_size, x_stride), np.float32)
+    lib().oracle_fp32_BinaryToReal_Backward(_ptr(dy), _ptr(dx), C.c_int(input_node_size // dy.shape[0]), C.c_int(frame_mux), C.c_int(dy.shape[0]),
+                                            C.c_int(x_stride), C.c_int(y_frame_size), C.c_int(dy.shape[1]))
+    return dx
+
+
+def binarize_forward(x, frame_size, th=0.0, low=-1.0, high=1.0, bit=False, y_stride=None):
+    """y = x > th ? high : low (include/bb/Binarize.h:196-213), or the packed bits of x > th."""
+    x = _c(x, np.float32)
+    if bit:
+        y_stride = (frame_size + 31) // 32 if y_stride is None else y_stride
+        y = np.zeros((x.shape[0], y_stride), np.int32)
+        lib().oracle_fp32_bit_Binarize_Forward(_ptr(x), _ptr(y), C.c_float(th), C.c_int(x.shape[0]), C.c_int(frame_size), C.c_int(x.shape[1]),
+                                               C.c_int(y_stride))
+        return y
+    y = np.zeros_like(x)
+    lib().oracle_fp32_Binarize_Forward(_ptr(x), _ptr(y), C.c_float(th), C.c_float(low), C.c_float(high), C.c_int(x.shape[0]), C.c_int(frame_size),
+                                       C.c_int(x.shape[1]))
+    return y
+
+
+def hard_tanh_forward(x, frame_size, lo=-1.0, hi=1.0):
+    x = _c(x, np.float32)
+    y = np.zeros_like(x)
+    lib().oracle_fp32_HardTanh_Forward(_ptr(x), _ptr(y), C.c_float(lo), C.c_float(hi), C.c_int(x.shape[0]), C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y
+
+
+def hard_tanh_backward(x, dy, frame_size, lo=-1.0, hi=1.0):
+    """dx = dy inside the open window (lo, hi), 0 elsewhere (include/bb/HardTanh.h:253-271); also the backward of Binarize."""
+    x = _c(x, np.float32); dy = _c(dy, np.float32)
+    dx = np.zeros_like(x)
+    lib().oracle_fp32_HardTanh_Backward(_ptr(x), _ptr(dy), _ptr(dx), C.c_float(lo), C.c_float(hi), C.c_int(x.shape[0]), C.c_int(frame_size),
+                                        C.c_int(x.shape[1]))
+    return dx
+
+
 def loss_mean_squared_error(y, t, frame_size, batch_size=None, reduction_sum=False, loss=0.0):
     """-> (dy, loss accumulator): the reference's host loop (include/bb/LossMeanSquaredError.h:121-169) for one batch; `loss` is the
     accumulator before the batch.  The layer's loss is accumulator / frames seen (the accumulator itself with reduction "sum")."""
@@ -810,6 +876,59 @@ def ref_reduce(x, output_node_size, frames, bit=False, integration_size=0, dy=No
     f.restype = C.c_long
     r = f(C.c_int(int(bit)), C.c_int(I), C.c_int(output_node_size), C.c_int(frames), C.c_int(integration_size), _ptr(x), _ptr(y), _ptr(dy),
           _ptr(dx), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
+
+
+def ref_real_to_binary(x, depth, points, frames, frame_mod=1, depth_mod=1, lo=0.0, hi=1.0, binary_mode=True, bit=False, name="",
+                       want_object=False):
+    """The reference's RealToBinary host path (no value generator) on a dense [depth * points, frames] array -> (y, object bytes);
+    y is [depth * depth_mod * points, frames * frame_mod] fp32, or rows of packed words."""
+    x = _c(x, np.float32)
+    out_nodes, out_frames = depth * depth_mod * points, frames * frame_mod
+    y = np.zeros((out_nodes, (out_frames + 31) // 32), np.int32) if bit else np.zeros((out_nodes, out_frames), np.float32)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_RealToBinary
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(depth), C.c_int(points), C.c_int(frames), C.c_int(frame_mod), C.c_int(depth_mod), C.c_float(lo),
+          C.c_float(hi), C.c_int(int(binary_mode)), _ptr(x), _ptr(y), C.c_char_p(name.encode()), _ptr(out),
+          C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, (out[:r].copy() if want_object else None)
+
+
+def ref_binary_to_real(x, output_node_size, frames, frame_mux=1, bit=False, dy=None, name="", want_object=False):
+    """The reference's BinaryToReal host path; x [I, frames] fp32 or [I, words] bits -> (y [O, frames / frame_mux], dx, object bytes)."""
+    x = _c(x, np.int32 if bit else np.float32)
+    I = x.shape[0]
+    y = np.zeros((output_node_size, frames // frame_mux), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((I, frames), np.float32)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_BinaryToReal
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(I), C.c_int(output_node_size), C.c_int(frames), C.c_int(frame_mux), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx),
+          C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
+
+
+def ref_activation(kind, x, frames, bit=False, th=0.0, low=-1.0, high=1.0, lo=-1.0, hi=1.0, dy=None, name="", want_object=False):
+    """The reference's Binarize (kind "binarize"), HardTanh ("hard_tanh") or HardTanh in binary mode ("hard_tanh_binary") host paths
+    on a dense [nodes, frames] array -> (y, dx, object bytes); y is packed words where the layer's output type is Bit."""
+    x = _c(x, np.float32)
+    nodes = x.shape[0]
+    y = np.zeros((nodes, (frames + 31) // 32), np.int32) if bit else np.zeros((nodes, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((nodes, frames), np.float32)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_Activation
+    f.restype = C.c_long
+    r = f(C.c_int({"binarize": 0, "hard_tanh": 1, "hard_tanh_binary": 2}[kind]), C.c_int(int(bit)), C.c_int(nodes), C.c_int(frames),
+          C.c_float(th), C.c_float(low), C.c_float(high), C.c_float(lo), C.c_float(hi), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx),
+          C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
     assert r >= 0, r
     return y, dx, (out[:r].copy() if want_object else None)
 

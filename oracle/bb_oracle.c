@@ -34,6 +34,11 @@
  *     vectors written from it (tests/golden/bn.npz) to 1e-6 of the terms that
  *     cancel (contraction, as above; the batch mean bit-exact), fp64 textbook
  *     statistics, the gradient's two vanishing sums and a finite difference.
+ *   - RealToBinary, BinaryToReal, Binarize, HardTanh: bit-exact against the
+ *     reference's classes (oracle/_ref), vectors written from them
+ *     (tests/golden/modulation.npz), the known answers of
+ *     tests/gtest/RealToBinaryTest.cpp, BinaryToRealTest.cpp, BinarizeTest.cpp,
+ *     and numpy restatements.
  *
  * Array conventions (the reference's FrameBuffer layout, include/bb/FrameBuffer.h:28-46,
  * 927-939): node-major, frame-minor; element (node n, frame f) of an fp32
@@ -1284,6 +1289,185 @@ void oracle_fp32_MetricsMeanSquaredError(float const *y, float const *t, double 
             float const grad = t[(long long)node * frame_stride + f] - y[(long long)node * frame_stride + f];
             float const error = grad * grad;
             *accuracy += error / (double)node_size;
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ *  The layers at either end of a binary network and the activations between its layers.
+ *
+ *  RealToBinary without a value generator (host loop include/bb/RealToBinary.h:300-344): input node (depth c, point p),
+ *  input frame g; output node (depth c * dm + d, point p), output frame g * fm + f:
+ *      v = (x - lo) * (1 / (hi - lo));  v = (v - d * (1/dm)) * dm;  v = (v - f * (1/fm)) * fm;  v = max(0, min(1, v))
+ *  every operation rounded to fp32 on its own, min and max as std::min / std::max evaluate them (a NaN becomes 1), and
+ *  in binary mode +1 where v > 0.5, else -1.  Packed output takes the bit of that value as Bit(v) does (DataType.h:278):
+ *  v > 0, which is v > 0.5 before the +1 / -1 in binary mode and v > 0 after the clamp otherwise.
+ *  BinaryToReal (include/bb/BinaryToReal.h:262-290, backward :333-352): output node o, frame g counts the inputs that are
+ *  > 0 (set bits) among input nodes o, O + o, 2 O + o, ... and frames g * fmux ... g * fmux + fmux - 1 and divides the count by their
+ *  number; backward sends dy * gain to each of them, gain = O / (I * fmux) in fp32.
+ *  Binarize (include/bb/Binarize.h:196-213): y = x > th ? high : low; its backward is HardTanh's with the layer's own window
+ *  (:268-285).  HardTanh (include/bb/HardTanh.h:176-193, :253-271): x <= min -> min, x >= max -> max; dx = 0 there, dy elsewhere.
+ *  Pinned by tests/test_oracle_modulation.py: the reference's classes (oracle/_ref), vectors written from them
+ *  (tests/golden/modulation.npz), the known answers of tests/gtest/RealToBinaryTest.cpp, BinaryToRealTest.cpp and
+ *  BinarizeTest.cpp, and numpy restatements in fp64 where fp32 rounding cannot matter.
+ * ------------------------------------------------------------------------------------------------------------------- */
+static inline float std_min_f(float a, float b) { return (b < a) ? b : a; }     /* std::min(a, b) */
+static inline float std_max_f(float a, float b) { return (a < b) ? b : a; }     /* std::max(a, b) */
+
+static inline float real_to_binary_value(float x, long long d, long long f, float lo, float x_scale, float depth_step,
+                                         float depth_step_recip, float frame_step, float frame_step_recip)
+{
+    float v = (x - lo) * x_scale;
+    v = (v - (float)((float)d * depth_step)) * depth_step_recip;
+    v = (v - (float)((float)f * frame_step)) * frame_step_recip;
+    return std_max_f(0.0f, std_min_f(1.0f, v));
+}
+
+void oracle_fp32_RealToBinary_Forward(float const *x, float *y, int depth_modulation_size, int frame_modulation_size,
+                                      float input_range_lo, float input_range_hi, int point_size, int x_depth_size,
+                                      int x_frame_size, int x_frame_stride, int y_frame_stride, int binarize)
+{
+    float const frame_step = 1.0f / (float)frame_modulation_size, frame_step_recip = (float)frame_modulation_size;
+    float const depth_step = 1.0f / (float)depth_modulation_size, depth_step_recip = (float)depth_modulation_size;
+    float const x_scale = 1.0f / (input_range_hi - input_range_lo);
+    for (int g = 0; g < x_frame_size; ++g) {
+        for (int f = 0; f < frame_modulation_size; ++f) {
+            long long const out_frame = (long long)g * frame_modulation_size + f;
+            for (int c = 0; c < x_depth_size; ++c) {
+                for (int p = 0; p < point_size; ++p) {
+                    float const xv = x[((long long)c * point_size + p) * x_frame_stride + g];
+                    for (int d = 0; d < depth_modulation_size; ++d) {
+                        long long const out_node = ((long long)c * depth_modulation_size + d) * point_size + p;
+                        float v = real_to_binary_value(xv, d, f, input_range_lo, x_scale, depth_step, depth_step_recip, frame_step, frame_step_recip);
+                        if (binarize) { v = (v > 0.5f) ? 1.0f : -1.0f; }
+                        y[out_node * y_frame_stride + out_frame] = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* y rows are y_frame_stride words; the caller clears them (bits past the last frame stay 0) */
+void oracle_bit_RealToBinary_Forward(float const *x, int *y, int depth_modulation_size, int frame_modulation_size,
+                                     float input_range_lo, float input_range_hi, int point_size, int x_depth_size,
+                                     int x_frame_size, int x_frame_stride, int y_frame_stride, int binarize)
+{
+    float const frame_step = 1.0f / (float)frame_modulation_size, frame_step_recip = (float)frame_modulation_size;
+    float const depth_step = 1.0f / (float)depth_modulation_size, depth_step_recip = (float)depth_modulation_size;
+    float const x_scale = 1.0f / (input_range_hi - input_range_lo);
+    for (int g = 0; g < x_frame_size; ++g) {
+        for (int f = 0; f < frame_modulation_size; ++f) {
+            long long const out_frame = (long long)g * frame_modulation_size + f;
+            for (int c = 0; c < x_depth_size; ++c) {
+                for (int p = 0; p < point_size; ++p) {
+                    float const xv = x[((long long)c * point_size + p) * x_frame_stride + g];
+                    for (int d = 0; d < depth_modulation_size; ++d) {
+                        long long const out_node = ((long long)c * depth_modulation_size + d) * point_size + p;
+                        float v = real_to_binary_value(xv, d, f, input_range_lo, x_scale, depth_step, depth_step_recip, frame_step, frame_step_recip);
+                        if (binarize) { v = (v > 0.5f) ? 1.0f : -1.0f; }
+                        if (v > 0) { y[out_node * y_frame_stride + (out_frame >> 5)] |= (int)(1u << (out_frame & 31)); }
+                    }
+                }
+            }
+        }
+    }
+}
+
+void oracle_fp32_BinaryToReal_Forward(float const *x, float *y, int node_mux_size, int frame_mux_size, int y_node_size,
+                                      int x_frame_stride, int y_frame_size, int y_frame_stride)
+{
+    for (int g = 0; g < y_frame_size; ++g) {
+        for (int o = 0; o < y_node_size; ++o) {
+            float v = 0;
+            int n = 0;
+            for (int m = 0; m < node_mux_size; ++m) {
+                for (int i = 0; i < frame_mux_size; ++i) {
+                    float const sig = x[((long long)m * y_node_size + o) * x_frame_stride + (long long)g * frame_mux_size + i];
+                    v += (sig > 0) ? 1 : 0;
+                    n += 1;
+                }
+            }
+            y[(long long)o * y_frame_stride + g] = v / (float)n;
+        }
+    }
+}
+
+void oracle_bit_fp32_BinaryToReal_Forward(int const *x, float *y, int node_mux_size, int frame_mux_size, int y_node_size,
+                                          int x_frame_stride, int y_frame_size, int y_frame_stride)
+{
+    for (int g = 0; g < y_frame_size; ++g) {
+        for (int o = 0; o < y_node_size; ++o) {
+            float v = 0;
+            int n = 0;
+            for (int m = 0; m < node_mux_size; ++m) {
+                for (int i = 0; i < frame_mux_size; ++i) {
+                    v += get_bit(x + ((long long)m * y_node_size + o) * x_frame_stride, (long long)g * frame_mux_size + i) ? 1 : 0;
+                    n += 1;
+                }
+            }
+            y[(long long)o * y_frame_stride + g] = v / (float)n;
+        }
+    }
+}
+
+void oracle_fp32_BinaryToReal_Backward(float const *dy, float *dx, int node_mux_size, int frame_mux_size, int y_node_size,
+                                       int x_frame_stride, int y_frame_size, int y_frame_stride)
+{
+    float const gain = (float)y_node_size / ((float)((long long)node_mux_size * y_node_size) * (float)frame_mux_size);
+    for (long long node = 0; node < (long long)node_mux_size * y_node_size; ++node) {
+        for (int g = 0; g < y_frame_size; ++g) {
+            for (int i = 0; i < frame_mux_size; ++i) {
+                float grad = dy[(node % y_node_size) * y_frame_stride + g];
+                grad *= gain;
+                dx[node * x_frame_stride + (long long)g * frame_mux_size + i] = grad;
+            }
+        }
+    }
+}
+
+void oracle_fp32_Binarize_Forward(float const *x, float *y, float binary_th, float binary_low, float binary_high,
+                                  int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            y[(long long)node * frame_stride + f] = x[(long long)node * frame_stride + f] > binary_th ? binary_high : binary_low;
+        }
+    }
+}
+
+/* y rows are y_frame_stride words; the caller clears them */
+void oracle_fp32_bit_Binarize_Forward(float const *x, int *y, float binary_th, int node_size, int frame_size,
+                                      int x_frame_stride, int y_frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            if (x[(long long)node * x_frame_stride + f] > binary_th) { y[(long long)node * y_frame_stride + (f >> 5)] |= (int)(1u << (f & 31)); }
+        }
+    }
+}
+
+void oracle_fp32_HardTanh_Forward(float const *x, float *y, float limit_min, float limit_max, int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float v = x[(long long)node * frame_stride + f];
+            if (v <= limit_min) { v = limit_min; }
+            if (v >= limit_max) { v = limit_max; }
+            y[(long long)node * frame_stride + f] = v;
+        }
+    }
+}
+
+void oracle_fp32_HardTanh_Backward(float const *x, float const *dy, float *dx, float limit_min, float limit_max,
+                                   int node_size, int frame_size, int frame_stride)
+{
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            float g = dy[(long long)node * frame_stride + f];
+            float const v = x[(long long)node * frame_stride + f];
+            if (v <= limit_min || v >= limit_max) { g = 0.0f; }
+            dx[(long long)node * frame_stride + f] = g;
         }
     }
 }

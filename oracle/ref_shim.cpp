@@ -37,6 +37,10 @@
 #include "bb/Convolution2d.h"
 #include "bb/Sequential.h"
 #include "bb/StochasticBatchNormalization.h"
+#include "bb/RealToBinary.h"
+#include "bb/BinaryToReal.h"
+#include "bb/Binarize.h"
+#include "bb/HardTanh.h"
 
 namespace {
 
@@ -865,4 +869,100 @@ extern "C" int bbref_MeanSquaredError(int nodes, int F, int batches, int reducti
     *loss = lossFunc->GetLoss();
     *metric = metrics->GetMetrics();
     return 0;
+}
+
+// RealToBinary<BinType, float> (host path, no value generator).  x: [depth * points][F]; y: [depth * depth_mod * points][F * frame_mod]
+// as fp32 or as rows of ceil(F * frame_mod / 32) words.
+namespace {
+template <typename BinType>
+long run_real_to_binary(int depth, int points, int F, int frame_mod, int depth_mod, float lo, float hi, int binary_mode,
+                        float const *x, void *y, char const *name, unsigned char *object_out, long cap)
+{
+    auto m = bb::RealToBinary<BinType, float>::Create((index_t)frame_mod, (index_t)depth_mod, nullptr, false, lo, hi);
+    if (name && *name) { m->SetName(name); }
+    m->SendCommand("binary " + onoff(binary_mode));
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)depth, (index_t)points}), BB_TYPE_FP32, true);
+    m->SetInputShape(xb.GetShape());
+    put_fp32(xb, x, (index_t)depth * points, F);
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    index_t const out_nodes = (index_t)depth * depth_mod * points, out_frames = (index_t)F * frame_mod;
+    if (yb.GetNodeSize() != out_nodes || yb.GetFrameSize() != out_frames) { return -2; }
+    if (bb::DataType<BinType>::type == BB_TYPE_BIT) { get_bit(yb, (std::int32_t *)y, out_nodes, (out_frames + 31) / 32); }
+    else                                            { get_fp32(yb, (float *)y, out_nodes, out_frames); }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+
+template <typename BinType>
+long run_binary_to_real(int I, int O, int F, int frame_mux, void const *x, float *y, float const *dy, float *dx, char const *name,
+                        unsigned char *object_out, long cap)
+{
+    auto m = bb::BinaryToReal<BinType, float>::Create((index_t)frame_mux, bb::indices_t({(index_t)O}));
+    if (name && *name) { m->SetName(name); }
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)I}), xtype, true);
+    m->SetInputShape(xb.GetShape());
+    if (xtype == BB_TYPE_BIT) { put_bit(xb, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(xb, (float const *)x, I, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (yb.GetNodeSize() != O || yb.GetFrameSize() != F / frame_mux) { return -2; }
+    get_fp32(yb, y, O, F / frame_mux);
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)(F / frame_mux), bb::indices_t({(index_t)O}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, O, F / frame_mux);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        if (dxb.GetNodeSize() != I || dxb.GetFrameSize() != F) { return -3; }
+        get_fp32(dxb, dx, I, F);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+
+// kind 0: Binarize<BinType>(th, low, high, lo, hi); kind 1: HardTanh<BinType>(lo, hi); kind 2: HardTanh in binary mode
+template <typename BinType>
+long run_activation(int kind, int nodes, int F, float th, float low, float high, float lo, float hi, float const *x, void *y,
+                    float const *dy, float *dx, char const *name, unsigned char *object_out, long cap)
+{
+    std::shared_ptr<bb::Binarize<BinType, float>> m;
+    if (kind == 0) { m = bb::Binarize<BinType, float>::Create(th, (double)low, (double)high, lo, hi); }
+    else {
+        m = bb::HardTanh<BinType, float>::Create(lo, hi);
+        if (kind == 2) { m->SendCommand("binary true"); }
+    }
+    if (name && *name) { m->SetName(name); }
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)nodes}), BB_TYPE_FP32, true);
+    m->SetInputShape(xb.GetShape());
+    put_fp32(xb, x, nodes, F);
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (yb.GetType() == BB_TYPE_BIT) { get_bit(yb, (std::int32_t *)y, nodes, (F + 31) / 32); }
+    else                             { get_fp32(yb, (float *)y, nodes, F); }
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, bb::indices_t({(index_t)nodes}), BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, nodes, F);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, nodes, F);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+}  // namespace
+
+extern "C" long bbref_RealToBinary(int bit, int depth, int points, int F, int frame_mod, int depth_mod, float lo, float hi, int binary_mode,
+                                   float const *x, void *y, char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_real_to_binary<bb::Bit>(depth, points, F, frame_mod, depth_mod, lo, hi, binary_mode, x, y, name, object_out, cap)
+               : run_real_to_binary<float>(depth, points, F, frame_mod, depth_mod, lo, hi, binary_mode, x, y, name, object_out, cap);
+}
+
+// BinaryToReal<BinType, float> (host path) with output shape {O}.  x: [I][F] fp32 or bits; y, dy: [O][F / frame_mux]; dx: [I][F].
+extern "C" long bbref_BinaryToReal(int bit, int I, int O, int F, int frame_mux, void const *x, float *y, float const *dy, float *dx,
+                                   char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_binary_to_real<bb::Bit>(I, O, F, frame_mux, x, y, dy, dx, name, object_out, cap)
+               : run_binary_to_real<float>(I, O, F, frame_mux, x, y, dy, dx, name, object_out, cap);
+}
+
+// Binarize / HardTanh (host paths), see run_activation.  y: fp32 [nodes][F], or bits when the layer's output type is Bit.
+extern "C" long bbref_Activation(int kind, int bit, int nodes, int F, float th, float low, float high, float lo, float hi,
+                                 float const *x, void *y, float const *dy, float *dx, char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_activation<bb::Bit>(kind, nodes, F, th, low, high, lo, hi, x, y, dy, dx, name, object_out, cap)
+               : run_activation<float>(kind, nodes, F, th, low, high, lo, hi, x, y, dy, dx, name, object_out, cap);
 }

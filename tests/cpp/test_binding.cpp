@@ -97,6 +97,17 @@ SAME(&bbcu_fp32_StochasticBatchNormalization_ForwardTraining, int (*)(float cons
 SAME(&bbcu_fp32_StochasticBatchNormalization_ReForward, int (*)(float const *, float *, float const *, float const *, float, float, int, int, int, S));
 SAME(&bbcu_fp32_StochasticBatchNormalization_ForwardInference, int (*)(float const *, float *, float const *, float const *, float, float, int, int, int, S));
 SAME(&bbcu_fp32_StochasticBatchNormalization_Backward, int (*)(float const *, float const *, float *, float const *, float const *, float, float, int, int, int, int, S));
+// bbcu.h:1223-1276, 1337-1413
+SAME(&bbcu_fp32_Binarize_Forward, int (*)(const float *, float *, float, float, float, int, int, int, S));
+SAME(&bbcu_fp32_bit_Binarize_Forward, int (*)(float const *, int *, float, int, int, int, int, S));
+SAME(&bbcu_fp32_HardTanh_Forward, int (*)(float const *, float *, float, float, int, int, int, S));
+SAME(&bbcu_fp32_HardTanh_Backward, int (*)(const float *, const float *, float *, float, float, int, int, int, S));
+SAME(&bbcu_RealToBinary_Forward<float>, int (*)(float const *, float *, unsigned int, unsigned int, float, float, unsigned int, unsigned int, unsigned int, unsigned int, unsigned int, bool, S));
+SAME(&bbcu_RealToBinary_Forward<>, decltype(&bbcu_RealToBinary_Forward<float>));
+SAME(&bbcu_bit_RealToBinary_Forward<float>, int (*)(float const *, int *, unsigned int, unsigned int, float, float, unsigned int, unsigned int, unsigned int, unsigned int, unsigned int, S));
+SAME(&bbcu_fp32_BinaryToReal_Forward, int (*)(float const *, float *, int, int, int, int, int, int, S));
+SAME(&bbcu_bit_fp32_BinaryToReal_Forward, int (*)(int const *, float *, int, int, int, int, int, int, S));
+SAME(&bbcu_fp32_BinaryToReal_Backward, int (*)(float const *, float *, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_Im2Col_Forward, int (*)(float const *, float *, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, float, S));
 SAME(&bbcu_bit_Im2Col_Forward, int (*)(int const *, int *, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_Im2Col_Backward, int (*)(float const *, float *, int, int, int, int, int, int, int, int, int, int, int, int, int, int, S));
@@ -167,7 +178,7 @@ static int run_on_gpu(void)
 
 int main(int argc, char **argv)
 {
-    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11;
+    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11 + 10;
     if (argc > 1 && !std::strcmp(argv[1], "--gpu")) {
         if (!bbcu_IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
         int const bad = run_on_gpu();
