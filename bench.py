@@ -228,6 +228,55 @@ def bench_stochastic_bn(args, lib):
     return out
 
 
+def bench_modulation(args, lib):
+    """RealToBinary, BinaryToReal, Binarize and HardTanh (secondary measurement).  The converters at the size of an MNIST-like input
+    batch (784 nodes x 4096 frames, 7 frames per input: 28672 modulated frames) and of a classifier's last binary layer (1024 nodes
+    folding into 128, 7 frames into 1); the activations at the size of a hidden layer of the headline configuration, 8192 nodes x
+    4096 frames.  Algorithmic bytes: every element of each input and output once (4 B per fp32 element, 1 bit per packed one)."""
+    import torch
+    from binarybrain_amd import ops, synth
+    g = torch.Generator(device="cuda"); g.manual_seed(0)
+    nodes, F, fm = 784, 4096, 7
+    yF = F * fm
+    x = torch.rand((nodes, synth.frame_stride_fp32(F)), device="cuda", generator=g)
+    ys, ws = synth.frame_stride_fp32(yF), synth.frame_stride_bit(yF)
+    I, O = 1024, 128
+    h = (torch.rand((I, ys), device="cuda", generator=g) - 0.5)
+    hb = ops.binarize_forward(h, yF, 0.0, bit=True, y_stride=ws)
+    dyo = torch.randn((O, synth.frame_stride_fp32(F)), device="cuda", generator=g)
+    an, aF = 8192, 4096
+    aS = synth.frame_stride_fp32(aF)
+    a = torch.randn((an, aS), device="cuda", generator=g)
+    da = torch.randn((an, aS), device="cuda", generator=g)
+    e = 4
+    cases = [
+        ("real_to_binary_kernel fp32 784x4096 x7", lambda: ops.real_to_binary_forward(x, 1, nodes, F, fm, y_stride=ys), e * nodes * (F + yF)),
+        ("real_to_binary_kernel bit 784x4096 x7", lambda: ops.real_to_binary_forward(x, 1, nodes, F, fm, bit=True, y_stride=ws), e * nodes * F + nodes * yF // 8),
+        ("binary_to_real_forward_kernel fp32 1024->128 /7", lambda: ops.binary_to_real_forward(h, O, F, fm), e * (I * yF + O * F)),
+        ("binary_to_real_forward_kernel bit 1024->128 /7", lambda: ops.binary_to_real_forward(hb, O, F, fm), I * yF // 8 + e * O * F),
+        ("binary_to_real_backward_kernel 128->1024 x7", lambda: ops.binary_to_real_backward(dyo, I, F, fm, x_stride=ys), e * (O * F + I * yF)),
+        ("row_map_kernel Binarize 8192x4096", lambda: ops.binarize_forward(a, aF), 2 * e * an * aF),
+        ("binarize_bits_kernel 8192x4096", lambda: ops.binarize_forward(a, aF, bit=True, y_stride=synth.frame_stride_bit(aF)), e * an * aF + an * aF // 8),
+        ("row_map_kernel HardTanh 8192x4096", lambda: ops.hard_tanh_forward(a, aF), 2 * e * an * aF),
+        ("row_map_kernel HardTanh backward 8192x4096", lambda: ops.hard_tanh_backward(a, da, aF), 3 * e * an * aF),
+    ]
+    kernels = {}
+    total_ms = 0.0
+    for name, fn, nbytes in cases:
+        med = library_timed_ms(lib, fn, args.steps, args.warmup)
+        total_ms += med
+        kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
+    dom = max(kernels, key=lambda k: kernels[k]["ms"])
+    out = {"metric": "RealToBinary + BinaryToReal + Binarize + HardTanh kernels, ms for one launch of each", "value": total_ms, "unit": "ms",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": total_ms, "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "converters at 784 nodes x 4096 frames x 7 and 1024 -> 128 nodes; activations at 8192 nodes x 4096 frames"},
+           "roofline": {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": kernels[dom]["achieved_GBps"] / HBM_PEAK_GBS, "traffic": None},
+           "kernels": kernels}
+    return out
+
+
 def bench_tail(args, lib):
     """The tail of the MNIST-like classifier (secondary measurement): AverageLut 7 -> 1 over 70 -> 10 nodes (and MaxLut at the same
     shape), softmax cross entropy and categorical accuracy over the 10 classes.  Measured at 65536 frames (streaming rate) and at the
@@ -843,7 +892,7 @@ def main():
                     help="headline workload only: skip the other BASELINE configurations that the default run reports under `configs`")
     ap.add_argument("--profile-copy", action="store_true",
                     help="after the timed region, copy x to y three times: a plain copy of known size for calibrating rocprofv3 byte counters")
-    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail", "stochastic_bn",
+    ap.add_argument("--workload", default="stochasticlut6", choices=["stochasticlut6", "binarylut6", "differentiablelut6", "differentiablelut6_bit", "mnist_step", "conv_block", "adam", "conv", "tail", "stochastic_bn", "modulation",
                              "forward_784x1024x64", "gather_ceiling"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
@@ -859,7 +908,7 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     lib = capi.lib()
-    secondary = {"binarylut6": bench_binarylut6, "adam": bench_adam, "conv": bench_conv, "tail": bench_tail, "stochastic_bn": bench_stochastic_bn,
+    secondary = {"binarylut6": bench_binarylut6, "adam": bench_adam, "conv": bench_conv, "tail": bench_tail, "stochastic_bn": bench_stochastic_bn, "modulation": bench_modulation,
                  "differentiablelut6": bench_differentiablelut6, "differentiablelut6_bit": bench_differentiablelut6,
                  "mnist_step": bench_mnist_step, "conv_block": bench_conv_block, "forward_784x1024x64": bench_forward_small,
                  "gather_ceiling": bench_gather_ceiling}

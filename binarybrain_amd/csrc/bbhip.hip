@@ -1889,15 +1889,16 @@ static int launch_real_to_binary(float const *x, void *y, bool bit, unsigned dep
         return fail("%s: sizes must be positive", name);
     }
     long long const y_frames = (long long)x_frame_size * frame_modulation_size;
-    long long const y_nodes = (long long)x_depth_size * depth_modulation_size * point_size;
-    if (y_frames > 0x7fffffffLL || y_nodes > 0x7fffffffLL) { return fail("%s: output too large", name); }
+    long long const y_planes = (long long)x_depth_size * depth_modulation_size;
+    long long const y_nodes = (y_planes <= 0x7fffffffLL) ? y_planes * point_size : -1;
+    if (y_frames > 0x7fffffffLL || y_nodes < 0 || y_nodes > 0x7fffffffLL) { return fail("%s: output too large", name); }
     if (x_frame_stride < x_frame_size || (long long)y_frame_stride < (bit ? (y_frames + 31) / 32 : y_frames)) {
         return fail("%s: frame stride shorter than the frames", name);
     }
     RealToBinaryArgs a{};
     a.x = x; a.y = y;
     a.x_frame_size = (int)x_frame_size; a.y_frame_size = (int)y_frames; a.x_stride = (int)x_frame_stride; a.y_stride = (int)y_frame_stride;
-    a.point_size = (int)point_size; a.depth_modulation_size = (int)depth_modulation_size;
+    a.points = make_tile_divisor((int)point_size); a.depth_modulation = make_tile_divisor((int)depth_modulation_size);
     a.lo = input_range_lo; a.x_scale = 1.0f / (input_range_hi - input_range_lo);
     a.depth_step = 1.0f / (float)depth_modulation_size; a.depth_step_recip = (float)depth_modulation_size;
     a.frame_step = 1.0f / (float)frame_modulation_size; a.frame_step_recip = (float)frame_modulation_size;

@@ -105,7 +105,8 @@ struct RealToBinaryArgs {
     float const *x;
     void        *y;                 // fp32 rows or rows of packed words
     int x_frame_size, y_frame_size, x_stride, y_stride;
-    int point_size, depth_modulation_size;
+    TileDivisor points;             // output node -> (depth plane, point)
+    TileDivisor depth_modulation;   // depth plane -> (input depth, depth step)
     float lo, x_scale, depth_step, depth_step_recip, frame_step, frame_step_recip;
     float threshold;                // packed output: 0.5 in binary mode, else 0 (the bit of the clamped value, v > 0)
     int binarize;                   // fp32 output: +1 / -1 by v > 0.5
@@ -113,36 +114,55 @@ struct RealToBinaryArgs {
     TileDivisor frame_modulation;   // output frame -> (input frame, step within the modulation)
 };
 
-// the modulated and clamped value of input x at depth step d and frame step r (include/bb/RealToBinary.h:318-330)
-__device__ __forceinline__ float real_to_binary_value(float x, float d, float r, RealToBinaryArgs const &a)
+// The value of an input before the frame step: brought to [0, 1] and through the depth step d (include/bb/RealToBinary.h:318-324)
+__device__ __forceinline__ float real_to_binary_depth_value(float x, float d, RealToBinaryArgs const &a)
 {
-    float v = rounded_mul(x - a.lo, a.x_scale);
-    v = rounded_mul(v - rounded_mul(d, a.depth_step), a.depth_step_recip);
-    v = rounded_mul(v - rounded_mul(r, a.frame_step), a.frame_step_recip);
+    float const v = rounded_mul(x - a.lo, a.x_scale);
+    return rounded_mul(v - rounded_mul(d, a.depth_step), a.depth_step_recip);
+}
+
+// ... and through frame step r, clamped (:326-330)
+__device__ __forceinline__ float real_to_binary_frame_value(float t, float r, RealToBinaryArgs const &a)
+{
+    float v = rounded_mul(t - rounded_mul(r, a.frame_step), a.frame_step_recip);
     v = (v < 1.0f) ? v : 1.0f;      // std::min(1, v): a NaN becomes 1
     v = (0.0f < v) ? v : 0.0f;      // std::max(0, v)
     return v;
 }
 
+// A thread's W output frames are consecutive, so their (input frame, frame step) pairs follow from the first by counting:
+// one division per thread.  The inputs of all W frames are requested before the first is used (neighbouring frames mostly
+// share one, which the cache serves; a load that waits for the previous frame's arithmetic would cost a round trip each).
 template <bool BIT, int W>
 __global__ __launch_bounds__(kModBlock) void real_to_binary_kernel(RealToBinaryArgs a)
 {
     int node, block;
     split_tile(blockIdx.x, a.f_blocks, node, block);
     // output node = (c * dm + d) * points + p  reads input node c * points + p
-    int const plane = node / a.point_size, p = node - plane * a.point_size;
-    int const c = plane / a.depth_modulation_size, d = plane - c * a.depth_modulation_size;
-    float const *__restrict__ xr = a.x + (size_t)(c * a.point_size + p) * a.x_stride;
+    int plane, p, c, d;
+    split_tile(node, a.points, plane, p);
+    split_tile(plane, a.depth_modulation, c, d);
+    float const *__restrict__ xr = a.x + (size_t)(c * a.points.count + p) * a.x_stride;
     int const f = (block * kModBlock + threadIdx.x) * W;
     float v[W];
     uint32_t bits = 0;
     if (f < a.y_frame_size) {
+        int g, r;
+        split_tile(f, a.frame_modulation, g, r);
+        float xv[W];
+        int step[W];
 #pragma unroll
         for (int j = 0; j < W; ++j) {
-            int g, r;
-            split_tile(f + j, a.frame_modulation, g, r);
-            float const xv = (f + j < a.y_frame_size) ? xr[g] : 0.0f;
-            v[j] = real_to_binary_value(xv, (float)d, (float)r, a);
+            xv[j] = xr[g];
+            step[j] = r;
+            if (++r == a.frame_modulation.count) {
+                r = 0;
+                g = (g + 1 < a.x_frame_size) ? g + 1 : g;          // frames past the end of the row are computed but not stored
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+            v[j] = real_to_binary_frame_value(real_to_binary_depth_value(xv[j], (float)d, a), (float)step[j], a);
             if (BIT) { if (f + j < a.y_frame_size && v[j] > a.threshold) { bits |= 1u << j; } }
             else if (a.binarize) { v[j] = (v[j] > 0.5f) ? 1.0f : -1.0f; }
         }

@@ -25,6 +25,10 @@
 #define BB_TYPE_INT32   (0x0200 + 32)
 #define BB_TYPE_UINT8   (0x0300 + 8)
 
+// the two values of a binary signal held as a number (reference: include/bb/DataType.h:48-49)
+#define BB_BINARY_HI    (+1)
+#define BB_BINARY_LO    (-1)
+
 namespace bb {
 
 using index_t   = std::int64_t;

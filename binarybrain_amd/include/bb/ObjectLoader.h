@@ -1,6 +1,6 @@
 // Reconstruct a serialized object from its recorded type name (reference: include/bb/ObjectLoader.h:407-447
 // `Object_Load` / `Object_LoadFromFile`).  Known here: the LUT layers of widths 2..6 on fp32 or packed-bit frames,
-// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
+// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, Binarize, HardTanh, RealToBinary, BinaryToReal, BinaryModulation, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
 #pragma once
 
 #include "bb/StochasticLutN.h"
@@ -14,6 +14,11 @@
 #include "bb/MaxLut.h"
 #include "bb/AverageLut.h"
 #include "bb/Reduce.h"
+#include "bb/Binarize.h"
+#include "bb/HardTanh.h"
+#include "bb/RealToBinary.h"
+#include "bb/BinaryToReal.h"
+#include "bb/BinaryModulation.h"
 
 namespace bb {
 
@@ -44,6 +49,16 @@ inline std::shared_ptr<Object> CreateByName(std::string const &name)
     if (name == Reduce<float, float>::ObjectName())               { return Reduce<float, float>::Create(); }
     if (name == Reduce<Bit, float>::ObjectName())                 { return Reduce<Bit, float>::Create(); }
     if (name == MaxLut<Bit, float>::ObjectName())                 { return MaxLut<Bit, float>::Create(); }
+    if (name == Binarize<float, float>::ObjectName())             { return Binarize<float, float>::Create(); }
+    if (name == Binarize<Bit, float>::ObjectName())               { return Binarize<Bit, float>::Create(); }
+    if (name == HardTanh<float, float>::ObjectName())             { return HardTanh<float, float>::Create(); }
+    if (name == HardTanh<Bit, float>::ObjectName())               { return HardTanh<Bit, float>::Create(); }
+    if (name == RealToBinary<float, float>::ObjectName())         { return RealToBinary<float, float>::Create(); }
+    if (name == RealToBinary<Bit, float>::ObjectName())           { return RealToBinary<Bit, float>::Create(); }
+    if (name == BinaryToReal<float, float>::ObjectName())         { return BinaryToReal<float, float>::Create(); }
+    if (name == BinaryToReal<Bit, float>::ObjectName())           { return BinaryToReal<Bit, float>::Create(); }
+    if (name == BinaryModulation<float, float>::ObjectName())     { return BinaryModulation<float, float>::Create(); }
+    if (name == BinaryModulation<Bit, float>::ObjectName())       { return BinaryModulation<Bit, float>::Create(); }
     if (name == Convolution2d<float, float>::ObjectName())        { return Convolution2d<float, float>::Create(); }
     if (name == Convolution2d<Bit, float>::ObjectName())          { return Convolution2d<Bit, float>::Create(); }
     if (name == ConvolutionIm2Col<float, float>::ObjectName())    { return ConvolutionIm2Col<float, float>::Create(1, 1); }

@@ -933,6 +933,17 @@ def ref_activation(kind, x, frames, bit=False, th=0.0, low=-1.0, high=1.0, lo=-1
     return y, dx, (out[:r].copy() if want_object else None)
 
 
+def ref_dump_binary_modulation_object(input_nodes, o1, o2, train_mod, infer_mod=0, depth_mod=1, bit=False, seed=1, run_inference=False, name=""):
+    """The bytes of a BinaryModulation around a list of two DifferentiableLut6 layers as the reference's DumpObject writes them."""
+    out = np.zeros(1 << 22, np.uint8)
+    f = ref().bbref_DumpBinaryModulationObject
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(input_nodes), C.c_int(o1), C.c_int(o2), C.c_int(train_mod), C.c_int(infer_mod), C.c_int(depth_mod),
+          C.c_int(seed), C.c_int(int(run_inference)), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size))
+    assert r > 0, r
+    return out[:r].copy()
+
+
 def ref_mean_squared_error(y, t, frames, batches=1, reduction_sum=False):
     """The reference's LossMeanSquaredError and MetricsMeanSquaredError host paths over `batches` batches of `frames` frames held side
     by side in y and t -> (dy, loss, metric)."""

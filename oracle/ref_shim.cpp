@@ -41,6 +41,7 @@
 #include "bb/BinaryToReal.h"
 #include "bb/Binarize.h"
 #include "bb/HardTanh.h"
+#include "bb/BinaryModulation.h"
 
 namespace {
 
@@ -965,4 +966,41 @@ extern "C" long bbref_Activation(int kind, int bit, int nodes, int F, float th, 
 {
     return bit ? run_activation<bb::Bit>(kind, nodes, F, th, low, high, lo, hi, x, y, dy, dx, name, object_out, cap)
                : run_activation<float>(kind, nodes, F, th, low, high, lo, hi, x, y, dy, dx, name, object_out, cap);
+}
+
+// A BinaryModulation<BinType, float> around a Sequential of two DifferentiableLut6 layers (I -> o1 -> o2 nodes, wired and initialised
+// by the reference from the seed), dumped after SetInputShape({I}) and, with run_inference, after one inference pass over four zero
+// frames (which leaves the converters at the inference modulation size).  Returns the object's size, negative on error.
+namespace {
+template <typename BinType>
+long dump_binary_modulation(int I, int o1, int o2, int train_mod, int infer_mod, int depth_mod, int seed, int run_inference, char const *name,
+                            unsigned char *out, long cap)
+{
+    auto make_lut = [&](int o, int s) {
+        typename bb::DifferentiableLutN<6, BinType, float>::create_t cr;
+        cr.output_shape = {(index_t)o};
+        cr.seed = (std::uint64_t)s;
+        return bb::DifferentiableLutN<6, BinType, float>::Create(cr);
+    };
+    auto body = bb::Sequential::Create();
+    body->Add(make_lut(o1, seed));
+    body->Add(make_lut(o2, seed + 1));
+    auto m = bb::BinaryModulation<BinType, float>::Create(body, (index_t)train_mod, (index_t)infer_mod, (index_t)depth_mod);
+    if (name && *name) { m->SetName(name); }
+    m->SendCommand("host_only true");
+    m->SetInputShape(bb::indices_t({(index_t)I}));
+    if (run_inference) {
+        bb::FrameBuffer xb((index_t)4, bb::indices_t({(index_t)I}), BB_TYPE_FP32, true);
+        xb.FillZero();
+        (void)m->Forward(xb, false);
+    }
+    return emit(*m, out, cap);
+}
+}  // namespace
+
+extern "C" long bbref_DumpBinaryModulationObject(int bit, int I, int o1, int o2, int train_mod, int infer_mod, int depth_mod, int seed,
+                                                 int run_inference, char const *name, unsigned char *out, long cap)
+{
+    return bit ? dump_binary_modulation<bb::Bit>(I, o1, o2, train_mod, infer_mod, depth_mod, seed, run_inference, name, out, cap)
+               : dump_binary_modulation<float>(I, o1, o2, train_mod, infer_mod, depth_mod, seed, run_inference, name, out, cap);
 }

@@ -26,6 +26,11 @@
 #include "bb/Convolution2d.h"
 #include "bb/Sequential.h"
 #include "bb/StochasticBatchNormalization.h"
+#include "bb/Binarize.h"
+#include "bb/HardTanh.h"
+#include "bb/RealToBinary.h"
+#include "bb/BinaryToReal.h"
+#include "bb/BinaryModulation.h"
 #include "bb/ObjectLoader.h"
 
 extern "C" {
@@ -50,6 +55,13 @@ void oracle_fp32_Reduce_Forward(float const *x, float *y, int input_node_size, i
 void oracle_fp32_Reduce_Backward(float const *dy, float *dx, int input_node_size, int output_node_size, int frame_size, int frame_stride);
 void oracle_fp32_LossMeanSquaredError(float const *y, float const *t, float *dy, double *loss, int node_size, int frame_size, int frame_stride, float grad_reduction, double loss_reduction);
 void oracle_fp32_MetricsMeanSquaredError(float const *y, float const *t, double *accuracy, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_RealToBinary_Forward(float const *x, float *y, int depth_modulation_size, int frame_modulation_size, float input_range_lo, float input_range_hi, int point_size, int x_depth_size, int x_frame_size, int x_frame_stride, int y_frame_stride, int binarize);
+void oracle_bit_RealToBinary_Forward(float const *x, int *y, int depth_modulation_size, int frame_modulation_size, float input_range_lo, float input_range_hi, int point_size, int x_depth_size, int x_frame_size, int x_frame_stride, int y_frame_stride, int binarize);
+void oracle_fp32_BinaryToReal_Forward(float const *x, float *y, int node_mux_size, int frame_mux_size, int y_node_size, int x_frame_stride, int y_frame_size, int y_frame_stride);
+void oracle_fp32_BinaryToReal_Backward(float const *dy, float *dx, int node_mux_size, int frame_mux_size, int y_node_size, int x_frame_stride, int y_frame_size, int y_frame_stride);
+void oracle_fp32_Binarize_Forward(float const *x, float *y, float binary_th, float binary_low, float binary_high, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_HardTanh_Forward(float const *x, float *y, float limit_min, float limit_max, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_HardTanh_Backward(float const *x, float const *dy, float *dx, float limit_min, float limit_max, int node_size, int frame_size, int frame_stride);
 void oracle_bit_BinaryLut6_Forward(std::int32_t const *x, std::int32_t *y, std::int32_t const *idx, std::int32_t const *table, int node_size, int frame_size, int frame_stride);
 }
 
@@ -619,6 +631,139 @@ static void test_reduce_and_mean_squared_error(void)
     }
 }
 
+// The converters at either end of a binary network, the activations, and the three-part container around a layer list.
+static void test_binary_modulation(void)
+{
+    std::mt19937_64 mt(23);
+    std::uniform_real_distribution<float> uni(-0.1f, 1.1f);
+    std::vector<float> x, y, dy, dx, ref;
+    {   // RealToBinary over shape {2, 5}: 3 frames and 2 depth steps per input; fp32 and packed outputs, binary and real mode
+        int const D = 2, P = 5, F = 37, fm = 3, dm = 2;
+        bb::FrameBuffer x_buf(F, {D, P}, BB_TYPE_FP32);
+        for (int n = 0; n < D * P; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, uni(mt)); }
+        read_fp32(x_buf, x);
+        auto r2b = bb::RealToBinary<float>::Create(fm, dm);
+        auto r2b_bit = bb::RealToBinary<bb::Bit>::Create(fm, dm);
+        CHECK(r2b->SetInputShape({D, P}) == bb::indices_t({D * dm, P}), "RealToBinary output shape");
+        for (int binary = 1; binary >= 0; --binary) {
+            r2b->SendCommand(binary ? "binary true" : "binary false"); r2b_bit->SendCommand(binary ? "binary true" : "binary false");
+            bb::FrameBuffer y_buf = r2b->Forward(x_buf), yb_buf = r2b_bit->Forward(x_buf);
+            CHECK(y_buf.GetFrameSize() == F * fm && y_buf.GetNodeSize() == D * dm * P && yb_buf.GetType() == BB_TYPE_BIT, "RealToBinary output size");
+            read_fp32(y_buf, y);
+            ref.assign(y.size(), 0.0f);
+            oracle_fp32_RealToBinary_Forward(x.data(), ref.data(), dm, fm, 0.0f, 1.0f, P, D, F, F, F * fm, binary);
+            CHECK(max_diff(y, ref) == 0.0, "RealToBinary (binary %d) differs by %g", binary, max_diff(y, ref));
+            size_t bad = 0;
+            // the packed output is Bit(v), v > 0, of the fp32 output: of +1 / -1 in binary mode, of the clamped value otherwise
+            for (int n = 0; n < D * dm * P; ++n) for (int f = 0; f < F * fm; ++f) { bad += (yb_buf.GetBit(f, n) != (ref[(size_t)n * F * fm + f] > 0.0f)); }
+            CHECK(bad == 0, "RealToBinary packed output (binary %d): %zu bits differ", binary, bad);
+        }
+        auto plain = bb::RealToBinary<float>::Create(fm);
+        plain->SendCommand("binary false");
+        bb::FrameBuffer same = plain->Forward(x_buf);
+        CHECK(same_bits(same, x_buf), "RealToBinary out of binary mode without depth modulation hands its input through");
+    }
+    {   // BinaryToReal: 70 nodes fold into 10, 7 frames into 1; fp32 and packed input, backward
+        int const I = 70, O = 10, Fy = 33, fm = 7, F = Fy * fm;
+        bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), xb_buf(F, {I}, BB_TYPE_BIT), dy_buf(Fy, {O}, BB_TYPE_FP32);
+        for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { float const v = uni(mt) - 0.5f; x_buf.SetFP32(f, n, v); xb_buf.SetBit(f, n, v > 0); }
+        for (int n = 0; n < O; ++n) for (int f = 0; f < Fy; ++f) { dy_buf.SetFP32(f, n, uni(mt) - 0.5f); }
+        read_fp32(x_buf, x); read_fp32(dy_buf, dy);
+        auto b2r = bb::BinaryToReal<float>::Create(fm, bb::indices_t({O}));
+        auto b2r_bit = bb::BinaryToReal<bb::Bit>::Create(fm, bb::indices_t({O}));
+        bb::FrameBuffer y_buf = b2r->Forward(x_buf), yb_buf = b2r_bit->Forward(xb_buf);
+        read_fp32(y_buf, y);
+        ref.assign((size_t)O * Fy, 0.0f);
+        oracle_fp32_BinaryToReal_Forward(x.data(), ref.data(), I / O, fm, O, F, Fy, Fy);
+        CHECK(max_diff(y, ref) == 0.0 && same_bits(y_buf, yb_buf), "BinaryToReal forward differs by %g", max_diff(y, ref));
+        bb::FrameBuffer dx_buf = b2r->Backward(dy_buf);
+        read_fp32(dx_buf, dx);
+        ref.assign((size_t)I * F, 0.0f);
+        oracle_fp32_BinaryToReal_Backward(dy.data(), ref.data(), I / O, fm, O, F, Fy, Fy);
+        CHECK(dx_buf.GetFrameSize() == F && max_diff(dx, ref) == 0.0, "BinaryToReal backward differs by %g", max_diff(dx, ref));
+        auto by_depth = bb::BinaryToReal<float>::Create(fm, 7);
+        CHECK(by_depth->SetInputShape({I}) == bb::indices_t({O}), "BinaryToReal output shape from the depth integration size");
+    }
+    {   // Binarize and HardTanh
+        int const N = 9, F = 130;
+        bb::FrameBuffer x_buf(F, {N}, BB_TYPE_FP32), dy_buf(F, {N}, BB_TYPE_FP32);
+        for (int n = 0; n < N; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, 3.0f * (uni(mt) - 0.5f)); dy_buf.SetFP32(f, n, uni(mt)); }
+        read_fp32(x_buf, x); read_fp32(dy_buf, dy);
+        auto bin = bb::Binarize<float>::Create(0.1f, 0.0, 1.0, -0.7f, 0.9f);
+        auto bin_bit = bb::Binarize<bb::Bit>::Create(0.1f);
+        auto tanh = bb::HardTanh<float>::Create(-0.5f, 0.75f);
+        bb::FrameBuffer y_buf = bin->Forward(x_buf), yb_buf = bin_bit->Forward(x_buf, false), t_buf = tanh->Forward(x_buf);
+        read_fp32(y_buf, y);
+        ref.assign(x.size(), 0.0f);
+        oracle_fp32_Binarize_Forward(x.data(), ref.data(), 0.1f, 0.0f, 1.0f, N, F, F);
+        size_t bad = 0;
+        for (int n = 0; n < N; ++n) for (int f = 0; f < F; ++f) { bad += (yb_buf.GetBit(f, n) != (ref[(size_t)n * F + f] > 0.5f)); }
+        CHECK(max_diff(y, ref) == 0.0 && bad == 0, "Binarize forward differs by %g, %zu bits", max_diff(y, ref), bad);
+        bb::FrameBuffer dx_buf = bin->Backward(dy_buf);
+        read_fp32(dx_buf, dx);
+        oracle_fp32_HardTanh_Backward(x.data(), dy.data(), ref.data(), -0.7f, 0.9f, N, F, F);
+        CHECK(max_diff(dx, ref) == 0.0, "Binarize backward differs by %g", max_diff(dx, ref));
+        read_fp32(t_buf, y);
+        oracle_fp32_HardTanh_Forward(x.data(), ref.data(), -0.5f, 0.75f, N, F, F);
+        CHECK(max_diff(y, ref) == 0.0, "HardTanh forward differs by %g", max_diff(y, ref));
+        dx_buf = tanh->Backward(dy_buf);
+        read_fp32(dx_buf, dx);
+        oracle_fp32_HardTanh_Backward(x.data(), dy.data(), ref.data(), -0.5f, 0.75f, N, F, F);
+        CHECK(max_diff(dx, ref) == 0.0, "HardTanh backward differs by %g", max_diff(dx, ref));
+        tanh->SendCommand("binary true");
+        t_buf = tanh->Forward(x_buf, false);
+        read_fp32(t_buf, y);
+        oracle_fp32_Binarize_Forward(x.data(), ref.data(), 0.125f, -1.0f, 1.0f, N, F, F);
+        CHECK(max_diff(y, ref) == 0.0, "HardTanh in binary mode differs by %g", max_diff(y, ref));
+        CHECK(tanh->ForwardNode(0, {0.2, 0.1})[0] == 0.75 && tanh->ForwardNode(0, {0.2, 0.1})[1] == -0.5, "HardTanh::ForwardNode in binary mode");
+    }
+    {   // BinaryModulation around two layers = its three parts called one after the other; training and inference sizes; a reload
+        int const I = 20, O1 = 36, O2 = 12, F = 50, train_mod = 3, infer_mod = 5;
+        auto make_body = [&](void) {
+            auto body = bb::Sequential::Create();
+            body->Add(bb::DifferentiableLutN<6, float>::Create((bb::index_t)O1));
+            body->Add(bb::DifferentiableLutN<6, float>::Create((bb::index_t)O2));
+            return body;
+        };
+        auto net = bb::BinaryModulation<float>::Create(make_body(), train_mod, infer_mod);
+        CHECK(net->SetInputShape({I}) == bb::indices_t({O2}), "BinaryModulation output shape");
+        auto body = make_body();
+        {   // a second copy of the layers with the same contents, for the parts called by hand
+            std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+            net->GetLayer()->DumpObject(ss);
+            body->SetInputShape({I});
+            body->LoadObject(ss);
+        }
+        bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), dy_buf(F, {O2}, BB_TYPE_FP32);
+        for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, uni(mt)); }
+        for (int n = 0; n < O2; ++n) for (int f = 0; f < F; ++f) { dy_buf.SetFP32(f, n, uni(mt) - 0.5f); }
+        auto r2b = bb::RealToBinary<float>::Create(train_mod);
+        auto b2r = bb::BinaryToReal<float>::Create(train_mod, bb::indices_t({O2}));
+        bb::FrameBuffer y_buf = net->Forward(x_buf, true);
+        bb::FrameBuffer h_buf = b2r->Forward(body->Forward(r2b->Forward(x_buf, true), true), true);
+        CHECK(y_buf.GetFrameSize() == F && same_bits(y_buf, h_buf), "BinaryModulation forward differs from its three parts");
+        bb::FrameBuffer dx_buf = net->Backward(dy_buf);
+        bb::FrameBuffer g_buf = body->Backward(b2r->Backward(dy_buf));
+        CHECK(dx_buf.GetFrameSize() == F && dx_buf.GetNodeSize() == I && g_buf.GetFrameSize() == F * train_mod, "BinaryModulation backward shapes");
+        {
+            auto a = net->GetGradients(), b = body->GetGradients();
+            CHECK(a.GetSize() == b.GetSize() && a.GetSize() == 2, "BinaryModulation hands the layers' gradients through");
+        }
+        r2b->SetModulationSize(infer_mod); b2r->SetFrameIntegrationSize(infer_mod);
+        y_buf = net->Forward(x_buf, false);
+        h_buf = b2r->Forward(body->Forward(r2b->Forward(x_buf, false), false), false);
+        CHECK(y_buf.GetFrameSize() == F && same_bits(y_buf, h_buf), "BinaryModulation inference differs from its three parts");
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        net->DumpObject(ss);
+        auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)again && again->GetObjectName() == "BinaryModulation_fp32_fp32" && again->GetOutputNodeSize() == O2, "BinaryModulation reload");
+        if (again) { bb::FrameBuffer y3 = again->Forward(x_buf, false); CHECK(same_bits(y3, y_buf), "reloaded BinaryModulation differs"); }
+        net->SendCommand("binary false");
+        y_buf = net->Forward(x_buf, false);
+        CHECK(y_buf.GetFrameSize() == F, "BinaryModulation out of binary mode runs the layer on the unconverted input");
+    }
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -776,6 +921,7 @@ int main(void)
         test_stochastic_batch_normalization();
         test_max_lut();
         test_reduce_and_mean_squared_error();
+        test_binary_modulation();
         test_tail();
         test_hand_off_through_files();
     }

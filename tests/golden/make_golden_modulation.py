@@ -1,6 +1,7 @@
 """Writes tests/golden/modulation.npz: inputs and outputs of the reference's own RealToBinary, BinaryToReal, Binarize and HardTanh host
 classes (include/bb/RealToBinary.h:266-344, BinaryToReal.h:205-352, Binarize.h:142-285, HardTanh.h:133-271), run through
-oracle/_ref/libbbref.so, with the objects they serialize to.
+oracle/_ref/libbbref.so, with the objects they serialize to, and BinaryModulation objects (include/bb/BinaryModulation.h:370-394) around
+two DifferentiableLut6 layers that the reference wired and initialised from a seed.
 
 RealToBinary cases come in two kinds.  "dyadic": inputs on a grid of 1/256 with the range [0, 1] and modulation sizes that are powers
 of two, so that every operation of the layer is exact and the reference's build flags (which fuse some multiply-add pairs) cannot
@@ -31,6 +32,10 @@ BINARY_TO_REAL = [(10, 10, 16, 1, ""), (70, 10, 9, 7, ""), (12, 3, 40, 15, "b2r"
 ACTIVATION = [("binarize", 5, 33, 0.0, -1.0, 1.0, -1.0, 1.0, ""), ("binarize", 3, 64, 0.1, 0.0, 1.0, -0.7, 0.9, "bin"),
               ("hard_tanh", 7, 100, 0.0, -1.0, 1.0, -1.0, 1.0, ""), ("hard_tanh", 4, 31, 0.0, -1.0, 1.0, 0.0, 1.0, "ht"),
               ("hard_tanh_binary", 6, 70, 0.0, -1.0, 1.0, -0.5, 0.75, "")]
+# BinaryModulation around two DifferentiableLut6 layers: bit activations, input nodes, o1, o2, training modulation, inference
+# modulation, depth modulation, seed, dumped after an inference pass, name
+MODULATION = [(False, 20, 36, 12, 7, 0, 1, 3, False, ""), (False, 12, 24, 6, 3, 15, 2, 5, True, "net"), (True, 20, 36, 12, 7, 0, 1, 3, False, ""),
+              (True, 16, 30, 10, 1, 4, 1, 8, True, "bits")]
 
 
 def clear_tail(words, frames):
@@ -89,6 +94,12 @@ def main():
         out[q + "name"] = np.frombuffer(name.encode(), np.uint8)
         for key, val in (("x", x), ("dy", dy), ("y", y), ("y_bits", clear_tail(yb, F)), ("dx", dx), ("object", obj), ("object_bit", objb)):
             out[q + key] = val
+    out["mod_count"] = np.array([len(MODULATION)], np.int32)
+    for k, (bit, I, o1, o2, tm, im, dm, seed, infer, name) in enumerate(MODULATION):
+        q = "n%d_" % k
+        out[q + "args"] = np.array([int(bit), I, o1, o2, tm, im, dm, seed, int(infer)], np.int64)
+        out[q + "name"] = np.frombuffer(name.encode(), np.uint8)
+        out[q + "object"] = oracle.ref_dump_binary_modulation_object(I, o1, o2, tm, im, dm, bit=bit, seed=seed, run_inference=infer, name=name)
     np.savez_compressed(os.path.join(OUT, "modulation.npz"), **out)
     print("wrote modulation.npz")
 

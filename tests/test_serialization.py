@@ -343,3 +343,71 @@ def test_reference_reduce_objects_load_and_survive_a_round_trip(tmp_path, k):
         if oracle.have_ref():                           # the reference's loader lists this type: it reads what was written here
             back = oracle.ref_reload_container_object(np.frombuffer(open(dst, "rb").read(), np.uint8))
             assert back is not None and back.tobytes() == data
+
+
+# ----------------------------------------------------------------------------------------------
+#  RealToBinary, BinaryToReal, Binarize, HardTanh, BinaryModulation (include/bb/RealToBinary.h:501-548, BinaryToReal.h:352-380,
+#  Binarize.h:286-308, HardTanh.h:262-289, BinaryModulation.h:370-420): objects written by the reference's classes
+#  (tests/golden/modulation.npz) load here, report their shapes and names, and are written again byte for byte; the reference's
+#  loader, which lists all of these type names, reads what was written here and writes the same bytes.
+# ----------------------------------------------------------------------------------------------
+MODULATION = np.load(os.path.join(HERE, "golden", "modulation.npz"))
+
+
+def _reload_and_compare(tmp_path, data, type_name, name, default_name, in_nodes, out_nodes):
+    src, dst = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    open(src, "wb").write(data)
+    out = tool("reload", src, dst).stdout.split()
+    assert out[0] == type_name and out[1] == (name if name else default_name)
+    assert (int(out[3]), int(out[5])) == (in_nodes, out_nodes)
+    assert open(dst, "rb").read() == data
+    if oracle.have_ref():
+        back = oracle.ref_reload_container_object(np.frombuffer(open(dst, "rb").read(), np.uint8))
+        assert back is not None and back.tobytes() == data
+
+
+@pytest.mark.parametrize("k", range(int(MODULATION["r2b_count"][0])))
+def test_reference_real_to_binary_objects(tmp_path, k):
+    q = "m%d_" % k
+    d, p, F, fm, dm, _ = [int(v) for v in MODULATION[q + "geom"]]
+    name = MODULATION[q + "name"].tobytes().decode()
+    for key, type_name in (("object", "RealToBinary_fp32_fp32"), ("object_bit", "RealToBinary_bit_fp32")):
+        _reload_and_compare(tmp_path, MODULATION[q + key].tobytes(), type_name, name, "RealToBinary", d * p, d * dm * p)
+
+
+@pytest.mark.parametrize("k", range(int(MODULATION["b2r_count"][0])))
+def test_reference_binary_to_real_objects(tmp_path, k):
+    q = "b%d_" % k
+    I, O, Fy, fm = [int(v) for v in MODULATION[q + "geom"]]
+    name = MODULATION[q + "name"].tobytes().decode()
+    for key, type_name in (("object", "BinaryToReal_fp32_fp32"), ("object_bit", "BinaryToReal_bit_fp32")):
+        _reload_and_compare(tmp_path, MODULATION[q + key].tobytes(), type_name, name, "BinaryToReal", I, O)
+
+
+@pytest.mark.parametrize("k", range(int(MODULATION["act_count"][0])))
+def test_reference_activation_objects(tmp_path, k):
+    q = "a%d_" % k
+    kind = bytes(MODULATION[q + "kind"]).decode()
+    nodes, F = [int(v) for v in MODULATION[q + "geom"]]
+    name = MODULATION[q + "name"].tobytes().decode()
+    model = "Binarize" if kind == "binarize" else "HardTanh"
+    for key, suffix in (("object", "_fp32_fp32"), ("object_bit", "_bit_fp32")):
+        _reload_and_compare(tmp_path, MODULATION[q + key].tobytes(), model + suffix, name, model, nodes, nodes)
+
+
+@pytest.mark.parametrize("k", range(int(MODULATION["mod_count"][0])))
+def test_reference_binary_modulation_objects(tmp_path, k):
+    q = "n%d_" % k
+    bit, I, o1, o2, tm, im, dm, seed, infer = [int(v) for v in MODULATION[q + "args"]]
+    name = MODULATION[q + "name"].tobytes().decode()
+    _reload_and_compare(tmp_path, MODULATION[q + "object"].tobytes(), "BinaryModulation_bit_fp32" if bit else "BinaryModulation_fp32_fp32",
+                        name, "BinaryModulation", I, o2)
+
+
+def test_truncated_modulation_objects_are_rejected(tmp_path):
+    data = MODULATION["n1_object"].tobytes()
+    for cut in (len(data) // 3, len(data) - 9):
+        src = str(tmp_path / ("cut%d.bin" % cut))
+        open(src, "wb").write(data[:cut])
+        res = subprocess.run([TOOL, "reload", src, str(tmp_path / "out.bin")], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        assert res.returncode != 0
