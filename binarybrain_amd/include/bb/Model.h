@@ -82,6 +82,10 @@ public:
     // (reference: include/bb/Model.h:312-315)
     virtual FrameBuffer ReForward(FrameBuffer x_buf) { return Forward(x_buf, true); }
 
+    // drops what a training forward pass kept for the backward pass (reference: include/bb/Model.h:362-367); used by layers
+    // that recompute their intermediate results instead of keeping them
+    virtual void Clear(void) { while (!m_bufs.empty()) { m_bufs.pop(); } }
+
     // value of one output node for one vector of input values (used to tabulate a trained layer)
     virtual std::vector<double> ForwardNode(index_t, std::vector<double> input_value) const { return input_value; }
 };

@@ -1,6 +1,6 @@
 // Reconstruct a serialized object from its recorded type name (reference: include/bb/ObjectLoader.h:407-447
 // `Object_Load` / `Object_LoadFromFile`).  Known here: the LUT layers of widths 2..6 on fp32 or packed-bit frames,
-// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, Binarize, HardTanh, RealToBinary, BinaryToReal, BinaryModulation, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
+// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, Binarize, HardTanh, RealToBinary, BinaryToReal, BinaryModulation, DifferentiableLutDiscreteN (the LUT layer put together from its parts), the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
 #pragma once
 
 #include "bb/StochasticLutN.h"
@@ -19,6 +19,7 @@
 #include "bb/RealToBinary.h"
 #include "bb/BinaryToReal.h"
 #include "bb/BinaryModulation.h"
+#include "bb/DifferentiableLutDiscreteN.h"
 
 namespace bb {
 
@@ -31,6 +32,8 @@ inline std::shared_ptr<Object> CreateLutByName(std::string const &name)
     if (name == StochasticLutN<N, Bit, float>::ObjectName())       { return StochasticLutN<N, Bit, float>::Create((index_t)1); }
     if (name == DifferentiableLutN<N, float, float>::ObjectName()) { return DifferentiableLutN<N, float, float>::Create((index_t)1); }
     if (name == DifferentiableLutN<N, Bit, float>::ObjectName())   { return DifferentiableLutN<N, Bit, float>::Create((index_t)1); }
+    if (name == DifferentiableLutDiscreteN<N, float, float>::ObjectName()) { return DifferentiableLutDiscreteN<N, float, float>::Create((index_t)1); }
+    if (name == DifferentiableLutDiscreteN<N, Bit, float>::ObjectName())   { return DifferentiableLutDiscreteN<N, Bit, float>::Create((index_t)1); }
     return std::shared_ptr<Object>();
 }
 

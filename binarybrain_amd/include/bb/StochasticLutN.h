@@ -219,6 +219,8 @@ public:
         return y_buf;
     }
 
+    void Clear(void) override { Model::Clear(); m_x_buf = FrameBuffer(); }
+
     FrameBuffer Backward(FrameBuffer dy_buf) override
     {
         if (dy_buf.Empty()) { return FrameBuffer(); }       // (the reference also drops its dW tensor here — a defect, not kept)

@@ -944,6 +944,17 @@ def ref_dump_binary_modulation_object(input_nodes, o1, o2, train_mod, infer_mod=
     return out[:r].copy()
 
 
+def ref_dump_discrete_lut_object(input_nodes, output_nodes, bit=False, seed=1, batch_norm=True, memory_saving=False, name=""):
+    """The bytes of a DifferentiableLutDiscrete6 (StochasticLut6 -> StochasticBatchNormalization -> HardTanh) as the reference writes them."""
+    out = np.zeros(1 << 22, np.uint8)
+    f = ref().bbref_DumpDiscreteLutObject
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(input_nodes), C.c_int(output_nodes), C.c_int(seed), C.c_int(int(batch_norm)), C.c_int(int(memory_saving)),
+          C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size))
+    assert r > 0, r
+    return out[:r].copy()
+
+
 def ref_mean_squared_error(y, t, frames, batches=1, reduction_sum=False):
     """The reference's LossMeanSquaredError and MetricsMeanSquaredError host paths over `batches` batches of `frames` frames held side
     by side in y and t -> (dy, loss, metric)."""

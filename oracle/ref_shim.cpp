@@ -42,6 +42,7 @@
 #include "bb/Binarize.h"
 #include "bb/HardTanh.h"
 #include "bb/BinaryModulation.h"
+#include "bb/DifferentiableLutDiscreteN.h"
 
 namespace {
 
@@ -1003,4 +1004,19 @@ extern "C" long bbref_DumpBinaryModulationObject(int bit, int I, int o1, int o2,
 {
     return bit ? dump_binary_modulation<bb::Bit>(I, o1, o2, train_mod, infer_mod, depth_mod, seed, run_inference, name, out, cap)
                : dump_binary_modulation<float>(I, o1, o2, train_mod, infer_mod, depth_mod, seed, run_inference, name, out, cap);
+}
+
+// A DifferentiableLutDiscreteN<6, BinType, float> (StochasticLutN -> StochasticBatchNormalization -> HardTanh), wired and initialised
+// by the reference from the seed, dumped after SetInputShape({I}).  Returns the object's size, negative on error.
+extern "C" long bbref_DumpDiscreteLutObject(int bit, int I, int O, int seed, int batch_norm, int memory_saving, char const *name,
+                                            unsigned char *out, long cap)
+{
+    auto fill = [&](auto m) {
+        if (name && *name) { m->SetName(name); }
+        m->SendCommand("memory_saving " + onoff(memory_saving));
+        m->SetInputShape(bb::indices_t({(index_t)I}));
+        return emit(*m, out, cap);
+    };
+    if (bit) { return fill(bb::DifferentiableLutDiscreteN<6, bb::Bit, float>::Create((index_t)O, batch_norm != 0, "", (std::uint64_t)seed)); }
+    return fill(bb::DifferentiableLutDiscreteN<6, float, float>::Create((index_t)O, batch_norm != 0, "", (std::uint64_t)seed));
 }

@@ -31,6 +31,7 @@
 #include "bb/RealToBinary.h"
 #include "bb/BinaryToReal.h"
 #include "bb/BinaryModulation.h"
+#include "bb/DifferentiableLutDiscreteN.h"
 #include "bb/ObjectLoader.h"
 
 extern "C" {
@@ -764,6 +765,76 @@ static void test_binary_modulation(void)
     }
 }
 
+// The LUT layer put together from its parts (StochasticLutN -> StochasticBatchNormalization -> HardTanh) against the fused
+// DifferentiableLutN with the same wiring and table, in the shape of the reference's own comparison of the two
+// (tests/gtest/SparseLutNTest.cpp:19-299), and with memory saving (intermediate results recomputed in the backward pass) against
+// without, which must give the same bits.
+template <int N>
+static void test_discrete(int I, int O, int F, bool binary)
+{
+    std::mt19937_64 mt(4242 + I + O + F + (binary ? 1 : 0));
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    constexpr int NN = 1 << N;
+    typename bb::DifferentiableLutN<N, float>::create_t fc;
+    fc.output_shape = {O}; fc.binary = binary; fc.momentum = 0.9f;
+    auto fused = bb::DifferentiableLutN<N, float>::Create(fc);
+    typename bb::DifferentiableLutDiscreteN<N, float>::create_t dc;
+    dc.output_shape = {O}; dc.momentum = 0.9f;
+    auto parts = bb::DifferentiableLutDiscreteN<N, float>::Create(dc);
+    auto saving = bb::DifferentiableLutDiscreteN<N, float>::Create(dc);
+    saving->SendCommand("memory_saving true");
+    std::vector<std::int32_t> idx; wire<N>(mt, I, O, idx);
+    std::vector<float> W((size_t)O * NN);
+    for (auto &w : W) { w = uni(mt); }
+    auto set_up = [&](auto &m) {
+        m->SendCommand(binary ? "binary true" : "binary false");
+        m->SendCommand("lut_binarize false");
+        m->SetInputShape({I});
+        for (int o = 0; o < O; ++o) for (int i = 0; i < N; ++i) { m->SetNodeConnectionIndex(o, i, idx[(size_t)o * N + i]); }
+        auto Wp = m->lock_W();
+        for (size_t k = 0; k < W.size(); ++k) { Wp[(bb::index_t)k] = W[k]; }
+    };
+    set_up(fused); set_up(parts); set_up(saving);
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), dy_buf(F, {O}, BB_TYPE_FP32);
+    for (int loop = 0; loop < 2; ++loop) {
+        for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, uni(mt)); }
+        for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dy_buf.SetFP32(f, n, uni(mt) - 0.5f); }
+        bb::FrameBuffer y0 = fused->Forward(x_buf, true), y1 = parts->Forward(x_buf, true), y2 = saving->Forward(x_buf, true);
+        bb::FrameBuffer dx0 = fused->Backward(dy_buf), dx1 = parts->Backward(dy_buf), dx2 = saving->Backward(dy_buf);
+        CHECK(same_bits(y1, y2) && same_bits(dx1, dx2), "DifferentiableLutDiscrete%d: memory saving changes the result", N);
+        std::vector<float> a, b;
+        read_fp32(y0, a); read_fp32(y1, b);
+        if (binary) {
+            size_t mism = 0;
+            for (size_t k = 0; k < a.size(); ++k) { mism += ((a[k] > 0.5f) != (b[k] > 0.0f)); }     // the fused layer writes 1 / 0, the activation +1 / -1
+            CHECK(mism <= 2 + a.size() / 10000, "DifferentiableLutDiscrete%d binary y: %zu of %zu differ from the fused layer", N, mism, a.size());
+        }
+        else {
+            CHECK(max_diff(a, b) <= 1e-5, "DifferentiableLutDiscrete%d y differs from the fused layer by %g", N, max_diff(a, b));
+            read_fp32(dx0, a); read_fp32(dx1, b);
+            CHECK(max_diff(a, b) <= 1e-4 * std::max(1e-3, max_abs(a)), "DifferentiableLutDiscrete%d dx differs from the fused layer by %g of %g", N, max_diff(a, b), max_abs(a));
+            std::vector<float> g0((size_t)O * NN), g1((size_t)O * NN);
+            { auto p = fused->lock_dW_const(); auto q = parts->lock_dW_const(); for (size_t k = 0; k < g0.size(); ++k) { g0[k] = p[(bb::index_t)k]; g1[k] = q[(bb::index_t)k]; } }
+            CHECK(max_diff(g0, g1) <= 1e-4 * std::max(1e-3, max_abs(g0)), "DifferentiableLutDiscrete%d dW differs from the fused layer by %g of %g", N, max_diff(g0, g1), max_abs(g0));
+        }
+        std::vector<float> m0((size_t)O), m1((size_t)O), v0((size_t)O), v1((size_t)O);
+        { auto p = fused->lock_mean_const(); auto q = parts->lock_mean_const(); auto r = fused->lock_var_const(); auto t = parts->lock_var_const();
+          for (int o = 0; o < O; ++o) { m0[(size_t)o] = p[o]; m1[(size_t)o] = q[o]; v0[(size_t)o] = r[o]; v1[(size_t)o] = t[o]; } }
+        CHECK(max_diff(m0, m1) <= 1e-5 && max_diff(v0, v1) <= 2e-5, "DifferentiableLutDiscrete%d running statistics differ by %g, %g", N, max_diff(m0, m1), max_diff(v0, v1));
+        { auto p = parts->lock_dW_const(); auto q = saving->lock_dW_const(); size_t bad = 0; for (bb::index_t k = 0; k < (bb::index_t)O * NN; ++k) { bad += (p[k] != q[k]); }
+          CHECK(bad == 0, "DifferentiableLutDiscrete%d: memory saving changes %zu table gradients", N, bad); }
+    }
+    // through a stream and back
+    std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+    parts->DumpObject(ss);
+    auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+    CHECK((bool)again && again->GetObjectName() == parts->GetObjectName() && again->GetOutputNodeSize() == O, "DifferentiableLutDiscrete reload");
+    if (again) {
+        bb::FrameBuffer y1 = parts->Forward(x_buf, false), y3 = again->Forward(x_buf, false);
+        CHECK(same_bits(y1, y3), "reloaded DifferentiableLutDiscrete%d differs", N);
+    }
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -922,6 +993,10 @@ int main(void)
         test_max_lut();
         test_reduce_and_mean_squared_error();
         test_binary_modulation();
+        test_discrete<6>(24, 16, 200, false);
+        test_discrete<6>(24, 16, 200, true);
+        test_discrete<4>(12, 30, 1024, false);
+        test_discrete<6>(6, 1, 39, false);
         test_tail();
         test_hand_off_through_files();
     }

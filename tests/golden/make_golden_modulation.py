@@ -1,7 +1,8 @@
 """Writes tests/golden/modulation.npz: inputs and outputs of the reference's own RealToBinary, BinaryToReal, Binarize and HardTanh host
 classes (include/bb/RealToBinary.h:266-344, BinaryToReal.h:205-352, Binarize.h:142-285, HardTanh.h:133-271), run through
 oracle/_ref/libbbref.so, with the objects they serialize to, and BinaryModulation objects (include/bb/BinaryModulation.h:370-394) around
-two DifferentiableLut6 layers that the reference wired and initialised from a seed.
+two DifferentiableLut6 layers, and DifferentiableLutDiscrete6 objects (include/bb/DifferentiableLutDiscreteN.h:392-407), whose LUT layers the
+reference wired and initialised from a seed.
 
 RealToBinary cases come in two kinds.  "dyadic": inputs on a grid of 1/256 with the range [0, 1] and modulation sizes that are powers
 of two, so that every operation of the layer is exact and the reference's build flags (which fuse some multiply-add pairs) cannot
@@ -36,6 +37,10 @@ ACTIVATION = [("binarize", 5, 33, 0.0, -1.0, 1.0, -1.0, 1.0, ""), ("binarize", 3
 # modulation, depth modulation, seed, dumped after an inference pass, name
 MODULATION = [(False, 20, 36, 12, 7, 0, 1, 3, False, ""), (False, 12, 24, 6, 3, 15, 2, 5, True, "net"), (True, 20, 36, 12, 7, 0, 1, 3, False, ""),
               (True, 16, 30, 10, 1, 4, 1, 8, True, "bits")]
+# DifferentiableLutDiscrete6 (StochasticLut6 -> StochasticBatchNormalization -> HardTanh): bit activations, input nodes, output nodes,
+# seed, batch normalisation, memory saving, name
+DISCRETE = [(False, 24, 16, 2, True, False, ""), (False, 12, 40, 6, False, True, "plain"), (True, 24, 16, 2, True, True, "packed"),
+            (True, 30, 7, 9, True, False, "")]
 
 
 def clear_tail(words, frames):
@@ -100,6 +105,12 @@ def main():
         out[q + "args"] = np.array([int(bit), I, o1, o2, tm, im, dm, seed, int(infer)], np.int64)
         out[q + "name"] = np.frombuffer(name.encode(), np.uint8)
         out[q + "object"] = oracle.ref_dump_binary_modulation_object(I, o1, o2, tm, im, dm, bit=bit, seed=seed, run_inference=infer, name=name)
+    out["discrete_count"] = np.array([len(DISCRETE)], np.int32)
+    for k, (bit, I, O, seed, bn, saving, name) in enumerate(DISCRETE):
+        q = "d%d_" % k
+        out[q + "args"] = np.array([int(bit), I, O, seed, int(bn), int(saving)], np.int64)
+        out[q + "name"] = np.frombuffer(name.encode(), np.uint8)
+        out[q + "object"] = oracle.ref_dump_discrete_lut_object(I, O, bit=bit, seed=seed, batch_norm=bn, memory_saving=saving, name=name)
     np.savez_compressed(os.path.join(OUT, "modulation.npz"), **out)
     print("wrote modulation.npz")
 
