@@ -19,6 +19,7 @@
 #include "tail_kernels.hpp"
 #include "bn_kernels.hpp"
 #include "modulation_kernels.hpp"
+#include "pooling_kernels.hpp"
 
 using namespace bbhip;
 
@@ -2008,6 +2009,184 @@ int bbhip_fp32_BinaryToReal_Backward(float const *dev_dy_buf, float *dev_dx_buf,
     else      { hipLaunchKernelGGL((binary_to_real_backward_kernel<1>), dim3(blocks), dim3(kModBlock), 0, st, a, x_frame_size); }
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+
+// ---- MaxPooling, UpSampling ----
+// rows = the rows of the launch's index space, an image of (row_h, row_w) pixels per channel; items = frames or words per row
+static int window_grid(WindowArgs &a, int c, int row_h, int row_w, int items, int per_thread, unsigned &blocks, char const *name)
+{
+    long long const rows = (long long)c * row_h * row_w;
+    int const per_row = ceil_div(items, kPoolBlock * per_thread);
+    if (rows > 0x7fffffffLL || rows * per_row > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    a.f_blocks = make_tile_divisor(per_row);
+    a.row_w = make_tile_divisor(row_w);
+    a.row_h = make_tile_divisor(row_h);
+    blocks = (unsigned)(rows * per_row);
+    return 0;
+}
+
+static int check_pooling(void const *p0, void const *p1, void const *p2, int fh, int fw, int w, int h, int ow, int oh, int c, int frame_size,
+                         char const *name)
+{
+    if (!(p0 && p1 && p2)) { return fail("%s: null buffer", name); }
+    if (!(fh > 0 && fw > 0 && w > 0 && h > 0 && c > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", name); }
+    if (ow != (w + fw - 1) / fw || oh != (h + fh - 1) / fh) { return fail("%s: output size must be ceil(input / filter)", name); }
+    if ((long long)c * h * w > 0x7fffffffLL) { return fail("%s: image too large", name); }
+    return 0;
+}
+
+int bbhip_fp32_MaxPooling_Forward(float const *dev_x_buf, float *dev_y_buf, int *dev_argmax_buf, int filter_h_size, int filter_w_size,
+                                  int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                  int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_pooling(dev_x_buf, dev_y_buf, dev_argmax_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size, output_h_size,
+                      c_size, frame_size, __func__)) { return 1; }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    WindowArgs a{};
+    a.x = dev_x_buf; a.out = dev_y_buf; a.argmax_out = dev_argmax_buf;
+    a.fh = filter_h_size; a.fw = filter_w_size; a.w = input_w_size; a.h = input_h_size; a.ow = output_w_size; a.oh = output_h_size;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    bool const wide = bn_rows_aligned(dev_x_buf, dev_y_buf, dev_argmax_buf, frame_stride, frame_stride);
+    bool const two = filter_h_size == 2 && filter_w_size == 2;
+    unsigned blocks;
+    if (window_grid(a, c_size, output_h_size, output_w_size, frame_size, wide ? 4 : 1, blocks, __func__)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    dim3 const grid(blocks), block(kPoolBlock);
+    if (wide) { if (two) { hipLaunchKernelGGL((max_pooling_forward_kernel<4, true>), grid, block, 0, st, a); }
+                else     { hipLaunchKernelGGL((max_pooling_forward_kernel<4, false>), grid, block, 0, st, a); } }
+    else      { if (two) { hipLaunchKernelGGL((max_pooling_forward_kernel<1, true>), grid, block, 0, st, a); }
+                else     { hipLaunchKernelGGL((max_pooling_forward_kernel<1, false>), grid, block, 0, st, a); } }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_bit_MaxPooling_Forward(int const *dev_x_buf, int *dev_y_buf, int filter_h_size, int filter_w_size, int input_w_size,
+                                 int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride,
+                                 void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_pooling(dev_x_buf, dev_y_buf, dev_y_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size, output_h_size,
+                      c_size, frame_size, __func__)) { return 1; }
+    int const words = (frame_size + 31) / 32;
+    if (frame_stride < words) { return fail("%s: frame stride shorter than the frames", __func__); }
+    WindowArgs a{};
+    a.x = dev_x_buf; a.out = dev_y_buf;
+    a.fh = filter_h_size; a.fw = filter_w_size; a.w = input_w_size; a.h = input_h_size; a.ow = output_w_size; a.oh = output_h_size;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    unsigned blocks;
+    if (window_grid(a, c_size, output_h_size, output_w_size, words, 1, blocks, __func__)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    hipLaunchKernelGGL(max_pooling_bit_forward_kernel, dim3(blocks), dim3(kPoolBlock), 0, st, a, words);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_MaxPooling_Backward(int const *dev_argmax_buf, float const *dev_dy_buf, float *dev_dx_buf, int filter_h_size, int filter_w_size,
+                                   int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                   int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_pooling(dev_argmax_buf, dev_dy_buf, dev_dx_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size,
+                      output_h_size, c_size, frame_size, __func__)) { return 1; }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    WindowArgs a{};
+    a.argmax_in = dev_argmax_buf; a.dy = dev_dy_buf; a.out = dev_dx_buf;
+    a.fh = filter_h_size; a.fw = filter_w_size; a.w = input_w_size; a.h = input_h_size; a.ow = output_w_size; a.oh = output_h_size;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    bool const wide = bn_rows_aligned(dev_argmax_buf, dev_dy_buf, dev_dx_buf, frame_stride, frame_stride);
+    unsigned blocks;
+    if (window_grid(a, c_size, output_h_size, output_w_size, frame_size, wide ? 4 : 1, blocks, __func__)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    if (wide) { hipLaunchKernelGGL((max_pooling_backward_kernel<4>), dim3(blocks), dim3(kPoolBlock), 0, st, a); }
+    else      { hipLaunchKernelGGL((max_pooling_backward_kernel<1>), dim3(blocks), dim3(kPoolBlock), 0, st, a); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_bit_fp32_MaxPooling_Backward(int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int filter_h_size, int filter_w_size,
+                                       int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                       int forward_frame_stride, int backward_frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    if (check_pooling(dev_x_buf, dev_dy_buf, dev_dx_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size, output_h_size,
+                      c_size, frame_size, __func__)) { return 1; }
+    if (forward_frame_stride < (frame_size + 31) / 32 || backward_frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    WindowArgs a{};
+    a.x = dev_x_buf; a.dy = dev_dy_buf; a.out = dev_dx_buf;
+    a.fh = filter_h_size; a.fw = filter_w_size; a.w = input_w_size; a.h = input_h_size; a.ow = output_w_size; a.oh = output_h_size;
+    a.frame_size = frame_size; a.x_stride = forward_frame_stride; a.out_stride = backward_frame_stride;
+    unsigned blocks;
+    if (window_grid(a, c_size, output_h_size, output_w_size, frame_size, 1, blocks, __func__)) { return 1; }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    hipLaunchKernelGGL(max_pooling_bit_backward_kernel, dim3(blocks), dim3(kPoolBlock), 0, st, a);
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int launch_up_sampling(void const *x, float const *dy, void *out, bool bit, bool backward, int input_w_size, int input_h_size, int c_size,
+                              int filter_w_size, int filter_h_size, int fill, int frame_size, int frame_stride, void *stream, char const *name)
+{
+    if (!((backward ? (void const *)dy : x) && out)) { return fail("%s: null buffer", name); }
+    if (!(filter_h_size > 0 && filter_w_size > 0 && input_w_size > 0 && input_h_size > 0 && c_size > 0 && frame_size > 0)) {
+        return fail("%s: sizes must be positive", name);
+    }
+    long long const out_pixels = (long long)c_size * input_h_size * filter_h_size * input_w_size * filter_w_size;
+    if ((long long)input_h_size * filter_h_size > 0x7fffffffLL || (long long)input_w_size * filter_w_size > 0x7fffffffLL || out_pixels > 0x7fffffffLL) {
+        return fail("%s: image too large", name);
+    }
+    int const items = bit ? (frame_size + 31) / 32 : frame_size;
+    if (frame_stride < items) { return fail("%s: frame stride shorter than the frames", name); }
+    WindowArgs a{};
+    a.x = x; a.dy = dy; a.out = out;
+    a.fh = filter_h_size; a.fw = filter_w_size; a.w = input_w_size; a.h = input_h_size; a.fill = fill;
+    a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
+    bool const wide = !bit && bn_rows_aligned(backward ? (void const *)dy : x, out, out, frame_stride, frame_stride);
+    unsigned blocks;
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    if (backward) {
+        if (window_grid(a, c_size, input_h_size, input_w_size, items, wide ? 4 : 1, blocks, name)) { return 1; }
+        ScopedTimer tm(kTimeOther, st);
+        if (wide) { hipLaunchKernelGGL((up_sampling_backward_kernel<4>), dim3(blocks), dim3(kPoolBlock), 0, st, a); }
+        else      { hipLaunchKernelGGL((up_sampling_backward_kernel<1>), dim3(blocks), dim3(kPoolBlock), 0, st, a); }
+    }
+    else {
+        if (window_grid(a, c_size, input_h_size * filter_h_size, input_w_size * filter_w_size, items, wide ? 4 : 1, blocks, name)) { return 1; }
+        ScopedTimer tm(kTimeOther, st);
+        if (bit)       { hipLaunchKernelGGL((up_sampling_forward_kernel<true, 1>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items); }
+        else if (wide) { hipLaunchKernelGGL((up_sampling_forward_kernel<false, 4>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items); }
+        else           { hipLaunchKernelGGL((up_sampling_forward_kernel<false, 1>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items); }
+    }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_fp32_UpSampling_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                  int filter_h_size, int fill, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_up_sampling(dev_x_buf, nullptr, dev_y_buf, false, false, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
+                              frame_size, frame_stride, stream, __func__);
+}
+
+int bbhip_bit_UpSampling_Forward(int const *dev_x_buf, int *dev_y_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                 int filter_h_size, int fill, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_up_sampling(dev_x_buf, nullptr, dev_y_buf, true, false, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
+                              frame_size, frame_stride, stream, __func__);
+}
+
+int bbhip_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                   int filter_h_size, int fill, int frame_size, int frame_stride, void *stream)
+{
+    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    return launch_up_sampling(nullptr, dev_dy_buf, dev_dx_buf, false, true, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
+                              frame_size, frame_stride, stream, __func__);
 }
 
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,

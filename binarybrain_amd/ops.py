@@ -392,6 +392,65 @@ def hard_tanh_backward(x, dy, frame_size, lo=-1.0, hi=1.0):
     return dx
 
 
+def _pool_out(h, w, fh, fw):
+    return (h + fh - 1) // fh, (w + fw - 1) // fw
+
+
+def max_pooling_forward(x, c, h, w, fh, fw, frame_size):
+    """fp32 x [c * h * w, stride] -> (y, argmax) [c * oh * ow, stride]"""
+    _dev(x)
+    oh, ow = _pool_out(h, w, fh, fw)
+    y = torch.empty((c * oh * ow, x.shape[1]), dtype=torch.float32, device=x.device)
+    arg = torch.empty((c * oh * ow, x.shape[1]), dtype=torch.int32, device=x.device)
+    check(lib().bbhip_fp32_MaxPooling_Forward(ptr(x), ptr(y), ptr(arg), fh, fw, w, h, ow, oh, c, frame_size, x.shape[1], stream_ptr()))
+    return y, arg
+
+
+def max_pooling_backward(argmax, dy, c, h, w, fh, fw, frame_size):
+    _dev(argmax, dy)
+    oh, ow = _pool_out(h, w, fh, fw)
+    dx = torch.empty((c * h * w, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_MaxPooling_Backward(ptr(argmax), ptr(dy), ptr(dx), fh, fw, w, h, ow, oh, c, frame_size, dy.shape[1], stream_ptr()))
+    return dx
+
+
+def bit_max_pooling_forward(xbits, c, h, w, fh, fw, frame_size):
+    _dev(xbits)
+    oh, ow = _pool_out(h, w, fh, fw)
+    y = torch.zeros((c * oh * ow, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    check(lib().bbhip_bit_MaxPooling_Forward(ptr(xbits), ptr(y), fh, fw, w, h, ow, oh, c, frame_size, xbits.shape[1], stream_ptr()))
+    return y
+
+
+def bit_max_pooling_backward(xbits, dy, c, h, w, fh, fw, frame_size):
+    _dev(xbits, dy)
+    oh, ow = _pool_out(h, w, fh, fw)
+    dx = torch.empty((c * h * w, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_bit_fp32_MaxPooling_Backward(ptr(xbits), ptr(dy), ptr(dx), fh, fw, w, h, ow, oh, c, frame_size, xbits.shape[1], dy.shape[1],
+                                                   stream_ptr()))
+    return dx
+
+
+def up_sampling_forward(x, c, h, w, fh, fw, frame_size, fill=True):
+    """x [c * h * w, stride], fp32 or int32 packed words -> y [c * h fh * w fw, stride] of the same type"""
+    _dev(x)
+    if x.dtype == torch.int32:
+        y = torch.zeros((c * h * fh * w * fw, x.shape[1]), dtype=torch.int32, device=x.device)
+        f = lib().bbhip_bit_UpSampling_Forward
+    else:
+        y = torch.empty((c * h * fh * w * fw, x.shape[1]), dtype=torch.float32, device=x.device)
+        f = lib().bbhip_fp32_UpSampling_Forward
+    check(f(ptr(x), ptr(y), w, h, c, fw, fh, int(fill), frame_size, x.shape[1], stream_ptr()))
+    return y
+
+
+def up_sampling_backward(dy, c, h, w, fh, fw, frame_size, fill=True):
+    _dev(dy)
+    dx = torch.empty((c * h * w, dy.shape[1]), dtype=torch.float32, device=dy.device)
+    check(lib().bbhip_fp32_UpSampling_Backward(ptr(dy), ptr(dx), w, h, c, fw, fh, int(fill), frame_size, dy.shape[1], stream_ptr()))
+    return dx
+
+
 def loss_mean_squared_error(y, t, frame_size, loss_buf, batch_size=None, reduction_sum=False):
     """-> dy; loss_buf (float64, device, any length >= 1) receives the batch's partial sums ON TOP of what it holds.  The layer's loss is
     loss_buf.sum() / frames seen (the sum itself with reduction "sum")."""

@@ -398,6 +398,61 @@ inline int bbcu_fp32_HardTanh_Backward(const float *dev_x_buf, const float *dev_
     return 0;
 }
 
+/* ---- MaxPooling / UpSampling, include/bbcu/bbcu.h:949-1068 ---- */
+inline int bbcu_fp32_MaxPooling_Forward(float const *dev_x_buf, float *dev_y_buf, int *dev_argmax_buf, int filter_h_size, int filter_w_size,
+        int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride,
+        cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_MaxPooling_Forward(dev_x_buf, dev_y_buf, dev_argmax_buf, filter_h_size, filter_w_size, input_w_size, input_h_size,
+                                                output_w_size, output_h_size, c_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_bit_MaxPooling_Forward(int const *dev_x_buf, int *dev_y_buf, int filter_h_size, int filter_w_size, int input_w_size,
+        int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_bit_MaxPooling_Forward(dev_x_buf, dev_y_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size,
+                                               output_h_size, c_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_MaxPooling_Backward(int const *dev_argmax_buf, float const *dev_dy_buf, float *dev_dx_buf, int filter_h_size,
+        int filter_w_size, int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+        int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_MaxPooling_Backward(dev_argmax_buf, dev_dy_buf, dev_dx_buf, filter_h_size, filter_w_size, input_w_size, input_h_size,
+                                                 output_w_size, output_h_size, c_size, frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_bit_fp32_MaxPooling_Backward(int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int filter_h_size,
+        int filter_w_size, int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+        int forward_frame_stride, int backward_frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_bit_fp32_MaxPooling_Backward(dev_x_buf, dev_dy_buf, dev_dx_buf, filter_h_size, filter_w_size, input_w_size, input_h_size,
+                                                     output_w_size, output_h_size, c_size, frame_size, forward_frame_stride,
+                                                     backward_frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_UpSampling_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size, int c_size,
+        int filter_w_size, int filter_h_size, int fill, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_UpSampling_Forward(dev_x_buf, dev_y_buf, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
+                                                frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_bit_UpSampling_Forward(int const *dev_x_buf, int *dev_y_buf, int input_w_size, int input_h_size, int c_size,
+        int filter_w_size, int filter_h_size, int fill, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_bit_UpSampling_Forward(dev_x_buf, dev_y_buf, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
+                                               frame_size, frame_stride, streamId));
+    return 0;
+}
+inline int bbcu_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_w_size, int input_h_size, int c_size,
+        int filter_w_size, int filter_h_size, int fill, int frame_size, int frame_stride, cudaStream_t streamId = 0)
+{
+    BBCU_HIP_CALL(bbhip_fp32_UpSampling_Backward(dev_dy_buf, dev_dx_buf, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
+                                                 frame_size, frame_stride, streamId));
+    return 0;
+}
+
 /* ---- Im2Col / Col2Im, include/bbcu/bbcu.h:1076-1186 ---- */
 inline int bbcu_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
         int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size, int output_w_size,

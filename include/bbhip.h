@@ -312,6 +312,39 @@ int bbhip_fp32_HardTanh_Forward(float const *dev_x_buf, float *dev_y_buf, float 
 int bbhip_fp32_HardTanh_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, float limit_min, float limit_max,
                                  int node_size, int frame_size, int frame_stride, void *stream);
 
+/* ---- MaxPooling, UpSampling ----
+ * Windows of filter_h x filter_w tile the image without overlap, the last ones cut off at the border: output = ceil(input / filter).
+ * Bit-exact with the reference's host loops. */
+/* bbcu_fp32_MaxPooling_Forward, include/bbcu/bbcu.h:949-964: y = the largest value of the window, argmax = the position of its first
+ * occurrence counted in (fy, fx) order over the window's positions inside the image (include/bb/MaxPooling.h:251-284) */
+int bbhip_fp32_MaxPooling_Forward(float const *dev_x_buf, float *dev_y_buf, int *dev_argmax_buf, int filter_h_size, int filter_w_size,
+                                  int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                  int frame_stride, void *stream);
+/* bbcu_bit_MaxPooling_Forward, include/bbcu/bbcu.h:966-980: packed rows, y = the OR of the window (bits past the last frame written as 0) */
+int bbhip_bit_MaxPooling_Forward(int const *dev_x_buf, int *dev_y_buf, int filter_h_size, int filter_w_size, int input_w_size,
+                                 int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride,
+                                 void *stream);
+/* bbcu_fp32_MaxPooling_Backward, include/bbcu/bbcu.h:983-998: the recorded position of each window receives dy, the others 0 */
+int bbhip_fp32_MaxPooling_Backward(int const *dev_argmax_buf, float const *dev_dy_buf, float *dev_dx_buf, int filter_h_size, int filter_w_size,
+                                   int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                   int frame_stride, void *stream);
+/* bbcu_bit_fp32_MaxPooling_Backward, include/bbcu/bbcu.h:1000-1016: dy goes to the first set input of each window in (fy, fx) order,
+ * to none when none is set (include/bb/MaxPooling.h:551-579); x is the packed forward input */
+int bbhip_bit_fp32_MaxPooling_Backward(int const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int filter_h_size, int filter_w_size,
+                                       int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                       int forward_frame_stride, int backward_frame_stride, void *stream);
+/* bbcu_fp32_UpSampling_Forward, include/bbcu/bbcu.h:1024-1037: every input pixel becomes a filter_h x filter_w block, all of it (fill)
+ * or only its position (filter_h / 2, filter_w / 2) with zeros around (include/bb/UpSampling.h:223-259) */
+int bbhip_fp32_UpSampling_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                  int filter_h_size, int fill, int frame_size, int frame_stride, void *stream);
+/* bbcu_bit_UpSampling_Forward, include/bbcu/bbcu.h:1039-1052: packed rows of frame_stride words */
+int bbhip_bit_UpSampling_Forward(int const *dev_x_buf, int *dev_y_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                 int filter_h_size, int fill, int frame_size, int frame_stride, void *stream);
+/* bbcu_fp32_UpSampling_Backward, include/bbcu/bbcu.h:1055-1068: dx = the sum of dy over the block in (fy, fx) order, or dy at the
+ * block's position (filter_h / 2, filter_w / 2) (include/bb/UpSampling.h:321-353) */
+int bbhip_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                   int filter_h_size, int fill, int frame_size, int frame_stride, void *stream);
+
 /* ---- mean squared error ---- */
 /* bbcu_fp32_LossMeanSquaredError, include/bbcu/bbcu.h:1487-1500: dy = (y - t) * grad_reduction (the caller passes 2 / (nodes * batch)
  * or 2); dev_loss_buf[s] += the sum over the frames s, s + loss_buf_size, ... and all nodes of (float)(y - t)^2 * loss_reduction in

@@ -388,6 +388,66 @@ def hard_tanh_backward(x, dy, frame_size, lo=-1.0, hi=1.0):
     return dx
 
 
+def _pool_geometry(h, w, fh, fw):
+    return (h + fh - 1) // fh, (w + fw - 1) // fw
+
+
+def max_pooling_forward(x, c, h, w, fh, fw, frame_size):
+    """fp32 x [c * h * w, stride] -> (y, argmax) [c * oh * ow, stride] (include/bb/MaxPooling.h:251-284)"""
+    x = _c(x, np.float32)
+    oh, ow = _pool_geometry(h, w, fh, fw)
+    y = np.zeros((c * oh * ow, x.shape[1]), np.float32); arg = np.zeros((c * oh * ow, x.shape[1]), np.int32)
+    lib().oracle_fp32_MaxPooling_Forward(_ptr(x), _ptr(y), _ptr(arg), C.c_int(fh), C.c_int(fw), C.c_int(w), C.c_int(h), C.c_int(ow), C.c_int(oh),
+                                         C.c_int(c), C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y, arg
+
+
+def max_pooling_backward(argmax, dy, c, h, w, fh, fw, frame_size):
+    argmax = _c(argmax, np.int32); dy = _c(dy, np.float32)
+    oh, ow = _pool_geometry(h, w, fh, fw)
+    dx = np.zeros((c * h * w, dy.shape[1]), np.float32)
+    lib().oracle_fp32_MaxPooling_Backward(_ptr(argmax), _ptr(dy), _ptr(dx), C.c_int(fh), C.c_int(fw), C.c_int(w), C.c_int(h), C.c_int(ow),
+                                          C.c_int(oh), C.c_int(c), C.c_int(frame_size), C.c_int(dy.shape[1]))
+    return dx
+
+
+def bit_max_pooling_forward(xbits, c, h, w, fh, fw, frame_size):
+    """packed x [c * h * w, words] -> packed y: the OR of each window (include/bb/MaxPooling.h:340-370)"""
+    xbits = _c(xbits, np.int32)
+    oh, ow = _pool_geometry(h, w, fh, fw)
+    y = np.zeros((c * oh * ow, xbits.shape[1]), np.int32)
+    lib().oracle_bit_MaxPooling_Forward(_ptr(xbits), _ptr(y), C.c_int(fh), C.c_int(fw), C.c_int(w), C.c_int(h), C.c_int(ow), C.c_int(oh),
+                                        C.c_int(c), C.c_int(frame_size), C.c_int(xbits.shape[1]))
+    return y
+
+
+def bit_max_pooling_backward(xbits, dy, c, h, w, fh, fw, frame_size):
+    """dy goes to the first set input of each window (include/bb/MaxPooling.h:551-579)"""
+    xbits = _c(xbits, np.int32); dy = _c(dy, np.float32)
+    oh, ow = _pool_geometry(h, w, fh, fw)
+    dx = np.zeros((c * h * w, dy.shape[1]), np.float32)
+    lib().oracle_bit_fp32_MaxPooling_Backward(_ptr(xbits), _ptr(dy), _ptr(dx), C.c_int(fh), C.c_int(fw), C.c_int(w), C.c_int(h), C.c_int(ow),
+                                              C.c_int(oh), C.c_int(c), C.c_int(frame_size), C.c_int(xbits.shape[1]), C.c_int(dy.shape[1]))
+    return dx
+
+
+def up_sampling_forward(x, c, h, w, fh, fw, frame_size, fill=True, bit=False):
+    """x [c * h * w, stride] (fp32 or packed words) -> y [c * h fh * w fw, stride] (include/bb/UpSampling.h:223-259)"""
+    x = _c(x, np.int32 if bit else np.float32)
+    y = np.zeros((c * h * fh * w * fw, x.shape[1]), x.dtype)
+    f = lib().oracle_bit_UpSampling_Forward if bit else lib().oracle_fp32_UpSampling_Forward
+    f(_ptr(x), _ptr(y), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(fw), C.c_int(fh), C.c_int(int(fill)), C.c_int(frame_size), C.c_int(x.shape[1]))
+    return y
+
+
+def up_sampling_backward(dy, c, h, w, fh, fw, frame_size, fill=True):
+    dy = _c(dy, np.float32)
+    dx = np.zeros((c * h * w, dy.shape[1]), np.float32)
+    lib().oracle_fp32_UpSampling_Backward(_ptr(dy), _ptr(dx), C.c_int(w), C.c_int(h), C.c_int(c), C.c_int(fw), C.c_int(fh), C.c_int(int(fill)),
+                                          C.c_int(frame_size), C.c_int(dy.shape[1]))
+    return dx
+
+
 def loss_mean_squared_error(y, t, frame_size, batch_size=None, reduction_sum=False, loss=0.0):
     """-> (dy, loss accumulator): the reference's host loop (include/bb/LossMeanSquaredError.h:121-169) for one batch; `loss` is the
     accumulator before the batch.  The layer's loss is accumulator / frames seen (the accumulator itself with reduction "sum")."""
@@ -953,6 +1013,41 @@ def ref_dump_discrete_lut_object(input_nodes, output_nodes, bit=False, seed=1, b
           C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size))
     assert r > 0, r
     return out[:r].copy()
+
+
+def ref_max_pooling(x, c, h, w, fh, fw, frames, bit=False, dy=None, name="", want_object=False):
+    """The reference's MaxPooling host path on dense arrays -> (y, dx, object bytes); x [c * h * w, frames] fp32 or [.., words] bits."""
+    x = _c(x, np.int32 if bit else np.float32)
+    oh, ow = _pool_geometry(h, w, fh, fw)
+    O = c * oh * ow
+    y = np.zeros((O, (frames + 31) // 32), np.int32) if bit else np.zeros((O, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((c * h * w, frames), np.float32)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_MaxPooling
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(fh), C.c_int(fw), C.c_int(frames), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx),
+          C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
+
+
+def ref_up_sampling(x, c, h, w, fh, fw, frames, fill=True, bit=False, dy=None, name="", want_object=False):
+    """The reference's UpSampling host path on dense arrays -> (y, dx, object bytes)."""
+    x = _c(x, np.int32 if bit else np.float32)
+    O = c * h * fh * w * fw
+    y = np.zeros((O, (frames + 31) // 32), np.int32) if bit else np.zeros((O, frames), np.float32)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, np.float32); dx = np.zeros((c * h * w, frames), np.float32)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_UpSampling
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(fh), C.c_int(fw), C.c_int(int(fill)), C.c_int(frames), _ptr(x), _ptr(y),
+          _ptr(dy), _ptr(dx), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
 
 
 def ref_mean_squared_error(y, t, frames, batches=1, reduction_sum=False):

@@ -39,6 +39,9 @@
  *     (tests/golden/modulation.npz), the known answers of
  *     tests/gtest/RealToBinaryTest.cpp, BinaryToRealTest.cpp, BinarizeTest.cpp,
  *     and numpy restatements.
+ *   - MaxPooling *, UpSampling *: bit-exact against the reference's classes
+ *     (oracle/_ref), vectors written from them (tests/golden/pooling.npz), the
+ *     known answers of tests/gtest/MaxPoolingTest.cpp and UpSamplingTest.cpp, numpy.
  *
  * Array conventions (the reference's FrameBuffer layout, include/bb/FrameBuffer.h:28-46,
  * 927-939): node-major, frame-minor; element (node n, frame f) of an fp32
@@ -1468,6 +1471,197 @@ void oracle_fp32_HardTanh_Backward(float const *x, float const *dy, float *dx, f
             float const v = x[(long long)node * frame_stride + f];
             if (v <= limit_min || v >= limit_max) { g = 0.0f; }
             dx[(long long)node * frame_stride + f] = g;
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ *  MaxPooling (include/bb/MaxPooling.h): windows of filter_h x filter_w tile the image without overlap, the last ones cut off at
+ *  the border (output = ceil(input / filter)).  fp32 forward (:251-284): the largest value of the window, found with a strict >
+ *  from the lowest float in (fy, fx) order, and the position of its first occurrence counted over the positions inside the image;
+ *  backward (:478-506): that position receives dy, the others 0.  Packed bits, windows below 32 positions (:340-370 forward: the
+ *  OR of the window; :551-579 backward: dy goes to the first set input in (fy, fx) order, nothing when none is set).
+ *  UpSampling (include/bb/UpSampling.h:223-259, :321-353): every input pixel becomes a filter_h x filter_w block, all of it (fill)
+ *  or only its position (filter_h / 2, filter_w / 2) with zeros around; backward sums dy over the block in (fy, fx) order in fp32,
+ *  or takes that one position.
+ *  Pinned by tests/test_oracle_pooling.py: the reference's classes (oracle/_ref), vectors written from them
+ *  (tests/golden/pooling.npz), the known answers of tests/gtest/MaxPoolingTest.cpp and UpSamplingTest.cpp, numpy.
+ * ------------------------------------------------------------------------------------------------------------------- */
+void oracle_fp32_MaxPooling_Forward(float const *x, float *y, int *argmax, int filter_h_size, int filter_w_size, int input_w_size,
+                                    int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride)
+{
+    for (int c = 0; c < c_size; ++c) {
+        for (int oy = 0; oy < output_h_size; ++oy) {
+            for (int ox = 0; ox < output_w_size; ++ox) {
+                long long const out = (((long long)c * output_h_size + oy) * output_w_size + ox) * frame_stride;
+                for (int f = 0; f < frame_size; ++f) {
+                    float max_val = -3.402823466e+38f;      /* std::numeric_limits<float>::lowest() */
+                    int best = 0, arg = 0;
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        int const iy = oy * filter_h_size + fy;
+                        if (iy >= input_h_size) { continue; }
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            int const ix = ox * filter_w_size + fx;
+                            if (ix >= input_w_size) { continue; }
+                            float const v = x[(((long long)c * input_h_size + iy) * input_w_size + ix) * frame_stride + f];
+                            if (v > max_val) { max_val = v; best = arg; }
+                            ++arg;
+                        }
+                    }
+                    y[out + f] = max_val;
+                    argmax[out + f] = best;
+                }
+            }
+        }
+    }
+}
+
+void oracle_fp32_MaxPooling_Backward(int const *argmax, float const *dy, float *dx, int filter_h_size, int filter_w_size, int input_w_size,
+                                     int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride)
+{
+    for (int c = 0; c < c_size; ++c) {
+        for (int oy = 0; oy < output_h_size; ++oy) {
+            for (int ox = 0; ox < output_w_size; ++ox) {
+                long long const out = (((long long)c * output_h_size + oy) * output_w_size + ox) * frame_stride;
+                for (int f = 0; f < frame_size; ++f) {
+                    int arg = 0;
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        int const iy = oy * filter_h_size + fy;
+                        if (iy >= input_h_size) { continue; }
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            int const ix = ox * filter_w_size + fx;
+                            if (ix >= input_w_size) { continue; }
+                            dx[(((long long)c * input_h_size + iy) * input_w_size + ix) * frame_stride + f] = (arg == argmax[out + f]) ? dy[out + f] : 0.0f;
+                            ++arg;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* y rows are frame_stride words; the caller clears them */
+void oracle_bit_MaxPooling_Forward(int const *x, int *y, int filter_h_size, int filter_w_size, int input_w_size, int input_h_size,
+                                   int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride)
+{
+    for (int c = 0; c < c_size; ++c) {
+        for (int oy = 0; oy < output_h_size; ++oy) {
+            for (int ox = 0; ox < output_w_size; ++ox) {
+                int *yr = y + (((long long)c * output_h_size + oy) * output_w_size + ox) * frame_stride;
+                for (int f = 0; f < frame_size; ++f) {
+                    int any = 0;
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        int const iy = oy * filter_h_size + fy;
+                        if (iy >= input_h_size) { continue; }
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            int const ix = ox * filter_w_size + fx;
+                            if (ix >= input_w_size) { continue; }
+                            any |= get_bit(x + (((long long)c * input_h_size + iy) * input_w_size + ix) * frame_stride, f);
+                        }
+                    }
+                    set_bit(yr, f, any);
+                }
+            }
+        }
+    }
+}
+
+void oracle_bit_fp32_MaxPooling_Backward(int const *x, float const *dy, float *dx, int filter_h_size, int filter_w_size, int input_w_size,
+                                         int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
+                                         int forward_frame_stride, int backward_frame_stride)
+{
+    for (int c = 0; c < c_size; ++c) {
+        for (int oy = 0; oy < output_h_size; ++oy) {
+            for (int ox = 0; ox < output_w_size; ++ox) {
+                long long const out = (((long long)c * output_h_size + oy) * output_w_size + ox) * backward_frame_stride;
+                for (int f = 0; f < frame_size; ++f) {
+                    float grad = dy[out + f];
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        int const iy = oy * filter_h_size + fy;
+                        if (iy >= input_h_size) { continue; }
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            int const ix = ox * filter_w_size + fx;
+                            if (ix >= input_w_size) { continue; }
+                            long long const in_node = ((long long)c * input_h_size + iy) * input_w_size + ix;
+                            int const sig = get_bit(x + in_node * forward_frame_stride, f);
+                            dx[in_node * backward_frame_stride + f] = sig ? grad : 0.0f;
+                            if (sig) { grad = 0.0f; }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+void oracle_fp32_UpSampling_Forward(float const *x, float *y, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                    int filter_h_size, int fill, int frame_size, int frame_stride)
+{
+    int const output_h_size = input_h_size * filter_h_size, output_w_size = input_w_size * filter_w_size;
+    for (int c = 0; c < c_size; ++c) {
+        for (int iy = 0; iy < input_h_size; ++iy) {
+            for (int ix = 0; ix < input_w_size; ++ix) {
+                long long const in_node = ((long long)c * input_h_size + iy) * input_w_size + ix;
+                for (int f = 0; f < frame_size; ++f) {
+                    float const v = x[in_node * frame_stride + f];
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            long long const out_node = ((long long)c * output_h_size + iy * filter_h_size + fy) * output_w_size + ix * filter_w_size + fx;
+                            int const centre = (fx == filter_w_size / 2 && fy == filter_h_size / 2);
+                            y[out_node * frame_stride + f] = (fill || centre) ? v : 0.0f;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* y rows are frame_stride words; the caller clears them */
+void oracle_bit_UpSampling_Forward(int const *x, int *y, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                   int filter_h_size, int fill, int frame_size, int frame_stride)
+{
+    int const output_h_size = input_h_size * filter_h_size, output_w_size = input_w_size * filter_w_size;
+    for (int c = 0; c < c_size; ++c) {
+        for (int iy = 0; iy < input_h_size; ++iy) {
+            for (int ix = 0; ix < input_w_size; ++ix) {
+                long long const in_node = ((long long)c * input_h_size + iy) * input_w_size + ix;
+                for (int f = 0; f < frame_size; ++f) {
+                    int const v = get_bit(x + in_node * frame_stride, f);
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            long long const out_node = ((long long)c * output_h_size + iy * filter_h_size + fy) * output_w_size + ix * filter_w_size + fx;
+                            int const centre = (fx == filter_w_size / 2 && fy == filter_h_size / 2);
+                            set_bit(y + out_node * frame_stride, f, (fill || centre) ? v : 0);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+void oracle_fp32_UpSampling_Backward(float const *dy, float *dx, int input_w_size, int input_h_size, int c_size, int filter_w_size,
+                                     int filter_h_size, int fill, int frame_size, int frame_stride)
+{
+    int const output_h_size = input_h_size * filter_h_size, output_w_size = input_w_size * filter_w_size;
+    for (int c = 0; c < c_size; ++c) {
+        for (int iy = 0; iy < input_h_size; ++iy) {
+            for (int ix = 0; ix < input_w_size; ++ix) {
+                long long const in_node = ((long long)c * input_h_size + iy) * input_w_size + ix;
+                for (int f = 0; f < frame_size; ++f) {
+                    float sum = 0;
+                    for (int fy = 0; fy < filter_h_size; ++fy) {
+                        for (int fx = 0; fx < filter_w_size; ++fx) {
+                            long long const out_node = ((long long)c * output_h_size + iy * filter_h_size + fy) * output_w_size + ix * filter_w_size + fx;
+                            int const centre = (fx == filter_w_size / 2 && fy == filter_h_size / 2);
+                            if (fill || centre) { sum += dy[out_node * frame_stride + f]; }
+                        }
+                    }
+                    dx[in_node * frame_stride + f] = sum;
+                }
+            }
         }
     }
 }

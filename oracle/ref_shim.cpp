@@ -43,6 +43,8 @@
 #include "bb/HardTanh.h"
 #include "bb/BinaryModulation.h"
 #include "bb/DifferentiableLutDiscreteN.h"
+#include "bb/MaxPooling.h"
+#include "bb/UpSampling.h"
 
 namespace {
 
@@ -1019,4 +1021,73 @@ extern "C" long bbref_DumpDiscreteLutObject(int bit, int I, int O, int seed, int
     };
     if (bit) { return fill(bb::DifferentiableLutDiscreteN<6, bb::Bit, float>::Create((index_t)O, batch_norm != 0, "", (std::uint64_t)seed)); }
     return fill(bb::DifferentiableLutDiscreteN<6, float, float>::Create((index_t)O, batch_norm != 0, "", (std::uint64_t)seed));
+}
+
+// MaxPooling<BinType, float> and UpSampling<BinType, float> (host paths).  x: [c * h * w][F] fp32 or bits; dy, y: the output shape.
+namespace {
+template <typename BinType>
+long run_max_pooling(int c, int h, int w, int fh, int fw, int F, void const *x, void *y, float const *dy, float *dx, char const *name,
+                     unsigned char *object_out, long cap)
+{
+    auto m = bb::MaxPooling<BinType, float>::Create((index_t)fh, (index_t)fw);
+    m->SendCommand("host_only true");
+    if (name && *name) { m->SetName(name); }
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)c, (index_t)h, (index_t)w}), xtype, true);
+    auto out_shape = m->SetInputShape(xb.GetShape());
+    index_t const I = (index_t)c * h * w, O = bb::CalcShapeSize(out_shape);
+    if (xtype == BB_TYPE_BIT) { put_bit(xb, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(xb, (float const *)x, I, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (yb.GetNodeSize() != O) { return -2; }
+    if (xtype == BB_TYPE_BIT) { get_bit(yb, (std::int32_t *)y, O, (F + 31) / 32); }
+    else                      { get_fp32(yb, (float *)y, O, F); }
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, out_shape, BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, O, F);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, I, F);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+
+template <typename BinType>
+long run_up_sampling(int c, int h, int w, int fh, int fw, int fill, int F, void const *x, void *y, float const *dy, float *dx, char const *name,
+                     unsigned char *object_out, long cap)
+{
+    auto m = bb::UpSampling<BinType, float>::Create((index_t)fh, (index_t)fw, fill != 0);
+    m->SendCommand("host_only true");
+    if (name && *name) { m->SetName(name); }
+    int const xtype = bb::DataType<BinType>::type;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({(index_t)c, (index_t)h, (index_t)w}), xtype, true);
+    auto out_shape = m->SetInputShape(xb.GetShape());
+    index_t const I = (index_t)c * h * w, O = bb::CalcShapeSize(out_shape);
+    if (xtype == BB_TYPE_BIT) { put_bit(xb, (std::int32_t const *)x, I, (F + 31) / 32); }
+    else                      { put_fp32(xb, (float const *)x, I, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (yb.GetNodeSize() != O) { return -2; }
+    if (xtype == BB_TYPE_BIT) { get_bit(yb, (std::int32_t *)y, O, (F + 31) / 32); }
+    else                      { get_fp32(yb, (float *)y, O, F); }
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, out_shape, BB_TYPE_FP32, true);
+        put_fp32(dyb, dy, O, F);
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        get_fp32(dxb, dx, I, F);
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
+}
+}  // namespace
+
+extern "C" long bbref_MaxPooling(int bit, int c, int h, int w, int fh, int fw, int F, void const *x, void *y, float const *dy, float *dx,
+                                 char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_max_pooling<bb::Bit>(c, h, w, fh, fw, F, x, y, dy, dx, name, object_out, cap)
+               : run_max_pooling<float>(c, h, w, fh, fw, F, x, y, dy, dx, name, object_out, cap);
+}
+
+extern "C" long bbref_UpSampling(int bit, int c, int h, int w, int fh, int fw, int fill, int F, void const *x, void *y, float const *dy,
+                                 float *dx, char const *name, unsigned char *object_out, long cap)
+{
+    return bit ? run_up_sampling<bb::Bit>(c, h, w, fh, fw, fill, F, x, y, dy, dx, name, object_out, cap)
+               : run_up_sampling<float>(c, h, w, fh, fw, fill, F, x, y, dy, dx, name, object_out, cap);
 }
