@@ -178,6 +178,23 @@ def bench_conv(args, lib):
         total_ms += med
         kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
     dom = max(kernels, key=lambda k: kernels[k]["ms"])
+    # MaxPooling (what binary networks pool with) and UpSampling at the same maps, listed beside the block's own kernels, not added
+    _, arg = ops.max_pooling_forward(maps, CO, OH, OW, 2, 2, F)
+    PO = CO * (OH // 2) * (OW // 2)
+    maps_bits = ops.binarize_forward(maps, F, 0.5, bit=True, y_stride=synth.frame_stride_bit(F))
+    dup = torch.rand_like(maps)
+    beside = [
+        ("max_pooling_forward_kernel 2x2", lambda: ops.max_pooling_forward(maps, CO, OH, OW, 2, 2, F), e * F * (CO * OH * OW + 2 * PO)),
+        ("max_pooling_backward_kernel 2x2", lambda: ops.max_pooling_backward(arg, dpooled, CO, OH, OW, 2, 2, F), e * F * (CO * OH * OW + 2 * PO)),
+        ("max_pooling_bit_forward_kernel 2x2", lambda: ops.bit_max_pooling_forward(maps_bits, CO, OH, OW, 2, 2, F), F // 8 * (CO * OH * OW + PO)),
+        ("max_pooling_bit_backward_kernel 2x2", lambda: ops.bit_max_pooling_backward(maps_bits, dpooled, CO, OH, OW, 2, 2, F),
+         F // 8 * CO * OH * OW + e * F * (CO * OH * OW + PO)),
+        ("up_sampling_forward_kernel 2x2", lambda: ops.up_sampling_forward(pooled, CO, OH // 2, OW // 2, 2, 2, F), e * F * (CO * OH * OW + PO)),
+        ("up_sampling_backward_kernel 2x2", lambda: ops.up_sampling_backward(dup, CO, OH // 2, OW // 2, 2, 2, F), e * F * (CO * OH * OW + PO)),
+    ]
+    for name, fn, nbytes in beside:
+        med = library_timed_ms(lib, fn, args.steps, args.warmup)
+        kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
     out = {"metric": "conv-block permutation kernels, ms per pass over 256 images (fwd+bwd)", "value": total_ms, "unit": "ms",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": total_ms, "higher_is_better": False, "scaling": "weak",
            "vs_baseline": None, "dtype": "f32", "data": "synthetic",

@@ -1311,12 +1311,19 @@ static int launch_pool(PoolArgs const &a, bool backward, void *stream, char cons
     if (!(a.w > 0 && a.h > 0 && a.c > 0 && a.frame_size > 0)) { return fail("%s: sizes must be positive", name); }
     if (a.ow != (a.w + 1) / 2 || a.oh != (a.h + 1) / 2) { return fail("%s: output size must be ceil(input / 2)", name); }
     if (a.frame_stride < a.frame_size) { return fail("%s: frame stride shorter than the frames", name); }
-    int const f_blocks = ceil_div(a.frame_size, kConvBlock);
+    // four frames per thread with 128-bit accesses where every row starts on 16 bytes
+    uintptr_t const bits = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.out) | reinterpret_cast<uintptr_t>(backward ? a.dy : a.x);
+    bool const wide = (bits & 15u) == 0 && (a.frame_stride & 3) == 0;
+    int const f_blocks = ceil_div(a.frame_size, kConvBlock * (wide ? 4 : 1));
     long long const blocks = (long long)a.c * a.oh * a.ow * f_blocks;
     if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
-    ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
-    if (backward) { hipLaunchKernelGGL(stochastic_maxpool2x2_backward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, f_blocks); }
-    else          { hipLaunchKernelGGL(stochastic_maxpool2x2_forward_kernel, dim3((unsigned)blocks), dim3(kConvBlock), 0, static_cast<hipStream_t>(stream), a, f_blocks); }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    dim3 const grid((unsigned)blocks), block(kConvBlock);
+    if (backward) { if (wide) { hipLaunchKernelGGL((stochastic_maxpool2x2_backward_kernel<4>), grid, block, 0, st, a, f_blocks); }
+                    else      { hipLaunchKernelGGL((stochastic_maxpool2x2_backward_kernel<1>), grid, block, 0, st, a, f_blocks); } }
+    else          { if (wide) { hipLaunchKernelGGL((stochastic_maxpool2x2_forward_kernel<4>), grid, block, 0, st, a, f_blocks); }
+                    else      { hipLaunchKernelGGL((stochastic_maxpool2x2_forward_kernel<1>), grid, block, 0, st, a, f_blocks); } }
     BBHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -2025,6 +2032,19 @@ static int window_grid(WindowArgs &a, int c, int row_h, int row_w, int items, in
     return 0;
 }
 
+// packed rows: (row, word) pairs numbered through, f_blocks = words per row
+static int window_grid_flat(WindowArgs &a, int c, int row_h, int row_w, int words, unsigned &blocks, long long &total, char const *name)
+{
+    long long const rows = (long long)c * row_h * row_w;
+    total = rows * words;
+    if (rows > 0x7fffffffLL || total > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    a.f_blocks = make_tile_divisor(words);
+    a.row_w = make_tile_divisor(row_w);
+    a.row_h = make_tile_divisor(row_h);
+    blocks = (unsigned)((total + kPoolBlock - 1) / kPoolBlock);
+    return 0;
+}
+
 static int check_pooling(void const *p0, void const *p1, void const *p2, int fh, int fw, int w, int h, int ow, int oh, int c, int frame_size,
                          char const *name)
 {
@@ -2076,10 +2096,11 @@ int bbhip_bit_MaxPooling_Forward(int const *dev_x_buf, int *dev_y_buf, int filte
     a.fh = filter_h_size; a.fw = filter_w_size; a.w = input_w_size; a.h = input_h_size; a.ow = output_w_size; a.oh = output_h_size;
     a.frame_size = frame_size; a.x_stride = frame_stride; a.out_stride = frame_stride;
     unsigned blocks;
-    if (window_grid(a, c_size, output_h_size, output_w_size, words, 1, blocks, __func__)) { return 1; }
+    long long total;
+    if (window_grid_flat(a, c_size, output_h_size, output_w_size, words, blocks, total, __func__)) { return 1; }
     hipStream_t const st = static_cast<hipStream_t>(stream);
     ScopedTimer tm(kTimeOther, st);
-    hipLaunchKernelGGL(max_pooling_bit_forward_kernel, dim3(blocks), dim3(kPoolBlock), 0, st, a, words);
+    hipLaunchKernelGGL(max_pooling_bit_forward_kernel, dim3(blocks), dim3(kPoolBlock), 0, st, a, words, total);
     BBHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -2155,11 +2176,13 @@ static int launch_up_sampling(void const *x, float const *dy, void *out, bool bi
         else      { hipLaunchKernelGGL((up_sampling_backward_kernel<1>), dim3(blocks), dim3(kPoolBlock), 0, st, a); }
     }
     else {
-        if (window_grid(a, c_size, input_h_size * filter_h_size, input_w_size * filter_w_size, items, wide ? 4 : 1, blocks, name)) { return 1; }
+        long long total = 0;
+        if (bit) { if (window_grid_flat(a, c_size, input_h_size * filter_h_size, input_w_size * filter_w_size, items, blocks, total, name)) { return 1; } }
+        else if (window_grid(a, c_size, input_h_size * filter_h_size, input_w_size * filter_w_size, items, wide ? 4 : 1, blocks, name)) { return 1; }
         ScopedTimer tm(kTimeOther, st);
-        if (bit)       { hipLaunchKernelGGL((up_sampling_forward_kernel<true, 1>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items); }
-        else if (wide) { hipLaunchKernelGGL((up_sampling_forward_kernel<false, 4>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items); }
-        else           { hipLaunchKernelGGL((up_sampling_forward_kernel<false, 1>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items); }
+        if (bit)       { hipLaunchKernelGGL((up_sampling_forward_kernel<true, 1>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items, total); }
+        else if (wide) { hipLaunchKernelGGL((up_sampling_forward_kernel<false, 4>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items, total); }
+        else           { hipLaunchKernelGGL((up_sampling_forward_kernel<false, 1>), dim3(blocks), dim3(kPoolBlock), 0, st, a, items, total); }
     }
     BBHIP_LAUNCH_CHECK();
     return 0;

@@ -13,6 +13,7 @@
 #include <stdint.h>
 
 #include "vector_kernels.hpp"
+#include "bn_kernels.hpp"
 
 namespace bbhip {
 
@@ -258,55 +259,83 @@ struct PoolArgs {
 };
 
 // y = 1 - prod over the window taps inside the image, (fy, fx) ascending, of (1 - x): the probability that at least one
-// of four independent binary inputs is 1 (include/bb/StochasticMaxPooling2x2.h:190-218).  One thread per (output node, frame).
+// of four independent binary inputs is 1 (include/bb/StochasticMaxPooling2x2.h:190-218).  One thread per (output node,
+// W frames), W = 4 with 128-bit accesses where rows are 16-byte aligned; the four taps are loaded before the first is used.
+template <int W>
 __global__ __launch_bounds__(kConvBlock) void stochastic_maxpool2x2_forward_kernel(PoolArgs a, int f_blocks)
 {
-    int const f = (int)(blockIdx.x % f_blocks) * kConvBlock + threadIdx.x;
+    int const f = ((int)(blockIdx.x % f_blocks) * kConvBlock + threadIdx.x) * W;
     int const node = blockIdx.x / f_blocks;
     if (f >= a.frame_size) { return; }
     int const ox = node % a.ow, oy = (node / a.ow) % a.oh, c = node / (a.ow * a.oh);
-    float out = 1.0f;
+    float v[2][2][W];
 #pragma unroll
     for (int fy = 0; fy < 2; ++fy) {
 #pragma unroll
         for (int fx = 0; fx < 2; ++fx) {
             int const iy = oy * 2 + fy, ix = ox * 2 + fx;
-            // the product is rounded on its own (not fused into the final 1 - out)
-            if (iy < a.h && ix < a.w) { out = rounded_mul(out, 1.0f - a.x[((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride + f]); }
+            if (iy < a.h && ix < a.w) { bn_load<W>(a.x + ((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride, f, a.frame_size, v[fy][fx]); }
         }
     }
-    a.out[(size_t)node * a.frame_stride + f] = 1.0f - out;
+    float out[W];
+#pragma unroll
+    for (int j = 0; j < W; ++j) { out[j] = 1.0f; }
+#pragma unroll
+    for (int fy = 0; fy < 2; ++fy) {
+#pragma unroll
+        for (int fx = 0; fx < 2; ++fx) {
+            int const iy = oy * 2 + fy, ix = ox * 2 + fx;
+            if (iy < a.h && ix < a.w) {
+                // the product is rounded on its own (not fused into the final 1 - out)
+#pragma unroll
+                for (int j = 0; j < W; ++j) { out[j] = rounded_mul(out[j], 1.0f - v[fy][fx][j]); }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < W; ++j) { out[j] = 1.0f - out[j]; }
+    bn_store<W>(a.out + (size_t)node * a.frame_stride, f, a.frame_size, out);
 }
 
 // dx of each tap = dy * prod over the other three taps of (1 - x), the product evaluated in double and rounded once, taps
 // outside the image reading as 0 (include/bb/StochasticMaxPooling2x2.h:262-306)
+template <int W>
 __global__ __launch_bounds__(kConvBlock) void stochastic_maxpool2x2_backward_kernel(PoolArgs a, int f_blocks)
 {
-    int const f = (int)(blockIdx.x % f_blocks) * kConvBlock + threadIdx.x;
+    int const f = ((int)(blockIdx.x % f_blocks) * kConvBlock + threadIdx.x) * W;
     int const node = blockIdx.x / f_blocks;
     if (f >= a.frame_size) { return; }
     int const ox = node % a.ow, oy = (node / a.ow) % a.oh, c = node / (a.ow * a.oh);
-    double in[2][2] = {{0.0, 0.0}, {0.0, 0.0}};
+    float v[2][2][W], gv[W];
 #pragma unroll
     for (int fy = 0; fy < 2; ++fy) {
 #pragma unroll
         for (int fx = 0; fx < 2; ++fx) {
             int const iy = oy * 2 + fy, ix = ox * 2 + fx;
-            if (iy < a.h && ix < a.w) { in[fy][fx] = (double)a.x[((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride + f]; }
+            if (iy < a.h && ix < a.w) { bn_load<W>(a.x + ((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride, f, a.frame_size, v[fy][fx]); }
+            else {
+#pragma unroll
+                for (int j = 0; j < W; ++j) { v[fy][fx][j] = 0.0f; }
+            }
         }
     }
-    double const g = (double)a.dy[(size_t)node * a.frame_stride + f];
-    float gr[2][2];
-    gr[0][0] = (float)(g * (1.0 - in[0][1]) * (1.0 - in[1][0]) * (1.0 - in[1][1]));
-    gr[0][1] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[1][0]) * (1.0 - in[1][1]));
-    gr[1][0] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[0][1]) * (1.0 - in[1][1]));
-    gr[1][1] = (float)(g * (1.0 - in[0][0]) * (1.0 - in[0][1]) * (1.0 - in[1][0]));
+    bn_load<W>(a.dy + (size_t)node * a.frame_stride, f, a.frame_size, gv);
+    float gr[2][2][W];
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+        double const g = (double)gv[j];
+        double const i00 = (double)v[0][0][j], i01 = (double)v[0][1][j], i10 = (double)v[1][0][j], i11 = (double)v[1][1][j];
+        gr[0][0][j] = (float)(g * (1.0 - i01) * (1.0 - i10) * (1.0 - i11));
+        gr[0][1][j] = (float)(g * (1.0 - i00) * (1.0 - i10) * (1.0 - i11));
+        gr[1][0][j] = (float)(g * (1.0 - i00) * (1.0 - i01) * (1.0 - i11));
+        gr[1][1][j] = (float)(g * (1.0 - i00) * (1.0 - i01) * (1.0 - i10));
+    }
 #pragma unroll
     for (int fy = 0; fy < 2; ++fy) {
 #pragma unroll
         for (int fx = 0; fx < 2; ++fx) {
             int const iy = oy * 2 + fy, ix = ox * 2 + fx;
-            if (iy < a.h && ix < a.w) { a.out[((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride + f] = gr[fy][fx]; }
+            if (iy < a.h && ix < a.w) { bn_store<W>(a.out + ((size_t)(c * a.h + iy) * a.w + ix) * a.frame_stride, f, a.frame_size, gr[fy][fx]); }
         }
     }
 }

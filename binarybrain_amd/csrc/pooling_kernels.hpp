@@ -138,13 +138,14 @@ __global__ __launch_bounds__(kPoolBlock) void max_pooling_backward_kernel(Window
 }
 
 // ---- MaxPooling, packed bits ---------------------------------------------------------------------------------------
-// y = the OR of the window; one thread per (window, word)
-__global__ __launch_bounds__(kPoolBlock) void max_pooling_bit_forward_kernel(WindowArgs a, int words)
+// y = the OR of the window; one thread per (window, word), the (window, word) pairs numbered through: a packed row of a
+// training batch is a few words, far fewer than a workgroup has threads
+__global__ __launch_bounds__(kPoolBlock) void max_pooling_bit_forward_kernel(WindowArgs a, int words, long long total)
 {
-    int node, block, c, oy, ox;
-    split_tile(blockIdx.x, a.f_blocks, node, block);
-    int const wd = block * kPoolBlock + threadIdx.x;
-    if (wd >= words) { return; }
+    long long const gid = (long long)blockIdx.x * kPoolBlock + threadIdx.x;
+    if (gid >= total) { return; }
+    int node, wd, c, oy, ox;
+    split_tile((int)gid, a.f_blocks, node, wd);         // f_blocks holds the words per row here
     split_pixel(node, a, c, oy, ox);
     uint32_t const *__restrict__ x = static_cast<uint32_t const *>(a.x);
     uint32_t any = 0;
@@ -190,12 +191,20 @@ __global__ __launch_bounds__(kPoolBlock) void max_pooling_bit_backward_kernel(Wi
 // Output pixel (oy, ox) reads input pixel (oy / fh, ox / fw): all of the block (fill) or only its position (fh / 2, fw / 2)
 // with zeros around.  One thread per (output pixel, W frames) or, packed, per (output pixel, word).
 template <bool BIT, int W>
-__global__ __launch_bounds__(kPoolBlock) void up_sampling_forward_kernel(WindowArgs a, int items)
+__global__ __launch_bounds__(kPoolBlock) void up_sampling_forward_kernel(WindowArgs a, int items, long long total)
 {
-    int node, block, c, oy, ox;
-    split_tile(blockIdx.x, a.f_blocks, node, block);
-    int const f = (block * kPoolBlock + threadIdx.x) * W;
-    if (f >= items) { return; }
+    int node, f, c, oy, ox;
+    if constexpr (BIT) {                                // (pixel, word) pairs numbered through, f_blocks = words per row
+        long long const gid = (long long)blockIdx.x * kPoolBlock + threadIdx.x;
+        if (gid >= total) { return; }
+        split_tile((int)gid, a.f_blocks, node, f);
+    }
+    else {
+        int block;
+        split_tile(blockIdx.x, a.f_blocks, node, block);
+        f = (block * kPoolBlock + threadIdx.x) * W;
+        if (f >= items) { return; }
+    }
     split_pixel(node, a, c, oy, ox);                    // extents: the output image
     int const iy = oy / a.fh, ix = ox / a.fw;
     bool const take = a.fill || (oy - iy * a.fh == a.fh / 2 && ox - ix * a.fw == a.fw / 2);

@@ -108,6 +108,14 @@ SAME(&bbcu_bit_RealToBinary_Forward<float>, int (*)(float const *, int *, unsign
 SAME(&bbcu_fp32_BinaryToReal_Forward, int (*)(float const *, float *, int, int, int, int, int, int, S));
 SAME(&bbcu_bit_fp32_BinaryToReal_Forward, int (*)(int const *, float *, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_BinaryToReal_Backward, int (*)(float const *, float *, int, int, int, int, int, int, S));
+// bbcu.h:949-1068
+SAME(&bbcu_fp32_MaxPooling_Forward, int (*)(float const *, float *, int *, int, int, int, int, int, int, int, int, int, S));
+SAME(&bbcu_bit_MaxPooling_Forward, int (*)(int const *, int *, int, int, int, int, int, int, int, int, int, S));
+SAME(&bbcu_fp32_MaxPooling_Backward, int (*)(int const *, float const *, float *, int, int, int, int, int, int, int, int, int, S));
+SAME(&bbcu_bit_fp32_MaxPooling_Backward, int (*)(int const *, float const *, float *, int, int, int, int, int, int, int, int, int, int, S));
+SAME(&bbcu_fp32_UpSampling_Forward, int (*)(float const *, float *, int, int, int, int, int, int, int, int, S));
+SAME(&bbcu_bit_UpSampling_Forward, int (*)(int const *, int *, int, int, int, int, int, int, int, int, S));
+SAME(&bbcu_fp32_UpSampling_Backward, int (*)(float const *, float *, int, int, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_Im2Col_Forward, int (*)(float const *, float *, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, float, S));
 SAME(&bbcu_bit_Im2Col_Forward, int (*)(int const *, int *, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_Im2Col_Backward, int (*)(float const *, float *, int, int, int, int, int, int, int, int, int, int, int, int, int, int, S));
@@ -178,7 +186,7 @@ static int run_on_gpu(void)
 
 int main(int argc, char **argv)
 {
-    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11 + 10;
+    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11 + 10 + 7;
     if (argc > 1 && !std::strcmp(argv[1], "--gpu")) {
         if (!bbcu_IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
         int const bad = run_on_gpu();

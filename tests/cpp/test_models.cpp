@@ -32,6 +32,8 @@
 #include "bb/BinaryToReal.h"
 #include "bb/BinaryModulation.h"
 #include "bb/DifferentiableLutDiscreteN.h"
+#include "bb/MaxPooling.h"
+#include "bb/UpSampling.h"
 #include "bb/ObjectLoader.h"
 
 extern "C" {
@@ -63,6 +65,10 @@ void oracle_fp32_BinaryToReal_Backward(float const *dy, float *dx, int node_mux_
 void oracle_fp32_Binarize_Forward(float const *x, float *y, float binary_th, float binary_low, float binary_high, int node_size, int frame_size, int frame_stride);
 void oracle_fp32_HardTanh_Forward(float const *x, float *y, float limit_min, float limit_max, int node_size, int frame_size, int frame_stride);
 void oracle_fp32_HardTanh_Backward(float const *x, float const *dy, float *dx, float limit_min, float limit_max, int node_size, int frame_size, int frame_stride);
+void oracle_fp32_MaxPooling_Forward(float const *x, float *y, int *argmax, int filter_h_size, int filter_w_size, int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride);
+void oracle_fp32_MaxPooling_Backward(int const *argmax, float const *dy, float *dx, int filter_h_size, int filter_w_size, int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride);
+void oracle_fp32_UpSampling_Forward(float const *x, float *y, int input_w_size, int input_h_size, int c_size, int filter_w_size, int filter_h_size, int fill, int frame_size, int frame_stride);
+void oracle_fp32_UpSampling_Backward(float const *dy, float *dx, int input_w_size, int input_h_size, int c_size, int filter_w_size, int filter_h_size, int fill, int frame_size, int frame_stride);
 void oracle_bit_BinaryLut6_Forward(std::int32_t const *x, std::int32_t *y, std::int32_t const *idx, std::int32_t const *table, int node_size, int frame_size, int frame_stride);
 }
 
@@ -835,6 +841,71 @@ static void test_discrete(int I, int O, int F, bool binary)
     }
 }
 
+// MaxPooling and UpSampling through the classes: fp32 against the oracle, the packed forms against the fp32 forms on 0 / 1 images
+// (OR = max; the first set input = the first largest value), shapes, and a trip through a stream.
+static void test_pooling(void)
+{
+    int const C = 3, H = 5, Wd = 7, FH = 2, FW = 3, F = 70;
+    int const OH = (H + FH - 1) / FH, OW = (Wd + FW - 1) / FW;
+    std::mt19937_64 mt(31);
+    std::uniform_real_distribution<float> uni(-1.0f, 1.0f);
+    bb::FrameBuffer x_buf(F, {C, H, Wd}, BB_TYPE_FP32), dy_buf(F, {C, OH, OW}, BB_TYPE_FP32);
+    for (int n = 0; n < C * H * Wd; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, (mt() % 5 == 0) ? 0.25f : uni(mt)); }
+    for (int n = 0; n < C * OH * OW; ++n) for (int f = 0; f < F; ++f) { dy_buf.SetFP32(f, n, uni(mt)); }
+    std::vector<float> x, dy, y, dx, y_ref((size_t)C * OH * OW * F), dx_ref((size_t)C * H * Wd * F);
+    std::vector<int> arg_ref(y_ref.size());
+    read_fp32(x_buf, x); read_fp32(dy_buf, dy);
+    auto pool = bb::MaxPooling<>::Create(FH, FW);
+    CHECK(pool->SetInputShape({C, H, Wd}) == bb::indices_t({C, OH, OW}), "MaxPooling output shape");
+    bb::FrameBuffer y_buf = pool->Forward(x_buf), dx_buf = pool->Backward(dy_buf);
+    read_fp32(y_buf, y); read_fp32(dx_buf, dx);
+    oracle_fp32_MaxPooling_Forward(x.data(), y_ref.data(), arg_ref.data(), FH, FW, Wd, H, OW, OH, C, F, F);
+    oracle_fp32_MaxPooling_Backward(arg_ref.data(), dy.data(), dx_ref.data(), FH, FW, Wd, H, OW, OH, C, F, F);
+    CHECK(max_diff(y, y_ref) == 0.0 && max_diff(dx, dx_ref) == 0.0, "MaxPooling differs by %g, %g", max_diff(y, y_ref), max_diff(dx, dx_ref));
+    {   // packed: a 0 / 1 image pooled as bits = the fp32 pooling of the same image
+        bb::FrameBuffer b_buf(F, {C, H, Wd}, BB_TYPE_BIT), f_buf(F, {C, H, Wd}, BB_TYPE_FP32);
+        for (int n = 0; n < C * H * Wd; ++n) for (int f = 0; f < F; ++f) { bool const v = (mt() % 4 == 0); b_buf.SetBit(f, n, v); f_buf.SetFP32(f, n, v ? 1.0f : 0.0f); }
+        auto pool_bit = bb::MaxPooling<bb::Bit>::Create(FH, FW);
+        auto pool_f = bb::MaxPooling<>::Create(FH, FW);
+        bb::FrameBuffer yb = pool_bit->Forward(b_buf), yf = pool_f->Forward(f_buf);
+        size_t bad = 0;
+        for (int n = 0; n < C * OH * OW; ++n) for (int f = 0; f < F; ++f) { bad += (yb.GetBit(f, n) != (yf.GetFP32(f, n) > 0.5f)); }
+        CHECK(yb.GetType() == BB_TYPE_BIT && bad == 0, "packed MaxPooling forward: %zu bits differ", bad);
+        bb::FrameBuffer gb = pool_bit->Backward(dy_buf), gf = pool_f->Backward(dy_buf);
+        // where a window holds a one both send dy to its first one; an empty window sends nothing (packed) or dy to its first input (fp32)
+        bad = 0;
+        for (int c = 0; c < C; ++c) for (int iy = 0; iy < H; ++iy) for (int ix = 0; ix < Wd; ++ix) for (int f = 0; f < F; ++f) {
+            int const n = (c * H + iy) * Wd + ix, o = (c * OH + iy / FH) * OW + ix / FW;
+            float const want = yb.GetBit(f, o) ? gf.GetFP32(f, n) : 0.0f;
+            bad += (gb.GetFP32(f, n) != want);
+        }
+        CHECK(bad == 0, "packed MaxPooling backward: %zu values differ", bad);
+    }
+    for (int fill = 1; fill >= 0; --fill) {
+        auto up = bb::UpSampling<>::Create(FH, FW, fill != 0);
+        CHECK(up->SetInputShape({C, OH, OW}) == bb::indices_t({C, OH * FH, OW * FW}), "UpSampling output shape");
+        bb::FrameBuffer u_buf = up->Forward(dy_buf);
+        bb::FrameBuffer g_buf(F, {C, OH * FH, OW * FW}, BB_TYPE_FP32);
+        for (int n = 0; n < C * OH * FH * OW * FW; ++n) for (int f = 0; f < F; ++f) { g_buf.SetFP32(f, n, uni(mt)); }
+        bb::FrameBuffer d_buf = up->Backward(g_buf);
+        std::vector<float> u, g, d, u_ref((size_t)C * OH * FH * OW * FW * F), d_ref(dy.size());
+        read_fp32(u_buf, u); read_fp32(g_buf, g); read_fp32(d_buf, d);
+        oracle_fp32_UpSampling_Forward(dy.data(), u_ref.data(), OW, OH, C, FW, FH, fill, F, F);
+        oracle_fp32_UpSampling_Backward(g.data(), d_ref.data(), OW, OH, C, FW, FH, fill, F, F);
+        CHECK(max_diff(u, u_ref) == 0.0 && max_diff(d, d_ref) == 0.0, "UpSampling (fill %d) differs by %g, %g", fill, max_diff(u, u_ref), max_diff(d, d_ref));
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        up->DumpObject(ss);
+        pool->DumpObject(ss);
+        auto up2 = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        auto pool2 = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)up2 && (bool)pool2 && up2->GetObjectName() == "UpSampling_fp32_fp32" && pool2->GetObjectName() == "MaxPooling_fp32_fp32", "pooling reload");
+        if (up2 && pool2) {
+            bb::FrameBuffer u2 = up2->Forward(dy_buf, false), y2 = pool2->Forward(x_buf, false);
+            CHECK(same_bits(u2, u_buf) && same_bits(y2, y_buf), "reloaded pooling layers differ");
+        }
+    }
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -993,6 +1064,7 @@ int main(void)
         test_max_lut();
         test_reduce_and_mean_squared_error();
         test_binary_modulation();
+        test_pooling();
         test_discrete<6>(24, 16, 200, false);
         test_discrete<6>(24, 16, 200, true);
         test_discrete<4>(12, 30, 1024, false);

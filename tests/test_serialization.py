@@ -423,3 +423,29 @@ def test_truncated_modulation_objects_are_rejected(tmp_path):
         open(src, "wb").write(data[:cut])
         res = subprocess.run([TOOL, "reload", src, str(tmp_path / "out.bin")], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
         assert res.returncode != 0
+
+
+# ----------------------------------------------------------------------------------------------
+#  MaxPooling, UpSampling (include/bb/MaxPooling.h:694-735, UpSampling.h:357-383): objects written by the reference's classes
+#  (tests/golden/pooling.npz), fp32 and packed, load here and are written again byte for byte; the reference's loader reads them back.
+# ----------------------------------------------------------------------------------------------
+POOLING = np.load(os.path.join(HERE, "golden", "pooling.npz"))
+
+
+@pytest.mark.parametrize("k", range(int(POOLING["pool_count"][0])))
+def test_reference_max_pooling_objects(tmp_path, k):
+    q = "p%d_" % k
+    c, h, w, fh, fw, F = [int(v) for v in POOLING[q + "geom"]]
+    name = POOLING[q + "name"].tobytes().decode()
+    out_nodes = c * ((h + fh - 1) // fh) * ((w + fw - 1) // fw)
+    for key, type_name in (("object", "MaxPooling_fp32_fp32"), ("object_bit", "MaxPooling_bit_fp32")):
+        _reload_and_compare(tmp_path, POOLING[q + key].tobytes(), type_name, name, "MaxPooling", c * h * w, out_nodes)
+
+
+@pytest.mark.parametrize("k", range(int(POOLING["up_count"][0])))
+def test_reference_up_sampling_objects(tmp_path, k):
+    q = "u%d_" % k
+    c, h, w, fh, fw, fill, F = [int(v) for v in POOLING[q + "geom"]]
+    name = POOLING[q + "name"].tobytes().decode()
+    for key, type_name in (("object", "UpSampling_fp32_fp32"), ("object_bit", "UpSampling_bit_fp32")):
+        _reload_and_compare(tmp_path, POOLING[q + key].tobytes(), type_name, name, "UpSampling", c * h * w, c * h * fh * w * fw)
