@@ -309,8 +309,101 @@ def test_random_shapes_of_the_classifier_tail_and_adam():
         run_tail_case(ops, torch, seed)
 
 
+def run_plumbing_case(ops, seed):
+    """RealToBinary, BinaryToReal, Binarize / HardTanh, MaxPooling and UpSampling at random shapes, row pitches and parameters: all of them
+    bit for bit against the oracle"""
+    F32 = np.float32
+    rng = np.random.default_rng(seed)
+    kind = str(rng.choice(["real_to_binary", "binary_to_real", "activation", "max_pooling", "up_sampling"]))
+
+    def pitch(n):
+        return int(rng.choice([synth.frame_stride_fp32(n), n, n + int(rng.integers(1, 9))]))
+
+    def words(n):
+        return int(rng.choice([synth.frame_stride_bit(n), (n + 31) // 32, (n + 31) // 32 + int(rng.integers(1, 4))]))
+
+    if kind == "real_to_binary":
+        d = int(rng.integers(1, 5)); p = int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(40, 900))])); F = int(rng.integers(1, 300))
+        fm = int(rng.choice([1, 2, 7, 15, int(rng.integers(1, 70))])); dm = int(rng.choice([1, 1, 2, int(rng.integers(1, 6))]))
+        lo, hi = [(0.0, 1.0), (-1.0, 1.0), (0.0, 255.0), (0.1, 0.9)][int(rng.integers(0, 4))]
+        binarize = bool(rng.integers(0, 2))
+        print("seed %d: real_to_binary d=%d p=%d F=%d fm=%d dm=%d range=(%g, %g) binarize=%d" % (seed, d, p, F, fm, dm, lo, hi, binarize), flush=True)
+        x = pad((rng.random((d * p, F)) * (hi - lo) * 1.2 + lo - 0.1 * (hi - lo)).astype(F32), pitch(F))
+        ys, ws = pitch(F * fm), words(F * fm)
+        got = host(ops.real_to_binary_forward(dev(x), d, p, F, fm, dm, lo, hi, binarize=binarize, y_stride=ys))
+        assert np.array_equal(got[:, :F * fm], oracle.real_to_binary_forward(x, d, p, F, fm, dm, lo, hi, binarize=binarize, y_stride=ys)[:, :F * fm])
+        got = host(ops.real_to_binary_forward(dev(x), d, p, F, fm, dm, lo, hi, binarize=binarize, bit=True, y_stride=ws))
+        assert np.array_equal(got, oracle.real_to_binary_forward(x, d, p, F, fm, dm, lo, hi, binarize=binarize, bit=True, y_stride=ws))
+    elif kind == "binary_to_real":
+        O = int(rng.integers(1, 200)); mux = int(rng.choice([1, 1, 7, int(rng.integers(1, 12))])); Fy = int(rng.integers(1, 300))
+        fm = int(rng.choice([1, 2, 7, 15, 32, int(rng.integers(1, 70))]))
+        I, F = O * mux, Fy * fm
+        print("seed %d: binary_to_real I=%d O=%d Fy=%d fm=%d" % (seed, I, O, Fy, fm), flush=True)
+        xs, ys, ws = pitch(F), pitch(Fy), words(F)
+        x = pad(rng.standard_normal((I, F)).astype(F32), xs)
+        x[:, F:] = 3.0
+        x[rng.random(x.shape) < 0.1] = 0.0
+        assert np.array_equal(host(ops.binary_to_real_forward(dev(x), O, Fy, fm, y_stride=ys))[:, :Fy], oracle.binary_to_real_forward(x, O, Fy, fm, y_stride=ys)[:, :Fy])
+        xb = synth.bernoulli_bits(rng, I, F, ws, p=float(rng.choice([0.1, 0.5, 0.9])))
+        xb[:, (F + 31) // 32:] = -1
+        assert np.array_equal(host(ops.binary_to_real_forward(dev(xb), O, Fy, fm, y_stride=ys))[:, :Fy],
+                              oracle.binary_to_real_forward(xb, O, Fy, fm, bit=True, y_stride=ys)[:, :Fy])
+        dy = pad(rng.standard_normal((O, Fy)).astype(F32), ys)
+        assert np.array_equal(host(ops.binary_to_real_backward(dev(dy), I, Fy, fm, x_stride=xs))[:, :F], oracle.binary_to_real_backward(dy, I, Fy, fm, x_stride=xs)[:, :F])
+    elif kind == "activation":
+        nodes = int(rng.integers(1, 400)); F = int(rng.choice([int(rng.integers(1, 70)), int(rng.integers(64, 5000))]))
+        lo, hi = sorted(float(v) for v in rng.standard_normal(2)); th = float(rng.standard_normal() * 0.3)
+        if lo == hi:
+            hi = lo + 1.0
+        print("seed %d: activation nodes=%d F=%d window=(%g, %g) th=%g" % (seed, nodes, F, lo, hi, th), flush=True)
+        st = pitch(F)
+        x = pad(rng.standard_normal((nodes, F)).astype(F32), st); dy = pad(rng.standard_normal((nodes, F)).astype(F32), st)
+        x.flat[:4] = [lo, hi, th, np.nan]
+        assert np.array_equal(host(ops.binarize_forward(dev(x), F, th, -1.0, 1.0))[:, :F], oracle.binarize_forward(x, F, th, -1.0, 1.0)[:, :F])
+        ws = words(F)
+        assert np.array_equal(host(ops.binarize_forward(dev(x), F, th, bit=True, y_stride=ws)), oracle.binarize_forward(x, F, th, bit=True, y_stride=ws))
+        assert np.array_equal(host(ops.hard_tanh_forward(dev(x), F, lo, hi))[:, :F], oracle.hard_tanh_forward(x, F, lo, hi)[:, :F], equal_nan=True)
+        assert np.array_equal(host(ops.hard_tanh_backward(dev(x), dev(dy), F, lo, hi))[:, :F], oracle.hard_tanh_backward(x, dy, F, lo, hi)[:, :F])
+    elif kind == "max_pooling":
+        c = int(rng.integers(1, 12)); h = int(rng.integers(1, 20)); w = int(rng.integers(1, 20)); fh = int(rng.choice([1, 2, 2, 3, int(rng.integers(1, 6))]))
+        fw = int(rng.choice([1, 2, 2, 3, int(rng.integers(1, 6))])); F = int(rng.integers(1, 400))
+        print("seed %d: max_pooling c=%d h=%d w=%d filter=%dx%d F=%d" % (seed, c, h, w, fh, fw, F), flush=True)
+        st = pitch(F)
+        x = pad(rng.standard_normal((c * h * w, F)).astype(F32), st)
+        x[rng.random(x.shape) < 0.2] = 0.5
+        O = c * ((h + fh - 1) // fh) * ((w + fw - 1) // fw)
+        dy = pad(rng.standard_normal((O, F)).astype(F32), st)
+        y, arg = ops.max_pooling_forward(dev(x), c, h, w, fh, fw, F)
+        y_ref, arg_ref = oracle.max_pooling_forward(x, c, h, w, fh, fw, F)
+        assert np.array_equal(host(y)[:, :F], y_ref[:, :F]) and np.array_equal(host(arg)[:, :F], arg_ref[:, :F])
+        assert np.array_equal(host(ops.max_pooling_backward(arg, dev(dy), c, h, w, fh, fw, F))[:, :F], oracle.max_pooling_backward(arg_ref, dy, c, h, w, fh, fw, F)[:, :F])
+        xb = synth.bernoulli_bits(rng, c * h * w, F, words(F), p=float(rng.choice([0.05, 0.3, 0.8])))
+        nw = (F + 31) // 32
+        assert np.array_equal(host(ops.bit_max_pooling_forward(dev(xb), c, h, w, fh, fw, F))[:, :nw], oracle.bit_max_pooling_forward(xb, c, h, w, fh, fw, F)[:, :nw])
+        assert np.array_equal(host(ops.bit_max_pooling_backward(dev(xb), dev(dy), c, h, w, fh, fw, F))[:, :F],
+                              oracle.bit_max_pooling_backward(xb, dy, c, h, w, fh, fw, F)[:, :F])
+    else:
+        c = int(rng.integers(1, 12)); h = int(rng.integers(1, 12)); w = int(rng.integers(1, 12)); fh = int(rng.integers(1, 5)); fw = int(rng.integers(1, 5))
+        F = int(rng.integers(1, 400)); fill = bool(rng.integers(0, 2))
+        print("seed %d: up_sampling c=%d h=%d w=%d filter=%dx%d F=%d fill=%d" % (seed, c, h, w, fh, fw, F, fill), flush=True)
+        st = pitch(F)
+        x = pad(rng.standard_normal((c * h * w, F)).astype(F32), st)
+        dy = pad(rng.standard_normal((c * h * fh * w * fw, F)).astype(F32), st)
+        assert np.array_equal(host(ops.up_sampling_forward(dev(x), c, h, w, fh, fw, F, fill))[:, :F], oracle.up_sampling_forward(x, c, h, w, fh, fw, F, fill)[:, :F])
+        assert np.array_equal(host(ops.up_sampling_backward(dev(dy), c, h, w, fh, fw, F, fill))[:, :F], oracle.up_sampling_backward(dy, c, h, w, fh, fw, F, fill)[:, :F])
+        xb = synth.bernoulli_bits(rng, c * h * w, F, words(F))
+        nw = (F + 31) // 32
+        assert np.array_equal(host(ops.up_sampling_forward(dev(xb), c, h, w, fh, fw, F, fill))[:, :nw], oracle.up_sampling_forward(xb, c, h, w, fh, fw, F, fill, bit=True)[:, :nw])
+
+
+def test_random_shapes_of_the_converters_activations_and_pooling():
+    from binarybrain_amd import ops
+    for seed in range(13000, 13250):
+        run_plumbing_case(ops, seed)
+
+
 def test_extended_random_run():
-    """The same three generators over further seeds, for a longer run on the device: set BBHIP_EXTENDED_CASES=N (N cases of each
+    """The same four generators over further seeds, for a longer run on the device: set BBHIP_EXTENDED_CASES=N (N cases of each
     generator, at most 200 000; seeds continue after the ones above).  Stops at the first failing case, whose seed the case
     prints.  Without the variable the test is skipped, so the default suite stays short:
         BBHIP_EXTENDED_CASES=10000 python -u -m pytest tests/test_gpu_random_shapes.py -k extended -x -s"""
@@ -326,6 +419,7 @@ def test_extended_random_run():
             run_case(ops, torch, 100000 + k)
             run_exact_case(ops, 400000 + k)
             run_tail_case(ops, torch, 700000 + k)
+            run_plumbing_case(ops, 900000 + k)
             if (k + 1) % 500 == 0:
                 print("extended run: %d of %d" % (k + 1, count), flush=True)
     finally:
