@@ -372,8 +372,10 @@ def bench_differentiablelut6(args, lib):
             y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=(0.0, 1.0))
             ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev)
         else:
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=(0.0, 1.0))
-            ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev)
+            # the model class keeps the packed copy of its binarized input from the forward to the backward call
+            packed = ops.packed_input_buffer(I, F)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=(0.0, 1.0), packed=packed)
+            ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev, packed=packed)
 
     t_ramp = time.perf_counter()
     while time.perf_counter() - t_ramp < args.ramp_seconds:
@@ -435,15 +437,17 @@ def bench_conv_block(args, lib):
         a = cols; acts = []
         for l in layers:
             # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=(0.0, 1.0))
-            acts.append((a, mean, rstd)); a = y
+            # ... and keeps the packed copy of its binarized input for the backward call
+            packed = ops.packed_input_buffer(a.shape[0], FW_FRAMES)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed)
+            acts.append((a, mean, rstd, packed)); a = y
         maps = ops.col2im_forward(a, CO, OH, OW, F)
         pooled = ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F)
         dmaps = ops.stochastic_maxpool2x2_backward(maps, dpooled, CO, OH, OW, F)
         dy = ops.col2im_backward(dmaps, CO, OH, OW, F)
-        for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
+        for l, (a_in, mean, rstd, packed) in zip(reversed(layers), reversed(acts)):
             l["dW"].zero_()
-            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"])
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"], packed=packed)
         return ops.im2col_backward(dy, C, H, W_, F, FH, FW), pooled
 
     t_ramp = time.perf_counter()
@@ -529,15 +533,17 @@ def bench_mnist_step(args, lib):
         acts = []
         for l in layers:
             # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0))
-            acts.append((a, mean, rstd)); a = y
+            # ... and keeps the packed copy of its binarized input for the backward call
+            packed = ops.packed_input_buffer(a.shape[0], F)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed)
+            acts.append((a, mean, rstd, packed)); a = y
         out = ops.average_lut_forward(a, idx_avg, F, False, False)
         dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
         acc, cat = ops.metrics_categorical_accuracy(out, t, CLASSES, 1, F)
         dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
-        for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
+        for l, (a_in, mean, rstd, packed) in zip(reversed(layers), reversed(acts)):
             # dW accumulates; it is zero here because the optimizer's Update() zeroed it after the previous step (Optimizer.h:31-35)
-            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"])
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"], packed=packed)
         keep["loss_buf"], keep["acc"] = loss_buf, acc
 
     def timed(fn):

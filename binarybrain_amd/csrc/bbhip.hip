@@ -66,6 +66,11 @@ bool g_host_only = false;
 int  g_dx_mode   = 0;
 bool g_average_lut_mean = false;             // bbhip_SetAverageLutMean: un-binarized AverageLut output is sum * (1 / n)
 thread_local int g_input_node_hint = 0;      // bbhip_HintInputNodeSize: rows of the next forward call's input, 0 = unknown
+// bbhip_HintPackedInput: a caller-owned buffer for the packed copy of the next LUT call's binarized fp32 input
+struct PackedInputHint { uint32_t *bits; int rows, row_words, holds_input; };
+thread_local PackedInputHint g_packed_hint = {nullptr, 0, 0, 0};
+// hints are for the next LUT call only: every entry spends them
+static inline void clear_hints(void) { g_input_node_hint = 0; g_packed_hint = PackedInputHint{nullptr, 0, 0, 0}; }
 
 // ------------------------------------------------------------------------------------------------
 //  optional kernel timer: HIP events around the dominant kernel of each entry point, on the launch stream
@@ -412,7 +417,8 @@ int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_s
 }
 
 template <int N>
-int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch const *fixed = nullptr)
+int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch const *fixed = nullptr,
+                PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0})
 {
     constexpr int NN = 1 << N;
     // input_rows: what the caller said about the input's row count (bbhip_HintInputNodeSize), 0 = nothing.
@@ -420,7 +426,10 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     // call is a packed-bit call (same outputs)
     ForwardCall c = call;
     bool const pack = (c.xmode == kXBinary) && input_rows > 0 && use_corner_values(kXBinary) && pack_binarized_input();
-    if (pack) { c.xmode = kXBit; c.x_stride = packed_row_words(c.frame_size); c.x = nullptr; }
+    // the packed copy goes to the caller's buffer where one was offered and fits (rows of whole 32-byte groups), else to the arena
+    bool const to_caller = pack && packed.bits != nullptr && packed.rows == input_rows && packed.row_words >= (c.frame_size + 31) / 32 &&
+                           packed.row_words % 8 == 0 && (reinterpret_cast<uintptr_t>(packed.bits) & 31u) == 0;
+    if (pack) { c.xmode = kXBit; c.x_stride = to_caller ? packed.row_words : packed_row_words(c.frame_size); c.x = nullptr; }
     bool const corner     = use_corner_values(c.xmode);
     int const npw         = corner ? 1 : fwd_nodes_per_wave();
     int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
@@ -435,14 +444,14 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     size_t const c_bytes    = align256((size_t)c.node_size * NN * sizeof(float));
     size_t const v_bytes    = corner ? c_bytes : 0;
     size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
-    size_t const bits_bytes = pack ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
+    size_t const bits_bytes = (pack && !to_caller) ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
     if (arena_get(c_bytes + v_bytes + stat_bytes + bits_bytes, &base, st, fixed)) { return 1; }
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
     if (pack) {
-        uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes);
+        uint32_t *bits = to_caller ? packed.bits : reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes);
         if (launch_pack_and_prep<N>(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size,
                                     c.W, C, V, c.node_size, c.lut_binarize, c.bias, st, c.clamp_W, c.clamp_lo, c.clamp_hi)) { return 1; }
         c.x = bits;
@@ -505,11 +514,13 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
 
 int forward_entry(ForwardCall const &c, void *stream, Scratch const *fixed = nullptr)
 {
-    int const input_rows = fixed ? 0 : g_input_node_hint;       // the hint is spent by this call, whatever becomes of it
-    g_input_node_hint = 0;
+    // the hints are spent by this call, whatever becomes of it; a buffer for the packed copy also says how many rows the input has
+    PackedInputHint const packed = fixed ? PackedInputHint{nullptr, 0, 0, 0} : g_packed_hint;
+    int const input_rows = fixed ? 0 : (packed.bits ? packed.rows : g_input_node_hint);
+    clear_hints();
     if (check_forward(c)) { return 1; }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed));
+    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed, packed));
     return 0;
 }
 
@@ -552,7 +563,7 @@ int check_backward(BackwardCall const &c, int dxmode)
 }
 
 template <int N>
-int run_backward(BackwardCall const &call, hipStream_t st)
+int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0})
 {
     constexpr int NN = 1 << N;
     int dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
@@ -572,7 +583,11 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     // kernels of this pass gain from packed rows); from here on the call is a packed-bit call
     BackwardCall c = call;
     bool const pack = (c.xmode == kXBinary) && dxmode == kDxNone && use_corner_values(kXBinary) && pack_binarized_input();
-    if (pack) { c.xmode = kXBit; c.x_stride = packed_row_words(c.frame_size); c.x = nullptr; }      // the packed rows get their place in the arena below
+    // a caller that kept the packed copy of this input from the forward call hands it back: nothing to pack
+    bool const have_bits = pack && packed.bits != nullptr && packed.holds_input && packed.rows == c.input_node_size &&
+                           packed.row_words >= (c.frame_size + 31) / 32 && packed.row_words % 8 == 0 &&
+                           (reinterpret_cast<uintptr_t>(packed.bits) & 31u) == 0;
+    if (pack) { c.xmode = kXBit; c.x_stride = have_bits ? packed.row_words : packed_row_words(c.frame_size); c.x = nullptr; }   // else: a place in the arena below
 
     int const tile_count = ceil_div(c.output_node_size, kWavesPerBlk);
     int const range      = (dxmode == kDxTmp) ? (c.tmp_frame_size < c.frame_size ? c.tmp_frame_size : c.frame_size) : c.frame_size;
@@ -611,7 +626,7 @@ int run_backward(BackwardCall const &call, hipStream_t st)
     size_t const dtab_bytes = align256(term_count * sizeof(int));
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     size_t const v_bytes = corner ? c_bytes : 0;
-    size_t const bits_bytes = pack ? align256((size_t)c.input_node_size * c.x_stride * sizeof(uint32_t)) : 0;
+    size_t const bits_bytes = (pack && !have_bits) ? align256((size_t)c.input_node_size * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
     if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes, &base, st)) { return 1; }
     float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
@@ -623,7 +638,14 @@ int run_backward(BackwardCall const &call, hipStream_t st)
 
     // centred coefficients: needed where the LUT output is recomputed (batch-norm) or per-connection gradients are formed
     bool const prep = c.bn || dxmode != kDxNone;
-    if (pack) {
+    if (have_bits) {
+        c.x = packed.bits;
+        if (prep) {
+            launch_table_prep<N>(c.W, C, c.output_node_size, c.lut_binarize, st, V, c.bias);
+            BBHIP_LAUNCH_CHECK();
+        }
+    }
+    else if (pack) {
         uint32_t *bits = reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes);
         float const *src = reinterpret_cast<float const *>(call.x);
         if (prep) {
@@ -765,9 +787,10 @@ int run_backward(BackwardCall const &call, hipStream_t st)
 
 int backward_entry(BackwardCall const &c, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next forward call only
+    PackedInputHint const packed = g_packed_hint;
+    clear_hints();                                  // hints are for the next LUT call only
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st));
+    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st, packed));
     return 0;
 }
 
@@ -1064,11 +1087,18 @@ int  bbhip_GetAverageLutMean(void) { return g_average_lut_mean ? 1 : 0; }
 
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
 void bbhip_HintInputNodeSize(int input_node_size) { g_input_node_hint = input_node_size > 0 ? input_node_size : 0; }
+int  bbhip_PackedRowWords(int frame_size) { return frame_size > 0 ? packed_row_words(frame_size) : 0; }
+void bbhip_HintPackedInput(int *dev_bits, int rows, int row_words, int holds_input)
+{
+    g_packed_hint = (dev_bits != nullptr && rows > 0 && row_words > 0)
+                  ? PackedInputHint{reinterpret_cast<uint32_t *>(dev_bits), rows, row_words, holds_input != 0}
+                  : PackedInputHint{nullptr, 0, 0, 0};
+}
 int  bbhip_GetDxMode(void) { return g_dx_mode; }
 
 int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_dst != nullptr && size >= 0);
     if (size == 0) { return 0; }
     hipLaunchKernelGGL(fill_kernel, dim3(ceil_div(size, kBlock * 4)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, a, (size_t)size);
@@ -1078,7 +1108,7 @@ int bbhip_fp32_Vector_set(float *dev_dst, float a, int size, void *stream)
 
 int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, float hi, int size, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_dst != nullptr && dev_src != nullptr && size >= 0);
     if (size == 0) { return 0; }
     hipLaunchKernelGGL(clamp_kernel, dim3(ceil_div(size, kBlock)), dim3(kBlock), 0, static_cast<hipStream_t>(stream), dev_dst, dev_src, lo, hi, size);
@@ -1088,55 +1118,55 @@ int bbhip_fp32_Vector_clamp(float *dev_dst, float const *dev_src, float lo, floa
 
 int bbhip_fp32_Vector_add_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecAddEx>(dev_dst, dev_src0, dev_src1, a, b, c, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_mul_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecMulEx>(dev_dst, dev_src0, dev_src1, a, b, 0.0f, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_div_ex(float *dev_dst, float const *dev_src0, float const *dev_src1, float a, float b, float c, float d, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecDivEx>(dev_dst, dev_src0, dev_src1, a, b, c, d, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_sqrt(float *dev_dst, float const *dev_src, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecSqrt>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_exp(float *dev_dst, float const *dev_src, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecExp>(dev_dst, dev_src, nullptr, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_min(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecMin>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_min_v(float *dev_dst, float const *dev_src, float a, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecMinV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_max(float *dev_dst, float const *dev_src0, float const *dev_src1, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecMax>(dev_dst, dev_src0, dev_src1, 0.0f, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
 int bbhip_fp32_Vector_max_v(float *dev_dst, float const *dev_src, float a, int size, void *stream)
 {
-    g_input_node_hint = 0;
+    clear_hints();
     return vector_op<kVecMaxV>(dev_dst, dev_src, nullptr, a, 0.0f, 0.0f, 0.0f, size, stream, __func__);
 }
 
@@ -1144,7 +1174,7 @@ namespace {
 int adam_entry(bool zero_grads, int size, int const *dev_size_table, float *const *dev_params_buf_table, float *const *dev_grads_buf_table,
                float *const *dev_m_buf_table, float *const *dev_v_buf_table, float lr_t, float beta1, float beta2, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(size >= 0 && size <= 65535);
     if (size == 0) { return 0; }
     BBHIP_REQUIRE(dev_size_table != nullptr && dev_params_buf_table != nullptr && dev_grads_buf_table != nullptr &&
@@ -1184,7 +1214,7 @@ int bbhip_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_st
                               int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
                               int border_mode, float border_value, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     Im2ColArgs a{dev_x_buf, dev_y_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  border_mode, border_value, 0, 0};
@@ -1205,7 +1235,7 @@ int bbhip_bit_Im2Col_Forward(int const *dev_x_buf, int *dev_y_buf, int x_stride,
                              int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
                              int border_mode, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     Im2ColArgs a{dev_x_buf, dev_y_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  border_mode, 0.0f, 0, 0};
@@ -1226,7 +1256,7 @@ int bbhip_fp32_Im2Col_Backward(float const *dev_dy_buf, float *dev_dx_buf, int x
                                int output_w_size, int output_h_size, int output_frame_stride, int filter_w_size, int filter_h_size,
                                void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     Im2ColArgs a{dev_dy_buf, dev_dx_buf, x_stride, y_stride, x_offset, y_offset, input_frame_size, input_frame_stride, input_w_size,
                  input_h_size, input_c_size, output_w_size, output_h_size, output_frame_stride, filter_w_size, filter_h_size,
                  0, 0.0f, 0, 0};
@@ -1261,7 +1291,7 @@ static int check_col2im(void const *p, void const *q, int w, int h, int c, int n
 int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
                               int output_frame_size, int output_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_col2im(dev_x_buf, dev_y_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, false, __func__)) { return 1; }
     int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
     long long const blocks = (long long)c_size * xy_tiles * f_tiles;
@@ -1276,7 +1306,7 @@ int bbhip_fp32_Col2Im_Forward(float const *dev_x_buf, float *dev_y_buf, int w_si
 int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w_size, int h_size, int c_size, int input_frame_stride,
                                int output_frame_size, int output_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_col2im(dev_dy_buf, dev_dx_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, false, __func__)) { return 1; }
     int const hw = h_size * w_size, xy_tiles = ceil_div(hw, kTile), f_tiles = ceil_div(output_frame_size, kTile);
     long long const blocks = (long long)c_size * xy_tiles * f_tiles;
@@ -1291,7 +1321,7 @@ int bbhip_fp32_Col2Im_Backward(float const *dev_dy_buf, float *dev_dx_buf, int w
 int bbhip_bit_Col2Im_Forward(int const *dev_x_buf, int *dev_y_buf, int w_size, int h_size, int c_size, int input_frame_stride,
                              int output_frame_size, int output_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_col2im(dev_x_buf, dev_y_buf, w_size, h_size, c_size, input_frame_stride, output_frame_size, output_frame_stride, true, __func__)) { return 1; }
     int const hw = h_size * w_size, words = (output_frame_size + 31) / 32;
     long long const total = (long long)c_size * hw * words;
@@ -1331,7 +1361,7 @@ static int launch_pool(PoolArgs const &a, bool backward, void *stream, char cons
 int bbhip_fp32_StochasticMaxPooling2x2_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size,
                                                int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     PoolArgs a{dev_x_buf, nullptr, dev_y_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
     return launch_pool(a, false, stream, __func__);
 }
@@ -1340,7 +1370,7 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
                                                 int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
                                                 int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     PoolArgs a{dev_x_buf, dev_dy_buf, dev_dx_buf, input_w_size, input_h_size, output_w_size, output_h_size, c_size, frame_size, frame_stride};
     return launch_pool(a, true, stream, __func__);
 }
@@ -1368,7 +1398,7 @@ static int check_average_lut(void const *a, void const *b, int const *idx, int n
 int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                                   int frame_stride, int binarize_input, int binarize_output, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
     int const f_blocks = ceil_div(frame_size, kTailBlock);
     long long const blocks = (long long)node_size * f_blocks;
@@ -1384,7 +1414,7 @@ int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int 
 int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                                  int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     int const words = (frame_size > 0) ? ceil_div(frame_size, 32) : 0;
     if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, words, __func__)) { return 1; }
     int const w_blocks = ceil_div(words, kTailBlock);
@@ -1416,7 +1446,7 @@ int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const
 int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
                                    int output_node_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_average_lut(dev_dy_buf, dev_dx_buf, dev_input_index, n, output_node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
     if (input_node_size <= 0) { return fail("%s: sizes must be positive", __func__); }
     int const total = output_node_size * n;
@@ -1448,7 +1478,7 @@ int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
 int bbhip_fp32_MaxLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                               int frame_stride, int binarize_input, int binarize_output, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
     int const f_blocks = ceil_div(frame_size, kTailBlock);
     long long const blocks = (long long)node_size * f_blocks;
@@ -1463,7 +1493,7 @@ int bbhip_fp32_MaxLut_Forward(float const *dev_x_buf, float *dev_y_buf, int cons
 int bbhip_bit_MaxLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                              int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     int const words = (frame_size > 0) ? ceil_div(frame_size, 32) : 0;
     if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, words, __func__)) { return 1; }
     int const w_blocks = ceil_div(words, kTailBlock);
@@ -1526,7 +1556,7 @@ static int launch_max_lut_backward(void const *x, bool bits, float const *dy, fl
 int bbhip_fp32_MaxLut_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n,
                                int input_node_size, int output_node_size, int frame_size, int frame_stride, int binarize_input, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_max_lut_backward(dev_x_buf, false, dev_dy_buf, dev_dx_buf, dev_input_index, n, input_node_size, output_node_size, frame_size,
                                    frame_stride, frame_stride, binarize_input, stream, __func__);
 }
@@ -1535,7 +1565,7 @@ int bbhip_bit_fp32_MaxLut_Backward(int const *dev_x_buf, float const *dev_dy_buf
                                    int input_node_size, int output_node_size, int frame_size, int x_frame_stride, int dy_frame_stride,
                                    void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_max_lut_backward(dev_x_buf, true, dev_dy_buf, dev_dx_buf, dev_input_index, n, input_node_size, output_node_size, frame_size,
                                    x_frame_stride, dy_frame_stride, 0, stream, __func__);
 }
@@ -1562,21 +1592,21 @@ static int launch_reduce_forward(void const *x, bool bits, float *y, int input_n
 int bbhip_fp32_Reduce_Forward(float const *dev_x_buf, float *dev_y_buf, int input_node_size, int output_node_size, int frame_size,
                               int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_reduce_forward(dev_x_buf, false, dev_y_buf, input_node_size, output_node_size, frame_size, frame_stride, frame_stride, stream, __func__);
 }
 
 int bbhip_bit_fp32_Reduce_Forward(int const *dev_x_buf, float *dev_y_buf, int input_node_size, int output_node_size, int frame_size,
                                   int x_frame_stride, int y_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_reduce_forward(dev_x_buf, true, dev_y_buf, input_node_size, output_node_size, frame_size, x_frame_stride, y_frame_stride, stream, __func__);
 }
 
 int bbhip_fp32_Reduce_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_node_size, int output_node_size, int frame_size,
                                int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (!(dev_dy_buf && dev_dx_buf)) { return fail("%s: null buffer", __func__); }
     if (!(input_node_size > 0 && output_node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (input_node_size % output_node_size != 0) { return fail("%s: the input nodes must be a multiple of the output nodes", __func__); }
@@ -1623,7 +1653,7 @@ static int launch_mean_squared_error(float const *y, float const *t, float *dy, 
 int bbhip_fp32_LossMeanSquaredError(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, int loss_buf_size,
                                     int node_size, int frame_size, int frame_stride, float grad_reduction, double loss_reduction, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_mean_squared_error(dev_y_buf, dev_t_buf, dev_dy_buf, dev_loss_buf, loss_buf_size, node_size, frame_size, frame_stride,
                                      grad_reduction, loss_reduction, true, stream, __func__);
 }
@@ -1631,7 +1661,7 @@ int bbhip_fp32_LossMeanSquaredError(float const *dev_y_buf, float const *dev_t_b
 int bbhip_fp32_MetricsMeanSquaredError(float const *dev_y_buf, float const *dev_t_buf, double *dev_accuracy_buf, int accuracy_buf_size,
                                        int node_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_mean_squared_error(dev_y_buf, dev_t_buf, nullptr, dev_accuracy_buf, accuracy_buf_size, node_size, frame_size, frame_stride,
                                      0.0f, (double)node_size, false, stream, __func__);
 }
@@ -1639,7 +1669,7 @@ int bbhip_fp32_MetricsMeanSquaredError(float const *dev_y_buf, float const *dev_
 int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, float t_sum,
                                        int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (!(dev_y_buf && dev_t_buf && dev_dy_buf && dev_loss_buf)) { return fail("%s: null buffer", __func__); }
     if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -1674,7 +1704,7 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
 int bbhip_fp32_MetricsCategoricalAccuracy(float const *dev_y_buf, float const *dev_t_buf, int *dev_accuracy_buf, int *dev_category_buf,
                                           int pix_size, int ch_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (!(dev_y_buf && dev_t_buf && dev_accuracy_buf && dev_category_buf)) { return fail("%s: null buffer", __func__); }
     if (!(pix_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -1747,7 +1777,7 @@ int bbhip_fp32_StochasticBatchNormalization_ForwardTraining(float const *dev_x_b
                                                             float *dev_running_mean_buf, float *dev_running_var_buf, float gamma, float beta,
                                                             float momentum, int node_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_bn(dev_x_buf, dev_y_buf, node_size, frame_size, frame_stride, frame_stride, __func__)) { return 1; }
     BBHIP_REQUIRE(dev_mean_buf != nullptr && dev_rstd_buf != nullptr && dev_running_mean_buf != nullptr && dev_running_var_buf != nullptr);
     BnArgs a{};
@@ -1762,7 +1792,7 @@ int bbhip_fp32_StochasticBatchNormalization_ReForward(float const *dev_x_buf, fl
                                                       float const *dev_rstd_buf, float gamma, float beta, int node_size, int frame_size,
                                                       int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_bn(dev_x_buf, dev_y_buf, node_size, frame_size, frame_stride, frame_stride, __func__)) { return 1; }
     BBHIP_REQUIRE(dev_mean_buf != nullptr && dev_rstd_buf != nullptr);
     BnArgs a{};
@@ -1776,7 +1806,7 @@ int bbhip_fp32_StochasticBatchNormalization_ForwardInference(float const *dev_x_
                                                              float const *dev_running_var_buf, float gamma, float beta, int node_size,
                                                              int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_bn(dev_x_buf, dev_y_buf, node_size, frame_size, frame_stride, frame_stride, __func__)) { return 1; }
     BBHIP_REQUIRE(dev_running_mean_buf != nullptr && dev_running_var_buf != nullptr);
     BnArgs a{};
@@ -1792,7 +1822,7 @@ int bbhip_fp32_StochasticBatchNormalization_Backward(float const *dev_x_buf, flo
                                                      float reciprocal_frame_size, int node_size, int frame_size, int frame_stride,
                                                      int x_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_bn(dev_x_buf, dev_dx_buf, node_size, frame_size, x_frame_stride, frame_stride, __func__)) { return 1; }
     BBHIP_REQUIRE(dev_dy_buf != nullptr && dev_mean_buf != nullptr && dev_rstd_buf != nullptr);
     BnArgs a{};
@@ -1848,7 +1878,7 @@ static int launch_row_map(int op, float const *x, float const *dy, float *out, f
 int bbhip_fp32_Binarize_Forward(float const *dev_x_buf, float *dev_y_buf, float binary_th, float binary_low, float binary_high,
                                 int node_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_row_map(kMapBinarize, dev_x_buf, nullptr, dev_y_buf, binary_th, binary_low, binary_high, node_size, frame_size, frame_stride,
                           stream, __func__);
 }
@@ -1856,7 +1886,7 @@ int bbhip_fp32_Binarize_Forward(float const *dev_x_buf, float *dev_y_buf, float 
 int bbhip_fp32_bit_Binarize_Forward(float const *dev_x_buf, int *dev_y_buf, float binary_th, int node_size, int frame_size,
                                     int x_frame_stride, int y_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (!(dev_x_buf && dev_y_buf)) { return fail("%s: null buffer", __func__); }
     if (!(node_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
     if (x_frame_stride < frame_size || y_frame_stride < (frame_size + 31) / 32) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -1876,14 +1906,14 @@ int bbhip_fp32_bit_Binarize_Forward(float const *dev_x_buf, int *dev_y_buf, floa
 int bbhip_fp32_HardTanh_Forward(float const *dev_x_buf, float *dev_y_buf, float limit_min, float limit_max, int node_size, int frame_size,
                                 int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_row_map(kMapHardTanh, dev_x_buf, nullptr, dev_y_buf, limit_min, limit_max, 0.0f, node_size, frame_size, frame_stride, stream, __func__);
 }
 
 int bbhip_fp32_HardTanh_Backward(float const *dev_x_buf, float const *dev_dy_buf, float *dev_dx_buf, float limit_min, float limit_max,
                                  int node_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_row_map(kMapHardTanhBackward, dev_x_buf, dev_dy_buf, dev_dx_buf, limit_min, limit_max, 0.0f, node_size, frame_size, frame_stride,
                           stream, __func__);
 }
@@ -1930,7 +1960,7 @@ int bbhip_fp32_RealToBinary_Forward(float const *dev_x_buf, float *dev_y_buf, un
                                     float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size,
                                     unsigned x_frame_size, unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_real_to_binary(dev_x_buf, dev_y_buf, false, depth_modulation_size, frame_modulation_size, input_range_lo, input_range_hi,
                                  point_size, x_depth_size, x_frame_size, x_frame_stride, y_frame_stride, binarize, stream, __func__);
 }
@@ -1939,7 +1969,7 @@ int bbhip_fp32_bit_RealToBinary_Forward(float const *dev_x_buf, int *dev_y_buf, 
                                         float input_range_lo, float input_range_hi, unsigned point_size, unsigned x_depth_size,
                                         unsigned x_frame_size, unsigned x_frame_stride, unsigned y_frame_stride, int binarize, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_real_to_binary(dev_x_buf, dev_y_buf, true, depth_modulation_size, frame_modulation_size, input_range_lo, input_range_hi,
                                  point_size, x_depth_size, x_frame_size, x_frame_stride, y_frame_stride, binarize, stream, __func__);
 }
@@ -1981,7 +2011,7 @@ static int launch_binary_to_real_forward(void const *x, bool bit, float *y, int 
 int bbhip_fp32_BinaryToReal_Forward(float const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
                                     int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_binary_to_real_forward(dev_x_buf, false, dev_y_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size,
                                          y_frame_stride, stream, __func__);
 }
@@ -1989,7 +2019,7 @@ int bbhip_fp32_BinaryToReal_Forward(float const *dev_x_buf, float *dev_y_buf, in
 int bbhip_bit_fp32_BinaryToReal_Forward(int const *dev_x_buf, float *dev_y_buf, int node_mux_size, int frame_mux_size, int y_node_size,
                                         int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_binary_to_real_forward(dev_x_buf, true, dev_y_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size,
                                          y_frame_stride, stream, __func__);
 }
@@ -1997,7 +2027,7 @@ int bbhip_bit_fp32_BinaryToReal_Forward(int const *dev_x_buf, float *dev_y_buf, 
 int bbhip_fp32_BinaryToReal_Backward(float const *dev_dy_buf, float *dev_dx_buf, int node_mux_size, int frame_mux_size, int y_node_size,
                                      int x_frame_stride, int y_frame_size, int y_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_binary_to_real(dev_dy_buf, dev_dx_buf, node_mux_size, frame_mux_size, y_node_size, x_frame_stride, y_frame_size, y_frame_stride,
                              __func__)) { return 1; }
     BinaryToRealArgs a{};
@@ -2059,7 +2089,7 @@ int bbhip_fp32_MaxPooling_Forward(float const *dev_x_buf, float *dev_y_buf, int 
                                   int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
                                   int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_pooling(dev_x_buf, dev_y_buf, dev_argmax_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size, output_h_size,
                       c_size, frame_size, __func__)) { return 1; }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -2086,7 +2116,7 @@ int bbhip_bit_MaxPooling_Forward(int const *dev_x_buf, int *dev_y_buf, int filte
                                  int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size, int frame_stride,
                                  void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_pooling(dev_x_buf, dev_y_buf, dev_y_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size, output_h_size,
                       c_size, frame_size, __func__)) { return 1; }
     int const words = (frame_size + 31) / 32;
@@ -2109,7 +2139,7 @@ int bbhip_fp32_MaxPooling_Backward(int const *dev_argmax_buf, float const *dev_d
                                    int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
                                    int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_pooling(dev_argmax_buf, dev_dy_buf, dev_dx_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size,
                       output_h_size, c_size, frame_size, __func__)) { return 1; }
     if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -2132,7 +2162,7 @@ int bbhip_bit_fp32_MaxPooling_Backward(int const *dev_x_buf, float const *dev_dy
                                        int input_w_size, int input_h_size, int output_w_size, int output_h_size, int c_size, int frame_size,
                                        int forward_frame_stride, int backward_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     if (check_pooling(dev_x_buf, dev_dy_buf, dev_dx_buf, filter_h_size, filter_w_size, input_w_size, input_h_size, output_w_size, output_h_size,
                       c_size, frame_size, __func__)) { return 1; }
     if (forward_frame_stride < (frame_size + 31) / 32 || backward_frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
@@ -2191,7 +2221,7 @@ static int launch_up_sampling(void const *x, float const *dy, void *out, bool bi
 int bbhip_fp32_UpSampling_Forward(float const *dev_x_buf, float *dev_y_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
                                   int filter_h_size, int fill, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_up_sampling(dev_x_buf, nullptr, dev_y_buf, false, false, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
                               frame_size, frame_stride, stream, __func__);
 }
@@ -2199,7 +2229,7 @@ int bbhip_fp32_UpSampling_Forward(float const *dev_x_buf, float *dev_y_buf, int 
 int bbhip_bit_UpSampling_Forward(int const *dev_x_buf, int *dev_y_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
                                  int filter_h_size, int fill, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_up_sampling(dev_x_buf, nullptr, dev_y_buf, true, false, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
                               frame_size, frame_stride, stream, __func__);
 }
@@ -2207,7 +2237,7 @@ int bbhip_bit_UpSampling_Forward(int const *dev_x_buf, int *dev_y_buf, int input
 int bbhip_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
                                    int filter_h_size, int fill, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     return launch_up_sampling(nullptr, dev_dy_buf, dev_dx_buf, false, true, input_w_size, input_h_size, c_size, filter_w_size, filter_h_size, fill,
                               frame_size, frame_stride, stream, __func__);
 }
@@ -2215,7 +2245,7 @@ int bbhip_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
                              int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr);
     BBHIP_REQUIRE(node_size > 0 && node_size <= 65535 * 1024 && frame_size > 0);
     BBHIP_REQUIRE(x_frame_stride >= (frame_size + 31) / 32 && y_frame_stride >= frame_size);
@@ -2511,7 +2541,7 @@ int bbhip_bit_fp32_DifferentiableLutN_Backward(int n, int const *dev_x_buf, floa
 int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
                                  int node_size, int frame_size, int frame_stride, void *stream)
 {
-    g_input_node_hint = 0;                          // a hint is for the next LUT forward call only
+    clear_hints();                                 // a hint is for the next LUT forward call only
     BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr && dev_input_index != nullptr && dev_table != nullptr);
     BBHIP_REQUIRE(node_size > 0 && node_size <= (0x7fffffff >> 6) && frame_size > 0);
     BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);

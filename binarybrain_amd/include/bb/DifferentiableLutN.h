@@ -7,6 +7,8 @@
 // hard-tanh window on dy in both binary and non-binary mode.  Frame work runs in the HIP library only.
 #pragma once
 
+#include <stack>
+
 #include <random>
 
 #include "bb/Model.h"
@@ -222,6 +224,29 @@ public:
         return std::vector<double>(1, (double)y);
     }
 
+private:
+    // A layer on fp32 frames in binary mode reads its input as bits.  The forward entry packs them into a buffer that the layer
+    // keeps beside the input it keeps anyway, and hands it back to the backward entry, which then does not pack again
+    // (bbhip_HintPackedInput).  One packed buffer per kept input, in the same order.
+    std::stack<FrameBuffer> m_packed_bufs;
+
+    // the hint for a call on x_buf: with `bits` the packed copy's place (or the copy itself, holds_input), else only the row count
+    void HintInput(FrameBuffer const &x_buf, FrameBuffer *bits, bool holds_input)
+    {
+        if (bits != nullptr && !bits->Empty()) {
+            auto p = bits->LockDeviceMemory(!holds_input);
+            bbhip_HintPackedInput((int *)p.GetAddr(), (int)x_buf.GetNodeSize(), (int)(bits->GetFrameStride() / 4), holds_input ? 1 : 0);
+        }
+        else { bbhip_HintInputNodeSize((int)x_buf.GetNodeSize()); }         // the forward signatures do not carry the input's row count
+    }
+
+public:
+    void Clear(void) override
+    {
+        Model::Clear();
+        while (!m_packed_bufs.empty()) { m_packed_bufs.pop(); }
+    }
+
     FrameBuffer Forward(FrameBuffer x_buf, bool train = true) override
     {
         RequireDevice("DifferentiableLutN::Forward");
@@ -239,6 +264,12 @@ public:
         int const O = (int)y_buf.GetNodeSize(), F = (int)y_buf.GetFrameSize();
         int const y_stride = (int)(y_buf.GetFrameStride() / 4), x_stride = (int)(x_buf.GetFrameStride() / 4);
         if (!kBitType) { BB_ASSERT(x_stride == y_stride); }
+        // the packed copy of a binarized fp32 input, kept for the backward pass of a training call
+        FrameBuffer bits_buf;
+        if (train) {
+            if (!kBitType && m_binary_mode) { bits_buf.Resize(x_buf.GetFrameSize(), m_input_shape, BB_TYPE_BIT); }
+            m_packed_bufs.push(bits_buf);
+        }
         auto x_ptr   = x_buf.LockDeviceMemoryConst();
         auto y_ptr   = y_buf.LockDeviceMemory(true);
         auto idx_ptr = m_connection_table.LockDeviceMemConst_InputTable();
@@ -255,7 +286,7 @@ public:
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, 0.0f, 1.0f, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW");
             }
             else {
-                bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
+                HintInput(x_buf, &bits_buf, false);
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float *)W_mut.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
                                 (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
@@ -278,7 +309,7 @@ public:
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTraining");
             }
             else {
-                bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
+                HintInput(x_buf, &bits_buf, false);
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTraining(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
                                 (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
@@ -308,7 +339,7 @@ public:
                             m_lut_binarize ? 1 : 0, m_unbinarize_bias, nullptr), "bbhip_bit_bit_fp32_StochasticLut_Forward");
         }
         else {
-            bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
+            HintInput(x_buf, &bits_buf, false);
             CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardNoBn(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                             (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), m_unbinarize_bias, O, F, y_stride,
                             m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_ForwardNoBn");
@@ -326,8 +357,11 @@ public:
         RequireDevice("DifferentiableLutN::Backward");
         m_flagClamp = true;
         FrameBuffer x_buf = this->PopFrameBuffer();
+        FrameBuffer bits_buf;
+        if (!m_packed_bufs.empty()) { bits_buf = m_packed_bufs.top(); m_packed_bufs.pop(); }
         if (!kBitType && x_buf.GetType() == BB_TYPE_BIT) { x_buf = x_buf.ConvertBitToFP32(); }
         BB_ASSERT(x_buf.GetType() == DataType<BinType>::type && x_buf.GetFrameSize() == dy_buf.GetFrameSize());
+        if (!bits_buf.Empty() && (bits_buf.GetFrameSize() != x_buf.GetFrameSize() || !m_binary_mode)) { bits_buf = FrameBuffer(); }
         FrameBuffer dx_buf(dy_buf.GetFrameSize(), m_input_shape, DataType<RealType>::type);
 
         FrameBuffer tmp_buf;
@@ -376,6 +410,7 @@ public:
                                 m_lut_binarize ? 1 : 0, nullptr), "bbhip_bit_fp32_DifferentiableLutN_Backward");
             }
             else {
+                if (!bits_buf.Empty()) { HintInput(x_buf, &bits_buf, true); }
                 CheckDevice(bbhip_fp32_DifferentiableLutN_Backward(N, (float const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
                                 tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),
                                 (float const *)mean_ptr.GetAddr(), (float const *)rstd_ptr.GetAddr(), (float *)dmean_ptr.GetAddr(), (float *)dvar_ptr.GetAddr(),
@@ -390,6 +425,7 @@ public:
                         "bbhip_bit_fp32_StochasticLut_Backward");
         }
         else {
+            if (!bits_buf.Empty()) { HintInput(x_buf, &bits_buf, true); }
             CheckDevice(bbhip_fp32_StochasticLut_Backward(N, (float const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
                             tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),
                             rev_stride, I, O, F, stride, (int)tmp_frame_size, tmp_stride, m_binary_mode ? 1 : 0, m_lut_binarize ? 1 : 0,

@@ -30,6 +30,7 @@ protected:
     std::string m_connection;
     indices_t   m_input_shape, m_output_shape;
     FrameBuffer m_x_buf;
+    FrameBuffer m_bits_buf;     // the packed copy of m_x_buf that the forward entry made (binary mode on fp32 frames)
     FixedSizeConnectionTable<N> m_connection_table;
     std::shared_ptr<Tensor> m_W, m_dW;
     std::mt19937_64 m_mt;
@@ -190,7 +191,13 @@ public:
         RequireDevice("StochasticLutN::Forward");
         if (x_buf.GetShape() != m_input_shape) { SetInputShape(x_buf.GetShape()); }
         FrameBuffer y_buf(x_buf.GetFrameSize(), m_output_shape, DataType<RealType>::type);
-        if (train) { m_x_buf = x_buf; }
+        if (train) {
+            m_x_buf = x_buf;
+            // in binary mode the layer reads fp32 frames as bits: the forward entry packs them into a buffer that is kept beside
+            // the input and handed back to the backward entry, which then does not pack again (bbhip_HintPackedInput)
+            m_bits_buf = FrameBuffer();
+            if (!kBitInput && m_binary_mode) { m_bits_buf.Resize(x_buf.GetFrameSize(), m_input_shape, BB_TYPE_BIT); }
+        }
 
         // The table is clamped to [0, 1] in place before every forward pass (reference: StochasticLutN.h:451): for fp32 frames
         // by the forward entry itself, in its table-preparation launch; for packed frames by a call of its own.
@@ -209,7 +216,11 @@ public:
         else {
             BB_ASSERT(x_buf.GetFrameStride() == y_buf.GetFrameStride());
             auto W_ptr = m_W->LockDeviceMemory();
-            bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
+            if (train && !m_bits_buf.Empty()) {
+                auto bits_ptr = m_bits_buf.LockDeviceMemory(true);
+                bbhip_HintPackedInput((int *)bits_ptr.GetAddr(), (int)x_buf.GetNodeSize(), (int)(m_bits_buf.GetFrameStride() / sizeof(int)), 0);
+            }
+            else { bbhip_HintInputNodeSize((int)x_buf.GetNodeSize()); }     // the forward signatures do not carry the input's row count
             CheckDevice(bbhip_fp32_StochasticLut_ForwardClampW(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                             (int const *)idx_ptr.GetAddr(), (float *)W_ptr.GetAddr(),
                             (int)y_buf.GetNodeSize(), (int)y_buf.GetFrameSize(), (int)(y_buf.GetFrameStride() / sizeof(float)),
@@ -219,15 +230,16 @@ public:
         return y_buf;
     }
 
-    void Clear(void) override { Model::Clear(); m_x_buf = FrameBuffer(); }
+    void Clear(void) override { Model::Clear(); m_x_buf = FrameBuffer(); m_bits_buf = FrameBuffer(); }
 
     FrameBuffer Backward(FrameBuffer dy_buf) override
     {
         if (dy_buf.Empty()) { return FrameBuffer(); }       // (the reference also drops its dW tensor here — a defect, not kept)
         BB_ASSERT(dy_buf.GetType() == DataType<RealType>::type);
         RequireDevice("StochasticLutN::Backward");
-        FrameBuffer x_buf = m_x_buf;
+        FrameBuffer x_buf = m_x_buf, bits_buf = m_bits_buf;
         m_x_buf = FrameBuffer();
+        m_bits_buf = FrameBuffer();
         BB_ASSERT(!x_buf.Empty() && x_buf.GetFrameSize() == dy_buf.GetFrameSize());
         FrameBuffer dx_buf(dy_buf.GetFrameSize(), m_input_shape, DataType<RealType>::type);
 
@@ -264,6 +276,10 @@ public:
                         "bbhip_bit_fp32_StochasticLut_Backward");
         }
         else {
+            if (!bits_buf.Empty() && m_binary_mode && bits_buf.GetFrameSize() == x_buf.GetFrameSize()) {
+                auto bits_ptr = bits_buf.LockDeviceMemory();
+                bbhip_HintPackedInput((int *)bits_ptr.GetAddr(), (int)x_buf.GetNodeSize(), (int)(bits_buf.GetFrameStride() / sizeof(int)), 1);
+            }
             CheckDevice(bbhip_fp32_StochasticLut_Backward(N, (float const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(),
                             (float *)dx_ptr.GetAddr(), tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(),
                             (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(), (int)m_connection_table.GetReverseTableStride(),

@@ -503,13 +503,29 @@ def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
     return y
 
 
-def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None, clamp_w=None):
+def packed_input_buffer(rows, frame_size, device="cuda"):
+    """A place for the packed copy of a binarized fp32 input of `rows` node rows (see `packed=` of the LUT forward / backward wrappers):
+    the forward call fills it, the backward call on the same input reads it instead of packing the input again."""
+    return torch.empty((rows, lib().bbhip_PackedRowWords(frame_size)), dtype=torch.int32, device=device)
+
+
+def _hint_input(x, packed, holds_input):
+    """what the wrapper knows about the next LUT call's input: its row count, and where its packed copy goes to / comes from"""
+    if packed is not None:
+        _dev(packed)
+        assert packed.dtype == torch.int32 and packed.shape[0] == x.shape[0]
+        lib().bbhip_HintPackedInput(ptr(packed), x.shape[0], packed.shape[1], int(holds_input))
+    elif not holds_input:
+        lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+
+
+def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None, clamp_w=None, packed=None):
     """clamp_w = (lo, hi): W is clamped in place first, as StochasticLutN::Forward does (include/bb/StochasticLutN.h:451),
     by the same launch that prepares the tables."""
     _dev(x, idx, W, out)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
-    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+    _hint_input(x, packed, False)
     if clamp_w is not None:
         check(lib().bbhip_fp32_StochasticLut_ForwardClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, frame_size, x.shape[1],
                                                            int(input_binary), int(lut_binarize), bias, float(clamp_w[0]), float(clamp_w[1]), stream_ptr()))
@@ -552,7 +568,7 @@ def _tmp_for(output_nodes, n, frame_size, device, max_tmp_bytes):
 
 
 def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_binary=False, lut_binarize=False, bias=0.25,
-                            dx_tmp=None, tmp_frame_size=None, max_tmp_bytes=256 * 1024 * 1024, out=None):
+                            dx_tmp=None, tmp_frame_size=None, max_tmp_bytes=256 * 1024 * 1024, out=None, packed=None):
     """dW is accumulated in place; returns dx [I, stride]. ``rev`` (reverse table) is needed by dx modes 0 and 2,
     dx_tmp by mode 2 only (allocated here when not given)."""
     _dev(x, dy, idx, W, dW, rev, dx_tmp, out)
@@ -564,6 +580,7 @@ def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_bi
         tf = min(ts, frame_size) if tmp_frame_size is None else tmp_frame_size
     elif lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
+    _hint_input(x, packed, True)
     check(lib().bbhip_fp32_StochasticLut_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                   0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,
                                                   int(input_binary), int(lut_binarize), bias, stream_ptr()))
@@ -585,8 +602,9 @@ def bit_stochastic_lut_backward(n, xbits, dy, idx, W, dW, frame_size, rev=None, 
 
 
 def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None):
+                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None, packed=None):
     """fp32 frames. running_mean / running_var are updated in place. returns (y, mean, rstd).
+    packed: a `packed_input_buffer` that receives the packed copy of the binarized input (binary mode), for the backward call.
     clamp_w = (lo, hi): W is clamped in place first, by the launch that prepares the tables (the model class's clamp before the
     first forward pass after a backward pass, include/bb/DifferentiableLutN.h:605-608)."""
     _dev(x, idx, W, running_mean, running_var)
@@ -594,7 +612,7 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
     mean = torch.empty(O, dtype=torch.float32, device=x.device)
     rstd = torch.empty(O, dtype=torch.float32, device=x.device)
-    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+    _hint_input(x, packed, False)
     if clamp_w is not None:
         check(lib().bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                                         ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
@@ -650,18 +668,19 @@ def bit_differentiable_lut_forward_inference(n, xbits, idx, W, frame_size, runni
     return y
 
 
-def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_binarize=False, binary_mode=True):
+def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_binarize=False, binary_mode=True, packed=None):
     _dev(x, idx, W)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
-    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+    _hint_input(x, packed, False)
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardNoBn(n, ptr(x), ptr(y), ptr(idx), ptr(W), bias, O, frame_size, x.shape[1],
                                                           int(lut_binarize), int(binary_mode), stream_ptr()))
     return y
 
 
 def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, rev=None, gamma=0.3, beta=0.5, bias=0.25,
-                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024):
+                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024, packed=None):
+    """packed: the buffer that the forward call on the same x filled (`packed_input_buffer`): the call reads it instead of packing x."""
     _dev(x, dy, idx, W, dW, mean, rstd, rev)
     I = x.shape[0]; O = idx.shape[0]
     dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=x.device)
@@ -670,6 +689,7 @@ def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, re
     dx_tmp, tf, ts = (None, 0, 0)
     if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
+    _hint_input(x, packed, True)
     check(lib().bbhip_fp32_DifferentiableLutN_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                        ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
                                                        0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,

@@ -105,6 +105,21 @@ int  bbhip_GetDxMode(void);
  * of them with it): the value is trusted like the sizes of any entry point.  Results do not depend on the hint. */
 void bbhip_HintInputNodeSize(int input_node_size);
 
+/* ---- a caller-owned place for the packed copy of a binarized fp32 input (no counterpart in the reference) ----
+ * In binary mode on fp32 frames a LUT layer reads bits: the forward and the backward entry each pack the binarized input once
+ * (bit = x > 0.5) into the library's scratch, because the entry points share no state.  A caller that keeps the layer's input
+ * between the two calls anyway (the model classes do) can keep the packed copy as well and save the backward pass its packing:
+ *   - right before the forward call, with holds_input = 0: dev_bits, `rows` rows (the input's node count: this also serves as
+ *     bbhip_HintInputNodeSize) of row_words 32-bit words each, receives the packed copy instead of the library's scratch;
+ *   - right before the backward call on the same input, with holds_input = 1: the buffer still holds that copy (the caller's
+ *     promise: x has not changed since), and the call reads it instead of packing x again.
+ * row_words must be a multiple of 8 and at least ceil(frame_size / 32) (bbhip_PackedRowWords(frame_size) gives the pitch the
+ * library itself would use), dev_bits 32-byte aligned; a buffer that does not fit the call is ignored (the library packs into its
+ * scratch as always).  Like the other hint it holds for the next LUT call of the same thread and is cleared by any entry.
+ * Results do not depend on it. */
+int  bbhip_PackedRowWords(int frame_size);
+void bbhip_HintPackedInput(int *dev_bits, int rows, int row_words, int holds_input);
+
 /* ---- kernel timer (instrumentation; no counterpart in the reference) ----
  * While enabled, every call brackets its dominant kernel (which: 0 = LUT forward kernel, 1 = LUT backward kernel,
  * 2 = BinaryLut6 kernel, 3 = input-centric dx kernel, 4 = the kernels of any other entry: vector operations, Adam, Im2Col,
