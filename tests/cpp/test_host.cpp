@@ -10,6 +10,10 @@
 #include "bb/DifferentiableLutN.h"
 #include "bb/BinaryLutN.h"
 #include "bb/ObjectLoader.h"
+#include "bb/BinaryModulation.h"
+#include "bb/DifferentiableLutDiscreteN.h"
+#include "bb/MaxPooling.h"
+#include "bb/UpSampling.h"
 #include "../../binarybrain_amd/csrc/tile_divisor.hpp"
 
 extern "C" int oracle_ReverseTable(int n, std::int32_t const *idx, int input_node_size, int output_node_size, std::int32_t *rev, int rev_cap);
@@ -186,6 +190,47 @@ int main(void)
         auto t2 = std::dynamic_pointer_cast<bb::Tensor_<std::int32_t>>(bb::Object_Load(s5));
         CHECK(t2 && t2->GetShape() == bb::indices_t({2, 3}));
         if (t2) { auto p = t2->LockConst(); CHECK(p(1, 1) == 5 && p(1, 2) == 6); }          // ObjectTest.cpp:185-186
+    }
+    // the layers around the LUT layers: shapes, commands, refusals, and the device path's refusal without a device
+    {
+        auto r2b = bb::RealToBinary<bb::Bit>::Create(7, 3);
+        CHECK(r2b->SetInputShape({2, 4, 5}) == bb::indices_t({6, 4, 5}) && r2b->GetInputNodeSize() == 40 && r2b->GetOutputNodeSize() == 120);
+        CHECK(r2b->GetObjectName() == "RealToBinary_bit_fp32" && r2b->GetModulationSize() == 7);
+        bool threw = false;
+        try { bb::RealToBinary<float>::Create(2, std::make_shared<bb::Tensor>()); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);                                                   // thresholds from a value generator are not provided
+        auto b2r = bb::BinaryToReal<bb::Bit>::Create(7, bb::indices_t({10}));
+        CHECK(b2r->SetInputShape({70}) == bb::indices_t({10}));
+        auto by_depth = bb::BinaryToReal<float>::Create(1, 7);
+        CHECK(by_depth->SetInputShape({70, 2}) == bb::indices_t({10, 2}));
+        threw = false;
+        try { bb::BinaryToReal<float>::Create(1, bb::indices_t({9}))->SetInputShape({70}); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);                                                   // 70 inputs do not fold into 9 outputs
+        auto pool = bb::MaxPooling<bb::Bit>::Create(2, 3);
+        CHECK(pool->SetInputShape({4, 5, 7}) == bb::indices_t({4, 3, 3}) && pool->GetFilterHeight() == 2 && pool->GetFilterWidth() == 3);
+        auto up = bb::UpSampling<>::Create(2, 3, false);
+        CHECK(up->SetInputShape({4, 5, 7}) == bb::indices_t({4, 10, 21}) && up->GetOutputNodeSize() == 840);
+        auto tanh = bb::HardTanh<>::Create(0.0f, 1.0f);
+        CHECK(tanh->ForwardNode(0, {-0.5, 0.25, 2.0}) == std::vector<double>({0.0, 0.25, 1.0}));
+        tanh->SendCommand("binary true");
+        CHECK(tanh->ForwardNode(0, {0.4, 0.6}) == std::vector<double>({0.0, 1.0}));
+        auto body = bb::Sequential::Create();
+        body->Add(bb::DifferentiableLutN<6, bb::Bit>::Create((bb::index_t)36));
+        body->Add(bb::DifferentiableLutDiscreteN<6, bb::Bit>::Create((bb::index_t)12));
+        auto net = bb::BinaryModulation<bb::Bit>::Create(body, 7, 15);
+        CHECK(net->SetInputShape({20}) == bb::indices_t({12}) && net->GetInputNodeSize() == 20 && net->GetLayer() == body);
+        CHECK(net->GetParameters().GetSize() == 2 && net->GetGradients().GetSize() == 2);
+        std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+        net->DumpObject(ss);
+        auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+        CHECK((bool)again && again->GetObjectName() == "BinaryModulation_bit_fp32" && again->GetOutputNodeSize() == 12);
+        std::stringstream s1(std::ios::in | std::ios::out | std::ios::binary), s2(std::ios::in | std::ios::out | std::ios::binary);
+        net->DumpObject(s1);
+        if (again) { again->DumpObject(s2); CHECK(s1.str() == s2.str()); }
+        bb::FrameBuffer x(8, {20}, BB_TYPE_FP32, true);
+        threw = false;
+        try { net->Forward(x); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);                                                   // no device: the layers refuse instead of computing on the host
     }
     // workgroup index -> (frame chunk, node tile) without an integer division: exact for every index below 2^31
     {
