@@ -178,7 +178,7 @@ def bench_conv(args, lib):
         total_ms += med
         kernels[name] = {"ms": med, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (med * 1e-3) / 1e9}
     dom = max(kernels, key=lambda k: kernels[k]["ms"])
-    # MaxPooling (what binary networks pool with) and UpSampling at the same maps, listed beside the block's own kernels, not added
+    # MaxPooling (what binary networks pool with), UpSampling and Shuffle at the same maps, listed beside the block's own kernels, not added
     _, arg = ops.max_pooling_forward(maps, CO, OH, OW, 2, 2, F)
     PO = CO * (OH // 2) * (OW // 2)
     maps_bits = ops.binarize_forward(maps, F, 0.5, bit=True, y_stride=synth.frame_stride_bit(F))
@@ -191,6 +191,8 @@ def bench_conv(args, lib):
          F // 8 * CO * OH * OW + e * F * (CO * OH * OW + PO)),
         ("up_sampling_forward_kernel 2x2", lambda: ops.up_sampling_forward(pooled, CO, OH // 2, OW // 2, 2, 2, F), e * F * (CO * OH * OW + PO)),
         ("up_sampling_backward_kernel 2x2", lambda: ops.up_sampling_backward(dup, CO, OH // 2, OW // 2, 2, 2, F), e * F * (CO * OH * OW + PO)),
+        ("row_shuffle_kernel unit 36", lambda: ops.shuffle_forward(maps, CO, F), 2 * e * F * CO * OH * OW),
+        ("row_shuffle_kernel unit 36, packed", lambda: ops.shuffle_forward(maps_bits, CO, F), 2 * 4 * maps_bits.shape[1] * CO * OH * OW),    # rows move whole
     ]
     for name, fn, nbytes in beside:
         med = library_timed_ms(lib, fn, args.steps, args.warmup)

@@ -98,6 +98,8 @@ _SIGNATURES = {
     "bbhip_fp32_UpSampling_Forward": (C.c_int, [_vp, _vp] + [_i] * 8 + [_vp]),
     "bbhip_bit_UpSampling_Forward": (C.c_int, [_vp, _vp] + [_i] * 8 + [_vp]),
     "bbhip_fp32_UpSampling_Backward": (C.c_int, [_vp, _vp] + [_i] * 8 + [_vp]),
+    "bbhip_Shuffle_Forward": (C.c_int, [_vp, _vp] + [_u] * 4 + [_vp]),
+    "bbhip_Shuffle_Backward": (C.c_int, [_vp, _vp] + [_u] * 4 + [_vp]),
     "bbhip_fp32_ConvBitToReal": (C.c_int, [_vp, _vp, _f, _f, _i, _i, _i, _i, _vp]),
     "bbhip_fp32_StochasticLut_Forward": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "bbhip_fp32_StochasticLut_Forward_NoAlloc": (C.c_int, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),

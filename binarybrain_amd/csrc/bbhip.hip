@@ -2242,6 +2242,47 @@ int bbhip_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, i
                               frame_size, frame_stride, stream, __func__);
 }
 
+// ---- Shuffle ----
+static int launch_shuffle(int const *src, int *dst, unsigned unit_size, unsigned group_size, unsigned node_size, unsigned frame_size,
+                          unsigned frame_stride, void *stream, char const *name)
+{
+    if (!(src && dst)) { return fail("%s: null buffer", name); }
+    if (unit_size == 0 || node_size == 0 || frame_size == 0 || frame_stride == 0) { return fail("%s: sizes must be positive", name); }
+    if ((unsigned long long)unit_size * group_size != node_size) { return fail("%s: node_size must be a multiple of the unit size", name); }
+    if (node_size > 0x7fffffffu || frame_stride > 0x7fffffffu) { return fail("%s: buffer too large", name); }
+    bool const wide = (frame_stride & 3u) == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0;
+    unsigned const pieces = wide ? frame_stride / 4 : frame_stride;
+    long long const total = (long long)node_size * pieces;
+    if (total > 0x7fffffffLL) { return fail("%s: grid too large", name); }
+    ShuffleArgs a{};
+    a.src = reinterpret_cast<uint32_t const *>(src); a.dst = reinterpret_cast<uint32_t *>(dst);
+    a.pieces = make_tile_divisor((int)pieces); a.unit = make_tile_divisor((int)unit_size);
+    a.group_size = (int)group_size; a.stride = (int)frame_stride;
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    dim3 const grid((unsigned)((total + kPoolBlock - 1) / kPoolBlock)), block(kPoolBlock);
+    if (wide) { hipLaunchKernelGGL(row_shuffle_kernel<4>, grid, block, 0, st, a, total); }
+    else      { hipLaunchKernelGGL(row_shuffle_kernel<1>, grid, block, 0, st, a, total); }
+    BBHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+int bbhip_Shuffle_Forward(int const *dev_x_buf, int *dev_y_buf, unsigned int y_unit_size, unsigned int node_size, unsigned int frame_size,
+                          unsigned int frame_stride, void *stream)
+{
+    clear_hints();                                 // a hint is for the next LUT forward call only
+    if (y_unit_size == 0) { return fail("%s: sizes must be positive", __func__); }
+    return launch_shuffle(dev_x_buf, dev_y_buf, y_unit_size, node_size / y_unit_size, node_size, frame_size, frame_stride, stream, __func__);
+}
+
+int bbhip_Shuffle_Backward(int const *dev_dy_buf, int *dev_dx_buf, unsigned int y_unit_size, unsigned int node_size, unsigned int frame_size,
+                           unsigned int frame_stride, void *stream)
+{
+    clear_hints();                                 // a hint is for the next LUT forward call only
+    if (y_unit_size == 0 || node_size % y_unit_size != 0) { return fail("%s: node_size must be a multiple of the unit size", __func__); }
+    return launch_shuffle(dev_dy_buf, dev_dx_buf, node_size / y_unit_size, y_unit_size, node_size, frame_size, frame_stride, stream, __func__);
+}
+
 int bbhip_fp32_ConvBitToReal(int const *dev_x_buf, float *dev_y_buf, float value0, float value1,
                              int node_size, int frame_size, int x_frame_stride, int y_frame_stride, void *stream)
 {

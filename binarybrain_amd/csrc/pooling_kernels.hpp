@@ -1,6 +1,6 @@
-// MaxPooling and UpSampling over images held as rows (channel, y, x) of frames
+// MaxPooling and UpSampling over images held as rows (channel, y, x) of frames, and Shuffle, a permutation of whole rows
 // (reference: include/bb/MaxPooling.h:251-284, 340-370, 478-506, 551-579; include/bb/UpSampling.h:223-259, 321-353;
-// entry points include/bbcu/bbcu.h:949-1016, 1024-1069).
+// include/bb/Shuffle.h:166-185, 225-243; entry points include/bbcu/bbcu.h:949-1016, 1024-1069, 1194-1216).
 //
 // Windows of filter_h x filter_w tile the image without overlap (the last ones are cut off at the border), so every input
 // element belongs to one window and every kernel writes each output element once: streaming maps with one thread per W
@@ -254,6 +254,32 @@ __global__ __launch_bounds__(kPoolBlock) void up_sampling_backward_kernel(Window
         for (int j = 0; j < W; ++j) { sum[j] += g[j]; }          // 0 + dy, as the host loop adds it
     }
     bn_store<W>(static_cast<float *>(a.out) + (size_t)node * a.out_stride, f, a.frame_size, sum);
+}
+
+// ---- Shuffle -------------------------------------------------------------------------------------------------------
+// Destination row group * unit.count + u takes source row u * group_size + group: the rows, seen as a [unit][group] matrix,
+// are transposed.  The backward pass is the same copy with the two extents exchanged.  Rows are copied whole, whatever they
+// hold; one thread per (destination row, piece of V words), pieces numbered through so that short rows still fill the chip.
+struct ShuffleArgs {
+    uint32_t const *src;
+    uint32_t       *dst;
+    TileDivisor     pieces;     // per row
+    TileDivisor     unit;
+    int             group_size;
+    int             stride;     // words per row
+};
+
+template <int V>
+__global__ __launch_bounds__(kPoolBlock) void row_shuffle_kernel(ShuffleArgs a, long long total)
+{
+    long long const gid = (long long)blockIdx.x * kPoolBlock + threadIdx.x;
+    if (gid >= total) { return; }
+    int row, piece, group, u;
+    split_tile((int)gid, a.pieces, row, piece);
+    split_tile(row, a.unit, group, u);
+    size_t const from = ((size_t)u * a.group_size + group) * a.stride, to = (size_t)row * a.stride;
+    if constexpr (V == 4) { reinterpret_cast<uint4 *>(a.dst + to)[piece] = reinterpret_cast<uint4 const *>(a.src + from)[piece]; }
+    else                  { a.dst[to + piece] = a.src[from + piece]; }
 }
 
 }  // namespace bbhip

@@ -1,6 +1,6 @@
 // Reconstruct a serialized object from its recorded type name (reference: include/bb/ObjectLoader.h:407-447
 // `Object_Load` / `Object_LoadFromFile`).  Known here: the LUT layers of widths 2..6 on fp32 or packed-bit frames,
-// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, Binarize, HardTanh, RealToBinary, BinaryToReal, BinaryModulation, DifferentiableLutDiscreteN (the LUT layer put together from its parts), MaxPooling, UpSampling, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
+// BinaryLut6, StochasticBatchNormalization, AverageLut, MaxLut, Reduce, Binarize, HardTanh, RealToBinary, BinaryToReal, BinaryModulation, DifferentiableLutDiscreteN (the LUT layer put together from its parts), MaxPooling, UpSampling, Shuffle, the convolution wrapper with its Im2Col / Col2Im, the layer list, and tensors.  An unknown name yields an empty pointer, as in the reference.
 #pragma once
 
 #include "bb/StochasticLutN.h"
@@ -22,6 +22,7 @@
 #include "bb/DifferentiableLutDiscreteN.h"
 #include "bb/MaxPooling.h"
 #include "bb/UpSampling.h"
+#include "bb/Shuffle.h"
 
 namespace bb {
 
@@ -68,6 +69,7 @@ inline std::shared_ptr<Object> CreateByName(std::string const &name)
     if (name == MaxPooling<Bit, float>::ObjectName())             { return MaxPooling<Bit, float>::Create(); }
     if (name == UpSampling<float, float>::ObjectName())           { return UpSampling<float, float>::Create(); }
     if (name == UpSampling<Bit, float>::ObjectName())             { return UpSampling<Bit, float>::Create(); }
+    if (name == Shuffle::ObjectName())                            { return Shuffle::Create(); }
     if (name == Convolution2d<float, float>::ObjectName())        { return Convolution2d<float, float>::Create(); }
     if (name == Convolution2d<Bit, float>::ObjectName())          { return Convolution2d<Bit, float>::Create(); }
     if (name == ConvolutionIm2Col<float, float>::ObjectName())    { return ConvolutionIm2Col<float, float>::Create(1, 1); }

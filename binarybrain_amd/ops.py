@@ -451,6 +451,21 @@ def up_sampling_backward(dy, c, h, w, fh, fw, frame_size, fill=True):
     return dx
 
 
+def shuffle_forward(x, shuffle_unit, frame_size):
+    """x [nodes, stride], fp32 or int32 packed words: row i * shuffle_unit + j of the result is row j * (nodes / shuffle_unit) + i"""
+    _dev(x)
+    y = torch.empty_like(x)
+    check(lib().bbhip_Shuffle_Forward(ptr(x), ptr(y), shuffle_unit, x.shape[0], frame_size, x.shape[1], stream_ptr()))
+    return y
+
+
+def shuffle_backward(dy, shuffle_unit, frame_size):
+    _dev(dy)
+    dx = torch.empty_like(dy)
+    check(lib().bbhip_Shuffle_Backward(ptr(dy), ptr(dx), shuffle_unit, dy.shape[0], frame_size, dy.shape[1], stream_ptr()))
+    return dx
+
+
 def loss_mean_squared_error(y, t, frame_size, loss_buf, batch_size=None, reduction_sum=False):
     """-> dy; loss_buf (float64, device, any length >= 1) receives the batch's partial sums ON TOP of what it holds.  The layer's loss is
     loss_buf.sum() / frames seen (the sum itself with reduction "sum")."""

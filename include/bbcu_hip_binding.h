@@ -453,6 +453,26 @@ inline int bbcu_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_
     return 0;
 }
 
+/* ---- bbcu_Shuffle_Forward<T> / bbcu_Shuffle_Backward<T>, include/bbcu/bbcu.h:1194-1216 (T = int or float: rows of 32-bit words) ---- */
+template <typename T>
+int bbcu_Shuffle_Forward(T const *dev_x_buf, T *dev_y_buf, unsigned int y_unit_size, unsigned int node_size, unsigned int frame_size,
+                         unsigned int frame_stride, cudaStream_t streamId = 0)
+{
+    static_assert(sizeof(T) == 4, "rows of 32-bit words");
+    BBCU_HIP_CALL(bbhip_Shuffle_Forward(reinterpret_cast<int const *>(dev_x_buf), reinterpret_cast<int *>(dev_y_buf), y_unit_size, node_size,
+                                        frame_size, frame_stride, streamId));
+    return 0;
+}
+template <typename T>
+int bbcu_Shuffle_Backward(T const *dev_dy_buf, T *dev_dx_buf, unsigned int y_unit_size, unsigned int node_size, unsigned int frame_size,
+                          unsigned int frame_stride, cudaStream_t streamId = 0)
+{
+    static_assert(sizeof(T) == 4, "rows of 32-bit words");
+    BBCU_HIP_CALL(bbhip_Shuffle_Backward(reinterpret_cast<int const *>(dev_dy_buf), reinterpret_cast<int *>(dev_dx_buf), y_unit_size, node_size,
+                                         frame_size, frame_stride, streamId));
+    return 0;
+}
+
 /* ---- Im2Col / Col2Im, include/bbcu/bbcu.h:1076-1186 ---- */
 inline int bbcu_fp32_Im2Col_Forward(float const *dev_x_buf, float *dev_y_buf, int x_stride, int y_stride, int x_offset, int y_offset,
         int input_frame_size, int input_frame_stride, int input_w_size, int input_h_size, int input_c_size, int output_w_size,

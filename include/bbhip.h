@@ -360,6 +360,17 @@ int bbhip_bit_UpSampling_Forward(int const *dev_x_buf, int *dev_y_buf, int input
 int bbhip_fp32_UpSampling_Backward(float const *dev_dy_buf, float *dev_dx_buf, int input_w_size, int input_h_size, int c_size, int filter_w_size,
                                    int filter_h_size, int fill, int frame_size, int frame_stride, void *stream);
 
+/* ---- Shuffle ----
+ * bbcu_Shuffle_Forward<T>, include/bbcu/bbcu.h:1194-1204: with x_unit_size = node_size / y_unit_size, output row i * y_unit_size + j is
+ * input row j * x_unit_size + i (include/bb/Shuffle.h:166-185).  Rows are frame_stride 32-bit words whatever they hold (fp32 frames or
+ * packed bits: the reference's class passes both as int) and are copied whole; node_size must be a multiple of y_unit_size. */
+int bbhip_Shuffle_Forward(int const *dev_x_buf, int *dev_y_buf, unsigned int y_unit_size, unsigned int node_size, unsigned int frame_size,
+                          unsigned int frame_stride, void *stream);
+/* bbcu_Shuffle_Backward<T>, include/bbcu/bbcu.h:1206-1216: input-gradient row i * x_unit_size + j is output-gradient row
+ * j * y_unit_size + i (include/bb/Shuffle.h:225-243) */
+int bbhip_Shuffle_Backward(int const *dev_dy_buf, int *dev_dx_buf, unsigned int y_unit_size, unsigned int node_size, unsigned int frame_size,
+                           unsigned int frame_stride, void *stream);
+
 /* ---- mean squared error ---- */
 /* bbcu_fp32_LossMeanSquaredError, include/bbcu/bbcu.h:1487-1500: dy = (y - t) * grad_reduction (the caller passes 2 / (nodes * batch)
  * or 2); dev_loss_buf[s] += the sum over the frames s, s + loss_buf_size, ... and all nodes of (float)(y - t)^2 * loss_reduction in

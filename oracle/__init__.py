@@ -448,6 +448,22 @@ def up_sampling_backward(dy, c, h, w, fh, fw, frame_size, fill=True):
     return dx
 
 
+def shuffle_forward(x, shuffle_unit):
+    """Rows of 32-bit words (fp32 or packed bits alike), x [nodes, stride] -> y (include/bb/Shuffle.h:166-185)"""
+    x = np.ascontiguousarray(x); assert x.dtype.itemsize == 4 and x.shape[0] % shuffle_unit == 0
+    y = np.zeros_like(x)
+    lib().oracle_Shuffle_Forward(_ptr(x), _ptr(y), C.c_int(shuffle_unit), C.c_int(x.shape[0]), C.c_int(x.shape[1]))
+    return y
+
+
+def shuffle_backward(dy, shuffle_unit):
+    """include/bb/Shuffle.h:225-243"""
+    dy = np.ascontiguousarray(dy); assert dy.dtype.itemsize == 4 and dy.shape[0] % shuffle_unit == 0
+    dx = np.zeros_like(dy)
+    lib().oracle_Shuffle_Backward(_ptr(dy), _ptr(dx), C.c_int(shuffle_unit), C.c_int(dy.shape[0]), C.c_int(dy.shape[1]))
+    return dx
+
+
 def loss_mean_squared_error(y, t, frame_size, batch_size=None, reduction_sum=False, loss=0.0):
     """-> (dy, loss accumulator): the reference's host loop (include/bb/LossMeanSquaredError.h:121-169) for one batch; `loss` is the
     accumulator before the batch.  The layer's loss is accumulator / frames seen (the accumulator itself with reduction "sum")."""
@@ -1046,6 +1062,23 @@ def ref_up_sampling(x, c, h, w, fh, fw, frames, fill=True, bit=False, dy=None, n
     f.restype = C.c_long
     r = f(C.c_int(int(bit)), C.c_int(c), C.c_int(h), C.c_int(w), C.c_int(fh), C.c_int(fw), C.c_int(int(fill)), C.c_int(frames), _ptr(x), _ptr(y),
           _ptr(dy), _ptr(dx), C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
+    assert r >= 0, r
+    return y, dx, (out[:r].copy() if want_object else None)
+
+
+def ref_shuffle(x, shuffle_unit, frames, bit=False, dy=None, name="", want_object=False):
+    """The reference's Shuffle host path on dense arrays (fp32 [nodes, frames] or packed words) -> (y, dx, object bytes)."""
+    dt = np.int32 if bit else np.float32
+    x = _c(x, dt)
+    y = np.zeros_like(x)
+    dx = None
+    if dy is not None:
+        dy = _c(dy, dt); dx = np.zeros_like(x)
+    out = np.zeros(1 << 16, np.uint8) if want_object else None
+    f = ref().bbref_Shuffle
+    f.restype = C.c_long
+    r = f(C.c_int(int(bit)), C.c_int(shuffle_unit), C.c_int(x.shape[0]), C.c_int(frames), _ptr(x), _ptr(y), _ptr(dy), _ptr(dx),
+          C.c_char_p(name.encode()), _ptr(out), C.c_long(out.size if want_object else 0))
     assert r >= 0, r
     return y, dx, (out[:r].copy() if want_object else None)
 

@@ -42,6 +42,9 @@
  *   - MaxPooling *, UpSampling *: bit-exact against the reference's classes
  *     (oracle/_ref), vectors written from them (tests/golden/pooling.npz), the
  *     known answers of tests/gtest/MaxPoolingTest.cpp and UpSamplingTest.cpp, numpy.
+ *   - Shuffle *: bit-exact against the reference's class (oracle/_ref), the known
+ *     answer of tests/gtest/ShuffleTest.cpp, numpy's transpose of the rows seen as
+ *     a [unit][group] matrix, and backward(forward(x)) == x.
  *
  * Array conventions (the reference's FrameBuffer layout, include/bb/FrameBuffer.h:28-46,
  * 927-939): node-major, frame-minor; element (node n, frame f) of an fp32
@@ -1662,6 +1665,31 @@ void oracle_fp32_UpSampling_Backward(float const *dy, float *dx, int input_w_siz
                     dx[in_node * frame_stride + f] = sum;
                 }
             }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------------------------------------------
+ *  Shuffle (include/bb/Shuffle.h:166-185, :225-243): a permutation of whole rows, whatever their element type.  With
+ *  x_unit_size = node_size / y_unit_size, output row i * y_unit_size + j is input row j * x_unit_size + i; backward undoes it.
+ *  Rows are frame_stride 32-bit words and are copied whole, as the reference's memcpy of one stride does.
+ * ---------------------------------------------------------------------------------------------------------------------------------- */
+void oracle_Shuffle_Forward(int const *x, int *y, int y_unit_size, int node_size, int frame_stride)
+{
+    int const x_unit_size = node_size / y_unit_size;
+    for (int i = 0; i < x_unit_size; ++i) {
+        for (int j = 0; j < y_unit_size; ++j) {
+            memcpy(y + (size_t)(i * y_unit_size + j) * frame_stride, x + (size_t)(j * x_unit_size + i) * frame_stride, (size_t)frame_stride * sizeof(int));
+        }
+    }
+}
+
+void oracle_Shuffle_Backward(int const *dy, int *dx, int y_unit_size, int node_size, int frame_stride)
+{
+    int const x_unit_size = node_size / y_unit_size;
+    for (int i = 0; i < y_unit_size; ++i) {
+        for (int j = 0; j < x_unit_size; ++j) {
+            memcpy(dx + (size_t)(i * x_unit_size + j) * frame_stride, dy + (size_t)(j * y_unit_size + i) * frame_stride, (size_t)frame_stride * sizeof(int));
         }
     }
 }

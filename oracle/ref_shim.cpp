@@ -45,6 +45,7 @@
 #include "bb/DifferentiableLutDiscreteN.h"
 #include "bb/MaxPooling.h"
 #include "bb/UpSampling.h"
+#include "bb/Shuffle.h"
 
 namespace {
 
@@ -1090,4 +1091,33 @@ extern "C" long bbref_UpSampling(int bit, int c, int h, int w, int fh, int fw, i
 {
     return bit ? run_up_sampling<bb::Bit>(c, h, w, fh, fw, fill, F, x, y, dy, dx, name, object_out, cap)
                : run_up_sampling<float>(c, h, w, fh, fw, fill, F, x, y, dy, dx, name, object_out, cap);
+}
+
+// Shuffle (host path): x [node_size][F] fp32 or bits -> y; dy of the same type -> dx.  output_node_size > 0 asks for that output
+// shape, 0 keeps the input shape.
+extern "C" long bbref_Shuffle(int bit, int shuffle_unit, int node_size, int F, void const *x, void *y, void const *dy, void *dx,
+                              char const *name, unsigned char *object_out, long cap)
+{
+    auto m = bb::Shuffle::Create((index_t)shuffle_unit);
+    m->SendCommand("host_only true");
+    if (name && *name) { m->SetName(name); }
+    int const xtype = bit ? BB_TYPE_BIT : BB_TYPE_FP32;
+    index_t const N = (index_t)node_size;
+    bb::FrameBuffer xb((index_t)F, bb::indices_t({N}), xtype, true);
+    auto out_shape = m->SetInputShape(xb.GetShape());
+    if (bb::CalcShapeSize(out_shape) != N) { return -2; }
+    if (bit) { put_bit(xb, (std::int32_t const *)x, N, (F + 31) / 32); }
+    else     { put_fp32(xb, (float const *)x, N, F); }
+    bb::FrameBuffer yb = m->Forward(xb, true);
+    if (bit) { get_bit(yb, (std::int32_t *)y, N, (F + 31) / 32); }
+    else     { get_fp32(yb, (float *)y, N, F); }
+    if (dy) {
+        bb::FrameBuffer dyb((index_t)F, out_shape, xtype, true);
+        if (bit) { put_bit(dyb, (std::int32_t const *)dy, N, (F + 31) / 32); }
+        else     { put_fp32(dyb, (float const *)dy, N, F); }
+        bb::FrameBuffer dxb = m->Backward(dyb);
+        if (bit) { get_bit(dxb, (std::int32_t *)dx, N, (F + 31) / 32); }
+        else     { get_fp32(dxb, (float *)dx, N, F); }
+    }
+    return object_out ? emit(*m, object_out, cap) : 0;
 }

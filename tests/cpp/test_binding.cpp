@@ -122,6 +122,10 @@ SAME(&bbcu_fp32_Im2Col_Backward, int (*)(float const *, float *, int, int, int, 
 SAME(&bbcu_fp32_Col2Im_Forward, int (*)(float const *, float *, int, int, int, int, int, int, S));
 SAME(&bbcu_bit_Col2Im_Forward, int (*)(int const *, int *, int, int, int, int, int, int, S));
 SAME(&bbcu_fp32_Col2Im_Backward, int (*)(float const *, float *, int, int, int, int, int, int, S));
+SAME(&bbcu_Shuffle_Forward<int>, int (*)(int const *, int *, unsigned int, unsigned int, unsigned int, unsigned int, S));
+SAME(&bbcu_Shuffle_Forward<float>, int (*)(float const *, float *, unsigned int, unsigned int, unsigned int, unsigned int, S));
+SAME(&bbcu_Shuffle_Backward<int>, int (*)(int const *, int *, unsigned int, unsigned int, unsigned int, unsigned int, S));
+SAME(&bbcu_Shuffle_Backward<float>, int (*)(float const *, float *, unsigned int, unsigned int, unsigned int, unsigned int, S));
 SAME(&bbcu_LossSoftmaxCrossEntropy<float>, int (*)(float const *, float const *, float *, double *, float, int, int, int, int, S));
 SAME(&bbcu_MetricsCategoricalAccuracy<float>, int (*)(float const *, float const *, int *, int *, int, int, int, int, S));
 SAME(&bbcu_fp32_OptimizerAdam, int (*)(int, int const *, float *const *, float *const *, float *const *, float *const *, float, float, float, S));
@@ -186,7 +190,7 @@ static int run_on_gpu(void)
 
 int main(int argc, char **argv)
 {
-    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11 + 10 + 7;
+    int const checks = 11 + 11 + 6 + 4 + 5 * LutSignatures<6>::kChecks + 4 + 4 + 1 + 11 + 10 + 7 + 4;
     if (argc > 1 && !std::strcmp(argv[1], "--gpu")) {
         if (!bbcu_IsDeviceAvailable()) { std::printf("no device available\n"); return 2; }
         int const bad = run_on_gpu();

@@ -14,6 +14,7 @@
 #include "bb/DifferentiableLutDiscreteN.h"
 #include "bb/MaxPooling.h"
 #include "bb/UpSampling.h"
+#include "bb/Shuffle.h"
 #include "../../binarybrain_amd/csrc/tile_divisor.hpp"
 
 extern "C" int oracle_ReverseTable(int n, std::int32_t const *idx, int input_node_size, int output_node_size, std::int32_t *rev, int rev_cap);
@@ -210,6 +211,17 @@ int main(void)
         CHECK(pool->SetInputShape({4, 5, 7}) == bb::indices_t({4, 3, 3}) && pool->GetFilterHeight() == 2 && pool->GetFilterWidth() == 3);
         auto up = bb::UpSampling<>::Create(2, 3, false);
         CHECK(up->SetInputShape({4, 5, 7}) == bb::indices_t({4, 10, 21}) && up->GetOutputNodeSize() == 840);
+        auto shuffle = bb::Shuffle::Create(3, bb::indices_t({2, 6}));
+        CHECK(shuffle->SetInputShape({12}) == bb::indices_t({2, 6}) && shuffle->SetInputShape({6}) == bb::indices_t({6}));
+        {
+            std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+            shuffle->DumpObject(ss);
+            auto back = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+            CHECK((bool)back && back->GetObjectName() == "Shuffle" && back->GetOutputShape() == bb::indices_t({6}));
+        }
+        threw = false;
+        try { bb::Shuffle::Create(4)->SetInputShape({6}); } catch (bb::Exception const &) { threw = true; }
+        CHECK(threw);                                                   // 6 nodes do not split into units of 4
         auto tanh = bb::HardTanh<>::Create(0.0f, 1.0f);
         CHECK(tanh->ForwardNode(0, {-0.5, 0.25, 2.0}) == std::vector<double>({0.0, 0.25, 1.0}));
         tanh->SendCommand("binary true");

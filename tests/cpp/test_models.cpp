@@ -34,6 +34,7 @@
 #include "bb/DifferentiableLutDiscreteN.h"
 #include "bb/MaxPooling.h"
 #include "bb/UpSampling.h"
+#include "bb/Shuffle.h"
 #include "bb/ObjectLoader.h"
 
 extern "C" {
@@ -906,6 +907,36 @@ static void test_pooling(void)
     }
 }
 
+// Shuffle through the class: fp32 and packed frames against the closed form (output node i * unit + j = input node
+// j * (nodes / unit) + i), backward(forward(x)) == x, and a trip through a stream.
+static void test_shuffle(void)
+{
+    int const N = 84, U = 7, X = N / U, F = 70;
+    std::mt19937_64 mt(47);
+    std::uniform_real_distribution<float> uni(-1.0f, 1.0f);
+    bb::FrameBuffer x_buf(F, {N}, BB_TYPE_FP32), b_buf(F, {N}, BB_TYPE_BIT);
+    for (int n = 0; n < N; ++n) for (int f = 0; f < F; ++f) { x_buf.SetFP32(f, n, uni(mt)); b_buf.SetBit(f, n, mt() % 2 == 0); }
+    auto shuffle = bb::Shuffle::Create(U, bb::indices_t({4, 21}));
+    CHECK(shuffle->SetInputShape({N}) == bb::indices_t({4, 21}), "Shuffle output shape");
+    bb::FrameBuffer y_buf = shuffle->Forward(x_buf), yb_buf = shuffle->Forward(b_buf);
+    CHECK(y_buf.GetType() == BB_TYPE_FP32 && yb_buf.GetType() == BB_TYPE_BIT && y_buf.GetShape() == bb::indices_t({4, 21}), "Shuffle output type");
+    size_t bad = 0;
+    for (int i = 0; i < X; ++i) for (int j = 0; j < U; ++j) for (int f = 0; f < F; ++f) {
+        bad += (y_buf.GetFP32(f, i * U + j) != x_buf.GetFP32(f, j * X + i));
+        bad += (yb_buf.GetBit(f, i * U + j) != b_buf.GetBit(f, j * X + i));
+    }
+    CHECK(bad == 0, "Shuffle forward: %zu values differ", bad);
+    bb::FrameBuffer dx_buf = shuffle->Backward(y_buf), dxb_buf = shuffle->Backward(yb_buf);
+    bad = 0;
+    for (int n = 0; n < N; ++n) for (int f = 0; f < F; ++f) { bad += (dx_buf.GetFP32(f, n) != x_buf.GetFP32(f, n)) + (dxb_buf.GetBit(f, n) != b_buf.GetBit(f, n)); }
+    CHECK(bad == 0 && dx_buf.GetShape() == bb::indices_t({N}), "Shuffle backward does not undo forward: %zu values differ", bad);
+    std::stringstream ss(std::ios::in | std::ios::out | std::ios::binary);
+    shuffle->DumpObject(ss);
+    auto again = std::dynamic_pointer_cast<bb::Model>(bb::Object_Load(ss));
+    CHECK((bool)again && again->GetObjectName() == "Shuffle" && again->GetOutputShape() == bb::indices_t({4, 21}), "Shuffle reload");
+    if (again) { bb::FrameBuffer y2 = again->Forward(x_buf, false); CHECK(same_bits(y2, y_buf), "reloaded Shuffle differs"); }
+}
+
 static void test_tail(void)
 {
     int const n = 7, O = 10, I = 70, F = 100;
@@ -1065,6 +1096,7 @@ int main(void)
         test_reduce_and_mean_squared_error();
         test_binary_modulation();
         test_pooling();
+        test_shuffle();
         test_discrete<6>(24, 16, 200, false);
         test_discrete<6>(24, 16, 200, true);
         test_discrete<4>(12, 30, 1024, false);

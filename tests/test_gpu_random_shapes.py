@@ -402,6 +402,27 @@ def test_random_shapes_of_the_converters_activations_and_pooling():
         run_plumbing_case(ops, seed)
 
 
+def run_shuffle_case(ops, seed):
+    """Shuffle at random node counts, units and row pitches, fp32 rows and packed rows: whole rows bit for bit against the oracle"""
+    rng = np.random.default_rng(seed)
+    unit = int(rng.choice([1, 2, 3, 7, 32, int(rng.integers(1, 100))])); group = int(rng.choice([1, 2, 5, 36, int(rng.integers(1, 200))]))
+    nodes = unit * group
+    F = int(rng.integers(1, 600))
+    stride = int(rng.choice([synth.frame_stride_fp32(F), F, F + int(rng.integers(1, 9))]))
+    print("seed %d: shuffle nodes=%d unit=%d F=%d stride=%d" % (seed, nodes, unit, F, stride), flush=True)
+    x = rng.integers(-2**31, 2**31, (nodes, stride)).astype(np.int32)
+    assert np.array_equal(host(ops.shuffle_forward(dev(x), unit, F)), oracle.shuffle_forward(x, unit))
+    assert np.array_equal(host(ops.shuffle_backward(dev(x), unit, F)), oracle.shuffle_backward(x, unit))
+    xf = x.view(np.float32)                                              # the same words as fp32 rows (NaN patterns included)
+    assert np.array_equal(host(ops.shuffle_forward(dev(xf), unit, F)).view(np.int32), oracle.shuffle_forward(x, unit))
+
+
+def test_random_shapes_of_shuffle():
+    from binarybrain_amd import ops
+    for seed in range(14000, 14100):
+        run_shuffle_case(ops, seed)
+
+
 def test_extended_random_run():
     """The same four generators over further seeds, for a longer run on the device: set BBHIP_EXTENDED_CASES=N (N cases of each
     generator, at most 200 000; seeds continue after the ones above).  Stops at the first failing case, whose seed the case

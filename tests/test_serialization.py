@@ -449,3 +449,12 @@ def test_reference_up_sampling_objects(tmp_path, k):
     name = POOLING[q + "name"].tobytes().decode()
     for key, type_name in (("object", "UpSampling_fp32_fp32"), ("object_bit", "UpSampling_bit_fp32")):
         _reload_and_compare(tmp_path, POOLING[q + key].tobytes(), type_name, name, "UpSampling", c * h * w, c * h * fh * w * fw)
+
+
+#  Shuffle (include/bb/Shuffle.h:270-301): version, Model part, host_only, the two shapes, the unit
+@pytest.mark.parametrize("k", range(int(POOLING["shuffle_count"][0])))
+def test_reference_shuffle_objects(tmp_path, k):
+    q = "s%d_" % k
+    nodes, unit, F = [int(v) for v in POOLING[q + "geom"]]
+    name = POOLING[q + "name"].tobytes().decode()
+    _reload_and_compare(tmp_path, POOLING[q + "object"].tobytes(), "Shuffle", name, "Shuffle", nodes, nodes)
