@@ -424,7 +424,7 @@ def test_random_shapes_of_shuffle():
 
 
 def test_extended_random_run():
-    """The same four generators over further seeds, for a longer run on the device: set BBHIP_EXTENDED_CASES=N (N cases of each
+    """The same five generators over further seeds, for a longer run on the device: set BBHIP_EXTENDED_CASES=N (N cases of each
     generator, at most 200 000; seeds continue after the ones above).  Stops at the first failing case, whose seed the case
     prints.  Without the variable the test is skipped, so the default suite stays short:
         BBHIP_EXTENDED_CASES=10000 python -u -m pytest tests/test_gpu_random_shapes.py -k extended -x -s"""
@@ -441,6 +441,7 @@ def test_extended_random_run():
             run_exact_case(ops, 400000 + k)
             run_tail_case(ops, torch, 700000 + k)
             run_plumbing_case(ops, 900000 + k)
+            run_shuffle_case(ops, 1200000 + k)
             if (k + 1) % 500 == 0:
                 print("extended run: %d of %d" % (k + 1, count), flush=True)
     finally:
