@@ -368,16 +368,18 @@ def bench_differentiablelut6(args, lib):
     if bits:
         xb = torch.from_numpy(synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))).cuda()
 
+    tables = ops.prepared_tables_buffer(6, idx.shape[0])     # the model class keeps the tables derived from W from forward to backward
+
     def step():
         # (the table is clamped to [0, 1] in place by the forward entry's table launch, as the model class does before a forward pass)
         if bits:
-            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=(0.0, 1.0))
-            ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev)
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=(0.0, 1.0), tables=tables)
+            ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev, tables=tables)
         else:
             # the model class keeps the packed copy of its binarized input from the forward to the backward call
             packed = ops.packed_input_buffer(I, F)
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=(0.0, 1.0), packed=packed)
-            ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev, packed=packed)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=(0.0, 1.0), packed=packed, tables=tables)
+            ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev, packed=packed, tables=tables)
 
     t_ramp = time.perf_counter()
     while time.perf_counter() - t_ramp < args.ramp_seconds:
@@ -441,7 +443,8 @@ def bench_conv_block(args, lib):
             # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
             # ... and keeps the packed copy of its binarized input for the backward call
             packed = ops.packed_input_buffer(a.shape[0], FW_FRAMES)
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed,
+                                                                    tables=l.setdefault("tables", ops.prepared_tables_buffer(6, l["idx"].shape[0])))
             acts.append((a, mean, rstd, packed)); a = y
         maps = ops.col2im_forward(a, CO, OH, OW, F)
         pooled = ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F)
@@ -449,7 +452,7 @@ def bench_conv_block(args, lib):
         dy = ops.col2im_backward(dmaps, CO, OH, OW, F)
         for l, (a_in, mean, rstd, packed) in zip(reversed(layers), reversed(acts)):
             l["dW"].zero_()
-            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"], packed=packed)
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"], packed=packed, tables=l["tables"])
         return ops.im2col_backward(dy, C, H, W_, F, FH, FW), pooled
 
     t_ramp = time.perf_counter()
@@ -537,7 +540,8 @@ def bench_mnist_step(args, lib):
             # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
             # ... and keeps the packed copy of its binarized input for the backward call
             packed = ops.packed_input_buffer(a.shape[0], F)
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed,
+                                                                    tables=l.setdefault("tables", ops.prepared_tables_buffer(6, l["idx"].shape[0])))
             acts.append((a, mean, rstd, packed)); a = y
         out = ops.average_lut_forward(a, idx_avg, F, False, False)
         dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
@@ -545,7 +549,7 @@ def bench_mnist_step(args, lib):
         dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
         for l, (a_in, mean, rstd, packed) in zip(reversed(layers), reversed(acts)):
             # dW accumulates; it is zero here because the optimizer's Update() zeroed it after the previous step (Optimizer.h:31-35)
-            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"], packed=packed)
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"], packed=packed, tables=l["tables"])
         keep["loss_buf"], keep["acc"] = loss_buf, acc
 
     def timed(fn):

@@ -42,6 +42,8 @@ _SIGNATURES = {
     "bbhip_HintInputNodeSize": (None, [_i]),
     "bbhip_PackedRowWords": (C.c_int, [_i]),
     "bbhip_HintPackedInput": (None, [_vp, _i, _i, _i]),
+    "bbhip_HintPreparedTables": (None, [_vp, C.c_size_t, _i]),
+    "bbhip_PreparedTablesBytes": (C.c_size_t, [_i, _i]),
     "bbhip_GetDxMode": (C.c_int, []),
     "bbhip_fp32_Vector_set": (C.c_int, [_vp, _f, _i, _vp]),
     "bbhip_fp32_Vector_clamp": (C.c_int, [_vp, _vp, _f, _f, _i, _vp]),

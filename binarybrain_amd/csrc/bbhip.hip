@@ -70,7 +70,17 @@ thread_local int g_input_node_hint = 0;      // bbhip_HintInputNodeSize: rows of
 struct PackedInputHint { uint32_t *bits; int rows, row_words, holds_input; };
 thread_local PackedInputHint g_packed_hint = {nullptr, 0, 0, 0};
 // hints are for the next LUT call only: every entry spends them
-static inline void clear_hints(void) { g_input_node_hint = 0; g_packed_hint = PackedInputHint{nullptr, 0, 0, 0}; }
+// bbhip_HintPreparedTables: a caller-owned place for the tables that a LUT call derives from W (centred coefficients, corner values)
+struct PreparedTablesHint { float *buf; size_t bytes; int holds_tables; };
+thread_local PreparedTablesHint g_tables_hint = {nullptr, 0, 0};
+static inline void clear_hints(void)
+{
+    g_input_node_hint = 0; g_packed_hint = PackedInputHint{nullptr, 0, 0, 0}; g_tables_hint = PreparedTablesHint{nullptr, 0, 0};
+}
+static inline bool tables_fit(PreparedTablesHint const &t, size_t bytes)
+{
+    return t.buf != nullptr && t.bytes >= bytes && (reinterpret_cast<uintptr_t>(t.buf) & 255u) == 0;
+}
 
 // ------------------------------------------------------------------------------------------------
 //  optional kernel timer: HIP events around the dominant kernel of each entry point, on the launch stream
@@ -418,7 +428,7 @@ int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_s
 
 template <int N>
 int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch const *fixed = nullptr,
-                PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0})
+                PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0}, PreparedTablesHint tables = PreparedTablesHint{nullptr, 0, 0})
 {
     constexpr int NN = 1 << N;
     // input_rows: what the caller said about the input's row count (bbhip_HintInputNodeSize), 0 = nothing.
@@ -450,6 +460,12 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
+    // the tables go to the caller's buffer where one was offered and fits: the backward call of the same step can take them from there
+    bool const tables_to_caller = tables_fit(tables, c_bytes + v_bytes);
+    if (tables_to_caller) {
+        C = tables.buf;
+        V = corner ? reinterpret_cast<float *>(reinterpret_cast<char *>(tables.buf) + c_bytes) : nullptr;
+    }
     if (pack) {
         uint32_t *bits = to_caller ? packed.bits : reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes);
         if (launch_pack_and_prep<N>(reinterpret_cast<float const *>(call.x), call.x_stride, bits, c.x_stride, input_rows, c.frame_size,
@@ -458,7 +474,7 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     }
     // plain output of a call with one unit per node on the polynomial kernel: the wavefronts prepare their node's table
     // themselves (FwdArgs::W_inline) and the table launch falls away
-    bool const inline_table = (c.bn == 0) && !corner && chunk_count == 1 && LutMatrixQ<N>::kUsable && c.clamp_W == nullptr;
+    bool const inline_table = (c.bn == 0) && !corner && chunk_count == 1 && LutMatrixQ<N>::kUsable && c.clamp_W == nullptr && !tables_to_caller;
     if (!pack && !inline_table) {
         launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias, c.clamp_W, c.clamp_lo, c.clamp_hi);
         BBHIP_LAUNCH_CHECK();
@@ -517,10 +533,11 @@ int forward_entry(ForwardCall const &c, void *stream, Scratch const *fixed = nul
     // the hints are spent by this call, whatever becomes of it; a buffer for the packed copy also says how many rows the input has
     PackedInputHint const packed = fixed ? PackedInputHint{nullptr, 0, 0, 0} : g_packed_hint;
     int const input_rows = fixed ? 0 : (packed.bits ? packed.rows : g_input_node_hint);
+    PreparedTablesHint const tables = fixed ? PreparedTablesHint{nullptr, 0, 0} : g_tables_hint;
     clear_hints();
     if (check_forward(c)) { return 1; }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed, packed));
+    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed, packed, tables));
     return 0;
 }
 
@@ -563,7 +580,8 @@ int check_backward(BackwardCall const &c, int dxmode)
 }
 
 template <int N>
-int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0})
+int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0},
+                 PreparedTablesHint tables = PreparedTablesHint{nullptr, 0, 0})
 {
     constexpr int NN = 1 << N;
     int dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
@@ -636,8 +654,14 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
     int   *term = reinterpret_cast<int *>(base + c_bytes + part_bytes + stat_bytes);
     float *dyh  = reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes);
 
-    // centred coefficients: needed where the LUT output is recomputed (batch-norm) or per-connection gradients are formed
-    bool const prep = c.bn || dxmode != kDxNone;
+    // centred coefficients: needed where the LUT output is recomputed (batch-norm) or per-connection gradients are formed;
+    // a caller that kept the tables of this step's forward call (same W, same kind of input) hands them back: nothing to prepare
+    bool const have_tables = tables.holds_tables && tables_fit(tables, c_bytes + v_bytes);
+    if (have_tables) {
+        C = tables.buf;
+        V = corner ? reinterpret_cast<float *>(reinterpret_cast<char *>(tables.buf) + c_bytes) : nullptr;
+    }
+    bool const prep = (c.bn || dxmode != kDxNone) && !have_tables;
     if (have_bits) {
         c.x = packed.bits;
         if (prep) {
@@ -788,9 +812,10 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
 int backward_entry(BackwardCall const &c, void *stream)
 {
     PackedInputHint const packed = g_packed_hint;
+    PreparedTablesHint const tables = g_tables_hint;
     clear_hints();                                  // hints are for the next LUT call only
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st, packed));
+    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st, packed, tables));
     return 0;
 }
 
@@ -1088,6 +1113,17 @@ int  bbhip_GetAverageLutMean(void) { return g_average_lut_mean ? 1 : 0; }
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
 void bbhip_HintInputNodeSize(int input_node_size) { g_input_node_hint = input_node_size > 0 ? input_node_size : 0; }
 int  bbhip_PackedRowWords(int frame_size) { return frame_size > 0 ? packed_row_words(frame_size) : 0; }
+void bbhip_HintPreparedTables(float *dev_tables, size_t bytes, int holds_tables)
+{
+    g_tables_hint = (dev_tables != nullptr && bytes > 0) ? PreparedTablesHint{dev_tables, bytes, holds_tables != 0} : PreparedTablesHint{nullptr, 0, 0};
+}
+
+size_t bbhip_PreparedTablesBytes(int n, int node_size)
+{
+    if (n < 2 || n > 6 || node_size <= 0) { return 0; }
+    return 2 * align256((size_t)node_size * ((size_t)1 << n) * sizeof(float));
+}
+
 void bbhip_HintPackedInput(int *dev_bits, int rows, int row_words, int holds_input)
 {
     g_packed_hint = (dev_bits != nullptr && rows > 0 && row_words > 0)

@@ -120,6 +120,7 @@ class Memory {
     bool        m_host_valid = false;   // host copy holds the current contents
     bool        m_dev_valid = false;    // device copy holds the current contents
     bool        m_host_pinned = false;
+    std::uint64_t m_writes = 0;         // writable locks handed out (WriteCount)
 
     void alloc_host(void)
     {
@@ -158,11 +159,15 @@ public:
     bool IsHostOnly(void) const { return m_host_only; }
     bool IsDeviceAvailable(void) const { return !m_host_only && Manager::IsDeviceAvailable(); }
 
-    void Resize(std::size_t size) { release(); m_size = size; }
+    void Resize(std::size_t size) { release(); m_size = size; ++m_writes; }
+
+    // how many writable locks were handed out so far: unchanged between two moments = nothing could write in between
+    std::uint64_t WriteCount(void) const { return m_writes; }
 
     // host side, read-write (discard = old contents not needed)
     void *Lock(bool discard = false)
     {
+        ++m_writes;
         alloc_host();
         if (!discard && !m_host_valid && m_dev_valid) { CheckDevice(bbhip_Memcpy(m_host, m_dev, m_size, 2), "bbhip_Memcpy(D2H)"); }
         m_host_valid = true;
@@ -179,6 +184,7 @@ public:
     // device side
     void *LockDevice(bool discard = false)
     {
+        ++m_writes;
         alloc_dev();
         if (!discard && !m_dev_valid && m_host_valid) { CheckDevice(bbhip_Memcpy(m_dev, m_host, m_size, 1), "bbhip_Memcpy(H2D)"); }
         m_dev_valid = true;

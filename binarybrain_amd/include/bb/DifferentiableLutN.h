@@ -240,11 +240,41 @@ private:
         else { bbhip_HintInputNodeSize((int)x_buf.GetNodeSize()); }         // the forward signatures do not carry the input's row count
     }
 
+    // The tables that the entry points derive from W before their kernels run (centred coefficients, corner values) are the same
+    // for every call between two changes of W.  A batch-norm training forward call writes them into a buffer of the layer's, and the
+    // backward calls that follow take them from there instead of preparing them again (bbhip_HintPreparedTables) — as long as nobody
+    // took a writable lock on W since and the layer's modes are those of the call that filled the buffer.
+    std::shared_ptr<Memory>                  m_tables;
+    std::pair<void const *, std::uint64_t>   m_tables_stamp{nullptr, 0};
+    int                                      m_tables_modes = -1;
+
+    int TableModes(void) const { return (m_lut_binarize ? 1 : 0) | (m_binary_mode ? 2 : 0); }
+
+    // before a training forward call, after its locks on W were taken
+    void OfferTables(void)
+    {
+        std::size_t const bytes = bbhip_PreparedTablesBytes(N, (int)this->GetOutputNodeSize());
+        if (bytes == 0) { return; }
+        if (!m_tables || m_tables->GetSize() != bytes) { m_tables = Memory::Create(bytes); }
+        bbhip_HintPreparedTables((float *)m_tables->LockDevice(true), bytes, 0);
+        m_tables_stamp = m_W->WriteStamp();
+        m_tables_modes = TableModes();
+    }
+
+    // before a backward call
+    void ReturnTables(void)
+    {
+        if (m_tables && m_tables_modes == TableModes() && m_tables_stamp == m_W->WriteStamp()) {
+            bbhip_HintPreparedTables((float *)m_tables->LockDevice(), m_tables->GetSize(), 1);
+        }
+    }
+
 public:
     void Clear(void) override
     {
         Model::Clear();
         while (!m_packed_bufs.empty()) { m_packed_bufs.pop(); }
+        m_tables_modes = -1;
     }
 
     FrameBuffer Forward(FrameBuffer x_buf, bool train = true) override
@@ -279,6 +309,7 @@ public:
             auto rstd_ptr = m_rstd.LockDeviceMemory(true);
             auto rm_ptr   = m_running_mean.LockDeviceMemory();
             auto rv_ptr   = m_running_var.LockDeviceMemory();
+            OfferTables();
             if (kBitType) {
                 CheckDevice(bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float *)W_mut.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
@@ -302,6 +333,7 @@ public:
             auto rstd_ptr = m_rstd.LockDeviceMemory(true);
             auto rm_ptr   = m_running_mean.LockDeviceMemory();
             auto rv_ptr   = m_running_var.LockDeviceMemory();
+            OfferTables();
             if (kBitType) {
                 CheckDevice(bbhip_bit_fp32_DifferentiableLutN_ForwardTraining(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
@@ -402,6 +434,7 @@ public:
             Tensor_<RealType> dmean(m_output_shape), dvar(m_output_shape);
             auto dmean_ptr = dmean.LockDeviceMemory(true);
             auto dvar_ptr  = dvar.LockDeviceMemory(true);
+            ReturnTables();
             if (kBitType) {
                 CheckDevice(bbhip_bit_fp32_DifferentiableLutN_Backward(N, (int const *)x_ptr.GetAddr(), (float const *)dy_ptr.GetAddr(), (float *)dx_ptr.GetAddr(),
                                 tmp_addr, (int const *)idx_ptr.GetAddr(), (int const *)rev_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)dW_ptr.GetAddr(),

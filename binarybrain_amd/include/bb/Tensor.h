@@ -130,6 +130,8 @@ public:
         BB_ASSERT(DataType<T>::type == m_type);
         return TensorView<T, void const *>(m_mem, m_mem->LockConst(), m_shape);
     }
+    // identifies the contents: the same stamp at two moments = no writable lock was taken and no new block was put in between
+    std::pair<void const *, std::uint64_t> WriteStamp(void) const { return {m_mem.get(), m_mem ? m_mem->WriteCount() : 0}; }
     DevicePtr      LockDeviceMemory(bool discard = false) { return DevicePtr(m_mem, m_mem->LockDevice(discard)); }
     DeviceConstPtr LockDeviceMemoryConst(void) const      { return DeviceConstPtr(m_mem, m_mem->LockDeviceConst()); }
 

@@ -524,6 +524,19 @@ def packed_input_buffer(rows, frame_size, device="cuda"):
     return torch.empty((rows, lib().bbhip_PackedRowWords(frame_size)), dtype=torch.int32, device=device)
 
 
+def prepared_tables_buffer(n, node_size, device="cuda"):
+    """A buffer for bbhip_HintPreparedTables: the tables that a LUT call derives from W, kept from a step's forward call for its
+    backward call (`tables=` of the DifferentiableLut wrappers)."""
+    return torch.empty(lib().bbhip_PreparedTablesBytes(n, node_size) // 4, dtype=torch.float32, device=device)
+
+
+def _hint_tables(tables, holds_tables):
+    if tables is not None:
+        _dev(tables)
+        assert tables.dtype == torch.float32
+        lib().bbhip_HintPreparedTables(ptr(tables), tables.numel() * 4, int(holds_tables))
+
+
 def _hint_input(x, packed, holds_input):
     """what the wrapper knows about the next LUT call's input: its row count, and where its packed copy goes to / comes from"""
     if packed is not None:
@@ -617,8 +630,9 @@ def bit_stochastic_lut_backward(n, xbits, dy, idx, W, dW, frame_size, rev=None, 
 
 
 def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None, packed=None):
+                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None, packed=None, tables=None):
     """fp32 frames. running_mean / running_var are updated in place. returns (y, mean, rstd).
+    tables: a `prepared_tables_buffer` that receives the tables derived from W, for the backward call of the same step.
     packed: a `packed_input_buffer` that receives the packed copy of the binarized input (binary mode), for the backward call.
     clamp_w = (lo, hi): W is clamped in place first, by the launch that prepares the tables (the model class's clamp before the
     first forward pass after a backward pass, include/bb/DifferentiableLutN.h:605-608)."""
@@ -628,6 +642,7 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
     mean = torch.empty(O, dtype=torch.float32, device=x.device)
     rstd = torch.empty(O, dtype=torch.float32, device=x.device)
     _hint_input(x, packed, False)
+    _hint_tables(tables, False)
     if clamp_w is not None:
         check(lib().bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                                         ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
@@ -642,12 +657,13 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
 
 
 def bit_differentiable_lut_forward_training(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                            momentum=0.9, bias=0.25, lut_binarize=False, clamp_w=None):
+                                            momentum=0.9, bias=0.25, lut_binarize=False, clamp_w=None, tables=None):
     _dev(xbits, idx, W, running_mean, running_var)
     O = idx.shape[0]
     y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
     mean = torch.empty(O, dtype=torch.float32, device=xbits.device)
     rstd = torch.empty(O, dtype=torch.float32, device=xbits.device)
+    _hint_tables(tables, False)
     if clamp_w is not None:
         check(lib().bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW(n, ptr(xbits), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                                             ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
@@ -694,8 +710,9 @@ def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_bin
 
 
 def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, rev=None, gamma=0.3, beta=0.5, bias=0.25,
-                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024, packed=None):
-    """packed: the buffer that the forward call on the same x filled (`packed_input_buffer`): the call reads it instead of packing x."""
+                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024, packed=None, tables=None):
+    """tables: the buffer that this step's forward call with the same W filled (`prepared_tables_buffer`): no preparation launch.
+    packed: the buffer that the forward call on the same x filled (`packed_input_buffer`): the call reads it instead of packing x."""
     _dev(x, dy, idx, W, dW, mean, rstd, rev)
     I = x.shape[0]; O = idx.shape[0]
     dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=x.device)
@@ -705,6 +722,7 @@ def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, re
     if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
     _hint_input(x, packed, True)
+    _hint_tables(tables, True)
     check(lib().bbhip_fp32_DifferentiableLutN_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                        ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
                                                        0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,
@@ -713,7 +731,7 @@ def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, re
 
 
 def bit_differentiable_lut_backward(n, xbits, dy, idx, W, dW, frame_size, mean, rstd, rev=None, gamma=0.3, beta=0.5,
-                                    bias=0.25, lut_binarize=False, max_tmp_bytes=256 * 1024 * 1024):
+                                    bias=0.25, lut_binarize=False, max_tmp_bytes=256 * 1024 * 1024, tables=None):
     _dev(xbits, dy, idx, W, dW, mean, rstd, rev)
     I = xbits.shape[0]; O = idx.shape[0]
     dx = torch.empty((I, dy.shape[1]), dtype=torch.float32, device=dy.device)
@@ -722,6 +740,7 @@ def bit_differentiable_lut_backward(n, xbits, dy, idx, W, dW, frame_size, mean, 
     dx_tmp, tf, ts = (None, 0, 0)
     if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, dy.device, max_tmp_bytes)
+    _hint_tables(tables, True)
     check(lib().bbhip_bit_fp32_DifferentiableLutN_Backward(n, ptr(xbits), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W),
                                                            ptr(dW), ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
                                                            0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1],

@@ -120,6 +120,16 @@ void bbhip_HintInputNodeSize(int input_node_size);
 int  bbhip_PackedRowWords(int frame_size);
 void bbhip_HintPackedInput(int *dev_bits, int rows, int row_words, int holds_input);
 
+/* No counterpart in the reference.  A caller-owned device buffer (256-byte aligned, bbhip_PreparedTablesBytes(n, node_size) bytes) for the
+ * tables that a LUT call derives from W before its kernels run (centred coefficients, corner values).  Given right before a forward call
+ * (holds_tables = 0), the call writes them there instead of into the library's scratch memory; given right before the backward call of
+ * the same step with holds_tables = 1, that call takes them from there and skips its own preparation launch.  holds_tables = 1 is the
+ * caller's promise that W, the LUT width, the node count, lut_binarize and the kind of input (two-valued or not) are those of the call
+ * that filled the buffer; a buffer that is too small or not aligned is ignored and not written.  Thread-local, spent by the next entry
+ * point called on the thread, like the other hints; results are the same bits with and without it. */
+void   bbhip_HintPreparedTables(float *dev_tables, size_t bytes, int holds_tables);
+size_t bbhip_PreparedTablesBytes(int n, int node_size);
+
 /* ---- kernel timer (instrumentation; no counterpart in the reference) ----
  * While enabled, every call brackets its dominant kernel (which: 0 = LUT forward kernel, 1 = LUT backward kernel,
  * 2 = BinaryLut6 kernel, 3 = input-centric dx kernel, 4 = the kernels of any other entry: vector operations, Adam, Im2Col,

@@ -222,6 +222,18 @@ int main(void)
         threw = false;
         try { bb::Shuffle::Create(4)->SetInputShape({6}); } catch (bb::Exception const &) { threw = true; }
         CHECK(threw);                                                   // 6 nodes do not split into units of 4
+        {   // the stamp that says whether a tensor could have been written to since it was last looked at
+            bb::Tensor_<float> t(bb::indices_t({4}));
+            { auto w = t.Lock(true); w[0] = 1.0f; }
+            auto const s0 = t.WriteStamp();
+            { auto r = t.LockConst(); CHECK(r[0] == 1.0f); }
+            CHECK(t.WriteStamp() == s0);                                // reading does not move it
+            { auto w = t.Lock(); w[1] = 2.0f; }
+            CHECK(t.WriteStamp() != s0);                                // a writable lock does
+            auto const s1 = t.WriteStamp();
+            t.Resize(bb::indices_t({8}));
+            CHECK(t.WriteStamp() != s1);                                // and so does a new block
+        }
         auto tanh = bb::HardTanh<>::Create(0.0f, 1.0f);
         CHECK(tanh->ForwardNode(0, {-0.5, 0.25, 2.0}) == std::vector<double>({0.0, 0.25, 1.0}));
         tanh->SendCommand("binary true");
