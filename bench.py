@@ -543,7 +543,7 @@ def bench_mnist_step(args, lib):
             y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed,
                                                                     tables=l.setdefault("tables", ops.prepared_tables_buffer(6, l["idx"].shape[0])))
             acts.append((a, mean, rstd, packed)); a = y
-        out = ops.average_lut_forward(a, idx_avg, F, False, False)
+        out = ops.average_lut_forward(a, idx_avg, F, False, False, mean=False)
         dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
         acc, cat = ops.metrics_categorical_accuracy(out, t, CLASSES, 1, F)
         dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
@@ -847,34 +847,54 @@ def bench_forward_small(args, lib):
     return out
 
 
+def gather_probe_library():
+    """bench_gather_probe.so: the bench's own instrumentation kernel, built from bench_gather_probe.hip beside this file
+    (by __graft_entry__.build(); here only when it is missing)."""
+    import ctypes as C
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    so, src = os.path.join(here, "bench_gather_probe.so"), os.path.join(here, "bench_gather_probe.hip")
+    if not os.path.exists(so):
+        subprocess.check_call([os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+                               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", src, "-o", so], cwd=here)
+    probe = C.CDLL(so)
+    probe.bench_row_gather_probe.restype = C.c_int
+    probe.bench_row_gather_probe.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 7 + [C.POINTER(C.c_float), C.c_void_p]
+    return probe
+
+
 def bench_gather_ceiling(args, lib):
-    """What the GPU sustains on the dx kernel's access pattern alone (instrumentation): per (input row, 128-frame window) 36
-    pseudo-randomly chosen rows' 512-byte segments are read and discarded — 6 consumers x (5 rows + dy) as in the headline
-    shape.  Reported as a rate through L1; the dx kernel moves the same bytes and does its arithmetic on top."""
+    """What the GPU sustains on the dx kernel's access pattern alone (instrumentation, a kernel of the bench's own): per (input row,
+    128-frame window) 36 pseudo-randomly chosen rows' 512-byte segments are read and discarded — 6 consumers x (5 rows + dy) as in the
+    headline shape.  Reported as a rate through L1; the dx kernel moves the same bytes and does its arithmetic on top."""
+    import ctypes as C
     import torch
-    from binarybrain_amd import capi, synth
+    from binarybrain_amd import synth
     from binarybrain_amd.capi import ptr, stream_ptr
+    probe = gather_probe_library()
     I, F = 4096, 8192
     S = synth.frame_stride_fp32(F)
     x = torch.rand((I, S), device="cuda")
     sink = torch.zeros(1, device="cuda")
     loads = 36
+    steps, warmup = max(args.steps, 20), max(args.warmup, 20)
 
-    def step():
-        capi.check(lib.bbhip_Probe_RowGather(ptr(x), ptr(sink), I, F, S, loads, stream_ptr()))
+    def mean_ms(seg):
+        ms = C.c_float(0)
+        rc = probe.bench_row_gather_probe(ptr(x), ptr(sink), I, F, S, loads, seg, warmup, steps, C.byref(ms), stream_ptr())
+        if rc != 0:
+            raise RuntimeError("bench_row_gather_probe failed: %d" % rc)
+        return ms.value
 
-    kernel_ms = library_timed_ms(lib, step, max(args.steps, 20), max(args.warmup, 20))
+    kernel_ms = mean_ms(128)
     nbytes = I * (F // 128) * loads * 512
     # the same bytes as longer or shorter row segments: the rate grows with the bytes per visited row until the window of all rows
     # (4096 rows x segment) no longer fits the 4 MiB L2 of an XCD
     by_segment = {}
     for seg in (64, 128, 256, 512):
-        def seg_step(seg=seg):
-            capi.check(lib.bbhip_Probe_RowGatherSegments(ptr(x), ptr(sink), I, F, S, loads, seg, stream_ptr()))
-        ms = library_timed_ms(lib, seg_step, max(args.steps, 20), max(args.warmup, 20))
-        by_segment["%d B" % (seg * 4)] = round(I * (F // seg) * loads * seg * 4 / (ms * 1e-3) / 1e12, 2)
+        by_segment["%d B" % (seg * 4)] = round(I * (F // seg) * loads * seg * 4 / (mean_ms(seg) * 1e-3) / 1e12, 2)
     return {"metric": "TB/s of gathered 512-byte row segments through L1 (access pattern of the dx kernel, no arithmetic)",
-            "value": nbytes / (kernel_ms * 1e-3) / 1e12, "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 20),
+            "value": nbytes / (kernel_ms * 1e-3) / 1e12, "unit": "TB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
             "ms_per_step": kernel_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": "row gather probe, 4096 rows x 8192 frames, 36 row segments per (row, 128 frames)", "bytes_per_launch": nbytes,
                        "TBps_by_segment_length": by_segment}}

@@ -33,6 +33,13 @@ def build_library(verbose=False):
     return LIB_PATH
 
 
+def build_bench_probe(verbose=False):
+    """bench_gather_probe.so beside bench.py: the instrumentation kernel of `bench.py --workload gather_ceiling` (not part of the library)."""
+    out = os.path.join(ROOT, "bench_gather_probe.so")
+    _run([HIPCC] + FLAGS + ["-I" + ROOT, os.path.join(ROOT, "bench_gather_probe.hip"), "-o", out], verbose)
+    return out
+
+
 def build_cpp_tests(verbose=False):
     """tests/cpp/test_host, object_tool and test_binding (CPU; test_binding --gpu runs on the device) and tests/cpp/test_models
     (GPU): plain host C++ over the C ABI; the oracle library is linked as the checker."""

@@ -34,10 +34,6 @@ _SIGNATURES = {
     "bbhip_ReleaseScratch": (C.c_int, []),
     "bbhip_GetScratchSize": (C.c_size_t, []),
     "bbhip_GetSwitch": (C.c_int, [C.c_char_p]),
-    "bbhip_Probe_RowGather": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _vp]),
-    "bbhip_Probe_RowGatherSegments": (C.c_int, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "bbhip_SetAverageLutMean": (None, [_i]),
-    "bbhip_GetAverageLutMean": (C.c_int, []),
     "bbhip_SetDxMode": (None, [_i]),
     "bbhip_HintInputNodeSize": (None, [_i]),
     "bbhip_PackedRowWords": (C.c_int, [_i]),
@@ -67,6 +63,7 @@ _SIGNATURES = {
     "bbhip_fp32_StochasticMaxPooling2x2_Forward": (C.c_int, [_vp, _vp] + [_i] * 7 + [_vp]),
     "bbhip_fp32_StochasticMaxPooling2x2_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 7 + [_vp]),
     "bbhip_fp32_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
+    "bbhip_fp32_AverageLut_ForwardSum": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_bit_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_AverageLut_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 5 + [_vp]),
     "bbhip_fp32_MaxLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),

@@ -64,7 +64,6 @@ int fail(char const *fmt, ...)
 // ------------------------------------------------------------------------------------------------
 bool g_host_only = false;
 int  g_dx_mode   = 0;
-bool g_average_lut_mean = false;             // bbhip_SetAverageLutMean: un-binarized AverageLut output is sum * (1 / n)
 thread_local int g_input_node_hint = 0;      // bbhip_HintInputNodeSize: rows of the next forward call's input, 0 = unknown
 // bbhip_HintPackedInput: a caller-owned buffer for the packed copy of the next LUT call's binarized fp32 input
 struct PackedInputHint { uint32_t *bits; int rows, row_words, holds_input; };
@@ -1071,45 +1070,6 @@ int bbhip_GetSwitch(char const *name)
     return -1;
 }
 
-static int launch_row_gather_probe(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
-                                   int segment_frames, void *stream, char const *name)
-{
-    if (!(dev_x != nullptr && dev_sink != nullptr && row_count > 0 && frame_size > 0 && frame_stride >= frame_size && loads_per_unit > 0)) {
-        return fail("%s: rejected argument", name);
-    }
-    if (!(segment_frames == 64 || segment_frames == 128 || segment_frames == 256 || segment_frames == 512)) {
-        return fail("%s: segments are 64, 128, 256 or 512 frames long", name);
-    }
-    int const chunk_count = ceil_div(frame_size, segment_frames), tile_count = ceil_div(row_count, kWavesPerBlk);
-    if ((long long)chunk_count * tile_count > 0x7fffffffLL) { return fail("%s: grid too large", name); }
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    dim3 const grid((unsigned)(chunk_count * tile_count)), block(kBlock);
-    TileDivisor const tiles = make_tile_divisor(tile_count);
-    ScopedTimer tm(kTimeOther, st);
-    switch (segment_frames / kWave) {
-    case 1: hipLaunchKernelGGL(row_gather_probe_kernel<1>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
-    case 2: hipLaunchKernelGGL(row_gather_probe_kernel<2>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
-    case 4: hipLaunchKernelGGL(row_gather_probe_kernel<4>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
-    default: hipLaunchKernelGGL(row_gather_probe_kernel<8>, grid, block, 0, st, dev_x, dev_sink, row_count, frame_stride, frame_size, chunk_count, tiles, loads_per_unit); break;
-    }
-    BBHIP_LAUNCH_CHECK();
-    return 0;
-}
-
-int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit, void *stream)
-{
-    return launch_row_gather_probe(dev_x, dev_sink, row_count, frame_size, frame_stride, loads_per_unit, 128, stream, __func__);
-}
-
-int bbhip_Probe_RowGatherSegments(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
-                                  int segment_frames, void *stream)
-{
-    return launch_row_gather_probe(dev_x, dev_sink, row_count, frame_size, frame_stride, loads_per_unit, segment_frames, stream, __func__);
-}
-
-void bbhip_SetAverageLutMean(int mean) { g_average_lut_mean = mean != 0; }
-int  bbhip_GetAverageLutMean(void) { return g_average_lut_mean ? 1 : 0; }
-
 void bbhip_SetDxMode(int mode) { g_dx_mode = (mode == 1 || mode == 2) ? mode : 0; }
 void bbhip_HintInputNodeSize(int input_node_size) { g_input_node_hint = input_node_size > 0 ? input_node_size : 0; }
 int  bbhip_PackedRowWords(int frame_size) { return frame_size > 0 ? packed_row_words(frame_size) : 0; }
@@ -1431,20 +1391,34 @@ static int check_average_lut(void const *a, void const *b, int const *idx, int n
     return 0;
 }
 
-int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
-                                  int frame_stride, int binarize_input, int binarize_output, void *stream)
+static int average_lut_forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                               int frame_stride, int binarize_input, int binarize_output, bool mean, void *stream, char const *name)
 {
     clear_hints();                                 // a hint is for the next LUT forward call only
-    if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, __func__)) { return 1; }
+    if (check_average_lut(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, frame_size, name)) { return 1; }
     int const f_blocks = ceil_div(frame_size, kTailBlock);
     long long const blocks = (long long)node_size * f_blocks;
-    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", __func__); }
+    if (blocks > 0x7fffffffLL) { return fail("%s: grid too large", name); }
     ScopedTimer tm(kTimeOther, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(average_lut_forward_kernel, dim3((unsigned)blocks), dim3(kTailBlock), 0, static_cast<hipStream_t>(stream), dev_x_buf,
                        dev_y_buf, dev_input_index, n, frame_size, frame_stride, binarize_input, binarize_output, f_blocks,
-                       g_average_lut_mean ? 1.0f / (float)n : 1.0f);
+                       mean ? 1.0f / (float)n : 1.0f);
     BBHIP_LAUNCH_CHECK();
     return 0;
+}
+
+int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                  int frame_stride, int binarize_input, int binarize_output, void *stream)
+{
+    return average_lut_forward(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, binarize_input, binarize_output,
+                               true, stream, __func__);
+}
+
+int bbhip_fp32_AverageLut_ForwardSum(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                     int frame_stride, int binarize_input, int binarize_output, void *stream)
+{
+    return average_lut_forward(dev_x_buf, dev_y_buf, dev_input_index, n, node_size, frame_size, frame_stride, binarize_input, binarize_output,
+                               false, stream, __func__);
 }
 
 int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,

@@ -1402,49 +1402,6 @@ __global__ __launch_bounds__(kBlock) void dx_gather_kernel(float const *__restri
 }
 
 // ------------------------------------------------------------------------------------------------
-//  Instrumentation: the gather pattern of lut_dx_kernel without its arithmetic.  One wavefront per (row, unit of P x 64 frames;
-//  P = 2 is the dx kernel's unit), units dealt to the XCDs as everywhere; it reads `loads` pseudo-randomly chosen rows'
-//  segments of its frame window (P x 256 bytes each), six rows' loads in flight at a time like a dx term, and adds them up.  What this kernel sustains is the rate at
-//  which this GPU delivers gathered row segments from L2 to the compute units — the practical ceiling of any kernel with
-//  the dx kernel's access pattern.
-// ------------------------------------------------------------------------------------------------
-template <int P>
-__global__ __launch_bounds__(kBlock) void row_gather_probe_kernel(float const *__restrict__ x, float *__restrict__ sink, int rows, int stride,
-                                                                  int frame_size, int chunk_count, TileDivisor tiles, int loads)
-{
-    // P: 64-frame steps per row segment (a segment is P x 256 bytes, read with P loads in flight)
-    int const B   = chunk_count * tiles.count;
-    int const lid = xcd_remap(blockIdx.x, B);
-    int ck, tile;
-    split_tile(lid, tiles, ck, tile);
-    int const lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    if (tile * kWavesPerBlk + wave >= rows) { return; }
-    uint32_t s = (uint32_t)(lid * kWavesPerBlk + wave) * 2654435761u + 12345u;
-    int const f_last = frame_size - 1;
-    uint32_t off[P];
-#pragma unroll
-    for (int q = 0; q < P; ++q) { off[q] = (uint32_t)min(ck * (P * kWave) + q * kWave + lane, f_last) * 4u; }
-    float acc = 0.0f;
-    for (int r = 0; r < loads; r += 6) {
-        float v[6][P];
-#pragma unroll
-        for (int j = 0; j < 6; ++j) {
-            s = s * 1664525u + 1013904223u;
-            int const row = __builtin_amdgcn_readfirstlane((int)((s >> 8) % (uint32_t)rows));
-            char const *p = reinterpret_cast<char const *>(x + (size_t)row * stride);
-#pragma unroll
-            for (int q = 0; q < P; ++q) { v[j][q] = *reinterpret_cast<float const *>(p + off[q]); }
-        }
-#pragma unroll
-        for (int j = 0; j < 6; ++j) {
-#pragma unroll
-            for (int q = 0; q < P; ++q) { acc += v[j][q]; }
-        }
-    }
-    if (acc == 123.456f) { sink[0] = acc; }                 // (never true for the buffers it is run on; keeps the loads alive)
-}
-
-// ------------------------------------------------------------------------------------------------
 //  elementwise helpers
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void fill_kernel(float *__restrict__ dst, float v, size_t size)

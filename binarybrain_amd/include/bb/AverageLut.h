@@ -2,7 +2,10 @@
 // it is the strict majority of the n inputs.  Reference API: include/bb/AverageLut.h:22-458 (Create(n, output_shape,
 // connection, binarize, binarize_input, seed); commands binary / binarize_input / binarize_output / host_only; connection
 // get/set; GetLutTable = majority of the index bits; wiring policies and serialized form: bb/WiredSelectModel.h).
-// Frame work runs in the HIP library only.
+// Frame work runs in the HIP library only.  Without binarize_output the reference disagrees with itself: its CUDA kernel writes
+// sum * (1 / n) (cuda/AverageLut.cu:46-54), its host loop the plain sum (include/bb/AverageLut.h:331-343).  The class follows
+// the device path, which is what the reference's class runs where a GPU is present; the command "host_sum true" selects the
+// host loop's sum (a run-time choice like host_only: not part of the serialized object).
 #pragma once
 
 #include "bb/WiredSelectModel.h"
@@ -25,8 +28,16 @@ public:
     };
 
 protected:
+    bool m_host_sum = false;
+
     explicit AverageLut(create_t const &create)
         : WiredSelectModel(create.n, create.output_shape, create.connection, create.binarize_input, create.binarize_output, create.seed) {}
+
+    void CommandProc(std::vector<std::string> args) override
+    {
+        WiredSelectModel::CommandProc(args);
+        if (args.size() == 2 && args[0] == "host_sum") { m_host_sum = EvalBool(args[1]); }
+    }
 
 public:
     static std::string ModelName(void)  { return "AverageLut"; }
@@ -72,7 +83,8 @@ public:
                         "bbhip_bit_AverageLut_Forward");
         }
         else {
-            CheckDevice(bbhip_fp32_AverageLut_Forward((float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(), (int const *)idx_ptr.GetAddr(), m_n,
+            auto const entry = m_host_sum ? bbhip_fp32_AverageLut_ForwardSum : bbhip_fp32_AverageLut_Forward;
+            CheckDevice(entry((float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(), (int const *)idx_ptr.GetAddr(), m_n,
                             (int)y_buf.GetNodeSize(), (int)y_buf.GetFrameSize(), (int)(y_buf.GetFrameStride() / sizeof(float)),
                             m_binarize_input ? 1 : 0, m_binarize_output ? 1 : 0, nullptr), "bbhip_fp32_AverageLut_Forward");
         }

@@ -18,11 +18,6 @@ def _dev(*ts):
             raise capi.BbhipError("bbhip ops need contiguous tensors")
 
 
-def set_average_lut_mean(mean):
-    """False (default): AverageLut writes the sum of its inputs (the reference's host path); True: sum * (1 / n) (its CUDA kernel)."""
-    lib().bbhip_SetAverageLutMean(int(bool(mean)))
-
-
 def set_dx_mode(mode):
     """0: deterministic dx, input-centric re-evaluation through the reverse table (default); 1: fp32 atomics;
     2: the reference's scheme (per-connection gradients in dx_tmp, summed through the reverse table)."""
@@ -237,13 +232,14 @@ def stochastic_bn_backward(x, dy, mean, rstd, frame_size, gamma=0.2):
     return dx
 
 
-def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True):
-    """fp32 x [I, stride] -> y [O, stride]: sum of the n wired inputs (their votes when binarize_input), or its sign."""
+def average_lut_forward(x, idx, frame_size, binarize_input=False, binarize_output=True, mean=True):
+    """fp32 x [I, stride] -> y [O, stride]: the sign of the sum of the n wired inputs (their votes when binarize_input) or, without
+    binarize_output, sum * (1 / n) as the reference's CUDA kernel writes it; mean=False: the plain sum of the reference's host loop."""
     _dev(x, idx)
     O, n = idx.shape
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
-    check(lib().bbhip_fp32_AverageLut_Forward(ptr(x), ptr(y), ptr(idx), n, O, frame_size, x.shape[1], int(binarize_input),
-                                              int(binarize_output), stream_ptr()))
+    entry = lib().bbhip_fp32_AverageLut_Forward if mean else lib().bbhip_fp32_AverageLut_ForwardSum
+    check(entry(ptr(x), ptr(y), ptr(idx), n, O, frame_size, x.shape[1], int(binarize_input), int(binarize_output), stream_ptr()))
     return y
 
 

@@ -96,8 +96,8 @@ inline int bbcu_bit_BinatyLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int
                                        int node_size, int frame_size, int frame_stride, cudaStream_t streamId = 0)
 { BBCU_HIP_CALL(bbhip_bit_BinaryLut6_Forward(dev_x_buf, dev_y_buf, dev_input_index, dev_table, node_size, frame_size, frame_stride, streamId)); return 0; }
 
-/* ---- AverageLut, include/bbcu/bbcu.h:321-361 (T = float).  Without binarize_output the library writes the sum of the
- * inputs, as the reference's host path does; its CUDA kernel writes sum / n (see bbhip.h) ---- */
+/* ---- AverageLut, include/bbcu/bbcu.h:321-361 (T = float).  Without binarize_output the forward entry writes sum * (1 / n), as the
+ * CUDA kernel of this name does (cuda/AverageLut.cu:46-54); the host loop's plain sum is bbhip_fp32_AverageLut_ForwardSum ---- */
 template <typename T>
 int bbcu_AverageLut_Forward(T const *dev_x_buf, T *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                             int frame_stride, bool binarize_input, bool binarize_output, cudaStream_t streamId = 0)

@@ -76,14 +76,6 @@ size_t bbhip_GetScratchSize(void);
  * number, and takes its default (on) when unset. */
 int bbhip_GetSwitch(char const *name);
 
-/* ---- which of the reference's two AverageLut conventions the forward entry follows (no counterpart in the reference) ----
- * The reference disagrees with itself: without binarize_output its host loop writes the SUM of the n inputs
- * (include/bb/AverageLut.h:331-343), its CUDA kernel writes sum * (1 / n) (cuda/AverageLut.cu:46-54); both backward paths
- * return dy / n.  0 (default): the host convention; 1: the CUDA kernel's (the fp32 reciprocal of n, then one multiply).
- * A process-wide switch like the dx mode; binarized outputs and the packed-bit entry do not depend on it. */
-void bbhip_SetAverageLutMean(int mean);
-int  bbhip_GetAverageLutMean(void);
-
 /* ---- how dx is accumulated over the fan-out of an input node (no counterpart in the reference) ----
  * 0 (default): deterministic, no scratch — one wavefront per (input node, frame chunk) walks reverse_index in the
  *              reference's order (cuda/Common.cuh:174-202, include/bb/FixedSizeConnectionTable.h:198-214) and
@@ -137,19 +129,6 @@ size_t bbhip_PreparedTablesBytes(int n, int node_size);
  * returns their summed duration and count, and forgets them. */
 void bbhip_KernelTimer_Enable(int enable);
 int  bbhip_KernelTimer_Read(int which, float *total_ms, int *launches);
-
-/* ---- gather probe (instrumentation; no counterpart in the reference) ----
- * Runs the memory access pattern of the input-centric dx kernel without its arithmetic: one wavefront per (row, 128-frame
- * window) reads `loads_per_unit` (rounded up to a multiple of 6) pseudo-randomly chosen rows' 512-byte segments of that
- * window from dev_x [row_count][frame_stride] and discards them.  Bytes moved per launch:
- * row_count * ceil(frame_size / 128) * loads_per_unit * 512.  Timed by the kernel timer as kind 4.  Used by bench.py to put
- * a measured ceiling next to the dx kernel's rate.  dev_sink: one float that is never written in practice. */
-int bbhip_Probe_RowGather(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
-                          void *stream);
-/* The same with windows of segment_frames = 64, 128, 256 or 512 frames (row segments of 256 bytes to 2 KiB): how the rate that the
- * GPU sustains depends on the bytes read per visited row, and where the window of all rows stops fitting an L2. */
-int bbhip_Probe_RowGatherSegments(float const *dev_x, float *dev_sink, int row_count, int frame_size, int frame_stride, int loads_per_unit,
-                                  int segment_frames, void *stream);
 
 /* ---- elementwise helpers ---- */
 /* bbcu_fp32_Vector_set, include/bbcu/bbcu.h:89-94 */
@@ -243,12 +222,17 @@ int bbhip_fp32_StochasticMaxPooling2x2_Backward(float const *dev_x_buf, float co
                                                 int frame_stride, void *stream);
 
 /* ---- AverageLut, softmax cross entropy, categorical accuracy (the tail of a LUT classifier) ---- */
-/* bbcu_AverageLut_Forward<float>, include/bbcu/bbcu.h:321-334.  y = sum over the n inputs dev_input_index[node*n + i] of x (each
- * replaced by +1 / -1 on x > 0 when binarize_input), written as +1 / -1 on sum > 0 when binarize_output.  Without
- * binarize_output the SUM is written, as by the reference's host loop (include/bb/AverageLut.h:331-343); its CUDA kernel
- * writes sum * (1 / n) (cuda/AverageLut.cu:46-54), which bbhip_SetAverageLutMean(1) selects. */
+/* bbcu_AverageLut_Forward<float>, include/bbcu/bbcu.h:321-334.  s = sum over the n inputs dev_input_index[node*n + i] of x (each
+ * replaced by +1 / -1 on x > 0 when binarize_input); with binarize_output y = +1 / -1 on s > 0, else y = s * (1 / n) with the fp32
+ * reciprocal of n, as the CUDA kernel of that name writes it (cuda/AverageLut.cu:46-54, 93) — the mean, whose gradient dy / n is
+ * what both backward paths of the reference return. */
 int bbhip_fp32_AverageLut_Forward(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
                                   int frame_stride, int binarize_input, int binarize_output, void *stream);
+/* The same with the convention of the reference's HOST loop, which disagrees with its CUDA kernel: without binarize_output the SUM s is
+ * written (include/bb/AverageLut.h:331-343).  No bbcu counterpart; for callers that reproduce networks trained on the reference's
+ * host path (bb::AverageLut takes it after the command "host_sum true").  Binarized outputs are the same in both. */
+int bbhip_fp32_AverageLut_ForwardSum(float const *dev_x_buf, float *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,
+                                     int frame_stride, int binarize_input, int binarize_output, void *stream);
 /* bbcu_bit_AverageLut_Forward, include/bbcu/bbcu.h:336-346: packed bits, y = strict majority of the n inputs (a tie of an even
  * n gives 0); frame_stride in 32-bit words */
 int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int n, int node_size, int frame_size,

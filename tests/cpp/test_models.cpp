@@ -954,10 +954,21 @@ static void test_tail(void)
         auto avg = bb::AverageLut<>::Create(n, (bb::index_t)O, "", binarize != 0);
         avg->SetInputShape({I});
         for (int o = 0; o < O; ++o) for (int i = 0; i < n; ++i) { avg->SetNodeConnectionIndex(o, i, idx[(size_t)o * n + i]); }
-        bb::FrameBuffer y_buf = avg->Forward(x_buf);
+        // the class follows the reference's device path: sum * (1 / n) where the output is not binarized; "host_sum true" gives
+        // the host loop's plain sum, which is what the oracle restates
         oracle_fp32_AverageLut_Forward(x.data(), y_ref.data(), idx.data(), n, O, F, F, 0, binarize);
+        bb::FrameBuffer y_buf = avg->Forward(x_buf);
         read_fp32(y_buf, got);
-        CHECK(got == y_ref, "AverageLut forward (binarize %d)", binarize);
+        {
+            std::vector<float> y_mean(y_ref);
+            float const reciprocal = 1.0f / (float)n;
+            if (!binarize) { for (auto &v : y_mean) { v = v * reciprocal; } }
+            CHECK(got == y_mean, "AverageLut forward, device convention (binarize %d)", binarize);
+        }
+        avg->SendCommand("host_sum true");
+        y_buf = avg->Forward(x_buf);
+        read_fp32(y_buf, got);
+        CHECK(got == y_ref, "AverageLut forward, host convention (binarize %d)", binarize);
         bb::FrameBuffer dx_buf = avg->Backward(dy_buf);
         oracle_fp32_AverageLut_Backward(dy.data(), dx_ref.data(), idx.data(), n, I, O, F, F);
         read_fp32(dx_buf, got);

@@ -59,9 +59,14 @@ def test_full_size_against_oracle_slice_and_stochastic_lut(ops):
     y = ops.binary_lut6_forward(dev(xb), dev(idx), dev(T), F)
     sel = np.arange(0, O, 509)                  # every position of a node within the group that shares a wavefront
     y_ref = oracle.binary_lut6_forward(xb, idx[sel], T[sel], F, words=True)
-    assert np.array_equal(host(y)[sel], y_ref)
+    yh = host(y)
+    assert np.array_equal(yh[sel], y_ref)
+    # every node: over the first and over the last 8192 frames (256 words each; a node's words do not depend on one another)
+    for w0 in (0, F // 32 - 256):
+        part = np.ascontiguousarray(xb[:, w0:w0 + 256])
+        assert np.array_equal(yh[:, w0:w0 + 256], oracle.binary_lut6_forward(part, idx, T, 8192, words=True)), w0
     # the same layer as a StochasticLut with W in {0,1} and bit inputs mapped to 0/1 (bias 0.5): y > 0.5 reproduces the table
     sel2 = sel[:8]
     W = np.array([[(int(np.uint32(T[o, b >> 5])) >> (b & 31)) & 1 for b in range(64)] for o in sel2], np.float32)
     yb = ops.bit_bit_stochastic_lut_forward(6, dev(xb), dev(idx[sel2]), dev(W), F, bias=0.5)
-    assert np.array_equal(host(yb), host(y)[sel2])
+    assert np.array_equal(host(yb), yh[sel2])

@@ -132,7 +132,7 @@ def test_classifier_training_step_at_full_size():
         a = y_ref
     # the tail: AverageLut (sum of seven 0/1 activations: exact), loss and its gradient, accuracy
     out_ref = oracle.average_lut_forward(a, idx_avg, F, False, False)
-    out = ops.average_lut_forward(dev(a), dev(idx_avg), F, False, False)
+    out = ops.average_lut_forward(dev(a), dev(idx_avg), F, False, False, mean=False)
     assert np.array_equal(host(out)[:, :F], out_ref[:, :F])
     dy_ref, loss_ref, tsum_ref = oracle.loss_softmax_cross_entropy(out_ref, t, CLASSES, 1, F)
     dy, loss_buf, t_sum = ops.loss_softmax_cross_entropy(dev(out_ref), dev(t), CLASSES, 1, F)

@@ -265,8 +265,9 @@ def run_tail_case(ops, torch, seed):
         dy = tail._pad(rng.standard_normal((O, F)).astype(F32), stride)
         for bin_in in (False, True):
             for bin_out in (False, True):
-                y = host(ops.average_lut_forward(dev(x), dev(idx), F, bin_in, bin_out))
-                assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, bin_in, bin_out)[:, :F]), (bin_in, bin_out)
+                mean = bool((bin_in + 2 * bin_out + F) & 1)          # both conventions for the un-binarized output
+                y = host(ops.average_lut_forward(dev(x), dev(idx), F, bin_in, bin_out, mean=mean))
+                assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, bin_in, bin_out, mean=mean)[:, :F]), (bin_in, bin_out, mean)
         dx = host(ops.average_lut_backward(dev(dy), dev(idx), I, F))
         assert np.array_equal(dx, oracle.average_lut_backward(dy, idx, I, F))
         xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))

@@ -267,6 +267,18 @@ def test_full_size_properties(ops):
     fs = 256
     dx_ref, _ = oracle.stochastic_lut_backward(6, np.ascontiguousarray(x[:, :fs]), np.ascontiguousarray(dy[:, :fs]), idx, W, fs)
     assert_bwd(host(dxb)[:, :fs], dx_ref)
+    # every node: y over a 512-frame slice in the middle of the batch, and dW of the full-size call when dy is zero outside that
+    # slice (then the table gradient is that of the slice alone, and so is dx inside it)
+    f0, fn = 4096 + 64, 512
+    xs_, dys_ = np.ascontiguousarray(x[:, f0:f0 + fn]), np.ascontiguousarray(dy[:, f0:f0 + fn])
+    assert_fwd(host(y)[:, f0:f0 + fn], oracle.stochastic_lut_forward(6, xs_, idx, W, fn))
+    dy_cut = np.zeros_like(dy); dy_cut[:, f0:f0 + fn] = dys_
+    dWs = torch.zeros((O, 64), device="cuda")
+    dxs = ops.stochastic_lut_backward(6, xd, dev(dy_cut), idxd, Wd, dWs, F, rev)
+    dx_ref, dW_ref = oracle.stochastic_lut_backward(6, xs_, dys_, idx, W, fn)
+    assert_bwd(host(dWs), dW_ref)
+    assert_bwd(host(dxs)[:, f0:f0 + fn], dx_ref)
+    assert not host(dxs)[:, :f0].any() and not host(dxs)[:, f0 + fn:].any()
 
 
 def test_full_size_properties_packed_bits(ops):

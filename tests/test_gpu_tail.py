@@ -55,8 +55,9 @@ def test_average_lut(ops, shape):
     dy = _pad(rng.standard_normal((O, F)).astype(F32), stride)
     for bin_in in (False, True):
         for bin_out in (False, True):
-            y = host(ops.average_lut_forward(dev(x), dev(idx), F, bin_in, bin_out))
-            assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, bin_in, bin_out)[:, :F]), (bin_in, bin_out)
+            for mean in (False, True):
+                y = host(ops.average_lut_forward(dev(x), dev(idx), F, bin_in, bin_out, mean=mean))
+                assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, bin_in, bin_out, mean=mean)[:, :F]), (bin_in, bin_out, mean)
     dx = host(ops.average_lut_backward(dev(dy), dev(idx), I, F))
     assert np.array_equal(dx, oracle.average_lut_backward(dy, idx, I, F))          # padding columns included: zero
     xb = synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))
@@ -68,7 +69,7 @@ def test_average_lut_reference_vectors(ops):
     for k in range(int(GOLD["average_count"][0])):
         n, I, O, F, bin_in, bin_out = [int(v) for v in GOLD["a%d_geom" % k]]; q = "a%d_" % k
         idx = GOLD[q + "idx"]
-        y = host(ops.average_lut_forward(dev(GOLD[q + "x"]), dev(idx), F, bool(bin_in), bool(bin_out)))
+        y = host(ops.average_lut_forward(dev(GOLD[q + "x"]), dev(idx), F, bool(bin_in), bool(bin_out), mean=False))      # vectors of the host loop
         assert np.array_equal(y, GOLD[q + "y"]), k
         dx = host(ops.average_lut_backward(dev(GOLD[q + "dy"]), dev(idx), I, F))
         assert np.array_equal(dx, GOLD[q + "dx"]), k
@@ -182,23 +183,23 @@ def test_rejected_arguments(ops):
         ops.metrics_categorical_accuracy(x, x, 4, 1, 0)
 
 
-def test_average_lut_mean_convention(ops):
-    """bbhip_SetAverageLutMean(1): the un-binarized forward follows the reference's CUDA kernel, sum * (1 / n), bit for bit;
-    binarized outputs and the backward (dy / n in both conventions) do not change."""
+def test_average_lut_both_conventions(ops):
+    """bbhip_fp32_AverageLut_Forward follows the reference's CUDA kernel of that name, sum * (1 / n), bit for bit;
+    bbhip_fp32_AverageLut_ForwardSum its host loop, the plain sum; binarized outputs are the same in both, and so is the
+    backward pass (dy / n)."""
     rng = np.random.default_rng(77)
-    try:
-        for n in (6, 7, 8):
-            I, O, F = 90, 15, 333
-            S = synth.frame_stride_fp32(F)
-            idx = rng.integers(0, I, (O, n)).astype(np.int32)
-            x = np.zeros((I, S), np.float32); x[:, :F] = rng.standard_normal((I, F))
-            ops.set_average_lut_mean(True)
-            y = host(ops.average_lut_forward(dev(x), dev(idx), F, False, False))
-            yb = host(ops.average_lut_forward(dev(x), dev(idx), F, True, True))
-            ops.set_average_lut_mean(False)
-            ys = host(ops.average_lut_forward(dev(x), dev(idx), F, False, False))
-            assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, False, False, mean=True)[:, :F])
-            assert np.array_equal(ys[:, :F], oracle.average_lut_forward(x, idx, F, False, False)[:, :F])
-            assert np.array_equal(yb[:, :F], oracle.average_lut_forward(x, idx, F, True, True)[:, :F])
-    finally:
-        ops.set_average_lut_mean(False)
+    for n in (6, 7, 8):
+        I, O, F = 90, 15, 333
+        S = synth.frame_stride_fp32(F)
+        idx = rng.integers(0, I, (O, n)).astype(np.int32)
+        x = np.zeros((I, S), np.float32); x[:, :F] = rng.standard_normal((I, F))
+        y = host(ops.average_lut_forward(dev(x), dev(idx), F, False, False))             # the entry's own convention: the mean
+        ys = host(ops.average_lut_forward(dev(x), dev(idx), F, False, False, mean=False))
+        yb = host(ops.average_lut_forward(dev(x), dev(idx), F, True, True))
+        ybs = host(ops.average_lut_forward(dev(x), dev(idx), F, True, True, mean=False))
+        assert np.array_equal(y[:, :F], oracle.average_lut_forward(x, idx, F, False, False, mean=True)[:, :F])
+        assert np.array_equal(ys[:, :F], oracle.average_lut_forward(x, idx, F, False, False)[:, :F])
+        assert np.array_equal(yb[:, :F], oracle.average_lut_forward(x, idx, F, True, True)[:, :F])
+        assert np.array_equal(yb[:, :F], ybs[:, :F])
+        # the two differ by exactly the fp32 reciprocal of n
+        assert np.array_equal(y[:, :F], (ys[:, :F] * (np.float32(1.0) / np.float32(n))).astype(np.float32))

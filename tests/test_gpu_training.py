@@ -53,7 +53,7 @@ def test_lut_network_learns():
         else:
             y1 = ops.differentiable_lut_forward_inference(6, x, d_idx1, W1, F, rm1, rv1); m1 = r1 = None
             y2 = ops.differentiable_lut_forward_inference(6, y1, d_idx2, W2, F, rm2, rv2); m2 = r2 = None
-        y3 = ops.average_lut_forward(y2, d_idx3, F, False, False)
+        y3 = ops.average_lut_forward(y2, d_idx3, F, False, False, mean=False)
         return y1, m1, r1, y2, m2, r2, y3
 
     losses, accuracies = [], []
