@@ -18,17 +18,103 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 
-# HBM-side bytes per launch at the default workloads, from the hardware counters FETCH_SIZE (x 2.000 KiB per count) and
-# WRITE_SIZE (x 1.000 KiB per count); each scale is what the same counter reads for a plain device copy of known size in
-# the same profiler run.  The counter tables and the commands are in profiles/*.md.  A kernel or workload that is not
-# listed reports null.
-MEASURED_TRAFFIC_BYTES = {
-    ("lut_dx_kernel<6>", 0):       (651415.9 * 2.0 + 132096.0) * 1024,
-    ("lut_forward_kernel<6>", 0):  (128472.4 * 2.0 + 131072.0) * 1024,
-    ("lut_backward_kernel<6>", 0): (352168.3 * 2.0 + 6391.2) * 1024,
-    ("binary_lut6_kernel", 0):     (348316.2 * 2.0 + 524288.0) * 1024,
-    ("adam_kernel", 0):            (527931.3 * 2.0 + 791860.5) * 1024,
+# HBM-side bytes per launch (per step, for the step workloads) come from the hardware counters FETCH_SIZE and WRITE_SIZE, collected with
+# rocprofv3 and written to profiles/traffic.json by `bench.py --write-traffic` (TRAFFIC_COMMANDS below); nothing is measured twice
+# here: the bench line carries what that file holds for the kernel, and the file's git blob hash, or null where the file has no entry.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+TRAFFIC_WORKLOADS = {          # workload -> (extra bench arguments, kernel that runs once per step)
+    "stochasticlut6": ("--no-configs --profile-copy", "lut_dx_kernel"),
+    "binarylut6": ("--profile-copy", "binary_lut6_kernel"),
+    "adam": ("", "adam_kernel"),
+    "mnist_step": ("", "adam_kernel"),
+    "conv_block": ("", "im2col_backward_kernel"),
 }
+TRAFFIC_COMMANDS = [
+    "rocprofv3 --pmc %s -d gpurun_out/traffic/%s/%s -o r -- python3 bench.py --workload %s --steps 5 --warmup 5 --ramp-seconds 0 --no-cpu %s"
+    % (counter, w, counter, w, extra) for w, (extra, _) in TRAFFIC_WORKLOADS.items() for counter in ("FETCH_SIZE", "WRITE_SIZE")
+] + ["python3 bench.py --write-traffic gpurun_out/traffic"]
+
+
+def _git_blob_hash(path):
+    import hashlib
+    data = open(path, "rb").read()
+    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+
+
+_traffic_cache = None
+
+
+def measured_traffic(section, name):
+    """bytes from profiles/traffic.json: section "kernels" (per launch) or "steps" (per step); None when the file has no such entry"""
+    global _traffic_cache
+    if _traffic_cache is None:
+        try:
+            _traffic_cache = json.load(open(TRAFFIC_FILE))
+            _traffic_cache["git_blob"] = _git_blob_hash(TRAFFIC_FILE)
+        except (OSError, ValueError):
+            _traffic_cache = {}
+    entry = _traffic_cache.get(section, {}).get(name)
+    return None if entry is None else entry["bytes"]
+
+
+def traffic_source():
+    measured_traffic("kernels", "")
+    return {"file": "profiles/traffic.json", "git_blob": _traffic_cache.get("git_blob")}
+
+
+def _short_kernel_name(name):
+    """'void bbhip::lut_dx_kernel<6, 0, 2>(bbhip::DxArgs)' -> 'lut_dx_kernel'"""
+    name = name.split("(")[0].replace("void ", "").strip()
+    return name.split("<")[0].split("::")[-1]
+
+
+def write_traffic(dirname):
+    """Reads the counter runs of TRAFFIC_COMMANDS under `dirname` (rocprofv3's r_results.db per workload and counter) and writes
+    profiles/traffic.json: per kernel of the library the mean FETCH_SIZE / WRITE_SIZE per dispatch in bytes, per step workload the sum
+    over one step.  A counter's unit is taken from what it reads for the plain device copies of known size at the end of the
+    `--profile-copy` runs (torch's copy kernel: x.numel() * 4 bytes read and as many written per copy)."""
+    import sqlite3
+
+    def counters(workload, counter):
+        db = os.path.join(dirname, workload, counter, "r_results.db")
+        con = sqlite3.connect(db)
+        rows = con.execute("select kernel_name, value from counters_collection where counter_name = ? order by rowid", (counter,)).fetchall()
+        con.close()
+        by = {}
+        for name, value in rows:
+            by.setdefault(name, []).append(float(value))
+        return by
+
+    copy_bytes = {"stochasticlut6": 4096 * 8320 * 4, "binarylut6": 8192 * 8288 * 4}
+    unit = {}
+    calibration = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        units = []
+        for w, nbytes in copy_bytes.items():
+            by = counters(w, counter)
+            copies = [v for name, vals in by.items() if ("copy" in name.lower() or "elementwise" in name.lower()) for v in vals[-3:]]
+            if copies:
+                units.append(nbytes / (sum(copies) / len(copies)))
+                calibration["%s, %s" % (counter, w)] = {"copy_bytes": nbytes, "counter_per_copy": sum(copies) / len(copies)}
+        unit[counter] = sum(units) / len(units)
+    out = {"made_by": TRAFFIC_COMMANDS, "counter_unit_bytes": unit, "calibration": calibration, "kernels": {}, "steps": {}}
+    for w, (_, marker) in TRAFFIC_WORKLOADS.items():
+        fetch, write = counters(w, "FETCH_SIZE"), counters(w, "WRITE_SIZE")
+        steps = max(len(v) for name, v in fetch.items() if marker in name)
+        step_bytes = 0.0
+        for name in fetch:
+            if "bbhip::" not in name:
+                continue
+            f = sum(fetch[name]) / len(fetch[name]) * unit["FETCH_SIZE"]
+            wr = sum(write.get(name, [0.0])) / max(1, len(write.get(name, [0.0]))) * unit["WRITE_SIZE"]
+            step_bytes += (f + wr) * len(fetch[name]) / steps
+            if w in ("stochasticlut6", "binarylut6", "adam"):
+                out["kernels"]["%s/%s" % (w, _short_kernel_name(name))] = {"bytes": f + wr, "fetch_bytes": f, "write_bytes": wr, "dispatches": len(fetch[name]), "workload": w}
+        out["steps"][w] = {"bytes": step_bytes, "steps_counted": steps}
+    with open(TRAFFIC_FILE, "w") as fh:
+        json.dump(out, fh, indent=1, sort_keys=True)
+        fh.write("\n")
+    print("wrote %s: %d kernels, %d step workloads" % (TRAFFIC_FILE, len(out["kernels"]), len(out["steps"])))
 
 
 def algorithmic_bytes(I, O, F):
@@ -109,7 +195,7 @@ def bench_adam(args, lib):
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
            "config": {"workload": "Adam step over %d tensors, %d elements" % (len(sizes), total)},
            "roofline": {"bound": "hbm", "kernel": "adam_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES[("adam_kernel", 0)]}}
+                        "frac": gbs / HBM_PEAK_GBS, "traffic": measured_traffic("kernels", "adam/adam_kernel"), "traffic_source": traffic_source()}}
     if not args.no_cpu:
         import oracle
         n = 1 << 22
@@ -369,31 +455,39 @@ def bench_differentiablelut6(args, lib):
         xb = torch.from_numpy(synth.bernoulli_bits(rng, I, F, synth.frame_stride_bit(F))).cuda()
 
     tables = ops.prepared_tables_buffer(6, idx.shape[0])     # the model class keeps the tables derived from W from forward to backward
+    packed = ops.packed_input_buffer(I, F)                   # ... and the packed copy of its binarized input
+    plain = getattr(args, "plain_signatures", False)
+    clamp_w = None if plain else (0.0, 1.0)
 
     def step():
-        # (the table is clamped to [0, 1] in place by the forward entry's table launch, as the model class does before a forward pass)
+        # (the table is clamped to [0, 1] in place by the forward entry, as the model class does before a forward pass; with the
+        # reference's plain signatures the clamp is a launch of its own)
+        if plain:
+            ops.vector_clamp_(W, 0.0, 1.0)
         if bits:
-            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=(0.0, 1.0), tables=tables)
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=clamp_w, tables=tables)
             ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev, tables=tables)
         else:
-            # the model class keeps the packed copy of its binarized input from the forward to the backward call
-            packed = ops.packed_input_buffer(I, F)
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=(0.0, 1.0), packed=packed, tables=tables)
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=clamp_w, packed=packed, tables=tables)
             ops.differentiable_lut_backward(6, x, dy, idx, W, dW, F, mean, rstd, rev, packed=packed, tables=tables)
 
-    t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < args.ramp_seconds:
-        for _ in range(10):
+    ops.HINTS = not plain
+    try:
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < args.ramp_seconds:
+            for _ in range(10):
+                step()
+            torch.cuda.synchronize()
+        for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+    finally:
+        ops.HINTS = True
     # every tensor once per pass: forward x, y, tables; backward x, dy, dx, tables, per-node statistics
     nbytes = 4 * F * (I + O) + 4 * F * (2 * I + O) + 4 * 280 * O + 32 * O
     if bits:      # packed x and y (1 bit per element), fp32 dy and dx
@@ -436,38 +530,57 @@ def bench_conv_block(args, lib):
     dpooled = torch.randn((CO * (OH // 2) * (OW // 2), synth.frame_stride_fp32(F)), device="cuda", generator=g)
     ops.set_dx_mode(0)
 
+    # what a caller that keeps a layer's input for the backward pass keeps as well (the model classes do): the packed copy of each
+    # layer's binarized input — the first layer's is packed by its forward call, the second layer's is written by the first layer's
+    # forward call as its packed output — and the tables derived from W
+    for l in layers:
+        l["packed_in"] = ops.packed_input_buffer(l["I"], FW_FRAMES)
+        l["tables"] = ops.prepared_tables_buffer(6, l["O"])
+
+    plain = getattr(args, "plain_signatures", False)
+    clamp_w = None if plain else (0.0, 1.0)
+
     def step():
         cols = ops.im2col_forward(img, C, H, W_, F, FH, FW)
         a = cols; acts = []
-        for l in layers:
-            # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
-            # ... and keeps the packed copy of its binarized input for the backward call
-            packed = ops.packed_input_buffer(a.shape[0], FW_FRAMES)
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed,
-                                                                    tables=l.setdefault("tables", ops.prepared_tables_buffer(6, l["idx"].shape[0])))
-            acts.append((a, mean, rstd, packed)); a = y
+        for k, l in enumerate(layers):
+            # the model class clamps its table before the first forward pass after a backward pass; the entry does it with its tables
+            # (with the reference's plain signatures the clamp is a launch of its own)
+            if plain:
+                ops.vector_clamp_(l["W"], 0.0, 1.0)
+            nxt = layers[k + 1]["packed_in"] if k + 1 < len(layers) else None
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], FW_FRAMES, l["rm"], l["rv"], clamp_w=clamp_w,
+                                                                    packed=l["packed_in"], packed_holds=(k > 0), packed_out=nxt, tables=l["tables"])
+            acts.append((a, mean, rstd)); a = y
         maps = ops.col2im_forward(a, CO, OH, OW, F)
         pooled = ops.stochastic_maxpool2x2_forward(maps, CO, OH, OW, F)
         dmaps = ops.stochastic_maxpool2x2_backward(maps, dpooled, CO, OH, OW, F)
         dy = ops.col2im_backward(dmaps, CO, OH, OW, F)
-        for l, (a_in, mean, rstd, packed) in zip(reversed(layers), reversed(acts)):
-            l["dW"].zero_()
-            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"], packed=packed, tables=l["tables"])
+        for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
+            # one backward pass per step and no optimizer in it: the table gradient is written, not accumulated (a fill launch otherwise)
+            if not ops.HINTS:
+                l["dW"].zero_()
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], FW_FRAMES, mean, rstd, l["rev"], packed=l["packed_in"],
+                                                 tables=l["tables"], overwrite_dw=ops.HINTS)
         return ops.im2col_backward(dy, C, H, W_, F, FH, FW), pooled
 
-    t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < args.ramp_seconds:
-        for _ in range(3):
+    ops.HINTS = not plain
+    try:
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < args.ramp_seconds:
+            for _ in range(3):
+                step()
+            torch.cuda.synchronize()
+        for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+    finally:
+        ops.HINTS = True
     node_evals = sum(l["O"] for l in layers) * FW_FRAMES
     e = 4
     # every activation and gradient once per pass: image, window columns, both LUT layers, maps, pooled maps
@@ -479,7 +592,8 @@ def bench_conv_block(args, lib):
            "config": {"workload": "Im2Col 3x3 -> DifferentiableLut6 27->216->36 (batch_norm, binary) -> Col2Im 36x30x30 -> StochasticMaxPooling2x2, "
                                   "256 images of 3x32x32, forward + backward", "images_per_s": F / dt},
            "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None if plain else measured_traffic("steps", "conv_block"),
+                        "traffic_source": traffic_source()}}
     if not args.no_cpu:
         import oracle
         Fs = 4                                                # images in the CPU sample
@@ -487,21 +601,45 @@ def bench_conv_block(args, lib):
         xs = np.zeros((C * H * W_, S), np.float32); xs[:, :Fs] = img[:, :Fs].cpu().numpy()
         Ws = [l["W"].cpu().numpy() for l in layers]; idxs = [l["idx"].cpu().numpy() for l in layers]
         dps = np.ascontiguousarray(dpooled[:, :Fs].cpu().numpy())          # the oracle's conv functions work on dense rows
-        t0 = time.perf_counter()
-        a = oracle.im2col_forward(xs, C, H, W_, Fs, FH, FW); acts = []
-        for l, Wt, idx in zip(layers, Ws, idxs):
-            y, mean, rstd, _, _ = oracle.differentiable_lut_forward_training(6, a, idx, Wt, FWs, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))
-            acts.append((a, mean, rstd)); a = y
-        maps = oracle.col2im_forward(a, CO, OH, OW, Fs)
-        oracle.stochastic_maxpool2x2_forward(maps, CO, OH, OW, Fs)
-        dy = oracle.col2im_backward(oracle.stochastic_maxpool2x2_backward(maps, dps, CO, OH, OW, Fs), CO, OH, OW, Fs)
-        for l, Wt, idx, (a_in, mean, rstd) in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(acts)):
-            dy, _ = oracle.differentiable_lut_backward(6, a_in, dy, idx, Wt, FWs, mean, rstd)
-        oracle.im2col_backward(dy, C, H, W_, Fs, FH, FW)
-        cpu_dt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": sum(l["O"] for l in layers) * FWs / cpu_dt / 1e9, "unit": "G node-evals/s", "cores": 1, "kind": "port",
-                               "sample": "the same block on %d images through the C restatement of the reference's host path (generic DifferentiableLut "
-                                         "algorithm, whose batch-norm backward is single-threaded in the reference too)" % Fs}
+        threads = min(os.cpu_count() or 1, 16)
+        if oracle.have_ref():
+            # the reference's own classes (oracle/_ref: its headers compiled in place; OpenMP forward, single-threaded batch-norm backward).
+            # Untimed: one forward pass for the activations.  Timed: every layer's Forward + Backward, last layer first.
+            os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+            dense = lambda a_, n_: np.ascontiguousarray(a_[:, :n_])
+            cols, _ = oracle.ref_im2col(dense(xs, Fs), C, H, W_, Fs, FH, FW)
+            a = cols; ins = []
+            for l, Wt, idx in zip(layers, Ws, idxs):
+                ins.append(a)
+                a = oracle.ref_differentiable_lut(6, a, idx, Wt, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))["y"]
+            maps, _ = oracle.ref_col2im(a, CO, OH, OW, Fs)
+            t0 = time.perf_counter()
+            oracle.ref_im2col(dense(xs, Fs), C, H, W_, Fs, FH, FW)
+            _, dmaps = oracle.ref_stochastic_maxpool2x2(maps, CO, OH, OW, Fs, dy=dps)
+            _, dy = oracle.ref_col2im(a, CO, OH, OW, Fs, dy=dmaps)
+            for l, Wt, idx, a_in in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(ins)):
+                dy = oracle.ref_differentiable_lut(6, a_in, idx, Wt, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32), dy=dy)["dx"]
+            oracle.ref_im2col(dense(xs, Fs), C, H, W_, Fs, FH, FW, dy=dy)
+            cpu_dt = time.perf_counter() - t0
+            out["cpu_baseline"] = {"value": sum(l["O"] for l in layers) * FWs / cpu_dt / 1e9, "unit": "G node-evals/s", "cores": threads, "kind": "reference",
+                                   "sample": "the same block on %d of the 256 images through the reference's own host classes (Forward + Backward of every layer incl. the "
+                                             "harness's buffer copies; its DifferentiableLut forward runs on the OpenMP threads, its batch-norm backward on one)" % Fs}
+        else:
+            t0 = time.perf_counter()
+            a = oracle.im2col_forward(xs, C, H, W_, Fs, FH, FW); acts = []
+            for l, Wt, idx in zip(layers, Ws, idxs):
+                y, mean, rstd, _, _ = oracle.differentiable_lut_forward_training(6, a, idx, Wt, FWs, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))
+                acts.append((a, mean, rstd)); a = y
+            maps = oracle.col2im_forward(a, CO, OH, OW, Fs)
+            oracle.stochastic_maxpool2x2_forward(maps, CO, OH, OW, Fs)
+            dy = oracle.col2im_backward(oracle.stochastic_maxpool2x2_backward(maps, dps, CO, OH, OW, Fs), CO, OH, OW, Fs)
+            for l, Wt, idx, (a_in, mean, rstd) in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(acts)):
+                dy, _ = oracle.differentiable_lut_backward(6, a_in, dy, idx, Wt, FWs, mean, rstd)
+            oracle.im2col_backward(dy, C, H, W_, Fs, FH, FW)
+            cpu_dt = time.perf_counter() - t0
+            out["cpu_baseline"] = {"value": sum(l["O"] for l in layers) * FWs / cpu_dt / 1e9, "unit": "G node-evals/s", "cores": 1, "kind": "port",
+                                   "sample": "the same block on %d images through the C restatement of the reference's host path (generic DifferentiableLut "
+                                             "algorithm, whose batch-norm backward is single-threaded in the reference too)" % Fs}
     return out
 
 
@@ -533,23 +671,38 @@ def bench_mnist_step(args, lib):
     ops.set_dx_mode(0)
     keep = {}
 
+    # what a caller that keeps a layer's input for the backward pass keeps as well (the model classes do): the packed copy of each
+    # layer's binarized input — the first layer's is packed by its forward call, every other layer's is written by the forward call of
+    # the layer before as its packed output — and the tables derived from W
+    for l in layers:
+        l["packed_in"] = ops.packed_input_buffer(l["I"], F)
+        l["tables"] = ops.prepared_tables_buffer(6, l["O"])
+
+    plain = getattr(args, "plain_signatures", False)
+    clamp_w = None if plain else (0.0, 1.0)
+
     def forward_backward():
         a = x
         acts = []
-        for l in layers:
-            # the model class clamps its table before the first forward pass after a backward pass; the entry does it in its table launch
-            # ... and keeps the packed copy of its binarized input for the backward call
-            packed = ops.packed_input_buffer(a.shape[0], F)
-            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=(0.0, 1.0), packed=packed,
-                                                                    tables=l.setdefault("tables", ops.prepared_tables_buffer(6, l["idx"].shape[0])))
-            acts.append((a, mean, rstd, packed)); a = y
-        out = ops.average_lut_forward(a, idx_avg, F, False, False, mean=False)
-        dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
-        acc, cat = ops.metrics_categorical_accuracy(out, t, CLASSES, 1, F)
-        dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
-        for l, (a_in, mean, rstd, packed) in zip(reversed(layers), reversed(acts)):
+        for k, l in enumerate(layers):
+            # the model class clamps its table before the first forward pass after a backward pass; the entry does it with its tables
+            # (with the reference's plain signatures the clamp is a launch of its own)
+            if plain:
+                ops.vector_clamp_(l["W"], 0.0, 1.0)
+            nxt = layers[k + 1]["packed_in"] if k + 1 < len(layers) else None
+            y, mean, rstd = ops.differentiable_lut_forward_training(6, a, l["idx"], l["W"], F, l["rm"], l["rv"], clamp_w=clamp_w,
+                                                                    packed=l["packed_in"], packed_holds=(k > 0), packed_out=nxt, tables=l["tables"])
+            acts.append((a, mean, rstd)); a = y
+        if plain:
+            out = ops.average_lut_forward(a, idx_avg, F, False, False, mean=False)
+            dy, loss_buf, _ = ops.loss_softmax_cross_entropy(out, t, CLASSES, 1, F, t_sum=float(F))
+            acc, cat = ops.metrics_categorical_accuracy(out, t, CLASSES, 1, F)
+            dy = ops.average_lut_backward(dy, idx_avg, sizes[-1], F)
+        else:       # the same four in one launch
+            out, dy, loss_buf, acc, cat, _ = ops.classifier_tail(a, idx_avg, t, F, t_sum=float(F), mean=False)
+        for l, (a_in, mean, rstd) in zip(reversed(layers), reversed(acts)):
             # dW accumulates; it is zero here because the optimizer's Update() zeroed it after the previous step (Optimizer.h:31-35)
-            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"], packed=packed, tables=l["tables"])
+            dy = ops.differentiable_lut_backward(6, a_in, dy, l["idx"], l["W"], l["dW"], F, mean, rstd, l["rev"], packed=l["packed_in"], tables=l["tables"])
         keep["loss_buf"], keep["acc"] = loss_buf, acc
 
     def timed(fn):
@@ -567,18 +720,30 @@ def bench_mnist_step(args, lib):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps
 
+    def optimizer_update():
+        if plain:               # bbcu_fp32_OptimizerAdam, then the gradients cleared tensor by tensor (Optimizer::Update, include/bb/Optimizer.h:31-35)
+            adam.step()
+            for l in layers:
+                ops.vector_set_(l["dW"], 0.0)
+        else:
+            adam.update()
+
     def eager_step():
-        forward_backward(); adam.update()
+        forward_backward(); optimizer_update()
 
-    dt_eager = timed(eager_step)
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        forward_backward()
+    ops.HINTS = not plain
+    try:
+        dt_eager = timed(eager_step)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            forward_backward()
 
-    def graph_step():
-        graph.replay(); adam.update()
+        def graph_step():
+            graph.replay(); optimizer_update()
 
-    dt_graph = timed(graph_step)
+        dt_graph = timed(graph_step)
+    finally:
+        ops.HINTS = True
     loss = -float(keep["loss_buf"].sum().item()) / F
     node_evals = sum(sizes[1:]) * F
     # every activation, gradient and table once per pass over the three LUT layers
@@ -591,25 +756,47 @@ def bench_mnist_step(args, lib):
                       "ms_per_step_host_launched": dt_eager * 1e3, "ms_per_step_graph_replay": dt_graph * 1e3,
                       "G_node_evals_per_s": node_evals / dt / 1e9, "loss_after_run": loss},
            "roofline": {"bound": "hbm", "kernel": "whole step (launch-bound)", "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "traffic": None if plain else measured_traffic("steps", "mnist_step"),
+                        "traffic_source": traffic_source()}}
     if not args.no_cpu:
         import oracle
         xs = x.cpu().numpy(); ts = t.cpu().numpy()
         Ws = [l["W"].cpu().numpy() for l in layers]; idxs = [l["idx"].cpu().numpy() for l in layers]
-        t0 = time.perf_counter()
-        a = xs; acts = []
-        for l, W, idx in zip(layers, Ws, idxs):
-            y, mean, rstd, _, _ = oracle.differentiable_lut_forward_training(6, a, idx, W, F, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))
-            acts.append((a, mean, rstd)); a = y
-        o = oracle.average_lut_forward(a, idx_avg.cpu().numpy(), F, False, False)
-        dy, _, _ = oracle.loss_softmax_cross_entropy(o, ts, CLASSES, 1, F)
-        dy = oracle.average_lut_backward(dy, idx_avg.cpu().numpy(), sizes[-1], F)
-        for l, W, idx, (a_in, mean, rstd) in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(acts)):
-            dy, _ = oracle.differentiable_lut_backward(6, a_in, dy, idx, W, F, mean, rstd)
-        cpu_dt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": 1.0 / cpu_dt, "unit": "steps/s", "cores": 1, "kind": "port",
-                               "sample": "one forward + backward of the same network through the C restatement of the reference's generic "
-                                         "DifferentiableLut path (its batch-norm backward is single-threaded in the reference too), Adam not included"}
+        threads = min(os.cpu_count() or 1, 16)
+        if oracle.have_ref():
+            # the reference's own classes (oracle/_ref).  Untimed: one forward pass for the activations.  Timed: the tail, then every
+            # layer's Forward + Backward, last layer first, each fed the gradient that the layer behind it returned.
+            os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+            a = np.ascontiguousarray(xs[:, :F]); ins = []
+            for l, W, idx in zip(layers, Ws, idxs):
+                ins.append(a)
+                a = oracle.ref_differentiable_lut(6, a, idx, W, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))["y"]
+            t0 = time.perf_counter()
+            o = oracle.average_lut_forward(a, idx_avg.cpu().numpy(), F, False, False)
+            dy, _, _ = oracle.loss_softmax_cross_entropy(o, np.ascontiguousarray(ts[:, :F]), CLASSES, 1, F)
+            dy = oracle.average_lut_backward(dy, idx_avg.cpu().numpy(), sizes[-1], F)
+            for l, W, idx, a_in in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(ins)):
+                dy = oracle.ref_differentiable_lut(6, a_in, idx, W, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32), dy=dy)["dx"]
+            cpu_dt = time.perf_counter() - t0
+            out["cpu_baseline"] = {"value": 1.0 / cpu_dt, "unit": "steps/s", "cores": threads, "kind": "reference",
+                                   "sample": "Forward + Backward of the three DifferentiableLut6 layers through the reference's own host class (incl. the harness's "
+                                             "buffer copies; its forward runs on the OpenMP threads, its batch-norm backward on one), the 70-node tail through "
+                                             "the C restatement, Adam not included"}
+        else:
+            t0 = time.perf_counter()
+            a = xs; acts = []
+            for l, W, idx in zip(layers, Ws, idxs):
+                y, mean, rstd, _, _ = oracle.differentiable_lut_forward_training(6, a, idx, W, F, np.zeros(l["O"], np.float32), np.ones(l["O"], np.float32))
+                acts.append((a, mean, rstd)); a = y
+            o = oracle.average_lut_forward(a, idx_avg.cpu().numpy(), F, False, False)
+            dy, _, _ = oracle.loss_softmax_cross_entropy(o, ts, CLASSES, 1, F)
+            dy = oracle.average_lut_backward(dy, idx_avg.cpu().numpy(), sizes[-1], F)
+            for l, W, idx, (a_in, mean, rstd) in zip(reversed(layers), reversed(Ws), reversed(idxs), reversed(acts)):
+                dy, _ = oracle.differentiable_lut_backward(6, a_in, dy, idx, W, F, mean, rstd)
+            cpu_dt = time.perf_counter() - t0
+            out["cpu_baseline"] = {"value": 1.0 / cpu_dt, "unit": "steps/s", "cores": 1, "kind": "port",
+                                   "sample": "one forward + backward of the same network through the C restatement of the reference's generic "
+                                             "DifferentiableLut path (its batch-norm backward is single-threaded in the reference too), Adam not included"}
     return out
 
 
@@ -652,7 +839,7 @@ def bench_binarylut6(args, lib):
            "config": {"workload": "BinaryLut6 packed inference, 8192 in x 16384 out x 262144 frames", "frame_stride_words": SW},
            "roofline": {"bound": "hbm", "kernel": "binary_lut6_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": gbs / HBM_PEAK_GBS,
-                        "traffic": MEASURED_TRAFFIC_BYTES.get(("binary_lut6_kernel", 0))}}
+                        "traffic": measured_traffic("kernels", "binarylut6/binary_lut6_kernel"), "traffic_source": traffic_source()}}
     if args.profile_copy:
         for _ in range(3):
             y[:I].copy_(x)
@@ -783,7 +970,8 @@ def bench_stochasticlut6(args, lib):
         "hbm_frac_step": (fwd_b + bwd_b) / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": dk["frac"],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((dominant, args.dx_mode))},
+                     "traffic": measured_traffic("kernels", "stochasticlut6/" + dominant.split("<")[0]) if args.dx_mode == 0 else None,
+                     "traffic_source": traffic_source()},
         "kernels": kernels,
     }
     if args.profile_copy:
@@ -916,9 +1104,27 @@ def other_configs(args, lib):
                                ("cfg5_conv_block", bench_conv_block, "conv_block"),
                                ("dx_gather_ceiling", bench_gather_ceiling, "gather_ceiling")):
         sub.workload = workload
+        sub.plain_signatures = False
         r = fn(sub, lib)
         out[name] = {k: r[k] for k in keep if k in r}
+        if name in ("cfg3_mnist_step", "cfg5_conv_block"):
+            out[name]["ms_per_step_without_hints"] = without_hints(fn, sub, lib)
+    sub.workload = "differentiablelut6"
+    sub.plain_signatures = False
+    r = bench_differentiablelut6(sub, lib)
+    out["differentiablelut6_4096x4096x8192"] = {k: r[k] for k in keep if k in r}
+    out["differentiablelut6_4096x4096x8192"]["ms_per_step_without_hints"] = without_hints(bench_differentiablelut6, sub, lib)
     return out
+
+
+def without_hints(fn, args, lib):
+    """ms per step of the same workload called as the reference's own classes would call it through include/bbcu_hip_binding.h: the
+    reference's signatures only (no bbhip_Hint* call, no entry that folds the table clamp or the gradient clear into another launch)"""
+    import copy
+    sub = copy.copy(args)
+    sub.plain_signatures = True
+    sub.no_cpu = True
+    return fn(sub, lib)["ms_per_step"]
 
 
 def main():
@@ -945,7 +1151,15 @@ def main():
                              "forward_784x1024x64", "gather_ceiling"],
                     help="stochasticlut6 (default, the headline metric) or binarylut6 (packed inference, 8192 -> 16384 nodes, 262144 frames)")
     ap.add_argument("--cpu-frames", type=int, default=8192)
+    ap.add_argument("--plain-signatures", action="store_true",
+                    help="workloads differentiablelut6, mnist_step, conv_block: call the library as the reference's own classes would through "
+                         "include/bbcu_hip_binding.h — no bbhip_Hint* call, table clamp and gradient clear as launches of their own")
+    ap.add_argument("--write-traffic", metavar="DIR", default=None,
+                    help="no benchmark: read the rocprofv3 counter runs under DIR (made by the commands in TRAFFIC_COMMANDS) and write profiles/traffic.json")
     args = ap.parse_args()
+    if args.write_traffic:
+        write_traffic(args.write_traffic)
+        return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path would shard over the "
               "frame axis; no multi-GPU code is built)" % args.gpus, file=sys.stderr)

@@ -38,6 +38,8 @@ _SIGNATURES = {
     "bbhip_HintInputNodeSize": (None, [_i]),
     "bbhip_PackedRowWords": (C.c_int, [_i]),
     "bbhip_HintPackedInput": (None, [_vp, _i, _i, _i]),
+    "bbhip_HintPackedOutput": (None, [_vp, _i, _i]),
+    "bbhip_HintTableGradientOverwrite": (None, [_i]),
     "bbhip_HintPreparedTables": (None, [_vp, C.c_size_t, _i]),
     "bbhip_PreparedTablesBytes": (C.c_size_t, [_i, _i]),
     "bbhip_GetDxMode": (C.c_int, []),
@@ -66,6 +68,7 @@ _SIGNATURES = {
     "bbhip_fp32_AverageLut_ForwardSum": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_bit_AverageLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_AverageLut_Backward": (C.c_int, [_vp, _vp, _vp] + [_i] * 5 + [_vp]),
+    "bbhip_fp32_ClassifierTail_ForwardBackward": (C.c_int, [_vp] * 9 + [_f] + [_i] * 7 + [_vp]),
     "bbhip_fp32_MaxLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 6 + [_vp]),
     "bbhip_bit_MaxLut_Forward": (C.c_int, [_vp, _vp, _vp] + [_i] * 4 + [_vp]),
     "bbhip_fp32_MaxLut_Backward": (C.c_int, [_vp, _vp, _vp, _vp] + [_i] * 6 + [_vp]),

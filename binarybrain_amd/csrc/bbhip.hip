@@ -72,9 +72,16 @@ thread_local PackedInputHint g_packed_hint = {nullptr, 0, 0, 0};
 // bbhip_HintPreparedTables: a caller-owned place for the tables that a LUT call derives from W (centred coefficients, corner values)
 struct PreparedTablesHint { float *buf; size_t bytes; int holds_tables; };
 thread_local PreparedTablesHint g_tables_hint = {nullptr, 0, 0};
+// bbhip_HintPackedOutput: a caller-owned buffer that receives the binarized output of the next forward call as packed bits
+struct PackedOutputHint { uint32_t *bits; int rows, row_words; };
+thread_local PackedOutputHint g_packed_out_hint = {nullptr, 0, 0};
+// bbhip_HintTableGradientOverwrite: the next backward call writes dW instead of adding to it
+thread_local int g_dw_overwrite_hint = 0;
 static inline void clear_hints(void)
 {
+    g_dw_overwrite_hint = 0;
     g_input_node_hint = 0; g_packed_hint = PackedInputHint{nullptr, 0, 0, 0}; g_tables_hint = PreparedTablesHint{nullptr, 0, 0};
+    g_packed_out_hint = PackedOutputHint{nullptr, 0, 0};
 }
 static inline bool tables_fit(PreparedTablesHint const &t, size_t bytes)
 {
@@ -134,6 +141,8 @@ bool use_corner_values(int xmode)
 }
 
 bool pack_binarized_input(void) { static bool const on = env_switch("BBHIP_PACK", true); return on; }
+// the corner-value forward kernel derives a node's tables in the wavefront where no packing launch carries the preparation (0 = a table launch)
+bool inline_tables(void) { static bool const on = env_switch("BBHIP_INLINE_TABLES", true); return on; }
 // packed rows in the dx kernel read with one scalar load per row and pass where pitch and alignment allow (0 = vector loads + read-lanes)
 bool dx_wide_rows(void) { static bool const on = env_switch("BBHIP_DX_WIDE", true); return on; }
 int dx_wide_max_rows(void) { static int const v = env_int("BBHIP_DX_WIDE_ROWS", 1024); return v; }
@@ -427,18 +436,23 @@ int launch_pack_and_prep(float const *x, int x_stride, uint32_t *bits, int bit_s
 
 template <int N>
 int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch const *fixed = nullptr,
-                PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0}, PreparedTablesHint tables = PreparedTablesHint{nullptr, 0, 0})
+                PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0}, PreparedTablesHint tables = PreparedTablesHint{nullptr, 0, 0},
+                PackedOutputHint packed_out = PackedOutputHint{nullptr, 0, 0})
 {
     constexpr int NN = 1 << N;
     // input_rows: what the caller said about the input's row count (bbhip_HintInputNodeSize), 0 = nothing.
     // fp32 frames that the layer binarizes at 0.5 are packed to bits once where the row count is known; from here on the
     // call is a packed-bit call (same outputs)
     ForwardCall c = call;
-    bool const pack = (c.xmode == kXBinary) && input_rows > 0 && use_corner_values(kXBinary) && pack_binarized_input();
+    bool const bits_wanted = (c.xmode == kXBinary) && input_rows > 0 && use_corner_values(kXBinary) && pack_binarized_input();
     // the packed copy goes to the caller's buffer where one was offered and fits (rows of whole 32-byte groups), else to the arena
-    bool const to_caller = pack && packed.bits != nullptr && packed.rows == input_rows && packed.row_words >= (c.frame_size + 31) / 32 &&
+    bool const to_caller = bits_wanted && packed.bits != nullptr && packed.rows == input_rows && packed.row_words >= (c.frame_size + 31) / 32 &&
                            packed.row_words % 8 == 0 && (reinterpret_cast<uintptr_t>(packed.bits) & 31u) == 0;
-    if (pack) { c.xmode = kXBit; c.x_stride = to_caller ? packed.row_words : packed_row_words(c.frame_size); c.x = nullptr; }
+    // ... unless the caller says that the buffer already holds the packed copy of this input (the packed output of the layer
+    // before, or of an earlier call on the same input): nothing to pack
+    bool const have_bits = to_caller && packed.holds_input;
+    bool const pack = bits_wanted && !have_bits;
+    if (bits_wanted) { c.xmode = kXBit; c.x_stride = to_caller ? packed.row_words : packed_row_words(c.frame_size); c.x = have_bits ? packed.bits : nullptr; }
     bool const corner     = use_corner_values(c.xmode);
     int const npw         = corner ? 1 : fwd_nodes_per_wave();
     int const tile_count  = ceil_div(c.node_size, kWavesPerBlk * npw);
@@ -474,13 +488,20 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     // plain output of a call with one unit per node on the polynomial kernel: the wavefronts prepare their node's table
     // themselves (FwdArgs::W_inline) and the table launch falls away
     bool const inline_table = (c.bn == 0) && !corner && chunk_count == 1 && LutMatrixQ<N>::kUsable && c.clamp_W == nullptr && !tables_to_caller;
-    if (!pack && !inline_table) {
+    // the corner-value kernel derives a node's tables in the wavefront in any case where no packing launch is there to carry the
+    // preparation: the first launch of the call does it and stores them for the launches (and the backward call) that follow
+    bool const inline_corner = corner && !pack && inline_tables();
+    if (!pack && !inline_table && !inline_corner) {
         launch_table_prep<N>(c.W, C, c.node_size, c.lut_binarize, st, V, c.bias, c.clamp_W, c.clamp_lo, c.clamp_hi);
         BBHIP_LAUNCH_CHECK();
     }
 
     FwdArgs a{};
     if (inline_table) { a.W_inline = c.W; a.lut_binarize = c.lut_binarize; }
+    if (inline_corner) {
+        a.W_inline = c.W; a.lut_binarize = c.lut_binarize; a.C_out = C; a.V_out = V;
+        a.clamp_W = c.clamp_W; a.clamp_lo = c.clamp_lo; a.clamp_hi = c.clamp_hi;
+    }
     a.x = c.x; a.y = c.y; a.idx = c.idx; a.C = C; a.V = V;
     a.node_size = c.node_size; a.frame_size = c.frame_size;
     a.x_stride = c.x_stride; a.y_stride = c.y_stride;
@@ -499,6 +520,7 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
         a.stat_partial = stat;
         if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
+        if (inline_corner) { a.W_inline = nullptr; a.C_out = nullptr; a.V_out = nullptr; a.clamp_W = nullptr; }      // stored by that launch
         if (chunk_count <= kInlineStatUnits) {
             // few units: every wavefront of the output pass adds up the partial sums of its node itself, and the wavefront of a
             // node's first unit stores the statistics; a launch that does it once per node would cost more than that
@@ -519,6 +541,11 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
         a.stat_mode = kStatRunning; a.mean = c.running_mean; a.rstd = c.running_var;       // rstd = 1 / sqrt(var) in the kernel
         kind = 1;
     }
+    // the binarized fp32 output as packed bits as well, where the caller offered a buffer that fits (rows of whole 32-byte groups)
+    if (c.ymode == kYBinarize && packed_out.bits != nullptr && packed_out.rows == c.node_size && packed_out.row_words >= (c.frame_size + 31) / 32 &&
+        packed_out.row_words % 8 == 0 && (reinterpret_cast<uintptr_t>(packed_out.bits) & 31u) == 0) {
+        a.y_bits = packed_out.bits; a.y_bits_stride = packed_out.row_words;
+    }
     {
         ScopedTimer tm(kTimeForward, st, fixed == nullptr);     // (event creation may allocate: not on the path that must not)
         if (dispatch_forward<N>(c.xmode, c.ymode, kind, a, npw, st)) { return 1; }
@@ -533,10 +560,11 @@ int forward_entry(ForwardCall const &c, void *stream, Scratch const *fixed = nul
     PackedInputHint const packed = fixed ? PackedInputHint{nullptr, 0, 0, 0} : g_packed_hint;
     int const input_rows = fixed ? 0 : (packed.bits ? packed.rows : g_input_node_hint);
     PreparedTablesHint const tables = fixed ? PreparedTablesHint{nullptr, 0, 0} : g_tables_hint;
+    PackedOutputHint const packed_out = fixed ? PackedOutputHint{nullptr, 0, 0} : g_packed_out_hint;
     clear_hints();
     if (check_forward(c)) { return 1; }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed, packed, tables));
+    BBHIP_SWITCH_N(c.n, return run_forward<N>(c, input_rows, st, fixed, packed, tables, packed_out));
     return 0;
 }
 
@@ -580,7 +608,7 @@ int check_backward(BackwardCall const &c, int dxmode)
 
 template <int N>
 int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packed = PackedInputHint{nullptr, 0, 0, 0},
-                 PreparedTablesHint tables = PreparedTablesHint{nullptr, 0, 0})
+                 PreparedTablesHint tables = PreparedTablesHint{nullptr, 0, 0}, int dw_overwrite = 0)
 {
     constexpr int NN = 1 << N;
     int dxmode = (g_dx_mode == 1) ? kDxAtomic : (g_dx_mode == 2) ? kDxTmp : kDxNone;
@@ -788,6 +816,7 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
                           (reinterpret_cast<uintptr_t>(c.x) % 32u) == 0;
         // folding the slab sums into dW rides at the end of this launch
         d.fin_partial = part; d.fin_dW = c.dW; d.fin_node_size = c.output_node_size; d.fin_slab_count = slab_total;
+        d.fin_overwrite = dw_overwrite;
         d.fin_blocks = (ceil_div(c.output_node_size * NN, kBlock) + 7) & ~7;
         if ((long long)d.fin_blocks + (long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
         {
@@ -803,7 +832,7 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
     }
 
     int const total = c.output_node_size * NN;
-    hipLaunchKernelGGL(dw_finalize_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, part, c.dW, c.output_node_size, slab_total);
+    hipLaunchKernelGGL(dw_finalize_kernel<N>, dim3(ceil_div(total, kBlock)), dim3(kBlock), 0, st, part, c.dW, c.output_node_size, slab_total, dw_overwrite);
     BBHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -812,9 +841,10 @@ int backward_entry(BackwardCall const &c, void *stream)
 {
     PackedInputHint const packed = g_packed_hint;
     PreparedTablesHint const tables = g_tables_hint;
+    int const dw_overwrite = g_dw_overwrite_hint;
     clear_hints();                                  // hints are for the next LUT call only
     hipStream_t st = static_cast<hipStream_t>(stream);
-    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st, packed, tables));
+    BBHIP_SWITCH_N(c.n, return run_backward<N>(c, st, packed, tables, dw_overwrite));
     return 0;
 }
 
@@ -1067,6 +1097,7 @@ int bbhip_GetSwitch(char const *name)
     if (!strcmp(name, "corner")) { return use_corner_values(kXBit) ? 1 : 0; }
     if (!strcmp(name, "pack"))   { return pack_binarized_input() ? 1 : 0; }
     if (!strcmp(name, "dx_wide")) { return dx_wide_rows() ? 1 : 0; }
+    if (!strcmp(name, "inline_tables")) { return inline_tables() ? 1 : 0; }
     return -1;
 }
 
@@ -1082,6 +1113,14 @@ size_t bbhip_PreparedTablesBytes(int n, int node_size)
 {
     if (n < 2 || n > 6 || node_size <= 0) { return 0; }
     return 2 * align256((size_t)node_size * ((size_t)1 << n) * sizeof(float));
+}
+
+void bbhip_HintTableGradientOverwrite(int overwrite) { g_dw_overwrite_hint = overwrite != 0; }
+
+void bbhip_HintPackedOutput(int *dev_bits, int rows, int row_words)
+{
+    g_packed_out_hint = (dev_bits != nullptr && rows > 0 && row_words > 0) ? PackedOutputHint{reinterpret_cast<uint32_t *>(dev_bits), rows, row_words}
+                                                                           : PackedOutputHint{nullptr, 0, 0};
 }
 
 void bbhip_HintPackedInput(int *dev_bits, int rows, int row_words, int holds_input)
@@ -1708,6 +1747,32 @@ int bbhip_fp32_LossSoftmaxCrossEntropy(float const *dev_y_buf, float const *dev_
         hipLaunchKernelGGL(loss_pixel_sum_kernel, dim3((unsigned)f_blocks), dim3(kTailBlock), 0, st, partial, dev_loss_buf, pix_size, frame_size);
         BBHIP_LAUNCH_CHECK();
     }
+    return 0;
+}
+
+int bbhip_fp32_ClassifierTail_ForwardBackward(float const *dev_x_buf, float *dev_y_buf, float *dev_dx_buf, int const *dev_input_index,
+                                              float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, int *dev_accuracy_buf,
+                                              int *dev_category_buf, float t_sum, int n, int input_node_size, int ch_size, int frame_size,
+                                              int frame_stride, int binarize_input, int output_sum, void *stream)
+{
+    clear_hints();
+    if (!(dev_x_buf && dev_dx_buf && dev_input_index && dev_t_buf && dev_loss_buf)) { return fail("%s: null buffer", __func__); }
+    if (!(n > 0 && input_node_size > 0 && ch_size > 0 && frame_size > 0)) { return fail("%s: sizes must be positive", __func__); }
+    if (frame_stride < frame_size) { return fail("%s: frame stride shorter than the frames", __func__); }
+    if (ch_size > 16) { return fail("%s: at most 16 classes (ch_size=%d): call the four entries one by one", __func__, ch_size); }
+    if ((long long)ch_size * n > 0x7fffffffLL) { return fail("%s: connection table too large", __func__); }
+    // per-input sums, logits and gradients of 64 frames, then the table: within 64 KiB of LDS
+    size_t const lds = ((size_t)input_node_size + 2 * 16) * 64 * sizeof(float) + (((size_t)ch_size * n + 3) & ~(size_t)3) * sizeof(int);
+    if (lds > 64u * 1024u) {
+        return fail("%s: input_node_size=%d nodes and ch_size*n=%d table entries need %zu bytes of LDS, 65536 are there (192 nodes with 2048 entries, "
+                    "216 with 512): call the four entries one by one", __func__, input_node_size, ch_size * n, lds);
+    }
+    hipStream_t const st = static_cast<hipStream_t>(stream);
+    ScopedTimer tm(kTimeOther, st);
+    hipLaunchKernelGGL(classifier_tail_kernel<16>, dim3((unsigned)ceil_div(frame_stride, 64)), dim3(64 * kClassifierTailWaves), lds, st, dev_x_buf, dev_y_buf, dev_dx_buf,
+                       dev_input_index, dev_t_buf, dev_dy_buf, dev_loss_buf, dev_accuracy_buf, dev_category_buf, t_sum,
+                       output_sum ? 1.0f : 1.0f / (float)n, n, input_node_size, ch_size, frame_size, frame_stride, binarize_input);
+    BBHIP_LAUNCH_CHECK();
     return 0;
 }
 

@@ -47,6 +47,30 @@ __device__ __forceinline__ float wave_sum(float v)
 //  clamp_W != nullptr: the table is first clamped to [clamp_lo, clamp_hi] and written back there (the model classes clamp
 //  their table in place before every forward pass, include/bb/StochasticLutN.h:451; folded in here the clamp costs no
 //  launch of its own).  clamp_W is W itself, so neither pointer is declared unaliased.
+// entry i of a table held by 2^N neighbouring lanes: W' -> centred coefficients, (a, b) -> ((a + b) / 2, b - a) per index bit ...
+template <int N>
+__device__ __forceinline__ float centred_butterfly(float v, int i)
+{
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float const o = __shfl_xor(v, 1 << j, 64);
+        v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f;
+    }
+    return v;
+}
+
+// ... and centred coefficients -> corner values, (a, b) -> (a - bias b, a + bias b) per index bit
+template <int N>
+__device__ __forceinline__ float corner_butterfly(float v, int i, float bias)
+{
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float const o = __shfl_xor(v, 1 << j, 64);
+        v = ((i >> j) & 1) ? __builtin_fmaf(bias, v, o) : __builtin_fmaf(-bias, o, v);
+    }
+    return v;
+}
+
 template <int N>
 __device__ __forceinline__ void table_prep_block(float const *W, float *__restrict__ C, int node_size, int lut_binarize,
                                                  float *__restrict__ V, float bias, int block,
@@ -66,18 +90,10 @@ __device__ __forceinline__ void table_prep_block(float const *W, float *__restri
         if (lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
     }
     int const i = t & (NN - 1);
-#pragma unroll
-    for (int j = 0; j < N; ++j) {
-        float const o = __shfl_xor(v, 1 << j, 64);
-        v = ((i >> j) & 1) ? (v - o) : (v + o) * 0.5f;
-    }
+    v = centred_butterfly<N>(v, i);
     if (t < total) { C[t] = v; }
     if (V == nullptr) { return; }           // same for every thread of the launch
-#pragma unroll
-    for (int j = 0; j < N; ++j) {
-        float const o = __shfl_xor(v, 1 << j, 64);
-        v = ((i >> j) & 1) ? __builtin_fmaf(bias, v, o) : __builtin_fmaf(-bias, o, v);
-    }
+    v = corner_butterfly<N>(v, i, bias);
     if (t < total) { V[t] = v; }
 }
 
@@ -90,9 +106,10 @@ __global__ __launch_bounds__(kBlock) void table_prep_kernel(float const *W, floa
     table_prep_block<N>(W, C, node_size, lut_binarize, V, bias, blockIdx.x, clamp_W, clamp_lo, clamp_hi);
 }
 
-// dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order)
+// dW[node][i] += (T^T sum_s partial[s][node])[i]   (T = the butterfly above; deterministic slab order); overwrite: = instead of +=
 template <int N>
-__device__ __forceinline__ void dw_finalize_block(float const *__restrict__ partial, float *__restrict__ dW, int node_size, int slab_count, int block)
+__device__ __forceinline__ void dw_finalize_block(float const *__restrict__ partial, float *__restrict__ dW, int node_size, int slab_count, int block,
+                                                  int overwrite = 0)
 {
     constexpr int NN = 1 << N;
     int const t = block * kBlock + threadIdx.x;
@@ -108,14 +125,14 @@ __device__ __forceinline__ void dw_finalize_block(float const *__restrict__ part
         float const o = __shfl_xor(v, 1 << j, 64);
         v = ((i >> j) & 1) ? (o * 0.5f + v) : (v * 0.5f - o);
     }
-    if (t < total) { dW[t] += v; }
+    if (t < total) { dW[t] = overwrite ? v : dW[t] + v; }
 }
 
 template <int N>
 __global__ __launch_bounds__(kBlock) void dw_finalize_kernel(float const *__restrict__ partial, float *__restrict__ dW,
-                                                            int node_size, int slab_count)
+                                                            int node_size, int slab_count, int overwrite)
 {
-    dw_finalize_block<N>(partial, dW, node_size, slab_count, blockIdx.x);
+    dw_finalize_block<N>(partial, dW, node_size, slab_count, blockIdx.x, overwrite);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -185,7 +202,7 @@ struct FwdArgs {
     float const *V;             // [O][2^N] corner values (two-valued inputs: lut_forward_corner_kernel)
     float const *mean;          // BN: per node (nullptr otherwise)
     float const *rstd;
-    float       *stat_partial;  // STATS: [chunk][O][2] partial sums of (v - C0), (v - C0)^2;  kind 3: of g, g (v - mean)
+    float       *stat_partial;  // STATS: [O][chunk][2] partial sums of (v - C0), (v - C0)^2;  kind 3: of g, g (v - mean)
     float const *dy;            // kind 3: [O][dy_stride]
     int   dy_stride;
     int   node_size, frame_size;
@@ -204,18 +221,29 @@ struct FwdArgs {
     // butterfly of table_prep_block over the lanes.  A call of a few hundred frames is two launches' worth of latency, not work.
     float const *W_inline;
     int   lut_binarize;
+    // lut_forward_corner_kernel with W_inline: the node's tables go to C_out / V_out as well (the wavefront of the node's first unit
+    // stores them: for a later launch of the same call, and for the caller that keeps them for the backward pass), and the table is
+    // first clamped to [clamp_lo, clamp_hi] and written back where clamp_W (W itself) is given — all as table_prep_block does
+    float *C_out, *V_out;
+    float *clamp_W;  float clamp_lo, clamp_hi;
+    // Not null (binarized fp32 output): the binarized output also goes here as packed bits, rows of y_bits_stride words — the packed
+    // copy that the next layer would otherwise make of y before it reads it
+    uint32_t *y_bits;
+    int   y_bits_stride;
 };
 
 // kStatInline: the call has one unit per node, so the wavefront that writes a node's output first sums the node's statistics
 // itself (a pass of its own over the unit) instead of reading them from a statistics launch
 enum StatMode : int { kStatGiven = 0, kStatRunning = 1, kStatPartial = 2, kStatInline = 3 };
-constexpr int kInlineStatUnits = kWave;     // most units whose partial sums a wavefront adds up itself: one load per lane
+constexpr int kInlineStatUnits = 4 * kWave; // most units whose partial sums a wavefront adds up itself: up to four loads per lane
 
 // What a forward kernel does with the LUT output v of (node, frame f = f0 + lane): accumulate statistics (kinds 2, 3) or
 // apply the batch-norm output stage (kind 1) and store.  ok: the frame belongs to the unit; live: the node exists.
+// bits_mask (binarized fp32 output with a packed copy): where given, the lane mask of the step's binarized output is handed back
+// instead of stored, and the caller stores the words of several steps together.
 template <int YMODE, int FWD_KIND>
 __device__ __forceinline__ void forward_stage(FwdArgs const &a, float v, bool ok, bool live, int lane, int node, int f0, int f, int f_end,
-                                              float mean, float rstd, float c0, float dyv, float &s1, float &s2)
+                                              float mean, float rstd, float c0, float dyv, float &s1, float &s2, uint64_t *bits_mask = nullptr)
 {
     if (FWD_KIND == 2) {
         float const d = ok ? (v - c0) : 0.0f;
@@ -243,10 +271,29 @@ __device__ __forceinline__ void forward_stage(FwdArgs const &a, float v, bool ok
         if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
     }
     else {
-        if (YMODE == kYBinarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
-        else                     { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+        if (YMODE == kYBinarize) {
+            if (a.y_bits != nullptr) {                // wave-uniform
+                uint64_t const m = __ballot(ok && (v > 0.5f));
+                if (bits_mask != nullptr) { *bits_mask = m; }
+                else {
+                    uint32_t *yr = a.y_bits + (size_t)node * a.y_bits_stride + (f0 >> 5);
+                    if (lane == 0)                          { yr[0] = (uint32_t)m; }
+                    if (lane == 32 && (f0 + 32) < f_end)    { yr[1] = (uint32_t)(m >> 32); }
+                }
+            }
+            v = (v > 0.5f) ? 1.0f : 0.0f;
+        }
+        else { v = __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
         if (ok) { __builtin_nontemporal_store(v, reinterpret_cast<float *>(a.y) + (size_t)node * a.y_stride + f); }
     }
+}
+
+// Packed copy of the output: the words of a node's row behind its last frame are written as 0 by the wavefront of the node's last
+// unit (the words of the frames themselves are whole: bits past the last frame are 0 in the ballot), as the packing kernels leave them.
+__device__ __forceinline__ void zero_packed_tail(FwdArgs const &a, int ck, int node, bool live, int lane)
+{
+    if (a.y_bits == nullptr || ck != a.chunk_count - 1 || !live) { return; }
+    for (int w = ((a.frame_size + 31) >> 5) + lane; w < a.y_bits_stride; w += kWave) { a.y_bits[(size_t)node * a.y_bits_stride + w] = 0u; }
 }
 
 // per (unit, node) partial sums of the statistics kinds
@@ -254,20 +301,32 @@ __device__ __forceinline__ void forward_store_stats(FwdArgs const &a, int ck, in
 {
     float const t1 = wave_sum(s1), t2 = wave_sum(s2);
     if (lane == 0 && live) {
-        float *q = a.stat_partial + ((size_t)ck * a.node_size + node) * 2;
+        float *q = a.stat_partial + ((size_t)node * a.chunk_count + ck) * 2;     // a node's units side by side: who adds them up reads a contiguous run
         q[0] = t1;
         q[1] = t2;
     }
 }
 
-// Sum of the per-unit partial sums [count][node_size][2] of one node by one wavefront, count <= kInlineStatUnits: lane l
-// holds unit l and wave_sum adds the lanes, a fixed order: every wavefront that sums a node gets the same bits.  With few
-// units this costs a wavefront one load and a dozen cross-lane steps, less than the launch that would do it once per node.
+// Sum of the per-unit partial sums [node_size][count][2] of one node by one wavefront, count <= kInlineStatUnits: lane l
+// adds units l, l + 64, l + 128, l + 192 in that order and wave_sum adds the lanes, a fixed order: every wavefront that sums a node
+// gets the same bits.  This costs a wavefront a few loads and a dozen cross-lane steps, less than the launch that would do it once per node.
 __device__ __forceinline__ void wave_stat_sums(float const *__restrict__ stat_partial, int node_size, int count, int node, int lane,
                                                float &s1, float &s2)
 {
     float2 v = make_float2(0.0f, 0.0f);
-    if (lane < count) { v = *reinterpret_cast<float2 const *>(stat_partial + ((size_t)lane * node_size + node) * 2); }
+    if (count <= kWave) {
+        if (lane < count) { v = *reinterpret_cast<float2 const *>(stat_partial + ((size_t)node * count + lane) * 2); }
+    }
+    else {
+        float2 p[kInlineStatUnits / kWave];
+#pragma unroll
+        for (int q = 0; q < kInlineStatUnits / kWave; ++q) {
+            int const u = lane + q * kWave;
+            p[q] = (u < count) ? *reinterpret_cast<float2 const *>(stat_partial + ((size_t)node * count + u) * 2) : make_float2(0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int q = 0; q < kInlineStatUnits / kWave; ++q) { v.x += p[q].x; v.y += p[q].y; }
+    }
     s1 = wave_sum(v.x);
     s2 = wave_sum(v.y);
 }
@@ -440,6 +499,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
         for (int p = 0; p < NPW; ++p) { forward_store_statistics(a, node[p], live[p], ck, lane, mean[p], var[p], rstd[p]); }
     }
+    if (YMODE == kYBinarize && (FWD_KIND == 0 || FWD_KIND == 1)) {
+#pragma unroll
+        for (int p = 0; p < NPW; ++p) { zero_packed_tail(a, ck, node[p], live[p], lane); }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -493,6 +556,8 @@ __device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(
                 if (KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
             }
         }
+        constexpr bool kPackedCopy = (YMODE == kYBinarize) && (KIND == 0 || KIND == 1);
+        uint32_t words = 0;                                  // lane l < 2 U: word l of the pass's packed output
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             int const f0 = fb + u * kWave;
@@ -501,8 +566,17 @@ __device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(
             bool const ok = f < f_end;
             uint32_t const index = corner_index<N, XMODE>(raw[u]);
             float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), corner));
+            uint64_t m = 0;
             forward_stage<YMODE, KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
-                                       (KIND == 3) ? dyv[u] : 0.0f, s1, s2);
+                                       (KIND == 3) ? dyv[u] : 0.0f, s1, s2, kPackedCopy ? &m : nullptr);
+            if (kPackedCopy) {
+                asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)m), "n"(2 * u));               // words[lane 2u] = low half
+                asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)(m >> 32)), "n"(2 * u + 1));
+            }
+        }
+        // the packed copy of the pass: its 2 U words by one store (a store per step would double the kernel's store instructions)
+        if (kPackedCopy && a.y_bits != nullptr && lane < 2 * U && fb + 32 * lane < f_end) {
+            a.y_bits[(size_t)node * a.y_bits_stride + (fb >> 5) + lane] = words;
         }
     }
 }
@@ -530,7 +604,28 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
 
-    int const corner = __float_as_int(a.V[(size_t)node * NN + (lane & (NN - 1))]);      // lane p holds V[p]
+    int corner;                                                                         // lane p holds V[p]
+    float c0 = 0.0f, table_c = 0.0f, table_w = 0.0f;
+    bool clamp_store = false;
+    if (a.W_inline != nullptr) {
+        // no table launch has run: the wavefront derives its node's tables itself, as table_prep_block would (same operations on
+        // the same values: same bits), and the wavefront of the node's first unit stores what later launches and the caller read
+        int const i = lane & (NN - 1);
+        float w = a.W_inline[(size_t)node * NN + i];
+        if (a.clamp_W != nullptr) {
+            float const wc = fminf(a.clamp_hi, fmaxf(a.clamp_lo, w));
+            clamp_store = (ck == 0) && (lane < NN) && (wc != w);
+            w = wc;
+        }
+        table_w = w;
+        if (a.lut_binarize) { w = (w > 0.5f) ? 1.0f : 0.0f; }
+        float const c = centred_butterfly<N>(w, i);
+        float const v = corner_butterfly<N>(c, i, a.bias);
+        table_c = c;                                        // stored at the end of the kernel: a store ahead of the unit's loads would be waited for with them
+        c0 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(c)));
+        corner = __float_as_int(v);
+    }
+    else { corner = __float_as_int(a.V[(size_t)node * NN + (lane & (NN - 1))]); }
     void const *rows[N];
 #pragma unroll
     for (int k = 0; k < N; ++k) {
@@ -538,8 +633,10 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
         rows[k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
                                    : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
     }
-    float mean = 0.0f, rstd = 1.0f, c0 = 0.0f;
-    if (FWD_KIND == 2 || (FWD_KIND == 1 && (a.stat_mode == kStatPartial || a.stat_mode == kStatInline))) { c0 = a.C[(size_t)node * NN]; }
+    float mean = 0.0f, rstd = 1.0f;
+    if (a.W_inline == nullptr && (FWD_KIND == 2 || (FWD_KIND == 1 && (a.stat_mode == kStatPartial || a.stat_mode == kStatInline)))) {
+        c0 = a.C[(size_t)node * NN];
+    }
     float var = 0.0f;
 
     int const f_begin = ck * a.chunk;
@@ -565,12 +662,18 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
     corner_unit_pass<N, XMODE, YMODE, FWD_KIND, WIDE>(a, rows, corner, node, lane, f_begin, f_end, f_last, mean, rstd, c0, s1, s2);
     if (FWD_KIND == 2 || FWD_KIND == 3) { forward_store_stats(a, ck, node, true, lane, s1, s2); }
     if (FWD_KIND == 1) { forward_store_statistics(a, node, true, ck, lane, mean, var, rstd); }
+    if (YMODE == kYBinarize && (FWD_KIND == 0 || FWD_KIND == 1)) { zero_packed_tail(a, ck, node, true, lane); }
+    if (a.W_inline != nullptr && ck == 0 && lane < NN) {
+        if (clamp_store)         { a.clamp_W[(size_t)node * NN + lane] = table_w; }
+        if (a.C_out != nullptr)  { a.C_out[(size_t)node * NN + lane] = table_c; }
+        if (a.V_out != nullptr)  { a.V_out[(size_t)node * NN + lane] = __int_as_float(corner); }
+    }
 }
 
-// Sum of the per-unit partial sums [count][node_size][2] of one node.  A workgroup owns nodes_per_block consecutive nodes
+// Sum of the per-unit partial sums [node_size][count][2] of one node.  A workgroup owns nodes_per_block consecutive nodes
 // (a power of two up to kBlock) and splits the units over its kBlock / nodes_per_block thread groups: group g adds units
 // g, g + G, ... in ascending order and the groups are added in ascending order through LDS — a fixed order, so the result
-// does not depend on the launch.  Consecutive threads of a group read consecutive nodes (8 bytes each).  Returns true in
+// does not depend on the launch.  Returns true in
 // the one thread per node that holds the sums.
 __device__ __forceinline__ bool sum_stat_partials(float const *__restrict__ stat_partial, int node_size, int count,
                                                   int nodes_per_block, int &node, float &s1, float &s2)
@@ -582,7 +685,7 @@ __device__ __forceinline__ bool sum_stat_partials(float const *__restrict__ stat
     if (node < node_size) {
 #pragma unroll 4
         for (int c = g; c < count; c += groups) {
-            float2 const v = *reinterpret_cast<float2 const *>(stat_partial + ((size_t)c * node_size + node) * 2);
+            float2 const v = *reinterpret_cast<float2 const *>(stat_partial + ((size_t)node * count + c) * 2);
             a += v.x;
             b += v.y;
         }
@@ -965,6 +1068,7 @@ struct DxArgs {
     float const *fin_partial;
     float       *fin_dW;
     int   fin_node_size, fin_slab_count, fin_blocks;
+    int   fin_overwrite;        // dW = instead of dW += (the caller's dW holds nothing: bbhip_HintTableGradientOverwrite)
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -1130,7 +1234,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_kernel(DxArgs a)
     // the end of this launch instead of taking a launch of its own
     int const bid = blockIdx.x;
     int const B   = a.chunk_count * a.tiles.count;
-    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B); return; }
+    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B, a.fin_overwrite); return; }
     int const lid  = xcd_remap(bid, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);
@@ -1206,7 +1310,7 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
     using T = DxTerm<N, XMODE, U>;
     int const bid = blockIdx.x;
     int const B   = a.chunk_count * a.tiles.count;
-    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B); return; }
+    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B, a.fin_overwrite); return; }
     int const lid  = xcd_remap(bid, B);
     int ck, tile;
     split_tile(lid, a.tiles, ck, tile);

@@ -435,6 +435,153 @@ __global__ __launch_bounds__(kTailBlock) void softmax_cross_entropy_few_kernel(f
     partial[(size_t)pix * frame_size + f] = loss;
 }
 
+// The whole tail of a LUT classifier in one launch: AverageLut forward over the last layer's output (un-binarized: the logits), softmax
+// cross entropy against t, categorical accuracy, and the AverageLut backward pass of the loss gradient — four launches of a few
+// microseconds each when called one by one, which at training batch sizes cost their launch latencies rather than their work.
+// A workgroup of kClassifierTailWaves wavefronts owns 64 frames of ALL nodes, one frame per lane.
+//   1. the table is staged in LDS;
+//   2. wavefront w computes the logits of the channels ch = w, w + waves, ...: the sum of the channel's n inputs in table order, times
+//      `scale` (as average_lut_forward_kernel), eight loads in flight at a time, and leaves them in LDS;
+//   3. every wavefront takes all logits and computes the loss terms (as softmax_cross_entropy_few_kernel, pix_size 1) and the accuracy
+//      (as categorical_accuracy_kernel) — the same values in each, cheaper than a second exchange; wavefront 0 stores them;
+//   4. the gradient dy / n of every logit goes through the table once more, in table order, into per-input sums in LDS
+//      (acc[input][lane] += dy[node] / n: the order of the host loop, include/bb/AverageLut.h:395-404, and of
+//      average_lut_backward_kernel); wavefront w takes the inputs with input % waves == w, so the chain of dependent LDS updates is a
+//      quarter as long, and writes their rows.
+// Columns between frame_size and frame_stride of dx are written as 0, as the backward kernels do.  Same bits as the four entries called
+// one after the other.  LDS: (input_node_size + 2 CH) x 64 floats + the table (padded to a multiple of four entries).
+constexpr int kClassifierTailWaves = 4;
+
+template <int CH>
+__global__ __launch_bounds__(64 * kClassifierTailWaves) void classifier_tail_kernel(float const *__restrict__ x, float *__restrict__ y, float *__restrict__ dx,
+                                                             int const *__restrict__ idx, float const *__restrict__ t,
+                                                             float *__restrict__ dy_out, double *__restrict__ loss_buf,
+                                                             int *__restrict__ accuracy_buf, int *__restrict__ category_buf,
+                                                             float t_sum, float scale, int n, int input_node_size, int ch_size,
+                                                             int frame_size, int frame_stride, int binarize_input)
+{
+    extern __shared__ __attribute__((aligned(16))) float tail_lds[];
+    constexpr int WAVES = kClassifierTailWaves;
+    int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int const total = ch_size * n, padded = (total + 3) & ~3;
+    float *acc   = tail_lds;                                                    // [input_node_size][64]
+    float *logit = tail_lds + (size_t)input_node_size * 64;                     // [CH][64]
+    float *dyn   = logit + CH * 64;                                             // [CH][64]: dy / n of the lane's frame
+    int *piece   = reinterpret_cast<int *>(dyn + CH * 64);                      // [padded]: the table
+    int const f = blockIdx.x * 64 + lane;
+    bool const in_row = f < frame_stride, live = f < frame_size;
+    int const fc = live ? f : 0;                                                // (a lane without a frame loads frame 0 and stores nothing)
+    for (int k = threadIdx.x; k < padded; k += 64 * WAVES) { piece[k] = (k < total) ? idx[k] : -1; }
+    // the targets do not depend on anything computed here: requested ahead of the logits
+    float tv[CH];
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) { tv[ch] = (ch < ch_size) ? t[(size_t)ch * frame_stride + fc] : 0.0f; }
+    __syncthreads();
+    {
+        // the wavefront's channels together, so that their loads are in flight together (a channel's sum stays in table order)
+        constexpr int PER = (CH + WAVES - 1) / WAVES;
+        float sum[PER];
+        int const *row[PER];
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            int const ch = wave + q * WAVES;
+            sum[q] = 0.0f;
+            row[q] = piece + ((ch < ch_size) ? ch : 0) * n;         // (a channel that does not exist reads channel 0's rows and stores nothing)
+        }
+        for (int i0 = 0; i0 < n; i0 += 8) {
+            float v[PER][8];
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) { v[q][j] = x[(size_t)row[q][(i0 + j < n) ? i0 + j : 0] * frame_stride + fc]; }
+            }
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (i0 + j < n) {
+                        float u = v[q][j];
+                        if (binarize_input) { u = (u > 0.0f) ? 1.0f : -1.0f; }
+                        sum[q] += u;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            int const ch = wave + q * WAVES;
+            if (ch < ch_size) {
+                float const out = rounded_mul(sum[q], scale);
+                logit[ch * 64 + lane] = out;
+                if (live && y != nullptr) { y[(size_t)ch * frame_stride + f] = out; }
+            }
+        }
+    }
+    __syncthreads();
+    float const eps = 1.0e-7f;
+    bool const first = (wave == 0) && live;
+    float yv[CH];
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) { yv[ch] = (ch < ch_size) ? logit[ch * 64 + lane] : 0.0f; }
+    // accuracy: the first largest logit sits on a channel with a positive target (one pixel per frame)
+    if (first) {
+        float max_y = -3.402823466e+38f, max_t = -3.402823466e+38f;
+        bool valid = false;
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            if (ch < ch_size) {
+                valid = valid || (tv[ch] > 0.0f);
+                if (yv[ch] > max_y) { max_y = yv[ch]; max_t = tv[ch]; }
+            }
+        }
+        if (accuracy_buf != nullptr) { accuracy_buf[f] = (valid && max_t > 0.0f) ? 1 : 0; }
+        if (category_buf != nullptr) { category_buf[f] = valid ? 1 : 0; }
+    }
+    // softmax cross entropy
+    float c = -3.402823466e+38f;
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) { if (ch < ch_size) { c = (c < yv[ch]) ? yv[ch] : c; } }
+    float y_sum = 0.0f, t_max = 0.0f;
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+        if (ch < ch_size) {
+            yv[ch] = expf(yv[ch] - c);
+            y_sum += yv[ch];
+            t_max += tv[ch];
+        }
+    }
+    if (y_sum <= eps) { y_sum = eps; }
+    double loss = 0.0;
+    float const fn = (float)n;
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+        if (ch < ch_size) {
+            float const softmax = yv[ch] / y_sum;
+            if (tv[ch] > 0.0f) { loss += (double)rounded_mul(logf(softmax + eps), t_max); }
+            float const g = (rounded_mul(t_max, softmax) - tv[ch]) / t_sum;
+            if (first && dy_out != nullptr) { dy_out[(size_t)ch * frame_stride + f] = g; }
+            dyn[ch * 64 + lane] = g / fn;           // (every wavefront writes the same values; each reads them after its own writes)
+        }
+    }
+    if (first) { loss_buf[f] = loss; }
+    // backward through the table, in table order; a lane only ever touches its own column of acc and dyn
+    for (int in = wave; in < input_node_size; in += WAVES) { acc[in * 64 + lane] = 0.0f; }
+    int node = 0, pos = 0;
+    for (int k = 0; k < padded; k += 4) {
+        int4 const e4 = *reinterpret_cast<int4 const *>(&piece[k]);
+        int const e[4] = {e4.x, e4.y, e4.z, e4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int const in = e[j];                            // the same for every lane
+            if ((unsigned)in < (unsigned)input_node_size && (in % WAVES) == wave) { acc[in * 64 + lane] += dyn[node * 64 + lane]; }
+            if (++pos == n) { pos = 0; ++node; }
+        }
+    }
+    if (in_row) {
+        for (int in = wave; in < input_node_size; in += WAVES) { dx[(size_t)in * frame_stride + f] = live ? acc[in * 64 + lane] : 0.0f; }
+    }
+}
+
 // loss_buf[frame] = sum over the pixels, ascending, of the per-pixel terms
 __global__ __launch_bounds__(kTailBlock) void loss_pixel_sum_kernel(double const *partial, double *loss_buf, int pix_size, int frame_size)
 {

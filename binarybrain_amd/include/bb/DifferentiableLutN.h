@@ -234,10 +234,23 @@ private:
     void HintInput(FrameBuffer const &x_buf, FrameBuffer *bits, bool holds_input)
     {
         if (bits != nullptr && !bits->Empty()) {
-            auto p = bits->LockDeviceMemory(!holds_input);
-            bbhip_HintPackedInput((int *)p.GetAddr(), (int)x_buf.GetNodeSize(), (int)(bits->GetFrameStride() / 4), holds_input ? 1 : 0);
+            int const rows = (int)x_buf.GetNodeSize(), words = (int)(bits->GetFrameStride() / 4);
+            if (holds_input) { bbhip_HintPackedInput((int *)bits->LockDeviceMemoryConst().GetAddr(), rows, words, 1); }
+            else             { bbhip_HintPackedInput((int *)bits->LockDeviceMemory(true).GetAddr(), rows, words, 0); }
         }
         else { bbhip_HintInputNodeSize((int)x_buf.GetNodeSize()); }         // the forward signatures do not carry the input's row count
+    }
+
+    // A layer in binary mode on fp32 frames binarizes its output; the layer behind it, if it is one of these too, reads that output as
+    // bits.  The forward entry writes the packed copy in the launch that binarizes (bbhip_HintPackedOutput) and it travels with the
+    // output buffer (FrameBuffer::AttachPackedTwin): the next layer's forward and backward calls then pack nothing.
+    FrameBuffer OfferPackedOutput(FrameBuffer const &y_buf)
+    {
+        FrameBuffer bits;
+        if (kBitType || !m_binary_mode) { return bits; }
+        bits.Resize(y_buf.GetFrameSize(), m_output_shape, BB_TYPE_BIT);
+        bbhip_HintPackedOutput((int *)bits.LockDeviceMemory(true).GetAddr(), (int)y_buf.GetNodeSize(), (int)(bits.GetFrameStride() / 4));
+        return bits;
     }
 
     // The tables that the entry points derive from W before their kernels run (centred coefficients, corner values) are the same
@@ -247,6 +260,7 @@ private:
     std::shared_ptr<Memory>                  m_tables;
     std::pair<void const *, std::uint64_t>   m_tables_stamp{nullptr, 0};
     int                                      m_tables_modes = -1;
+    float                                    m_tables_bias = 0.0f;      // the corner values depend on unbinarize_bias
 
     int TableModes(void) const { return (m_lut_binarize ? 1 : 0) | (m_binary_mode ? 2 : 0); }
 
@@ -257,14 +271,22 @@ private:
         if (bytes == 0) { return; }
         if (!m_tables || m_tables->GetSize() != bytes) { m_tables = Memory::Create(bytes); }
         bbhip_HintPreparedTables((float *)m_tables->LockDevice(true), bytes, 0);
+        m_tables_modes = -1;            // not filled yet: KeepTables() after the entry has returned success
+    }
+
+    // after the training forward entry returned success: the buffer holds the tables of this W and these modes
+    void KeepTables(void)
+    {
+        if (!m_tables) { return; }
         m_tables_stamp = m_W->WriteStamp();
         m_tables_modes = TableModes();
+        m_tables_bias  = m_unbinarize_bias;
     }
 
     // before a backward call
     void ReturnTables(void)
     {
-        if (m_tables && m_tables_modes == TableModes() && m_tables_stamp == m_W->WriteStamp()) {
+        if (m_tables && m_tables_modes == TableModes() && m_tables_bias == m_unbinarize_bias && m_tables_stamp == m_W->WriteStamp()) {
             bbhip_HintPreparedTables((float *)m_tables->LockDevice(), m_tables->GetSize(), 1);
         }
     }
@@ -294,14 +316,19 @@ public:
         int const O = (int)y_buf.GetNodeSize(), F = (int)y_buf.GetFrameSize();
         int const y_stride = (int)(y_buf.GetFrameStride() / 4), x_stride = (int)(x_buf.GetFrameStride() / 4);
         if (!kBitType) { BB_ASSERT(x_stride == y_stride); }
-        // the packed copy of a binarized fp32 input, kept for the backward pass of a training call
+        // the packed copy of a binarized fp32 input: the one that came with the buffer from the layer that wrote it, else (training) a
+        // place for the entry to pack into; kept for the backward pass of a training call
         FrameBuffer bits_buf;
-        if (train) {
-            if (!kBitType && m_binary_mode) { bits_buf.Resize(x_buf.GetFrameSize(), m_input_shape, BB_TYPE_BIT); }
-            m_packed_bufs.push(bits_buf);
+        bool have_bits = false;
+        if (!kBitType && m_binary_mode) {
+            bits_buf = x_buf.GetPackedTwin();
+            have_bits = !bits_buf.Empty();
+            if (!have_bits && train && !m_backward_break) { bits_buf.Resize(x_buf.GetFrameSize(), m_input_shape, BB_TYPE_BIT); }
         }
+        if (train) { m_packed_bufs.push(bits_buf); }
         auto x_ptr   = x_buf.LockDeviceMemoryConst();
         auto y_ptr   = y_buf.LockDeviceMemory(true);
+        FrameBuffer y_bits;
         auto idx_ptr = m_connection_table.LockDeviceMemConst_InputTable();
         if (clamp_in_entry) {
             auto W_mut    = m_W->LockDeviceMemory();
@@ -317,13 +344,16 @@ public:
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, 0.0f, 1.0f, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTrainingClampW");
             }
             else {
-                HintInput(x_buf, &bits_buf, false);
+                HintInput(x_buf, &bits_buf, have_bits);
+                y_bits = OfferPackedOutput(y_buf);
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float *)W_mut.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
                                 (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, 0.0f, 1.0f, nullptr),
                             "bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW");
             }
+            KeepTables();
+            if (!y_bits.Empty()) { y_buf.AttachPackedTwin(y_bits); }
             return y_buf;
         }
         auto W_ptr   = m_W->LockDeviceMemoryConst();
@@ -341,12 +371,14 @@ public:
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, nullptr), "bbhip_bit_fp32_DifferentiableLutN_ForwardTraining");
             }
             else {
-                HintInput(x_buf, &bits_buf, false);
+                HintInput(x_buf, &bits_buf, have_bits);
+                y_bits = OfferPackedOutput(y_buf);
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardTraining(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float *)mean_ptr.GetAddr(), (float *)rstd_ptr.GetAddr(),
                                 (float *)rm_ptr.GetAddr(), (float *)rv_ptr.GetAddr(), m_gamma, m_beta, m_momentum, m_unbinarize_bias,
                                 O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_ForwardTraining");
             }
+            KeepTables();
         }
         else if (m_batch_norm) {
             auto rm_ptr = m_running_mean.LockDeviceMemoryConst();
@@ -358,7 +390,8 @@ public:
                             "bbhip_bit_fp32_DifferentiableLutN_ForwardInference");
             }
             else {
-                bbhip_HintInputNodeSize((int)x_buf.GetNodeSize());      // the forward signatures do not carry the input's row count
+                HintInput(x_buf, &bits_buf, have_bits);
+                y_bits = OfferPackedOutput(y_buf);
                 CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardInference(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                                 (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), (float const *)rm_ptr.GetAddr(), (float const *)rv_ptr.GetAddr(),
                                 m_gamma, m_beta, m_unbinarize_bias, O, F, y_stride, m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr),
@@ -371,11 +404,13 @@ public:
                             m_lut_binarize ? 1 : 0, m_unbinarize_bias, nullptr), "bbhip_bit_bit_fp32_StochasticLut_Forward");
         }
         else {
-            HintInput(x_buf, &bits_buf, false);
+            HintInput(x_buf, &bits_buf, have_bits);
+            y_bits = OfferPackedOutput(y_buf);
             CheckDevice(bbhip_fp32_DifferentiableLutN_ForwardNoBn(N, (float const *)x_ptr.GetAddr(), (float *)y_ptr.GetAddr(),
                             (int const *)idx_ptr.GetAddr(), (float const *)W_ptr.GetAddr(), m_unbinarize_bias, O, F, y_stride,
                             m_lut_binarize ? 1 : 0, m_binary_mode ? 1 : 0, nullptr), "bbhip_fp32_DifferentiableLutN_ForwardNoBn");
         }
+        if (!y_bits.Empty()) { y_buf.AttachPackedTwin(y_bits); }
         return y_buf;
     }
 
@@ -383,6 +418,9 @@ public:
     {
         if (m_backward_break || dy_buf.Empty()) {          // a frozen layer: no gradient of its own, none passed on (reference :1015-1018)
             m_dW->FillZero();
+            // (what the matching forward pass kept is let go, or a frozen layer would hold one input and one packed copy per step)
+            if (!this->m_bufs.empty()) { this->m_bufs.pop(); }
+            if (!m_packed_bufs.empty()) { m_packed_bufs.pop(); }
             return FrameBuffer();
         }
         BB_ASSERT(dy_buf.GetType() == DataType<RealType>::type);

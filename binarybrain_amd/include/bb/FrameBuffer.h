@@ -65,8 +65,19 @@ class FrameBuffer {
     indices_t               m_shape;
     bool                    m_host_only = false;
     std::shared_ptr<Memory> m_mem;
+    // The packed copy (bit = value > 0.5) of a binarized fp32 buffer, written by the layer that produced the buffer in the same launch
+    // (bbhip_HintPackedOutput).  It travels with the buffer's copies and holds good while nobody has taken a writable lock on the
+    // fp32 memory since it was attached: the layer that reads the buffer next then takes the bits instead of packing the values again.
+    struct PackedTwin { std::shared_ptr<FrameBuffer> bits; std::uint64_t writes; };
+    std::shared_ptr<PackedTwin> m_twin;
 
 public:
+    // bits: a BB_TYPE_BIT buffer of the same shape and frame count.  Called by the producing layer after its launch, while the
+    // writable lock it took on this buffer for that launch is the last one handed out.
+    void AttachPackedTwin(FrameBuffer const &bits);
+    // the packed copy, or an empty buffer when there is none or the fp32 memory may have been written since
+    FrameBuffer GetPackedTwin(void) const;
+
     static index_t CalcFrameStride(int type, index_t frame_size)
     {
         index_t bytes = ((frame_size * DataType_GetBitSize(type) + 2047) / 2048) * 256;
@@ -88,6 +99,7 @@ public:
         m_node_size = shape.empty() ? 0 : CalcShapeSize(shape);
         m_frame_stride = CalcFrameStride(type, frame_size);
         m_mem = Memory::Create((std::size_t)(m_node_size * m_frame_stride), m_host_only);
+        m_twin.reset();
     }
 
     bool      Empty(void) const          { return m_frame_size == 0 || m_node_size == 0; }
@@ -151,5 +163,20 @@ public:
         return dst;
     }
 };
+
+inline void FrameBuffer::AttachPackedTwin(FrameBuffer const &bits)
+{
+    BB_ASSERT(bits.GetType() == BB_TYPE_BIT && bits.GetFrameSize() == m_frame_size && bits.GetNodeSize() == m_node_size);
+    m_twin = std::make_shared<PackedTwin>(PackedTwin{std::make_shared<FrameBuffer>(bits), m_mem->WriteCount()});
+}
+
+inline FrameBuffer FrameBuffer::GetPackedTwin(void) const
+{
+    if (m_twin && m_twin->bits && m_mem && m_twin->writes == m_mem->WriteCount() && m_twin->bits->GetFrameSize() == m_frame_size &&
+        m_twin->bits->GetNodeSize() == m_node_size) {
+        return *m_twin->bits;
+    }
+    return FrameBuffer();
+}
 
 }  // namespace bb

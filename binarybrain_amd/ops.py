@@ -506,6 +506,28 @@ def metrics_categorical_accuracy(y, t, ch_size, pix_size, frame_size):
     return acc, cat
 
 
+def classifier_tail(x, idx, t, frame_size, t_sum=None, binarize_input=False, mean=True, want_y=True, want_dy=False, want_accuracy=True):
+    """AverageLut forward (un-binarized) + softmax cross entropy + categorical accuracy + AverageLut backward in one launch; the same
+    bits as `average_lut_forward`, `loss_softmax_cross_entropy`, `metrics_categorical_accuracy` and `average_lut_backward` called one
+    after the other.  returns (y or None, dx, loss_buf, accuracy or None, category or None, dy or None)."""
+    _dev(x, idx, t)
+    ch, n = idx.shape
+    S = x.shape[1]
+    assert t.shape[1] == S
+    y = torch.empty((ch, S), dtype=torch.float32, device=x.device) if want_y else None
+    dy = torch.empty((ch, S), dtype=torch.float32, device=x.device) if want_dy else None
+    dx = torch.empty((x.shape[0], S), dtype=torch.float32, device=x.device)
+    loss_buf = torch.empty(frame_size, dtype=torch.float64, device=x.device)
+    acc = torch.empty(frame_size, dtype=torch.int32, device=x.device) if want_accuracy else None
+    cat = torch.empty(frame_size, dtype=torch.int32, device=x.device) if want_accuracy else None
+    if t_sum is None:
+        t_sum = float(t[:, :frame_size].sum(dtype=torch.float64).item())
+    check(lib().bbhip_fp32_ClassifierTail_ForwardBackward(ptr(x), ptr(y), ptr(dx), ptr(idx), ptr(t), ptr(dy), ptr(loss_buf), ptr(acc), ptr(cat),
+                                                          float(t_sum), n, x.shape[0], ch, frame_size, S,
+                                                          int(binarize_input), int(not mean), stream_ptr()))
+    return y, dx, loss_buf, acc, cat, dy
+
+
 def conv_bit_to_real(xbits, frame_size, y_stride, value0=0.0, value1=1.0):
     _dev(xbits)
     y = torch.empty((xbits.shape[0], y_stride), dtype=torch.float32, device=xbits.device)
@@ -527,29 +549,48 @@ def prepared_tables_buffer(n, node_size, device="cuda"):
 
 
 def _hint_tables(tables, holds_tables):
-    if tables is not None:
+    if tables is not None and HINTS:
         _dev(tables)
         assert tables.dtype == torch.float32
         lib().bbhip_HintPreparedTables(ptr(tables), tables.numel() * 4, int(holds_tables))
 
 
-def _hint_input(x, packed, holds_input):
+HINTS = True          # False: the wrappers pass no bbhip_Hint* at all (what a caller of the reference's plain signatures gets)
+
+
+def _hint_input(x, packed, holds_input, forward=True):
     """what the wrapper knows about the next LUT call's input: its row count, and where its packed copy goes to / comes from"""
+    if not HINTS:
+        return
     if packed is not None:
         _dev(packed)
         assert packed.dtype == torch.int32 and packed.shape[0] == x.shape[0]
         lib().bbhip_HintPackedInput(ptr(packed), x.shape[0], packed.shape[1], int(holds_input))
-    elif not holds_input:
+    elif forward:
         lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
 
 
-def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None, clamp_w=None, packed=None):
+def _hint_output(packed_out, rows):
+    """packed_out: a `packed_input_buffer(rows, frame_size)` that receives the binarized output as packed bits (for the next layer)"""
+    if packed_out is not None and HINTS:
+        _dev(packed_out)
+        assert packed_out.dtype == torch.int32 and packed_out.shape[0] == rows
+        lib().bbhip_HintPackedOutput(ptr(packed_out), rows, packed_out.shape[1])
+
+
+def _hint_overwrite(overwrite_dw):
+    if overwrite_dw:
+        lib().bbhip_HintTableGradientOverwrite(1)
+
+
+def stochastic_lut_forward(n, x, idx, W, frame_size, input_binary=False, lut_binarize=False, bias=0.25, out=None, clamp_w=None, packed=None,
+                           packed_holds=False):
     """clamp_w = (lo, hi): W is clamped in place first, as StochasticLutN::Forward does (include/bb/StochasticLutN.h:451),
     by the same launch that prepares the tables."""
     _dev(x, idx, W, out)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device) if out is None else out
-    _hint_input(x, packed, False)
+    _hint_input(x, packed, packed_holds)
     if clamp_w is not None:
         check(lib().bbhip_fp32_StochasticLut_ForwardClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, frame_size, x.shape[1],
                                                            int(input_binary), int(lut_binarize), bias, float(clamp_w[0]), float(clamp_w[1]), stream_ptr()))
@@ -592,7 +633,7 @@ def _tmp_for(output_nodes, n, frame_size, device, max_tmp_bytes):
 
 
 def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_binary=False, lut_binarize=False, bias=0.25,
-                            dx_tmp=None, tmp_frame_size=None, max_tmp_bytes=256 * 1024 * 1024, out=None, packed=None):
+                            dx_tmp=None, tmp_frame_size=None, max_tmp_bytes=256 * 1024 * 1024, out=None, packed=None, overwrite_dw=False):
     """dW is accumulated in place; returns dx [I, stride]. ``rev`` (reverse table) is needed by dx modes 0 and 2,
     dx_tmp by mode 2 only (allocated here when not given)."""
     _dev(x, dy, idx, W, dW, rev, dx_tmp, out)
@@ -604,7 +645,8 @@ def stochastic_lut_backward(n, x, dy, idx, W, dW, frame_size, rev=None, input_bi
         tf = min(ts, frame_size) if tmp_frame_size is None else tmp_frame_size
     elif lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
-    _hint_input(x, packed, True)
+    _hint_input(x, packed, True, forward=False)
+    _hint_overwrite(overwrite_dw)
     check(lib().bbhip_fp32_StochasticLut_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                   0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,
                                                   int(input_binary), int(lut_binarize), bias, stream_ptr()))
@@ -626,8 +668,11 @@ def bit_stochastic_lut_backward(n, xbits, dy, idx, W, dW, frame_size, rev=None, 
 
 
 def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None, packed=None, tables=None):
+                                        momentum=0.9, bias=0.25, lut_binarize=False, binary_mode=True, clamp_w=None, packed=None, tables=None,
+                                        packed_holds=False, packed_out=None):
     """fp32 frames. running_mean / running_var are updated in place. returns (y, mean, rstd).
+    packed_holds: `packed` already holds the packed copy of x (it was the `packed_out` of the layer before): nothing is packed.
+    packed_out: a `packed_input_buffer(O, frame_size)` that receives the binarized output as packed bits, for the next layer.
     tables: a `prepared_tables_buffer` that receives the tables derived from W, for the backward call of the same step.
     packed: a `packed_input_buffer` that receives the packed copy of the binarized input (binary mode), for the backward call.
     clamp_w = (lo, hi): W is clamped in place first, by the launch that prepares the tables (the model class's clamp before the
@@ -637,8 +682,9 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
     mean = torch.empty(O, dtype=torch.float32, device=x.device)
     rstd = torch.empty(O, dtype=torch.float32, device=x.device)
-    _hint_input(x, packed, False)
+    _hint_input(x, packed, packed_holds)
     _hint_tables(tables, False)
+    _hint_output(packed_out if binary_mode else None, O)
     if clamp_w is not None:
         check(lib().bbhip_fp32_DifferentiableLutN_ForwardTrainingClampW(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(mean), ptr(rstd),
                                                                         ptr(running_mean), ptr(running_var), gamma, beta, momentum, bias,
@@ -673,11 +719,12 @@ def bit_differentiable_lut_forward_training(n, xbits, idx, W, frame_size, runnin
 
 
 def differentiable_lut_forward_inference(n, x, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                         bias=0.25, lut_binarize=False, binary_mode=True):
+                                         bias=0.25, lut_binarize=False, binary_mode=True, packed=None, packed_holds=False, packed_out=None):
     _dev(x, idx, W, running_mean, running_var)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
-    lib().bbhip_HintInputNodeSize(x.shape[0])       # the forward signatures do not carry the row count of x
+    _hint_input(x, packed, packed_holds)
+    _hint_output(packed_out if binary_mode else None, O)
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardInference(n, ptr(x), ptr(y), ptr(idx), ptr(W), ptr(running_mean),
                                                                ptr(running_var), gamma, beta, bias, O, frame_size, x.shape[1],
                                                                int(lut_binarize), int(binary_mode), stream_ptr()))
@@ -695,18 +742,20 @@ def bit_differentiable_lut_forward_inference(n, xbits, idx, W, frame_size, runni
     return y
 
 
-def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_binarize=False, binary_mode=True, packed=None):
+def differentiable_lut_forward_nobn(n, x, idx, W, frame_size, bias=0.25, lut_binarize=False, binary_mode=True, packed=None, packed_holds=False,
+                                    packed_out=None):
     _dev(x, idx, W)
     O = idx.shape[0]
     y = torch.empty((O, x.shape[1]), dtype=torch.float32, device=x.device)
-    _hint_input(x, packed, False)
+    _hint_input(x, packed, packed_holds)
+    _hint_output(packed_out if binary_mode else None, O)
     check(lib().bbhip_fp32_DifferentiableLutN_ForwardNoBn(n, ptr(x), ptr(y), ptr(idx), ptr(W), bias, O, frame_size, x.shape[1],
                                                           int(lut_binarize), int(binary_mode), stream_ptr()))
     return y
 
 
 def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, rev=None, gamma=0.3, beta=0.5, bias=0.25,
-                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024, packed=None, tables=None):
+                                lut_binarize=False, binary_mode=True, max_tmp_bytes=256 * 1024 * 1024, packed=None, tables=None, overwrite_dw=False):
     """tables: the buffer that this step's forward call with the same W filled (`prepared_tables_buffer`): no preparation launch.
     packed: the buffer that the forward call on the same x filled (`packed_input_buffer`): the call reads it instead of packing x."""
     _dev(x, dy, idx, W, dW, mean, rstd, rev)
@@ -717,8 +766,9 @@ def differentiable_lut_backward(n, x, dy, idx, W, dW, frame_size, mean, rstd, re
     dx_tmp, tf, ts = (None, 0, 0)
     if lib().bbhip_GetDxMode() == 2:
         dx_tmp, tf, ts = _tmp_for(O, n, frame_size, x.device, max_tmp_bytes)
-    _hint_input(x, packed, True)
+    _hint_input(x, packed, True, forward=False)
     _hint_tables(tables, True)
+    _hint_overwrite(overwrite_dw)
     check(lib().bbhip_fp32_DifferentiableLutN_Backward(n, ptr(x), ptr(dy), ptr(dx), ptr(dx_tmp), ptr(idx), ptr(rev), ptr(W), ptr(dW),
                                                        ptr(mean), ptr(rstd), ptr(dmean), ptr(dvar), gamma, beta, bias,
                                                        0 if rev is None else rev.shape[1], I, O, frame_size, dy.shape[1], tf, ts,

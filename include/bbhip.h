@@ -104,7 +104,8 @@ void bbhip_HintInputNodeSize(int input_node_size);
  *   - right before the forward call, with holds_input = 0: dev_bits, `rows` rows (the input's node count: this also serves as
  *     bbhip_HintInputNodeSize) of row_words 32-bit words each, receives the packed copy instead of the library's scratch;
  *   - right before the backward call on the same input, with holds_input = 1: the buffer still holds that copy (the caller's
- *     promise: x has not changed since), and the call reads it instead of packing x again.
+ *     promise: x has not changed since), and the call reads it instead of packing x again.  A forward call takes holds_input = 1 the
+ *     same way (the buffer was filled as the packed output of the layer before, bbhip_HintPackedOutput, or by an earlier call).
  * row_words must be a multiple of 8 and at least ceil(frame_size / 32) (bbhip_PackedRowWords(frame_size) gives the pitch the
  * library itself would use), dev_bits 32-byte aligned; a buffer that does not fit the call is ignored (the library packs into its
  * scratch as always).  Like the other hint it holds for the next LUT call of the same thread and is cleared by any entry.
@@ -112,11 +113,31 @@ void bbhip_HintInputNodeSize(int input_node_size);
 int  bbhip_PackedRowWords(int frame_size);
 void bbhip_HintPackedInput(int *dev_bits, int rows, int row_words, int holds_input);
 
+/* ---- the binarized output of a forward call as packed bits as well (no counterpart in the reference) ----
+ * A layer in binary mode that follows another reads bits, and what it would pack is the output that the layer before has just
+ * binarized.  Given right before a forward call whose output is binarized fp32 (the fp32 entries in binary mode), the call writes its
+ * output to dev_y_buf as always AND as packed bits to dev_bits (`rows` = node_size rows of row_words words, row_words a multiple of 8
+ * and at least ceil(frame_size / 32), 32-byte aligned; bit f & 31 of word f >> 5 = y > 0.5, words behind the last frame 0): the
+ * wavefront that binarizes 64 frames stores their ballot, no extra launch.  The caller then hands that buffer to the next layer's
+ * forward call as bbhip_HintPackedInput(dev_bits, rows, row_words, 1) — "this already holds the packed copy of the input" — and that
+ * call packs nothing; its backward call takes it the same way.  holds_input = 1 is the caller's promise that the fp32 buffer has not
+ * been written since.  A buffer that does not fit the call is ignored and not written.  Thread-local and spent by the next entry
+ * called on the thread, like the other hints; the fp32 output is the same bits with and without it. */
+void bbhip_HintPackedOutput(int *dev_bits, int rows, int row_words);
+
+/* ---- table gradient written instead of accumulated (no counterpart in the reference) ----
+ * The backward entries add into dev_dW, as the reference's do (dW accumulates until the optimizer or ZeroGrad clears it).  A caller
+ * whose dW holds nothing worth keeping (it would zero it first) says so right before the backward call with overwrite = 1, and the
+ * call writes dW = (this call's gradient) in the launch that already folds the partial sums: the caller's fill launch falls away.
+ * Same bits as zero-fill followed by the plain call.  Thread-local, spent by the next entry called on the thread. */
+void bbhip_HintTableGradientOverwrite(int overwrite);
+
 /* No counterpart in the reference.  A caller-owned device buffer (256-byte aligned, bbhip_PreparedTablesBytes(n, node_size) bytes) for the
  * tables that a LUT call derives from W before its kernels run (centred coefficients, corner values).  Given right before a forward call
  * (holds_tables = 0), the call writes them there instead of into the library's scratch memory; given right before the backward call of
  * the same step with holds_tables = 1, that call takes them from there and skips its own preparation launch.  holds_tables = 1 is the
- * caller's promise that W, the LUT width, the node count, lut_binarize and the kind of input (two-valued or not) are those of the call
+ * caller's promise that W, the LUT width, the node count, lut_binarize, unbinarize_bias (the corner values depend on it) and the kind of
+ * input (two-valued or not) are those of the call
  * that filled the buffer; a buffer that is too small or not aligned is ignored and not written.  Thread-local, spent by the next entry
  * point called on the thread, like the other hints; results are the same bits with and without it. */
 void   bbhip_HintPreparedTables(float *dev_tables, size_t bytes, int holds_tables);
@@ -242,6 +263,20 @@ int bbhip_bit_AverageLut_Forward(int const *dev_x_buf, int *dev_y_buf, int const
  * the padding of every row, are written as 0.  Deterministic: the reverse wiring is built on the device in library scratch. */
 int bbhip_fp32_AverageLut_Backward(float const *dev_dy_buf, float *dev_dx_buf, int const *dev_input_index, int n, int input_node_size,
                                    int output_node_size, int frame_size, int frame_stride, void *stream);
+/* The tail of a LUT classifier in ONE launch (no counterpart in the reference, which calls the four parts one by one; for training
+ * loops at small batches, where each of those launches costs its latency rather than its work):
+ *   y  = bbhip_fp32_AverageLut_Forward(x) without binarize_output (output_sum = 1: bbhip_fp32_AverageLut_ForwardSum), ch_size nodes of n inputs;
+ *   dy, loss = bbhip_fp32_LossSoftmaxCrossEntropy(y, t) with pix_size 1;   accuracy, category = bbhip_fp32_MetricsCategoricalAccuracy(y, t);
+ *   dx = bbhip_fp32_AverageLut_Backward(dy)
+ * with the same bits in every output as those calls give.  dev_y_buf, dev_dy_buf ([ch_size][frame_stride]), dev_accuracy_buf and
+ * dev_category_buf ([frame_size]) may be NULL where the caller does not want them; dev_dx_buf [input_node_size][frame_stride] and
+ * dev_loss_buf [frame_size] are always written.  Limits: ch_size <= 16 and 256 * (input_node_size + 32) + 4 * ch_size * n <= 65536
+ * (the per-input sums of 64 frames and the table are kept in LDS: 192 input nodes with 2048 table entries, 216 with 512); larger tails
+ * are rejected — call the parts. */
+int bbhip_fp32_ClassifierTail_ForwardBackward(float const *dev_x_buf, float *dev_y_buf, float *dev_dx_buf, int const *dev_input_index,
+                                              float const *dev_t_buf, float *dev_dy_buf, double *dev_loss_buf, int *dev_accuracy_buf,
+                                              int *dev_category_buf, float t_sum, int n, int input_node_size, int ch_size, int frame_size,
+                                              int frame_stride, int binarize_input, int output_sum, void *stream);
 /* ---- MaxLut ----
  * The largest of n wired inputs, as the reference's host loop computes it (include/bb/MaxLut.h:293-318, 394-424): the running
  * maximum starts at -1 and is replaced by strictly larger values, so the output is never below -1 (the reference's device kernel

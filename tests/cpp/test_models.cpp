@@ -210,6 +210,61 @@ static void test_differentiable(int I, int O, int F, bool binary)
     CHECK(none.Empty() && max_abs(dW) == 0.0, "backward_break: the layer must return an empty buffer and zero its table gradient");
 }
 
+// Two DifferentiableLut6 layers in binary mode on fp32 frames: the first layer's forward call writes the packed copy of its binarized
+// output beside it and the copy travels with the buffer (FrameBuffer::GetPackedTwin), so the second layer packs nothing, forward or
+// backward.  A writable lock on the buffer in between makes the copy stale — the second layer then packs the values itself — and no
+// output may differ by a bit between the two ways; a frozen layer keeps nothing from its forward passes.
+static bool same_bits(bb::FrameBuffer &a, bb::FrameBuffer &b);
+static void test_packed_twin(int I, int H, int O, int F)
+{
+    std::mt19937_64 mt(4242 + I + H + O + F);
+    std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+    std::normal_distribution<float> nrm(0.0f, 1.0f);
+    bb::FrameBuffer x_buf(F, {I}, BB_TYPE_FP32), dy_buf(F, {O}, BB_TYPE_FP32);
+    { auto xp = x_buf.Lock<float>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { xp.Set(f, n, uni(mt)); } }
+    { auto dp = dy_buf.Lock<float>(true); for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { dp.Set(f, n, nrm(mt)); } }
+    std::vector<float> y[2], dx[2], dW1[2], dW2[2];
+    for (int pass = 0; pass < 2; ++pass) {
+        typename bb::DifferentiableLutN<6, float>::create_t c1, c2;
+        c1.output_shape = {H}; c1.seed = 11; c2.output_shape = {O}; c2.seed = 12;
+        auto l1 = bb::DifferentiableLutN<6, float>::Create(c1);
+        auto l2 = bb::DifferentiableLutN<6, float>::Create(c2);
+        l1->SetInputShape({I}); l2->SetInputShape({H});
+        for (int step = 0; step < 2; ++step) {                 // (the second step runs with the table clamp inside the forward entry)
+            bb::FrameBuffer h_buf = l1->Forward(x_buf, true);
+            if (step == 0) {
+                CHECK(!h_buf.GetPackedTwin().Empty(), "binary-mode layer on fp32 frames: the output carries no packed copy");
+                bb::FrameBuffer copy = h_buf;                   // the copy travels with copies of the buffer
+                CHECK(!copy.GetPackedTwin().Empty(), "the packed copy does not travel with a copy of the buffer");
+            }
+            if (pass == 1) {
+                h_buf.LockDeviceMemory();                       // somebody may have written: the packed copy is no longer trusted
+                CHECK(h_buf.GetPackedTwin().Empty(), "a writable lock must retire the packed copy");
+            }
+            bb::FrameBuffer y_buf = l2->Forward(h_buf, true);
+            bb::FrameBuffer dh_buf = l2->Backward(dy_buf);
+            bb::FrameBuffer dx_buf = l1->Backward(dh_buf);
+            if (step == 1) {
+                read_fp32(y_buf, y[pass]); read_fp32(dx_buf, dx[pass]);
+                { auto p = l1->lock_dW_const(); dW1[pass].resize((size_t)H * 64); for (size_t k = 0; k < dW1[pass].size(); ++k) { dW1[pass][k] = p[(bb::index_t)k]; } }
+                { auto p = l2->lock_dW_const(); dW2[pass].resize((size_t)O * 64); for (size_t k = 0; k < dW2[pass].size(); ++k) { dW2[pass][k] = p[(bb::index_t)k]; } }
+            }
+            else {
+                // an optimizer step's worth of change, so that the clamp has something to do
+                auto Wp = l1->lock_W(); for (bb::index_t k = 0; k < (bb::index_t)H * 64; k += 7) { Wp[k] = Wp[k] * 1.5f - 0.2f; }
+            }
+        }
+        // inference takes the copy as well
+        bb::FrameBuffer h_inf = l1->Forward(x_buf, false);
+        CHECK(!h_inf.GetPackedTwin().Empty(), "inference output carries no packed copy");
+        bb::FrameBuffer y_a = l2->Forward(h_inf, false);
+        h_inf.LockDeviceMemory();
+        bb::FrameBuffer y_b = l2->Forward(h_inf, false);
+        CHECK(same_bits(y_a, y_b), "inference: output differs with and without the packed copy");
+    }
+    CHECK(y[0] == y[1] && dx[0] == dx[1] && dW1[0] == dW1[1] && dW2[0] == dW2[1], "results differ with and without the packed copy of the hidden layer");
+}
+
 static void test_binary(int I, int O, int F)
 {
     std::mt19937_64 mt(99 + I + O + F);
@@ -1096,6 +1151,8 @@ int main(void)
             test_differentiable<4>(24, 20, 64, true);
         }
         bbhip_SetDxMode(0);
+        test_packed_twin(40, 70, 20, 1000);
+        test_packed_twin(27, 216, 36, 5000);
         test_binary(16, 16, 32);
         test_binary(70, 33, 1000);
         test_import_layer();

@@ -203,3 +203,44 @@ def test_average_lut_both_conventions(ops):
         assert np.array_equal(yb[:, :F], ybs[:, :F])
         # the two differ by exactly the fp32 reciprocal of n
         assert np.array_equal(y[:, :F], (ys[:, :F] * (np.float32(1.0) / np.float32(n))).astype(np.float32))
+
+
+@pytest.mark.parametrize("case", [(70, 10, 7, 1024, False), (70, 10, 7, 1000, True), (30, 5, 3, 5000, False), (176, 16, 9, 37, False), (12, 2, 6, 64, True)])
+@pytest.mark.parametrize("mean", [True, False])
+def test_classifier_tail_in_one_launch(ops, case, mean):
+    """bbhip_fp32_ClassifierTail_ForwardBackward = AverageLut forward + softmax cross entropy + accuracy + AverageLut backward: every output
+    equals, bit for bit, what the four entries give called one after the other (and those are checked against the oracle above)."""
+    import torch
+    I, CH, n, F, bin_in = case
+    rng = np.random.default_rng(I + CH + n + F)
+    S = synth.frame_stride_fp32(F)
+    idx = rng.integers(0, I - 2, (CH, n)).astype(np.int32)               # the last two inputs feed no node: their gradient is 0
+    if I == 70:
+        idx = np.arange(70, dtype=np.int32).reshape(10, 7)               # the classifier's own wiring
+    x = np.zeros((I, S), np.float32); x[:, :F] = rng.integers(0, 2, (I, F)) if I == 70 else rng.standard_normal((I, F))
+    t = np.zeros((CH, S), np.float32)
+    label = rng.integers(0, CH, F)
+    t[label, np.arange(F)] = 1.0
+    t[:, F // 2] = 0.0                                                   # a frame without a target: not counted by the accuracy
+    xd, td, idxd = dev(x), dev(t), dev(idx)
+    y0 = ops.average_lut_forward(xd, idxd, F, bin_in, False, mean=mean)
+    dy0, loss0, t_sum = ops.loss_softmax_cross_entropy(y0, td, CH, 1, F)
+    acc0, cat0 = ops.metrics_categorical_accuracy(y0, td, CH, 1, F)
+    dx0 = ops.average_lut_backward(dy0, idxd, I, F)
+    y1, dx1, loss1, acc1, cat1, dy1 = ops.classifier_tail(xd, idxd, td, F, t_sum=t_sum, binarize_input=bin_in, mean=mean, want_dy=True)
+    assert torch.equal(y0[:, :F], y1[:, :F]) and torch.equal(dy0[:, :F], dy1[:, :F])
+    assert torch.equal(loss0, loss1) and torch.equal(acc0, acc1) and torch.equal(cat0, cat1)
+    assert torch.equal(dx0, dx1)                                         # whole rows: the columns past the last frame are 0 in both
+    assert I == 70 or not host(dx1)[I - 2:].any()
+    # the outputs that the caller does not want may be left out
+    _, dx2, loss2, acc2, _, _ = ops.classifier_tail(xd, idxd, td, F, t_sum=t_sum, binarize_input=bin_in, mean=mean, want_y=False, want_accuracy=False)
+    assert torch.equal(dx0, dx2) and torch.equal(loss0, loss2) and acc2 is None
+
+
+def test_classifier_tail_limits(ops):
+    import torch
+    x = torch.zeros((300, 64), device="cuda"); t = torch.zeros((4, 64), device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.classifier_tail(x, torch.zeros((4, 3), dtype=torch.int32, device="cuda"), t, 64, t_sum=1.0)          # too many input nodes for one launch
+    with pytest.raises(RuntimeError):
+        ops.classifier_tail(x[:20], torch.zeros((17, 3), dtype=torch.int32, device="cuda"), torch.zeros((17, 64), device="cuda"), 64, t_sum=1.0)
