@@ -78,7 +78,7 @@ def write_traffic(dirname):
     def counters(workload, counter):
         db = os.path.join(dirname, workload, counter, "r_results.db")
         con = sqlite3.connect(db)
-        rows = con.execute("select kernel_name, value from counters_collection where counter_name = ? order by rowid", (counter,)).fetchall()
+        rows = con.execute("select kernel_name, value from counters_collection where counter_name = ? order by dispatch_id", (counter,)).fetchall()
         con.close()
         by = {}
         for name, value in rows:
@@ -92,7 +92,7 @@ def write_traffic(dirname):
         units = []
         for w, nbytes in copy_bytes.items():
             by = counters(w, counter)
-            copies = [v for name, vals in by.items() if ("copy" in name.lower() or "elementwise" in name.lower()) for v in vals[-3:]]
+            copies = [v for name, vals in by.items() if "copybuffer" in name.lower() for v in vals[-3:]]      # torch's device-to-device copy
             if copies:
                 units.append(nbytes / (sum(copies) / len(copies)))
                 calibration["%s, %s" % (counter, w)] = {"copy_bytes": nbytes, "counter_per_copy": sum(copies) / len(copies)}
