@@ -120,6 +120,7 @@ _SIGNATURES = {
     "bbhip_bit_fp32_DifferentiableLutN_Backward": (C.c_int, [_i] + [_vp] * 12 + [_f] * 3 + [_i] * 9 + [_vp]),
     "bbhip_fp32_DifferentiableLutN_ForwardNoBn": (C.c_int, [_i] + [_vp] * 4 + [_f] + [_i] * 5 + [_vp]),
     "bbhip_bit_BinaryLut6_Forward": (C.c_int, [_vp] * 4 + [_i] * 3 + [_vp]),
+    "bbhip_bit_BinaryLutN_Forward": (C.c_int, [_i] + [_vp] * 4 + [_i] * 3 + [_vp]),
 }
 
 

@@ -2697,4 +2697,31 @@ int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const
     return 0;
 }
 
+int bbhip_bit_BinaryLutN_Forward(int n, int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
+                                 int node_size, int frame_size, int frame_stride, void *stream)
+{
+    if (n == 6) { return bbhip_bit_BinaryLut6_Forward(dev_x_buf, dev_y_buf, dev_input_index, dev_table, node_size, frame_size, frame_stride, stream); }
+    clear_hints();
+    if (n < 2 || n > 6) { return fail("%s: LUT width n=%d not in 2..6", __func__, n); }
+    BBHIP_REQUIRE(dev_x_buf != nullptr && dev_y_buf != nullptr && dev_input_index != nullptr && dev_table != nullptr);
+    BBHIP_REQUIRE(node_size > 0 && node_size <= (0x7fffffff >> 6) && frame_size > 0);
+    BBHIP_REQUIRE(frame_stride >= (frame_size + 31) / 32);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint32_t const *x = reinterpret_cast<uint32_t const *>(dev_x_buf);
+    uint32_t *y = reinterpret_cast<uint32_t *>(dev_y_buf);
+    int const words = (frame_size + 31) / 32;
+    ScopedTimer tm(kTimeBinary, st);
+    for (int n0 = 0; n0 < node_size; n0 += 65535) {            // grid.y is limited to 65535 nodes per launch
+        dim3 const grid(ceil_div(words, kBlock), (node_size - n0 < 65535) ? node_size - n0 : 65535), block(kBlock);
+        switch (n) {
+        case 2: hipLaunchKernelGGL(binary_lutn_kernel<2>, grid, block, 0, st, x, y, dev_input_index, dev_table, n0, frame_size, frame_stride); break;
+        case 3: hipLaunchKernelGGL(binary_lutn_kernel<3>, grid, block, 0, st, x, y, dev_input_index, dev_table, n0, frame_size, frame_stride); break;
+        case 4: hipLaunchKernelGGL(binary_lutn_kernel<4>, grid, block, 0, st, x, y, dev_input_index, dev_table, n0, frame_size, frame_stride); break;
+        default: hipLaunchKernelGGL(binary_lutn_kernel<5>, grid, block, 0, st, x, y, dev_input_index, dev_table, n0, frame_size, frame_stride); break;
+        }
+        BBHIP_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
 }  // extern "C"

@@ -1794,4 +1794,37 @@ __global__ __launch_bounds__(kBlock) void binary_lut6_kernel(BinArgs a)
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+//  BinaryLutN for N = 2 .. 5 (reference: the generic loop of BinaryLutN<N>::Forward, include/bb/BinaryLutN.h:436-463; the
+//  reference has a device kernel for N = 6 only).  A table of 2^N <= 32 entries is one word per node.  One thread per (node, word of
+//  32 frames): the N input words are the select lines of a multiplexer tree over the table's entries, each entry spread to a word of
+//  all ones or all zeros — 2^N - 1 bit-selects per word, whose first level folds into constants.  The node (blockIdx.y), its wiring
+//  and its table are the same for the whole workgroup: scalar loads.  Bits of the last word beyond frame_size are written as 0.
+// ------------------------------------------------------------------------------------------------
+template <int N>
+__global__ __launch_bounds__(kBlock) void binary_lutn_kernel(uint32_t const *__restrict__ x, uint32_t *__restrict__ y, int const *__restrict__ idx,
+                                                            int const *__restrict__ table, int node0, int frame_size, int stride)
+{
+    static_assert(N >= 2 && N <= 5, "one table word per node");
+    int const node = node0 + (int)blockIdx.y;
+    int const w = blockIdx.x * kBlock + threadIdx.x;
+    int const words = (frame_size + 31) >> 5;
+    if (w >= words) { return; }
+    uint32_t const t = (uint32_t)table[node];
+    uint32_t sel[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) { sel[k] = x[(size_t)idx[node * N + k] * stride + w]; }
+    uint32_t v[1 << N];
+#pragma unroll
+    for (int i = 0; i < (1 << N); ++i) { v[i] = ((t >> i) & 1u) ? 0xffffffffu : 0u; }
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+#pragma unroll
+        for (int i = 0; i < (1 << (N - 1 - k)); ++i) { v[i] = (sel[k] & v[2 * i + 1]) | (~sel[k] & v[2 * i]); }
+    }
+    uint32_t out = v[0];
+    if (w == words - 1 && (frame_size & 31)) { out &= (1u << (frame_size & 31)) - 1u; }
+    y[(size_t)node * stride + w] = out;
+}
+
 }  // namespace bbhip

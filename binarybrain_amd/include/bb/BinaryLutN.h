@@ -1,7 +1,8 @@
-// BinaryLutN<6, Bit>: inference-only layer of 6-input binary look-up tables on bit-packed frames, with the reference's
+// BinaryLutN<N, Bit>, N = 2 .. 6: inference-only layer of N-input binary look-up tables on bit-packed frames, with the reference's
 // model API (include/bb/BinaryLutN.h:20-523, table helpers in include/bb/BinaryLutModel.h:45-91): Create, SetInputShape,
 // connection get/set, GetLutTable / SetLutTable, ImportLayer, Forward.  Input k of a node is bit k of the table index;
-// entries 0-31 of a node's 64-entry table live in word 0 of its int32 [2] row.  Frame work runs in the HIP library only.
+// a node's table is (2^N + 31) / 32 words of its int32 row, entry i = bit i & 31 of word i >> 5 (one word up to N = 5, two for N = 6).
+// Frame work runs in the HIP library only (the reference has a device kernel for N = 6 and runs the other widths on the host).
 #pragma once
 
 #include <random>
@@ -13,17 +14,17 @@ namespace bb {
 
 template <int N = 6, typename FT = Bit, typename BT = float>
 class BinaryLutN : public Model {
-    static_assert(N == 6 && std::is_same<FT, Bit>::value, "the device path covers 6-input tables on packed bits");
+    static_assert(N >= 2 && N <= 6 && std::is_same<FT, Bit>::value, "the device path covers 2- to 6-input tables on packed bits");
     static constexpr int kTableSize = 1 << N;
-    static constexpr int kTableUnit = kTableSize / 32;
+    static constexpr int kTableUnit = (kTableSize + 31) / 32;
 
 protected:
     bool        m_host_only = false;
     bool        m_host_simd = true;             // carried through serialization only: there is no host path here
     std::string m_connection;
     indices_t   m_input_shape, m_output_shape;
-    Tensor_<std::int32_t> m_table;          // [output nodes][2]
-    Tensor_<std::int32_t> m_input_index;    // [output nodes][6]
+    Tensor_<std::int32_t> m_table;          // [output nodes][kTableUnit]
+    Tensor_<std::int32_t> m_input_index;    // [output nodes][N]
     std::mt19937_64 m_mt;
 
     void CommandProc(std::vector<std::string> args) override
@@ -191,9 +192,9 @@ public:
         auto y_ptr   = y_buf.LockDeviceMemory(true);
         auto idx_ptr = m_input_index.LockDeviceMemoryConst();
         auto tbl_ptr = m_table.LockDeviceMemoryConst();
-        CheckDevice(bbhip_bit_BinaryLut6_Forward((int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(), (int const *)idx_ptr.GetAddr(),
+        CheckDevice(bbhip_bit_BinaryLutN_Forward(N, (int const *)x_ptr.GetAddr(), (int *)y_ptr.GetAddr(), (int const *)idx_ptr.GetAddr(),
                         (int const *)tbl_ptr.GetAddr(), (int)y_buf.GetNodeSize(), (int)y_buf.GetFrameSize(),
-                        (int)(y_buf.GetFrameStride() / sizeof(int)), nullptr), "bbhip_bit_BinaryLut6_Forward");
+                        (int)(y_buf.GetFrameStride() / sizeof(int)), nullptr), "bbhip_bit_BinaryLutN_Forward");
         return y_buf;
     }
 

@@ -47,6 +47,10 @@ inline std::shared_ptr<Object> CreateByName(std::string const &name)
     if (name == "Tensor_fp64")  { return std::make_shared<Tensor_<double>>(); }
     if (name == "Tensor_int32") { return std::make_shared<Tensor_<std::int32_t>>(); }
     if (name == BinaryLutN<6, Bit, float>::ObjectName()) { return BinaryLutN<6, Bit, float>::Create((index_t)1); }
+    if (name == BinaryLutN<5, Bit, float>::ObjectName()) { return BinaryLutN<5, Bit, float>::Create((index_t)1); }
+    if (name == BinaryLutN<4, Bit, float>::ObjectName()) { return BinaryLutN<4, Bit, float>::Create((index_t)1); }
+    if (name == BinaryLutN<3, Bit, float>::ObjectName()) { return BinaryLutN<3, Bit, float>::Create((index_t)1); }
+    if (name == BinaryLutN<2, Bit, float>::ObjectName()) { return BinaryLutN<2, Bit, float>::Create((index_t)1); }
     if (name == Sequential::ObjectName())                         { return Sequential::Create(); }
     if (name == StochasticBatchNormalization<float>::ObjectName()) { return StochasticBatchNormalization<float>::Create(); }
     if (name == AverageLut<float, float>::ObjectName())           { return AverageLut<float, float>::Create(); }

@@ -802,6 +802,16 @@ def binary_lut6_forward(xbits, idx, table, frame_size, out=None):
     return y
 
 
+def binary_lutn_forward(n, xbits, idx, table, frame_size, out=None):
+    """BinaryLutN<n> on packed bits, n = 2 .. 6: table [O, 1] words for n <= 5 (entry i = bit i), [O, 2] for n = 6"""
+    _dev(xbits, idx, table, out)
+    O = idx.shape[0]
+    assert idx.shape[1] == n and table.shape == (O, 2 if n == 6 else 1)
+    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device) if out is None else out
+    check(lib().bbhip_bit_BinaryLutN_Forward(n, ptr(xbits), ptr(y), ptr(idx), ptr(table), O, frame_size, xbits.shape[1], stream_ptr()))
+    return y
+
+
 def reverse_table(idx, input_nodes):
     """Reverse connection table as the reference builds it (include/bb/FixedSizeConnectionTable.h:180-215):
     ``[input_nodes, 1 + max fan-out]`` int32, row r = [count, node*n + input ... ascending, zero tail].

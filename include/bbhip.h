@@ -561,6 +561,13 @@ int bbhip_fp32_DifferentiableLutN_ForwardNoBn(int n, float const *dev_x_buf, flo
 int bbhip_bit_BinaryLut6_Forward(int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
                                  int node_size, int frame_size, int frame_stride, void *stream);
 
+/* BinaryLutN<N> for n = 2 .. 6 on packed bits.  The reference has a device entry for n = 6 only (above; n = 6 is forwarded to it) and runs
+ * the other widths in its generic host loop (include/bb/BinaryLutN.h:436-463), which is what this entry computes: input k of a node is
+ * bit k of the table index, dev_table is [node_size][1] words for n <= 5 (entry i = bit i), [node_size][2] for n = 6.  With it a layer
+ * trained at any width (StochasticLutN / DifferentiableLutN, n = 2 .. 6) can be tabulated and run packed on the device. */
+int bbhip_bit_BinaryLutN_Forward(int n, int const *dev_x_buf, int *dev_y_buf, int const *dev_input_index, int const *dev_table,
+                                 int node_size, int frame_size, int frame_stride, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

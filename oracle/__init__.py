@@ -693,6 +693,17 @@ def reverse_table(n, idx, input_node_size):
 #  the real reference headers (oracle/_ref/libbbref.so) — dense [nodes, frames] arrays, no stride
 # ----------------------------------------------------------------------------------------------
 
+def binary_lutn_forward(n, xbits, idx, table, frame_size):
+    """BinaryLutN<n>, n = 2 .. 6: packed x [I, stride_words] -> packed y [O, stride_words]; table [O, (2^n + 31) // 32] words, entry i = bit
+    i & 31 of word i >> 5; bits of frames >= frame_size stay zero (the reference's generic loop, include/bb/BinaryLutN.h:436-463)."""
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); table = _c(table, np.int32)
+    O = idx.shape[0]; stride = xbits.shape[1]
+    assert idx.shape[1] == n and table.shape == (O, ((1 << n) + 31) // 32)
+    y = np.zeros((O, stride), np.int32)
+    lib().oracle_bit_BinaryLutN_Forward(C.c_int(n), _ptr(xbits), _ptr(y), _ptr(idx), _ptr(table), C.c_int(O), C.c_int(frame_size), C.c_int(stride))
+    return y
+
+
 def ref_stochastic_lut(n, x, idx, W, dy=None, dW_init=None, bit_input=False, binary_mode=False, lut_binarize=False,
                        host_simd=True, frame_size=None):
     """Runs bb::StochasticLutN<n,...>::Forward (+Backward). Returns dict(y, W, dx, dW)."""
@@ -751,6 +762,17 @@ def ref_binary_lut6(xbits, idx, table, frame_size, host_simd=True):
     y = np.zeros((O, xbits.shape[1]), np.int32)
     rc = ref().bbref_BinaryLut6(C.c_int(I), C.c_int(O), C.c_int(frame_size), _ptr(xbits), _ptr(idx), _ptr(table), _ptr(y),
                                 C.c_int(int(host_simd)))
+    assert rc == 0
+    return y
+
+
+def ref_binary_lutn(n, xbits, idx, table, frame_size):
+    """bb::BinaryLutN<n, Bit>::Forward of the reference (host path), n = 2 .. 6; dense packed arrays [rows, ceil(frames / 32)]"""
+    xbits = _c(xbits, np.int32); idx = _c(idx, np.int32); table = _c(table, np.int32)
+    I = xbits.shape[0]; O = idx.shape[0]
+    assert xbits.shape[1] == (frame_size + 31) // 32 and idx.shape[1] == n
+    y = np.zeros((O, xbits.shape[1]), np.int32)
+    rc = ref().bbref_BinaryLutN(C.c_int(n), C.c_int(I), C.c_int(O), C.c_int(frame_size), _ptr(xbits), _ptr(idx), _ptr(table), _ptr(y))
     assert rc == 0
     return y
 

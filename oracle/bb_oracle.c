@@ -605,6 +605,26 @@ void oracle_bit_BinaryLut6_Forward(int32_t const *x, int32_t *y, int32_t const *
     }
 }
 
+/* The same loop for any width n = 2 .. 6 (BinaryLutN<N,Bit>::Forward is this loop for every N but 6 with host_simd,
+ * include/bb/BinaryLutN.h:436-463): a node's table is (2^n + 31) / 32 words, entry i = bit i & 31 of word i >> 5 (:43-46, 170-171). */
+void oracle_bit_BinaryLutN_Forward(int n, int32_t const *x, int32_t *y, int32_t const *idx, int32_t const *table,
+                                   int node_size, int frame_size, int frame_stride)
+{
+    int const unit = ((1 << n) + 31) / 32;
+    #pragma omp parallel for
+    for (int node = 0; node < node_size; ++node) {
+        for (int f = 0; f < frame_size; ++f) {
+            int index = 0, mask = 1;
+            for (int i = 0; i < n; ++i) {
+                if (read_bit(x + (size_t)idx[node * n + i] * frame_stride, f)) { index |= mask; }
+                mask <<= 1;
+            }
+            int v = (int)(((uint32_t)table[node * unit + (index >> 5)] >> (index & 31)) & 1u);
+            write_bit(y + (size_t)node * frame_stride, f, v);
+        }
+    }
+}
+
 /* Word-parallel form of the AVX2 loop (BinaryLutN.h:322-433): y = OR_k (T_k & AND_j (bit_j(k) ? x_j : ~x_j)),
  * evaluated on whole 32-bit words, padding bits included — used as the timed CPU baseline. */
 void oracle_bit_BinaryLut6_Forward_words(int32_t const *x, int32_t *y, int32_t const *idx, int32_t const *table,

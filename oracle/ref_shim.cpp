@@ -208,6 +208,25 @@ int run_differentiable(int I, int O, int F, void const *x, std::int32_t const *i
 }  // namespace
 
 
+// BinaryLutN<N,Bit>::Forward for any width N = 2 .. 6 (host path; N = 6 with its AVX2 loop); table [O][(2^N + 31) / 32] words
+template <int N>
+static int binary_lut_n(int I, int O, int F, std::int32_t const *x, std::int32_t const *idx, std::int32_t const *table, std::int32_t *y)
+{
+    auto lut = bb::BinaryLutN<N, bb::Bit, float>::Create((index_t)O);
+    lut->SendCommand("host_only true");
+    bb::FrameBuffer x_buf((index_t)F, {(index_t)I}, BB_TYPE_BIT, true);
+    lut->SetInputShape(x_buf.GetShape());
+    int const unit = ((1 << N) + 31) / 32;
+    for (int nd = 0; nd < O; ++nd) {
+        for (int i = 0; i < N; ++i) { lut->SetNodeConnectionIndex(nd, i, idx[nd * N + i]); }
+        for (int b = 0; b < (1 << N); ++b) { lut->SetLutTable(nd, b, ((table[nd * unit + (b >> 5)] >> (b & 31)) & 1) != 0); }
+    }
+    put_bit(x_buf, x, I, (F + 31) / 32);
+    auto y_buf = lut->Forward(x_buf, false);
+    get_bit(y_buf, y, O, (F + 31) / 32);
+    return 0;
+}
+
 extern "C" {
 
 // StochasticLutN<N,float|Bit,float>::Forward (+Backward when dy != NULL) on the host-only path.
@@ -284,6 +303,18 @@ int bbref_BinaryLut6(int I, int O, int F, std::int32_t const *x, std::int32_t co
     auto y_buf = lut->Forward(x_buf, false);
     get_bit(y_buf, y, O, (F + 31) / 32);
     return 0;
+}
+
+int bbref_BinaryLutN(int n, int I, int O, int F, std::int32_t const *x, std::int32_t const *idx, std::int32_t const *table, std::int32_t *y)
+{
+    switch (n) {
+    case 2: return binary_lut_n<2>(I, O, F, x, idx, table, y);
+    case 3: return binary_lut_n<3>(I, O, F, x, idx, table, y);
+    case 4: return binary_lut_n<4>(I, O, F, x, idx, table, y);
+    case 5: return binary_lut_n<5>(I, O, F, x, idx, table, y);
+    case 6: return binary_lut_n<6>(I, O, F, x, idx, table, y);
+    }
+    return 1;
 }
 
 // FixedSizeConnectionTable<6>: reverse table for a given input table.

@@ -286,27 +286,43 @@ static void test_binary(int I, int O, int F)
     CHECK(mism == 0, "BinaryLut6 %dx%dx%d: %zu mismatching bits", I, O, F, mism);
 }
 
-// trained-layer hand-off: a StochasticLut6 with binarized tables tabulated into a BinaryLut6 gives the same bits
+// trained-layer hand-off at every width: a StochasticLut<N> with binarized tables tabulated into a BinaryLut<N> gives the same bits,
+// and the tabulated layer survives a trip through a stream under its own type name
+template <int N>
 static void test_import_layer(void)
 {
     int const I = 32, O = 24, F = 200;
-    std::mt19937_64 mt(5);
+    std::mt19937_64 mt(5 + N);
     std::uniform_real_distribution<float> uni(0.0f, 1.0f);
-    auto src = bb::StochasticLutN<6, bb::Bit>::Create(O);
+    auto src = bb::StochasticLutN<N, bb::Bit>::Create(O);
     src->SendCommand("lut_binarize true");
     bb::FrameBuffer x_buf(F, {I}, BB_TYPE_BIT);
     src->SetInputShape(x_buf.GetShape());
-    { auto Wp = src->lock_W(); for (int k = 0; k < O * 64; ++k) { Wp[k] = uni(mt); } }
+    { auto Wp = src->lock_W(); for (int k = 0; k < O * (1 << N); ++k) { Wp[k] = uni(mt); } }
     { auto xp = x_buf.Lock<bb::Bit>(true); for (int n = 0; n < I; ++n) for (int f = 0; f < F; ++f) { xp.Set(f, n, bb::Bit((mt() & 1) != 0)); } }
-    auto dst = bb::BinaryLutN<6, bb::Bit>::Create(O);
+    auto dst = bb::BinaryLutN<N, bb::Bit>::Create(O);
     dst->SetInputShape(x_buf.GetShape());
+    CHECK(dst->GetLutTableSize(0) == (1 << N) && dst->GetNodeConnectionSize(0) == N, "BinaryLut%d: table size and fan-in", N);
     dst->ImportLayer(src);
     auto y_src = src->Forward(x_buf, false);          // fp32 in [0,1]; with binarized tables and bits at 0.5+-0.25 it is > 0.5 iff the table bit is 1
     auto y_dst = dst->Forward(x_buf);
-    auto a = y_src.LockConst<float>(); auto b = y_dst.LockConst<bb::Bit>();
-    size_t mism = 0;
-    for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { mism += ((a.Get(f, n) > 0.5f) != (bool)b.Get(f, n)); }
-    CHECK(mism == 0, "ImportLayer: %zu mismatching bits", mism);
+    {
+        auto a = y_src.template LockConst<float>(); auto b = y_dst.template LockConst<bb::Bit>();
+        size_t mism = 0;
+        for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { mism += ((a.Get(f, n) > 0.5f) != (bool)b.Get(f, n)); }
+        CHECK(mism == 0, "ImportLayer<%d>: %zu mismatching bits", N, mism);
+    }
+    std::stringstream ss;
+    dst->DumpObject(ss);
+    auto again = std::dynamic_pointer_cast<bb::BinaryLutN<N, bb::Bit>>(bb::Object_Load(ss));
+    CHECK((bool)again && again->GetObjectName() == "BinaryLut" + std::to_string(N) + "_bit_fp32", "BinaryLut%d does not come back from a stream", N);
+    if (again) {
+        auto y_again = again->Forward(x_buf);
+        auto a = y_dst.template LockConst<bb::Bit>(); auto b = y_again.template LockConst<bb::Bit>();
+        size_t mism = 0;
+        for (int n = 0; n < O; ++n) for (int f = 0; f < F; ++f) { mism += ((bool)a.Get(f, n) != (bool)b.Get(f, n)); }
+        CHECK(mism == 0, "BinaryLut%d: output differs after a trip through a stream (%zu bits)", N, mism);
+    }
 }
 
 // Shaped like the reference's optimizer test (tests/gtest/OptimizerAdamTest.cpp:44-96): parameters follow a model of the
@@ -1155,7 +1171,11 @@ int main(void)
         test_packed_twin(27, 216, 36, 5000);
         test_binary(16, 16, 32);
         test_binary(70, 33, 1000);
-        test_import_layer();
+        test_import_layer<6>();
+        test_import_layer<5>();
+        test_import_layer<4>();
+        test_import_layer<3>();
+        test_import_layer<2>();
         test_adam();
         test_conv_plumbing();
         test_convolution2d();
