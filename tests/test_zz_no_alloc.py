@@ -11,9 +11,8 @@ from util import dev, host
 pytestmark = pytest.mark.gpu
 
 
-def _forward(entry, n, x, idx, W, O, F, stride, input_binary, lut_binarize):
+def _forward(entry, n, x, idx, W, y, O, F, stride, input_binary, lut_binarize):
     import torch
-    y = torch.full((O, stride), -7.0, device="cuda")
     check(getattr(lib(), entry)(n, ptr(x), ptr(y), ptr(idx), ptr(W), O, F, stride, input_binary, lut_binarize, 0.25, stream_ptr()))
     torch.cuda.synchronize()
     return host(y)
@@ -21,13 +20,25 @@ def _forward(entry, n, x, idx, W, O, F, stride, input_binary, lut_binarize):
 
 @pytest.mark.parametrize("input_binary,lut_binarize", [(0, 0), (1, 0), (0, 1)])
 def test_no_alloc_forward_equals_forward(input_binary, lut_binarize):
+    import torch
     rng = np.random.default_rng(31 + input_binary + 2 * lut_binarize)
     for n, I, O, F in ((6, 300, 2000, 1100), (6, 64, 70, 130), (4, 50, 33, 64)):      # second and third calls: smaller layers
         stride = synth.frame_stride_fp32(F)
         idx = dev(synth.wiring(rng, I, O, n)); W = dev(synth.lut_tables(rng, O, n))
         x = dev(synth.uniform_frames(rng, I, F, stride, -0.1, 1.1))
-        want = _forward("bbhip_fp32_StochasticLut_Forward", n, x, idx, W, O, F, stride, input_binary, lut_binarize)
-        got = _forward("bbhip_fp32_StochasticLut_Forward_NoAlloc", n, x, idx, W, O, F, stride, input_binary, lut_binarize)
+        y_got = torch.full((O, stride), -7.0, device="cuda"); y_want = torch.full((O, stride), -7.0, device="cuda")
+        # The call must allocate nothing: with the library's own scratch arena given back first, it may not grow it again, and the
+        # device's free memory is the same after the call as before (the outputs were allocated above).
+        capi.check(lib().bbhip_fp32_Vector_set(ptr(y_want), -7.0, 1, stream_ptr()))     # (in a fresh process: the library's code is loaded by its first launch)
+        torch.cuda.synchronize()
+        check(lib().bbhip_ReleaseScratch())
+        assert lib().bbhip_GetScratchSize() == 0
+        free_before = torch.cuda.mem_get_info()[0]
+        got = _forward("bbhip_fp32_StochasticLut_Forward_NoAlloc", n, x, idx, W, y_got, O, F, stride, input_binary, lut_binarize)
+        assert lib().bbhip_GetScratchSize() == 0, "the entry that allocates nothing grew the scratch arena"
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated during the call"
+        want = _forward("bbhip_fp32_StochasticLut_Forward", n, x, idx, W, y_want, O, F, stride, input_binary, lut_binarize)
+        assert lib().bbhip_GetScratchSize() > 0                       # (the arena path does use the arena)
         # same kernels, same tables: identical bits (with input_binary the arena path may pack the input first when it is
         # told the row count; it is not told here)
         assert np.array_equal(got[:, :F], want[:, :F]), (n, I, O, F)
