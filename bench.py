@@ -29,10 +29,14 @@ TRAFFIC_WORKLOADS = {          # workload -> (extra bench arguments, kernel that
     "mnist_step": ("", "adam_kernel"),
     "conv_block": ("", "im2col_backward_kernel"),
 }
-TRAFFIC_COMMANDS = [
-    "rocprofv3 --pmc %s -d gpurun_out/traffic/%s/%s -o r -- python3 bench.py --workload %s --steps 5 --warmup 5 --ramp-seconds 0 --no-cpu %s"
-    % (counter, w, counter, w, extra) for w, (extra, _) in TRAFFIC_WORKLOADS.items() for counter in ("FETCH_SIZE", "WRITE_SIZE")
-] + ["python3 bench.py --write-traffic gpurun_out/traffic"]
+def traffic_commands(dirname="traffic_runs"):
+    """the counter runs behind profiles/traffic.json (one counter per run), then the call that writes the file from them"""
+    runs = ["rocprofv3 --pmc %s -d %s/%s/%s -o r -- python3 bench.py --workload %s --steps 5 --warmup 5 --ramp-seconds 0 --no-cpu %s"
+            % (counter, dirname, w, counter, w, extra) for w, (extra, _) in TRAFFIC_WORKLOADS.items() for counter in ("FETCH_SIZE", "WRITE_SIZE")]
+    return runs + ["python3 bench.py --write-traffic %s" % dirname]
+
+
+TRAFFIC_COMMANDS = traffic_commands()
 
 
 def _git_blob_hash(path):
