@@ -40,6 +40,14 @@ def main():
     dW = dev(np.zeros((O, 64), np.float32))
     dx = ops.differentiable_lut_backward(6, dev(x), dev(dy), dev(idx), dev(W), dW, F, dev(m_ref), dev(r_ref), rev)
     assert_bwd(host(dx)[:, :F], dx_ref[:, :F], "binary dx"); assert_bwd(host(dW), dW_ref, "binary dW")
+    # the binarized output as packed bits as well, under whichever kernels serve the call: the bits of y > 0.5, zeros behind the last frame
+    for kw in ({}, {"packed": ops.packed_input_buffer(I, F)}):
+        bits = ops.packed_input_buffer(O, F); bits.fill_(0x5a5a5a5a)
+        y2, _, _ = ops.differentiable_lut_forward_training(6, dev(x), dev(idx), dev(W), F, torch.zeros(O, device="cuda"), torch.ones(O, device="cuda"),
+                                                           packed_out=bits, **kw)
+        assert torch.equal(y2[:, :F], y[:, :F])
+        nw = (F + 31) // 32
+        assert np.array_equal(host(bits)[:, :nw], oracle.binarize_forward(host(y2), F, 0.5, bit=True)[:, :nw]) and not host(bits)[:, nw:].any()
     # continuous fp32 frames (the polynomial kernels under whatever unit sizes the environment sets)
     xc = synth.uniform_frames(rng, I, F, ys, -0.1, 1.1)
     assert_fwd(host(ops.stochastic_lut_forward(6, dev(xc), dev(idx), dev(W), F))[:, :F], oracle.stochastic_lut_forward(6, xc, idx, W, F, 0, 0, 0.25, False)[:, :F], "fp32")
