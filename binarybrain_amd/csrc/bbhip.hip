@@ -254,6 +254,12 @@ void launch_forward(FwdArgs const &a, int npw, hipStream_t st)
     if constexpr (XMODE == kXBit || XMODE == kXBinary) {
         // two-valued inputs: the corner-value kernel wherever the caller prepared the values (one node per wavefront)
         if (a.V != nullptr) {
+            if constexpr (XMODE == kXBit && YMODE == kYBinarize && KIND == 1) {
+                if (a.own_index != nullptr) {      // corner indices kept by the statistics launch of the same call
+                    hipLaunchKernelGGL((lut_forward_corner_kernel<N, XMODE, YMODE, KIND, false, kOwnMemory>), grid, block, 0, st, a);
+                    return;
+                }
+            }
             if constexpr (XMODE == kXBit) {
                 // 32-byte scalar loads where they stay inside the row pitch and never straddle a unit
                 if (a.x_stride % 8 == 0 && a.chunk % 256 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 3u) == 0) {
@@ -363,6 +369,8 @@ struct ForwardCall {
 
 // the kernels address a frame inside its node row with a 32-bit byte offset
 constexpr int kMaxFrames = 1 << 29;
+// most scratch that a forward call takes for the corner indices that its statistics launch keeps for its output launch (run_forward)
+constexpr size_t kOwnIndexMaxBytes = (size_t)1 << 30;
 
 int check_forward(ForwardCall const &c)
 {
@@ -468,8 +476,16 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     size_t const v_bytes    = corner ? c_bytes : 0;
     size_t const stat_bytes = (c.bn == 1) ? align256((size_t)chunk_count * c.node_size * 2 * sizeof(float)) : 0;
     size_t const bits_bytes = (pack && !to_caller) ? align256((size_t)input_rows * c.x_stride * sizeof(uint32_t)) : 0;
+    // fp32 frames of binary mode whose row count nobody told (nothing to pack ahead), batch-norm training pass in two launches: the
+    // statistics launch keeps the corner index that it forms of every (node, frame), a byte each, and the output launch reads those
+    // instead of gathering the fp32 frames again (FwdArgs::own_index_out).  Up to kOwnIndexMaxBytes of scratch.
+    int const own_words = ceil_div(c.frame_size, 256) * kWave;
+    bool const own_index = (c.xmode == kXBinary) && corner && pack_binarized_input() && c.bn == 1 && !one_unit && chunk_count > 1 &&
+                           chunk % 256 == 0 && c.ymode == kYBinarize && fixed == nullptr &&
+                           (size_t)c.node_size * own_words * sizeof(uint32_t) <= kOwnIndexMaxBytes;
+    size_t const own_bytes = own_index ? align256((size_t)c.node_size * own_words * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + v_bytes + stat_bytes + bits_bytes, &base, st, fixed)) { return 1; }
+    if (arena_get(c_bytes + v_bytes + stat_bytes + bits_bytes + own_bytes, &base, st, fixed)) { return 1; }
     float *C        = reinterpret_cast<float *>(base);
     float *V        = corner ? reinterpret_cast<float *>(base + c_bytes) : nullptr;
     float *stat     = reinterpret_cast<float *>(base + c_bytes + v_bytes);
@@ -518,9 +534,19 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     }
     else if (c.bn == 1) {
         a.stat_partial = stat;
+        if (own_index) { a.own_index_out = reinterpret_cast<uint32_t *>(base + c_bytes + v_bytes + stat_bytes + bits_bytes); a.own_stride = own_words; }
         if (dispatch_forward<N>(c.xmode, kYClamp, 2, a, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
         if (inline_corner) { a.W_inline = nullptr; a.C_out = nullptr; a.V_out = nullptr; a.clamp_W = nullptr; }      // stored by that launch
+        if (own_index) {
+            // the output launch reads the kept indices, a coalesced word per lane and four steps: longer units than the gathers of
+            // fp32 frames want (a unit's set-up weighs less), halved while they would leave the launch short of workgroups
+            a.own_index = a.own_index_out; a.own_index_out = nullptr; a.stat_units = chunk_count;
+            c.xmode = kXBit;
+            int own_chunk = 1024;
+            while (own_chunk > 256 && (long long)ceil_div(c.frame_size, own_chunk) * tile_count < 2048) { own_chunk /= 2; }
+            a.chunk = own_chunk; a.chunk_count = ceil_div(c.frame_size, own_chunk);
+        }
         if (chunk_count <= kInlineStatUnits) {
             // few units: every wavefront of the output pass adds up the partial sums of its node itself, and the wavefront of a
             // node's first unit stores the statistics; a launch that does it once per node would cost more than that

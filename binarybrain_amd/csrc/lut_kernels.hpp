@@ -230,11 +230,22 @@ struct FwdArgs {
     // copy that the next layer would otherwise make of y before it reads it
     uint32_t *y_bits;
     int   y_bits_stride;
+    // lut_forward_corner_kernel on fp32 frames, statistics kind: not null = the corner index that each lane forms of its frame's
+    // inputs is kept, one byte per (node, frame) (the index times 4, as ds_bpermute takes it): word (f / 256) * 64 + l of a node's
+    // row of own_stride words holds frames f + l, f + 64 + l, f + 128 + l, f + 192 + l.  The output launch of the same call
+    // (own_index: the same buffer) then reads a word per lane and four steps instead of gathering the fp32 frames a second time.
+    // Units of both launches begin at multiples of 256 frames.  Needs no count of the input's rows.
+    uint32_t       *own_index_out;
+    uint32_t const *own_index;
+    int   own_stride;
+    // kStatPartial: units per node of the launch that left the partial sums, where the output launch has other units (0: the same)
+    int   stat_units;
 };
 
 // kStatInline: the call has one unit per node, so the wavefront that writes a node's output first sums the node's statistics
 // itself (a pass of its own over the unit) instead of reading them from a statistics launch
 enum StatMode : int { kStatGiven = 0, kStatRunning = 1, kStatPartial = 2, kStatInline = 3 };
+constexpr int kInlineUnitPasses = 4;         // kStatInline over fp32 frames: passes (of 256 frames) whose corner indices a wavefront keeps in registers
 constexpr int kInlineStatUnits = 4 * kWave; // most units whose partial sums a wavefront adds up itself: up to four loads per lane
 
 // What a forward kernel does with the LUT output v of (node, frame f = f0 + lane): accumulate statistics (kinds 2, 3) or
@@ -359,7 +370,7 @@ __device__ __forceinline__ void forward_statistics(FwdArgs const &a, int node, i
     var = 0.0f;
     if (a.stat_mode == kStatPartial) {
         float s1, s2;
-        wave_stat_sums(a.stat_partial, a.node_size, a.chunk_count, node, lane, s1, s2);
+        wave_stat_sums(a.stat_partial, a.node_size, a.stat_units > 0 ? a.stat_units : a.chunk_count, node, lane, s1, s2);
         batch_statistics(s1, s2, c0, a.frame_size, mean, var, rstd);
     }
     else {
@@ -538,45 +549,71 @@ __device__ __forceinline__ uint32_t corner_index(Raw const (&raw)[N])
     return index;
 }
 
-// One pass of a corner-value wavefront over its unit (see lut_forward_corner_kernel): KIND says what is done with the LUT
-// output of a frame (forward_stage).
-template <int N, int XMODE, int YMODE, int KIND, bool WIDE>
+// A corner-value wavefront's pass over U wavefront-steps from frame fb of its unit (see lut_forward_corner_kernel): KIND says what is
+// done with the LUT output of a frame (forward_stage).
+// OWN: where the corner indices come from.  kOwnNone: from the gathered inputs; kOwnMemory: from the bytes that the statistics launch
+// of the call kept (FwdArgs::own_index); kOwnRegister: from `own`, which an earlier pass of the same wavefront over the same frames
+// left there.  `own` always returns the indices of the pass, byte u = 4 x the index of frame fb + 64 u + lane.
+enum OwnIndex : int { kOwnNone = 0, kOwnMemory = 1, kOwnRegister = 2 };
+template <int N, int XMODE, int YMODE, int KIND, bool WIDE, int OWN>
+__device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows)[N], int corner, int node, int lane, int fb,
+                                            int f_end, int f_last, float mean, float rstd, float c0, float &s1, float &s2, uint32_t &own)
+{
+    constexpr int U = (XMODE == kXBit && !WIDE && OWN == kOwnNone) ? 2 : 4;  // wavefront-steps whose loads are issued together
+    typename Gather<N, XMODE>::Raw raw[U][N];
+    float dyv[U];
+    if constexpr (OWN == kOwnNone)   { own = 0; }
+    if constexpr (OWN == kOwnMemory) { own = a.own_index[(size_t)node * a.own_stride + (fb >> 8) * kWave + lane]; }
+    if constexpr (WIDE && OWN == kOwnNone) { corner_masks_wide<N>(rows, fb, raw); }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
+            if constexpr (!WIDE && OWN == kOwnNone) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
+            if (KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
+        }
+    }
+    constexpr bool kPackedCopy = (YMODE == kYBinarize) && (KIND == 0 || KIND == 1);
+    uint32_t words = 0;                                  // lane l < 2 U: word l of the pass's packed output
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        int const f0 = fb + u * kWave;
+        if (f0 >= f_end) { break; }
+        int const  f  = f0 + lane;
+        bool const ok = f < f_end;
+        uint32_t index4;
+        if constexpr (OWN != kOwnNone) { index4 = (own >> (8 * u)) & 0xffu; }
+        else {
+            index4 = corner_index<N, XMODE>(raw[u]) << 2;
+            if (U == 4) { own |= index4 << (8 * u); }
+        }
+        float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index4, corner));
+        uint64_t m = 0;
+        forward_stage<YMODE, KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
+                                   (KIND == 3) ? dyv[u] : 0.0f, s1, s2, kPackedCopy ? &m : nullptr);
+        if (kPackedCopy) {
+            asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)m), "n"(2 * u));               // words[lane 2u] = low half
+            asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)(m >> 32)), "n"(2 * u + 1));
+        }
+    }
+    // the packed copy of the pass: its 2 U words by one store (a store per step would double the kernel's store instructions)
+    if (kPackedCopy && a.y_bits != nullptr && lane < 2 * U && fb + 32 * lane < f_end) {
+        a.y_bits[(size_t)node * a.y_bits_stride + (fb >> 5) + lane] = words;
+    }
+}
+
+// The passes of a corner-value wavefront over its unit.  OWN as in corner_pass (kOwnNone or kOwnMemory); the statistics kind over
+// fp32 frames keeps its corner indices for the output launch where the call asks for it (FwdArgs::own_index_out).
+template <int N, int XMODE, int YMODE, int KIND, bool WIDE, int OWN = kOwnNone>
 __device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(&rows)[N], int corner, int node, int lane,
                                                  int f_begin, int f_end, int f_last, float mean, float rstd, float c0, float &s1, float &s2)
 {
-    constexpr int U = (XMODE == kXBit && !WIDE) ? 2 : 4;  // wavefront-steps whose loads are issued together
+    constexpr int U = (XMODE == kXBit && !WIDE && OWN == kOwnNone) ? 2 : 4;
+    constexpr bool kKeepIndex = (XMODE == kXBinary) && (KIND == 2);
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
-        typename Gather<N, XMODE>::Raw raw[U][N];
-        float dyv[U];
-        if constexpr (WIDE) { corner_masks_wide<N>(rows, fb, raw); }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
-                if constexpr (!WIDE) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
-                if (KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
-            }
-        }
-        constexpr bool kPackedCopy = (YMODE == kYBinarize) && (KIND == 0 || KIND == 1);
-        uint32_t words = 0;                                  // lane l < 2 U: word l of the pass's packed output
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int const f0 = fb + u * kWave;
-            if (f0 >= f_end) { break; }
-            int const  f  = f0 + lane;
-            bool const ok = f < f_end;
-            uint32_t const index = corner_index<N, XMODE>(raw[u]);
-            float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(index << 2), corner));
-            uint64_t m = 0;
-            forward_stage<YMODE, KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
-                                       (KIND == 3) ? dyv[u] : 0.0f, s1, s2, kPackedCopy ? &m : nullptr);
-            if (kPackedCopy) {
-                asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)m), "n"(2 * u));               // words[lane 2u] = low half
-                asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)(m >> 32)), "n"(2 * u + 1));
-            }
-        }
-        // the packed copy of the pass: its 2 U words by one store (a store per step would double the kernel's store instructions)
-        if (kPackedCopy && a.y_bits != nullptr && lane < 2 * U && fb + 32 * lane < f_end) {
-            a.y_bits[(size_t)node * a.y_bits_stride + (fb >> 5) + lane] = words;
+        uint32_t own;
+        corner_pass<N, XMODE, YMODE, KIND, WIDE, OWN>(a, rows, corner, node, lane, fb, f_end, f_last, mean, rstd, c0, s1, s2, own);
+        if (kKeepIndex && a.own_index_out != nullptr) {      // (wave-uniform; steps beyond the unit left their byte 0)
+            a.own_index_out[(size_t)node * a.own_stride + (fb >> 8) * kWave + lane] = own;
         }
     }
 }
@@ -590,11 +627,14 @@ __device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(
 // ------------------------------------------------------------------------------------------------
 //  WIDE (packed bits, row pitch a multiple of 8 words, units a multiple of 256 frames): the bits of 256 frames of an input
 //  are one 32-byte scalar load, so a unit costs N scalar loads per four steps instead of 2 N per step.
-template <int N, int XMODE, int YMODE, int FWD_KIND, bool WIDE = false>
+//  OWN (output launch of a batch-norm training pass over fp32 frames): the corner indices are read from the bytes that the
+//  statistics launch kept (FwdArgs::own_index); instantiated on the packed-bit mode, whose gathers it does not use.
+template <int N, int XMODE, int YMODE, int FWD_KIND, bool WIDE = false, int OWN = kOwnNone>
 __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
 {
     static_assert(XMODE == kXBit || XMODE == kXBinary, "corner values need two-valued inputs");
     static_assert(!WIDE || XMODE == kXBit, "wide loads are for packed bits");
+    static_assert(OWN == kOwnNone || (OWN == kOwnMemory && XMODE == kXBit && !WIDE && FWD_KIND == 1), "kept corner indices: output launch only");
     constexpr int NN = 1 << N;
     int const B    = a.chunk_count * a.tiles.count;
     int const lid  = xcd_remap(blockIdx.x, B);
@@ -629,7 +669,7 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
     void const *rows[N];
 #pragma unroll
     for (int k = 0; k < N; ++k) {
-        int const in = a.idx[node * N + k];
+        int const in = (OWN == kOwnMemory) ? 0 : a.idx[node * N + k];
         rows[k] = (XMODE == kXBit) ? (void const *)(reinterpret_cast<uint32_t const *>(a.x) + (size_t)in * a.x_stride)
                                    : (void const *)(reinterpret_cast<float const *>(a.x) + (size_t)in * a.x_stride);
     }
@@ -643,23 +683,49 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
     int const f_end   = min(f_begin + a.chunk, a.frame_size);
     int const f_last  = a.frame_size - 1;
     float s1 = 0.0f, s2 = 0.0f;
+    bool f_done = false;
 
     if (FWD_KIND == 1) {
         if (a.stat_mode == kStatInline) {
             // one unit per node: the sums of the statistics kind, by the same steps in the same order, then what the
             // statistics launch and the partial-sum read would have delivered (same bits)
-            corner_unit_pass<N, XMODE, YMODE, 2, WIDE>(a, rows, corner, node, lane, f_begin, f_end, f_last, 0.0f, 1.0f, c0, s1, s2);
+            // fp32 frames, up to kInlineUnitPasses passes: the corner indices of the passes stay in registers for the output pass,
+            // which then gathers nothing
+            constexpr bool kKeep = (XMODE == kXBinary) && (OWN == kOwnNone);
+            bool const keep = kKeep && (f_end - f_begin <= kInlineUnitPasses * 4 * kWave);      // wave-uniform
+            uint32_t kept[kInlineUnitPasses];
+            if (keep) {
+                if constexpr (kKeep) {
+#pragma unroll
+                    for (int q = 0; q < kInlineUnitPasses; ++q) {
+                        int const fb = f_begin + q * 4 * kWave;
+                        kept[q] = 0;
+                        if (fb < f_end) { corner_pass<N, XMODE, YMODE, 2, WIDE, kOwnNone>(a, rows, corner, node, lane, fb, f_end, f_last, 0.0f, 1.0f, c0, s1, s2, kept[q]); }
+                    }
+                }
+            }
+            else { corner_unit_pass<N, XMODE, YMODE, 2, WIDE, OWN>(a, rows, corner, node, lane, f_begin, f_end, f_last, 0.0f, 1.0f, c0, s1, s2); }
             batch_statistics(wave_sum(s1), wave_sum(s2), c0, a.frame_size, mean, var, rstd);
             mean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mean)));
             var  = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(var)));
             rstd = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(rstd)));
             s1 = 0.0f; s2 = 0.0f;
+            if (keep) {
+                if constexpr (kKeep) {
+#pragma unroll
+                    for (int q = 0; q < kInlineUnitPasses; ++q) {
+                        int const fb = f_begin + q * 4 * kWave;
+                        if (fb < f_end) { corner_pass<N, XMODE, YMODE, FWD_KIND, WIDE, kOwnRegister>(a, rows, corner, node, lane, fb, f_end, f_last, mean, rstd, c0, s1, s2, kept[q]); }
+                    }
+                }
+                f_done = true;
+            }
         }
         else { forward_statistics(a, node, lane, c0, mean, var, rstd); }
     }
     if (FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
 
-    corner_unit_pass<N, XMODE, YMODE, FWD_KIND, WIDE>(a, rows, corner, node, lane, f_begin, f_end, f_last, mean, rstd, c0, s1, s2);
+    if (!f_done) { corner_unit_pass<N, XMODE, YMODE, FWD_KIND, WIDE, OWN>(a, rows, corner, node, lane, f_begin, f_end, f_last, mean, rstd, c0, s1, s2); }
     if (FWD_KIND == 2 || FWD_KIND == 3) { forward_store_stats(a, ck, node, true, lane, s1, s2); }
     if (FWD_KIND == 1) { forward_store_statistics(a, node, true, ck, lane, mean, var, rstd); }
     if (YMODE == kYBinarize && (FWD_KIND == 0 || FWD_KIND == 1)) { zero_packed_tail(a, ck, node, true, lane); }
