@@ -15,7 +15,7 @@ from util import assert_bwd, dev, host, rel_err
 
 pytestmark = pytest.mark.gpu
 
-FRAMES = [1, 39, 64, 1024, 32, 131]
+FRAMES = [1, 39, 64, 1024, 32, 131, 2048 + 17]     # (the last: several units per node, ragged last pass)
 
 
 @pytest.fixture(scope="module")
