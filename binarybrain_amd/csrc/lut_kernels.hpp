@@ -245,7 +245,7 @@ struct FwdArgs {
 // kStatInline: the call has one unit per node, so the wavefront that writes a node's output first sums the node's statistics
 // itself (a pass of its own over the unit) instead of reading them from a statistics launch
 enum StatMode : int { kStatGiven = 0, kStatRunning = 1, kStatPartial = 2, kStatInline = 3 };
-constexpr int kInlineUnitPasses = 4;         // kStatInline over fp32 frames: passes (of 256 frames) whose corner indices a wavefront keeps in registers
+constexpr int kInlineUnitPasses = 4;         // kStatInline: passes (of 256 frames) whose corner indices a wavefront keeps in registers
 constexpr int kInlineStatUnits = 4 * kWave; // most units whose partial sums a wavefront adds up itself: up to four loads per lane
 
 // What a forward kernel does with the LUT output v of (node, frame f = f0 + lane): accumulate statistics (kinds 2, 3) or
@@ -689,9 +689,9 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
         if (a.stat_mode == kStatInline) {
             // one unit per node: the sums of the statistics kind, by the same steps in the same order, then what the
             // statistics launch and the partial-sum read would have delivered (same bits)
-            // fp32 frames, up to kInlineUnitPasses passes: the corner indices of the passes stay in registers for the output pass,
+            // up to kInlineUnitPasses passes of four steps: the corner indices of the passes stay in registers for the output pass,
             // which then gathers nothing
-            constexpr bool kKeep = (XMODE == kXBinary) && (OWN == kOwnNone);
+            constexpr bool kKeep = (XMODE == kXBinary || WIDE) && (OWN == kOwnNone);
             bool const keep = kKeep && (f_end - f_begin <= kInlineUnitPasses * 4 * kWave);      // wave-uniform
             uint32_t kept[kInlineUnitPasses];
             if (keep) {
