@@ -502,8 +502,8 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
         c.x = bits;
     }
     // plain output of a call with one unit per node on the polynomial kernel: the wavefronts prepare their node's table
-    // themselves (FwdArgs::W_inline) and the table launch falls away
-    bool const inline_table = (c.bn == 0) && !corner && chunk_count == 1 && LutMatrixQ<N>::kUsable && c.clamp_W == nullptr && !tables_to_caller;
+    // themselves (FwdArgs::W_inline), clamp it in place where the entry asks for that, and the table launch falls away
+    bool const inline_table = (c.bn == 0) && !corner && chunk_count == 1 && LutMatrixQ<N>::kUsable && !tables_to_caller;
     // the corner-value kernel derives a node's tables in the wavefront in any case where no packing launch is there to carry the
     // preparation: the first launch of the call does it and stores them for the launches (and the backward call) that follow
     bool const inline_corner = corner && !pack && inline_tables();
@@ -513,7 +513,7 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
     }
 
     FwdArgs a{};
-    if (inline_table) { a.W_inline = c.W; a.lut_binarize = c.lut_binarize; }
+    if (inline_table) { a.W_inline = c.W; a.lut_binarize = c.lut_binarize; a.clamp_W = c.clamp_W; a.clamp_lo = c.clamp_lo; a.clamp_hi = c.clamp_hi; }
     if (inline_corner) {
         a.W_inline = c.W; a.lut_binarize = c.lut_binarize; a.C_out = C; a.V_out = V;
         a.clamp_W = c.clamp_W; a.clamp_lo = c.clamp_lo; a.clamp_hi = c.clamp_hi;

@@ -219,6 +219,7 @@ struct FwdArgs {
     // Not null (plain output, one unit per node, widths whose table fits one vector register): no table-preparation launch has
     // run; the wavefront brings its node's table W' into the centred basis itself — 2^N loads, one per lane, and the
     // butterfly of table_prep_block over the lanes.  A call of a few hundred frames is two launches' worth of latency, not work.
+    // With clamp_W (below) the table is first clamped and written back, as in the corner-value kernel.
     float const *W_inline;
     int   lut_binarize;
     // lut_forward_corner_kernel with W_inline: the node's tables go to C_out / V_out as well (the wavefront of the node's first unit
@@ -418,6 +419,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     float mean[NPW], rstd[NPW], var[NPW], c0[NPW];
     int node[NPW];
     bool live[NPW];
+    bool clamp_store[NPW];
+    float clamp_w[NPW];
+#pragma unroll
+    for (int p = 0; p < NPW; ++p) { clamp_store[p] = false; clamp_w[p] = 0.0f; }
     // (the statistics first: what they need in registers is gone before the tables arrive)
 #pragma unroll
     for (int p = 0; p < NPW; ++p) {
@@ -433,6 +438,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         if constexpr (kMatrix) {
             if (FWD_KIND == 0 && a.W_inline != nullptr) {
                 float v = a.W_inline[(size_t)node[p] * D::NN + (lane & (D::NN - 1))];
+                if (a.clamp_W != nullptr) {                   // the table clamped in place as well, by the wavefront of the node's first unit
+                    float const wc = fminf(a.clamp_hi, fmaxf(a.clamp_lo, v));
+                    clamp_store[p] = (ck == 0) && live[p] && (lane < D::NN) && (wc != v);
+                    v = wc;
+                    clamp_w[p] = wc;
+                }
                 if (a.lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
 #pragma unroll
                 for (int j = 0; j < N; ++j) {                 // as table_prep_block: (a, b) -> ((a + b) / 2, b - a) per index bit
@@ -513,6 +524,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     if (YMODE == kYBinarize && (FWD_KIND == 0 || FWD_KIND == 1)) {
 #pragma unroll
         for (int p = 0; p < NPW; ++p) { zero_packed_tail(a, ck, node[p], live[p], lane); }
+    }
+    if (FWD_KIND == 0 && kMatrix) {           // (at the end: a store ahead of the unit's loads would be waited for with them)
+#pragma unroll
+        for (int p = 0; p < NPW; ++p) {
+            if (clamp_store[p]) { a.clamp_W[(size_t)node[p] * D::NN + lane] = clamp_w[p]; }
+        }
     }
 }
 

@@ -57,13 +57,14 @@ def test_lut6_forward_backward(ops, shape, lut_binarize, input_binary):
     ops.set_dx_mode(0)
 
 
+@pytest.mark.parametrize("F", [700, 200])     # several units per node (the table launch clamps); one (the wavefronts clamp their node's table)
 @pytest.mark.parametrize("n,input_binary,lut_binarize", [(6, 0, 0), (6, 1, 0), (6, 0, 1), (4, 0, 0), (2, 1, 1)])
-def test_forward_that_clamps_the_table_in_place(ops, n, input_binary, lut_binarize):
+def test_forward_that_clamps_the_table_in_place(ops, n, input_binary, lut_binarize, F):
     """bbhip_fp32_StochasticLut_ForwardClampW = bbhip_fp32_Vector_clamp on W + bbhip_fp32_StochasticLut_Forward, bit for bit
     (what StochasticLutN::Forward does before every pass, include/bb/StochasticLutN.h:451): W afterwards equals the oracle's
     clamp, y equals the forward pass on the clamped table; a table already inside the range is left untouched."""
     rng = np.random.default_rng(77 + n)
-    I, O, F = 40, 37, 700
+    I, O = 40, 37
     stride = synth.frame_stride_fp32(F)
     idx = synth.wiring(rng, I, O, n)
     W0 = synth.lut_tables(rng, O, n, -0.3, 1.3)
