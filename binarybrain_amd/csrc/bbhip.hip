@@ -156,8 +156,14 @@ int fwd_chunk_frames_env(void) { static int env = env_int("BBHIP_FWD_CHUNK", 0);
 int fwd_chunk_frames(int xmode, int frame_size, int tile_count)
 {
     if (fwd_chunk_frames_env() > 0) { return fwd_chunk_frames_env(); }
-    int chunk = (xmode == kXBit) ? 1024 : 256;
-    while (chunk > 256 && (long long)((frame_size + chunk - 1) / chunk) * tile_count < 2048) { chunk /= 2; }
+    int chunk = (xmode == kXBit) ? 2048 : 256;
+    while (chunk > 256 && (long long)((frame_size + chunk - 1) / chunk) * tile_count < 2048) {
+        // ... but not past the number of units whose batch-norm partial sums the wavefronts add up themselves while the launch still
+        // has a thousand workgroups: halving would bring the finalize launches back (5.6 us each) for a few idle compute units
+        int const units = (frame_size + chunk - 1) / chunk;
+        if (units <= kInlineStatUnits && 2 * units > kInlineStatUnits && (long long)units * tile_count >= 1024) { break; }
+        chunk /= 2;
+    }
     return chunk;
 }
 int bwd_slab_frames(void)  { static int v = env_int("BBHIP_BWD_SLAB", 0);  return ((v + 63) / 64) * 64; }       // 0: chosen per call
@@ -543,7 +549,7 @@ int run_forward(ForwardCall const &call, int input_rows, hipStream_t st, Scratch
             // fp32 frames want (a unit's set-up weighs less), halved while they would leave the launch short of workgroups
             a.own_index = a.own_index_out; a.own_index_out = nullptr; a.stat_units = chunk_count;
             c.xmode = kXBit;
-            int own_chunk = 1024;
+            int own_chunk = 2048;
             while (own_chunk > 256 && (long long)ceil_div(c.frame_size, own_chunk) * tile_count < 2048) { own_chunk /= 2; }
             a.chunk = own_chunk; a.chunk_count = ceil_div(c.frame_size, own_chunk);
         }

@@ -253,6 +253,12 @@ constexpr int kInlineStatUnits = 4 * kWave; // most units whose partial sums a w
 // apply the batch-norm output stage (kind 1) and store.  ok: the frame belongs to the unit; live: the node exists.
 // bits_mask (binarized fp32 output with a packed copy): where given, the lane mask of the step's binarized output is handed back
 // instead of stored, and the caller stores the words of several steps together.
+// the batch-norm output of a LUT output v (reference: DifferentiableLutN.h:831-835); one expression for every kernel that forms it
+__device__ __forceinline__ float batch_norm_output(float v, float mean, float rstd, float gamma, float beta)
+{
+    return ((v - mean) * rstd) * gamma + beta;
+}
+
 template <int YMODE, int FWD_KIND>
 __device__ __forceinline__ void forward_stage(FwdArgs const &a, float v, bool ok, bool live, int lane, int node, int f0, int f, int f_end,
                                               float mean, float rstd, float c0, float dyv, float &s1, float &s2, uint64_t *bits_mask = nullptr)
@@ -264,17 +270,14 @@ __device__ __forceinline__ void forward_stage(FwdArgs const &a, float v, bool ok
         return;
     }
     if (FWD_KIND == 3) {
-        float const t = ((v - mean) * rstd) * a.gamma + a.beta;
+        float const t = batch_norm_output(v, mean, rstd, a.gamma, a.beta);
         float d = ok ? dyv : 0.0f;
         if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
         s1 += d;
         s2 = __builtin_fmaf(d, v - mean, s2);
         return;
     }
-    if (FWD_KIND == 1) {
-        v = (v - mean) * rstd;
-        v = v * a.gamma + a.beta;
-    }
+    if (FWD_KIND == 1) { v = batch_norm_output(v, mean, rstd, a.gamma, a.beta); }
     if (!live) { return; }
     if (YMODE == kYBit) {
         uint64_t const m = __ballot(ok && (v > 0.5f));
@@ -566,15 +569,42 @@ __device__ __forceinline__ uint32_t corner_index(Raw const (&raw)[N])
     return index;
 }
 
-// A corner-value wavefront's pass over U wavefront-steps from frame fb of its unit (see lut_forward_corner_kernel): KIND says what is
-// done with the LUT output of a frame (forward_stage).
+// What a corner-value wavefront looks up per frame.  The LUT output of a frame is one of the node's 2^N corner values, so everything
+// that a kind computes from it alone is computed once per corner — by lane p for corner p, with the operations the polynomial
+// kernels apply per frame (same bits) — and the frames fetch the finished value from the lane that holds it:
+//   kinds 0, 1: tab0 = the output (batch-norm stage for kind 1, then clamped to [0, 1], or 1 / 0 where the output is binarized)
+//   kind 2    : tab0 = V - C0, the term of the statistics sums
+//   kind 3    : tab0 = 1 / 0, whether the batch-norm output lies inside the hard-tanh window;  tab1 = V - mean
+struct CornerTables { int tab0, tab1; };
+
+template <int YMODE, int KIND>
+__device__ __forceinline__ CornerTables corner_tables(FwdArgs const &a, float v, float mean, float rstd, float c0)
+{
+    CornerTables t{0, 0};
+    if (KIND == 2) { t.tab0 = __float_as_int(v - c0); }
+    else if (KIND == 3) {
+        float const b = batch_norm_output(v, mean, rstd, a.gamma, a.beta);
+        t.tab0 = __float_as_int((b <= 0.0f || b >= 1.0f) ? 0.0f : 1.0f);
+        t.tab1 = __float_as_int(v - mean);
+    }
+    else {
+        float y = (KIND == 1) ? batch_norm_output(v, mean, rstd, a.gamma, a.beta) : v;
+        if (YMODE == kYClamp) { y = __builtin_amdgcn_fmed3f(y, 0.0f, 1.0f); }
+        else                  { y = (y > 0.5f) ? 1.0f : 0.0f; }
+        t.tab0 = __float_as_int(y);
+    }
+    return t;
+}
+
+// A corner-value wavefront's pass over U wavefront-steps from frame fb of its unit (see lut_forward_corner_kernel).
 // OWN: where the corner indices come from.  kOwnNone: from the gathered inputs; kOwnMemory: from the bytes that the statistics launch
 // of the call kept (FwdArgs::own_index); kOwnRegister: from `own`, which an earlier pass of the same wavefront over the same frames
 // left there.  `own` always returns the indices of the pass, byte u = 4 x the index of frame fb + 64 u + lane.
 enum OwnIndex : int { kOwnNone = 0, kOwnMemory = 1, kOwnRegister = 2 };
-template <int N, int XMODE, int YMODE, int KIND, bool WIDE, int OWN>
-__device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows)[N], int corner, int node, int lane, int fb,
-                                            int f_end, int f_last, float mean, float rstd, float c0, float &s1, float &s2, uint32_t &own)
+// RAGGED: the pass may reach beyond the unit's last frame (else all of its U steps are whole, and nothing is masked)
+template <int N, int XMODE, int YMODE, int KIND, bool WIDE, int OWN, bool RAGGED = true>
+__device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows)[N], CornerTables tabs, int node, int lane, int fb,
+                                            int f_end, int f_last, float &s1, float &s2, uint32_t &own)
 {
     constexpr int U = (XMODE == kXBit && !WIDE && OWN == kOwnNone) ? 2 : 4;  // wavefront-steps whose loads are issued together
     typename Gather<N, XMODE>::Raw raw[U][N];
@@ -584,9 +614,9 @@ __device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows
     if constexpr (WIDE && OWN == kOwnNone) { corner_masks_wide<N>(rows, fb, raw); }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        if (fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
+        if (!RAGGED || fb + u * kWave < f_end) {            // wave-uniform: steps beyond the unit load nothing
             if constexpr (!WIDE && OWN == kOwnNone) { Gather<N, XMODE>::load_raw(rows, fb + u * kWave, lane, f_last, raw[u]); }
-            if (KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + min(fb + u * kWave + lane, f_last)]; }
+            if (KIND == 3) { dyv[u] = a.dy[(size_t)node * a.dy_stride + (RAGGED ? min(fb + u * kWave + lane, f_last) : fb + u * kWave + lane)]; }
         }
     }
     constexpr bool kPackedCopy = (YMODE == kYBinarize) && (KIND == 0 || KIND == 1);
@@ -594,41 +624,73 @@ __device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         int const f0 = fb + u * kWave;
-        if (f0 >= f_end) { break; }
+        if (RAGGED && f0 >= f_end) { break; }
         int const  f  = f0 + lane;
-        bool const ok = f < f_end;
+        bool const ok = !RAGGED || f < f_end;
         uint32_t index4;
         if constexpr (OWN != kOwnNone) { index4 = (own >> (8 * u)) & 0xffu; }
         else {
             index4 = corner_index<N, XMODE>(raw[u]) << 2;
             if (U == 4) { own |= index4 << (8 * u); }
         }
-        float const v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index4, corner));
-        uint64_t m = 0;
-        forward_stage<YMODE, KIND>(a, v, ok, true, lane, node, f0, f, f_end, mean, rstd, c0,
-                                   (KIND == 3) ? dyv[u] : 0.0f, s1, s2, kPackedCopy ? &m : nullptr);
-        if (kPackedCopy) {
-            asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)m), "n"(2 * u));               // words[lane 2u] = low half
-            asm("v_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)(m >> 32)), "n"(2 * u + 1));
+        float const t0 = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index4, tabs.tab0));
+        if (KIND == 2) {
+            float const d = ok ? t0 : 0.0f;
+            s1 += d;
+            s2 = __builtin_fmaf(d, d, s2);
+        }
+        else if (KIND == 3) {
+            // (reference: DifferentiableLutN.h:1206-1222: dy behind the hard-tanh window, summed alone and times the centred output)
+            float const t1 = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index4, tabs.tab1));
+            float const d  = (ok && t0 != 0.0f) ? dyv[u] : 0.0f;
+            s1 += d;
+            s2 = __builtin_fmaf(d, t1, s2);
+        }
+        else if (YMODE == kYBit) {
+            uint64_t const m = __ballot(ok && (t0 > 0.5f));
+            uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
+            if (lane == 0)                                      { yr[0] = (uint32_t)m; }
+            if (lane == 32 && (!RAGGED || (f0 + 32) < f_end))   { yr[1] = (uint32_t)(m >> 32); }
+        }
+        else {
+            if (kPackedCopy && a.y_bits != nullptr) {         // wave-uniform
+                uint64_t const m = __ballot(ok && (t0 > 0.5f));
+                // words[lane 2u] = low half, words[lane 2u + 1] = high half.  The mask may come straight from a vector compare, and
+                // v_writelane_b32 must not read a scalar register in the wait states after a vector instruction wrote it (the
+                // compiler does not look into the asm): both instructions wait for themselves.
+                asm("s_nop 3\n\tv_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)m), "n"(2 * u));
+                asm("s_nop 3\n\tv_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)(m >> 32)), "n"(2 * u + 1));
+            }
+            if (ok) { __builtin_nontemporal_store(t0, reinterpret_cast<float *>(a.y) + (size_t)node * a.y_stride + f); }
         }
     }
     // the packed copy of the pass: its 2 U words by one store (a store per step would double the kernel's store instructions)
-    if (kPackedCopy && a.y_bits != nullptr && lane < 2 * U && fb + 32 * lane < f_end) {
+    if (kPackedCopy && a.y_bits != nullptr && lane < 2 * U && (!RAGGED || fb + 32 * lane < f_end)) {
         a.y_bits[(size_t)node * a.y_bits_stride + (fb >> 5) + lane] = words;
     }
+}
+
+// corner_pass, whole or ragged as the pass lies in the unit (wave-uniform)
+template <int N, int XMODE, int YMODE, int KIND, bool WIDE, int OWN>
+__device__ __forceinline__ void corner_pass_any(FwdArgs const &a, void const *(&rows)[N], CornerTables tabs, int node, int lane, int fb,
+                                                int f_end, int f_last, float &s1, float &s2, uint32_t &own)
+{
+    constexpr int U = (XMODE == kXBit && !WIDE && OWN == kOwnNone) ? 2 : 4;
+    if (fb + kWave * U <= f_end) { corner_pass<N, XMODE, YMODE, KIND, WIDE, OWN, false>(a, rows, tabs, node, lane, fb, f_end, f_last, s1, s2, own); }
+    else                         { corner_pass<N, XMODE, YMODE, KIND, WIDE, OWN, true>(a, rows, tabs, node, lane, fb, f_end, f_last, s1, s2, own); }
 }
 
 // The passes of a corner-value wavefront over its unit.  OWN as in corner_pass (kOwnNone or kOwnMemory); the statistics kind over
 // fp32 frames keeps its corner indices for the output launch where the call asks for it (FwdArgs::own_index_out).
 template <int N, int XMODE, int YMODE, int KIND, bool WIDE, int OWN = kOwnNone>
-__device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(&rows)[N], int corner, int node, int lane,
-                                                 int f_begin, int f_end, int f_last, float mean, float rstd, float c0, float &s1, float &s2)
+__device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(&rows)[N], CornerTables tabs, int node, int lane,
+                                                 int f_begin, int f_end, int f_last, float &s1, float &s2)
 {
     constexpr int U = (XMODE == kXBit && !WIDE && OWN == kOwnNone) ? 2 : 4;
     constexpr bool kKeepIndex = (XMODE == kXBinary) && (KIND == 2);
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
         uint32_t own;
-        corner_pass<N, XMODE, YMODE, KIND, WIDE, OWN>(a, rows, corner, node, lane, fb, f_end, f_last, mean, rstd, c0, s1, s2, own);
+        corner_pass_any<N, XMODE, YMODE, KIND, WIDE, OWN>(a, rows, tabs, node, lane, fb, f_end, f_last, s1, s2, own);
         if (kKeepIndex && a.own_index_out != nullptr) {      // (wave-uniform; steps beyond the unit left their byte 0)
             a.own_index_out[(size_t)node * a.own_stride + (fb >> 8) * kWave + lane] = own;
         }
@@ -711,17 +773,18 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
             constexpr bool kKeep = (XMODE == kXBinary || WIDE) && (OWN == kOwnNone);
             bool const keep = kKeep && (f_end - f_begin <= kInlineUnitPasses * 4 * kWave);      // wave-uniform
             uint32_t kept[kInlineUnitPasses];
+            CornerTables const stat_tabs = corner_tables<YMODE, 2>(a, __int_as_float(corner), 0.0f, 1.0f, c0);
             if (keep) {
                 if constexpr (kKeep) {
 #pragma unroll
                     for (int q = 0; q < kInlineUnitPasses; ++q) {
                         int const fb = f_begin + q * 4 * kWave;
                         kept[q] = 0;
-                        if (fb < f_end) { corner_pass<N, XMODE, YMODE, 2, WIDE, kOwnNone>(a, rows, corner, node, lane, fb, f_end, f_last, 0.0f, 1.0f, c0, s1, s2, kept[q]); }
+                        if (fb < f_end) { corner_pass_any<N, XMODE, YMODE, 2, WIDE, kOwnNone>(a, rows, stat_tabs, node, lane, fb, f_end, f_last, s1, s2, kept[q]); }
                     }
                 }
             }
-            else { corner_unit_pass<N, XMODE, YMODE, 2, WIDE, OWN>(a, rows, corner, node, lane, f_begin, f_end, f_last, 0.0f, 1.0f, c0, s1, s2); }
+            else { corner_unit_pass<N, XMODE, YMODE, 2, WIDE, OWN>(a, rows, stat_tabs, node, lane, f_begin, f_end, f_last, s1, s2); }
             batch_statistics(wave_sum(s1), wave_sum(s2), c0, a.frame_size, mean, var, rstd);
             mean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mean)));
             var  = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(var)));
@@ -729,10 +792,11 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
             s1 = 0.0f; s2 = 0.0f;
             if (keep) {
                 if constexpr (kKeep) {
+                    CornerTables const out_tabs = corner_tables<YMODE, FWD_KIND>(a, __int_as_float(corner), mean, rstd, c0);
 #pragma unroll
                     for (int q = 0; q < kInlineUnitPasses; ++q) {
                         int const fb = f_begin + q * 4 * kWave;
-                        if (fb < f_end) { corner_pass<N, XMODE, YMODE, FWD_KIND, WIDE, kOwnRegister>(a, rows, corner, node, lane, fb, f_end, f_last, mean, rstd, c0, s1, s2, kept[q]); }
+                        if (fb < f_end) { corner_pass_any<N, XMODE, YMODE, FWD_KIND, WIDE, kOwnRegister>(a, rows, out_tabs, node, lane, fb, f_end, f_last, s1, s2, kept[q]); }
                     }
                 }
                 f_done = true;
@@ -742,7 +806,10 @@ __global__ __launch_bounds__(kBlock) void lut_forward_corner_kernel(FwdArgs a)
     }
     if (FWD_KIND == 3) { mean = a.mean[node]; rstd = a.rstd[node]; }
 
-    if (!f_done) { corner_unit_pass<N, XMODE, YMODE, FWD_KIND, WIDE, OWN>(a, rows, corner, node, lane, f_begin, f_end, f_last, mean, rstd, c0, s1, s2); }
+    if (!f_done) {
+        CornerTables const tabs = corner_tables<YMODE, FWD_KIND>(a, __int_as_float(corner), mean, rstd, c0);
+        corner_unit_pass<N, XMODE, YMODE, FWD_KIND, WIDE, OWN>(a, rows, tabs, node, lane, f_begin, f_end, f_last, s1, s2);
+    }
     if (FWD_KIND == 2 || FWD_KIND == 3) { forward_store_stats(a, ck, node, true, lane, s1, s2); }
     if (FWD_KIND == 1) { forward_store_statistics(a, node, true, ck, lane, mean, var, rstd); }
     if (YMODE == kYBinarize && (FWD_KIND == 0 || FWD_KIND == 1)) { zero_packed_tail(a, ck, node, true, lane); }
