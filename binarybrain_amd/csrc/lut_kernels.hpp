@@ -1071,6 +1071,11 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
         dvarf = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(dvarf)));
     }
     float const grs = a.gamma * rstd;
+    int corner_open = 0;        // lane p: 1 where the batch-norm output of corner p lies inside the hard-tanh window, else 0
+    if (CORNER) {
+        float const t = batch_norm_output(__int_as_float(corner), mean, rstd, a.gamma, a.beta);
+        corner_open = (t <= 0.0f || t >= 1.0f) ? 0 : 1;
+    }
 
     int const f_begin = a.f_base + sl * a.slab;
     int const f_end   = min(f_begin + a.slab, a.f_limit);
@@ -1116,10 +1121,17 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
             if (BWD_KIND != 0) {
                 // hard-tanh window on the batch-norm output (reference: DifferentiableLutN.h:1206-1211, 1241-1246)
                 float v;
-                if constexpr (CORNER) { v = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(corner_index<N, XMODE>(raw[u]) << 2), corner)); }
-                else                  { v = LutEval<N>::combine(h, q); }
-                float const t = ((v - mean) * rstd) * a.gamma + a.beta;
-                if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
+                if constexpr (CORNER) {
+                    // the window depends on the corner alone: lane p decided it for corner p before the loop (same operations)
+                    int const index4 = (int)(corner_index<N, XMODE>(raw[u]) << 2);
+                    v = __int_as_float(__builtin_amdgcn_ds_bpermute(index4, corner));
+                    if (__builtin_amdgcn_ds_bpermute(index4, corner_open) == 0) { d = 0.0f; }
+                }
+                else {
+                    v = LutEval<N>::combine(h, q);
+                    float const t = batch_norm_output(v, mean, rstd, a.gamma, a.beta);
+                    if (t <= 0.0f || t >= 1.0f) { d = 0.0f; }
+                }
                 // dL/d(LUT output) (reference: DifferentiableLutN.h:1248-1250)
                 d = ok ? (__builtin_fmaf(d, grs, dmean) + v * dvarf) : 0.0f;
                 if (DXMODE == kDxNone && ok) { a.dx[(size_t)node * a.dx_stride + f] = d; }
