@@ -648,9 +648,8 @@ __device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows
         }
         else if (YMODE == kYBit) {
             uint64_t const m = __ballot(ok && (t0 > 0.5f));
-            uint32_t *yr = reinterpret_cast<uint32_t *>(a.y) + (size_t)node * a.y_stride + (f0 >> 5);
-            if (lane == 0)                                      { yr[0] = (uint32_t)m; }
-            if (lane == 32 && (!RAGGED || (f0 + 32) < f_end))   { yr[1] = (uint32_t)(m >> 32); }
+            asm("s_nop 3\n\tv_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)m), "n"(2 * u));         // (as below)
+            asm("s_nop 3\n\tv_writelane_b32 %0, %1, %2" : "+v"(words) : "s"((uint32_t)(m >> 32)), "n"(2 * u + 1));
         }
         else {
             if (kPackedCopy && a.y_bits != nullptr) {         // wave-uniform
@@ -667,6 +666,10 @@ __device__ __forceinline__ void corner_pass(FwdArgs const &a, void const *(&rows
     // the packed copy of the pass: its 2 U words by one store (a store per step would double the kernel's store instructions)
     if (kPackedCopy && a.y_bits != nullptr && lane < 2 * U && (!RAGGED || fb + 32 * lane < f_end)) {
         a.y_bits[(size_t)node * a.y_bits_stride + (fb >> 5) + lane] = words;
+    }
+    // packed output: the same, to the words of the output row that hold frames of the unit
+    if (YMODE == kYBit && (KIND == 0 || KIND == 1) && lane < 2 * U && (!RAGGED || fb + 32 * lane < f_end)) {
+        reinterpret_cast<uint32_t *>(a.y)[(size_t)node * a.y_stride + (fb >> 5) + lane] = words;
     }
 }
 
