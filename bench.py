@@ -465,6 +465,7 @@ def bench_differentiablelut6(args, lib):
     packed = ops.packed_input_buffer(I, F)                   # ... and the packed copy of its binarized input
     plain = getattr(args, "plain_signatures", False)
     clamp_w = None if plain else (0.0, 1.0)
+    yb = torch.zeros((idx.shape[0], xb.shape[1]), dtype=torch.int32, device="cuda") if bits else None      # the layer's packed output buffer
 
     def step():
         # (the table is clamped to [0, 1] in place by the forward entry, as the model class does before a forward pass; with the
@@ -472,7 +473,7 @@ def bench_differentiablelut6(args, lib):
         if plain:
             ops.vector_clamp_(W, 0.0, 1.0)
         if bits:
-            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=clamp_w, tables=tables)
+            y, mean, rstd = ops.bit_differentiable_lut_forward_training(6, xb, idx, W, F, rm, rv, clamp_w=clamp_w, tables=tables, out=yb)
             ops.bit_differentiable_lut_backward(6, xb, dy, idx, W, dW, F, mean, rstd, rev, tables=tables)
         else:
             y, mean, rstd = ops.differentiable_lut_forward_training(6, x, idx, W, F, rm, rv, clamp_w=clamp_w, packed=packed, tables=tables)

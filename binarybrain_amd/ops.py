@@ -699,10 +699,13 @@ def differentiable_lut_forward_training(n, x, idx, W, frame_size, running_mean, 
 
 
 def bit_differentiable_lut_forward_training(n, xbits, idx, W, frame_size, running_mean, running_var, gamma=0.3, beta=0.5,
-                                            momentum=0.9, bias=0.25, lut_binarize=False, clamp_w=None, tables=None):
+                                            momentum=0.9, bias=0.25, lut_binarize=False, clamp_w=None, tables=None, out=None):
+    """out: a packed output buffer [O, words] to write into (a layer keeps one); None: a new zero-filled one."""
     _dev(xbits, idx, W, running_mean, running_var)
     O = idx.shape[0]
-    y = torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    y = out if out is not None else torch.zeros((O, xbits.shape[1]), dtype=torch.int32, device=xbits.device)
+    if tuple(y.shape) != (O, xbits.shape[1]) or y.dtype != torch.int32:
+        raise ValueError("out must be int32 [%d, %d]" % (O, xbits.shape[1]))
     mean = torch.empty(O, dtype=torch.float32, device=xbits.device)
     rstd = torch.empty(O, dtype=torch.float32, device=xbits.device)
     _hint_tables(tables, False)
