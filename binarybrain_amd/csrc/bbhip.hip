@@ -827,7 +827,20 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
     if (dxmode == kDxNone) {
         bool const bit_corner = (c.xmode == kXBit) && use_corner_values(c.xmode);
         int const steps  = dx_pass_steps_env() ? dx_pass_steps_env() : (bit_corner ? 4 : 2);        // wavefront-steps per pass: {1, 2, 4}
-        int const frames = dx_chunk_frames_env() ? dx_chunk_frames_env() : (bit_corner ? 256 : 128);
+        // Packed rows with up to about a thousand input nodes (the layers of a convolution: tens to hundreds of channels x taps, very
+        // many frames): the words of a pass are read with one scalar load per row — the rows then stay in the scalar cache.  With
+        // more rows they do not, and the vector loads are faster (dx kernel at 324 / 512 / 1024 / 2048 rows: 94 / 107 / 138 / 141 us
+        // against 104 / 127 / 147 / 135 us; 4096 rows: 385 against 319 us per step).
+        bool const wide = bit_corner && dx_wide_rows() && steps == 4 && c.input_node_size <= dx_wide_max_rows() && c.x_stride % 8 == 0 &&
+                          (reinterpret_cast<uintptr_t>(c.x) % 32u) == 0;
+        int frames = dx_chunk_frames_env() ? dx_chunk_frames_env() : (bit_corner ? 256 : 128);
+        if (wide && dx_chunk_frames_env() == 0) {
+            // ... and such layers have few wavefronts' worth of input nodes and many frames: units of 1024 frames, so that a
+            // wavefront's set-up (its list, its share of it) serves four passes, halved while the launch would fall short of workgroups
+            // (conv block 0.602 -> 0.590 ms; the same units for a 4096-row layer: 0.338 -> 0.358 ms, hence only here)
+            frames = 1024;
+            while (frames > 256 && (long long)ceil_div(c.frame_size, frames) * ceil_div(c.input_node_size, kWavesPerBlk) < 2048) { frames /= 2; }
+        }
         int const chunk  = ((frames + kWave * steps - 1) / (kWave * steps)) * (kWave * steps);
         int const chunk_count = ceil_div(c.frame_size, chunk);
         // few input nodes with long work lists: the four wavefronts of a workgroup share one input node (DxArgs::split)
@@ -840,12 +853,6 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
         d.x_stride = c.x_stride; d.dy_stride = c.frame_stride; d.dx_stride = c.frame_stride;
         d.chunk = chunk; d.chunk_count = chunk_count; d.tiles = make_tile_divisor(in_tiles);
         d.bias = c.bias; d.split = split ? 1 : 0;
-        // Packed rows with up to about a thousand input nodes (the layers of a convolution: tens to hundreds of channels x taps, very
-        // many frames): the words of a pass are read with one scalar load per row — the rows then stay in the scalar cache.  With
-        // more rows they do not, and the vector loads are faster (dx kernel at 324 / 512 / 1024 / 2048 rows: 94 / 107 / 138 / 141 us
-        // against 104 / 127 / 147 / 135 us; 4096 rows: 385 against 319 us per step).
-        bool const wide = bit_corner && dx_wide_rows() && steps == 4 && c.input_node_size <= dx_wide_max_rows() && c.x_stride % 8 == 0 &&
-                          (reinterpret_cast<uintptr_t>(c.x) % 32u) == 0;
         // folding the slab sums into dW rides at the end of this launch
         d.fin_partial = part; d.fin_dW = c.dW; d.fin_node_size = c.output_node_size; d.fin_slab_count = slab_total;
         d.fin_overwrite = dw_overwrite;
