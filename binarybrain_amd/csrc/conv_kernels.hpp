@@ -71,12 +71,16 @@ __global__ __launch_bounds__(kConvBlock) void im2col_forward_kernel(Im2ColArgs a
     // all loads of a wavefront's 16 rows are issued before the first of them is used (one round trip instead of sixteen)
     constexpr int kRows = kTile / (kConvBlock / 64);
     float v[kRows];
+    int oy = (q0 + wave) / a.ow, ox = (q0 + wave) - oy * a.ow;      // of the wavefront's first row; the next rows step on from it
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
         int const q = q0 + wave + r * (kConvBlock / 64);
         v[r] = a.border_value;
+        if (r > 0) {
+            ox += kConvBlock / 64;
+            while (ox >= a.ow) { ox -= a.ow; ++oy; }
+        }
         if (q < plane) {
-            int const oy = q / a.ow, ox = q - oy * a.ow;
             int iy, ix;
             bool const have = im2col_source(a, oy, ox, fy, fx, iy, ix);  // wave-uniform
             if (have && f0 + lane < a.input_frame_size) {
@@ -149,7 +153,36 @@ __global__ __launch_bounds__(kConvBlock) void im2col_backward_kernel(Im2ColArgs 
 
     int const iy_limit = (a.oh - 1) * a.y_stride, ix_limit = (a.ow - 1) * a.x_stride;
     size_t const plane = (size_t)a.oh * a.ow;
-    if (p < hw) {
+    if (kPer <= 4 && a.x_stride == 1 && a.y_stride == 1 && a.fh <= 3 && a.fw <= 3) {
+        // Filters up to 3 x 3 at stride 1 (workgroup-uniform): the loads of all taps go out together — nine round trips become one —
+        // and the sums are formed in the same (fy, fx) order afterwards.  A tap outside the window contributes +0, which leaves a
+        // sum that started at +0 unchanged.
+        float v[3][3][kPer];
+        int const y = (p < hw) ? p / a.w : 0, x = (p < hw) ? p - y * a.w : 0;
+#pragma unroll
+        for (int fy = 0; fy < 3; ++fy) {
+#pragma unroll
+            for (int fx = 0; fx < 3; ++fx) {
+                int const iy = y - fy + a.y_offset, ix = x - fx + a.x_offset;
+                bool const have = (p < hw) && fy < a.fh && fx < a.fw && iy >= 0 && iy <= iy_limit && ix >= 0 && ix <= ix_limit;
+                float const *row = dy + (size_t)((c * a.fh + fy) * a.fw + fx) * a.output_frame_stride + (size_t)iy * a.ow + ix;
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) {
+                    int const f = f0 + wave + j * kWaves;
+                    v[fy][fx][j] = (have && f < a.input_frame_size) ? row[(size_t)f * plane] : 0.0f;
+                }
+            }
+        }
+#pragma unroll
+        for (int fy = 0; fy < 3; ++fy) {
+#pragma unroll
+            for (int fx = 0; fx < 3; ++fx) {
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) { acc[j] += v[fy][fx][j]; }
+            }
+        }
+    }
+    else if (p < hw) {
         int const y = p / a.w, x = p - y * a.w;
         int const x_align = x % a.x_stride, y_align = y % a.y_stride;
         for (int fy = y_align; fy < a.fh; fy += a.y_stride) {
