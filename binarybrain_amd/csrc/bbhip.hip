@@ -144,6 +144,7 @@ bool pack_binarized_input(void) { static bool const on = env_switch("BBHIP_PACK"
 // the corner-value forward kernel derives a node's tables in the wavefront where no packing launch carries the preparation (0 = a table launch)
 bool inline_tables(void) { static bool const on = env_switch("BBHIP_INLINE_TABLES", true); return on; }
 // packed rows in the dx kernel read with one scalar load per row and pass where pitch and alignment allow (0 = vector loads + read-lanes)
+bool term_from_corner_values(void) { static bool const on = env_switch("BBHIP_TERM_NODES", true); return on; }
 bool dx_wide_rows(void) { static bool const on = env_switch("BBHIP_DX_WIDE", true); return on; }
 int dx_wide_max_rows(void) { static int const v = env_int("BBHIP_DX_WIDE_ROWS", 1024); return v; }
 
@@ -758,6 +759,10 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
         tt.blocks = (int)blocks;
         tt.corner = use_corner_values(c.xmode) ? 1 : 0;
         tt.lo = 0.5f - c.bias; tt.hi = 0.5f + c.bias;
+        if (corner && term_from_corner_values()) {      // the nodes' corner values are at hand: the records are built node by node from them
+            tt.V = V; tt.node_size = c.output_node_size;
+            tt.blocks = (ceil_div(c.output_node_size, kWavesPerBlk) + 7) & ~7;
+        }
     }
 
     BwdArgs a{};
