@@ -145,6 +145,7 @@ bool pack_binarized_input(void) { static bool const on = env_switch("BBHIP_PACK"
 bool inline_tables(void) { static bool const on = env_switch("BBHIP_INLINE_TABLES", true); return on; }
 // packed rows in the dx kernel read with one scalar load per row and pass where pitch and alignment allow (0 = vector loads + read-lanes)
 bool term_from_corner_values(void) { static bool const on = env_switch("BBHIP_TERM_NODES", true); return on; }
+bool dx_indexed(void) { static bool const on = env_switch("BBHIP_DX_INDEXED", true); return on; }
 bool dx_wide_rows(void) { static bool const on = env_switch("BBHIP_DX_WIDE", true); return on; }
 int dx_wide_max_rows(void) { static int const v = env_int("BBHIP_DX_WIDE_ROWS", 1024); return v; }
 
@@ -700,13 +701,26 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
     int const stat_chunk       = fwd_chunk_frames(c.xmode, c.frame_size, ceil_div(c.output_node_size, kWavesPerBlk * stat_npw));
     int const stat_chunk_count = ceil_div(c.frame_size, stat_chunk);
     size_t const stat_bytes = c.bn ? align256((size_t)stat_chunk_count * c.output_node_size * 2 * sizeof(float)) : 0;
-    size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + NN / 2) : 0;
+    // Batch-norm backward of a small batch over packed rows: the statistics pass (passes of four steps over 32-byte groups of the rows)
+    // keeps the corner index it forms of every (node, frame), a byte each, and the dx kernel looks a term's value up at that index
+    // instead of reading the consumer's other five rows and forming the index again (lut_dx_indexed_kernel): a third of the vector
+    // instructions per term.  That pays where dy and the indices stay close to the compute units (classifier step: dx of the three
+    // layers 43.9 -> 38 us); at 4096 x 4096 x 8192 and at the conv block's 230 400 frames the dx kernel is bound by the gather of its
+    // dy rows and the kept bytes only add traffic (128.5 vs 128.1 us, 121 vs 114 us, statistics pass + 6 us): up to 32 MiB of both.
+    int const own_words = ceil_div(c.frame_size, 256) * kWave;
+    bool const indexed = c.bn && dxmode == kDxNone && corner && term_from_corner_values() && c.xmode == kXBit && dx_indexed() &&
+                         dx_pass_steps_env() == 0 && (dx_chunk_frames_env() == 0 || dx_chunk_frames_env() % 256 == 0) &&
+                         c.x_stride % 8 == 0 && stat_chunk % 256 == 0 &&
+                         (size_t)c.output_node_size * c.frame_size * 5 <= ((size_t)32 << 20);
+    size_t const own_bytes = indexed ? align256((size_t)c.output_node_size * own_words * sizeof(uint32_t)) : 0;
+    size_t const term_count = (dxmode == kDxNone) ? (size_t)c.input_node_size * (size_t)(c.rev_stride - 1) * (kTermHead + (indexed ? NN : NN / 2)) : 0;
     size_t const dtab_bytes = align256(term_count * sizeof(int));
     size_t const dyh_bytes  = (dxmode == kDxNone && c.bn) ? align256((size_t)c.output_node_size * c.frame_stride * sizeof(float)) : 0;
     size_t const v_bytes = corner ? c_bytes : 0;
     size_t const bits_bytes = (pack && !have_bits) ? align256((size_t)c.input_node_size * c.x_stride * sizeof(uint32_t)) : 0;
     char *base = nullptr;
-    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes, &base, st)) { return 1; }
+    if (arena_get(c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes + own_bytes, &base, st)) { return 1; }
+    uint32_t *own = indexed ? reinterpret_cast<uint32_t *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes + v_bytes + bits_bytes) : nullptr;
     float *V    = corner ? reinterpret_cast<float *>(base + c_bytes + part_bytes + stat_bytes + dtab_bytes + dyh_bytes) : nullptr;
     float *C    = reinterpret_cast<float *>(base);
     float *part = reinterpret_cast<float *>(base + c_bytes);
@@ -762,6 +776,10 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
         if (corner && term_from_corner_values()) {      // the nodes' corner values are at hand: the records are built node by node from them
             tt.V = V; tt.node_size = c.output_node_size;
             tt.blocks = (ceil_div(c.output_node_size, kWavesPerBlk) + 7) & ~7;
+            if (indexed) {      // ... and point at the rows of kept corner indices instead of the input rows
+                tt.indexed = 1;
+                tt.x_base = (unsigned long long)(uintptr_t)own; tt.x_row_pitch_bytes = (unsigned long long)own_words * 4ULL;
+            }
         }
     }
 
@@ -786,6 +804,7 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
         f.node_size = c.output_node_size; f.frame_size = c.frame_size; f.x_stride = c.x_stride;
         f.chunk = stat_chunk; f.chunk_count = stat_chunk_count; f.tiles = make_tile_divisor(stat_tiles);
         f.bias = c.bias; f.gamma = c.gamma; f.beta = c.beta;
+        if (indexed) { f.own_index_out = own; f.own_stride = own_words; }
         if (dispatch_forward<N>(c.xmode, kYClamp, 3, f, npw, st)) { return 1; }
         BBHIP_LAUNCH_CHECK();
         if (stat_chunk_count <= kInlineStatUnits) {
@@ -863,9 +882,14 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
         d.fin_overwrite = dw_overwrite;
         d.fin_blocks = (ceil_div(c.output_node_size * NN, kBlock) + 7) & ~7;
         if ((long long)d.fin_blocks + (long long)chunk_count * in_tiles > 0x7fffffffLL) { return fail("backward: grid too large"); }
+        d.own_stride = own_words;
         {
             ScopedTimer tm(kTimeDx, st);
-            if (wide) {
+            if (indexed) {
+                dim3 const grid(d.fin_blocks + d.chunk_count * d.tiles.count), block(kBlock);
+                hipLaunchKernelGGL((lut_dx_indexed_kernel<N>), grid, block, 0, st, d);
+            }
+            else if (wide) {
                 dim3 const grid(d.fin_blocks + d.chunk_count * d.tiles.count), block(kBlock);
                 hipLaunchKernelGGL((lut_dx_corner_kernel<N, kXBit, 4, true>), grid, block, 0, st, d);
             }

@@ -236,6 +236,7 @@ struct FwdArgs {
     // row of own_stride words holds frames f + l, f + 64 + l, f + 128 + l, f + 192 + l.  The output launch of the same call
     // (own_index: the same buffer) then reads a word per lane and four steps instead of gathering the fp32 frames a second time.
     // Units of both launches begin at multiples of 256 frames.  Needs no count of the input's rows.
+    // The statistics pass of a backward call (kind 3, passes of four steps) keeps them the same way for lut_dx_indexed_kernel.
     uint32_t       *own_index_out;
     uint32_t const *own_index;
     int   own_stride;
@@ -690,7 +691,9 @@ __device__ __forceinline__ void corner_unit_pass(FwdArgs const &a, void const *(
                                                  int f_begin, int f_end, int f_last, float &s1, float &s2)
 {
     constexpr int U = (XMODE == kXBit && !WIDE && OWN == kOwnNone) ? 2 : 4;
-    constexpr bool kKeepIndex = (XMODE == kXBinary) && (KIND == 2);
+    // passes of four steps leave their corner indices in `own`: the statistics kinds keep them where the call asks for it
+    // (kind 2 over fp32 frames: for the output launch; kind 3: for the dx kernel of the same backward call, lut_dx_indexed_kernel)
+    constexpr bool kKeepIndex = (U == 4) && (OWN == kOwnNone) && ((XMODE == kXBinary && KIND == 2) || KIND == 3);
     for (int fb = f_begin; fb < f_end; fb += kWave * U) {
         uint32_t own;
         corner_pass_any<N, XMODE, YMODE, KIND, WIDE, OWN>(a, rows, tabs, node, lane, fb, f_end, f_last, s1, s2, own);
@@ -894,6 +897,10 @@ struct TermArgs {
     // (term_table_node_block: `blocks` then counts workgroups of kWavesPerBlk nodes)
     float const *V;             // [O][2^N]
     int node_size;
+    // ... and indexed != 0: the records are those of lut_dx_indexed_kernel: kTermHead + 2^N dwords, head = the address of the consumer's
+    // row of kept corner indices (x_base / x_row_pitch_bytes describe that buffer) and of its dy row, then the value at every corner of
+    // the node (all N inputs: the two corners that differ in input k hold the same)
+    int indexed;
 };
 
 // input j of a node's connections with connection k left out (j < N - 1, may differ per lane; k and the array index are compile-time)
@@ -993,7 +1000,8 @@ __device__ __forceinline__ void term_table_block(TermArgs const &a, int block)
 template <int N>
 __device__ __forceinline__ void term_table_node_block(TermArgs const &a, int block)
 {
-    constexpr int NN = 1 << N, HN = NN / 2, REC = kTermHead + HN;
+    constexpr int NN = 1 << N, HN = NN / 2;
+    int const REC = kTermHead + (a.indexed ? NN : HN);
     int const node = __builtin_amdgcn_readfirstlane(block * kWavesPerBlk + (int)(threadIdx.x / kWave));
     if (node >= a.node_size) { return; }
     int const lane = threadIdx.x & (kWave - 1);
@@ -1019,13 +1027,24 @@ __device__ __forceinline__ void term_table_node_block(TermArgs const &a, int blo
         }
         if (slot < 0) { continue; }                                             // (a reverse table that does not list the connection: nothing to write)
         int *out = a.term + ((size_t)ins[k] * a.fan.count + slot) * REC;
+        float const other = __shfl_xor(v, 1 << k, 64);
+        if (a.indexed) {
+            // the node's row of kept corner indices and its dy row; the value at every corner of the node (both corners of input k)
+            if (lane < 4) {
+                unsigned long long const addr = (lane < 2) ? a.x_base + (unsigned long long)(unsigned)node * a.x_row_pitch_bytes
+                                                           : a.dy_base + (unsigned long long)(unsigned)node * a.dy_row_pitch_bytes;
+                out[lane] = (lane & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
+            }
+            float const step = ((lane >> k) & 1) ? (v - other) : (other - v);
+            if (lane < NN) { out[kTermHead + lane] = __float_as_int(step * inv_step); }
+            continue;
+        }
         if (lane < 2 * N) {
             int const j = lane >> 1;
             unsigned long long const addr = (j < N - 1) ? a.x_base + (unsigned long long)(unsigned)ins_other<N>(ins, k, j) * a.x_row_pitch_bytes
                                                         : a.dy_base + (unsigned long long)(unsigned)node * a.dy_row_pitch_bytes;
             out[lane] = (lane & 1) ? (int)(addr >> 32) : (int)(addr & 0xffffffffULL);
         }
-        float const other = __shfl_xor(v, 1 << k, 64);
         if (lane < NN && ((lane >> k) & 1)) {
             int const sidx = (lane & ((1 << k) - 1)) | ((lane >> (k + 1)) << k);          // the corner's index with bit k taken out
             out[kTermHead + sidx] = __float_as_int((v - other) * inv_step);
@@ -1301,6 +1320,7 @@ struct DxArgs {
     float       *fin_dW;
     int   fin_node_size, fin_slab_count, fin_blocks;
     int   fin_overwrite;        // dW = instead of dW += (the caller's dW holds nothing: bbhip_HintTableGradientOverwrite)
+    int   own_stride;           // lut_dx_indexed_kernel: words per node row of the kept corner indices
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -1698,6 +1718,90 @@ __global__ __launch_bounds__(kBlock) void lut_dx_corner_kernel(DxArgs a)
                 for (int j = 0; j < T::M; ++j) { index |= (__uint_as_float(st.raw[u][j]) > 0.5f) ? (4u << j) : 0u; }
                 float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)index, values));
                 acc[u] = __builtin_fmaf(st.dyv[u], d, acc[u]);
+            }
+        }
+        dx_store_pass<U>(a, part, in, wave, lane, f_begin, acc);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+//  Input-centric dx from kept corner indices (batch-norm backward over two-valued inputs).  The statistics pass of the same
+//  call has formed the corner index of every (node, frame) and kept it, a byte each (FwdArgs::own_index_out); a term's
+//  dy/dx_k is its record's value at that corner (term_table_node_block with indexed = 1), so a term costs per pass one word of
+//  indices and four of dy per lane, and per step a byte extract, ds_bpermute and the multiply-add: no row of the other inputs
+//  is read and no index is formed.  Units (multiples of 256 frames), work list, split mode and the dW rider are those of
+//  lut_dx_corner_kernel, and so is the order of the sums: the same bits.
+// ------------------------------------------------------------------------------------------------
+template <int N>
+__global__ __launch_bounds__(kBlock) void lut_dx_indexed_kernel(DxArgs a)
+{
+    constexpr int U = 4, NN = 1 << N, REC = kTermHead + NN, HEAD = 4;
+    int const bid = blockIdx.x;
+    int const B   = a.chunk_count * a.tiles.count;
+    if (bid >= B) { dw_finalize_block<N>(a.fin_partial, a.fin_dW, a.fin_node_size, a.fin_slab_count, bid - B, a.fin_overwrite); return; }
+    int const lid  = xcd_remap(bid, B);
+    int ck, tile;
+    split_tile(lid, a.tiles, ck, tile);
+    __shared__ float part[kWavesPerBlk][U][kWave];
+    int const wave = threadIdx.x / kWave;
+    int in, share;
+    dx_list_share(a, tile, wave, in, share);
+    if (in >= a.input_node_size) { return; }            // (workgroup-uniform in split mode)
+    int const lane = threadIdx.x & (kWave - 1);
+
+    int const cnt = a.rev[(size_t)in * a.rev_stride];
+    int t_begin, t_end;
+    dx_list_range(cnt, share, t_begin, t_end);
+    typedef __attribute__((address_space(4))) int const const_int;
+    const_int *rec = (const_int *)(a.term + (size_t)in * (a.rev_stride - 1) * REC);
+    int const *rec_v = a.term + (size_t)in * (a.rev_stride - 1) * REC + kTermHead + (lane & (NN - 1));
+    uint32_t const y_row_bytes = (uint32_t)a.frame_size * 4u;
+    uint32_t const i_row_bytes = (uint32_t)a.own_stride * 4u;
+
+    for (int f_begin = ck * a.chunk; f_begin < min((ck + 1) * a.chunk, a.frame_size); f_begin += kWave * U) {
+        uint32_t const yoff = (uint32_t)(f_begin + lane) * 4u;
+        uint32_t const ioff = ((uint32_t)(f_begin >> 8) * kWave + (uint32_t)lane) * 4u;     // byte u of the word: frame f_begin + 64 u + lane
+        float acc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { acc[u] = 0.0f; }
+
+        // two terms in flight, as in lut_dx_corner_kernel: while term t is evaluated, the words of term t + 1 have been
+        // requested and the head of term t + 2 is on its way (four in flight measured slower: 136 vs 128 us at 4096 x 4096 x 8192)
+        int head[HEAD];
+        uint32_t iw_next = 0;
+        float dy_next[U];
+        int values_next = 0;
+        auto load_head = [&](int t) {
+#pragma unroll
+            for (int i = 0; i < HEAD; ++i) { head[i] = rec[(size_t)t * REC + i]; }
+        };
+        auto request = [&](int t) {                           // of the term whose head is in `head`
+            __amdgpu_buffer_rsrc_t const ir = address_descriptor((uint32_t)head[0], (uint32_t)head[1], i_row_bytes);
+            iw_next = __builtin_amdgcn_raw_buffer_load_b32(ir, ioff, 0, 0);
+            __amdgpu_buffer_rsrc_t const dyr = address_descriptor((uint32_t)head[2], (uint32_t)head[3], y_row_bytes);
+#pragma unroll
+            for (int u = 0; u < U; ++u) { dy_next[u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(dyr, yoff + u * (kWave * 4u), 0, 0)); }
+            values_next = rec_v[(size_t)t * REC];              // lane p: the term's value at corner p
+        };
+        if (t_begin < t_end) {
+            load_head(t_begin);
+            request(t_begin);
+            if (t_begin + 1 < t_end) { load_head(t_begin + 1); }
+        }
+        for (int t = t_begin; t < t_end; ++t) {
+            uint32_t const iw = iw_next;
+            float dyv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) { dyv[u] = dy_next[u]; }
+            int const values = values_next;
+            if (t + 1 < t_end) {
+                request(t + 1);
+                if (t + 2 < t_end) { load_head(t + 2); }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float const d = __int_as_float(__builtin_amdgcn_ds_bpermute((int)((iw >> (8 * u)) & 0xffu), values));
+                acc[u] = __builtin_fmaf(dyv[u], d, acc[u]);
             }
         }
         dx_store_pass<U>(a, part, in, wave, lane, f_begin, acc);

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
                                  {"BBHIP_DX_STEPS": "1", "BBHIP_DX_CHUNK": "64", "BBHIP_BIN_NODES": "1", "BBHIP_BIN_CHUNK": "64"},
                                  {"BBHIP_DX_STEPS": "4", "BBHIP_DX_CHUNK": "512", "BBHIP_FWD_CHUNK": "512", "BBHIP_BIN_NODES": "2", "BBHIP_BIN_CHUNK": "256"},
                                  {"BBHIP_DX_SPLIT": "1"}, {"BBHIP_DX_SPLIT": "0", "BBHIP_BIN_NODES": "4"},
-                                 {"BBHIP_DX_WIDE": "0"}, {"BBHIP_INLINE_TABLES": "0"}, {"BBHIP_FWD_CHUNK": "2048"}])
+                                 {"BBHIP_DX_WIDE": "0"}, {"BBHIP_INLINE_TABLES": "0"}, {"BBHIP_FWD_CHUNK": "2048"}, {"BBHIP_DX_INDEXED": "0"}, {"BBHIP_TERM_NODES": "0"}])
 def test_two_valued_inputs_under_switches(env):
     child_env = dict(os.environ)
     child_env.update(env)
