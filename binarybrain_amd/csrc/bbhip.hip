@@ -773,8 +773,9 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
         tt.blocks = (int)blocks;
         tt.corner = use_corner_values(c.xmode) ? 1 : 0;
         tt.lo = 0.5f - c.bias; tt.hi = 0.5f + c.bias;
-        if (corner && term_from_corner_values()) {      // the nodes' corner values are at hand: the records are built node by node from them
-            tt.V = V; tt.node_size = c.output_node_size;
+        // node by node: coefficient records always, value records where the nodes' corner values are at hand (batch-norm backward)
+        if (term_from_corner_values() && (corner || tt.corner == 0)) {
+            tt.V = corner ? V : nullptr; tt.node_size = c.output_node_size;
             tt.blocks = (ceil_div(c.output_node_size, kWavesPerBlk) + 7) & ~7;
             if (indexed) {      // ... and point at the rows of kept corner indices instead of the input rows
                 tt.indexed = 1;

@@ -893,9 +893,9 @@ struct TermArgs {
     int blocks;                 // workgroups that build records (kWavesPerBlk * kTermRecordsPerWave records each); 0 = nothing to build
     int corner;                 // 1: records hold the derivative's corner values for two-valued inputs (lut_dx_corner_kernel)
     float lo, hi;               //    the two input values, 1/2 -+ bias
-    // Not null (two-valued inputs, the call has the nodes' corner values at hand): the records are built node by node from them
-    // (term_table_node_block: `blocks` then counts workgroups of kWavesPerBlk nodes)
-    float const *V;             // [O][2^N]
+    // node_size > 0: the records are built node by node (term_table_node_block: `blocks` then counts workgroups of kWavesPerBlk nodes) —
+    // coefficient records (corner = 0) from W, value records from the nodes' corner values V, which the call then has at hand
+    float const *V;             // [O][2^N], or null
     int node_size;
     // ... and indexed != 0: the records are those of lut_dx_indexed_kernel: kTermHead + 2^N dwords, head = the address of the consumer's
     // row of kept corner indices (x_base / x_row_pitch_bytes describe that buffer) and of its dy row, then the value at every corner of
@@ -991,12 +991,13 @@ __device__ __forceinline__ void term_table_block(TermArgs const &a, int block)
     }
 }
 
-// The same records built node by node, for two-valued inputs whose corner values V the call has already derived: a wavefront takes a
-// node, and for each of its N connections finds the connection's place in the reverse-table row of its input (the lanes compare a row's
-// entries with the connection id), and writes the record there.  y is linear in input k between its two values, so dy/dx_k at a corner of
-// the other inputs is (V[k at hi] - V[k at lo]) / (hi - lo): one cross-lane exchange instead of a butterfly per record.  The work is
-// O x N records, not I x (largest fan-out) slots, and about a third of the instructions per record: for a layer of 784 inputs and 6144
-// nodes 2.5 us instead of 10.5 us.
+// The same records built node by node: a wavefront takes a node, and for each of its N connections finds the connection's place in the
+// reverse-table row of its input (the lanes compare a row's entries with the connection id), and writes the record there.  Coefficient
+// records share one butterfly per node (the plain-basis table does not depend on the connection).  Value records (two-valued inputs) are
+// built where the call has already derived the node's corner values V: y is linear in input k between its two values, so dy/dx_k at a
+// corner of the other inputs is (V[k at hi] - V[k at lo]) / (hi - lo), one cross-lane exchange instead of a butterfly per record.  The
+// work is O x N records, not I x (largest fan-out) slots, and a fraction of the instructions per record: for a layer of 784 inputs and
+// 6144 nodes 2.5 us instead of 10.5 us.
 template <int N>
 __device__ __forceinline__ void term_table_node_block(TermArgs const &a, int block)
 {
@@ -1008,7 +1009,20 @@ __device__ __forceinline__ void term_table_node_block(TermArgs const &a, int blo
     typedef __attribute__((address_space(4))) int const const_int;
     const_int *rev = (const_int *)a.rev;
     const_int *idx = (const_int *)a.idx;
-    float const v = a.V[(size_t)node * NN + (lane & (NN - 1))];
+    float v;
+    if (a.V != nullptr) { v = a.V[(size_t)node * NN + (lane & (NN - 1))]; }
+    else {
+        // coefficient records: P = plain-basis coefficients of W' (W' = lut_binarize ? W > 0.5 : W), the butterfly (a, b) -> (a, b - a)
+        // per index bit, as term_table_block forms them per record (same operations: same bits); a record takes the entries whose
+        // index has the connection's bit set
+        v = a.W[(size_t)node * NN + (lane & (NN - 1))];
+        if (a.lut_binarize) { v = (v > 0.5f) ? 1.0f : 0.0f; }
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            float const o = __shfl_xor(v, 1 << j, 64);
+            v = ((lane >> j) & 1) ? (v - o) : v;
+        }
+    }
     float const inv_step = 1.0f / (a.hi - a.lo);
     int ins[N], cnt[N];
 #pragma unroll
@@ -1047,7 +1061,7 @@ __device__ __forceinline__ void term_table_node_block(TermArgs const &a, int blo
         }
         if (lane < NN && ((lane >> k) & 1)) {
             int const sidx = (lane & ((1 << k) - 1)) | ((lane >> (k + 1)) << k);          // the corner's index with bit k taken out
-            out[kTermHead + sidx] = __float_as_int((v - other) * inv_step);
+            out[kTermHead + sidx] = __float_as_int((a.V != nullptr) ? (v - other) * inv_step : v);
         }
     }
 }
@@ -1110,7 +1124,7 @@ __global__ __launch_bounds__(kBlock) void lut_backward_kernel(BwdArgs a)
     int const B   = a.slab_count * a.tiles.count;
     if (DXMODE == kDxNone) {
         if (bid >= B) {
-            if (a.tt.V != nullptr) { term_table_node_block<N>(a.tt, bid - B); }
+            if (a.tt.node_size > 0) { term_table_node_block<N>(a.tt, bid - B); }
             else                   { term_table_block<N>(a.tt, bid - B); }
             return;
         }
