@@ -677,8 +677,17 @@ int run_backward(BackwardCall const &call, hipStream_t st, PackedInputHint packe
     // stay below 256 MiB
     int slab = bwd_slab_frames();
     if (slab == 0) {
+        // The kernel keeps five workgroups per compute unit: a launch runs in ceil(workgroups / 1280) rounds of them, and a slab costs
+        // its frames plus about 384 frames' worth of set-up and reduction (fitted to 112 / 121 / 122 us at slabs of 4096 / 2048 / 1024
+        // frames for 4096 nodes x 8192 frames).  The slab length with the least rounds x cost: 4096 there (two rounds), 2048 for
+        // 216 nodes x 230 400 frames (five rounds against three twice as long) and for 36 nodes (one round), 512 / 256 for the layers
+        // of the classifier at 1024 frames.
+        auto cost = [&](int frames) {
+            long long const groups = (long long)tile_count * range_count * ceil_div(range, frames);
+            return ((groups + 1279) / 1280) * (long long)(frames + 384);
+        };
         slab = 4096;
-        while (slab > 256 && (long long)tile_count * range_count * ceil_div(range, slab) < 2048) { slab /= 2; }
+        for (int cand = 2048; cand >= 256; cand /= 2) { if (cost(cand) < cost(slab)) { slab = cand; } }
     }
     for (;;) {
         long long slabs = (long long)range_count * ceil_div(range, slab);
